@@ -1,0 +1,214 @@
+"""ctypes front end of the CPU oracle (``oracle/tacker_oracle.c``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke``
+and by the ``cpu_baseline`` leg of ``bench.py``; the product package never
+imports it.  All functions take and return numpy arrays.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtacker_oracle.so")
+_lib = None
+
+
+def build(force=False):
+    """Compile the oracle with gcc (see ``oracle/Makefile``)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.run(["make", "-C", _HERE, "-B", "libtacker_oracle.so"], check=True,
+                       stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        build()
+        _lib = C.CDLL(_LIB_PATH)
+        _declare(_lib)
+    return _lib
+
+
+_f32p = np.ctypeslib.ndpointer(np.float32, flags="C_CONTIGUOUS")
+_u16p = np.ctypeslib.ndpointer(np.uint16, flags="C_CONTIGUOUS")
+_i32p = np.ctypeslib.ndpointer(np.int32, flags="C_CONTIGUOUS")
+
+
+def _declare(l):
+    l.orc_num_threads.restype = C.c_int
+    l.orc_tzgemm_dims.argtypes = [C.c_int, C.c_int, C.c_int, _i32p]
+    l.orc_tzgemm_tile_origin.argtypes = [C.c_uint, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    l.orc_tzgemm.argtypes = [_u16p, _u16p, _f32p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_int,
+                             C.c_int, C.c_int]
+    l.orc_gptb_index.argtypes = [C.c_uint, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i32p]
+    l.orc_stencil_gptb.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int,
+                                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    l.orc_stencil.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+    l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    l.orc_mriq_gptb.argtypes = [C.c_int, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, C.c_int,
+                                C.c_int, C.c_int, C.c_int]
+    l.orc_cp_initatoms.argtypes = [_f32p, C.c_int, C.c_uint, C.c_uint, C.c_uint, C.c_float]
+    l.orc_cp_atoms_to_const.argtypes = [_f32p, C.c_int, C.c_float, _f32p]
+    l.orc_cp_gptb.argtypes = [C.c_int, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+    l.orc_mnk_from_conv_args.argtypes = [_i32p, _i32p]
+    l.orc_im2col.argtypes = [C.c_int, _f32p] + [C.c_int] * 12 + [_f32p]
+
+
+def num_threads():
+    return int(lib().orc_num_threads())
+
+
+# --------------------------------------------------------------------------- tzgemm
+ALPHA = np.float32(1.1)  # alpha_g, src/header/tzgemm_header.h:64
+
+
+def tzgemm_dims(m, n, k):
+    out = np.zeros(4, np.int32)
+    lib().orc_tzgemm_dims(m, n, k, out)
+    return [int(v) for v in out]
+
+
+def tzgemm_tile_origin(pos, N):
+    r, c = C.c_int(), C.c_int()
+    lib().orc_tzgemm_tile_origin(pos, N, C.byref(r), C.byref(c))
+    return r.value, c.value
+
+
+def tzgemm(A, B, C_init=None, alpha=ALPHA, start=0, end=None, f64=False):
+    """A [M][K] float16, B [N][K] float16 -> C [M][N] float32 (tiles [start,end))."""
+    A = np.ascontiguousarray(A, np.float16)
+    B = np.ascontiguousarray(B, np.float16)
+    M, K = A.shape
+    N = B.shape[0]
+    assert B.shape[1] == K
+    if end is None:
+        end = (M // 64) * (N // 64)
+    out = np.zeros((M, N), np.float32) if C_init is None else np.array(C_init, np.float32, order="C")
+    lib().orc_tzgemm(A.view(np.uint16), B.view(np.uint16), out, M, N, K, float(alpha), start, end,
+                     1 if f64 else 0)
+    return out
+
+
+def gptb_index(block_pos, t, gdx, gdy, bdx, bdy):
+    out = np.zeros(4, np.int32)
+    lib().orc_gptb_index(block_pos, t, gdx, gdy, bdx, bdy, out)
+    return tuple(int(v) for v in out)
+
+
+# --------------------------------------------------------------------------- stencil
+def stencil_grid(nx, ny):
+    """Natural launch grid of ori_stencil (src/ori_kernel/stencil_kernel.cu:166-173)."""
+    return (nx + 63) // 64, (ny + 3) // 4
+
+
+def stencil(c0, c1, A0, Anext):
+    """One sweep; arrays are [nz][ny][nx] float32. Returns the new Anext."""
+    nz, ny, nx = A0.shape
+    out = np.array(Anext, np.float32, order="C")
+    lib().orc_stencil(c0, c1, np.ascontiguousarray(A0, np.float32), out, nx, ny, nz)
+    return out
+
+
+def stencil_gptb(c0, c1, A0, Anext, start, end, gdx=None, gdy=None, bdx=32, bdy=4):
+    nz, ny, nx = A0.shape
+    if gdx is None:
+        gdx, gdy = stencil_grid(nx, ny)
+    out = np.array(Anext, np.float32, order="C")
+    lib().orc_stencil_gptb(c0, c1, np.ascontiguousarray(A0, np.float32), out, nx, ny, nz, gdx, gdy,
+                           bdx, bdy, start, end)
+    return out
+
+
+# --------------------------------------------------------------------------- lbm
+LBM_ENTRIES = 20
+
+
+def lbm(src, dst, sx, sy, sz, start=0, end=None):
+    """src/dst are flat float32 arrays of 20*cells (entry-major SoA). Returns new dst."""
+    if end is None:
+        end = sy * sz
+    src = np.ascontiguousarray(src, np.float32)
+    out = np.array(dst, np.float32, order="C")
+    assert src.size == 20 * sx * sy * sz and out.size == src.size
+    lib().orc_lbm_gptb(src, out, sx, sy, sz, start, end)
+    return out
+
+
+# --------------------------------------------------------------------------- mri-q
+def mriq_phimag(phiR, phiI):
+    out = np.zeros_like(phiR, dtype=np.float32)
+    lib().orc_mriq_phimag(np.ascontiguousarray(phiR, np.float32),
+                          np.ascontiguousarray(phiI, np.float32), out, phiR.size)
+    return out
+
+
+def mriq(kvals, x, y, z, Qr, Qi, start=0, end=None, gdx=None, f64=False):
+    """kvals is [numK][4] float32 {Kx,Ky,Kz,PhiMag}. Returns (Qr, Qi)."""
+    kvals = np.ascontiguousarray(kvals, np.float32)
+    numK = kvals.shape[0]
+    numX = x.size
+    if gdx is None:
+        gdx = numX // 256
+    if end is None:
+        end = gdx
+    qr = np.array(Qr, np.float32, order="C")
+    qi = np.array(Qi, np.float32, order="C")
+    lib().orc_mriq_gptb(numK, kvals.reshape(-1), np.ascontiguousarray(x, np.float32),
+                        np.ascontiguousarray(y, np.float32), np.ascontiguousarray(z, np.float32),
+                        qr, qi, gdx, start, end, 1 if f64 else 0)
+    return qr, qi
+
+
+# --------------------------------------------------------------------------- cp
+def cp_initatoms(count=4000, volx=4096, voly=4096, volz=1, gridspacing=0.1):
+    atoms = np.zeros(count * 4, np.float32)
+    lib().orc_cp_initatoms(atoms, count, volx, voly, volz, gridspacing)
+    return atoms.reshape(count, 4)
+
+
+def cp_atoms_to_const(atoms, zplane=0.0):
+    atoms = np.ascontiguousarray(atoms, np.float32).reshape(-1)
+    out = np.zeros_like(atoms)
+    lib().orc_cp_atoms_to_const(atoms, atoms.size // 4, zplane, out)
+    return out.reshape(-1, 4)
+
+
+def cp(atominfo, energygrid, gridspacing=0.1, start=0, end=None):
+    """energygrid is [voly][volx] float32 (volx multiple of 128, voly multiple of 8)."""
+    voly, volx = energygrid.shape
+    gdx, gdy = volx // 128, voly // 8
+    if end is None:
+        end = gdx * gdy
+    atominfo = np.ascontiguousarray(atominfo, np.float32).reshape(-1)
+    out = np.array(energygrid, np.float32, order="C")
+    lib().orc_cp_gptb(atominfo.size // 4, gridspacing, out.reshape(-1), atominfo, gdx, gdy, start, end)
+    return out
+
+
+# --------------------------------------------------------------------------- conv helpers
+def mnk_from_conv_args(args14):
+    a = np.asarray(args14, np.int32)
+    out = np.zeros(3, np.int32)
+    lib().orc_mnk_from_conv_args(a, out)
+    return [int(v) for v in out]
+
+
+def im2col(data_im, kernel, pad, stride, dilation=(1, 1)):
+    """data_im [C][H][W] -> col [C*kh*kw][Ho][Wo] (Caffe layout)."""
+    data_im = np.ascontiguousarray(data_im, np.float32)
+    Cc, H, W = data_im.shape
+    kh, kw = kernel
+    ph, pw = pad
+    sh, sw = stride
+    dh, dw = dilation
+    Ho = (H + 2 * ph - (dh * (kh - 1) + 1)) // sh + 1
+    Wo = (W + 2 * pw - (dw * (kw - 1) + 1)) // sw + 1
+    col = np.zeros((Cc * kh * kw, Ho, Wo), np.float32)
+    lib().orc_im2col(Cc * Ho * Wo, data_im.reshape(-1), H, W, kh, kw, ph, pw, sh, sw, dh, dw, Ho, Wo,
+                     col.reshape(-1))
+    return col

@@ -1,0 +1,575 @@
+/*
+ * tacker_oracle.c -- CPU restatement of the reference's hot-path kernels.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This file is the parity checker for the HIP path
+ * and the "port" CPU baseline of the benchmark.  Nothing in the product
+ * (tacker_amd/) may include, link, load or call it.
+ *
+ * Every function restates one reference function in plain C with the
+ * reference's own operation order (compile with -ffp-contract=off so that no
+ * multiply-add is fused behind our back).  Citations are relative to the
+ * reference tree (sjtu-epcc/Tacker).
+ *
+ * Pinning status (what fixes each function besides "we typed it"):
+ *   orc_tzgemm_dims       known answers held by the reference: the K keys
+ *                         128/512/1152/2304/4608 of src/config/kinfo-vgg16.json:8-12
+ *                         and (12800,512,4096) of src/Creator.cu:255-261.
+ *   orc_tzgemm_*          closed forms (A=I, all-ones), bijection of the tile
+ *                         map, numpy float64 matmul.
+ *   orc_stencil*          harmonic fields -> 0, constant field, numpy roll
+ *                         formulation in float64, boundary invariance.
+ *   orc_lbm*              obstacle = exact permutation, mass / momentum
+ *                         conservation, rest-equilibrium fixed point,
+ *                         independent numpy formulation.
+ *   orc_mriq*             x=0 closed form, single-k closed form, numpy
+ *                         float64 brute force.
+ *   orc_cp*               single atom closed form, numpy float64 brute force,
+ *                         ori_blks = 16384 held by fusion/code/kinfo.json.
+ *   orc_im2col            direct convolution brute force.
+ *   orc_gptb_index        partition invariance (any launch grid covers every
+ *                         block once).
+ * Unpinned at the bit level (tolerance applies): the reference's WMMA
+ * accumulation order and the CUDA libdevice sin/cos last-ulp behaviour; no
+ * reference file holds golden outputs for them.
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+#define ORC_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------ */
+/* fp16 helpers                                                             */
+/* ------------------------------------------------------------------------ */
+
+static float half_bits_to_float(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1fu;
+    uint32_t man = h & 0x3ffu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: renormalise */
+            int e = -1;
+            do {
+                man <<= 1;
+                e++;
+            } while (!(man & 0x400u));
+            man &= 0x3ffu;
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+ORC_API int orc_num_threads(void)
+{
+#ifdef _OPENMP
+    return omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+/* ------------------------------------------------------------------------ */
+/* tzgemm                                                                   */
+/* ------------------------------------------------------------------------ */
+
+/* src/tzgemm_kernel.h:30-48 getTZGEMMGridDim: floor to multiples of 128 (min
+ * 128); tiles = (M/16 * N/16) / (4*4) 64x64 CTA tiles. */
+ORC_API void orc_tzgemm_dims(int m, int n, int k, int out[4])
+{
+    int M = (m < 128) ? 128 : (m / 128) * 128;
+    int N = (n < 128) ? 128 : (n / 128) * 128;
+    int K = (k < 128) ? 128 : (k / 128) * 128;
+    int m_tiles = M / 16, n_tiles = N / 16;
+    out[0] = M;
+    out[1] = N;
+    out[2] = K;
+    out[3] = (m_tiles * n_tiles) / (4 * 4);
+}
+
+/* src/mix_kernel/tzgemm_stencil.cu:54-56: origin (in elements) of CTA tile
+ * block_pos.  tile_i = ((pos*4)/N_TILES)*4, tile_j = (pos*4)%N_TILES in units
+ * of 16. */
+ORC_API void orc_tzgemm_tile_origin(unsigned pos, int N, int *row0, int *col0)
+{
+    unsigned n_tiles = (unsigned)N / 16u;
+    unsigned ti = ((pos * 4u) / n_tiles) * 4u;
+    unsigned tj = (pos * 4u) % n_tiles;
+    *row0 = (int)(ti * 16u);
+    *col0 = (int)(tj * 16u);
+}
+
+/* src/mix_kernel/tzgemm_stencil.cu:5-172 (fp16 branch, int2 store):
+ * C[i][j] = alpha * sum_k float(A[i][k]) * float(B[j][k]) for the 64x64 tiles
+ * block_pos in [start,end); other elements of C are left untouched.  A is
+ * [M][K], B is [N][K], C is [M][N], all row-major.  accumulate_f64 = 0: fp32
+ * sequential accumulation (tolerance witness); 1: fp64 accumulation (truth).
+ * alpha is applied once after the K reduction (:152), in fp32. */
+ORC_API void orc_tzgemm(const uint16_t *A, const uint16_t *B, float *C, int M, int N, int K,
+                        float alpha, int start, int end, int accumulate_f64)
+{
+    (void)M;
+    float *Af = (float *)malloc(sizeof(float) * (size_t)M * K);
+    float *Bf = (float *)malloc(sizeof(float) * (size_t)N * K);
+    for (size_t i = 0; i < (size_t)M * K; i++) Af[i] = half_bits_to_float(A[i]);
+    for (size_t i = 0; i < (size_t)N * K; i++) Bf[i] = half_bits_to_float(B[i]);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int pos = start; pos < end; pos++) {
+        int r0, c0;
+        orc_tzgemm_tile_origin((unsigned)pos, N, &r0, &c0);
+        for (int i = r0; i < r0 + 64; i++) {
+            const float *a = Af + (size_t)i * K;
+            for (int j = c0; j < c0 + 64; j++) {
+                const float *b = Bf + (size_t)j * K;
+                if (accumulate_f64) {
+                    double acc = 0.0;
+                    for (int k = 0; k < K; k++) acc += (double)a[k] * (double)b[k];
+                    C[(size_t)i * N + j] = (float)((double)alpha * acc);
+                } else {
+                    float acc = 0.0f;
+                    for (int k = 0; k < K; k++) acc = acc + a[k] * b[k];
+                    C[(size_t)i * N + j] = acc * alpha;
+                }
+            }
+        }
+    }
+    free(Af);
+    free(Bf);
+}
+
+/* ------------------------------------------------------------------------ */
+/* GPTB index reconstruction                                                */
+/* ------------------------------------------------------------------------ */
+
+/* src/gptb_kernel/stencil_kernel.cu:6-24, cp_kernel.cu:13-41: a linear
+ * block_pos and a role-local thread index t = threadIdx.x - thread_base are
+ * unfolded into (block_id_x, block_id_y) and (thread_id_x, thread_id_y).
+ * block_id_y wraps modulo grid_dimension_y. out = {bx, by, tx, ty}. */
+ORC_API void orc_gptb_index(unsigned block_pos, int t, int grid_dimension_x, int grid_dimension_y,
+                            int block_dimension_x, int block_dimension_y, int out[4])
+{
+    out[0] = (int)(block_pos % (unsigned)grid_dimension_x);
+    out[1] = (int)((block_pos / (unsigned)grid_dimension_x) % (unsigned)grid_dimension_y);
+    out[2] = t % block_dimension_x;
+    out[3] = (t / block_dimension_x) % block_dimension_y;
+}
+
+/* ------------------------------------------------------------------------ */
+/* stencil                                                                  */
+/* ------------------------------------------------------------------------ */
+
+#define IDX3(nx, ny, i, j, k) ((size_t)(i) + (size_t)(nx) * ((size_t)(j) + (size_t)(ny) * (size_t)(k)))
+
+/* One block of src/ori_kernel/stencil_kernel.cu:9-94 (= general_ptb_stencil
+ * body, src/gptb_kernel/stencil_kernel.cu:26-102): block (bx,by) of
+ * block_dimension (bdx,bdy) covers x in [2*bdx*bx, 2*bdx*bx + 2*bdx),
+ * y in [bdy*by, bdy*by + bdy), marches k = 1..nz-2. */
+static void stencil_block(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz,
+                          int bx, int by, int bdx, int bdy)
+{
+    for (int ty = 0; ty < bdy; ty++) {
+        int j = by * bdy + ty;
+        for (int half = 0; half < 2; half++) {
+            for (int tx = 0; tx < bdx; tx++) {
+                int i = bx * bdx * 2 + tx + half * bdx;
+                /* :26-27 write regions */
+                int w = (half == 0) ? (i > 0 && j > 0 && i < nx - 1 && j < ny - 1)
+                                    : (j > 0 && i < nx - 1 && j < ny - 1);
+                if (!w) continue;
+                for (int k = 1; k < nz - 1; k++) {
+                    float top = A0[IDX3(nx, ny, i, j, k + 1)];
+                    float bottom = A0[IDX3(nx, ny, i, j, k - 1)];
+                    float up = A0[IDX3(nx, ny, i, j + 1, k)];
+                    float down = A0[IDX3(nx, ny, i, j - 1, k)];
+                    float right = A0[IDX3(nx, ny, i + 1, j, k)];
+                    float left = A0[IDX3(nx, ny, i - 1, j, k)];
+                    float centre = A0[IDX3(nx, ny, i, j, k)];
+                    /* :68-69 and :82-83: same association order for both halves */
+                    float s = top + bottom;
+                    s = s + up;
+                    s = s + down;
+                    s = s + right;
+                    s = s + left;
+                    float p = s * c1;
+                    float q = centre * c0;
+                    Anext[IDX3(nx, ny, i, j, k)] = p - q;
+                }
+            }
+        }
+    }
+}
+
+/* GPTB form: blocks block_pos in [start,end) of a (gdx,gdy) grid of (bdx,bdy)
+ * blocks; by wraps modulo gdy (src/gptb_kernel/stencil_kernel.cu:22-24). */
+ORC_API void orc_stencil_gptb(float c0, float c1, const float *A0, float *Anext, int nx, int ny,
+                              int nz, int gdx, int gdy, int bdx, int bdy, int start, int end)
+{
+#pragma omp parallel for schedule(static)
+    for (int pos = start; pos < end; pos++) {
+        int bx = pos % gdx;
+        int by = (pos / gdx) % gdy;
+        stencil_block(c0, c1, A0, Anext, nx, ny, nz, bx, by, bdx, bdy);
+    }
+}
+
+/* Ori form: the natural grid (ceil(nx/64), ceil(ny/4)) of (32,4) blocks,
+ * src/ori_kernel/stencil_kernel.cu:166-173. */
+ORC_API void orc_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz)
+{
+    int gdx = (nx + 32 * 2 - 1) / (32 * 2);
+    int gdy = (ny + 4 - 1) / 4;
+    orc_stencil_gptb(c0, c1, A0, Anext, nx, ny, nz, gdx, gdy, 32, 4, 0, gdx * gdy);
+}
+
+/* ------------------------------------------------------------------------ */
+/* lbm                                                                      */
+/* ------------------------------------------------------------------------ */
+
+/* Entry order, src/header/lbm_header.h:228-233. */
+enum { LC = 0, LN, LS, LE, LW, LT, LB, LNE, LNW, LSE, LSW, LNT, LNB, LST, LSB, LET, LEB, LWT, LWB,
+       LFLAGS, L_ENTRIES };
+
+/* Direction of each entry, src/header/lbm_header.h:102-121. */
+static const int lbm_dx[19] = {0, 0, 0, +1, -1, 0, 0, +1, -1, +1, -1, 0, 0, 0, 0, +1, +1, -1, -1};
+static const int lbm_dy[19] = {0, +1, -1, 0, 0, 0, 0, +1, +1, -1, -1, +1, +1, -1, -1, 0, 0, 0, 0};
+static const int lbm_dz[19] = {0, 0, 0, 0, 0, +1, -1, 0, 0, 0, 0, +1, -1, +1, -1, +1, -1, +1, -1};
+
+/* One cell of src/ori_kernel/lbm_kernel.cu:9-154.  src/dst point at entry
+ * plane 0 of cell (0,0,0) (i.e. base + REAL_MARGIN).  SoA layout
+ * CALC_INDEX(x,y,z,e) = cells*e + x + y*sx + z*sx*sy (lbm_header.h:43-44),
+ * SCATTER mode (:47-51), no boundary clamping: the neighbour is reached by
+ * linear index arithmetic.
+ *
+ * A scatter whose linear target cell index falls outside [0, cells) would land
+ * in the adjacent entry plane, where the reference has a write-write race with
+ * that plane's in-range writer (two threads, two values, one address).  This
+ * restatement resolves the race the same way on every run: the in-range
+ * writer wins, i.e. the out-of-range store is dropped. */
+static void lbm_cell(const float *src, float *dst, long cells, long c, const long off[19])
+{
+    float f[19];
+    for (int e = 0; e < 19; e++) f[e] = src[cells * e + c];
+    uint32_t flags;
+    memcpy(&flags, &src[cells * LFLAGS + c], 4);
+
+    if (flags & 1u) { /* OBSTACLE: :49-57 */
+        float t;
+        t = f[LN]; f[LN] = f[LS]; f[LS] = t;
+        t = f[LE]; f[LE] = f[LW]; f[LW] = t;
+        t = f[LT]; f[LT] = f[LB]; f[LB] = t;
+        t = f[LNE]; f[LNE] = f[LSW]; f[LSW] = t;
+        t = f[LNW]; f[LNW] = f[LSE]; f[LSE] = t;
+        t = f[LNT]; f[LNT] = f[LSB]; f[LSB] = t;
+        t = f[LNB]; f[LNB] = f[LST]; f[LST] = t;
+        t = f[LET]; f[LET] = f[LWB]; f[LWB] = t;
+        t = f[LEB]; f[LEB] = f[LWT]; f[LWT] = t;
+    } else {
+        float ux, uy, uz, rho, u2, temp1, temp2, temp_base;
+        /* :63-72 */
+        rho = f[LC] + f[LN];
+        rho = rho + f[LS]; rho = rho + f[LE]; rho = rho + f[LW]; rho = rho + f[LT];
+        rho = rho + f[LB]; rho = rho + f[LNE]; rho = rho + f[LNW]; rho = rho + f[LSE];
+        rho = rho + f[LSW]; rho = rho + f[LNT]; rho = rho + f[LNB]; rho = rho + f[LST];
+        rho = rho + f[LSB]; rho = rho + f[LET]; rho = rho + f[LEB]; rho = rho + f[LWT];
+        rho = rho + f[LWB];
+        /* :74-88 (unary plus, then left to right) */
+        ux = f[LE] - f[LW];
+        ux = ux + f[LNE]; ux = ux - f[LNW]; ux = ux + f[LSE]; ux = ux - f[LSW];
+        ux = ux + f[LET]; ux = ux + f[LEB]; ux = ux - f[LWT]; ux = ux - f[LWB];
+        uy = f[LN] - f[LS];
+        uy = uy + f[LNE]; uy = uy + f[LNW]; uy = uy - f[LSE]; uy = uy - f[LSW];
+        uy = uy + f[LNT]; uy = uy + f[LNB]; uy = uy - f[LST]; uy = uy - f[LSB];
+        uz = f[LT] - f[LB];
+        uz = uz + f[LNT]; uz = uz - f[LNB]; uz = uz + f[LST]; uz = uz - f[LSB];
+        uz = uz + f[LET]; uz = uz - f[LEB]; uz = uz + f[LWT]; uz = uz - f[LWB];
+        ux = ux / rho; /* :90-92 */
+        uy = uy / rho;
+        uz = uz / rho;
+        if (flags & 2u) { /* ACCEL :93-97 */
+            ux = 0.005f;
+            uy = 0.002f;
+            uz = 0.000f;
+        }
+        {
+            float a = ux * ux, b = uy * uy, cc = uz * uz;
+            float s = a + b;
+            s = s + cc;
+            u2 = 1.5f * s;
+            u2 = u2 - 1.0f; /* :98 */
+        }
+        const float OMEGA = 1.95f;
+        const float DFL1 = 1.0f / 3.0f, DFL2 = 1.0f / 18.0f, DFL3 = 1.0f / 36.0f;
+        temp_base = OMEGA * rho;
+        temp1 = DFL1 * temp_base;
+        temp2 = 1.0f - OMEGA;
+#define LBM_RELAX(entry, expr)                 \
+    do {                                       \
+        float lhs_ = temp2 * f[entry];         \
+        float e_ = (expr);                     \
+        float rhs_ = temp1 * e_;               \
+        f[entry] = lhs_ + rhs_;                \
+    } while (0)
+#define LBM_Q(v, sgn) ((v) * (4.5f * (v) + (sgn)) - u2)
+        LBM_RELAX(LC, -u2); /* :105 */
+        temp1 = DFL2 * temp_base;
+        LBM_RELAX(LN, LBM_Q(uy, 3.0f));
+        LBM_RELAX(LS, uy * (4.5f * uy - 3.0f) - u2);
+        LBM_RELAX(LT, LBM_Q(uz, 3.0f));
+        LBM_RELAX(LB, uz * (4.5f * uz - 3.0f) - u2);
+        LBM_RELAX(LE, LBM_Q(ux, 3.0f));
+        LBM_RELAX(LW, ux * (4.5f * ux - 3.0f) - u2);
+        temp1 = DFL3 * temp_base;
+        {
+            float v;
+            v = (+uy + uz); LBM_RELAX(LNT, LBM_Q(v, 3.0f));
+            v = (+uy - uz); LBM_RELAX(LNB, LBM_Q(v, 3.0f));
+            v = (-uy + uz); LBM_RELAX(LST, LBM_Q(v, 3.0f));
+            v = (-uy - uz); LBM_RELAX(LSB, LBM_Q(v, 3.0f));
+            v = (+ux + uy); LBM_RELAX(LNE, LBM_Q(v, 3.0f));
+            v = (+ux - uy); LBM_RELAX(LSE, LBM_Q(v, 3.0f));
+            v = (+ux + uz); LBM_RELAX(LET, LBM_Q(v, 3.0f));
+            v = (+ux - uz); LBM_RELAX(LEB, LBM_Q(v, 3.0f));
+            v = (-ux + uy); LBM_RELAX(LNW, LBM_Q(v, 3.0f));
+            v = (-ux - uy); LBM_RELAX(LSW, LBM_Q(v, 3.0f));
+            v = (-ux + uz); LBM_RELAX(LWT, LBM_Q(v, 3.0f));
+            v = (-ux - uz); LBM_RELAX(LWB, LBM_Q(v, 3.0f));
+        }
+#undef LBM_RELAX
+#undef LBM_Q
+    }
+    for (int e = 0; e < 19; e++) { /* :133-153 scatter */
+        long t = c + off[e];
+        if (t >= 0 && t < cells) dst[cells * e + t] = f[e];
+    }
+}
+
+/* GPTB form (src/gptb_kernel/lbm_kernel.cu:3-178): block_pos -> (y,z) with
+ * y = pos % sy, z = (pos / sy) % sz; thread_id_x = x in [0,sx).  The grid is
+ * (sy,sz) blocks of sx threads (src/ori_kernel/lbm_kernel.cu:218-222). */
+ORC_API void orc_lbm_gptb(const float *src, float *dst, int sx, int sy, int sz, int start, int end)
+{
+    long cells = (long)sx * sy * sz;
+    long off[19];
+    for (int e = 0; e < 19; e++) off[e] = lbm_dx[e] + (long)lbm_dy[e] * sx + (long)lbm_dz[e] * sx * sy;
+#pragma omp parallel for schedule(static)
+    for (int pos = start; pos < end; pos++) {
+        int y = pos % sy;
+        int z = (pos / sy) % sz;
+        for (int x = 0; x < sx; x++) {
+            long c = x + (long)y * sx + (long)z * sx * sy;
+            lbm_cell(src, dst, cells, c, off);
+        }
+    }
+}
+
+ORC_API void orc_lbm(const float *src, float *dst, int sx, int sy, int sz)
+{
+    orc_lbm_gptb(src, dst, sx, sy, sz, 0, sy * sz);
+}
+
+/* ------------------------------------------------------------------------ */
+/* mri-q                                                                    */
+/* ------------------------------------------------------------------------ */
+
+/* src/ori_kernel/mriq_kernel.cu:47-54 */
+ORC_API void orc_mriq_phimag(const float *phiR, const float *phiI, float *phiMag, int numK)
+{
+    for (int k = 0; k < numK; k++) {
+        float real = phiR[k];
+        float imag = phiI[k];
+        float a = real * real, b = imag * imag;
+        phiMag[k] = a + b;
+    }
+}
+
+/* src/ori_kernel/mriq_kernel.cu:56-105 with the k loop running over all numK
+ * samples (the reference's "QGrid < 1" loop stops after the first 1024-sample
+ * chunk, :58-59; the intended Parboil semantics is every chunk in order, which
+ * for one voxel is simply k = 0..numK-1 in sequence).  kvals is the AoS table
+ * {Kx,Ky,Kz,PhiMag} (src/header/mriq_header.h:12-17).  GPTB form: voxel blocks
+ * of 256 (KERNEL_Q_THREADS_PER_BLOCK) in [start,end), block_id_x wraps modulo
+ * grid_dimension_x (src/gptb_kernel/mriq_kernel.cu:17-33).  Read-modify-write
+ * on Qr/Qi.  f64 = 1: double arithmetic throughout (truth), written back as
+ * float. */
+ORC_API void orc_mriq_gptb(int numK, const float *kvals, const float *x, const float *y,
+                           const float *z, float *Qr, float *Qi, int gdx, int start, int end, int f64)
+{
+    const float PIx2 = 6.2831853071795864769252867665590058f;
+#pragma omp parallel for schedule(static)
+    for (int pos = start; pos < end; pos++) {
+        int bx = pos % gdx;
+        for (int t = 0; t < 256; t++) {
+            int xi = bx * 256 + t;
+            if (f64) {
+                double sx = x[xi], sy = y[xi], sz = z[xi];
+                double qr = Qr[xi], qi = Qi[xi];
+                for (int k = 0; k < numK; k++) {
+                    const float *kv = kvals + 4 * (size_t)k;
+                    double arg = 6.2831853071795864769252867665590058 *
+                                 ((double)kv[0] * sx + (double)kv[1] * sy + (double)kv[2] * sz);
+                    qr += (double)kv[3] * cos(arg);
+                    qi += (double)kv[3] * sin(arg);
+                }
+                Qr[xi] = (float)qr;
+                Qi[xi] = (float)qi;
+            } else {
+                float sx = x[xi], sy = y[xi], sz = z[xi];
+                float qr = Qr[xi], qi = Qi[xi];
+                for (int k = 0; k < numK; k++) {
+                    const float *kv = kvals + 4 * (size_t)k;
+                    float a = kv[0] * sx, b = kv[1] * sy, c = kv[2] * sz;
+                    float d = a + b;
+                    d = d + c;
+                    float arg = PIx2 * d;
+                    float pc = kv[3] * cosf(arg);
+                    float ps = kv[3] * sinf(arg);
+                    qr = qr + pc;
+                    qi = qi + ps;
+                }
+                Qr[xi] = qr;
+                Qi[xi] = qi;
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* cp                                                                       */
+/* ------------------------------------------------------------------------ */
+
+/* src/ori_kernel/cp_kernel.cu:185-209 initatoms: glibc srand(54321), four
+ * rand() per atom in the order x,y,z,q.  The box is dim3 (unsigned) so
+ * gridspacing*volsize truncates: 0.1f*4096 -> 409, 0.1f*1 -> 0. */
+ORC_API void orc_cp_initatoms(float *atoms, int count, unsigned volx, unsigned voly, unsigned volz,
+                              float gridspacing)
+{
+    unsigned sizex = (unsigned)(gridspacing * volx);
+    unsigned sizey = (unsigned)(gridspacing * voly);
+    unsigned sizez = (unsigned)(gridspacing * volz);
+    srand(54321);
+    for (int i = 0; i < count; i++) {
+        int addr = i * 4;
+        atoms[addr] = (rand() / (float)RAND_MAX) * sizex;
+        atoms[addr + 1] = (rand() / (float)RAND_MAX) * sizey;
+        atoms[addr + 2] = (rand() / (float)RAND_MAX) * sizez;
+        atoms[addr + 3] = (float)(((rand() / (float)RAND_MAX) * 2.0) - 1.0);
+    }
+}
+
+/* src/ori_kernel/cp_kernel.cu:159-179 copyatomstoconstbuf: z is replaced by
+ * (zplane - z)^2. */
+ORC_API void orc_cp_atoms_to_const(const float *atoms, int count, float zplane, float *atominfo)
+{
+    for (int i = 0; i < count * 4; i += 4) {
+        atominfo[i] = atoms[i];
+        atominfo[i + 1] = atoms[i + 1];
+        float dz = zplane - atoms[i + 2];
+        atominfo[i + 2] = dz * dz;
+        atominfo[i + 3] = atoms[i + 3];
+    }
+}
+
+/* src/gptb_kernel/cp_kernel.cu:8-96 (= ori_cp, src/ori_kernel/cp_kernel.cu:26-79,
+ * with blockIdx reconstructed): grid (gdx,gdy) of (16,8) blocks, each thread 8
+ * x-points 16 apart.  energygrid has row pitch gdx*16*8.  Blocks [start,end). */
+ORC_API void orc_cp_gptb(int numatoms, float gridspacing, float *energygrid, const float *atominfo,
+                         int gdx, int gdy, int start, int end)
+{
+    const int BX = 16, BY = 8, UNROLLX = 8;
+#pragma omp parallel for schedule(static)
+    for (int pos = start; pos < end; pos++) {
+        unsigned bx = (unsigned)pos % (unsigned)gdx;
+        unsigned by = ((unsigned)pos / (unsigned)gdx) % (unsigned)gdy;
+        for (unsigned ty = 0; ty < (unsigned)BY; ty++) {
+            for (unsigned tx = 0; tx < (unsigned)BX; tx++) {
+                unsigned xindex = bx * BX * UNROLLX + tx;
+                unsigned yindex = by * BY + ty;
+                unsigned outaddr = ((unsigned)gdx * BX * UNROLLX) * yindex + xindex;
+                float coory = gridspacing * yindex;
+                float coorx = gridspacing * xindex;
+                float e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                float gridspacing_u = gridspacing * BX;
+                for (int a = 0; a < numatoms; a++) {
+                    const float *at = atominfo + 4 * a;
+                    float dy = coory - at[1];
+                    float dy2 = dy * dy;
+                    float dyz2 = dy2 + at[2];
+                    float dx = coorx - at[0];
+                    for (int n = 0; n < 8; n++) {
+                        float dx2 = dx * dx;
+                        float r2 = dx2 + dyz2;
+                        float inv = 1.0f / sqrtf(r2);
+                        float contrib = at[3] * inv;
+                        e[n] = e[n] + contrib;
+                        dx = dx + gridspacing_u;
+                    }
+                }
+                for (int n = 0; n < 8; n++) {
+                    float *p = &energygrid[outaddr + (unsigned)n * BX];
+                    *p = *p + e[n];
+                }
+            }
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* conv -> GEMM helpers                                                     */
+/* ------------------------------------------------------------------------ */
+
+/* src/TaskManager.cu:92-123 get_mnk_from_cudnn_args: 14 ints
+ * {n,c,h,w, k,c,kh,kw, pad_h,pad_w, stride_h,stride_w, dil_h,dil_w}. */
+ORC_API void orc_mnk_from_conv_args(const int a[14], int mnk[3])
+{
+    int height_col = (a[2] + 2 * a[8] - (a[12] * (a[6] - 1) + 1)) / a[10] + 1;
+    int width_col = (a[3] + 2 * a[9] - (a[13] * (a[7] - 1) + 1)) / a[11] + 1;
+    mnk[0] = a[0] * height_col * width_col;
+    mnk[1] = a[4];
+    mnk[2] = a[6] * a[7] * a[1];
+}
+
+/* src/TaskManager.cu:48-82 im2col_gpu_kernel_ (Caffe im2col, NCHW): n =
+ * channels*height_col*width_col work items (the batch dimension is folded into
+ * channels by the caller). */
+ORC_API void orc_im2col(int n, const float *data_im, int height, int width, int kernel_h,
+                        int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
+                        int dilation_h, int dilation_w, int height_col, int width_col,
+                        float *data_col)
+{
+    for (int i = 0; i < n; i++) {
+        int h_index = i / width_col;
+        int h_col = h_index % height_col;
+        int w_col = i % width_col;
+        int c_im = h_index / height_col;
+        int c_col = c_im * kernel_h * kernel_w;
+        int h_offset = h_col * stride_h - pad_h;
+        int w_offset = w_col * stride_w - pad_w;
+        float *col = data_col + ((size_t)c_col * height_col + h_col) * width_col + w_col;
+        const float *im = data_im + ((long)c_im * height + h_offset) * width + w_offset;
+        for (int ki = 0; ki < kernel_h; ki++) {
+            for (int kj = 0; kj < kernel_w; kj++) {
+                int h_im = h_offset + ki * dilation_h;
+                int w_im = w_offset + kj * dilation_w;
+                *col = (h_im >= 0 && w_im >= 0 && h_im < height && w_im < width)
+                           ? im[ki * dilation_h * width + kj * dilation_w]
+                           : 0.0f;
+                col += (size_t)height_col * width_col;
+            }
+        }
+    }
+}
