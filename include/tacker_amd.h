@@ -1,0 +1,280 @@
+/*
+ * tacker_amd.h -- C-ABI of libtacker_amd.so (MI355X / gfx950).
+ *
+ * Two layers, both plain C (pointers, sizes, ints; no C++ or torch types):
+ *
+ *  1. tk*        : the thin device layer the host runtime (Kernel / GPTBKernel /
+ *                  MixKernel / Creator / TaskManager) is written against.  It
+ *                  replaces the CUDA runtime + driver calls the reference makes
+ *                  directly (cudaMalloc, cudaLaunchKernel, cuModuleLoad, ...).
+ *                  Two implementations exist: the HIP one (tk_hip.cpp, in
+ *                  libtacker_amd.so) and a recording fake (tk_fake.cpp, in
+ *                  libtacker_host_fake.so) used by CPU-only tests.
+ *  2. tacker_*   : the entry points of the hot path.  Each one drives the same
+ *                  C++ objects a reference caller would build by hand and
+ *                  launches the same device function; the comment on each names
+ *                  the reference interface it stands in for.
+ *
+ * Every function returns 0 on success and a non-zero code on failure unless
+ * stated otherwise; tkGetErrorString / tacker_last_error give the text.
+ * All device pointers are ordinary HIP device pointers (hipMalloc, torch, ...).
+ * Streams are hipStream_t passed as void* (NULL = the default stream).
+ * The library is single-host-thread like the reference (GPTBKernel::executeImpl
+ * pushes/pops its own parameter vector, src/GPTBKernel.h:99-119).
+ */
+#ifndef TACKER_AMD_H
+#define TACKER_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TK_API __attribute__((visibility("default")))
+
+/* ------------------------------------------------------------------------- */
+/* 1. thin device layer                                                       */
+/* ------------------------------------------------------------------------- */
+
+typedef void *tkStream_t;
+typedef void *tkEvent_t;
+typedef void *tkModule_t;
+typedef void *tkFunction_t;
+typedef struct tkDim3 {
+    unsigned x, y, z;
+} tkDim3;
+
+enum { TK_MEMCPY_H2D = 1, TK_MEMCPY_D2H = 2, TK_MEMCPY_D2D = 3 };
+enum {
+    TK_SUCCESS = 0,
+    TK_ERROR_INVALID_VALUE = 1,
+    TK_ERROR_NOT_FOUND = 2,      /* unknown kernel / symbol / function key */
+    TK_ERROR_UNSUPPORTED = 3,    /* shape the gfx950 kernels do not cover */
+    TK_ERROR_DEVICE = 4          /* a HIP call failed; see tkGetErrorString */
+};
+
+/* replaces initCUDA (src/main.cu:166-184): select the device, create a context */
+TK_API int tkInit(int device);
+TK_API const char *tkGetErrorString(int code);
+/* number of compute units (replaces the SM_NUM macro, src/header/pets_common.h:4-6) */
+TK_API int tkGetCuCount(int *cu_count);
+TK_API int tkGetDeviceName(char *buf, size_t len);
+
+TK_API int tkMalloc(void **ptr, size_t bytes);                           /* cudaMalloc */
+TK_API int tkFree(void *ptr);                                            /* cudaFree */
+TK_API int tkMemcpy(void *dst, const void *src, size_t bytes, int kind); /* cudaMemcpy */
+TK_API int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int kind, tkStream_t s);
+TK_API int tkMemset(void *ptr, int value, size_t bytes);                 /* cudaMemset */
+/* cudaMemcpyToSymbol for the two constant tables of the path: "ck" (mri-q k
+ * table, src/ori_kernel/mriq_kernel.cu:9) and "atominfo" (cp atoms,
+ * src/ori_kernel/cp_kernel.cu:23). */
+TK_API int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset);
+/* cudaMemcpyFromSymbol; also serves "tk_spin_fail", the word a role-local
+ * barrier raises when it gives up waiting. */
+TK_API int tkMemcpyFromSymbol(void *dst, const char *symbol, size_t bytes, size_t offset);
+
+TK_API int tkStreamCreate(tkStream_t *s);
+TK_API int tkStreamDestroy(tkStream_t s);
+TK_API int tkStreamSynchronize(tkStream_t s);
+TK_API int tkDeviceSynchronize(void);
+TK_API int tkEventCreate(tkEvent_t *e);
+TK_API int tkEventDestroy(tkEvent_t e);
+TK_API int tkEventRecord(tkEvent_t e, tkStream_t s);
+TK_API int tkEventSynchronize(tkEvent_t e);
+TK_API int tkEventElapsedTime(float *ms, tkEvent_t start, tkEvent_t stop);
+
+/* cudaLaunchKernel (src/GPTBKernel.h:109, src/MixKernel.h:100): func is a value
+ * of the function registry, args is an array of pointers to each argument. */
+TK_API int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, size_t shmem,
+                          tkStream_t stream);
+
+/* cuModuleLoad / cuModuleGetFunction / cuLaunchKernel (src/ModuleCenter.cu): code
+ * objects (.hsaco / .co) instead of cubins. */
+TK_API int tkModuleLoad(tkModule_t *m, const char *path);
+TK_API int tkModuleUnload(tkModule_t m);
+TK_API int tkModuleGetFunction(tkFunction_t *f, tkModule_t m, const char *name);
+TK_API int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void **args,
+                                size_t shmem, tkStream_t stream);
+
+/* Fills the string-keyed device-function registry (the global `fmap` of
+ * src/main.cu:108-159) without the host translation unit including device
+ * sources: insert(key, function, ctx) is called once per kernel. Keys on the
+ * hot path: ori_{stencil,lbm,mriq,cp}, gptb_{tzgemm,stencil,lbm,mriq,cp},
+ * tzgemm_{stencil,lbm,mriq,cp}, plus variant keys "<key>@<variant>". */
+typedef void (*tk_kernel_insert_fn)(const char *key, const void *func, void *ctx);
+TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx);
+
+/* ------------------------------------------------------------------------- */
+/* 2. hot-path entry points                                                   */
+/* ------------------------------------------------------------------------- */
+
+/* One-time set-up: tkInit(device), registry, kinfo JSON ("" or NULL = the
+ * built-in gfx950 table). Replaces main()'s read_json + initCUDA + fmap
+ * initialiser (src/main.cu:108-159,266-281). Idempotent. */
+TK_API int tacker_init(int device, const char *kinfo_json_path);
+TK_API const char *tacker_last_error(void);
+
+/* getTZGEMMGridDim (src/tzgemm_kernel.h:30-48): out = {M_GLOBAL, N_GLOBAL,
+ * K_GLOBAL, tiles}, dimensions floored to multiples of 128 (min 128), tiles in
+ * units of the reference's 64x64 CTA tile. */
+TK_API int tacker_tzgemm_grid_dim(int m, int n, int k, int out[4]);
+
+/* general_ptb_tzgemm through GPTBKernel (src/gptb_kernel/tzgemm_kernel.cu:430-449,
+ * src/GPTBKernel.h:99-119, src/TaskManager.cu:238-248): C[M][N] f32 =
+ * 1.1 * A[M][K] f16 * (B[N][K] f16)^T for the 64x64 tiles [tile_start, tile_end).
+ * M, N, K must already be multiples of 128. launch_grid = number of persistent
+ * workgroups (0 = one per tile group, capped at 2 per CU). */
+TK_API int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int K,
+                              int tile_start, int tile_end, int launch_grid, tkStream_t stream);
+
+/* ori_stencil through OriSTENCILKernel::executeImpl
+ * (src/ori_kernel/stencil_kernel.cu:9-94,189-201): one Jacobi sweep A0 -> Anext. */
+TK_API int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny,
+                              int nz, tkStream_t stream);
+/* general_ptb_stencil through GPTBKernel (src/gptb_kernel/stencil_kernel.cu:3-104,
+ * src/Creator.cu:179-192): blocks [block_start, block_end) of the ori grid
+ * (ceil(nx/64), ceil(ny/4)). launch_grid workgroups of launch_block threads
+ * (0 = the Creator default for this GPU). */
+TK_API int tacker_gptb_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny,
+                               int nz, int block_start, int block_end, int launch_grid,
+                               int launch_block, tkStream_t stream);
+
+/* ori_lbm / general_ptb_lbm (src/ori_kernel/lbm_kernel.cu:9-154,
+ * src/gptb_kernel/lbm_kernel.cu:3-178): one D3Q19 collide+scatter step. src and
+ * dst point at entry plane 0 of cell (0,0,0) of a 20*sx*sy*sz float SoA grid.
+ * Blocks are rows (y,z): block = y + sy*z. */
+TK_API int tacker_ori_lbm(const float *src, float *dst, int sx, int sy, int sz, tkStream_t stream);
+TK_API int tacker_gptb_lbm(const float *src, float *dst, int sx, int sy, int sz, int block_start,
+                           int block_end, int launch_grid, int launch_block, tkStream_t stream);
+
+/* ori_ComputePhiMag (src/ori_kernel/mriq_kernel.cu:47-54) */
+TK_API int tacker_mriq_phimag(const float *phiR, const float *phiI, float *phiMag, int numK,
+                              tkStream_t stream);
+/* cudaMemcpyToSymbol(ck, ...) (src/ori_kernel/mriq_kernel.cu:254-256): host table
+ * of numK {Kx,Ky,Kz,PhiMag} records, numK <= TACKER_MRIQ_MAX_K. */
+#define TACKER_MRIQ_MAX_K 4096
+TK_API int tacker_mriq_set_kvalues(const float *kvals_host, int numK);
+/* ori_mriq / g_general_ptb_mriq (src/ori_kernel/mriq_kernel.cu:56-105,
+ * src/gptb_kernel/mriq_kernel.cu:3-70): Q += sum over all numK samples for voxel
+ * blocks (256 voxels each) [block_start, block_end). numX multiple of 256. */
+TK_API int tacker_ori_mriq(int numK, const float *x, const float *y, const float *z, float *Qr,
+                           float *Qi, int numX, tkStream_t stream);
+TK_API int tacker_gptb_mriq(int numK, const float *x, const float *y, const float *z, float *Qr,
+                            float *Qi, int numX, int block_start, int block_end, int launch_grid,
+                            int launch_block, tkStream_t stream);
+
+/* copyatomstoconstbuf (src/ori_kernel/cp_kernel.cu:159-179): host array of
+ * count (<= 64) {x,y,z,q}; z is replaced by (zplane - z)^2 on the way. */
+TK_API int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane);
+/* initatoms (src/ori_kernel/cp_kernel.cu:185-209): glibc srand(54321) stream. */
+TK_API int tacker_cp_initatoms(float *atoms_host, int count, unsigned volx, unsigned voly,
+                               unsigned volz, float gridspacing);
+/* ori_cp / g_general_ptb_cp (src/ori_kernel/cp_kernel.cu:26-79,
+ * src/gptb_kernel/cp_kernel.cu:8-96): energygrid[voly][volx] += potential of the
+ * atoms set by tacker_cp_set_atoms; volx multiple of 128, voly multiple of 8;
+ * blocks [block_start, block_end) of the (volx/128, voly/8) grid. */
+TK_API int tacker_ori_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly,
+                         tkStream_t stream);
+TK_API int tacker_gptb_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly,
+                          int block_start, int block_end, int launch_grid, int launch_block,
+                          tkStream_t stream);
+
+/* The fused launches: <be>_tzgemm_mix through MixKernel
+ * (src/mix_kernel/tzgemm_{stencil,lbm,mriq,cp}.cu, src/MixKernel.h:55-104,
+ * src/TaskManager.cu:253-264).  One launch carries the vector kernel's blocks
+ * [be_start, be_end) and the GEMM tiles [tile_start, tile_end).  variant selects
+ * the fused code path ("" or NULL = the kinfo default; "wg" = workgroup-split;
+ * "wave" = wave-split inside each workgroup). launch_grid / launch_block 0 =
+ * kinfo's gridsize * CUs / blocksize. */
+TK_API int tacker_mix_tzgemm_stencil(float c0, float c1, const float *A0, float *Anext, int nx,
+                                     int ny, int nz, int be_start, int be_end, const void *A,
+                                     const void *B, float *C, int M, int N, int K, int tile_start,
+                                     int tile_end, const char *variant, int launch_grid,
+                                     int launch_block, tkStream_t stream);
+TK_API int tacker_mix_tzgemm_lbm(const float *src, float *dst, int sx, int sy, int sz, int be_start,
+                                 int be_end, const void *A, const void *B, float *C, int M, int N,
+                                 int K, int tile_start, int tile_end, const char *variant,
+                                 int launch_grid, int launch_block, tkStream_t stream);
+TK_API int tacker_mix_tzgemm_mriq(int numK, const float *x, const float *y, const float *z,
+                                  float *Qr, float *Qi, int numX, int be_start, int be_end,
+                                  const void *A, const void *B, float *C, int M, int N, int K,
+                                  int tile_start, int tile_end, const char *variant,
+                                  int launch_grid, int launch_block, tkStream_t stream);
+TK_API int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx,
+                                int voly, int be_start, int be_end, const void *A, const void *B,
+                                float *C, int M, int N, int K, int tile_start, int tile_end,
+                                const char *variant, int launch_grid, int launch_block,
+                                tkStream_t stream);
+
+/* im2col_gpu_kernel_ and convertFp32ToFp16_ (src/TaskManager.cu:48-90) */
+TK_API int tacker_im2col(const float *data_im, int channels, int height, int width, int kernel_h,
+                         int kernel_w, int pad_h, int pad_w, int stride_h, int stride_w,
+                         int dilation_h, int dilation_w, float *data_col, tkStream_t stream);
+TK_API int tacker_convert_fp32_to_fp16(void *out_f16, const float *in, int n, tkStream_t stream);
+/* get_mnk_from_cudnn_args (src/TaskManager.cu:92-123) */
+TK_API int tacker_mnk_from_conv_args(const int args[14], int mnk[3]);
+
+/* kinfo lookups (src/json.cc:9-42): get_kernel_info / fget_kernel_info; a missing
+ * key gives JSON_NOT_FOUND = -32767. */
+TK_API int tacker_get_kernel_info(const char *kernel, const char *key);
+TK_API float tacker_fget_kernel_info(const char *kernel, const char *key);
+
+/* ---- object API: the class layer itself, one handle per C++ object ---------- */
+typedef void *tacker_kernel_t;
+
+/* createKernel (src/Creator.cu:21-337) for the names cp, lbm, mriq, stencil,
+ * tzgemm: the memoised GPTBKernel that owns seeded device buffers exactly as the
+ * reference's Ori*Kernel::initParams builds them. Never destroy these. */
+TK_API tacker_kernel_t tacker_create_kernel(const char *name);
+
+/* Ori*Kernel objects over caller-owned device buffers (the reference's
+ * Ori*Kernel(id) constructors allocate their own; see tacker_create_kernel). */
+TK_API tacker_kernel_t tacker_ori_stencil_create(float c0, float c1, const float *A0, float *Anext,
+                                                 int nx, int ny, int nz);
+TK_API tacker_kernel_t tacker_ori_lbm_create(const float *src, float *dst, int sx, int sy, int sz);
+TK_API tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y,
+                                              const float *z, float *Qr, float *Qi, int numX);
+TK_API tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid,
+                                            int volx, int voly);
+/* OriTZGEMMKernel(id, m, n, k) (src/tzgemm_kernel.h:56-147); m, n, k are rounded
+ * by getTZGEMMGridDim's rule. A == NULL selects the global ori_wmma_* buffers. */
+TK_API tacker_kernel_t tacker_ori_tzgemm_create(const void *A, const void *B, float *C, int m, int n,
+                                                int k);
+/* new GPTBKernel(id, name, "gptb_<name>", ori, dim3(launch_grid), dim3(launch_block),
+ * start, end) (src/GPTBKernel.h:14-70). launch_grid / launch_block 0 = the
+ * Creator geometry for this GPU. */
+TK_API tacker_kernel_t tacker_gptb_create(tacker_kernel_t ori, int launch_grid, int launch_block,
+                                          int ptb_start_block_pos, int ptb_end_block_pos);
+TK_API int tacker_gptb_set_range(tacker_kernel_t gptb, int ptb_start_block_pos, int ptb_end_block_pos);
+/* new MixKernel(id, "tzgemm_<be>", be, tz, grid, block, be_start, be_end,
+ * tile_start, tile_end) with grid and block from kinfo (src/TaskManager.cu:253-264). */
+TK_API tacker_kernel_t tacker_mix_create(tacker_kernel_t be_gptb, tacker_kernel_t tz_gptb,
+                                         int be_start, int be_end, int tile_start, int tile_end,
+                                         const char *variant, int launch_grid, int launch_block);
+TK_API int tacker_mix_set_range(tacker_kernel_t mix, int be_start, int be_end, int tile_start,
+                                int tile_end);
+/* Kernel::execute(stream) */
+TK_API int tacker_kernel_execute(tacker_kernel_t kernel, tkStream_t stream);
+/* exchange the input and output grid of a stencil / lbm ori object (the
+ * ping-pong between iterations); fused and GPTB objects built on it follow,
+ * because their parameter vectors alias the ori object's fields */
+TK_API int tacker_kernel_swap_buffers(tacker_kernel_t ori);
+/* out = {launch grid x, launch block x, ptb_start, ptb_end, number of kernel
+ * parameters, smem, ori grid x, ori grid y} (start/end are 0 for non-GPTB objects) */
+TK_API int tacker_kernel_info(tacker_kernel_t kernel, int out[8]);
+TK_API int tacker_kernel_destroy(tacker_kernel_t kernel);
+/* value of the device flag a role-local barrier raises when it gives up waiting
+ * (wave-split fused kernels); reading clears it. 0 = no barrier ever timed out */
+TK_API int tacker_spin_fail_flag(int *flag);
+/* host half conversion used for the synthetic GEMM operands (round to nearest even) */
+TK_API uint16_t tacker_float_to_half_bits(float f);
+/* the seeded generator behind every synthetic input: fills out[n] with uniform
+ * [lo,hi) floats of the stream started by seed */
+TK_API int tacker_rng_uniform(uint64_t seed, float lo, float hi, float *out, size_t n);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TACKER_AMD_H */

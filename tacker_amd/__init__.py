@@ -1,0 +1,412 @@
+"""Python face of libtacker_amd.so (ctypes over the C-ABI of include/tacker_amd.h).
+
+PyTorch is used by callers only as the owner of device memory and streams; every
+compute call here goes through the C entry points, which launch the hand-written
+gfx950 kernels.  There is no fallback: if the library is missing or a call fails,
+an exception is raised.
+
+    import tacker_amd as ta
+    ta.init()                                  # tacker_init(0, builtin kinfo)
+    ta.gptb_tzgemm(A, B, C)                    # torch tensors on cuda:0
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libtacker_amd.so")
+FAKE_LIB_PATH = os.path.join(_HERE, "lib", "libtacker_host_fake.so")
+KINFO_PATH = os.path.join(_HERE, "config", "kinfo-gfx950.json")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "tacker_amd.h")
+
+JSON_NOT_FOUND = -32767
+ALPHA = 1.1
+
+
+class TackerError(RuntimeError):
+    pass
+
+
+def _declare(lib):
+    vp, i, f, cp = C.c_void_p, C.c_int, C.c_float, C.c_char_p
+    lib.tacker_init.argtypes = [i, cp]
+    lib.tacker_last_error.restype = cp
+    lib.tkGetErrorString.restype = cp
+    lib.tkGetErrorString.argtypes = [i]
+    lib.tkGetCuCount.argtypes = [C.POINTER(i)]
+    lib.tkGetDeviceName.argtypes = [C.c_char_p, C.c_size_t]
+    lib.tacker_tzgemm_grid_dim.argtypes = [i, i, i, C.POINTER(i)]
+    lib.tacker_gptb_tzgemm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp]
+    lib.tacker_ori_stencil.argtypes = [f, f, vp, vp, i, i, i, vp]
+    lib.tacker_gptb_stencil.argtypes = [f, f, vp, vp, i, i, i, i, i, i, i, vp]
+    lib.tacker_ori_lbm.argtypes = [vp, vp, i, i, i, vp]
+    lib.tacker_gptb_lbm.argtypes = [vp, vp, i, i, i, i, i, i, i, vp]
+    lib.tacker_mriq_phimag.argtypes = [vp, vp, vp, i, vp]
+    lib.tacker_mriq_set_kvalues.argtypes = [vp, i]
+    lib.tacker_ori_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, vp]
+    lib.tacker_gptb_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    lib.tacker_cp_set_atoms.argtypes = [vp, i, f]
+    lib.tacker_cp_initatoms.argtypes = [vp, i, C.c_uint, C.c_uint, C.c_uint, f]
+    lib.tacker_ori_cp.argtypes = [i, f, vp, i, i, vp]
+    lib.tacker_gptb_cp.argtypes = [i, f, vp, i, i, i, i, i, i, vp]
+    gemm = [vp, vp, vp, i, i, i, i, i, cp, i, i, vp]
+    lib.tacker_mix_tzgemm_stencil.argtypes = [f, f, vp, vp, i, i, i, i, i] + gemm
+    lib.tacker_mix_tzgemm_lbm.argtypes = [vp, vp, i, i, i, i, i] + gemm
+    lib.tacker_mix_tzgemm_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, i, i] + gemm
+    lib.tacker_mix_tzgemm_cp.argtypes = [i, f, vp, i, i, i, i] + gemm
+    lib.tacker_im2col.argtypes = [vp] + [i] * 11 + [vp, vp]
+    lib.tacker_convert_fp32_to_fp16.argtypes = [vp, vp, i, vp]
+    lib.tacker_mnk_from_conv_args.argtypes = [C.POINTER(i), C.POINTER(i)]
+    lib.tacker_get_kernel_info.argtypes = [cp, cp]
+    lib.tacker_fget_kernel_info.argtypes = [cp, cp]
+    lib.tacker_fget_kernel_info.restype = f
+    for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
+                 "tacker_ori_mriq_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
+                 "tacker_gptb_create", "tacker_mix_create"):
+        getattr(lib, name).restype = vp
+    lib.tacker_create_kernel.argtypes = [cp]
+    lib.tacker_ori_stencil_create.argtypes = [f, f, vp, vp, i, i, i]
+    lib.tacker_ori_lbm_create.argtypes = [vp, vp, i, i, i]
+    lib.tacker_ori_mriq_create.argtypes = [i, vp, vp, vp, vp, vp, i]
+    lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
+    lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
+    lib.tacker_gptb_create.argtypes = [vp, i, i, i, i]
+    lib.tacker_gptb_set_range.argtypes = [vp, i, i]
+    lib.tacker_mix_create.argtypes = [vp, vp, i, i, i, i, cp, i, i]
+    lib.tacker_mix_set_range.argtypes = [vp, i, i, i, i]
+    lib.tacker_kernel_execute.argtypes = [vp, vp]
+    lib.tacker_kernel_swap_buffers.argtypes = [vp]
+    lib.tacker_kernel_info.argtypes = [vp, C.POINTER(i)]
+    lib.tacker_kernel_destroy.argtypes = [vp]
+    lib.tacker_spin_fail_flag.argtypes = [C.POINTER(i)]
+    lib.tacker_float_to_half_bits.argtypes = [f]
+    lib.tacker_float_to_half_bits.restype = C.c_uint16
+    lib.tacker_rng_uniform.argtypes = [C.c_uint64, f, f, vp, C.c_size_t]
+    return lib
+
+
+def load_library(path=LIB_PATH):
+    """dlopen a build of the host runtime (the HIP one by default)."""
+    if not os.path.exists(path):
+        raise TackerError(f"{path} is missing: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                          "(or make -C tacker_amd/csrc) first; there is no fallback path")
+    return _declare(C.CDLL(path))
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = load_library()
+    return _lib
+
+
+def check(rc, what="tacker call"):
+    if rc != 0:
+        raise TackerError(f"{what} failed ({rc}): {lib().tacker_last_error().decode()}")
+
+
+def init(device=0, kinfo=None):
+    """tacker_init: device, kernel registry, kinfo table (None = built-in)."""
+    check(lib().tacker_init(device, kinfo.encode() if kinfo else None), "tacker_init")
+
+
+def cu_count():
+    n = C.c_int()
+    check(lib().tkGetCuCount(C.byref(n)), "tkGetCuCount")
+    return n.value
+
+
+def device_name():
+    buf = C.create_string_buffer(256)
+    check(lib().tkGetDeviceName(buf, 256), "tkGetDeviceName")
+    return buf.value.decode()
+
+
+def tzgemm_grid_dim(m, n, k):
+    out = (C.c_int * 4)()
+    lib().tacker_tzgemm_grid_dim(m, n, k, out)
+    return list(out)
+
+
+def get_kernel_info(kernel, key):
+    return lib().tacker_get_kernel_info(kernel.encode(), key.encode())
+
+
+def fget_kernel_info(kernel, key):
+    return lib().tacker_fget_kernel_info(kernel.encode(), key.encode())
+
+
+def _ptr(t):
+    """Device pointer of a torch tensor (must be contiguous and on the GPU)."""
+    if t is None:
+        return None
+    if not t.is_cuda or not t.is_contiguous():
+        raise TackerError("tensors must be contiguous CUDA/HIP tensors")
+    return t.data_ptr()
+
+
+def _stream(stream):
+    if stream is None:
+        import torch
+        return torch.cuda.current_stream().cuda_stream
+    return getattr(stream, "cuda_stream", stream)
+
+
+def _v(variant):
+    return variant.encode() if variant else None
+
+
+# ----------------------------------------------------------------------------- one-shot calls
+def gptb_tzgemm(A, B, Cm, tile_start=0, tile_end=None, launch_grid=0, stream=None):
+    M, K = A.shape
+    N = B.shape[0]
+    if tile_end is None:
+        tile_end = (M // 64) * (N // 64)
+    check(lib().tacker_gptb_tzgemm(_ptr(A), _ptr(B), _ptr(Cm), M, N, K, tile_start, tile_end,
+                                   launch_grid, _stream(stream)), "tacker_gptb_tzgemm")
+
+
+def stencil_blocks(nx, ny):
+    return ((nx + 63) // 64) * ((ny + 3) // 4)
+
+
+def ori_stencil(c0, c1, A0, Anext, stream=None):
+    nz, ny, nx = A0.shape
+    check(lib().tacker_ori_stencil(c0, c1, _ptr(A0), _ptr(Anext), nx, ny, nz, _stream(stream)),
+          "tacker_ori_stencil")
+
+
+def gptb_stencil(c0, c1, A0, Anext, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    nz, ny, nx = A0.shape
+    if end is None:
+        end = stencil_blocks(nx, ny)
+    check(lib().tacker_gptb_stencil(c0, c1, _ptr(A0), _ptr(Anext), nx, ny, nz, start, end, launch_grid,
+                                    launch_block, _stream(stream)), "tacker_gptb_stencil")
+
+
+def ori_lbm(src, dst, sx, sy, sz, stream=None):
+    check(lib().tacker_ori_lbm(_ptr(src), _ptr(dst), sx, sy, sz, _stream(stream)), "tacker_ori_lbm")
+
+
+def gptb_lbm(src, dst, sx, sy, sz, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    if end is None:
+        end = sy * sz
+    check(lib().tacker_gptb_lbm(_ptr(src), _ptr(dst), sx, sy, sz, start, end, launch_grid, launch_block,
+                                _stream(stream)), "tacker_gptb_lbm")
+
+
+def mriq_phimag(phiR, phiI, phiMag, stream=None):
+    check(lib().tacker_mriq_phimag(_ptr(phiR), _ptr(phiI), _ptr(phiMag), phiR.numel(), _stream(stream)),
+          "tacker_mriq_phimag")
+
+
+def mriq_set_kvalues(kvals_np):
+    """kvals_np: host numpy float32 [numK][4] = {Kx,Ky,Kz,PhiMag}."""
+    import numpy as np
+    kv = np.ascontiguousarray(kvals_np, np.float32)
+    check(lib().tacker_mriq_set_kvalues(kv.ctypes.data, kv.shape[0]), "tacker_mriq_set_kvalues")
+
+
+def ori_mriq(numK, x, y, z, Qr, Qi, stream=None):
+    check(lib().tacker_ori_mriq(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi), x.numel(),
+                                _stream(stream)), "tacker_ori_mriq")
+
+
+def gptb_mriq(numK, x, y, z, Qr, Qi, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    if end is None:
+        end = x.numel() // 256
+    check(lib().tacker_gptb_mriq(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi), x.numel(), start,
+                                 end, launch_grid, launch_block, _stream(stream)), "tacker_gptb_mriq")
+
+
+def cp_initatoms(count=4000, volx=4096, voly=4096, volz=1, gridspacing=0.1):
+    import numpy as np
+    atoms = np.zeros((count, 4), np.float32)
+    check(lib().tacker_cp_initatoms(atoms.ctypes.data, count, volx, voly, volz, gridspacing),
+          "tacker_cp_initatoms")
+    return atoms
+
+
+def cp_set_atoms(atoms_np, zplane=0.0):
+    import numpy as np
+    a = np.ascontiguousarray(atoms_np, np.float32)
+    check(lib().tacker_cp_set_atoms(a.ctypes.data, a.shape[0], zplane), "tacker_cp_set_atoms")
+
+
+def ori_cp(numatoms, gridspacing, grid, stream=None):
+    voly, volx = grid.shape
+    check(lib().tacker_ori_cp(numatoms, gridspacing, _ptr(grid), volx, voly, _stream(stream)),
+          "tacker_ori_cp")
+
+
+def gptb_cp(numatoms, gridspacing, grid, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    voly, volx = grid.shape
+    if end is None:
+        end = (volx // 128) * (voly // 8)
+    check(lib().tacker_gptb_cp(numatoms, gridspacing, _ptr(grid), volx, voly, start, end, launch_grid,
+                               launch_block, _stream(stream)), "tacker_gptb_cp")
+
+
+def _gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream):
+    M, K = A.shape
+    N = B.shape[0]
+    if tile_end is None:
+        tile_end = (M // 64) * (N // 64)
+    return [_ptr(A), _ptr(B), _ptr(Cm), M, N, K, tile_start, tile_end, _v(variant), launch_grid,
+            launch_block, _stream(stream)]
+
+
+def mix_tzgemm_stencil(c0, c1, A0, Anext, A, B, Cm, be_start=0, be_end=None, tile_start=0,
+                       tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    nz, ny, nx = A0.shape
+    if be_end is None:
+        be_end = stencil_blocks(nx, ny)
+    check(lib().tacker_mix_tzgemm_stencil(
+        c0, c1, _ptr(A0), _ptr(Anext), nx, ny, nz, be_start, be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_stencil")
+
+
+def mix_tzgemm_lbm(src, dst, sx, sy, sz, A, B, Cm, be_start=0, be_end=None, tile_start=0,
+                   tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    if be_end is None:
+        be_end = sy * sz
+    check(lib().tacker_mix_tzgemm_lbm(
+        _ptr(src), _ptr(dst), sx, sy, sz, be_start, be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_lbm")
+
+
+def mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, A, B, Cm, be_start=0, be_end=None, tile_start=0,
+                    tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    if be_end is None:
+        be_end = x.numel() // 256
+    check(lib().tacker_mix_tzgemm_mriq(
+        numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi), x.numel(), be_start, be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_mriq")
+
+
+def mix_tzgemm_cp(numatoms, gridspacing, grid, A, B, Cm, be_start=0, be_end=None, tile_start=0,
+                  tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    voly, volx = grid.shape
+    if be_end is None:
+        be_end = (volx // 128) * (voly // 8)
+    check(lib().tacker_mix_tzgemm_cp(
+        numatoms, gridspacing, _ptr(grid), volx, voly, be_start, be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_cp")
+
+
+def im2col(data_im, kernel, pad, stride, dilation, data_col, stream=None):
+    Cc, H, W = data_im.shape
+    check(lib().tacker_im2col(_ptr(data_im), Cc, H, W, kernel[0], kernel[1], pad[0], pad[1], stride[0],
+                              stride[1], dilation[0], dilation[1], _ptr(data_col), _stream(stream)),
+          "tacker_im2col")
+
+
+def convert_fp32_to_fp16(out, inp, stream=None):
+    check(lib().tacker_convert_fp32_to_fp16(_ptr(out), _ptr(inp), inp.numel(), _stream(stream)),
+          "tacker_convert_fp32_to_fp16")
+
+
+def mnk_from_conv_args(args14):
+    a = (C.c_int * 14)(*args14)
+    out = (C.c_int * 3)()
+    lib().tacker_mnk_from_conv_args(a, out)
+    return list(out)
+
+
+def spin_fail_flag():
+    v = C.c_int()
+    check(lib().tacker_spin_fail_flag(C.byref(v)), "tacker_spin_fail_flag")
+    return v.value
+
+
+# ----------------------------------------------------------------------------- object API
+class KernelHandle:
+    """Owner of one C++ Kernel object (Ori*, GPTBKernel or MixKernel)."""
+
+    def __init__(self, handle, what, owned=True, keep=()):
+        if not handle:
+            raise TackerError(f"{what} failed: {lib().tacker_last_error().decode()}")
+        self.handle = handle
+        self.owned = owned
+        self.keep = keep          # objects (tensors, handles) that must outlive this one
+
+    def execute(self, stream=None):
+        check(lib().tacker_kernel_execute(self.handle, _stream(stream)), "tacker_kernel_execute")
+
+    def swap_buffers(self):
+        check(lib().tacker_kernel_swap_buffers(self.handle), "tacker_kernel_swap_buffers")
+
+    def info(self):
+        out = (C.c_int * 8)()
+        check(lib().tacker_kernel_info(self.handle, out), "tacker_kernel_info")
+        keys = ("grid", "block", "ptb_start", "ptb_end", "nparams", "smem", "ori_grid_x", "ori_grid_y")
+        return dict(zip(keys, out))
+
+    def set_range(self, *r):
+        if len(r) == 2:
+            check(lib().tacker_gptb_set_range(self.handle, *r), "tacker_gptb_set_range")
+        else:
+            check(lib().tacker_mix_set_range(self.handle, *r), "tacker_mix_set_range")
+
+    def close(self):
+        if self.owned and self.handle:
+            lib().tacker_kernel_destroy(self.handle)
+        self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def create_kernel(name):
+    return KernelHandle(lib().tacker_create_kernel(name.encode()), f"createKernel({name})", owned=False)
+
+
+def ori_stencil_create(c0, c1, A0, Anext):
+    nz, ny, nx = A0.shape
+    return KernelHandle(lib().tacker_ori_stencil_create(c0, c1, _ptr(A0), _ptr(Anext), nx, ny, nz),
+                        "OriSTENCILKernel", keep=(A0, Anext))
+
+
+def ori_lbm_create(src, dst, sx, sy, sz):
+    return KernelHandle(lib().tacker_ori_lbm_create(_ptr(src), _ptr(dst), sx, sy, sz), "OriLBMKernel",
+                        keep=(src, dst))
+
+
+def ori_mriq_create(numK, x, y, z, Qr, Qi):
+    return KernelHandle(lib().tacker_ori_mriq_create(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi),
+                                                     x.numel()), "OriMRIQKernel", keep=(x, y, z, Qr, Qi))
+
+
+def ori_cp_create(numatoms, gridspacing, grid):
+    voly, volx = grid.shape
+    return KernelHandle(lib().tacker_ori_cp_create(numatoms, gridspacing, _ptr(grid), volx, voly),
+                        "OriCPKernel", keep=(grid,))
+
+
+def ori_tzgemm_create(A, B, Cm, m=None, n=None, k=None):
+    if A is not None:
+        m, k = A.shape
+        n = B.shape[0]
+    return KernelHandle(lib().tacker_ori_tzgemm_create(_ptr(A), _ptr(B), _ptr(Cm), m, n, k),
+                        "OriTZGEMMKernel", keep=(A, B, Cm))
+
+
+def gptb_create(ori, launch_grid=0, launch_block=0, start=0, end=0):
+    return KernelHandle(lib().tacker_gptb_create(ori.handle, launch_grid, launch_block, start, end),
+                        "GPTBKernel", keep=(ori,))
+
+
+def mix_create(be_gptb, tz_gptb, be_start, be_end, tile_start, tile_end, variant=None, launch_grid=0,
+               launch_block=0):
+    return KernelHandle(lib().tacker_mix_create(be_gptb.handle, tz_gptb.handle, be_start, be_end,
+                                                tile_start, tile_end, _v(variant), launch_grid,
+                                                launch_block), "MixKernel", keep=(be_gptb, tz_gptb))

@@ -1,0 +1,69 @@
+// Kernel.h -- base of every launchable object of the runtime.
+//
+// Public surface of src/Kernel.h of the reference (Kernel, lmode, GPTBParams):
+// same member names, same void*-per-argument parameter vector, same
+// execute()/initParams()/loadKernel()/getArgs() protocol, so TaskManager, Task
+// and Creator code written against the reference compiles against this.
+// Launches go through tkLaunchKernel (HIP: hipLaunchKernel) instead of
+// cudaLaunchKernel.
+#pragma once
+
+#include <string>
+#include <utility>
+#include <vector>
+
+#include "util.h"
+
+enum lmode { DRIVER_LAUNCH = 0, RUNTIME_LAUNCH };
+
+class Kernel {
+public:
+    virtual ~Kernel() = default;
+
+    // execute(stream): the one entry point callers use
+    template <typename... Args>
+    void execute(Args &&...args)
+    {
+        executeImpl(std::forward<Args>(args)...);
+    }
+    virtual void initParams() = 0;
+    virtual void loadKernel() = 0;
+    // integer description of the launch for the scheduler: {m,n,k} for a GEMM
+    // (mixable == 1), the 14 convolution ints (mixable == 2), empty otherwise
+    virtual std::vector<int> getArgs() = 0;
+
+    int getKernelId() { return Id; }
+    std::string &getKernelName() { return kernelName; }
+
+    int Id = 0;
+    std::string kernelName;
+    std::string moduleName;
+    std::string funcKey;
+    CUfunction function = nullptr;        // set when loaded through ModuleCenter
+    unsigned int smem = 0;                // LDS bytes the device function declares
+    std::vector<void *> kernelParams;     // one pointer per kernel argument, in order
+    std::vector<void *> cudaFreeList;     // device buffers this object owns
+    dim3 launchGridDim;
+    dim3 launchBlockDim;
+    lmode launchMode = RUNTIME_LAUNCH;
+    void *kernelFunc = nullptr;           // registry value for tkLaunchKernel
+    unsigned int mixable = 0;             // 0 solo only, 1 GEMM-shaped, 2 convolution-shaped
+    bool initialized = false;
+
+protected:
+    virtual void executeImpl(cudaStream_t stream) = 0;
+};
+
+// The uniform tail of every GPTB kernel's parameter list (thread_base follows
+// and is supplied at launch time).
+struct GPTBParams {
+    int grid_dimension_x;
+    int grid_dimension_y;
+    int grid_dimension_z;
+    int block_dimension_x;
+    int block_dimension_y;
+    int block_dimension_z;
+    int ptb_start_block_pos;
+    int ptb_iter_block_step;
+    int ptb_end_block_pos;
+};

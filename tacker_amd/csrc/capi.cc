@@ -1,0 +1,596 @@
+// capi.cc -- the tacker_* entry points of include/tacker_amd.h.
+// Each one validates its arguments (returning a code instead of letting the
+// class layer's logger.ERROR end the process), then builds and runs the same
+// Kernel / GPTBKernel / MixKernel objects a C++ caller would.
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+
+#include "Creator.h"
+#include "Logger.h"
+#include "json.h"
+#include "rng.h"
+
+extern Logger logger;
+extern std::unordered_map<std::string, void *> fmap;
+int tacker_runtime_init(int device, const char *kinfo_json_path);
+bool tacker_runtime_ready();
+
+namespace {
+thread_local std::string g_error;
+
+int fail(int code, const std::string &msg)
+{
+    g_error = msg;
+    return code;
+}
+
+// run f(), mapping exceptions of the class layer to an error code
+template <class F>
+int guarded(F &&f)
+{
+    try {
+        return f();
+    } catch (const std::exception &e) {
+        return fail(TK_ERROR_DEVICE, e.what());
+    }
+}
+
+#define REQUIRE_INIT()                                                             \
+    do {                                                                           \
+        if (!tacker_runtime_ready()) return fail(TK_ERROR_INVALID_VALUE, "tacker_init has not been called"); \
+    } while (0)
+
+bool has_key(const std::string &key) { return fmap.find(key) != fmap.end(); }
+
+// Creator geometry of the plain GPTB launch of a kernel on this GPU
+int default_block(const std::string &name)
+{
+    const int bs = get_kernel_info(name, "blocksize");
+    return bs == JSON_NOT_FOUND ? 256 : bs;
+}
+int default_grid(const std::string &name)
+{
+    int per_cu = get_kernel_info(name, "solo_ptb_blks");
+    if (per_cu == JSON_NOT_FOUND || per_cu < 1) per_cu = 1;
+    return cuCount() * per_cu;
+}
+
+int check_block(const std::string &name, int block)
+{
+    if (block <= 0 || block % 64 || block > 1024)
+        return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 64 in [64,1024]");
+    if (name == "tzgemm" && block != TZ_THREADS)
+        return fail(TK_ERROR_INVALID_VALUE, "tzgemm: launch_block must be 256");
+    if (name == "mriq" && block % 256)
+        return fail(TK_ERROR_INVALID_VALUE, "mriq: launch_block must be a multiple of 256");
+    if (name == "cp" && block % 128)
+        return fail(TK_ERROR_INVALID_VALUE, "cp: launch_block must be a multiple of 128");
+    return TK_SUCCESS;
+}
+
+GPTBKernel *make_gptb(Kernel *ori, int launch_grid, int launch_block, int start, int end)
+{
+    const std::string &name = ori->kernelName;
+    const int grid = launch_grid > 0 ? launch_grid : default_grid(name);
+    const int block = launch_block > 0 ? launch_block : default_block(name);
+    return new GPTBKernel(ori->Id, name, "gptb_" + name, ori, dim3(grid, 1, 1), dim3(block, 1, 1), start, end);
+}
+
+int natural_blocks(Kernel *ori)
+{
+    return (int)(ori->launchGridDim.x * ori->launchGridDim.y * ori->launchGridDim.z);
+}
+
+int check_range(Kernel *ori, int start, int end)
+{
+    if (start < 0 || end < start) return fail(TK_ERROR_INVALID_VALUE, ori->kernelName + ": bad block range");
+    if (ori->kernelName == "tzgemm" && end > natural_blocks(ori))
+        return fail(TK_ERROR_INVALID_VALUE, "tzgemm: tile range exceeds the tile count");
+    return TK_SUCCESS;
+}
+
+int check_stencil(const float *A0, float *Anext, int nx, int ny, int nz)
+{
+    if (!A0 || !Anext || nx < 1 || ny < 1 || nz < 1) return fail(TK_ERROR_INVALID_VALUE, "stencil: bad arguments");
+    if ((long long)nx * ny * nz >= (1LL << 40)) return fail(TK_ERROR_UNSUPPORTED, "stencil: grid too large");
+    return TK_SUCCESS;
+}
+int check_lbm(const float *src, float *dst, int sx, int sy, int sz)
+{
+    if (!src || !dst || sx < 1 || sy < 1 || sz < 1) return fail(TK_ERROR_INVALID_VALUE, "lbm: bad arguments");
+    if ((long long)sx * sy * sz * 20 >= (1LL << 31)) return fail(TK_ERROR_UNSUPPORTED, "lbm: grid too large for 32-bit cell indices");
+    return TK_SUCCESS;
+}
+int check_mriq(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi, int numX)
+{
+    if (!x || !y || !z || !Qr || !Qi || numK < 0 || numK > MRIQ_MAX_K || numX < 0)
+        return fail(TK_ERROR_INVALID_VALUE, "mriq: bad arguments");
+    if (numX % KERNEL_Q_THREADS_PER_BLOCK) return fail(TK_ERROR_UNSUPPORTED, "mriq: numX must be a multiple of 256");
+    return TK_SUCCESS;
+}
+int check_cp(int numatoms, float *grid, int volx, int voly)
+{
+    if (!grid || numatoms < 0 || numatoms > MAXATOMS) return fail(TK_ERROR_INVALID_VALUE, "cp: bad arguments");
+    if (volx < 128 || voly < 8 || volx % (BLOCKSIZEX * UNROLLX) || voly % BLOCKSIZEY)
+        return fail(TK_ERROR_UNSUPPORTED, "cp: volx must be a multiple of 128 and voly of 8");
+    return TK_SUCCESS;
+}
+int check_gemm(const void *A, const void *B, float *C, int M, int N, int K)
+{
+    if (!A || !B || !C) return fail(TK_ERROR_INVALID_VALUE, "tzgemm: null operand");
+    if (M < 128 || N < 128 || K < 128 || M % 128 || N % 128 || K % 128)
+        return fail(TK_ERROR_UNSUPPORTED, "tzgemm: M, N, K must be multiples of 128");
+    return TK_SUCCESS;
+}
+
+// launch an ori object once and drop it
+int run_once(Kernel *k, tkStream_t stream)
+{
+    std::unique_ptr<Kernel> hold(k);
+    return guarded([&]() -> int {
+        k->execute(stream);
+        return TK_SUCCESS;
+    });
+}
+int run_gptb_once(Kernel *ori, int start, int end, int grid, int block, tkStream_t stream)
+{
+    std::unique_ptr<Kernel> hold_ori(ori);
+    int rc = check_range(ori, start, end);
+    if (rc) return rc;
+    rc = check_block(ori->kernelName, block > 0 ? block : default_block(ori->kernelName));
+    if (rc) return rc;
+    return guarded([&]() -> int {
+        std::unique_ptr<GPTBKernel> g(make_gptb(ori, grid, block, start, end));
+        g->execute(stream);
+        return TK_SUCCESS;
+    });
+}
+int run_mix_once(Kernel *be_ori, int be_start, int be_end, const void *A, const void *B, float *C, int M,
+                 int N, int K, int tile_start, int tile_end, const char *variant, int grid, int block,
+                 tkStream_t stream)
+{
+    std::unique_ptr<Kernel> hold_be(be_ori);
+    int rc = check_gemm(A, B, C, M, N, K);
+    if (rc) return rc;
+    rc = check_range(be_ori, be_start, be_end);
+    if (rc) return rc;
+    const std::string v = variant ? variant : "";
+    const std::string key = "tzgemm_" + be_ori->kernelName + (v.empty() ? "" : "@" + v);
+    if (!has_key(key)) return fail(TK_ERROR_NOT_FOUND, "no fused kernel {" + key + "}");
+    if (get_kernel_info(key, "blocksize") == JSON_NOT_FOUND) return fail(TK_ERROR_NOT_FOUND, "kinfo has no entry for {" + key + "}");
+    if (block > 0 && block != get_kernel_info(key, "blocksize"))
+        return fail(TK_ERROR_INVALID_VALUE, "{" + key + "} is built for " + std::to_string(get_kernel_info(key, "blocksize")) + " threads");
+    return guarded([&]() -> int {
+        std::unique_ptr<OriTZGEMMKernel> tz_ori(new OriTZGEMMKernel(0, M, N, K, A, B, C));
+        int rc2 = check_range(tz_ori.get(), tile_start, tile_end);
+        if (rc2) return rc2;
+        std::unique_ptr<GPTBKernel> be(make_gptb(be_ori, 0, 0, be_start, be_end));
+        std::unique_ptr<GPTBKernel> tz(make_gptb(tz_ori.get(), 0, TZ_THREADS, tile_start, tile_end));
+        std::unique_ptr<MixKernel> mix(createTzgemmMix(be.get(), tz.get(), be_start, be_end, tile_start, tile_end, v, grid, block));
+        mix->execute(stream);
+        return TK_SUCCESS;
+    });
+}
+}  // namespace
+
+extern "C" {
+
+int tacker_init(int device, const char *kinfo_json_path)
+{
+    return guarded([&]() -> int {
+        const int rc = tacker_runtime_init(device, kinfo_json_path);
+        if (rc) g_error = tkGetErrorString(rc);
+        return rc;
+    });
+}
+
+const char *tacker_last_error(void) { return g_error.c_str(); }
+
+int tacker_tzgemm_grid_dim(int m, int n, int k, int out[4])
+{
+    const std::vector<int> d = getTZGEMMGridDim(m, n, k);
+    for (int i = 0; i < 4; ++i) out[i] = d[i];
+    return TK_SUCCESS;
+}
+
+int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                       int tile_end, int launch_grid, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_gemm(A, B, C, M, N, K);
+    if (rc) return rc;
+    return run_gptb_once(new OriTZGEMMKernel(0, M, N, K, A, B, C), tile_start, tile_end, launch_grid,
+                         TZ_THREADS, stream);
+}
+
+int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_stencil(A0, Anext, nx, ny, nz);
+    if (rc) return rc;
+    return run_once(new OriSTENCILKernel(0, c0, c1, A0, Anext, nx, ny, nz), stream);
+}
+
+int tacker_gptb_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz,
+                        int block_start, int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_stencil(A0, Anext, nx, ny, nz);
+    if (rc) return rc;
+    return run_gptb_once(new OriSTENCILKernel(0, c0, c1, A0, Anext, nx, ny, nz), block_start, block_end,
+                         launch_grid, launch_block, stream);
+}
+
+int tacker_ori_lbm(const float *src, float *dst, int sx, int sy, int sz, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_lbm(src, dst, sx, sy, sz);
+    if (rc) return rc;
+    if (sx > 1024) return fail(TK_ERROR_UNSUPPORTED, "ori_lbm: sx above 1024 needs the GPTB form");
+    return run_once(new OriLBMKernel(0, src, dst, sx, sy, sz), stream);
+}
+
+int tacker_gptb_lbm(const float *src, float *dst, int sx, int sy, int sz, int block_start, int block_end,
+                    int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_lbm(src, dst, sx, sy, sz);
+    if (rc) return rc;
+    return run_gptb_once(new OriLBMKernel(0, src, dst, sx, sy, sz), block_start, block_end, launch_grid,
+                         launch_block, stream);
+}
+
+int tacker_mriq_phimag(const float *phiR, const float *phiI, float *phiMag, int numK, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    if (!phiR || !phiI || !phiMag || numK < 0) return fail(TK_ERROR_INVALID_VALUE, "mriq_phimag: bad arguments");
+    if (numK == 0) return TK_SUCCESS;
+    void *args[] = {&phiR, &phiI, &phiMag, &numK};
+    const dim3 grid((numK + KERNEL_PHI_MAG_THREADS_PER_BLOCK - 1) / KERNEL_PHI_MAG_THREADS_PER_BLOCK);
+    const int rc = tkLaunchKernel(fmap["ori_ComputePhiMag"], grid.raw(), dim3(KERNEL_PHI_MAG_THREADS_PER_BLOCK).raw(), args, 0, stream);
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+int tacker_mriq_set_kvalues(const float *kvals_host, int numK)
+{
+    REQUIRE_INIT();
+    if (!kvals_host || numK < 0 || numK > MRIQ_MAX_K) return fail(TK_ERROR_INVALID_VALUE, "mriq: numK out of range");
+    const int rc = OriMRIQKernel::setKValues(reinterpret_cast<const mriq_kValues *>(kvals_host), numK);
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+int tacker_ori_mriq(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi, int numX, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_mriq(numK, x, y, z, Qr, Qi, numX);
+    if (rc) return rc;
+    if (numX == 0) return TK_SUCCESS;
+    return run_once(new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX), stream);
+}
+
+int tacker_gptb_mriq(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi, int numX,
+                     int block_start, int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_mriq(numK, x, y, z, Qr, Qi, numX);
+    if (rc) return rc;
+    if (numX == 0) return TK_SUCCESS;
+    return run_gptb_once(new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX), block_start, block_end, launch_grid,
+                         launch_block, stream);
+}
+
+int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane)
+{
+    REQUIRE_INIT();
+    if (!atoms_host || count < 0 || count > MAXATOMS) return fail(TK_ERROR_INVALID_VALUE, "cp: atom count out of range");
+    const int rc = cpCopyAtomsToConstBuf(atoms_host, count, zplane);
+    return rc ? fail(rc < 0 ? TK_ERROR_INVALID_VALUE : rc, "cp: loading the atom table failed") : rc;
+}
+
+int tacker_cp_initatoms(float *atoms_host, int count, unsigned volx, unsigned voly, unsigned volz, float gridspacing)
+{
+    if (!atoms_host || count < 0) return fail(TK_ERROR_INVALID_VALUE, "cp_initatoms: bad arguments");
+    cpInitAtoms(atoms_host, count, volx, voly, volz, gridspacing);
+    return TK_SUCCESS;
+}
+
+int tacker_ori_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_cp(numatoms, energygrid, volx, voly);
+    if (rc) return rc;
+    return run_once(new OriCPKernel(0, numatoms, gridspacing, energygrid, volx, voly), stream);
+}
+
+int tacker_gptb_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, int block_start,
+                   int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_cp(numatoms, energygrid, volx, voly);
+    if (rc) return rc;
+    return run_gptb_once(new OriCPKernel(0, numatoms, gridspacing, energygrid, volx, voly), block_start, block_end,
+                         launch_grid, launch_block, stream);
+}
+
+int tacker_mix_tzgemm_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz,
+                              int be_start, int be_end, const void *A, const void *B, float *C, int M, int N,
+                              int K, int tile_start, int tile_end, const char *variant, int launch_grid,
+                              int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_stencil(A0, Anext, nx, ny, nz);
+    if (rc) return rc;
+    return run_mix_once(new OriSTENCILKernel(0, c0, c1, A0, Anext, nx, ny, nz), be_start, be_end, A, B, C, M, N, K,
+                        tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
+int tacker_mix_tzgemm_lbm(const float *src, float *dst, int sx, int sy, int sz, int be_start, int be_end,
+                          const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                          int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_lbm(src, dst, sx, sy, sz);
+    if (rc) return rc;
+    return run_mix_once(new OriLBMKernel(0, src, dst, sx, sy, sz), be_start, be_end, A, B, C, M, N, K, tile_start,
+                        tile_end, variant, launch_grid, launch_block, stream);
+}
+
+int tacker_mix_tzgemm_mriq(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi,
+                           int numX, int be_start, int be_end, const void *A, const void *B, float *C, int M,
+                           int N, int K, int tile_start, int tile_end, const char *variant, int launch_grid,
+                           int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_mriq(numK, x, y, z, Qr, Qi, numX);
+    if (rc) return rc;
+    return run_mix_once(new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX), be_start, be_end, A, B, C, M, N, K,
+                        tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
+int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, int be_start,
+                         int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                         int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_cp(numatoms, energygrid, volx, voly);
+    if (rc) return rc;
+    return run_mix_once(new OriCPKernel(0, numatoms, gridspacing, energygrid, volx, voly), be_start, be_end, A, B, C,
+                        M, N, K, tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
+int tacker_im2col(const float *data_im, int channels, int height, int width, int kernel_h, int kernel_w,
+                  int pad_h, int pad_w, int stride_h, int stride_w, int dilation_h, int dilation_w,
+                  float *data_col, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    if (!data_im || !data_col || channels < 1 || height < 1 || width < 1 || kernel_h < 1 || kernel_w < 1 ||
+        stride_h < 1 || stride_w < 1 || dilation_h < 1 || dilation_w < 1 || pad_h < 0 || pad_w < 0)
+        return fail(TK_ERROR_INVALID_VALUE, "im2col: bad arguments");
+    int height_col = (height + 2 * pad_h - (dilation_h * (kernel_h - 1) + 1)) / stride_h + 1;
+    int width_col = (width + 2 * pad_w - (dilation_w * (kernel_w - 1) + 1)) / stride_w + 1;
+    if (height_col < 1 || width_col < 1) return fail(TK_ERROR_INVALID_VALUE, "im2col: empty output");
+    int n = channels * height_col * width_col;
+    int im_size = channels * height * width;
+    int col_size = channels * kernel_h * kernel_w * height_col * width_col;
+    void *args[] = {&n, &data_im, &height, &width, &kernel_h, &kernel_w, &pad_h, &pad_w, &stride_h, &stride_w,
+                    &dilation_h, &dilation_w, &height_col, &width_col, &data_col, &im_size, &col_size};
+    // grid-stride launch: 2 workgroups of 256 per CU, as the reference's SM_NUM*2
+    const int rc = tkLaunchKernel(fmap["im2col"], dim3(cuCount() * 2).raw(), dim3(256).raw(), args, 0, stream);
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+int tacker_convert_fp32_to_fp16(void *out_f16, const float *in, int n, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    if (!out_f16 || !in || n < 0) return fail(TK_ERROR_INVALID_VALUE, "convert: bad arguments");
+    if (n == 0) return TK_SUCCESS;
+    void *args[] = {&out_f16, &in, &n};
+    const int rc = tkLaunchKernel(fmap["convert_fp32_to_fp16"], dim3((n + 255) / 256).raw(), dim3(256).raw(), args, 0, stream);
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+int tacker_mnk_from_conv_args(const int a[14], int mnk[3])
+{
+    const int height_col = (a[2] + 2 * a[8] - (a[12] * (a[6] - 1) + 1)) / a[10] + 1;
+    const int width_col = (a[3] + 2 * a[9] - (a[13] * (a[7] - 1) + 1)) / a[11] + 1;
+    mnk[0] = a[0] * height_col * width_col;
+    mnk[1] = a[4];
+    mnk[2] = a[6] * a[7] * a[1];
+    return TK_SUCCESS;
+}
+
+int tacker_get_kernel_info(const char *kernel, const char *key) { return get_kernel_info(kernel, key); }
+float tacker_fget_kernel_info(const char *kernel, const char *key) { return fget_kernel_info(kernel, key); }
+
+// ---- object API -------------------------------------------------------------
+
+tacker_kernel_t tacker_create_kernel(const char *name)
+{
+    if (!tacker_runtime_ready() || !name) {
+        fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
+        return nullptr;
+    }
+    static const char *known[] = {"cp", "lbm", "mriq", "stencil", "tzgemm"};
+    bool ok = false;
+    for (auto k : known) ok |= (strcmp(k, name) == 0);
+    if (!ok) {
+        fail(TK_ERROR_NOT_FOUND, std::string("Creator: Kernel not found: ") + name);
+        return nullptr;
+    }
+    tacker_kernel_t out = nullptr;
+    guarded([&]() -> int {
+        out = static_cast<Kernel *>(createKernel(name));
+        return TK_SUCCESS;
+    });
+    return out;
+}
+
+#define CREATE(check_expr, new_expr)                          \
+    do {                                                      \
+        if (!tacker_runtime_ready()) {                        \
+            fail(TK_ERROR_INVALID_VALUE, "not initialised");  \
+            return nullptr;                                   \
+        }                                                     \
+        if (check_expr) return nullptr;                       \
+        tacker_kernel_t out_ = nullptr;                       \
+        guarded([&]() -> int {                                         \
+            out_ = static_cast<Kernel *>(new_expr);           \
+            return TK_SUCCESS;                                \
+        });                                                   \
+        return out_;                                          \
+    } while (0)
+
+tacker_kernel_t tacker_ori_stencil_create(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz)
+{
+    CREATE(check_stencil(A0, Anext, nx, ny, nz), new OriSTENCILKernel(0, c0, c1, A0, Anext, nx, ny, nz));
+}
+tacker_kernel_t tacker_ori_lbm_create(const float *src, float *dst, int sx, int sy, int sz)
+{
+    CREATE(check_lbm(src, dst, sx, sy, sz), new OriLBMKernel(0, src, dst, sx, sy, sz));
+}
+tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi, int numX)
+{
+    CREATE(check_mriq(numK, x, y, z, Qr, Qi, numX), new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX));
+}
+tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid, int volx, int voly)
+{
+    CREATE(check_cp(numatoms, energygrid, volx, voly), new OriCPKernel(0, numatoms, gridspacing, energygrid, volx, voly));
+}
+tacker_kernel_t tacker_ori_tzgemm_create(const void *A, const void *B, float *C, int m, int n, int k)
+{
+    if (m < 1 || n < 1 || k < 1) {
+        fail(TK_ERROR_INVALID_VALUE, "tzgemm: bad dimensions");
+        return nullptr;
+    }
+    if (!A) CREATE(0, new OriTZGEMMKernel(0, m, n, k));
+    CREATE((!B || !C) ? fail(TK_ERROR_INVALID_VALUE, "tzgemm: null operand") : 0, new OriTZGEMMKernel(0, m, n, k, A, B, C));
+}
+
+tacker_kernel_t tacker_gptb_create(tacker_kernel_t ori_handle, int launch_grid, int launch_block, int start, int end)
+{
+    Kernel *ori = static_cast<Kernel *>(ori_handle);
+    if (!ori || dynamic_cast<GPTBKernel *>(ori) || dynamic_cast<MixKernel *>(ori)) {
+        fail(TK_ERROR_INVALID_VALUE, "tacker_gptb_create: handle is not an ori kernel");
+        return nullptr;
+    }
+    const int block = launch_block > 0 ? launch_block : (ori->kernelName == "tzgemm" ? TZ_THREADS : default_block(ori->kernelName));
+    CREATE(check_range(ori, start, end) || check_block(ori->kernelName, block), make_gptb(ori, launch_grid, block, start, end));
+}
+
+int tacker_gptb_set_range(tacker_kernel_t h, int start, int end)
+{
+    GPTBKernel *g = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(h));
+    if (!g) return fail(TK_ERROR_INVALID_VALUE, "not a GPTB kernel");
+    const int rc = check_range(g->kernel_, start, end);
+    if (rc) return rc;
+    g->gptbParams.ptb_start_block_pos = start;
+    g->gptbParams.ptb_end_block_pos = end;
+    return TK_SUCCESS;
+}
+
+tacker_kernel_t tacker_mix_create(tacker_kernel_t be_h, tacker_kernel_t tz_h, int be_start, int be_end,
+                                  int tile_start, int tile_end, const char *variant, int launch_grid, int launch_block)
+{
+    GPTBKernel *be = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(be_h));
+    GPTBKernel *tz = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(tz_h));
+    if (!be || !tz || tz->kernelName != "tzgemm" || be->kernelName == "tzgemm") {
+        fail(TK_ERROR_INVALID_VALUE, "tacker_mix_create: need a best-effort GPTB kernel and a tzgemm GPTB kernel");
+        return nullptr;
+    }
+    const std::string v = variant ? variant : "";
+    const std::string key = "tzgemm_" + be->kernelName + (v.empty() ? "" : "@" + v);
+    if (!has_key(key) || get_kernel_info(key, "blocksize") == JSON_NOT_FOUND) {
+        fail(TK_ERROR_NOT_FOUND, "no fused kernel {" + key + "}");
+        return nullptr;
+    }
+    if (launch_block > 0 && launch_block != get_kernel_info(key, "blocksize")) {
+        fail(TK_ERROR_INVALID_VALUE, "{" + key + "} is built for another workgroup size");
+        return nullptr;
+    }
+    CREATE(check_range(be->kernel_, be_start, be_end) || check_range(tz->kernel_, tile_start, tile_end),
+           createTzgemmMix(be, tz, be_start, be_end, tile_start, tile_end, v, launch_grid, launch_block));
+}
+
+int tacker_mix_set_range(tacker_kernel_t h, int be_start, int be_end, int tile_start, int tile_end)
+{
+    MixKernel *m = dynamic_cast<MixKernel *>(static_cast<Kernel *>(h));
+    if (!m) return fail(TK_ERROR_INVALID_VALUE, "not a mix kernel");
+    if (be_start < 0 || be_end < be_start || tile_start < 0 || tile_end < tile_start)
+        return fail(TK_ERROR_INVALID_VALUE, "bad range");
+    m->kernel1_start_block_pos = be_start;
+    m->kernel1_end_block_pos = be_end;
+    m->kernel2_start_block_pos = tile_start;
+    m->kernel2_end_block_pos = tile_end;
+    return TK_SUCCESS;
+}
+
+int tacker_kernel_execute(tacker_kernel_t h, tkStream_t stream)
+{
+    Kernel *k = static_cast<Kernel *>(h);
+    if (!k) return fail(TK_ERROR_INVALID_VALUE, "null kernel");
+    if (dynamic_cast<OriTZGEMMKernel *>(k)) return fail(TK_ERROR_UNSUPPORTED, "the GEMM runs only in GPTB or fused form");
+    return guarded([&]() -> int {
+        k->execute(stream);
+        return TK_SUCCESS;
+    });
+}
+
+int tacker_kernel_swap_buffers(tacker_kernel_t h)
+{
+    Kernel *k = static_cast<Kernel *>(h);
+    if (auto *g = dynamic_cast<GPTBKernel *>(k)) k = g->kernel_;
+    if (auto *s = dynamic_cast<OriSTENCILKernel *>(k)) { s->swapGrids(); return TK_SUCCESS; }
+    if (auto *l = dynamic_cast<OriLBMKernel *>(k)) { l->swapGrids(); return TK_SUCCESS; }
+    return fail(TK_ERROR_INVALID_VALUE, "only stencil and lbm objects ping-pong");
+}
+
+int tacker_kernel_info(tacker_kernel_t h, int out[8])
+{
+    Kernel *k = static_cast<Kernel *>(h);
+    if (!k) return fail(TK_ERROR_INVALID_VALUE, "null kernel");
+    memset(out, 0, 8 * sizeof(int));
+    out[0] = (int)k->launchGridDim.x;
+    out[1] = (int)(k->launchBlockDim.x * k->launchBlockDim.y * k->launchBlockDim.z);
+    out[4] = (int)k->kernelParams.size();
+    out[5] = (int)k->smem;
+    Kernel *ori = k;
+    if (auto *g = dynamic_cast<GPTBKernel *>(k)) {
+        out[2] = g->gptbParams.ptb_start_block_pos;
+        out[3] = g->gptbParams.ptb_end_block_pos;
+        ori = g->kernel_;
+    }
+    out[6] = (int)ori->launchGridDim.x;
+    out[7] = (int)ori->launchGridDim.y;
+    return TK_SUCCESS;
+}
+
+int tacker_kernel_destroy(tacker_kernel_t h)
+{
+    delete static_cast<Kernel *>(h);
+    return TK_SUCCESS;
+}
+
+int tacker_spin_fail_flag(int *flag)
+{
+    REQUIRE_INIT();
+    if (!flag) return fail(TK_ERROR_INVALID_VALUE, "null output");
+    unsigned v = 0, zero = 0;
+    int rc = tkMemcpyFromSymbol(&v, "tk_spin_fail", sizeof(v), 0);
+    if (!rc && v) rc = tkMemcpyToSymbol("tk_spin_fail", &zero, sizeof(zero), 0);
+    *flag = (int)v;
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+uint16_t tacker_float_to_half_bits(float f) { return tk::float_to_half_bits(f); }
+
+int tacker_rng_uniform(uint64_t seed, float lo, float hi, float *out, size_t n)
+{
+    if (!out) return fail(TK_ERROR_INVALID_VALUE, "null output");
+    tk::Rng rng(seed);
+    for (size_t i = 0; i < n; ++i) out[i] = rng.uniform(lo, hi);
+    return TK_SUCCESS;
+}
+
+}  // extern "C"

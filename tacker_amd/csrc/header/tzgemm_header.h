@@ -1,0 +1,21 @@
+// tzgemm tile constants.
+// The reference (src/header/tzgemm_header.h) describes a 64x64 CTA tile built
+// from 16x16x16 WMMA fragments by 4 warps of 32.  Its tile is kept as the unit
+// of the [start,end) range interface (TZ_REF_TILE); the gfx950 kernel computes a
+// 128x128 macro tile (2x2 reference tiles) per 256-thread workgroup with
+// v_mfma_f32_16x16x32_f16, one reference tile per 64-wide wavefront.
+#pragma once
+#include "pets_common.h"
+
+#define TZ_REF_TILE 64            // BLOCK_ROW_TILES * WMMA_N of the reference
+#define TZ_MACRO_TILE 128         // rows and columns of C per workgroup
+#define TZ_THREADS 256            // 4 wavefronts, 2x2 over the macro tile
+#define TZ_MFMA_M 16
+#define TZ_MFMA_N 16
+#define TZ_MFMA_K 32
+#define TZ_BLOCK_K 32             // K extent staged in LDS per stage
+#define TZ_LDS_ROW_BYTES (TZ_BLOCK_K * 2 + 16)   // 16 B skew against bank conflicts
+#define TZ_LDS_STAGES 2
+#define TZ_LDS_BYTES (TZ_LDS_STAGES * 2 * TZ_MACRO_TILE * TZ_LDS_ROW_BYTES)
+
+#define TZ_ALPHA 1.1f             // alpha_g, src/header/tzgemm_header.h:64

@@ -1,0 +1,200 @@
+// Single device translation unit of libtacker_amd.so: the natural-grid ("ori")
+// kernels, their persistent-workgroup GPTB forms, the generated fused kernels,
+// the small data-movement kernels of the conv->GEMM path, and the registry that
+// hands all of them to the host by name.
+//
+// Names follow the reference: ori_<k> (src/ori_kernel/*.cu), gptb keys of
+// src/main.cu:108-125 (general_ptb_* / g_general_ptb_*), <be>_tzgemm_mix
+// (src/mix_kernel/tzgemm_*.cu).  Parameter lists are the reference's, so the
+// host marshals arguments exactly as GPTBKernel / MixKernel do.
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include "../../../include/tacker_amd.h"
+#include "cp_role.h"
+#include "lbm_role.h"
+#include "mriq_role.h"
+#include "stencil_role.h"
+#include "tzgemm_role.h"
+
+#define GPTB_TRAILER                                                                            \
+    int grid_dimension_x, int grid_dimension_y, int grid_dimension_z, int block_dimension_x,    \
+        int block_dimension_y, int block_dimension_z, int ptb_start_block_pos,                  \
+        int ptb_iter_block_step, int ptb_end_block_pos, int thread_base
+
+// ------------------------------------------------------------------ ori kernels
+
+// grid (ceil(nx/64), ceil(ny/4)), block (32,4): wave w of the 2 takes rows 2w, 2w+1.
+extern "C" __global__ __launch_bounds__(128) void ori_stencil(float c0, float c1, float *A0,
+                                                              float *Anext, int nx, int ny, int nz)
+{
+    const int tid = threadIdx.x + threadIdx.y * blockDim.x;
+    const int wave = tid >> 6;
+    tk::stencil_wave_block<2>(c0, c1, A0, Anext, nx, ny, nz, blockIdx.x * 2 * STENCIL_TILE_X,
+                              blockIdx.y * STENCIL_TILE_Y + 2 * wave, tid & 63);
+}
+
+// grid (sy, sz), block sx
+extern "C" __global__ void ori_lbm(float *srcGrid, float *dstGrid)
+{
+    const int sx = blockDim.x, sy = gridDim.x, sz = gridDim.y;
+    const int c = threadIdx.x + blockIdx.x * sx + blockIdx.y * sx * sy;
+    tk::lbm_cell(srcGrid, dstGrid, sx * sy * sz, c, sx, sx * sy);
+}
+
+extern "C" __global__ void ori_ComputePhiMag(float *phiR, float *phiI, float *phiMag, int numK)
+{
+    const int indexK = blockIdx.x * blockDim.x + threadIdx.x;
+    if (indexK < numK) {
+        const float real = phiR[indexK];
+        const float imag = phiI[indexK];
+        phiMag[indexK] = real * real + imag * imag;
+    }
+}
+
+// grid numX/256, block 256
+extern "C" __global__ __launch_bounds__(256) void ori_mriq(int numK, int kGlobalIndex, float *x,
+                                                           float *y, float *z, float *Qr, float *Qi)
+{
+    (void)kGlobalIndex;
+    tk::mriq_voxel(numK, x, y, z, Qr, Qi, blockIdx.x * KERNEL_Q_THREADS_PER_BLOCK + threadIdx.x);
+}
+
+// grid (volx/128, voly/8), block (16,8)
+extern "C" __global__ __launch_bounds__(128) void ori_cp(int numatoms, float gridspacing,
+                                                         float *energygrid)
+{
+    tk::cp_block(numatoms, gridspacing, energygrid, blockIdx.x, blockIdx.y, gridDim.x, threadIdx.x,
+                 threadIdx.y);
+}
+
+// ------------------------------------------------------------------ GPTB kernels
+
+extern "C" __global__ __launch_bounds__(TZ_THREADS) void general_ptb_tzgemm(
+    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, GPTB_TRAILER)
+{
+    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
+    tk::WorkgroupSync sync;
+    tk::tzgemm_role(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x, ptb_iter_block_step,
+                    ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base, tz_lds,
+                    sync);
+}
+
+extern "C" __global__ void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
+                                               int ny, int nz, GPTB_TRAILER)
+{
+    tk::stencil_role(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y,
+                     (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
+                     (int)threadIdx.x - thread_base, (int)blockDim.x);
+}
+
+extern "C" __global__ void general_ptb_lbm(float *srcGrid, float *dstGrid, GPTB_TRAILER)
+{
+    tk::lbm_role(srcGrid, dstGrid, grid_dimension_x, grid_dimension_y, block_dimension_x,
+                 (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
+                 (int)threadIdx.x - thread_base, (int)blockDim.x);
+}
+
+extern "C" __global__ void g_general_ptb_mriq(int numK, int kGlobalIndex, float *x, float *y,
+                                              float *z, float *Qr, float *Qi, GPTB_TRAILER)
+{
+    (void)kGlobalIndex;
+    tk::mriq_role(numK, x, y, z, Qr, Qi, grid_dimension_x, (int)blockIdx.x, ptb_iter_block_step,
+                  ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base,
+                  (int)blockDim.x);
+}
+
+extern "C" __global__ void g_general_ptb_cp(int numatoms, float gridspacing, float *energygrid,
+                                            GPTB_TRAILER)
+{
+    tk::cp_role(numatoms, gridspacing, energygrid, grid_dimension_x, grid_dimension_y,
+                (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
+                (int)threadIdx.x - thread_base, (int)blockDim.x);
+}
+
+// ------------------------------------------------------------------ conv -> GEMM helpers
+
+// Caffe im2col, NCHW (src/TaskManager.cu:48-82): grid-stride over
+// channels*height_col*width_col work items.
+extern "C" __global__ void im2col_gpu_kernel_(int n, float *data_im, int height, int width,
+                                              int kernel_h, int kernel_w, int pad_h, int pad_w,
+                                              int stride_h, int stride_w, int dilation_h,
+                                              int dilation_w, int height_col, int width_col,
+                                              float *data_col, int data_im_size, int data_col_size)
+{
+    (void)data_im_size;
+    (void)data_col_size;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += blockDim.x * gridDim.x) {
+        const int h_index = i / width_col;
+        const int h_col = h_index % height_col;
+        const int w_col = i % width_col;
+        const int c_im = h_index / height_col;
+        const int c_col = c_im * kernel_h * kernel_w;
+        const int h_offset = h_col * stride_h - pad_h;
+        const int w_offset = w_col * stride_w - pad_w;
+        float *data_col_ptr = data_col + ((size_t)c_col * height_col + h_col) * width_col + w_col;
+        const float *data_im_ptr = data_im + ((long)c_im * height + h_offset) * width + w_offset;
+        for (int ki = 0; ki < kernel_h; ++ki) {
+            for (int kj = 0; kj < kernel_w; ++kj) {
+                const int h_im = h_offset + ki * dilation_h;
+                const int w_im = w_offset + kj * dilation_w;
+                *data_col_ptr = (h_im >= 0 && w_im >= 0 && h_im < height && w_im < width)
+                                    ? data_im_ptr[ki * dilation_h * width + kj * dilation_w]
+                                    : 0.0f;
+                data_col_ptr += (size_t)height_col * width_col;
+            }
+        }
+    }
+}
+
+// src/TaskManager.cu:85-90
+extern "C" __global__ void convertFp32ToFp16_(_Float16 *out, float *in, int n)
+{
+    const int idx = blockDim.x * blockIdx.x + threadIdx.x;
+    if (idx < n) out[idx] = (_Float16)in[idx];
+}
+
+// ------------------------------------------------------------------ fused kernels (generated)
+#include "../mix_kernel/mix_kernels.inc"
+
+// ------------------------------------------------------------------ registry
+extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
+{
+    if (!insert) return TK_ERROR_INVALID_VALUE;
+    insert("ori_stencil", (const void *)ori_stencil, ctx);
+    insert("ori_lbm", (const void *)ori_lbm, ctx);
+    insert("ori_ComputePhiMag", (const void *)ori_ComputePhiMag, ctx);
+    insert("ori_mriq", (const void *)ori_mriq, ctx);
+    insert("ori_cp", (const void *)ori_cp, ctx);
+    insert("gptb_tzgemm", (const void *)general_ptb_tzgemm, ctx);
+    insert("gptb_stencil", (const void *)general_ptb_stencil, ctx);
+    insert("gptb_lbm", (const void *)general_ptb_lbm, ctx);
+    insert("gptb_mriq", (const void *)g_general_ptb_mriq, ctx);
+    insert("gptb_cp", (const void *)g_general_ptb_cp, ctx);
+    insert("im2col", (const void *)im2col_gpu_kernel_, ctx);
+    insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);
+    tk_register_mix_kernels(insert, ctx);
+    return TK_SUCCESS;
+}
+
+// Device symbols the host fills by name (cudaMemcpyToSymbol in the reference).
+extern "C" int tk_device_symbol(const char *name, const void **symbol, size_t *bytes)
+{
+    if (!name) return TK_ERROR_INVALID_VALUE;
+    if (__builtin_strcmp(name, "ck") == 0) {
+        *symbol = (const void *)&ck;
+        *bytes = sizeof(ck);
+        return TK_SUCCESS;
+    }
+    if (__builtin_strcmp(name, "atominfo") == 0) {
+        *symbol = (const void *)&atominfo;
+        *bytes = sizeof(atominfo);
+        return TK_SUCCESS;
+    }
+    if (__builtin_strcmp(name, "tk_spin_fail") == 0) {
+        *symbol = (const void *)&tk_spin_fail;
+        *bytes = sizeof(tk_spin_fail);
+        return TK_SUCCESS;
+    }
+    return TK_ERROR_NOT_FOUND;
+}

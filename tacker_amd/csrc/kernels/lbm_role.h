@@ -1,0 +1,164 @@
+// D3Q19 lattice-Boltzmann role (collide + scatter, one time step).
+//
+// Replaces ori_lbm / general_ptb_lbm / lbm_tzgemm_lbm0 of the reference
+// (src/ori_kernel/lbm_kernel.cu:9-154, src/gptb_kernel/lbm_kernel.cu:3-178,
+// src/mix_kernel/tzgemm_lbm.cu:6-181) with run-time grid extents.  Kept: SoA
+// layout CALC_INDEX(x,y,z,e) = cells*e + x + y*sx + z*sx*sy, SCATTER streaming
+// by linear index arithmetic without boundary clamping, obstacle bounce-back,
+// ACCEL override, and the exact fp32 operation order of the collision.
+//
+// One departure, on purpose: a scatter whose linear target cell lies outside
+// [0, cells) would land in the neighbouring entry plane, where the reference
+// races with that plane's own writer.  Here such a store is dropped, i.e. the
+// race is always resolved in favour of the in-range writer, so results are
+// reproducible.
+//
+// gfx950 design: a block is one x-row (y,z); lane = x, so each of the 20 loads
+// and 19 stores of a wave is one contiguous row segment.  No LDS, no barrier.
+// A role of T threads processes T / roundup64(sx) rows at once.
+#pragma once
+#include "role_common.h"
+#include "../header/lbm_header.h"
+
+namespace tk {
+
+// All indices are 32-bit: the host refuses grids with 20*cells >= 2^31.
+__device__ __forceinline__ void lbm_cell(const float *__restrict__ src, float *__restrict__ dst,
+                                         int cells, int c, int sx, int sxy)
+{
+    float tempC = src[cells * LBM_C + c];
+    float tempN = src[cells * LBM_N + c];
+    float tempS = src[cells * LBM_S + c];
+    float tempE = src[cells * LBM_E + c];
+    float tempW = src[cells * LBM_W + c];
+    float tempT = src[cells * LBM_T + c];
+    float tempB = src[cells * LBM_B + c];
+    float tempNE = src[cells * LBM_NE + c];
+    float tempNW = src[cells * LBM_NW + c];
+    float tempSE = src[cells * LBM_SE + c];
+    float tempSW = src[cells * LBM_SW + c];
+    float tempNT = src[cells * LBM_NT + c];
+    float tempNB = src[cells * LBM_NB + c];
+    float tempST = src[cells * LBM_ST + c];
+    float tempSB = src[cells * LBM_SB + c];
+    float tempET = src[cells * LBM_ET + c];
+    float tempEB = src[cells * LBM_EB + c];
+    float tempWT = src[cells * LBM_WT + c];
+    float tempWB = src[cells * LBM_WB + c];
+    const unsigned flags = __float_as_uint(src[cells * LBM_FLAGS + c]);
+
+    if (flags & LBM_OBSTACLE) {
+        float t;
+        t = tempN; tempN = tempS; tempS = t;
+        t = tempE; tempE = tempW; tempW = t;
+        t = tempT; tempT = tempB; tempB = t;
+        t = tempNE; tempNE = tempSW; tempSW = t;
+        t = tempNW; tempNW = tempSE; tempSE = t;
+        t = tempNT; tempNT = tempSB; tempSB = t;
+        t = tempNB; tempNB = tempST; tempST = t;
+        t = tempET; tempET = tempWB; tempWB = t;
+        t = tempEB; tempEB = tempWT; tempWT = t;
+    } else {
+        float ux, uy, uz, rho, u2, temp1, temp2, temp_base;
+        rho = tempC + tempN + tempS + tempE + tempW + tempT + tempB + tempNE + tempNW + tempSE +
+              tempSW + tempNT + tempNB + tempST + tempSB + tempET + tempEB + tempWT + tempWB;
+        ux = +tempE - tempW + tempNE - tempNW + tempSE - tempSW + tempET + tempEB - tempWT - tempWB;
+        uy = +tempN - tempS + tempNE + tempNW - tempSE - tempSW + tempNT + tempNB - tempST - tempSB;
+        uz = +tempT - tempB + tempNT - tempNB + tempST - tempSB + tempET - tempEB + tempWT - tempWB;
+        ux /= rho;
+        uy /= rho;
+        uz /= rho;
+        if (flags & LBM_ACCEL) {
+            ux = 0.005f;
+            uy = 0.002f;
+            uz = 0.000f;
+        }
+        u2 = 1.5f * (ux * ux + uy * uy + uz * uz) - 1.0f;
+        temp_base = LBM_OMEGA * rho;
+        temp1 = LBM_DFL1 * temp_base;
+        temp2 = 1.0f - LBM_OMEGA;
+        tempC = temp2 * tempC + temp1 * (-u2);
+        temp1 = LBM_DFL2 * temp_base;
+        tempN = temp2 * tempN + temp1 * (uy * (4.5f * uy + 3.0f) - u2);
+        tempS = temp2 * tempS + temp1 * (uy * (4.5f * uy - 3.0f) - u2);
+        tempT = temp2 * tempT + temp1 * (uz * (4.5f * uz + 3.0f) - u2);
+        tempB = temp2 * tempB + temp1 * (uz * (4.5f * uz - 3.0f) - u2);
+        tempE = temp2 * tempE + temp1 * (ux * (4.5f * ux + 3.0f) - u2);
+        tempW = temp2 * tempW + temp1 * (ux * (4.5f * ux - 3.0f) - u2);
+        temp1 = LBM_DFL3 * temp_base;
+        tempNT = temp2 * tempNT + temp1 * ((+uy + uz) * (4.5f * (+uy + uz) + 3.0f) - u2);
+        tempNB = temp2 * tempNB + temp1 * ((+uy - uz) * (4.5f * (+uy - uz) + 3.0f) - u2);
+        tempST = temp2 * tempST + temp1 * ((-uy + uz) * (4.5f * (-uy + uz) + 3.0f) - u2);
+        tempSB = temp2 * tempSB + temp1 * ((-uy - uz) * (4.5f * (-uy - uz) + 3.0f) - u2);
+        tempNE = temp2 * tempNE + temp1 * ((+ux + uy) * (4.5f * (+ux + uy) + 3.0f) - u2);
+        tempSE = temp2 * tempSE + temp1 * ((+ux - uy) * (4.5f * (+ux - uy) + 3.0f) - u2);
+        tempET = temp2 * tempET + temp1 * ((+ux + uz) * (4.5f * (+ux + uz) + 3.0f) - u2);
+        tempEB = temp2 * tempEB + temp1 * ((+ux - uz) * (4.5f * (+ux - uz) + 3.0f) - u2);
+        tempNW = temp2 * tempNW + temp1 * ((-ux + uy) * (4.5f * (-ux + uy) + 3.0f) - u2);
+        tempSW = temp2 * tempSW + temp1 * ((-ux - uy) * (4.5f * (-ux - uy) + 3.0f) - u2);
+        tempWT = temp2 * tempWT + temp1 * ((-ux + uz) * (4.5f * (-ux + uz) + 3.0f) - u2);
+        tempWB = temp2 * tempWB + temp1 * ((-ux - uz) * (4.5f * (-ux - uz) + 3.0f) - u2);
+    }
+
+#define TK_LBM_SCATTER(entry, dx, dy, dz, value)                          \
+    do {                                                                  \
+        const int t_ = c + (dx) + (dy) * sx + (dz) * sxy;                 \
+        if (t_ >= 0 && t_ < cells) dst[cells * (entry) + t_] = (value);   \
+    } while (0)
+    TK_LBM_SCATTER(LBM_C, 0, 0, 0, tempC);
+    TK_LBM_SCATTER(LBM_N, 0, +1, 0, tempN);
+    TK_LBM_SCATTER(LBM_S, 0, -1, 0, tempS);
+    TK_LBM_SCATTER(LBM_E, +1, 0, 0, tempE);
+    TK_LBM_SCATTER(LBM_W, -1, 0, 0, tempW);
+    TK_LBM_SCATTER(LBM_T, 0, 0, +1, tempT);
+    TK_LBM_SCATTER(LBM_B, 0, 0, -1, tempB);
+    TK_LBM_SCATTER(LBM_NE, +1, +1, 0, tempNE);
+    TK_LBM_SCATTER(LBM_NW, -1, +1, 0, tempNW);
+    TK_LBM_SCATTER(LBM_SE, +1, -1, 0, tempSE);
+    TK_LBM_SCATTER(LBM_SW, -1, -1, 0, tempSW);
+    TK_LBM_SCATTER(LBM_NT, 0, +1, +1, tempNT);
+    TK_LBM_SCATTER(LBM_NB, 0, +1, -1, tempNB);
+    TK_LBM_SCATTER(LBM_ST, 0, -1, +1, tempST);
+    TK_LBM_SCATTER(LBM_SB, 0, -1, -1, tempSB);
+    TK_LBM_SCATTER(LBM_ET, +1, 0, +1, tempET);
+    TK_LBM_SCATTER(LBM_EB, +1, 0, -1, tempEB);
+    TK_LBM_SCATTER(LBM_WT, -1, 0, +1, tempWT);
+    TK_LBM_SCATTER(LBM_WB, -1, 0, -1, tempWB);
+#undef TK_LBM_SCATTER
+}
+
+// grid_dimension_x = sy, grid_dimension_y = sz, block_dimension_x = sx
+// (src/ori_kernel/lbm_kernel.cu:218-222).
+__device__ __forceinline__ void lbm_role(const float *__restrict__ src, float *__restrict__ dst,
+                                         int grid_dimension_x, int grid_dimension_y,
+                                         int block_dimension_x, int role_block, int role_blocks,
+                                         int start, int end, int tid, int role_threads)
+{
+    const int sx = block_dimension_x, sy = grid_dimension_x, sz = grid_dimension_y;
+    const int sxy = sx * sy;
+    const int cells = sxy * sz;
+    const int lanes_per_row = ((sx + TK_WAVE_SIZE - 1) / TK_WAVE_SIZE) * TK_WAVE_SIZE;
+    int rows_at_once = role_threads / lanes_per_row;
+    int row_slot, x_first, x_step;
+    if (rows_at_once >= 1) {
+        row_slot = tid / lanes_per_row;
+        x_first = tid % lanes_per_row;
+        x_step = lanes_per_row;
+        if (row_slot >= rows_at_once) return;
+    } else {   // row longer than the role: the role's threads sweep it
+        rows_at_once = 1;
+        row_slot = 0;
+        x_first = tid;
+        x_step = role_threads;
+    }
+    const unsigned stride = (unsigned)role_blocks * rows_at_once;
+    for (unsigned pos = (unsigned)start + role_block * rows_at_once + row_slot; pos < (unsigned)end;
+         pos += stride) {
+        const int y = pos % sy;
+        const int z = (pos / sy) % sz;
+        for (int x = x_first; x < sx; x += x_step)
+            lbm_cell(src, dst, cells, x + y * sx + z * sxy, sx, sxy);
+    }
+}
+
+}  // namespace tk

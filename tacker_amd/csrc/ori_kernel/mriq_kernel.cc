@@ -1,0 +1,115 @@
+#include "mriq_kernel.h"
+
+#include <unordered_map>
+#include <vector>
+
+#include "../Logger.h"
+#include "../rng.h"
+
+extern Logger logger;
+extern std::unordered_map<std::string, void *> fmap;
+
+OriMRIQKernel::OriMRIQKernel(int id)
+{
+    Id = id;
+    this->kernelName = "mriq";
+    initParams();
+}
+
+OriMRIQKernel::OriMRIQKernel(int id, int numK, const float *x, const float *y, const float *z,
+                             float *Qr, float *Qi, int numX)
+    : numX_(numX)
+{
+    Id = id;
+    this->kernelName = "mriq";
+    MRIQKernelParams = new OriMRIQParamsStruct{numK, 0, const_cast<float *>(x), const_cast<float *>(y),
+                                               const_cast<float *>(z), Qr, Qi};
+    bind();
+}
+
+OriMRIQKernel::~OriMRIQKernel()
+{
+    for (auto &ptr : cudaFreeList) tkErrCheck(tkFree(ptr));
+    delete MRIQKernelParams;
+}
+
+int OriMRIQKernel::setKValues(const mriq_kValues *kvals, int numK)
+{
+    if (numK < 0 || numK > MRIQ_MAX_K) return TK_ERROR_INVALID_VALUE;
+    return tkMemcpyToSymbol("ck", kvals, (size_t)numK * sizeof(mriq_kValues), 0);
+}
+
+// The reference reads an input file that is not shipped and then forces numK to
+// 2097152 while only the first 1024 samples are ever used
+// (src/ori_kernel/mriq_kernel.cu:17,147,58-59).  Here: numK = 2048, numX =
+// 262144, kx,ky,kz and voxel coordinates uniform[-0.5,0.5), phi uniform[0,1),
+// Q = 0, same flow (device ComputePhiMag -> host AoS table -> constant memory).
+void OriMRIQKernel::initParams()
+{
+    const int numK = 2048;
+    numX_ = 262144;
+    tk::Rng rng(1337ULL);
+    std::vector<float> kx(numK), ky(numK), kz(numK), phiR(numK), phiI(numK);
+    std::vector<float> x(numX_), y(numX_), z(numX_);
+    for (int k = 0; k < numK; ++k) kx[k] = rng.uniform(-0.5f, 0.5f);
+    for (int k = 0; k < numK; ++k) ky[k] = rng.uniform(-0.5f, 0.5f);
+    for (int k = 0; k < numK; ++k) kz[k] = rng.uniform(-0.5f, 0.5f);
+    for (int i = 0; i < numX_; ++i) x[i] = rng.uniform(-0.5f, 0.5f);
+    for (int i = 0; i < numX_; ++i) y[i] = rng.uniform(-0.5f, 0.5f);
+    for (int i = 0; i < numX_; ++i) z[i] = rng.uniform(-0.5f, 0.5f);
+    for (int k = 0; k < numK; ++k) phiR[k] = rng.uniform();
+    for (int k = 0; k < numK; ++k) phiI[k] = rng.uniform();
+
+    float *d_phiR, *d_phiI, *d_phiMag, *d_x, *d_y, *d_z, *d_Qr, *d_Qi;
+    auto dev = [&](float **p, size_t n) {
+        TK_SAFE_CALL(tkMalloc((void **)p, n * sizeof(float)));
+        cudaFreeList.push_back(*p);
+    };
+    dev(&d_phiR, numK); dev(&d_phiI, numK); dev(&d_phiMag, numK);
+    dev(&d_x, numX_); dev(&d_y, numX_); dev(&d_z, numX_); dev(&d_Qr, numX_); dev(&d_Qi, numX_);
+    TK_SAFE_CALL(tkMemcpy(d_phiR, phiR.data(), numK * sizeof(float), TK_MEMCPY_H2D));
+    TK_SAFE_CALL(tkMemcpy(d_phiI, phiI.data(), numK * sizeof(float), TK_MEMCPY_H2D));
+    TK_SAFE_CALL(tkMemcpy(d_x, x.data(), numX_ * sizeof(float), TK_MEMCPY_H2D));
+    TK_SAFE_CALL(tkMemcpy(d_y, y.data(), numX_ * sizeof(float), TK_MEMCPY_H2D));
+    TK_SAFE_CALL(tkMemcpy(d_z, z.data(), numX_ * sizeof(float), TK_MEMCPY_H2D));
+    TK_SAFE_CALL(tkMemset(d_Qr, 0, numX_ * sizeof(float)));
+    TK_SAFE_CALL(tkMemset(d_Qi, 0, numX_ * sizeof(float)));
+
+    // phiMag on the device (ori_ComputePhiMag), then back for the AoS table
+    auto it = fmap.find("ori_ComputePhiMag");
+    if (it == fmap.end()) logger.ERROR("load kernel {ori_ComputePhiMag} failed!");
+    int nk = numK;
+    void *args[] = {&d_phiR, &d_phiI, &d_phiMag, &nk};
+    const dim3 grid((numK + KERNEL_PHI_MAG_THREADS_PER_BLOCK - 1) / KERNEL_PHI_MAG_THREADS_PER_BLOCK);
+    TK_SAFE_CALL(tkLaunchKernel(it->second, grid.raw(), dim3(KERNEL_PHI_MAG_THREADS_PER_BLOCK).raw(),
+                                args, 0, nullptr));
+    std::vector<float> phiMag(numK);
+    TK_SAFE_CALL(tkMemcpy(phiMag.data(), d_phiMag, numK * sizeof(float), TK_MEMCPY_D2H));
+    std::vector<mriq_kValues> kVals(numK);
+    for (int k = 0; k < numK; ++k) kVals[k] = mriq_kValues{kx[k], ky[k], kz[k], phiMag[k]};
+    TK_SAFE_CALL(setKValues(kVals.data(), numK));
+
+    MRIQKernelParams = new OriMRIQParamsStruct{numK, 0, d_x, d_y, d_z, d_Qr, d_Qi};
+    bind();
+}
+
+void OriMRIQKernel::bind()
+{
+    if (numX_ % KERNEL_Q_THREADS_PER_BLOCK != 0)
+        logger.ERROR("mriq: numX must be a multiple of 256");
+    launchGridDim = dim3(numX_ / KERNEL_Q_THREADS_PER_BLOCK, 1, 1);
+    launchBlockDim = dim3(KERNEL_Q_THREADS_PER_BLOCK, 1, 1);
+    OriMRIQParamsStruct *p = MRIQKernelParams;
+    kernelParams = {&p->numK, &p->kGlobalIndex, &p->x, &p->y, &p->z, &p->Qr, &p->Qi};
+    this->smem = 0;
+    auto it = fmap.find("ori_mriq");
+    this->kernelFunc = it == fmap.end() ? nullptr : it->second;
+    this->initialized = true;
+}
+
+void OriMRIQKernel::executeImpl(cudaStream_t stream)
+{
+    if (!kernelFunc) logger.ERROR("load kernel {ori_mriq} failed!");
+    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
+                                (void **)this->kernelParams.data(), 0, stream));
+}

@@ -1,0 +1,84 @@
+// runtime.cc -- process-wide state of the host runtime: the objects the
+// reference defines in src/main.cu (logger, recorder, moduleCenter, fmap) and in
+// src/TaskManager.cu:19-46 (global GEMM buffers), and the one-time set-up.
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "Logger.h"
+#include "ModuleCenter.h"
+#include "Recorder.h"
+#include "json.h"
+#include "rng.h"
+#include "tzgemm_kernel.h"
+#include "mix_kernel/kinfo_builtin.inc"
+
+Logger logger("", getenv("TACKER_QUIET") == nullptr, false);
+Recorder recorder;
+ModuleCenter moduleCenter;
+std::unordered_map<std::string, void *> fmap;
+
+long long MAX_ORI_WMMA_A = 0;
+long long MAX_ORI_WMMA_B = 0;
+long long MAX_ORI_WMMA_C = 0;
+bool gemm_malloced = false;
+void *ori_wmma_A = nullptr;
+void *ori_wmma_B = nullptr;
+float *ori_wmma_C = nullptr;
+
+static void grow(void **ptr, long long *have, long long need, bool seed_halves)
+{
+    if (need <= *have) return;
+    TK_SAFE_CALL(tkDeviceSynchronize());   // nothing may still be using the old buffer
+    if (*ptr) TK_SAFE_CALL(tkFree(*ptr));
+    TK_SAFE_CALL(tkMalloc(ptr, (size_t)need));
+    *have = need;
+    if (seed_halves) {
+        std::vector<uint16_t> host((size_t)need / 2);
+        tk::Rng rng(1337ULL + (uint64_t)need);
+        for (auto &h : host) h = tk::float_to_half_bits(rng.uniform(-1.0f, 1.0f));
+        TK_SAFE_CALL(tkMemcpy(*ptr, host.data(), (size_t)need, TK_MEMCPY_H2D));
+    } else {
+        TK_SAFE_CALL(tkMemset(*ptr, 0, (size_t)need));
+    }
+}
+
+void ensureGlobalGemmBuffers(int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
+{
+    const long long a = 2LL * M_GLOBAL * K_GLOBAL;
+    const long long b = 2LL * N_GLOBAL * K_GLOBAL;
+    const long long c = 4LL * M_GLOBAL * N_GLOBAL;
+    if (!gemm_malloced)
+        logger.INFO("[ori_tzgemm][initParams] allocating global GEMM buffers A " + std::to_string(a >> 20) +
+                    " MB, B " + std::to_string(b >> 20) + " MB, C " + std::to_string(c >> 20) + " MB");
+    grow(&ori_wmma_A, &MAX_ORI_WMMA_A, a, true);
+    grow(&ori_wmma_B, &MAX_ORI_WMMA_B, b, true);
+    grow((void **)&ori_wmma_C, &MAX_ORI_WMMA_C, c, false);
+    gemm_malloced = true;
+}
+
+static void fmap_insert(const char *key, const void *func, void *)
+{
+    fmap[key] = const_cast<void *>(func);
+}
+
+static bool g_initialised = false;
+
+// tkInit + registry + kinfo; returns a tk error code
+int tacker_runtime_init(int device, const char *kinfo_json_path)
+{
+    if (g_initialised) {
+        if (kinfo_json_path && *kinfo_json_path) read_json(kinfo_json_path);
+        return TK_SUCCESS;
+    }
+    int rc = tkInit(device);
+    if (rc) return rc;
+    rc = tk_register_kernels(fmap_insert, nullptr);
+    if (rc) return rc;
+    if (kinfo_json_path && *kinfo_json_path) read_json(kinfo_json_path);
+    else read_json_text(TK_KINFO_BUILTIN);
+    g_initialised = true;
+    return TK_SUCCESS;
+}
+
+bool tacker_runtime_ready() { return g_initialised; }

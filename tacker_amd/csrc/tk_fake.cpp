@@ -1,0 +1,202 @@
+// tk_fake.cpp -- recording stand-in for the device layer, for CPU-only tests of
+// the host runtime.  "Device" memory is host memory, every launch is appended to
+// a log (function key, grid, block, raw bytes of each argument) that tests read
+// back through tk_fake_* functions, and nothing is computed.  A launch can be
+// made to fail on demand to exercise the error conventions.
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "../../include/tacker_amd.h"
+
+namespace {
+struct FakeKernel {
+    std::string key;
+    std::vector<int> arg_sizes;   // bytes of each argument, in order
+};
+struct Launch {
+    std::string key;
+    tkDim3 grid, block;
+    std::vector<std::vector<unsigned char>> args;
+    void *stream;
+};
+std::vector<FakeKernel *> &kernels()
+{
+    static std::vector<FakeKernel *> k;
+    return k;
+}
+std::vector<Launch> g_launches;
+int g_fail_next_launch = 0;
+int g_cu_count = 256;
+float g_event_ms = 1.0f;
+std::map<std::string, std::vector<unsigned char>> g_symbols;
+
+const int P = 8, I = 4, F = 4;   // pointer, int, float
+std::vector<int> trailer(bool with_thread_base)
+{
+    std::vector<int> t(9, I);
+    if (with_thread_base) t.push_back(I);
+    return t;
+}
+std::vector<int> cat(std::vector<int> a, const std::vector<int> &b)
+{
+    a.insert(a.end(), b.begin(), b.end());
+    return a;
+}
+const std::vector<int> STENCIL = {F, F, P, P, I, I, I};
+const std::vector<int> LBM = {P, P};
+const std::vector<int> MRIQ = {I, I, P, P, P, P, P};
+const std::vector<int> CP = {I, F, P};
+const std::vector<int> TZ = {P, P, P, I, I, I};
+}  // namespace
+
+extern "C" {
+
+int tkInit(int) { return TK_SUCCESS; }
+const char *tkGetErrorString(int code)
+{
+    switch (code) {
+        case TK_SUCCESS: return "success";
+        case TK_ERROR_INVALID_VALUE: return "invalid value";
+        case TK_ERROR_NOT_FOUND: return "not found";
+        case TK_ERROR_UNSUPPORTED: return "unsupported shape";
+        case TK_ERROR_DEVICE: return "fake device error";
+        default: return "unknown error";
+    }
+}
+int tkGetCuCount(int *cu_count) { *cu_count = g_cu_count; return TK_SUCCESS; }
+int tkGetDeviceName(char *buf, size_t len) { snprintf(buf, len, "fake device"); return TK_SUCCESS; }
+int tkMalloc(void **ptr, size_t bytes) { *ptr = calloc(1, bytes ? bytes : 1); return *ptr ? TK_SUCCESS : TK_ERROR_DEVICE; }
+int tkFree(void *ptr) { free(ptr); return TK_SUCCESS; }
+int tkMemcpy(void *dst, const void *src, size_t bytes, int) { memmove(dst, src, bytes); return TK_SUCCESS; }
+int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int, tkStream_t) { memmove(dst, src, bytes); return TK_SUCCESS; }
+int tkMemset(void *ptr, int value, size_t bytes) { memset(ptr, value, bytes); return TK_SUCCESS; }
+int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset)
+{
+    if (strcmp(symbol, "ck") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail"))
+        return TK_ERROR_NOT_FOUND;
+    auto &buf = g_symbols[symbol];
+    if (buf.size() < offset + bytes) buf.resize(offset + bytes);
+    memcpy(buf.data() + offset, src, bytes);
+    return TK_SUCCESS;
+}
+int tkMemcpyFromSymbol(void *dst, const char *symbol, size_t bytes, size_t offset)
+{
+    auto it = g_symbols.find(symbol);
+    memset(dst, 0, bytes);
+    if (it == g_symbols.end()) return strcmp(symbol, "tk_spin_fail") ? TK_ERROR_NOT_FOUND : TK_SUCCESS;
+    if (offset + bytes <= it->second.size()) memcpy(dst, it->second.data() + offset, bytes);
+    return TK_SUCCESS;
+}
+int tkStreamCreate(tkStream_t *s) { *s = malloc(1); return TK_SUCCESS; }
+int tkStreamDestroy(tkStream_t s) { free(s); return TK_SUCCESS; }
+int tkStreamSynchronize(tkStream_t) { return TK_SUCCESS; }
+int tkDeviceSynchronize(void) { return TK_SUCCESS; }
+int tkEventCreate(tkEvent_t *e) { *e = malloc(1); return TK_SUCCESS; }
+int tkEventDestroy(tkEvent_t e) { free(e); return TK_SUCCESS; }
+int tkEventRecord(tkEvent_t, tkStream_t) { return TK_SUCCESS; }
+int tkEventSynchronize(tkEvent_t) { return TK_SUCCESS; }
+int tkEventElapsedTime(float *ms, tkEvent_t, tkEvent_t) { *ms = g_event_ms; return TK_SUCCESS; }
+
+int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, size_t, tkStream_t stream)
+{
+    if (g_fail_next_launch) {
+        g_fail_next_launch--;
+        return TK_ERROR_DEVICE;
+    }
+    const FakeKernel *k = nullptr;
+    for (auto *cand : kernels())
+        if (cand == func) k = cand;
+    if (!k) return TK_ERROR_INVALID_VALUE;
+    Launch l;
+    l.key = k->key;
+    l.grid = grid;
+    l.block = block;
+    l.stream = stream;
+    for (size_t i = 0; i < k->arg_sizes.size(); ++i) {
+        const unsigned char *p = (const unsigned char *)args[i];
+        l.args.emplace_back(p, p + k->arg_sizes[i]);
+    }
+    g_launches.push_back(std::move(l));
+    return TK_SUCCESS;
+}
+
+int tkModuleLoad(tkModule_t *m, const char *path)
+{
+    FILE *f = fopen(path, "rb");
+    if (!f) return TK_ERROR_DEVICE;
+    fclose(f);
+    *m = malloc(1);
+    return TK_SUCCESS;
+}
+int tkModuleUnload(tkModule_t m) { free(m); return TK_SUCCESS; }
+int tkModuleGetFunction(tkFunction_t *f, tkModule_t, const char *name)
+{
+    for (auto *k : kernels())
+        if (k->key == name) { *f = k; return TK_SUCCESS; }
+    return TK_ERROR_NOT_FOUND;
+}
+int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void **args, size_t shmem, tkStream_t s)
+{
+    return tkLaunchKernel(f, grid, block, args, shmem, s);
+}
+
+int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
+{
+    if (kernels().empty()) {
+        auto add = [](const char *key, std::vector<int> sizes) {
+            kernels().push_back(new FakeKernel{key, std::move(sizes)});
+        };
+        add("ori_stencil", STENCIL);
+        add("ori_lbm", LBM);
+        add("ori_ComputePhiMag", {P, P, P, I});
+        add("ori_mriq", MRIQ);
+        add("ori_cp", CP);
+        add("gptb_tzgemm", cat(TZ, trailer(true)));
+        add("gptb_stencil", cat(STENCIL, trailer(true)));
+        add("gptb_lbm", cat(LBM, trailer(true)));
+        add("gptb_mriq", cat(MRIQ, trailer(true)));
+        add("gptb_cp", cat(CP, trailer(true)));
+        add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
+        add("convert_fp32_to_fp16", {P, P, I});
+        add("tzgemm_stencil", cat(cat(STENCIL, trailer(false)), cat(TZ, trailer(false))));
+        add("tzgemm_lbm", cat(cat(LBM, trailer(false)), cat(TZ, trailer(false))));
+        add("tzgemm_mriq", cat(cat(MRIQ, trailer(false)), cat(TZ, trailer(false))));
+        add("tzgemm_cp", cat(cat(CP, trailer(false)), cat(TZ, trailer(false))));
+    }
+    for (auto *k : kernels()) insert(k->key.c_str(), k, ctx);
+    return TK_SUCCESS;
+}
+
+// ---- inspection interface for tests --------------------------------------
+TK_API int tk_fake_launch_count(void) { return (int)g_launches.size(); }
+TK_API void tk_fake_reset(void) { g_launches.clear(); g_fail_next_launch = 0; }
+TK_API void tk_fake_fail_next_launches(int n) { g_fail_next_launch = n; }
+TK_API void tk_fake_set_cu_count(int n) { g_cu_count = n; }
+TK_API void tk_fake_set_event_ms(float ms) { g_event_ms = ms; }
+TK_API const char *tk_fake_launch_key(int i) { return g_launches[i].key.c_str(); }
+TK_API int tk_fake_launch_nargs(int i) { return (int)g_launches[i].args.size(); }
+TK_API void tk_fake_launch_dims(int i, unsigned out[6])
+{
+    const Launch &l = g_launches[i];
+    out[0] = l.grid.x; out[1] = l.grid.y; out[2] = l.grid.z;
+    out[3] = l.block.x; out[4] = l.block.y; out[5] = l.block.z;
+}
+// copies argument a of launch i into out (up to cap bytes), returns its size
+TK_API int tk_fake_launch_arg(int i, int a, void *out, int cap)
+{
+    const auto &v = g_launches[i].args[a];
+    memcpy(out, v.data(), (size_t)cap < v.size() ? (size_t)cap : v.size());
+    return (int)v.size();
+}
+TK_API int tk_fake_symbol(const char *name, void *out, int cap)
+{
+    auto it = g_symbols.find(name);
+    if (it == g_symbols.end()) return -1;
+    memcpy(out, it->second.data(), (size_t)cap < it->second.size() ? (size_t)cap : it->second.size());
+    return (int)it->second.size();
+}
+
+}  // extern "C"

@@ -1,0 +1,160 @@
+// tk_hip.cpp -- the HIP implementation of the thin device layer (tk*).
+// One function per CUDA runtime / driver call the reference's host code makes;
+// HIP error codes are folded into TK_ERROR_DEVICE with the HIP text kept for
+// tkGetErrorString.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <string>
+
+#include "../../include/tacker_amd.h"
+
+extern "C" int tk_device_symbol(const char *name, const void **symbol, size_t *bytes);
+
+namespace {
+thread_local std::string g_last_hip_error;
+
+int fold(hipError_t e, const char *what)
+{
+    if (e == hipSuccess) return TK_SUCCESS;
+    g_last_hip_error = std::string(what) + ": " + hipGetErrorString(e);
+    (void)hipGetLastError();   // clear the sticky error
+    return TK_ERROR_DEVICE;
+}
+hipMemcpyKind kind_of(int kind)
+{
+    switch (kind) {
+        case TK_MEMCPY_H2D: return hipMemcpyHostToDevice;
+        case TK_MEMCPY_D2H: return hipMemcpyDeviceToHost;
+        case TK_MEMCPY_D2D: return hipMemcpyDeviceToDevice;
+        default: return hipMemcpyDefault;
+    }
+}
+}  // namespace
+
+#define FOLD(call) fold((call), #call)
+
+extern "C" {
+
+int tkInit(int device)
+{
+    int count = 0;
+    int rc = FOLD(hipGetDeviceCount(&count));
+    if (rc) return rc;
+    if (device < 0 || device >= count) {
+        g_last_hip_error = "tkInit: no such device";
+        return TK_ERROR_INVALID_VALUE;
+    }
+    rc = FOLD(hipSetDevice(device));
+    if (rc) return rc;
+    return FOLD(hipFree(0));   // force context creation, as initCUDA does
+}
+
+const char *tkGetErrorString(int code)
+{
+    switch (code) {
+        case TK_SUCCESS: return "success";
+        case TK_ERROR_INVALID_VALUE: return g_last_hip_error.empty() ? "invalid value" : g_last_hip_error.c_str();
+        case TK_ERROR_NOT_FOUND: return "not found";
+        case TK_ERROR_UNSUPPORTED: return "unsupported shape";
+        case TK_ERROR_DEVICE: return g_last_hip_error.c_str();
+        default: return "unknown error";
+    }
+}
+
+int tkGetCuCount(int *cu_count)
+{
+    int dev = 0;
+    int rc = FOLD(hipGetDevice(&dev));
+    if (rc) return rc;
+    return FOLD(hipDeviceGetAttribute(cu_count, hipDeviceAttributeMultiprocessorCount, dev));
+}
+
+int tkGetDeviceName(char *buf, size_t len)
+{
+    int dev = 0;
+    int rc = FOLD(hipGetDevice(&dev));
+    if (rc) return rc;
+    hipDeviceProp_t prop;
+    rc = FOLD(hipGetDeviceProperties(&prop, dev));
+    if (rc) return rc;
+    snprintf(buf, len, "%s (%s)", prop.name, prop.gcnArchName);
+    return TK_SUCCESS;
+}
+
+int tkMalloc(void **ptr, size_t bytes) { return FOLD(hipMalloc(ptr, bytes)); }
+int tkFree(void *ptr) { return FOLD(hipFree(ptr)); }
+int tkMemcpy(void *dst, const void *src, size_t bytes, int kind)
+{
+    return FOLD(hipMemcpy(dst, src, bytes, kind_of(kind)));
+}
+int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int kind, tkStream_t s)
+{
+    return FOLD(hipMemcpyAsync(dst, src, bytes, kind_of(kind), (hipStream_t)s));
+}
+int tkMemset(void *ptr, int value, size_t bytes) { return FOLD(hipMemset(ptr, value, bytes)); }
+
+int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset)
+{
+    const void *sym = nullptr;
+    size_t cap = 0;
+    const int rc = tk_device_symbol(symbol, &sym, &cap);
+    if (rc) return rc;
+    if (offset + bytes > cap) {
+        g_last_hip_error = "tkMemcpyToSymbol: range exceeds the symbol";
+        return TK_ERROR_INVALID_VALUE;
+    }
+    return FOLD(hipMemcpyToSymbol(sym, src, bytes, offset, hipMemcpyHostToDevice));
+}
+
+int tkMemcpyFromSymbol(void *dst, const char *symbol, size_t bytes, size_t offset)
+{
+    const void *sym = nullptr;
+    size_t cap = 0;
+    const int rc = tk_device_symbol(symbol, &sym, &cap);
+    if (rc) return rc;
+    if (offset + bytes > cap) {
+        g_last_hip_error = "tkMemcpyFromSymbol: range exceeds the symbol";
+        return TK_ERROR_INVALID_VALUE;
+    }
+    return FOLD(hipMemcpyFromSymbol(dst, sym, bytes, offset, hipMemcpyDeviceToHost));
+}
+
+int tkStreamCreate(tkStream_t *s) { return FOLD(hipStreamCreate((hipStream_t *)s)); }
+int tkStreamDestroy(tkStream_t s) { return FOLD(hipStreamDestroy((hipStream_t)s)); }
+int tkStreamSynchronize(tkStream_t s) { return FOLD(hipStreamSynchronize((hipStream_t)s)); }
+int tkDeviceSynchronize(void) { return FOLD(hipDeviceSynchronize()); }
+int tkEventCreate(tkEvent_t *e) { return FOLD(hipEventCreate((hipEvent_t *)e)); }
+int tkEventDestroy(tkEvent_t e) { return FOLD(hipEventDestroy((hipEvent_t)e)); }
+int tkEventRecord(tkEvent_t e, tkStream_t s) { return FOLD(hipEventRecord((hipEvent_t)e, (hipStream_t)s)); }
+int tkEventSynchronize(tkEvent_t e) { return FOLD(hipEventSynchronize((hipEvent_t)e)); }
+int tkEventElapsedTime(float *ms, tkEvent_t start, tkEvent_t stop)
+{
+    return FOLD(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+}
+
+int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, size_t shmem,
+                   tkStream_t stream)
+{
+    if (!func) {
+        g_last_hip_error = "tkLaunchKernel: null function";
+        return TK_ERROR_INVALID_VALUE;
+    }
+    return FOLD(hipLaunchKernel(func, dim3(grid.x, grid.y, grid.z), dim3(block.x, block.y, block.z),
+                                args, shmem, (hipStream_t)stream));
+}
+
+int tkModuleLoad(tkModule_t *m, const char *path) { return FOLD(hipModuleLoad((hipModule_t *)m, path)); }
+int tkModuleUnload(tkModule_t m) { return FOLD(hipModuleUnload((hipModule_t)m)); }
+int tkModuleGetFunction(tkFunction_t *f, tkModule_t m, const char *name)
+{
+    return FOLD(hipModuleGetFunction((hipFunction_t *)f, (hipModule_t)m, name));
+}
+int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void **args, size_t shmem,
+                         tkStream_t stream)
+{
+    return FOLD(hipModuleLaunchKernel((hipFunction_t)f, grid.x, grid.y, grid.z, block.x, block.y,
+                                      block.z, (unsigned)shmem, (hipStream_t)stream, args, nullptr));
+}
+
+}  // extern "C"

@@ -1,0 +1,115 @@
+"""Emit the text of fused ("mix") HIP kernels.
+
+Counterpart of ``fusion/code/gen_mix.py`` of the reference
+(``generate_mixed_kernel`` :16-76): one ``__global__`` whose parameter list is
+the concatenation of both kernels' GPTB parameter lists, and whose body sends
+each thread to one kernel's device-side role.  The reference splits by
+``threadIdx.x`` thresholds and keeps each role's barriers apart with PTX named
+barriers (``bar.sync id, n``).  gfx950 has one hardware barrier per workgroup,
+so two forms are emitted:
+
+* ``wg``   -- workgroup split: role = f(blockIdx); a group of ``a + b``
+  consecutive XCD-slots holds ``a`` workgroups of the first kernel and ``b`` of
+  the second (``tk::wg_split``).  Each role owns whole workgroups, so a role
+  that needs a barrier uses the hardware one.
+* ``wave`` -- wave split: every workgroup holds both roles, threads
+  ``[0, t0)`` run the first kernel and ``[t0, t0 + t1)`` the second, the way the
+  reference does; a role that needs a barrier uses an LDS arrival counter
+  private to its waves (``tk::RoleSpinSync``).
+"""
+from kernel_code import ROLES, signature
+
+
+def _params_text(sig_a, sig_b):
+    return ",\n    ".join(f"{t} {n}" for t, n in sig_a + sig_b)
+
+
+def _void_unused(sig, body):
+    """(void) casts for parameters the dispatcher body does not read."""
+    import re
+    return "".join(f"    (void){n};\n" for _, n in sig if not re.search(rf"\b{n}\b", body))
+
+
+def mix_kernel_name(be, variant):
+    return f"{be}_tzgemm_mix_{variant}"
+
+
+def generate_wg_split(be, tz_wgs, be_wgs, threads=256):
+    """Workgroup-split fused kernel of ``be`` with tzgemm; tz_wgs : be_wgs per group."""
+    variant = f"wg_{tz_wgs}_{be_wgs}"
+    p_be, sig_be = signature(be, 0)
+    p_tz, sig_tz = signature("tzgemm", 1)
+    tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="sp.role_block", blocks="sp.role_blocks",
+                                             tid="(int)threadIdx.x")
+    be_call = ROLES[be]["call"].format(p=p_be, block="sp.role_block", blocks="sp.role_blocks",
+                                       tid="(int)threadIdx.x", threads=threads)
+    name = mix_kernel_name(be, variant)
+    text = f"""// {be}-tzgemm  workgroup split  {tz_wgs} tzgemm : {be_wgs} {be} workgroups per group
+extern "C" __global__ __launch_bounds__({threads}) void {name}(
+    {_params_text(sig_be, sig_tz)})
+{{
+{_void_unused(sig_be + sig_tz, tz_call + be_call)}    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
+    const tk::WgSplit sp = tk::wg_split((int)blockIdx.x, (int)gridDim.x, {tz_wgs}, {be_wgs});
+    if (sp.role == 0) {{
+        tk::WorkgroupSync sync;
+        {tz_call}
+    }} else {{
+        {be_call}
+    }}
+}}
+"""
+    meta = {"variant": variant, "symbol": name, "blocksize": threads,
+            "group": tz_wgs + be_wgs, "tz_share": tz_wgs, "be_share": be_wgs, "kind": "wg"}
+    return text, meta
+
+
+def generate_wave_split(be, be_threads, tz_first=True):
+    """Wave-split fused kernel: 256 tzgemm threads + be_threads of ``be`` per workgroup."""
+    variant = f"wave_{be_threads}"
+    tz_threads = 256
+    total = tz_threads + be_threads
+    p_be, sig_be = signature(be, 0)
+    p_tz, sig_tz = signature("tzgemm", 1)
+    if tz_first:
+        tz_lo, be_lo = 0, tz_threads
+    else:
+        be_lo, tz_lo = 0, be_threads
+    tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="(int)blockIdx.x",
+                                             blocks=f"{p_tz}ptb_iter_block_step",
+                                             tid=f"(int)threadIdx.x - {tz_lo}")
+    be_call = ROLES[be]["call"].format(p=p_be, block="(int)blockIdx.x",
+                                       blocks=f"{p_be}ptb_iter_block_step",
+                                       tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads)
+    tz_cond = (f"threadIdx.x < {tz_threads}" if tz_first else f"threadIdx.x >= {be_threads}")
+    name = mix_kernel_name(be, variant)
+    unused = _void_unused(sig_be + sig_tz, tz_call + be_call)
+    text = f"""// {be}-tzgemm  wave split  {tz_threads} tzgemm threads + {be_threads} {be} threads per workgroup
+extern "C" __global__ __launch_bounds__({total}) void {name}(
+    {_params_text(sig_be, sig_tz)})
+{{
+{unused}    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
+    __shared__ unsigned tz_arrivals;
+    if (threadIdx.x == 0) tz_arrivals = 0u;
+    __syncthreads();   // the only workgroup-wide barrier: before the roles part ways
+    if ({tz_cond}) {{
+        tk::RoleSpinSync sync(&tz_arrivals, {tz_threads // 64}, &tk_spin_fail);
+        {tz_call}
+    }} else {{
+        {be_call}
+    }}
+}}
+"""
+    meta = {"variant": variant, "symbol": name, "blocksize": total, "group": 1,
+            "tz_share": 1, "be_share": 1, "kind": "wave"}
+    return text, meta
+
+
+def generate_pair(be, candidates):
+    """All fused kernels of one (be, tzgemm) pair: yields (text, meta)."""
+    for cand in candidates:
+        if cand[0] == "wg":
+            yield generate_wg_split(be, cand[1], cand[2])
+        elif cand[0] == "wave":
+            yield generate_wave_split(be, cand[1])
+        else:
+            raise ValueError(cand)

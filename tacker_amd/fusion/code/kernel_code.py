@@ -1,0 +1,73 @@
+"""Role descriptions the generator stitches together.
+
+Each entry plays the part of one ``<kernel>_code.py`` of the reference
+(fusion/code/cp_code.py, lbm_code.py, mriq_code.py, stencil_code.py and the
+truncated tzgemm_code.py): the kernel's parameter list in reference order and
+how to call its device-side role.  The role bodies themselves live in
+``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
+the reference's generated ``__global__`` functions call ``<a>_<b>_<k><i>()``
+device functions.
+
+``params``   -- (C type, name) in the order of the reference kernel's signature,
+               without the 10-int GPTB trailer.
+``call``     -- format string of the role call; ``{p}`` is the parameter prefix,
+               ``{block}``, ``{blocks}`` the role-local persistent-workgroup id
+               and count, ``{tid}`` the role-local thread id, ``{threads}`` the
+               role's thread count, ``{extra}`` role-specific trailing arguments.
+"""
+
+GPTB_DIMS = ["grid_dimension_x", "grid_dimension_y", "grid_dimension_z",
+             "block_dimension_x", "block_dimension_y", "block_dimension_z"]
+GPTB_RANGE = ["ptb_start_block_pos", "ptb_iter_block_step", "ptb_end_block_pos"]
+
+ROLES = {
+    "tzgemm": {
+        "params": [("_Float16*", "A"), ("_Float16*", "B"), ("float*", "C"),
+                   ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K")],
+        "needs_sync": True,
+        "lds_bytes": "TZ_LDS_BYTES",
+        "call": ("tk::tzgemm_role({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, "
+                 "{block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "tz_lds, sync);"),
+    },
+    "stencil": {
+        "params": [("float", "c0"), ("float", "c1"), ("float*", "A0"), ("float*", "Anext"),
+                   ("int", "nx"), ("int", "ny"), ("int", "nz")],
+        "needs_sync": False,
+        "call": ("tk::stencil_role({p}c0, {p}c1, {p}A0, {p}Anext, {p}nx, {p}ny, {p}nz, "
+                 "{p}grid_dimension_x, {p}grid_dimension_y, {block}, {blocks}, "
+                 "{p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+    "lbm": {
+        "params": [("float*", "srcGrid"), ("float*", "dstGrid")],
+        "needs_sync": False,
+        "call": ("tk::lbm_role({p}srcGrid, {p}dstGrid, {p}grid_dimension_x, {p}grid_dimension_y, "
+                 "{p}block_dimension_x, {block}, {blocks}, {p}ptb_start_block_pos, "
+                 "{p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+    "mriq": {
+        "params": [("int", "numK"), ("int", "kGlobalIndex"), ("float*", "x"), ("float*", "y"),
+                   ("float*", "z"), ("float*", "Qr"), ("float*", "Qi")],
+        "needs_sync": False,
+        "call": ("tk::mriq_role({p}numK, {p}x, {p}y, {p}z, {p}Qr, {p}Qi, {p}grid_dimension_x, "
+                 "{block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "{threads});"),
+    },
+    "cp": {
+        "params": [("int", "numatoms"), ("float", "gridspacing"), ("float*", "energygrid")],
+        "needs_sync": False,
+        "call": ("tk::cp_role({p}numatoms, {p}gridspacing, {p}energygrid, {p}grid_dimension_x, "
+                 "{p}grid_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, "
+                 "{p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+}
+
+
+def signature(name, index):
+    """Parameter list of role ``name`` as the index-th kernel of a fused launch:
+    ori params, 6 GPTB dims, start/step/end -- the concatenation MixKernel builds
+    (src/MixKernel.h:55-73 of the reference); no thread_base (it is baked in)."""
+    prefix = f"{name}{index}_"
+    out = [(t, prefix + n) for t, n in ROLES[name]["params"]]
+    out += [("int", prefix + n) for n in GPTB_DIMS + GPTB_RANGE]
+    return prefix, out

@@ -1,0 +1,323 @@
+"""GPU parity: every kernel of the path, in ori, GPTB and fused form, against the
+CPU oracle on the same seeded inputs, through the C-ABI.
+
+Bars: bit-exact for stencil, lbm, cp (ordered fp32, contraction off on both
+sides), for all [start,end) bookkeeping, and for fused-vs-unfused device output;
+tzgemm |d| <= 5e-3 + 1e-5|ref| and rel-Frobenius <= 1e-5 against the fp64 oracle;
+mri-q |d| <= 1e-3 + 1e-4|ref| against the fp64 oracle.
+"""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import tacker_amd as ta
+from gpu_util import (C0, C1, dev, gemm_inputs, gemm_tolerance_ok, host, lbm_inputs, mriq_inputs, setup,
+                      stencil_inputs)
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    setup()
+
+
+# ------------------------------------------------------------------ tzgemm
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 128), (1024, 1024, 1024), (384, 128, 640)])
+def test_gptb_tzgemm_matches_fp64_oracle(M, N, K):
+    A, B = gemm_inputs(M, N, K)
+    Cd = torch.full((M, N), -7.0, device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), Cd)
+    got = host(Cd)
+    truth = oracle.tzgemm(A, B, f64=True)
+    ok, fro, dmax = gemm_tolerance_ok(got, truth, K)
+    assert ok and fro <= 1e-5, (fro, dmax)
+
+
+def test_tzgemm_closed_forms():
+    K = 256
+    A = np.eye(128, K, dtype=np.float16)
+    rng = np.random.default_rng(3)
+    B = rng.uniform(-1, 1, (256, K)).astype(np.float16)
+    Cd = torch.zeros((128, 256), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), Cd)
+    assert np.array_equal(host(Cd), B.astype(np.float32).T * np.float32(1.1))
+    ones = np.ones((128, K), np.float16)
+    Cd2 = torch.zeros((128, 128), device="cuda:0")
+    ta.gptb_tzgemm(dev(ones), dev(ones), Cd2)
+    assert np.all(host(Cd2) == np.float32(K) * np.float32(1.1))
+
+
+@pytest.mark.parametrize("start,end,grid", [(0, 5, 0), (3, 9, 8), (7, 8, 16), (0, 0, 0), (0, 24, 3)])
+def test_tzgemm_tile_range_writes_only_its_tiles(start, end, grid):
+    M, N, K = 256, 384, 128
+    A, B = gemm_inputs(M, N, K, seed=5)
+    full = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), full)
+    full = host(full)
+    Cd = torch.full((M, N), -7.0, device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), Cd, tile_start=start, tile_end=end, launch_grid=grid)
+    got = host(Cd)
+    want = oracle.tzgemm(A, B, C_init=np.full((M, N), -7.0, np.float32), start=start, end=end)
+    mask = want != -7.0
+    assert np.array_equal(got[~mask], want[~mask])       # untouched outside the range
+    assert np.array_equal(got[mask], full[mask])         # same values as the full launch
+
+
+# ------------------------------------------------------------------ stencil
+@pytest.mark.parametrize("shape", [(8, 8, 64), (6, 10, 70), (5, 7, 130), (4, 9, 33), (64, 64, 128)])
+def test_stencil_ori_and_gptb_bit_exact(shape):
+    A0 = stencil_inputs(*shape)
+    want = oracle.stencil(C0, C1, A0, A0)
+    a0 = dev(A0)
+    out = a0.clone()
+    ta.ori_stencil(C0, C1, a0, out)
+    assert np.array_equal(host(out), want)
+    out2 = a0.clone()
+    ta.gptb_stencil(C0, C1, a0, out2)
+    assert np.array_equal(host(out2), want)
+    out3 = a0.clone()
+    ta.gptb_stencil(C0, C1, a0, out3, launch_grid=3, launch_block=128)
+    assert np.array_equal(host(out3), want)
+
+
+def test_stencil_gptb_ranges_and_wrap():
+    A0 = stencil_inputs(5, 12, 130)
+    nblk = ta.stencil_blocks(130, 12)
+    a0 = dev(A0)
+    acc = torch.full_like(a0, -3.0)
+    want = np.full_like(A0, -3.0)
+    for s, e in [(0, 2), (2, 7), (7, nblk)]:
+        ta.gptb_stencil(C0, C1, a0, acc, start=s, end=e, launch_grid=2, launch_block=64)
+        want = oracle.stencil_gptb(C0, C1, A0, want, s, e)
+        assert np.array_equal(host(acc), want)
+    ta.gptb_stencil(C0, C1, a0, acc, start=nblk, end=2 * nblk)      # wraps: same cells again
+    assert np.array_equal(host(acc), want)
+    ta.gptb_stencil(C0, C1, a0, acc, start=4, end=4)                # empty range
+    assert np.array_equal(host(acc), want)
+
+
+def test_stencil_iterations_ping_pong():
+    A0 = stencil_inputs(6, 16, 128)
+    a, b = dev(A0), dev(A0)
+    ha, hb = A0.copy(), A0.copy()
+    for _ in range(5):
+        ta.gptb_stencil(C0, C1, a, b)
+        hb = oracle.stencil(C0, C1, ha, hb)
+        a, b = b, a
+        ha, hb = hb, ha
+    assert np.array_equal(host(a), ha)
+
+
+# ------------------------------------------------------------------ lbm
+@pytest.mark.parametrize("dims", [(4, 4, 4), (12, 5, 6), (64, 3, 5), (120, 6, 4), (128, 4, 4), (200, 3, 3)])
+def test_lbm_ori_and_gptb_bit_exact(dims):
+    sx, sy, sz = dims
+    src = lbm_inputs(sx, sy, sz, obstacle_p=0.2, accel_p=0.1)
+    dst0 = np.full_like(src, -5.0)
+    want = oracle.lbm(src, dst0, sx, sy, sz)
+    s = dev(src)
+    d = dev(dst0)
+    ta.ori_lbm(s, d, sx, sy, sz)
+    assert np.array_equal(host(d).view(np.uint32), want.view(np.uint32))
+    d2 = dev(dst0)
+    ta.gptb_lbm(s, d2, sx, sy, sz)
+    assert np.array_equal(host(d2).view(np.uint32), want.view(np.uint32))
+    d3 = dev(dst0)
+    ta.gptb_lbm(s, d3, sx, sy, sz, launch_grid=2, launch_block=64)
+    assert np.array_equal(host(d3).view(np.uint32), want.view(np.uint32))
+
+
+def test_lbm_ranges():
+    sx, sy, sz = 16, 4, 3
+    src = lbm_inputs(sx, sy, sz)
+    s = dev(src)
+    d = torch.zeros_like(s)
+    want = np.zeros_like(src)
+    for a, b in [(0, 5), (5, 6), (6, 12)]:
+        ta.gptb_lbm(s, d, sx, sy, sz, start=a, end=b)
+        want = oracle.lbm(src, want, sx, sy, sz, a, b)
+        assert np.array_equal(host(d), want)
+
+
+# ------------------------------------------------------------------ mri-q
+def mriq_close(got, truth):
+    return np.all(np.abs(got.astype(np.float64) - truth) <= 1e-3 + 1e-4 * np.abs(truth))
+
+
+@pytest.mark.parametrize("numK,numX", [(64, 256), (1024, 1024), (2048, 512), (3, 256)])
+def test_mriq_matches_fp64_oracle(numK, numX):
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX)
+    pm = torch.zeros(numK, device="cuda:0")
+    ta.mriq_phimag(dev(phiR), dev(phiI), pm)
+    phimag = host(pm)
+    assert np.array_equal(phimag, oracle.mriq_phimag(phiR, phiI))
+    kv = np.concatenate([k, phimag[:, None]], 1).astype(np.float32)
+    ta.mriq_set_kvalues(kv)
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    q0 = np.full(numX, 0.5, np.float32)
+    tr, ti = oracle.mriq(kv, xyz[0], xyz[1], xyz[2], q0, q0, f64=True)
+    for form in ("ori", "gptb"):
+        Qr, Qi = dev(q0), dev(q0)
+        if form == "ori":
+            ta.ori_mriq(numK, x, y, z, Qr, Qi)
+        else:
+            ta.gptb_mriq(numK, x, y, z, Qr, Qi, launch_grid=3)
+        assert mriq_close(host(Qr), tr.astype(np.float64)) and mriq_close(host(Qi), ti.astype(np.float64))
+
+
+def test_mriq_closed_forms_and_ranges():
+    numK, numX = 128, 1024
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX, seed=2)
+    kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+    ta.mriq_set_kvalues(kv)
+    zero = torch.zeros(numX, device="cuda:0")
+    Qr, Qi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    ta.gptb_mriq(numK, zero, zero, zero, Qr, Qi)
+    np.testing.assert_allclose(host(Qr), kv[:, 3].astype(np.float64).sum(), rtol=1e-5)
+    assert np.all(host(Qi) == 0)
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    full_r = torch.zeros(numX, device="cuda:0")
+    full_i = torch.zeros(numX, device="cuda:0")
+    ta.gptb_mriq(numK, x, y, z, full_r, full_i)
+    pr, pi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    ta.gptb_mriq(numK, x, y, z, pr, pi, start=1, end=3)
+    pr, fr = host(pr), host(full_r)
+    assert np.array_equal(pr[256:768], fr[256:768]) and np.all(pr[:256] == 0) and np.all(pr[768:] == 0)
+
+
+# ------------------------------------------------------------------ cp
+def cp_atoms():
+    atoms = ta.cp_initatoms(4000)
+    assert np.array_equal(atoms, oracle.cp_initatoms(4000))
+    return atoms[1:65]
+
+
+@pytest.mark.parametrize("shape", [(8, 128), (24, 384), (64, 1024)])
+def test_cp_bit_exact(shape):
+    atoms = cp_atoms()
+    ta.cp_set_atoms(atoms, 0.0)
+    info = oracle.cp_atoms_to_const(atoms, 0.0)
+    rng = np.random.default_rng(4)
+    g0 = rng.uniform(-1, 1, shape).astype(np.float32)
+    want = oracle.cp(info, g0)
+    g = dev(g0)
+    ta.ori_cp(64, 0.1, g)
+    assert np.array_equal(host(g).view(np.uint32), want.view(np.uint32))
+    g2 = dev(g0)
+    ta.gptb_cp(64, 0.1, g2, launch_grid=5)
+    assert np.array_equal(host(g2).view(np.uint32), want.view(np.uint32))
+    g3 = dev(g0)
+    nblk = (shape[1] // 128) * (shape[0] // 8)
+    want3 = g0
+    for s, e in [(0, 1), (1, nblk)]:
+        ta.gptb_cp(64, 0.1, g3, start=s, end=e, launch_block=256)
+        want3 = oracle.cp(info, want3, start=s, end=e)
+    assert np.array_equal(host(g3).view(np.uint32), want3.view(np.uint32))
+    assert np.array_equal(want3, want)
+
+
+def test_cp_fewer_atoms():
+    atoms = cp_atoms()[:7]
+    ta.cp_set_atoms(atoms, 0.5)
+    info = oracle.cp_atoms_to_const(atoms, 0.5)
+    g = torch.zeros((16, 256), device="cuda:0")
+    ta.gptb_cp(7, 0.1, g)
+    assert np.array_equal(host(g), oracle.cp(info, np.zeros((16, 256), np.float32)))
+
+
+# ------------------------------------------------------------------ fused
+VARIANTS = [None, "wg_1_1", "wg_2_1", "wg_1_2"]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_mix_tzgemm_stencil(variant):
+    M, N, K = 256, 384, 256
+    A, B = gemm_inputs(M, N, K, seed=7)
+    A0 = stencil_inputs(6, 20, 200)
+    a0 = dev(A0)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), solo_c)
+    solo_s = a0.clone()
+    ta.gptb_stencil(C0, C1, a0, solo_s)
+    mix_c = torch.full((M, N), -7.0, device="cuda:0")
+    mix_s = a0.clone()
+    ta.mix_tzgemm_stencil(C0, C1, a0, mix_s, dev(A), dev(B), mix_c, variant=variant)
+    assert np.array_equal(host(mix_c), host(solo_c))             # fused == unfused, bit-exact
+    assert np.array_equal(host(mix_s), host(solo_s))
+    assert np.array_equal(host(mix_s), oracle.stencil(C0, C1, A0, A0))
+    ok, fro, _ = gemm_tolerance_ok(host(mix_c), oracle.tzgemm(A, B, f64=True), K)
+    assert ok and fro <= 1e-5
+
+
+def test_mix_tzgemm_stencil_partial_ranges():
+    M, N, K = 256, 256, 128
+    A, B = gemm_inputs(M, N, K, seed=8)
+    A0 = stencil_inputs(5, 12, 130)
+    a0 = dev(A0)
+    mix_c = torch.full((M, N), -7.0, device="cuda:0")
+    mix_s = torch.full_like(a0, -3.0)
+    ta.mix_tzgemm_stencil(C0, C1, a0, mix_s, dev(A), dev(B), mix_c, be_start=2, be_end=7, tile_start=3, tile_end=11)
+    assert np.array_equal(host(mix_s), oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), 2, 7))
+    want_c = oracle.tzgemm(A, B, C_init=np.full((M, N), -7.0, np.float32), start=3, end=11)
+    got_c = host(mix_c)
+    assert np.array_equal(got_c == -7.0, want_c == -7.0)
+    ta.mix_tzgemm_stencil(C0, C1, a0, mix_s, dev(A), dev(B), mix_c, be_start=0, be_end=0, tile_start=0, tile_end=0)
+    assert np.array_equal(host(mix_c), got_c)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_mix_tzgemm_lbm(variant):
+    M, N, K = 256, 256, 256
+    A, B = gemm_inputs(M, N, K, seed=9)
+    sx, sy, sz = 120, 6, 5
+    src = lbm_inputs(sx, sy, sz)
+    s = dev(src)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), solo_c)
+    mix_c = torch.zeros((M, N), device="cuda:0")
+    d = torch.zeros_like(s)
+    ta.mix_tzgemm_lbm(s, d, sx, sy, sz, dev(A), dev(B), mix_c, variant=variant)
+    assert np.array_equal(host(mix_c), host(solo_c))
+    want = oracle.lbm(src, np.zeros_like(src), sx, sy, sz)
+    assert np.array_equal(host(d).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_mix_tzgemm_mriq(variant):
+    M, N, K = 256, 256, 256
+    A, B = gemm_inputs(M, N, K, seed=10)
+    numK, numX = 256, 2048
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX)
+    kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+    ta.mriq_set_kvalues(kv)
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    solo_r, solo_i = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    ta.gptb_mriq(numK, x, y, z, solo_r, solo_i)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), solo_c)
+    mix_c = torch.zeros((M, N), device="cuda:0")
+    Qr, Qi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    ta.mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, dev(A), dev(B), mix_c, variant=variant)
+    assert np.array_equal(host(mix_c), host(solo_c))
+    assert np.array_equal(host(Qr), host(solo_r)) and np.array_equal(host(Qi), host(solo_i))
+    zq = np.zeros(numX, np.float32)
+    tr, ti = oracle.mriq(kv, xyz[0], xyz[1], xyz[2], zq, zq, f64=True)
+    assert mriq_close(host(Qr), tr.astype(np.float64)) and mriq_close(host(Qi), ti.astype(np.float64))
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_mix_tzgemm_cp(variant):
+    M, N, K = 256, 256, 256
+    A, B = gemm_inputs(M, N, K, seed=11)
+    atoms = cp_atoms()
+    ta.cp_set_atoms(atoms, 0.0)
+    info = oracle.cp_atoms_to_const(atoms, 0.0)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), solo_c)
+    mix_c = torch.zeros((M, N), device="cuda:0")
+    g = torch.zeros((32, 512), device="cuda:0")
+    ta.mix_tzgemm_cp(64, 0.1, g, dev(A), dev(B), mix_c, variant=variant)
+    assert np.array_equal(host(mix_c), host(solo_c))
+    assert np.array_equal(host(g).view(np.uint32), oracle.cp(info, np.zeros((32, 512), np.float32)).view(np.uint32))
