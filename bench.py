@@ -1,0 +1,183 @@
+#!/usr/bin/env python3
+"""Benchmark of the hot path on one MI355X: the fused tzgemm + stencil launch
+against serial launches of the same two kernels.
+
+Workload (BASELINE config 2): tzgemm fp16 2048x2048x2048 (uniform[-1,1], fp32
+accumulate, alpha 1.1) + Parboil 7-point Jacobi stencil on an fp32 512x512x64 grid
+(uniform[0,1], c0=1/6, c1=1/36), 100 iterations with pointer swap.  One "step" is
+the whole 100-iteration job: serial = 100 x (1 GEMM launch + 1 sweep launch) on one
+stream, fused = 100 fused launches (GEMM tiles [0,1024) + stencil blocks [0,1024)).
+
+Prints ONE JSON line: value = serial time / fused time, with the roofline of the
+fused kernel and the CPU baseline (the oracle restatement on the host cores).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK = 8.0e12          # B/s, MI355X HBM3E
+MFMA_F16_PEAK = 2.5e15     # flop/s, dense fp16 MFMA
+
+GEMM_MNK = (2048, 2048, 2048)
+STENCIL_DIMS = (64, 512, 512)      # nz, ny, nx
+ITERATIONS = 100
+
+
+def trimmed_mean(xs):
+    xs = sorted(xs)
+    if len(xs) >= 5:
+        k = len(xs) // 4
+        xs = xs[k:len(xs) - k]
+    return sum(xs) / len(xs)
+
+
+def cpu_baseline(A, B, A0, c0, c1):
+    """The oracle (CPU port of the reference kernels) on the host cores: 1 GEMM and
+    10 sweeps timed, scaled to the job's 100 + 100."""
+    import numpy as np
+    import oracle
+    t0 = time.perf_counter()
+    oracle.tzgemm(A, B)
+    t_gemm = time.perf_counter() - t0
+    a, b = A0.copy(), A0.copy()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        b = oracle.stencil(c0, c1, a, b)
+        a, b = b, a
+    t_sweep = (time.perf_counter() - t0) / 10
+    ms = (t_gemm + t_sweep) * ITERATIONS * 1e3
+    return {"value": round(ms, 1), "unit": "ms_per_step", "cores": oracle.num_threads(), "kind": "port",
+            "sample": "oracle/tacker_oracle.c with OpenMP: 1 tzgemm 2048^3 (%.2f s) + 10 stencil sweeps "
+                      "512x512x64 (%.4f s each), scaled to 100 + 100" % (t_gemm, t_sweep)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--variant", default=None, help="fused kernel variant (default: kinfo)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+    import tacker_amd as ta
+
+    ta.init(0)
+    M, N, K = GEMM_MNK
+    nz, ny, nx = STENCIL_DIMS
+    rng = np.random.default_rng(1337)
+    A = rng.uniform(-1, 1, (M, K)).astype(np.float16)
+    B = rng.uniform(-1, 1, (N, K)).astype(np.float16)
+    A0 = rng.uniform(0, 1, (nz, ny, nx)).astype(np.float32)
+    c0, c1 = float(np.float32(1.0 / 6.0)), float(np.float32(1.0 / 6.0 / 6.0))
+
+    dA, dB = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+    dC = torch.zeros((M, N), device="cuda:0")
+    g0 = torch.from_numpy(A0).cuda()
+    g1 = g0.clone()
+    stream = torch.cuda.current_stream()
+
+    tiles = ta.tzgemm_grid_dim(M, N, K)[3]
+    blocks = ta.stencil_blocks(nx, ny)
+    st_ori = ta.ori_stencil_create(c0, c1, g0, g1)
+    st = ta.gptb_create(st_ori, 0, 0, 0, blocks)
+    tz_ori = ta.ori_tzgemm_create(dA, dB, dC)
+    tz = ta.gptb_create(tz_ori, 0, 0, 0, tiles)
+    mix = ta.mix_create(st, tz, 0, blocks, 0, tiles, variant=args.variant)
+
+    def job(kind):
+        for _ in range(ITERATIONS):
+            if kind == "serial":
+                tz.execute(stream)
+                st.execute(stream)
+            elif kind == "fused":
+                mix.execute(stream)
+            elif kind == "gemm":
+                tz.execute(stream)
+            elif kind == "stencil":
+                st.execute(stream)
+            if kind != "gemm":
+                st_ori.swap_buffers()
+
+    e0, e1 = ta.Event(), ta.Event()
+
+    def timed(kind):
+        torch.cuda.synchronize()
+        e0.record(stream)
+        job(kind)
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_ms(e1)
+
+    for kind in ("gemm", "stencil", "serial", "fused"):
+        for _ in range(args.warmup):
+            job(kind)
+    torch.cuda.synchronize()
+
+    samples = {k: [] for k in ("gemm", "stencil", "serial", "fused")}
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter()
+    for _ in range(args.steps):                      # EXACTLY K timed steps of each form
+        for kind in samples:
+            samples[kind].append(timed(kind))
+    torch.cuda.synchronize()
+    t_wall = time.perf_counter() - t_wall
+    ms = {k: trimmed_mean(v) for k, v in samples.items()}
+
+    gemm_flop = 2.0 * M * N * K
+    stencil_bytes = 2.0 * nx * ny * nz * 4
+    fused_launch_s = ms["fused"] / ITERATIONS * 1e-3
+    speedup = ms["serial"] / ms["fused"]
+    info = mix.info()
+    out = {
+        "metric": "fused-pair speedup vs serial (tzgemm 2048^3 + stencil 512x512x64, 100 iterations)",
+        "value": round(speedup, 4), "unit": "x", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms["fused"], 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 in / f32 accumulate (tzgemm), f32 (stencil)",
+        "data": "synthetic (numpy default_rng(1337): A,B uniform[-1,1] -> f16; grid uniform[0,1])",
+        "config": {"workload": "configs[1]: fused tzgemm fp16 2048x2048x2048 + 7-point stencil fp32 "
+                               "512x512x64, c0=1/6, c1=1/36, 100 iterations",
+                   "fused_kernel": "tzgemm_stencil@" + (args.variant or ta.lib().tacker_last_error() and "default" or "default"),
+                   "fused_grid": info["grid"], "fused_block": info["block"], "device": ta.device_name()},
+        "serial_ms_per_step": round(ms["serial"], 4),
+        "gemm_alone_ms_per_100": round(ms["gemm"], 4), "stencil_alone_ms_per_100": round(ms["stencil"], 4),
+        "overlap_efficiency": round(max(ms["gemm"], ms["stencil"]) / ms["fused"], 4),
+        "roofline": {"bound": "hbm", "achieved": round(stencil_bytes / fused_launch_s / 1e9, 1),
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(stencil_bytes / fused_launch_s / HBM_PEAK, 4), "traffic": None,
+                     "kernel": "stencil_tzgemm_mix (one fused launch: 1 GEMM + 1 sweep)",
+                     "algorithmic_bytes_per_launch": stencil_bytes,
+                     "avg_launch_us": round(fused_launch_s * 1e6, 2)},
+        "roofline_mfma": {"bound": "mfma", "achieved": round(gemm_flop / fused_launch_s / 1e12, 1),
+                          "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s",
+                          "frac": round(gemm_flop / fused_launch_s / MFMA_F16_PEAK, 4),
+                          "flop_per_launch": gemm_flop},
+        "alone": {
+            "tzgemm": {"avg_launch_us": round(ms["gemm"] * 10, 2),
+                       "tflops": round(gemm_flop / (ms["gemm"] / ITERATIONS * 1e-3) / 1e12, 1),
+                       "frac_of_mfma_peak": round(gemm_flop / (ms["gemm"] / ITERATIONS * 1e-3) / MFMA_F16_PEAK, 4)},
+            "stencil": {"avg_launch_us": round(ms["stencil"] * 10, 2),
+                        "gbps": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / 1e9, 1),
+                        "frac_of_hbm_peak": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / HBM_PEAK, 4)}},
+        "wall_s_timed_region": round(t_wall, 3),
+    }
+    out["config"]["fused_kernel"] = "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)")
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(A, B, A0, c0, c1)
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

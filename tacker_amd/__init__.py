@@ -410,3 +410,35 @@ def mix_create(be_gptb, tz_gptb, be_start, be_end, tile_start, tile_end, variant
     return KernelHandle(lib().tacker_mix_create(be_gptb.handle, tz_gptb.handle, be_start, be_end,
                                                 tile_start, tile_end, _v(variant), launch_grid,
                                                 launch_block), "MixKernel", keep=(be_gptb, tz_gptb))
+
+
+# ----------------------------------------------------------------------------- events
+class Event:
+    """tkEvent (hipEvent) recorded on the stream the kernels are launched on."""
+
+    def __init__(self):
+        self.h = C.c_void_p()
+        lib().tkEventCreate.argtypes = [C.POINTER(C.c_void_p)]
+        lib().tkEventRecord.argtypes = [C.c_void_p, C.c_void_p]
+        lib().tkEventSynchronize.argtypes = [C.c_void_p]
+        lib().tkEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
+        lib().tkEventDestroy.argtypes = [C.c_void_p]
+        check(lib().tkEventCreate(C.byref(self.h)), "tkEventCreate")
+
+    def record(self, stream=None):
+        check(lib().tkEventRecord(self.h, _stream(stream)), "tkEventRecord")
+
+    def synchronize(self):
+        check(lib().tkEventSynchronize(self.h), "tkEventSynchronize")
+
+    def elapsed_ms(self, later):
+        ms = C.c_float()
+        check(lib().tkEventElapsedTime(C.byref(ms), self.h, later.h), "tkEventElapsedTime")
+        return ms.value
+
+    def __del__(self):
+        try:
+            if self.h:
+                lib().tkEventDestroy(self.h)
+        except Exception:
+            pass

@@ -42,7 +42,7 @@ def test_tzgemm_closed_forms():
     B = rng.uniform(-1, 1, (256, K)).astype(np.float16)
     Cd = torch.zeros((128, 256), device="cuda:0")
     ta.gptb_tzgemm(dev(A), dev(B), Cd)
-    assert np.array_equal(host(Cd), B.astype(np.float32).T * np.float32(1.1))
+    assert np.array_equal(host(Cd), B.astype(np.float32).T[:128] * np.float32(1.1))
     ones = np.ones((128, K), np.float16)
     Cd2 = torch.zeros((128, 128), device="cuda:0")
     ta.gptb_tzgemm(dev(ones), dev(ones), Cd2)
