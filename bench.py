@@ -62,6 +62,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--variant", default=None, help="fused kernel variant (default: kinfo)")
+    ap.add_argument("--grid", type=int, default=0, help="fused launch grid (default: kinfo gridsize x CUs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -94,7 +95,7 @@ def main():
     st = ta.gptb_create(st_ori, 0, 0, 0, blocks)
     tz_ori = ta.ori_tzgemm_create(dA, dB, dC)
     tz = ta.gptb_create(tz_ori, 0, 0, 0, tiles)
-    mix = ta.mix_create(st, tz, 0, blocks, 0, tiles, variant=args.variant)
+    mix = ta.mix_create(st, tz, 0, blocks, 0, tiles, variant=args.variant, launch_grid=args.grid)
 
     def job(kind):
         for _ in range(ITERATIONS):

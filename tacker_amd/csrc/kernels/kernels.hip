@@ -30,8 +30,11 @@ extern "C" __global__ __launch_bounds__(128) void ori_stencil(float c0, float c1
 {
     const int tid = threadIdx.x + threadIdx.y * blockDim.x;
     const int wave = tid >> 6;
-    tk::stencil_wave_block<2>(c0, c1, A0, Anext, nx, ny, nz, blockIdx.x * 2 * STENCIL_TILE_X,
-                              blockIdx.y * STENCIL_TILE_Y + 2 * wave, tid & 63);
+    for (int k_first = 1; k_first <= nz - 2; k_first += STENCIL_Z_RUN)
+        tk::stencil_wave_run<2, STENCIL_Z_RUN>(c0, c1, A0, Anext, nx, ny, k_first,
+                                               min(STENCIL_Z_RUN, nz - 1 - k_first),
+                                               blockIdx.x * 2 * STENCIL_TILE_X,
+                                               blockIdx.y * STENCIL_TILE_Y + 2 * wave, tid & 63);
 }
 
 // grid (sy, sz), block sx

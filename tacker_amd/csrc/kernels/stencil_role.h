@@ -8,99 +8,104 @@
 //   Anext = (top + bottom + up + down + right + left)*c1 - centre*c0   (:68-69,:82-83)
 // so that results are bit-identical to an ordered fp32 evaluation.
 //
-// gfx950 design: one wave64 per reference block, no LDS and no barrier.  Lane l
-// owns column x = 64*bx + l and keeps ROWS rows of three consecutive z planes in
-// registers (bottom / centre / top); y neighbours inside the block are the
-// lane's own registers, x neighbours are the adjacent lanes' registers (wave
-// shuffle), and only the halo (row above/below the block, column left/right of
-// the wave) is read a second time, from L2.  Every global access of a wave is a
-// contiguous 256-byte row segment.  Because a block needs no workgroup-level
-// cooperation the role runs unchanged as a whole launch or as some waves of a
-// fused workgroup.
+// gfx950 design: one wave64 per reference block and run of STENCIL_Z_RUN centre
+// planes, no LDS and no barrier.  Lane l owns column x = 64*bx + l.  A wave first
+// issues every load of its run -- ROWS rows of Z+2 planes, the rows above and
+// below the block for Z planes, and one gathered load that brings the 2*ROWS*Z
+// values left and right of the wave's 64 columns (lane i < 32 fetches the left
+// neighbour of row i/Z, plane i%Z; lanes 32.. the right ones) -- so that about 60
+// independent 256-byte requests are in flight per wave, then computes from
+// registers: y neighbours are the lane's own registers, x neighbours the adjacent
+// lanes' (wave shuffle), the two outermost lanes read theirs out of the gathered
+// register with v_readlane.  Every global access of a wave is a contiguous row
+// segment.  Because a block needs no workgroup-level cooperation the role runs
+// unchanged as a whole launch or as some waves of a fused workgroup.
 #pragma once
 #include "role_common.h"
 #include "../header/stencil_header.h"
 
 namespace tk {
 
-// March one block column: x = x0 + lane, rows j0 .. j0+ROWS-1, k = 1 .. nz-2.
-template <int ROWS>
-__device__ __forceinline__ void stencil_wave_block(float c0, float c1, const float *__restrict__ A0,
-                                                   float *__restrict__ Anext, int nx, int ny, int nz,
-                                                   int x0, int j0, int lane)
+// One run: x = x0 + lane, rows j0 .. j0+ROWS-1, centre planes k_first ..
+// k_first+nplanes-1 with 1 <= nplanes <= Z (and k_first+nplanes-1 <= nz-2).
+template <int ROWS, int Z>
+__device__ __forceinline__ void stencil_wave_run(float c0, float c1, const float *__restrict__ A0,
+                                                 float *__restrict__ Anext, int nx, int ny,
+                                                 int k_first, int nplanes, int x0, int j0, int lane)
 {
+    static_assert(ROWS * Z <= 32, "the edge gather gives each half-wave one value per (row, plane)");
     const int x = x0 + lane;
     const size_t plane = (size_t)nx * (size_t)ny;
     const bool xin = x < nx;
+    const float *col = A0 + (size_t)x + (size_t)nx * j0 + plane * (k_first - 1);
+
+    // own rows: planes k_first-1 .. k_first+nplanes
+    float own[Z + 2][ROWS];
+#pragma unroll
+    for (int p = 0; p < Z + 2; ++p)
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r)
+            own[p][r] = (xin && (j0 + r) < ny && p <= nplanes + 1) ? col[plane * p + (size_t)nx * r] : 0.f;
+    // rows below (j0-1) and above (j0+ROWS) the block, centre planes only
+    float dn[Z], up[Z];
     const bool halo_dn = xin && j0 > 0;
     const bool halo_up = xin && (j0 + ROWS) < ny;
-    // lane 0 fetches the column left of the wave, lane 63 the column right of it
-    const bool edge_l = lane == 0 && x > 0 && xin;
-    const bool edge_r = lane == 63 && (x + 1) < nx;
-    const int edge_x = edge_l ? x - 1 : x + 1;
+#pragma unroll
+    for (int p = 0; p < Z; ++p) {
+        dn[p] = (halo_dn && p < nplanes) ? col[plane * (p + 1) - (size_t)nx] : 0.f;
+        up[p] = (halo_up && p < nplanes) ? col[plane * (p + 1) + (size_t)nx * ROWS] : 0.f;
+    }
+    // columns left (x0-1) and right (x0+64) of the wave: one gathered load
+    float edge = 0.f;
+    {
+        const int side = lane >> 5;
+        const int idx = lane & 31;
+        const int er = idx / Z, ep = idx % Z;
+        const int ex = side ? x0 + 64 : x0 - 1;
+        if (idx < ROWS * Z && ex >= 0 && ex < nx && (j0 + er) < ny && ep < nplanes)
+            edge = A0[(size_t)ex + (size_t)nx * (j0 + er) + plane * (k_first + ep)];
+    }
 
-    float bot[ROWS], cur[ROWS], top[ROWS], edge[ROWS];
-    float dn = 0.f, up = 0.f;
-    bool rin[ROWS], win[ROWS];
+    bool win[ROWS];
 #pragma unroll
     for (int r = 0; r < ROWS; ++r) {
         const int j = j0 + r;
-        rin[r] = xin && j < ny;
         win[r] = x > 0 && x < nx - 1 && j > 0 && j < ny - 1;
     }
-
-    auto load_rows = [&](int k, float (&dst)[ROWS]) {
+    float *out = Anext + (size_t)x + (size_t)nx * j0 + plane * k_first;
 #pragma unroll
-        for (int r = 0; r < ROWS; ++r)
-            dst[r] = rin[r] ? A0[(size_t)x + (size_t)nx * (j0 + r) + plane * k] : 0.f;
-    };
-    auto load_halo = [&](int k, float &d, float &u, float (&e)[ROWS]) {
-        d = halo_dn ? A0[(size_t)x + (size_t)nx * (j0 - 1) + plane * k] : 0.f;
-        u = halo_up ? A0[(size_t)x + (size_t)nx * (j0 + ROWS) + plane * k] : 0.f;
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r)
-            e[r] = ((edge_l || edge_r) && (j0 + r) < ny)
-                       ? A0[(size_t)edge_x + (size_t)nx * (j0 + r) + plane * k]
-                       : 0.f;
-    };
-
-    load_rows(0, bot);
-    load_rows(1, cur);
-    load_halo(1, dn, up, edge);
-    for (int k = 1; k < nz - 1; ++k) {
-        float ndn, nup, nedge[ROWS];
-        load_rows(k + 1, top);
-        load_halo(k + 1, ndn, nup, nedge);   // neighbours of the next centre plane
+    for (int p = 0; p < Z; ++p) {
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            float left = __shfl_up(cur[r], 1, 64);
-            float right = __shfl_down(cur[r], 1, 64);
-            if (lane == 0) left = edge[r];
-            if (lane == 63) right = edge[r];
-            const float a_up = (r + 1 < ROWS) ? cur[(r + 1 < ROWS) ? r + 1 : r] : up;
-            const float a_dn = (r > 0) ? cur[(r > 0) ? r - 1 : r] : dn;
-            if (win[r]) {
-                float s = top[r] + bot[r];
+            const float centre = own[p + 1][r];
+            float left = __shfl_up(centre, 1, 64);
+            float right = __shfl_down(centre, 1, 64);
+            const float edge_l = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge), r * Z + p));
+            const float edge_r = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge), 32 + r * Z + p));
+            if (lane == 0) left = edge_l;
+            if (lane == 63) right = edge_r;
+            const float a_up = (r + 1 < ROWS) ? own[p + 1][(r + 1 < ROWS) ? r + 1 : r] : up[p];
+            const float a_dn = (r > 0) ? own[p + 1][(r > 0) ? r - 1 : r] : dn[p];
+            if (win[r] && p < nplanes) {
+                float s = own[p + 2][r] + own[p][r];   // top + bottom
                 s = s + a_up;
                 s = s + a_dn;
                 s = s + right;
                 s = s + left;
-                Anext[(size_t)x + (size_t)nx * (j0 + r) + plane * k] = s * c1 - cur[r] * c0;
+                out[plane * p + (size_t)nx * r] = s * c1 - centre * c0;
             }
         }
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r) {
-            bot[r] = cur[r];
-            cur[r] = top[r];
-            edge[r] = nedge[r];
-        }
-        dn = ndn;
-        up = nup;
     }
 }
 
-// GPTB form: virtual block = one wave.  The role's waves enumerate block
-// positions start + (role_block*waves + wave) + i*(role_blocks*waves).
+// GPTB form.  The unit of work of a wave is one reference block cut into runs of
+// STENCIL_Z_RUN centre planes: a 512x512x64 grid has only 1024 blocks, far fewer
+// than the waves a 256-CU part needs in flight to pull HBM bandwidth, so the z
+// march of a block is shared out.  The waves of one workgroup take consecutive
+// runs of the same block (their overlap planes hit in the CU's own cache).
+// Task t of the range: block = start + t / runs, run = t % runs; the role's waves
+// enumerate t = role_block*waves + wave, stepping by role_blocks*waves.
+#define STENCIL_Z_RUN 8
 __device__ __forceinline__ void stencil_role(float c0, float c1, const float *__restrict__ A0,
                                              float *__restrict__ Anext, int nx, int ny, int nz,
                                              int grid_dimension_x, int grid_dimension_y,
@@ -110,13 +115,20 @@ __device__ __forceinline__ void stencil_role(float c0, float c1, const float *__
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int waves = role_threads >> 6;
+    const int planes = nz - 2;
+    if (planes < 1 || end <= start) return;
+    const unsigned runs = (unsigned)(planes + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
+    const unsigned tasks = (unsigned)(end - start) * runs;
     const unsigned stride = (unsigned)role_blocks * waves;
-    for (unsigned pos = (unsigned)start + role_block * waves + wave; pos < (unsigned)end;
-         pos += stride) {
+    for (unsigned t = (unsigned)role_block * waves + wave; t < tasks; t += stride) {
+        const unsigned pos = (unsigned)start + t / runs;
+        const int run = (int)(t % runs);
         const int bx = pos % grid_dimension_x;
         const int by = (pos / grid_dimension_x) % grid_dimension_y;
-        stencil_wave_block<STENCIL_TILE_Y>(c0, c1, A0, Anext, nx, ny, nz, bx * 2 * STENCIL_TILE_X,
-                                           by * STENCIL_TILE_Y, lane);
+        const int k_first = 1 + run * STENCIL_Z_RUN;
+        const int nplanes = min(STENCIL_Z_RUN, nz - 1 - k_first);
+        stencil_wave_run<STENCIL_TILE_Y, STENCIL_Z_RUN>(c0, c1, A0, Anext, nx, ny, k_first, nplanes,
+                                                        bx * 2 * STENCIL_TILE_X, by * STENCIL_TILE_Y, lane);
     }
 }
 
