@@ -274,6 +274,62 @@ TK_API uint16_t tacker_float_to_half_bits(float f);
  * [lo,hi) floats of the stream started by seed */
 TK_API int tacker_rng_uniform(uint64_t seed, float lo, float hi, float *out, size_t n);
 
+/* ---- the latency-critical task and the scheduler ------------------------------ */
+typedef void *tacker_task_t;
+typedef void *tacker_task_manager_t;
+
+/* createTask (src/main.cu:227-244): "vgg16" builds VGG16 at batch 1 with
+ * random-initialised f16 weights; height/width 0 = 224. */
+TK_API tacker_task_t tacker_task_create(const char *model, int height, int width);
+TK_API int tacker_task_destroy(tacker_task_t task);
+/* Task::initExecution + every kernel's execute(stream) (the warm-up loop of
+ * src/main.cu:290-297) */
+TK_API int tacker_task_execute(tacker_task_t task, tkStream_t stream);
+TK_API int tacker_task_kernel_count(tacker_task_t task);
+/* name (up to name_cap bytes), mixable flag, getArgs() (up to 14 ints, count in *nargs) */
+TK_API int tacker_task_kernel_info(tacker_task_t task, int index, char *name, int name_cap,
+                                   int *mixable, int args[14], int *nargs);
+/* VGG16 only: output of convolution conv_index after bias+ReLU: device pointer and
+ * dims = {H, W, channels, channel stride}; logits = column 0 of the last GEMM */
+TK_API int tacker_task_activation(tacker_task_t task, int conv_index, float **ptr, int dims[4]);
+TK_API int tacker_task_logits(tacker_task_t task, const float **ptr, long *stride, int *count);
+/* VGG16 only: weights (f16 [dims[0]][dims[1]] = [Cout padded][9*Cin padded], k =
+ * (kh*3+kw)*Cin + c) and bias (f32 [dims[0]]) of convolution conv_index */
+TK_API int tacker_task_conv_params(tacker_task_t task, int conv_index, void **weights, float **bias,
+                                   int dims[2]);
+TK_API int tacker_task_input(tacker_task_t task, float **host_ptr, int *bytes);
+
+/* TaskManager(lc_task, be1, be2) (src/TaskManager.h:7-18) */
+TK_API tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const char *be_task1,
+                                                        const char *be_task2);
+TK_API int tacker_task_manager_destroy(tacker_task_manager_t tm);
+/* the constants the reference hard-codes: 50 ms budget, 4 ms guard, 5 warm-up,
+ * 10 profiling and 5 co-located queries (src/TaskManager.cu:430,446,569-586);
+ * a negative value keeps the current setting */
+TK_API int tacker_task_manager_configure(tacker_task_manager_t tm, float qos_budget_ms, float guard_ms,
+                                         int warmup_queries, int profile_queries, int queries,
+                                         int verbose);
+/* executeAllTasks (second_stage != 0) or execute_with_one_cd_kernel; mode 0 = Aker
+ * (ratio-limited BE slice per GEMM), 1 = Tacker (whole BE kernel per GEMM) */
+TK_API int tacker_task_manager_run(tacker_task_manager_t tm, int mode, tkStream_t stream,
+                                   int second_stage);
+/* out = {lc_solo_ms, be1_solo_ms, be2_solo_ms, be_blocks_executed, mix_times,
+ * mixable_times, time_earned_ms, qos_headroom_left_ms, stage1_be_ms, stage2_be_ms,
+ * be_task_finish_num, n co-located latencies, n solo latencies} */
+TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
+/* which = 0: per-query latency of the co-located queries, 1: of the solo profiling queries */
+TK_API int tacker_task_manager_latencies(tacker_task_manager_t tm, int which, float *out, int cap);
+
+/* the scheduler's arithmetic on its own (src/TaskManager.cu:586-640) */
+TK_API float tacker_qos_block_ratio(const char *be_name, int K_GLOBAL);
+TK_API int tacker_qos_colocated_blocks(int mode, const char *be_name, int tiles, int K_GLOBAL,
+                                       int be_total_blocks);
+TK_API int tacker_qos_must_run_solo(float budget_ms, float guard_ms, float qos_headroom,
+                                    float lc_time_remaining);
+/* out = {counted_as_mixed, charged_ms, earned_ms} */
+TK_API int tacker_qos_account(int mixable, float measured_ms, float solo_lc_ms, float be_ms,
+                              int cd_blocks, int be_total_blocks, float out[3]);
+
 #ifdef __cplusplus
 }
 #endif

@@ -81,6 +81,29 @@ def _declare(lib):
     lib.tacker_float_to_half_bits.argtypes = [f]
     lib.tacker_float_to_half_bits.restype = C.c_uint16
     lib.tacker_rng_uniform.argtypes = [C.c_uint64, f, f, vp, C.c_size_t]
+    lib.tacker_task_create.restype = vp
+    lib.tacker_task_create.argtypes = [cp, i, i]
+    lib.tacker_task_destroy.argtypes = [vp]
+    lib.tacker_task_execute.argtypes = [vp, vp]
+    lib.tacker_task_kernel_count.argtypes = [vp]
+    lib.tacker_task_kernel_info.argtypes = [vp, i, C.c_char_p, i, C.POINTER(i), C.POINTER(i), C.POINTER(i)]
+    lib.tacker_task_activation.argtypes = [vp, i, C.POINTER(vp), C.POINTER(i)]
+    lib.tacker_task_conv_params.argtypes = [vp, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(i)]
+    lib.tkMemcpy.argtypes = [vp, vp, C.c_size_t, i]
+    lib.tacker_task_logits.argtypes = [vp, C.POINTER(vp), C.POINTER(C.c_long), C.POINTER(i)]
+    lib.tacker_task_input.argtypes = [vp, C.POINTER(vp), C.POINTER(i)]
+    lib.tacker_task_manager_create.restype = vp
+    lib.tacker_task_manager_create.argtypes = [vp, cp, cp]
+    lib.tacker_task_manager_destroy.argtypes = [vp]
+    lib.tacker_task_manager_configure.argtypes = [vp, f, f, i, i, i, i]
+    lib.tacker_task_manager_run.argtypes = [vp, i, vp, i]
+    lib.tacker_task_manager_report.argtypes = [vp, C.POINTER(f)]
+    lib.tacker_task_manager_latencies.argtypes = [vp, i, C.POINTER(f), i]
+    lib.tacker_qos_block_ratio.argtypes = [cp, i]
+    lib.tacker_qos_block_ratio.restype = f
+    lib.tacker_qos_colocated_blocks.argtypes = [i, cp, i, i, i]
+    lib.tacker_qos_must_run_solo.argtypes = [f, f, f, f]
+    lib.tacker_qos_account.argtypes = [i, f, f, f, i, i, C.POINTER(f)]
     return lib
 
 
@@ -442,3 +465,123 @@ class Event:
                 lib().tkEventDestroy(self.h)
         except Exception:
             pass
+
+
+def device_to_host(ptr, shape, dtype, library=None):
+    """tkMemcpy device -> host of a raw device pointer into a fresh numpy array."""
+    import numpy as np
+    out = np.empty(shape, dtype)
+    l = library or lib()
+    rc = l.tkMemcpy(out.ctypes.data, ptr, out.nbytes, 2)
+    if rc:
+        raise TackerError(f"tkMemcpy failed ({rc})")
+    return out
+
+
+# ----------------------------------------------------------------------------- LC task + scheduler
+REPORT_KEYS = ("lc_solo_ms", "be1_solo_ms", "be2_solo_ms", "be_blocks_executed", "mix_times",
+               "mixable_times", "time_earned_ms", "qos_headroom_left_ms", "stage1_be_ms", "stage2_be_ms",
+               "be_task_finish_num", "n_colocated", "n_solo")
+
+
+class LcTask:
+    """createTask(model): the latency-critical job (VGG16 at batch 1)."""
+
+    def __init__(self, model="vgg16", height=0, width=0, library=None):
+        self.l = library or lib()
+        self.h = self.l.tacker_task_create(model.encode(), height, width)
+        if not self.h:
+            raise TackerError(f"createTask({model}) failed: {self.l.tacker_last_error().decode()}")
+
+    def execute(self, stream=None, raw_stream=...):
+        st = raw_stream if raw_stream is not ... else _stream(stream)
+        rc = self.l.tacker_task_execute(self.h, st)
+        if rc:
+            raise TackerError(f"task execute failed ({rc}): {self.l.tacker_last_error().decode()}")
+
+    def kernels(self):
+        out = []
+        for idx in range(self.l.tacker_task_kernel_count(self.h)):
+            name = C.create_string_buffer(128)
+            mix, n = C.c_int(), C.c_int()
+            args = (C.c_int * 14)()
+            self.l.tacker_task_kernel_info(self.h, idx, name, 128, C.byref(mix), args, C.byref(n))
+            out.append({"name": name.value.decode(), "mixable": mix.value, "args": list(args)[:n.value]})
+        return out
+
+    def activation(self, conv_index):
+        p = C.c_void_p()
+        dims = (C.c_int * 4)()
+        rc = self.l.tacker_task_activation(self.h, conv_index, C.byref(p), dims)
+        if rc:
+            raise TackerError(self.l.tacker_last_error().decode())
+        return p.value, tuple(dims)
+
+    def conv_params(self, conv_index):
+        """(weights f16 [Np][Kp], bias f32 [Np]) of a convolution, copied to the host."""
+        import numpy as np
+        w, b = C.c_void_p(), C.c_void_p()
+        dims = (C.c_int * 2)()
+        rc = self.l.tacker_task_conv_params(self.h, conv_index, C.byref(w), C.byref(b), dims)
+        if rc:
+            raise TackerError(self.l.tacker_last_error().decode())
+        return (device_to_host(w.value, (dims[0], dims[1]), np.float16, self.l),
+                device_to_host(b.value, (dims[0],), np.float32, self.l))
+
+    def logits(self):
+        p = C.c_void_p()
+        stride, n = C.c_long(), C.c_int()
+        rc = self.l.tacker_task_logits(self.h, C.byref(p), C.byref(stride), C.byref(n))
+        if rc:
+            raise TackerError(self.l.tacker_last_error().decode())
+        return p.value, stride.value, n.value
+
+    def host_input(self):
+        import numpy as np
+        p = C.c_void_p()
+        nbytes = C.c_int()
+        self.l.tacker_task_input(self.h, C.byref(p), C.byref(nbytes))
+        buf = (C.c_float * (nbytes.value // 4)).from_address(p.value)
+        return np.frombuffer(buf, dtype=np.float32)
+
+    def close(self):
+        if self.h:
+            self.l.tacker_task_destroy(self.h)
+            self.h = None
+
+
+class TaskManager:
+    """TaskManager(lc_task, be1, be2) with the reference's constants exposed."""
+
+    def __init__(self, task, be1, be2=None, library=None):
+        self.l = library or lib()
+        self.task = task
+        self.h = self.l.tacker_task_manager_create(task.h, be1.encode(), be2.encode() if be2 else None)
+        if not self.h:
+            raise TackerError(f"TaskManager failed: {self.l.tacker_last_error().decode()}")
+
+    def configure(self, qos_budget_ms=-1.0, guard_ms=-1.0, warmup=-1, profile=-1, queries=-1, verbose=-1):
+        self.l.tacker_task_manager_configure(self.h, qos_budget_ms, guard_ms, warmup, profile, queries, verbose)
+
+    def run(self, mode="aker", stream=None, second_stage=False, raw_stream=...):
+        st = raw_stream if raw_stream is not ... else _stream(stream)
+        rc = self.l.tacker_task_manager_run(self.h, 0 if mode == "aker" else 1, st, 1 if second_stage else 0)
+        if rc:
+            raise TackerError(f"TaskManager run failed ({rc}): {self.l.tacker_last_error().decode()}")
+        return self.report()
+
+    def report(self):
+        out = (C.c_float * 13)()
+        self.l.tacker_task_manager_report(self.h, out)
+        return dict(zip(REPORT_KEYS, out))
+
+    def latencies(self, solo=False):
+        cap = 1 << 20
+        buf = (C.c_float * cap)()
+        n = self.l.tacker_task_manager_latencies(self.h, 1 if solo else 0, buf, cap)
+        return list(buf[:n])
+
+    def close(self):
+        if self.h:
+            self.l.tacker_task_manager_destroy(self.h)
+            self.h = None

@@ -1,0 +1,90 @@
+// TaskManager.h -- QoS-aware co-location of one latency-critical (LC) task with
+// best-effort (BE) kernels (src/TaskManager.h of the reference).
+//
+// Same public surface: TaskManager(Task*, be1, be2), executeAllTasks(mode, stream),
+// execute_with_one_cd_kernel(mode, stream), the free functions
+// mixcudnnConvolutionForward / mixcublasSgemm / get_mnk_from_cudnn_args.  The
+// decision arithmetic of the reference's hot loop (src/TaskManager.cu:586-640) is
+// factored into QosPolicy so that it can be exercised with synthetic durations.
+#pragma once
+
+#include <string>
+#include <vector>
+
+#include "GPTBKernel.h"
+#include "Task.h"
+
+// {M, N, K} of the GEMM a convolution lowers to, from the 14 ints
+// {n,c,h,w, k,c,kh,kw, pad_h,pad_w, stride_h,stride_w, dil_h,dil_w}
+// (src/TaskManager.cu:92-123).
+std::vector<int> get_mnk_from_cudnn_args(std::vector<int> &cudnn_args);
+
+// One fused launch: the LC convolution's GEMM (after im2col) together with blocks
+// [cd_start_blk, cd_end_blk) of the BE kernel (src/TaskManager.cu:125-306).
+void mixcudnnConvolutionForward(std::vector<int> &cudnn_args, GPTBKernel *gptb_cd_kernel,
+                                int cd_start_blk, int cd_end_blk, cudaStream_t stream);
+// One fused launch: an LC fully-connected GEMM {m,n,k} + BE blocks (src/TaskManager.cu:309-400).
+void mixcublasSgemm(std::vector<int> &gemm_args, GPTBKernel *gptb_cd_kernel, int cd_start_blk,
+                    int cd_end_blk, cudaStream_t stream);
+
+// The per-query accounting of the scheduler, free of any device call.
+struct QosPolicy {
+    float qos_budget_ms = 50.0f;   // per LC query (src/TaskManager.cu:571)
+    float guard_ms = 4.0f;         // headroom guard band (:586)
+
+    // BE blocks per 64x64 GEMM tile for a GEMM of depth K_GLOBAL: kinfo entry
+    // "tzgemm_<be>"[K]; when absent, the K=4096 entry scaled linearly by K (:593-598).
+    static float blockRatio(const std::string &be_name, int K_GLOBAL);
+    // how many BE blocks ride along with a GEMM of `tiles` tiles (:599-600)
+    static int coLocatedBlocks(ExecutionMode mode, const std::string &be_name, int tiles, int K_GLOBAL,
+                               int be_total_blocks);
+    // solo if the remaining budget cannot cover the rest of the query plus the guard (:586)
+    bool mustRunSolo(float qos_headroom, float lc_time_remaining) const
+    {
+        return qos_headroom < lc_time_remaining + guard_ms;
+    }
+    struct Outcome {
+        bool counted_as_mixed;   // the fused launch beat "LC alone then BE share alone"
+        float charged_ms;        // what the query's budget is charged
+        float earned_ms;         // time saved against serial execution (0 if not mixed)
+    };
+    // (:628-640) solo_lc_ms = profiled LC kernel time; be_ms = BE kernel's full solo time
+    static Outcome account(unsigned mixable, float measured_ms, float solo_lc_ms, float be_ms,
+                           int cd_blocks, int be_total_blocks);
+};
+
+struct TaskManagerReport {
+    float lc_solo_ms = 0.0f;            // sum of profiled LC kernel times ("[PRE]")
+    float be1_solo_ms = 0.0f, be2_solo_ms = 0.0f;
+    long long be_blocks_executed = 0;   // BE blocks carried by fused launches in the last query
+    int mix_times = 0, mixable_times = 0;
+    float time_earned_ms = 0.0f;
+    float qos_headroom_left_ms = 0.0f;
+    float stage1_be_ms = 0.0f, stage2_be_ms = 0.0f;
+    std::vector<float> query_latency_ms;   // one entry per co-located LC query
+    std::vector<float> solo_latency_ms;    // one entry per solo LC query (profiling passes)
+};
+
+class TaskManager {
+public:
+    TaskManager(Task *lc_task, const std::string &be_task1, const std::string &be_task2);
+    ~TaskManager();
+    void executeAllTasks(ExecutionMode mode, cudaStream_t stream);
+    void execute_with_one_cd_kernel(ExecutionMode mode, cudaStream_t stream);
+
+    Task *lc_task;
+    std::string be_task1_name;
+    std::string be_task2_name;
+    int be_task_finish_num = 0;   // complete passes over the BE kernel's blocks
+
+    // knobs the reference hard-codes
+    QosPolicy policy;
+    int warmup_queries = 5;
+    int profile_queries = 10;
+    int queries = 5;
+    bool verbose = true;
+    TaskManagerReport report;
+
+private:
+    void run(ExecutionMode mode, cudaStream_t stream, bool with_second_stage);
+};

@@ -11,6 +11,8 @@
 #include "Logger.h"
 #include "json.h"
 #include "rng.h"
+#include "TaskManager.h"
+#include "dnn/vgg16.h"
 
 extern Logger logger;
 extern std::unordered_map<std::string, void *> fmap;
@@ -590,6 +592,214 @@ int tacker_rng_uniform(uint64_t seed, float lo, float hi, float *out, size_t n)
     if (!out) return fail(TK_ERROR_INVALID_VALUE, "null output");
     tk::Rng rng(seed);
     for (size_t i = 0; i < n; ++i) out[i] = rng.uniform(lo, hi);
+    return TK_SUCCESS;
+}
+
+
+// ---- LC task and scheduler ----------------------------------------------------
+
+tacker_task_t tacker_task_create(const char *model, int height, int width)
+{
+    if (!tacker_runtime_ready() || !model) {
+        fail(TK_ERROR_INVALID_VALUE, "tacker_task_create: not initialised");
+        return nullptr;
+    }
+    if (strcmp(model, "vgg16")) {
+        fail(TK_ERROR_NOT_FOUND, std::string("createTask: model not found: ") + model);
+        return nullptr;
+    }
+    VGG16Options opt;
+    if (height > 0) opt.height = height;
+    if (width > 0) opt.width = width;
+    if (opt.height % 32 || opt.width % 32) {
+        fail(TK_ERROR_UNSUPPORTED, "vgg16: input resolution must be a multiple of 32");
+        return nullptr;
+    }
+    tacker_task_t out = nullptr;
+    guarded([&]() -> int {
+        out = static_cast<Task *>(new VGG16(1, opt));
+        return TK_SUCCESS;
+    });
+    return out;
+}
+
+int tacker_task_destroy(tacker_task_t task)
+{
+    delete static_cast<Task *>(task);
+    return TK_SUCCESS;
+}
+
+int tacker_task_execute(tacker_task_t h, tkStream_t stream)
+{
+    Task *t = static_cast<Task *>(h);
+    if (!t) return fail(TK_ERROR_INVALID_VALUE, "null task");
+    return guarded([&]() -> int {
+        t->initExecution();
+        for (auto *k : t->kernels) k->execute(stream);
+        return TK_SUCCESS;
+    });
+}
+
+int tacker_task_kernel_count(tacker_task_t h)
+{
+    Task *t = static_cast<Task *>(h);
+    return t ? (int)t->kernels.size() : -1;
+}
+
+int tacker_task_kernel_info(tacker_task_t h, int index, char *name, int name_cap, int *mixable, int args[14], int *nargs)
+{
+    Task *t = static_cast<Task *>(h);
+    if (!t || index < 0 || index >= (int)t->kernels.size()) return fail(TK_ERROR_INVALID_VALUE, "bad kernel index");
+    Kernel *k = t->kernels[index];
+    if (name && name_cap > 0) snprintf(name, name_cap, "%s", k->kernelName.c_str());
+    if (mixable) *mixable = (int)k->mixable;
+    const std::vector<int> a = k->getArgs();
+    if (nargs) *nargs = (int)a.size();
+    if (args)
+        for (size_t i = 0; i < a.size() && i < 14; ++i) args[i] = a[i];
+    return TK_SUCCESS;
+}
+
+int tacker_task_activation(tacker_task_t h, int conv_index, float **ptr, int dims[4])
+{
+    VGG16 *v = dynamic_cast<VGG16 *>(static_cast<Task *>(h));
+    if (!v || conv_index < 0 || conv_index >= 13) return fail(TK_ERROR_INVALID_VALUE, "bad activation index");
+    const VGG16::Act a = v->activation(conv_index);
+    *ptr = a.ptr;
+    dims[0] = a.H; dims[1] = a.W; dims[2] = a.C; dims[3] = a.ld;
+    return TK_SUCCESS;
+}
+
+int tacker_task_conv_params(tacker_task_t h, int conv_index, void **weights, float **bias, int dims[2])
+{
+    VGG16 *v = dynamic_cast<VGG16 *>(static_cast<Task *>(h));
+    if (!v || conv_index < 0 || conv_index >= 13) return fail(TK_ERROR_INVALID_VALUE, "bad convolution index");
+    const VGG16::Act a = v->activation(conv_index);
+    *weights = a.weights;
+    *bias = a.bias;
+    dims[0] = a.Np;
+    dims[1] = a.Kp;
+    return TK_SUCCESS;
+}
+
+int tacker_task_logits(tacker_task_t h, const float **ptr, long *stride, int *count)
+{
+    VGG16 *v = dynamic_cast<VGG16 *>(static_cast<Task *>(h));
+    if (!v) return fail(TK_ERROR_INVALID_VALUE, "not a vgg16 task");
+    *ptr = v->logits(stride);
+    if (count) *count = v->opt.classes;
+    return TK_SUCCESS;
+}
+
+int tacker_task_input(tacker_task_t h, float **host_ptr, int *bytes)
+{
+    Task *t = static_cast<Task *>(h);
+    if (!t) return fail(TK_ERROR_INVALID_VALUE, "null task");
+    *host_ptr = static_cast<float *>(t->InputHost[0]);
+    *bytes = t->InputSize[0];
+    return TK_SUCCESS;
+}
+
+tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const char *be1, const char *be2)
+{
+    if (!lc_task || !be1) {
+        fail(TK_ERROR_INVALID_VALUE, "tacker_task_manager_create: bad arguments");
+        return nullptr;
+    }
+    static const char *known[] = {"cp", "lbm", "mriq", "stencil"};
+    bool ok1 = false, ok2 = !be2 || !*be2;
+    for (auto k : known) {
+        ok1 |= strcmp(k, be1) == 0;
+        if (be2) ok2 |= strcmp(k, be2) == 0;
+    }
+    if (!ok1 || !ok2) {
+        fail(TK_ERROR_NOT_FOUND, "Creator: Kernel not found");
+        return nullptr;
+    }
+    return new TaskManager(static_cast<Task *>(lc_task), be1, be2 ? be2 : "");
+}
+
+int tacker_task_manager_destroy(tacker_task_manager_t tm)
+{
+    delete static_cast<TaskManager *>(tm);
+    return TK_SUCCESS;
+}
+
+int tacker_task_manager_configure(tacker_task_manager_t h, float qos_budget_ms, float guard_ms, int warmup_queries,
+                                  int profile_queries, int queries, int verbose)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm) return fail(TK_ERROR_INVALID_VALUE, "null task manager");
+    if (qos_budget_ms >= 0) tm->policy.qos_budget_ms = qos_budget_ms;
+    if (guard_ms >= 0) tm->policy.guard_ms = guard_ms;
+    if (warmup_queries >= 0) tm->warmup_queries = warmup_queries;
+    if (profile_queries >= 0) tm->profile_queries = profile_queries;
+    if (queries >= 0) tm->queries = queries;
+    if (verbose >= 0) tm->verbose = verbose != 0;
+    return TK_SUCCESS;
+}
+
+int tacker_task_manager_run(tacker_task_manager_t h, int mode, tkStream_t stream, int second_stage)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm) return fail(TK_ERROR_INVALID_VALUE, "null task manager");
+    if (mode != 0 && mode != 1) return fail(TK_ERROR_INVALID_VALUE, "mode must be 0 (Aker) or 1 (Tacker)");
+    if (second_stage && tm->be_task2_name.empty()) return fail(TK_ERROR_INVALID_VALUE, "no second BE kernel");
+    return guarded([&]() -> int {
+        const ExecutionMode m = mode ? ExecutionMode::Tacker : ExecutionMode::Aker;
+        if (second_stage) tm->executeAllTasks(m, stream);
+        else tm->execute_with_one_cd_kernel(m, stream);
+        return TK_SUCCESS;
+    });
+}
+
+int tacker_task_manager_report(tacker_task_manager_t h, float out[13])
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm) return fail(TK_ERROR_INVALID_VALUE, "null task manager");
+    const TaskManagerReport &r = tm->report;
+    const float v[13] = {r.lc_solo_ms, r.be1_solo_ms, r.be2_solo_ms, (float)r.be_blocks_executed,
+                         (float)r.mix_times, (float)r.mixable_times, r.time_earned_ms, r.qos_headroom_left_ms,
+                         r.stage1_be_ms, r.stage2_be_ms, (float)tm->be_task_finish_num,
+                         (float)r.query_latency_ms.size(), (float)r.solo_latency_ms.size()};
+    memcpy(out, v, sizeof(v));
+    return TK_SUCCESS;
+}
+
+int tacker_task_manager_latencies(tacker_task_manager_t h, int which, float *out, int cap)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || !out) return -1;
+    const std::vector<float> &v = which ? tm->report.solo_latency_ms : tm->report.query_latency_ms;
+    const int n = std::min((int)v.size(), cap);
+    memcpy(out, v.data(), (size_t)n * sizeof(float));
+    return n;
+}
+
+float tacker_qos_block_ratio(const char *be_name, int K_GLOBAL) { return QosPolicy::blockRatio(be_name, K_GLOBAL); }
+
+int tacker_qos_colocated_blocks(int mode, const char *be_name, int tiles, int K_GLOBAL, int be_total_blocks)
+{
+    return QosPolicy::coLocatedBlocks(mode ? ExecutionMode::Tacker : ExecutionMode::Aker, be_name, tiles, K_GLOBAL,
+                                      be_total_blocks);
+}
+
+int tacker_qos_must_run_solo(float budget_ms, float guard_ms, float qos_headroom, float lc_time_remaining)
+{
+    QosPolicy p;
+    p.qos_budget_ms = budget_ms;
+    p.guard_ms = guard_ms;
+    return p.mustRunSolo(qos_headroom, lc_time_remaining) ? 1 : 0;
+}
+
+int tacker_qos_account(int mixable, float measured_ms, float solo_lc_ms, float be_ms, int cd_blocks,
+                       int be_total_blocks, float out[3])
+{
+    const QosPolicy::Outcome o = QosPolicy::account((unsigned)mixable, measured_ms, solo_lc_ms, be_ms, cd_blocks,
+                                                    be_total_blocks);
+    out[0] = o.counted_as_mixed ? 1.0f : 0.0f;
+    out[1] = o.charged_ms;
+    out[2] = o.earned_ms;
     return TK_SUCCESS;
 }
 

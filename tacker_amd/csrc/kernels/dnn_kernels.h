@@ -1,0 +1,78 @@
+// Data-movement kernels of the latency-critical DNN task (VGG16, batch 1), whose
+// convolutions and fully-connected layers run on tzgemm.
+//
+// The reference lowers a convolution with a Caffe NCHW im2col into an fp32 column
+// buffer and then times ptb_tzgemm on unrelated global operands
+// (src/include/dnn.h:554-803): a timing proxy.  Here the GEMM consumes the real
+// activations, so im2col writes the operand tzgemm wants directly: A[M][K] f16
+// with K contiguous, from NHWC fp32 activations.
+#pragma once
+#include <hip/hip_runtime.h>
+
+// A[m][k] for m = (h*W + w), k = (kh*KW + kw)*C + c; zero for padding taps and for
+// k in [KH*KW*C, K_pad).  Rows m >= H*W of A are never written (they stay zero).
+// act is [H][W][c_stride] with c < C used.  3x3/stride-1 style parameters general.
+extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C, int c_stride,
+                                           int KH, int KW, int pad, int stride, int Ho, int Wo,
+                                           _Float16 *A, int K_pad)
+{
+    const long total = (long)Ho * Wo * K_pad;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)blockDim.x * gridDim.x) {
+        const int k = (int)(i % K_pad);
+        const long m = i / K_pad;
+        float v = 0.0f;
+        if (k < KH * KW * C) {
+            const int c = k % C;
+            const int tap = k / C;
+            const int kw = tap % KW, kh = tap / KW;
+            const int wo = (int)(m % Wo), ho = (int)(m / Wo);
+            const int h = ho * stride - pad + kh, w = wo * stride - pad + kw;
+            if (h >= 0 && h < H && w >= 0 && w < W) v = act[((long)h * W + w) * c_stride + c];
+        }
+        A[i] = (_Float16)v;
+    }
+}
+
+// y[m][n] = max(0, y[m][n] + bias[n]) over rows < M of a [M][ld] matrix
+extern "C" __global__ void bias_relu_rows(float *y, const float *bias, int M, int ld, int relu)
+{
+    const long total = (long)M * ld;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)blockDim.x * gridDim.x) {
+        float v = y[i] + bias[i % ld];
+        y[i] = (relu && v < 0.0f) ? 0.0f : v;
+    }
+}
+
+// 2x2 / stride 2 max pooling, NHWC with channel stride ld
+extern "C" __global__ void maxpool2x2_nhwc(const float *in, int H, int W, int ld, float *out)
+{
+    const int Ho = H / 2, Wo = W / 2;
+    const long total = (long)Ho * Wo * ld;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long)blockDim.x * gridDim.x) {
+        const int c = (int)(i % ld);
+        const long p = i / ld;
+        const int wo = (int)(p % Wo), ho = (int)(p / Wo);
+        const float *src = in + ((long)(2 * ho) * W + 2 * wo) * ld + c;
+        const float a = src[0], b = src[ld], d = src[(long)W * ld], e = src[(long)W * ld + ld];
+        out[i] = fmaxf(fmaxf(a, b), fmaxf(d, e));
+    }
+}
+
+// Fully-connected layers run as C[out][128] = W[out][K] * X[128][K]^T with the
+// batch-1 activation in row 0 of X: pack an fp32 vector (taken with a stride, so
+// it can be column 0 of the previous layer's output) into that f16 row, with an
+// optional bias + ReLU on the way.
+extern "C" __global__ void pack_fc_input(const float *src, long src_stride, const float *bias, int relu,
+                                         int n, _Float16 *x_row)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        float v = src[(long)i * src_stride];
+        if (bias) v += bias[i];
+        if (relu && v < 0.0f) v = 0.0f;
+        x_row[i] = (_Float16)v;
+    }
+}

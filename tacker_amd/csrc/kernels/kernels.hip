@@ -12,6 +12,7 @@
 
 #include "../../../include/tacker_amd.h"
 #include "cp_role.h"
+#include "dnn_kernels.h"
 #include "lbm_role.h"
 #include "mriq_role.h"
 #include "stencil_role.h"
@@ -176,6 +177,10 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("gptb_cp", (const void *)g_general_ptb_cp, ctx);
     insert("im2col", (const void *)im2col_gpu_kernel_, ctx);
     insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);
+    insert("im2col_nhwc_f16", (const void *)im2col_nhwc_f16, ctx);
+    insert("bias_relu_rows", (const void *)bias_relu_rows, ctx);
+    insert("maxpool2x2_nhwc", (const void *)maxpool2x2_nhwc, ctx);
+    insert("pack_fc_input", (const void *)pack_fc_input, ctx);
     tk_register_mix_kernels(insert, ctx);
     return TK_SUCCESS;
 }

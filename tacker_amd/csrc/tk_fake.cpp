@@ -31,6 +31,7 @@ std::vector<Launch> g_launches;
 int g_fail_next_launch = 0;
 int g_cu_count = 256;
 float g_event_ms = 1.0f;
+std::vector<float> g_event_queue;   // scripted durations, consumed first
 std::map<std::string, std::vector<unsigned char>> g_symbols;
 
 const int P = 8, I = 4, F = 4;   // pointer, int, float
@@ -98,7 +99,16 @@ int tkEventCreate(tkEvent_t *e) { *e = malloc(1); return TK_SUCCESS; }
 int tkEventDestroy(tkEvent_t e) { free(e); return TK_SUCCESS; }
 int tkEventRecord(tkEvent_t, tkStream_t) { return TK_SUCCESS; }
 int tkEventSynchronize(tkEvent_t) { return TK_SUCCESS; }
-int tkEventElapsedTime(float *ms, tkEvent_t, tkEvent_t) { *ms = g_event_ms; return TK_SUCCESS; }
+int tkEventElapsedTime(float *ms, tkEvent_t, tkEvent_t)
+{
+    if (!g_event_queue.empty()) {
+        *ms = g_event_queue.front();
+        g_event_queue.erase(g_event_queue.begin());
+    } else {
+        *ms = g_event_ms;
+    }
+    return TK_SUCCESS;
+}
 
 int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, size_t, tkStream_t stream)
 {
@@ -146,7 +156,7 @@ int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void **args,
 int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
 {
     if (kernels().empty()) {
-        auto add = [](const char *key, std::vector<int> sizes) {
+        auto add = [](const std::string &key, std::vector<int> sizes) {
             kernels().push_back(new FakeKernel{key, std::move(sizes)});
         };
         add("ori_stencil", STENCIL);
@@ -161,10 +171,17 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("gptb_cp", cat(CP, trailer(true)));
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
-        add("tzgemm_stencil", cat(cat(STENCIL, trailer(false)), cat(TZ, trailer(false))));
-        add("tzgemm_lbm", cat(cat(LBM, trailer(false)), cat(TZ, trailer(false))));
-        add("tzgemm_mriq", cat(cat(MRIQ, trailer(false)), cat(TZ, trailer(false))));
-        add("tzgemm_cp", cat(cat(CP, trailer(false)), cat(TZ, trailer(false))));
+        add("im2col_nhwc_f16", {P, I, I, I, I, I, I, I, I, I, I, P, I});
+        add("bias_relu_rows", {P, P, I, I, I});
+        add("maxpool2x2_nhwc", {P, I, I, I, P});
+        add("pack_fc_input", {P, 8, P, I, I, P});
+        const std::pair<const char *, const std::vector<int> *> bes[] = {
+            {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}};
+        static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1", "@wave_256", "@wave_512"};
+        for (auto &be : bes)
+            for (auto v : variants)
+                add((std::string("tzgemm_") + be.first + v).c_str(),
+                    cat(cat(*be.second, trailer(false)), cat(TZ, trailer(false))));
     }
     for (auto *k : kernels()) insert(k->key.c_str(), k, ctx);
     return TK_SUCCESS;
@@ -172,10 +189,12 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
 
 // ---- inspection interface for tests --------------------------------------
 TK_API int tk_fake_launch_count(void) { return (int)g_launches.size(); }
-TK_API void tk_fake_reset(void) { g_launches.clear(); g_fail_next_launch = 0; }
+TK_API void tk_fake_reset(void) { g_launches.clear(); g_fail_next_launch = 0; g_event_queue.clear(); }
 TK_API void tk_fake_fail_next_launches(int n) { g_fail_next_launch = n; }
 TK_API void tk_fake_set_cu_count(int n) { g_cu_count = n; }
 TK_API void tk_fake_set_event_ms(float ms) { g_event_ms = ms; }
+TK_API void tk_fake_push_event_ms(const float *ms, int n) { g_event_queue.insert(g_event_queue.end(), ms, ms + n); }
+TK_API int tk_fake_event_queue_len(void) { return (int)g_event_queue.size(); }
 TK_API const char *tk_fake_launch_key(int i) { return g_launches[i].key.c_str(); }
 TK_API int tk_fake_launch_nargs(int i) { return (int)g_launches[i].args.size(); }
 TK_API void tk_fake_launch_dims(int i, unsigned out[6])

@@ -1,0 +1,113 @@
+"""GPU tests of the conv->GEMM helpers, the VGG16 latency-critical task and the
+TaskManager on the real device."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import tacker_amd as ta
+from gpu_util import dev, host, setup
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _init():
+    setup()
+
+
+@pytest.mark.parametrize("pad,stride,dil", [((1, 1), (1, 1), (1, 1)), ((0, 1), (2, 1), (1, 1)), ((2, 2), (1, 2), (2, 1))])
+def test_im2col_bit_exact(pad, stride, dil):
+    rng = np.random.default_rng(12)
+    im = rng.uniform(-1, 1, (5, 17, 19)).astype(np.float32)
+    want = oracle.im2col(im, (3, 3), pad, stride, dil)
+    col = torch.zeros(want.shape, device="cuda:0")
+    ta.im2col(dev(im), (3, 3), pad, stride, dil, col)
+    assert np.array_equal(host(col), want)
+
+
+def test_convert_fp32_to_fp16_rounds_to_nearest_even():
+    rng = np.random.default_rng(13)
+    x = np.concatenate([rng.uniform(-2, 2, 5000), rng.uniform(-1e-5, 1e-5, 1000), [0.0, 65504.0, 1e-8]]).astype(np.float32)
+    out = torch.zeros(x.size, dtype=torch.float16, device="cuda:0")
+    ta.convert_fp32_to_fp16(out, dev(x))
+    assert np.array_equal(host(out).view(np.uint16), x.astype(np.float16).view(np.uint16))
+
+
+def conv_reference(x_hwc, w, bias, C, Cout):
+    """relu(1.1 * conv3x3(f16(x), w) + bias) in float64; x [H][W][>=C], w f16 [Np][Kp], k = (kh*3+kw)*C + c."""
+    H, W = x_hwc.shape[:2]
+    xp = np.zeros((H + 2, W + 2, C))
+    xp[1:-1, 1:-1] = x_hwc[:, :, :C].astype(np.float16).astype(np.float64)
+    wk = w[:Cout, :9 * C].astype(np.float64).reshape(Cout, 3, 3, C)
+    out = np.zeros((H, W, Cout))
+    for kh in range(3):
+        for kw in range(3):
+            out += np.einsum("hwc,nc->hwn", xp[kh:kh + H, kw:kw + W], wk[:, kh, kw])
+    return np.maximum(float(np.float32(1.1)) * out + bias[:Cout].astype(np.float64), 0.0)
+
+
+def read_act(task, idx):
+    ptr, (H, W, C, ld) = task.activation(idx)
+    return ta.device_to_host(ptr, (H, W, ld), np.float32), C
+
+
+def test_vgg16_layers_match_direct_convolution():
+    task = ta.LcTask("vgg16", 32, 64)
+    task.execute()
+    torch.cuda.synchronize()
+    x = task.host_input().reshape(32, 64, 3)
+    prev, prevC = x, 3
+    for idx in range(4):                      # conv1_1, conv1_2, [pool], conv2_1, conv2_2
+        w, b = task.conv_params(idx)
+        got, Cout = read_act(task, idx)
+        if idx == 2:                          # a 2x2 max pool sits between conv1_2 and conv2_1
+            H, W = prev.shape[:2]
+            prev = prev.reshape(H // 2, 2, W // 2, 2, -1).max(axis=(1, 3))
+        want = conv_reference(prev, w, b, prevC, Cout)
+        np.testing.assert_allclose(got[:, :, :Cout], want, rtol=2e-4, atol=2e-4)
+        assert np.all(got[:, :, Cout:] == 0)  # padded channels stay zero
+        prev, prevC = got, Cout
+    # kernel list as the scheduler sees it
+    ks = task.kernels()
+    assert [k["mixable"] for k in ks].count(2) == 13 and [k["mixable"] for k in ks].count(1) == 3
+    task.close()
+
+
+def test_task_manager_colocation_keeps_lc_results_and_reports():
+    task = ta.LcTask("vgg16", 64, 64)
+    task.execute()
+    torch.cuda.synchronize()
+    p, stride, n = task.logits()
+    solo_logits = ta.device_to_host(p, (n, stride), np.float32)[:, 0].copy()
+    assert np.isfinite(solo_logits).all() and np.abs(solo_logits).max() > 0
+
+    tm = ta.TaskManager(task, "stencil", "lbm")
+    tm.configure(qos_budget_ms=50.0, guard_ms=0.5, warmup=1, profile=3, queries=4, verbose=0)
+    rep = tm.run("aker", second_stage=True)
+    torch.cuda.synchronize()
+    mixed_logits = ta.device_to_host(p, (n, stride), np.float32)[:, 0]
+    assert np.array_equal(mixed_logits, solo_logits)      # fused launches leave the LC numerics untouched
+    assert rep["mixable_times"] == 16 and rep["lc_solo_ms"] > 0 and rep["be1_solo_ms"] > 0
+    assert rep["n_colocated"] == 4 and rep["n_solo"] == 3
+    lat = tm.latencies()
+    assert len(lat) == 4 and all(0 < v < 50.0 for v in lat)
+    assert rep["qos_headroom_left_ms"] > 0
+    rep2 = tm.run("tacker", second_stage=False)
+    assert rep2["n_colocated"] == 4
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
+    tm.close()
+    task.close()
+
+
+def test_create_kernel_objects_run_and_match_oracle_for_cp():
+    k = ta.create_kernel("cp")
+    info = k.info()
+    assert (info["ptb_start"], info["ptb_end"]) == (0, 16384) and info["ori_grid_x"] == 32 and info["ori_grid_y"] == 512
+    k.execute()
+    torch.cuda.synchronize()
+    for name in ("stencil", "lbm", "mriq"):
+        ta.create_kernel(name).execute()
+    torch.cuda.synchronize()
+    assert ta.spin_fail_flag() == 0

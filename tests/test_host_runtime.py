@@ -1,0 +1,396 @@
+"""CPU tests of the host runtime (Kernel / GPTBKernel / MixKernel / Creator /
+TaskManager / json) over the recording fake device layer, plus the export check
+of both shared libraries.  No GPU, no compute calls."""
+import ctypes as C
+import os
+import re
+import struct
+
+import numpy as np
+import pytest
+
+import tacker_amd as ta
+
+HEADER = open(ta.HEADER_PATH).read()
+DECLARED = sorted(set(re.findall(r"TK_API\s+[\w\s\*]+?\b(\w+)\s*\(", HEADER)))
+
+
+@pytest.fixture(scope="module")
+def fake():
+    l = ta.load_library(ta.FAKE_LIB_PATH)
+    assert l.tacker_init(0, None) == 0
+    l.tk_fake_launch_key.restype = C.c_char_p
+    l.tk_fake_push_event_ms.argtypes = [C.POINTER(C.c_float), C.c_int]
+    l.tk_fake_set_event_ms.argtypes = [C.c_float]
+    l.tk_fake_symbol.argtypes = [C.c_char_p, C.c_void_p, C.c_int]
+    l.tk_fake_launch_arg.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_int]
+    l.tk_fake_launch_dims.argtypes = [C.c_int, C.POINTER(C.c_uint)]
+    return l
+
+
+def launches(l):
+    out = []
+    for i in range(l.tk_fake_launch_count()):
+        dims = (C.c_uint * 6)()
+        l.tk_fake_launch_dims(i, dims)
+        args = []
+        for a in range(l.tk_fake_launch_nargs(i)):
+            buf = C.create_string_buffer(8)
+            n = l.tk_fake_launch_arg(i, a, buf, 8)
+            args.append(buf.raw[:n])
+        out.append({"key": l.tk_fake_launch_key(i).decode(), "grid": tuple(dims[:3]), "block": tuple(dims[3:]),
+                    "args": args})
+    return out
+
+
+def as_int(b):
+    return struct.unpack("<i", b)[0]
+
+
+def as_float(b):
+    return struct.unpack("<f", b)[0]
+
+
+def as_ptr(b):
+    return struct.unpack("<Q", b)[0]
+
+
+# ------------------------------------------------------------------ exports
+def test_header_declares_something_and_both_libraries_export_all_of_it():
+    assert len(DECLARED) > 70
+    for path in (ta.LIB_PATH, ta.FAKE_LIB_PATH):
+        lib = C.CDLL(path)
+        missing = [n for n in DECLARED if not hasattr(lib, n)]
+        assert not missing, (path, missing)
+
+
+def test_product_library_does_not_link_the_oracle():
+    import subprocess
+    out = subprocess.run(["ldd", ta.LIB_PATH], capture_output=True, text=True).stdout
+    assert "oracle" not in out
+    syms = subprocess.run(["nm", "-D", ta.LIB_PATH], capture_output=True, text=True).stdout
+    assert "orc_" not in syms
+
+
+# ------------------------------------------------------------------ shape rule, kinfo
+def test_tzgemm_grid_dim_known_answers(fake):
+    out = (C.c_int * 4)()
+    for (m, n, k), want in [((128, 128, 27), [128, 128, 128, 4]), ((12800, 512, 4096), [12800, 512, 4096, 1600]),
+                            ((50176, 64, 576), [50176, 128, 512, 1568]), ((3136, 256, 1152), [3072, 256, 1152, 192]),
+                            ((1024, 1024, 1024), [1024, 1024, 1024, 256])]:
+        fake.tacker_tzgemm_grid_dim(m, n, k, out)
+        assert list(out) == want
+
+
+def test_kinfo_lookups_and_missing_keys(fake):
+    assert fake.tacker_get_kernel_info(b"tzgemm_stencil", b"blocksize") in (256, 512, 768, 1024)
+    assert fake.tacker_get_kernel_info(b"tzgemm_stencil", b"no_such_key") == ta.JSON_NOT_FOUND
+    assert fake.tacker_get_kernel_info(b"no_such_kernel", b"blocksize") == ta.JSON_NOT_FOUND
+    assert fake.tacker_fget_kernel_info(b"tzgemm_stencil", b"4096") > 0
+    assert fake.tacker_fget_kernel_info(b"nope", b"4096") == float(ta.JSON_NOT_FOUND)
+
+
+def test_block_ratio_table_and_k_extrapolation(fake):
+    r4096 = fake.tacker_fget_kernel_info(b"tzgemm_stencil", b"4096")
+    assert fake.tacker_qos_block_ratio(b"stencil", 4096) == pytest.approx(r4096)
+    assert fake.tacker_qos_block_ratio(b"stencil", 1152) == pytest.approx(
+        fake.tacker_fget_kernel_info(b"tzgemm_stencil", b"1152"))
+    # K absent from the table: the K=4096 entry scaled by K/4096 (src/TaskManager.cu:593-598)
+    assert fake.tacker_qos_block_ratio(b"stencil", 2048) == pytest.approx(r4096 * 2048 / 4096)
+    assert fake.tacker_qos_block_ratio(b"stencil", 8192) == pytest.approx(r4096 * 2)
+
+
+def test_colocated_blocks_aker_vs_tacker(fake):
+    ratio = fake.tacker_qos_block_ratio(b"stencil", 4608)
+    assert fake.tacker_qos_colocated_blocks(0, b"stencil", 96, 4608, 1024) == min(int(96 * ratio), 1024)
+    assert fake.tacker_qos_colocated_blocks(0, b"stencil", 100000, 4608, 1024) == 1024
+    assert fake.tacker_qos_colocated_blocks(1, b"stencil", 96, 4608, 1024) == 1024   # Tacker: everything
+
+
+# ------------------------------------------------------------------ QoS accounting (table driven)
+@pytest.mark.parametrize("mixable,measured,solo,be_ms,cd,total,want", [
+    (0, 9.0, 2.0, 10.0, 0, 100, (0, 2.0, 0.0)),          # not mixable: charged the profiled solo time
+    (2, 2.5, 2.0, 10.0, 10, 100, (1, 2.5, 0.5)),         # fused 2.5 < 2.0 + 10*10/100 = 3.0
+    (2, 3.5, 2.0, 10.0, 10, 100, (0, 2.0, 0.0)),         # fused slower than serial: modelled as "would not fuse"
+    (1, 3.0, 2.0, 10.0, 10, 100, (1, 3.0, 0.0)),         # equality counts as mixed (strict > in the reference)
+    (1, 1.0, 2.0, 4.0, 100, 100, (1, 1.0, 5.0)),
+])
+def test_qos_account_table(fake, mixable, measured, solo, be_ms, cd, total, want):
+    out = (C.c_float * 3)()
+    fake.tacker_qos_account(mixable, measured, solo, be_ms, cd, total, out)
+    assert (int(out[0]), out[1], out[2]) == pytest.approx(want)
+
+
+def test_qos_guard(fake):
+    # solo iff headroom < remaining LC time + guard (src/TaskManager.cu:586)
+    assert fake.tacker_qos_must_run_solo(50.0, 4.0, 10.0, 6.5) == 1
+    assert fake.tacker_qos_must_run_solo(50.0, 4.0, 10.5, 6.5) == 0
+    assert fake.tacker_qos_must_run_solo(50.0, 0.0, 6.5, 6.5) == 0
+
+
+# ------------------------------------------------------------------ marshalling
+def test_gptb_stencil_parameter_vector(fake):
+    fake.tk_fake_reset()
+    a0 = np.zeros((6, 10, 70), np.float32)
+    a1 = np.zeros_like(a0)
+    rc = fake.tacker_gptb_stencil(0.5, 0.25, a0.ctypes.data, a1.ctypes.data, 70, 10, 6, 2, 5, 24, 128, None)
+    assert rc == 0
+    (l,) = launches(fake)
+    # general_ptb_stencil(c0,c1,A0,Anext,nx,ny,nz, 6 dims, start,step,end, thread_base)
+    # src/gptb_kernel/stencil_kernel.cu:3-5
+    assert l["key"] == "gptb_stencil" and len(l["args"]) == 17
+    assert l["grid"] == (24, 1, 1) and l["block"] == (128, 1, 1)
+    a = l["args"]
+    assert (as_float(a[0]), as_float(a[1])) == (0.5, 0.25)
+    assert (as_ptr(a[2]), as_ptr(a[3])) == (a0.ctypes.data, a1.ctypes.data)
+    assert [as_int(x) for x in a[4:7]] == [70, 10, 6]
+    assert [as_int(x) for x in a[7:13]] == [2, 3, 1, 32, 4, 1]      # ori grid (ceil(70/64), ceil(10/4)), block (32,4)
+    assert [as_int(x) for x in a[13:17]] == [2, 24, 5, 0]           # start, step = launch grid, end, thread_base
+
+
+def test_mix_parameter_vector_matches_reference_signature(fake):
+    fake.tk_fake_reset()
+    a0 = np.zeros((6, 10, 70), np.float32)
+    a1 = np.zeros_like(a0)
+    A = np.zeros((256, 128), np.float16)
+    B = np.zeros((384, 128), np.float16)
+    Cm = np.zeros((256, 384), np.float32)
+    rc = fake.tacker_mix_tzgemm_stencil(0.5, 0.25, a0.ctypes.data, a1.ctypes.data, 70, 10, 6, 1, 4,
+                                        A.ctypes.data, B.ctypes.data, Cm.ctypes.data, 256, 384, 128, 3, 20,
+                                        b"wg_1_1", 0, 0, None)
+    assert rc == 0, fake.tacker_last_error()
+    (l,) = launches(fake)
+    # stencil_tzgemm_mix has 16 + 15 = 31 parameters (src/mix_kernel/tzgemm_stencil.cu:281-283):
+    # [stencil 7 + 6 dims + start,step,end][A,B,C,M,N,K + 6 dims + start,step,end]
+    assert l["key"] == "tzgemm_stencil@wg_1_1" and len(l["args"]) == 31
+    a = l["args"]
+    grid = l["grid"][0]
+    assert grid % 16 == 0 and l["block"] == (256, 1, 1)
+    assert [as_int(x) for x in a[7:13]] == [2, 3, 1, 32, 4, 1]
+    assert [as_int(x) for x in a[13:16]] == [1, grid, 4]            # start1, step = fused grid, end1
+    assert [as_ptr(x) for x in a[16:19]] == [A.ctypes.data, B.ctypes.data, Cm.ctypes.data]
+    assert [as_int(x) for x in a[19:22]] == [256, 384, 128]
+    assert [as_int(x) for x in a[22:28]] == [24, 1, 1, 256, 1, 1]   # tzgemm ori grid = tile count, block 256
+    assert [as_int(x) for x in a[28:31]] == [3, grid, 20]
+
+
+@pytest.mark.parametrize("be,n_be", [("lbm", 2), ("mriq", 7), ("cp", 3)])
+def test_other_mix_vectors_have_reference_lengths(fake, be, n_be):
+    fake.tk_fake_reset()
+    buf = np.zeros(1 << 16, np.float32)
+    A = np.zeros((128, 128), np.float16)
+    Cm = np.zeros((128, 128), np.float32)
+    g = [A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 128, 128, 128, 0, 4, None, 0, 0, None]
+    p = buf.ctypes.data
+    if be == "lbm":
+        rc = fake.tacker_mix_tzgemm_lbm(p, p, 8, 4, 4, 0, 16, *g)
+    elif be == "mriq":
+        rc = fake.tacker_mix_tzgemm_mriq(16, p, p, p, p, p, 512, 0, 2, *g)
+    else:
+        rc = fake.tacker_mix_tzgemm_cp(64, 0.1, p, 256, 16, 0, 4, *g)
+    assert rc == 0, fake.tacker_last_error()
+    (l,) = launches(fake)
+    # lbm_tzgemm_mix 11+15, mriq_tzgemm_mix 16+15, cp_tzgemm_mix 12+15
+    # (src/mix_kernel/tzgemm_{lbm,mriq,cp}.cu dispatcher signatures)
+    assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 15
+
+
+def test_gptb_vector_is_restored_after_launch_and_after_failure(fake):
+    fake.tk_fake_reset()
+    a0 = np.zeros((6, 10, 70), np.float32)
+    ori = fake.tacker_ori_stencil_create(0.5, 0.25, a0.ctypes.data, a0.ctypes.data, 70, 10, 6)
+    g = fake.tacker_gptb_create(ori, 8, 128, 0, 6)
+    info = (C.c_int * 8)()
+    fake.tacker_kernel_info(g, info)
+    assert info[4] == 13 and list(info[:4]) == [8, 128, 0, 6] and (info[6], info[7]) == (2, 3)
+    assert fake.tacker_kernel_execute(g, None) == 0
+    fake.tacker_kernel_info(g, info)
+    assert info[4] == 13                                  # start/step/end/thread_base popped again
+    fake.tk_fake_fail_next_launches(1)
+    rc = fake.tacker_kernel_execute(g, None)
+    # a failed launch surfaces as the runtime_error text of TK_SAFE_CALL: file, line, message
+    assert rc == 4 and b"GPTBKernel.h" in fake.tacker_last_error() and b"fake device error" in fake.tacker_last_error()
+    fake.tacker_kernel_info(g, info)
+    assert info[4] == 13
+    assert fake.tacker_kernel_execute(g, None) == 0       # still usable
+    assert len(launches(fake)[-1]["args"]) == 17
+    fake.tacker_kernel_destroy(g)
+    fake.tacker_kernel_destroy(ori)
+
+
+def test_mix_follows_ori_buffer_swap_but_not_gptb_range_edits(fake):
+    fake.tk_fake_reset()
+    a0 = np.zeros((6, 10, 70), np.float32)
+    a1 = np.zeros_like(a0)
+    A = np.zeros((128, 128), np.float16)
+    Cm = np.zeros((128, 128), np.float32)
+    st_ori = fake.tacker_ori_stencil_create(0.5, 0.25, a0.ctypes.data, a1.ctypes.data, 70, 10, 6)
+    st = fake.tacker_gptb_create(st_ori, 0, 0, 0, 6)
+    tz_ori = fake.tacker_ori_tzgemm_create(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 128, 128, 128)
+    tz = fake.tacker_gptb_create(tz_ori, 0, 0, 0, 4)
+    mix = fake.tacker_mix_create(st, tz, 0, 6, 0, 4, None, 0, 0)
+    assert mix, fake.tacker_last_error()
+    fake.tacker_kernel_execute(mix, None)
+    fake.tacker_kernel_swap_buffers(st_ori)               # parameter pointers alias the ori struct
+    fake.tacker_gptb_set_range(st, 2, 3)                  # the mix owns its own start/end ints
+    fake.tacker_kernel_execute(mix, None)
+    first, second = launches(fake)
+    assert [as_ptr(x) for x in first["args"][2:4]] == [a0.ctypes.data, a1.ctypes.data]
+    assert [as_ptr(x) for x in second["args"][2:4]] == [a1.ctypes.data, a0.ctypes.data]
+    assert [as_int(second["args"][13]), as_int(second["args"][15])] == [0, 6]
+    fake.tacker_mix_set_range(mix, 1, 2, 0, 4)
+    fake.tacker_kernel_execute(mix, None)
+    assert [as_int(launches(fake)[-1]["args"][13]), as_int(launches(fake)[-1]["args"][15])] == [1, 2]
+
+
+def test_argument_validation_returns_codes_instead_of_exiting(fake):
+    buf = np.zeros(1024, np.float32)
+    p = buf.ctypes.data
+    assert fake.tacker_gptb_tzgemm(p, p, p, 100, 128, 128, 0, 1, 0, None) == 3        # not a multiple of 128
+    assert fake.tacker_gptb_tzgemm(p, p, p, 128, 128, 128, 0, 5, 0, None) == 1        # range beyond the 4 tiles
+    assert fake.tacker_gptb_stencil(0.1, 0.1, p, p, 8, 8, 8, 0, 1, 4, 100, None) == 1  # block not a multiple of 64
+    assert fake.tacker_ori_mriq(8, p, p, p, p, p, 100, None) == 3
+    assert fake.tacker_ori_cp(65, 0.1, p, 128, 8, None) == 1
+    assert fake.tacker_mix_tzgemm_stencil(0.1, 0.1, p, p, 8, 8, 8, 0, 1, p, p, p, 128, 128, 128, 0, 4,
+                                          b"no_such_variant", 0, 0, None) == 2
+    assert not fake.tacker_create_kernel(b"no_such_kernel")
+    assert b"Kernel not found" in fake.tacker_last_error()
+    assert not fake.tacker_task_create(b"resnet50", 0, 0)
+
+
+def test_constant_tables_reach_the_device_layer(fake):
+    kv = np.arange(12, dtype=np.float32).reshape(3, 4)
+    assert fake.tacker_mriq_set_kvalues(kv.ctypes.data, 3) == 0
+    out = np.zeros(12, np.float32)
+    assert fake.tk_fake_symbol(b"ck", out.ctypes.data, 48) >= 48
+    assert np.array_equal(out, kv.reshape(-1))
+    atoms = np.array([[1, 2, 3, 0.5], [4, 5, -1, -0.25]], np.float32)
+    assert fake.tacker_cp_set_atoms(atoms.ctypes.data, 2, 1.0) == 0
+    out = np.zeros(8, np.float32)
+    fake.tk_fake_symbol(b"atominfo", out.ctypes.data, 32)
+    assert np.array_equal(out.reshape(2, 4), np.array([[1, 2, 4, 0.5], [4, 5, 4, -0.25]], np.float32))
+    assert fake.tacker_mriq_set_kvalues(kv.ctypes.data, 5000) == 1
+
+
+def test_create_kernel_geometry_and_memoisation(fake):
+    fake.tk_fake_set_cu_count(256)
+    k1 = fake.tacker_create_kernel(b"stencil")
+    k2 = fake.tacker_create_kernel(b"stencil")
+    assert k1 and k1 == k2
+    info = (C.c_int * 8)()
+    fake.tacker_kernel_info(k1, info)
+    per_cu = fake.tacker_get_kernel_info(b"stencil", b"solo_ptb_blks")
+    assert info[0] == 256 * per_cu and info[1] == fake.tacker_get_kernel_info(b"stencil", b"blocksize")
+    assert (info[2], info[3]) == (0, 1024) and (info[6], info[7]) == (8, 128)
+    fake.tk_fake_reset()
+    assert fake.tacker_kernel_execute(k1, None) == 0
+    assert launches(fake)[0]["key"] == "gptb_stencil"
+
+
+def test_host_half_conversion_matches_numpy():
+    lib = ta.load_library(ta.FAKE_LIB_PATH)
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([rng.uniform(-1, 1, 2000), rng.uniform(-7e4, 7e4, 200), rng.uniform(-1e-4, 1e-4, 500),
+                           rng.uniform(-1e-7, 1e-7, 500), [0.0, -0.0, 65504.0, 65520.0, 1e9, 5.96e-8, 2.98e-8,
+                                                           2.9802322e-08, 8.9406967e-08, 6.1035156e-05]]).astype(np.float32)
+    got = np.array([lib.tacker_float_to_half_bits(float(v)) for v in vals], np.uint16)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    assert np.array_equal(got, want)
+
+
+def test_rng_is_deterministic_and_uniform():
+    lib = ta.load_library(ta.FAKE_LIB_PATH)
+    a = np.zeros(100000, np.float32)
+    b = np.zeros(100000, np.float32)
+    lib.tacker_rng_uniform(1337, -1.0, 1.0, a.ctypes.data, a.size)
+    lib.tacker_rng_uniform(1337, -1.0, 1.0, b.ctypes.data, b.size)
+    assert np.array_equal(a, b) and a.min() >= -1 and a.max() < 1
+    assert abs(a.mean()) < 0.01 and abs(a.std() - 1 / np.sqrt(3)) < 0.01
+    lib.tacker_rng_uniform(1338, -1.0, 1.0, b.ctypes.data, b.size)
+    assert not np.array_equal(a, b)
+
+
+# ------------------------------------------------------------------ LC task + TaskManager
+@pytest.fixture(scope="module")
+def small_vgg(fake):
+    t = ta.LcTask("vgg16", 32, 32, library=fake)
+    yield t
+    t.close()
+
+
+def test_vgg16_task_structure(small_vgg):
+    ks = small_vgg.kernels()
+    convs = [k for k in ks if k["mixable"] == 2]
+    fcs = [k for k in ks if k["mixable"] == 1]
+    assert len(convs) == 13 and len(fcs) == 3 and len([k for k in ks if "MaxPool" in k["name"]]) == 5
+    assert convs[0]["args"] == [1, 3, 32, 32, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1]
+    assert convs[-1]["args"] == [1, 512, 2, 2, 512, 512, 3, 3, 1, 1, 1, 1, 1, 1]
+    assert [k["args"] for k in fcs] == [[4096, 128, 512], [4096, 128, 4096], [1024, 128, 4096]]
+    assert ta.LcTask.__init__  # keep the class referenced
+
+
+def test_vgg16_solo_pass_launches_every_layer(fake, small_vgg):
+    fake.tk_fake_reset()
+    small_vgg.execute(raw_stream=None)
+    keys = [l["key"] for l in launches(fake)]
+    assert keys.count("gptb_tzgemm") == 16 and keys.count("im2col_nhwc_f16") == 13
+    assert keys.count("maxpool2x2_nhwc") == 5 and keys.count("bias_relu_rows") == 13 and keys.count("pack_fc_input") == 3
+
+
+def run_manager(fake, task, durations=None, **cfg):
+    tm = ta.TaskManager(task, "stencil", "lbm", library=fake)
+    tm.configure(warmup=1, profile=2, verbose=0, **cfg)
+    fake.tk_fake_reset()
+    if durations is not None:
+        arr = (C.c_float * len(durations))(*durations)
+        fake.tk_fake_push_event_ms(arr, len(durations))
+    rep = tm.run("aker", raw_stream=None)
+    lat = tm.latencies()
+    tm.close()
+    return rep, lat
+
+
+def test_task_manager_fuses_when_budget_allows(fake, small_vgg):
+    fake.tk_fake_set_event_ms(0.01)      # every timed region "takes" 10 us
+    rep, lat = run_manager(fake, small_vgg, qos_budget_ms=50.0, guard_ms=4.0, queries=2)
+    n = len(small_vgg.kernels())
+    assert rep["mixable_times"] == 16 and rep["lc_solo_ms"] == pytest.approx(0.01 * n, rel=1e-4)
+    keys = [l["key"] for l in launches(fake)]
+    assert any(k.startswith("tzgemm_stencil") for k in keys)
+    assert len(lat) == 2 and lat[0] == pytest.approx(0.01 * n, rel=1e-4)
+    assert rep["qos_headroom_left_ms"] == pytest.approx(50.0 - 0.01 * n, rel=1e-3)
+    assert rep["mix_times"] > 0 and rep["be_blocks_executed"] > 0
+
+
+def test_task_manager_falls_back_to_solo_when_headroom_is_short(fake, small_vgg):
+    fake.tk_fake_set_event_ms(0.01)
+    n = len(small_vgg.kernels())
+    # budget below "rest of the query + guard" from the first kernel on: nothing may be fused
+    rep, lat = run_manager(fake, small_vgg, qos_budget_ms=0.01 * n + 1.0, guard_ms=4.0, queries=1)
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_")]
+    assert not fused and rep["mix_times"] == 0 and rep["be_blocks_executed"] == 0
+
+
+def test_task_manager_cursor_advances_and_wraps(fake, small_vgg):
+    fake.tk_fake_set_event_ms(0.01)
+    tm = ta.TaskManager(small_vgg, "stencil", None, library=fake)
+    tm.configure(warmup=0, profile=1, queries=3, verbose=0, qos_budget_ms=50.0, guard_ms=0.0)
+    fake.tk_fake_reset()
+    tm.run("tacker", raw_stream=None, second_stage=False)      # Tacker mode: the whole BE kernel per GEMM
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
+    assert len(fused) == 3 * 16
+    for l in fused:
+        assert (as_int(l["args"][13]), as_int(l["args"][15])) == (0, 1024)
+    assert tm.report()["be_task_finish_num"] == 48
+    tm.close()
+    tm = ta.TaskManager(small_vgg, "stencil", None, library=fake)
+    tm.configure(warmup=0, profile=1, queries=1, verbose=0, qos_budget_ms=50.0, guard_ms=0.0)
+    fake.tk_fake_reset()
+    tm.run("aker", raw_stream=None, second_stage=False)
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
+    ranges = [(as_int(l["args"][13]), as_int(l["args"][15])) for l in fused]
+    assert ranges and all(b > a for a, b in ranges)
+    for (a0, b0), (a1, b1) in zip(ranges, ranges[1:]):
+        assert a1 == b0 or a1 == 0           # each slice starts where the last one ended (or wrapped)
+    tm.close()
