@@ -1,0 +1,103 @@
+"""The fused-kernel generator: its candidate rule against the candidate lists and
+generated file names the reference ships, and the text it emits."""
+import itertools
+import json
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+GEN = os.path.join(ROOT, "tacker_amd", "fusion", "code")
+sys.path.insert(0, GEN)
+
+import data  # noqa: E402
+import gen_mix  # noqa: E402
+import gen_run  # noqa: E402
+import kernel_code  # noqa: E402
+
+FIX = json.load(open(os.path.join(ROOT, "tests", "golden", "generator_candidates.json")))
+T = data.REFERENCE_KERNEL_INFO
+
+
+def test_candidate_rule_reproduces_reference_log():
+    # fusion/code/log.txt: unreduced (n1, n2, blks) with summed register use
+    assert len(FIX["log"]) == 28
+    for key, want in FIX["log"].items():
+        a, b = key.split()
+        got = [[n1, n2, blks, *data.candidate_resources(a, b, (blks, n1, n2), T)]
+               for blks, n1, n2 in data.fuse_kernel_info(a, b, T, data.TURING_SM, reduce_gcd=False)]
+        assert got == want, key
+
+
+def test_candidate_rule_reproduces_reference_mix_kernel_info():
+    # fusion/code/mix_kernel_info.txt: both kernels as main in turn; the second
+    # direction skips ratios the first already produced; registers = max * threads
+    assert len(FIX["mix_kernel_info"]) == 42
+    for key, want in FIX["mix_kernel_info"].items():
+        a, b, main = key.split()
+        other = b if main == a else a
+        first = [(n1, n2) for _, n1, n2 in data.fuse_kernel_info(a, b, T, data.TURING_SM, reduce_gcd=False)]
+        got = []
+        for blks, n1, n2 in data.fuse_kernel_info(main, other, T, data.TURING_SM, reduce_gcd=False):
+            na, nb = (n1, n2) if main == a else (n2, n1)
+            if main == b and (na, nb) in first:
+                continue
+            _, smem, thr = data.candidate_resources(main, other, (blks, n1, n2), T)
+            got.append([na, nb, blks, max(T[a]["register"], T[b]["register"]) * thr, smem, thr])
+        assert got == want, key
+
+
+def test_generated_file_names_match_reference_mix_kernel_directory():
+    kernels = sorted(k for k in T if k != "tpacf")
+    names = set()
+    for a, b in itertools.combinations(kernels, 2):
+        names |= set(data.pair_file_names(a, b, T, data.TURING_SM))
+    assert sorted(names) == FIX["mix_kernel_files"] and len(names) == 143
+
+
+def test_cdna4_candidates_fit_one_compute_unit():
+    for be in gen_run.BE_KERNELS:
+        cands = data.fuse_kernel_info("tzgemm", be)
+        assert cands, be
+        for c in cands:
+            regs, lds, threads = data.candidate_resources("tzgemm", be, c)
+            assert regs <= data.CDNA4_CU.registers and lds <= data.CDNA4_CU.shared_memory
+            assert threads <= data.CDNA4_CU.thread_slots
+        for v in gen_run.pair_candidates(be):
+            if v[0] == "wave":
+                assert (256 + v[1]) % 64 == 0 and 256 + v[1] <= 1024
+
+
+def test_committed_generated_sources_are_fresh():
+    rc = subprocess.run([sys.executable, os.path.join(GEN, "gen_run.py"), "--check"], capture_output=True, text=True)
+    assert rc.returncode == 0, rc.stdout + rc.stderr
+
+
+@pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27)])
+def test_emitted_dispatcher_signature(be, n_params):
+    # parameter count = the reference dispatcher's (src/mix_kernel/tzgemm_<be>.cu), order: be first
+    text, meta = gen_mix.generate_wg_split(be, 1, 1)
+    sig = re.search(r"void (\w+)\(\s*(.*?)\)\s*\{", text, re.S)
+    params = [p.strip() for p in sig.group(2).split(",")]
+    assert len(params) == n_params and sig.group(1) == f"{be}_tzgemm_mix_wg_1_1"
+    names = [p.split()[-1] for p in params]
+    assert names[0].startswith(f"{be}0_") and names[-1] == "tzgemm1_ptb_end_block_pos"
+    assert names[-15:-12] == ["tzgemm1_A", "tzgemm1_B", "tzgemm1_C"]
+    assert names[-3:] == ["tzgemm1_ptb_start_block_pos", "tzgemm1_ptb_iter_block_step", "tzgemm1_ptb_end_block_pos"]
+    assert meta["blocksize"] == 256 and meta["group"] == 2
+    wave, wmeta = gen_mix.generate_wave_split(be, 256)
+    assert "RoleSpinSync" in wave and wave.count("__syncthreads()") == 1 and wmeta["blocksize"] == 512
+    assert f"(int)threadIdx.x - 256" in wave
+
+
+def test_kinfo_emitted_for_every_variant():
+    kinfo = json.load(open(os.path.join(ROOT, "tacker_amd", "config", "kinfo-gfx950.json")))
+    for be in gen_run.BE_KERNELS:
+        base = kinfo[f"tzgemm_{be}"]
+        assert {"gridsize", "blocksize", "variant", "block_ratio", "4096"} <= set(base)
+        assert f"tzgemm_{be}@{base['variant']}" in kinfo
+        assert {"register", "shared_memory", "blocksize", "solo_ptb_blks", "ori_blks"} <= set(kinfo[be])
+    assert set(kinfo["throughput_test"]) == {"a", "b"}

@@ -1,0 +1,71 @@
+"""Committed golden vectors (tests/golden/kernels_small.npz): the oracle must keep
+reproducing them (CPU), and the HIP path must match them (GPU)."""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+
+G = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kernels_small.npz"))
+C0, C1 = np.float32(1 / 6), np.float32(1 / 36)
+
+
+def test_oracle_reproduces_golden_vectors():
+    assert np.array_equal(oracle.tzgemm(G["gemm_A"], G["gemm_B"], f64=True), G["gemm_C64"])
+    assert np.array_equal(oracle.tzgemm(G["gemm_A"], G["gemm_B"]), G["gemm_C32"])
+    a, b = G["stencil_A0"].copy(), G["stencil_A0"].copy()
+    for _ in range(3):
+        b = oracle.stencil(C0, C1, a, b)
+        a, b = b, a
+    assert np.array_equal(a, G["stencil_after3"])
+    sx, sy, sz = (int(v) for v in G["lbm_dims"])
+    d1 = oracle.lbm(G["lbm_src"], G["lbm_src"].copy(), sx, sy, sz)
+    assert np.array_equal(d1, G["lbm_step1"])
+    assert np.array_equal(oracle.lbm(d1, G["lbm_src"].copy(), sx, sy, sz), G["lbm_step2"])
+    z = np.zeros(512, np.float32)
+    qr, qi = oracle.mriq(G["mriq_kvals"], *G["mriq_xyz"], z, z, f64=True)
+    assert np.array_equal(qr, G["mriq_Qr"]) and np.array_equal(qi, G["mriq_Qi"])
+    assert np.array_equal(oracle.cp_initatoms(70)[1:65], G["cp_atoms"])
+    assert np.array_equal(oracle.cp(oracle.cp_atoms_to_const(G["cp_atoms"], 0.0), np.zeros((16, 256), np.float32)),
+                          G["cp_grid"])
+    assert np.array_equal(oracle.im2col(G["im2col_im"], (3, 3), (1, 1), (1, 1)), G["im2col_col"])
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_golden_vectors():
+    import torch
+    import tacker_amd as ta
+    from gpu_util import dev, host, setup
+    setup()
+    Cd = torch.zeros((128, 256), device="cuda:0")
+    ta.gptb_tzgemm(dev(G["gemm_A"]), dev(G["gemm_B"]), Cd)
+    d = np.abs(host(Cd).astype(np.float64) - G["gemm_C64"])
+    assert np.all(d <= 5e-3 + 1e-5 * np.abs(G["gemm_C64"]))
+    a, b = dev(G["stencil_A0"]), dev(G["stencil_A0"])
+    for _ in range(3):
+        ta.gptb_stencil(float(C0), float(C1), a, b)
+        a, b = b, a
+    assert np.array_equal(host(a), G["stencil_after3"])
+    sx, sy, sz = (int(v) for v in G["lbm_dims"])
+    s, d1, d2 = dev(G["lbm_src"]), dev(G["lbm_src"]), dev(G["lbm_src"])
+    ta.gptb_lbm(s, d1, sx, sy, sz)
+    ta.gptb_lbm(d1, d2, sx, sy, sz)
+    assert np.array_equal(host(d1).view(np.uint32), G["lbm_step1"].view(np.uint32))
+    assert np.array_equal(host(d2).view(np.uint32), G["lbm_step2"].view(np.uint32))
+    pm = torch.zeros(96, device="cuda:0")
+    ta.mriq_phimag(dev(G["mriq_phiR"]), dev(G["mriq_phiI"]), pm)
+    assert np.array_equal(host(pm), G["mriq_kvals"][:, 3])
+    ta.mriq_set_kvalues(G["mriq_kvals"])
+    Qr, Qi = torch.zeros(512, device="cuda:0"), torch.zeros(512, device="cuda:0")
+    x, y, z = (dev(v) for v in G["mriq_xyz"])
+    ta.gptb_mriq(96, x, y, z, Qr, Qi)
+    for got, want in ((host(Qr), G["mriq_Qr"]), (host(Qi), G["mriq_Qi"])):
+        assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-3 + 1e-4 * np.abs(want))
+    ta.cp_set_atoms(G["cp_atoms"], 0.0)
+    g = torch.zeros((16, 256), device="cuda:0")
+    ta.gptb_cp(64, 0.1, g)
+    assert np.array_equal(host(g).view(np.uint32), G["cp_grid"].view(np.uint32))
+    col = torch.zeros(G["im2col_col"].shape, device="cuda:0")
+    ta.im2col(dev(G["im2col_im"]), (3, 3), (1, 1), (1, 1), (1, 1), col)
+    assert np.array_equal(host(col), G["im2col_col"])
