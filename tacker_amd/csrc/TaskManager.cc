@@ -64,7 +64,7 @@ static void launchMixedGemm(int M_INPUT, int N_INPUT, int K_INPUT, GPTBKernel *g
 {
     const std::vector<int> d = getTZGEMMGridDim(M_INPUT, N_INPUT, K_INPUT);
     OriTZGEMMKernel ori_tzgemm(0, d[0], d[1], d[2]);
-    GPTBKernel gptb_tzgemm_kernel(1, "tzgemm", "gptb_tzgemm", &ori_tzgemm, dim3(cuCount() * 2, 1, 1),
+    GPTBKernel gptb_tzgemm_kernel(1, "tzgemm", "gptb_tzgemm", &ori_tzgemm, dim3(cuCount(), 1, 1),
                                   dim3(TZ_THREADS, 1, 1), 0, d[3]);
     if (cd_end_blk <= cd_start_blk) {   // nothing to co-locate: the GEMM alone
         gptb_tzgemm_kernel.execute(stream);

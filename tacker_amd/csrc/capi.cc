@@ -61,8 +61,8 @@ int default_grid(const std::string &name)
 
 int check_block(const std::string &name, int block)
 {
-    if (block <= 0 || block % 64 || block > 1024)
-        return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 64 in [64,1024]");
+    if (block <= 0 || block % 64 || block > 256)
+        return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 64 in [64,256]");
     if (name == "tzgemm" && block != TZ_THREADS)
         return fail(TK_ERROR_INVALID_VALUE, "tzgemm: launch_block must be 256");
     if (name == "mriq" && block % 256)

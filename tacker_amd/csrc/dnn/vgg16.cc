@@ -66,7 +66,7 @@ public:
         this->kernelName = name;
         ori_.reset(new OriTZGEMMKernel(id, M, N, K, A, B, C));
         tiles_ = getTZGEMMGridDim(M, N, K)[3];
-        gptb_.reset(new GPTBKernel(id, "tzgemm", "gptb_tzgemm", ori_.get(), dim3(cuCount() * 2, 1, 1),
+        gptb_.reset(new GPTBKernel(id, "tzgemm", "gptb_tzgemm", ori_.get(), dim3(cuCount(), 1, 1),
                                    dim3(TZ_THREADS, 1, 1), 0, tiles_));
     }
     std::vector<int> gemmDims() const override { return {M_, N_, K_}; }

@@ -3,7 +3,8 @@
 // from 16x16x16 WMMA fragments by 4 warps of 32.  Its tile is kept as the unit
 // of the [start,end) range interface (TZ_REF_TILE); the gfx950 kernel computes a
 // 128x128 macro tile (2x2 reference tiles) per 256-thread workgroup with
-// v_mfma_f32_16x16x32_f16, one reference tile per 64-wide wavefront.
+// v_mfma_f32_16x16x32_f16, one reference tile per 64-wide wavefront, fed by a
+// ring of LDS stages that the global loads fill directly (no register staging).
 #pragma once
 #include "pets_common.h"
 
@@ -13,9 +14,11 @@
 #define TZ_MFMA_M 16
 #define TZ_MFMA_N 16
 #define TZ_MFMA_K 32
-#define TZ_BLOCK_K 32             // K extent staged in LDS per stage
-#define TZ_LDS_ROW_BYTES (TZ_BLOCK_K * 2 + 16)   // 16 B skew against bank conflicts
-#define TZ_LDS_STAGES 2
-#define TZ_LDS_BYTES (TZ_LDS_STAGES * 2 * TZ_MACRO_TILE * TZ_LDS_ROW_BYTES)
+#define TZ_BLOCK_K 64             // K extent of one LDS stage (128-byte tile rows)
+#define TZ_STAGE_BYTES (2 * TZ_MACRO_TILE * TZ_BLOCK_K * 2)   // A rows then B rows: 32 KiB
+#define TZ_STAGES 4               // LDS ring depth where the GEMM has the CU's LDS to itself
+#define TZ_STAGES_WG 3            // ring depth of workgroup-split fused kernels
+#define TZ_LDS_BYTES (TZ_STAGES * TZ_STAGE_BYTES)
+#define TZ_LDS_BYTES_WG (TZ_STAGES_WG * TZ_STAGE_BYTES)
 
 #define TZ_ALPHA 1.1f             // alpha_g, src/header/tzgemm_header.h:64

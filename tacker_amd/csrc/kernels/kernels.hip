@@ -74,17 +74,17 @@ extern "C" __global__ __launch_bounds__(128) void ori_cp(int numatoms, float gri
 
 // ------------------------------------------------------------------ GPTB kernels
 
-extern "C" __global__ __launch_bounds__(TZ_THREADS) void general_ptb_tzgemm(
+extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void general_ptb_tzgemm(
     _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, GPTB_TRAILER)
 {
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
     tk::WorkgroupSync sync;
-    tk::tzgemm_role(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x, ptb_iter_block_step,
+    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x, ptb_iter_block_step,
                     ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base, tz_lds,
                     sync);
 }
 
-extern "C" __global__ void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
+extern "C" __global__ __launch_bounds__(256) void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
                                                int ny, int nz, GPTB_TRAILER)
 {
     tk::stencil_role(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y,

@@ -23,8 +23,16 @@ typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
 
 // Barrier among all threads of a workgroup: usable when the role owns every wave
 // of the workgroup (plain GPTB kernels and workgroup-split fused kernels).
+// Only LDS traffic is ordered (s_waitcnt lgkmcnt(0)); global loads in flight are
+// deliberately left in flight -- the GEMM role keeps several chunks of
+// LDS-direct loads outstanding across its barriers and tracks them itself.
 struct WorkgroupSync {
-    __device__ __forceinline__ void sync() { __syncthreads(); }
+    __device__ __forceinline__ void sync()
+    {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    }
 };
 
 // Barrier among the waves of ONE role inside a workgroup that also hosts
@@ -47,7 +55,7 @@ struct RoleSpinSync {
         : counter(c), waves(w), expected(0), fail(f), spin_limit(limit) {}
     __device__ __forceinline__ void sync()
     {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // LDS reads/writes of this wave are done
         expected += waves;
         if ((threadIdx.x & (TK_WAVE_SIZE - 1)) == 0)
             __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -60,7 +68,7 @@ struct RoleSpinSync {
                 break;
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+        asm volatile("" ::: "memory");
     }
 };
 

@@ -26,38 +26,43 @@
 
 namespace tk {
 
-// One run: x = x0 + lane, rows j0 .. j0+ROWS-1, centre planes k_first ..
+// One run of a wave: x = x0 + lane, rows j0 .. j0+ROWS-1, centre planes k_first ..
 // k_first+nplanes-1 with 1 <= nplanes <= Z (and k_first+nplanes-1 <= nz-2).
+// issue() starts every load of the run; finish() computes and stores.  Keeping the
+// two apart lets a wave issue the loads of its next run before it computes the
+// current one, so its memory pipeline never drains.
 template <int ROWS, int Z>
-__device__ __forceinline__ void stencil_wave_run(float c0, float c1, const float *__restrict__ A0,
-                                                 float *__restrict__ Anext, int nx, int ny,
-                                                 int k_first, int nplanes, int x0, int j0, int lane)
-{
+struct StencilRun {
     static_assert(ROWS * Z <= 32, "the edge gather gives each half-wave one value per (row, plane)");
-    const int x = x0 + lane;
-    const size_t plane = (size_t)nx * (size_t)ny;
-    const bool xin = x < nx;
-    const float *col = A0 + (size_t)x + (size_t)nx * j0 + plane * (k_first - 1);
+    float own[Z + 2][ROWS];   // planes k_first-1 .. k_first+nplanes
+    float dn[Z], up[Z];       // rows j0-1 and j0+ROWS of the centre planes
+    float edge;               // gathered: columns x0-1 (lanes 0..31) and x0+64 (lanes 32..63)
+    int k_first, nplanes, x0, j0;
 
-    // own rows: planes k_first-1 .. k_first+nplanes
-    float own[Z + 2][ROWS];
-#pragma unroll
-    for (int p = 0; p < Z + 2; ++p)
-#pragma unroll
-        for (int r = 0; r < ROWS; ++r)
-            own[p][r] = (xin && (j0 + r) < ny && p <= nplanes + 1) ? col[plane * p + (size_t)nx * r] : 0.f;
-    // rows below (j0-1) and above (j0+ROWS) the block, centre planes only
-    float dn[Z], up[Z];
-    const bool halo_dn = xin && j0 > 0;
-    const bool halo_up = xin && (j0 + ROWS) < ny;
-#pragma unroll
-    for (int p = 0; p < Z; ++p) {
-        dn[p] = (halo_dn && p < nplanes) ? col[plane * (p + 1) - (size_t)nx] : 0.f;
-        up[p] = (halo_up && p < nplanes) ? col[plane * (p + 1) + (size_t)nx * ROWS] : 0.f;
-    }
-    // columns left (x0-1) and right (x0+64) of the wave: one gathered load
-    float edge = 0.f;
+    __device__ __forceinline__ void issue(const float *__restrict__ A0, int nx, int ny, int k_first_,
+                                          int nplanes_, int x0_, int j0_, int lane)
     {
+        k_first = k_first_;
+        nplanes = nplanes_;
+        x0 = x0_;
+        j0 = j0_;
+        const int x = x0 + lane;
+        const size_t plane = (size_t)nx * (size_t)ny;
+        const bool xin = x < nx;
+        const float *col = A0 + (size_t)x + (size_t)nx * j0 + plane * (k_first - 1);
+#pragma unroll
+        for (int p = 0; p < Z + 2; ++p)
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r)
+                own[p][r] = (xin && (j0 + r) < ny && p <= nplanes + 1) ? col[plane * p + (size_t)nx * r] : 0.f;
+        const bool halo_dn = xin && j0 > 0;
+        const bool halo_up = xin && (j0 + ROWS) < ny;
+#pragma unroll
+        for (int p = 0; p < Z; ++p) {
+            dn[p] = (halo_dn && p < nplanes) ? col[plane * (p + 1) - (size_t)nx] : 0.f;
+            up[p] = (halo_up && p < nplanes) ? col[plane * (p + 1) + (size_t)nx * ROWS] : 0.f;
+        }
+        edge = 0.f;
         const int side = lane >> 5;
         const int idx = lane & 31;
         const int er = idx / Z, ep = idx % Z;
@@ -66,36 +71,52 @@ __device__ __forceinline__ void stencil_wave_run(float c0, float c1, const float
             edge = A0[(size_t)ex + (size_t)nx * (j0 + er) + plane * (k_first + ep)];
     }
 
-    bool win[ROWS];
-#pragma unroll
-    for (int r = 0; r < ROWS; ++r) {
-        const int j = j0 + r;
-        win[r] = x > 0 && x < nx - 1 && j > 0 && j < ny - 1;
-    }
-    float *out = Anext + (size_t)x + (size_t)nx * j0 + plane * k_first;
-#pragma unroll
-    for (int p = 0; p < Z; ++p) {
+    __device__ __forceinline__ void finish(float c0, float c1, float *__restrict__ Anext, int nx, int ny,
+                                           int lane) const
+    {
+        const int x = x0 + lane;
+        const size_t plane = (size_t)nx * (size_t)ny;
+        bool win[ROWS];
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            const float centre = own[p + 1][r];
-            float left = __shfl_up(centre, 1, 64);
-            float right = __shfl_down(centre, 1, 64);
-            const float edge_l = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge), r * Z + p));
-            const float edge_r = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge), 32 + r * Z + p));
-            if (lane == 0) left = edge_l;
-            if (lane == 63) right = edge_r;
-            const float a_up = (r + 1 < ROWS) ? own[p + 1][(r + 1 < ROWS) ? r + 1 : r] : up[p];
-            const float a_dn = (r > 0) ? own[p + 1][(r > 0) ? r - 1 : r] : dn[p];
-            if (win[r] && p < nplanes) {
-                float s = own[p + 2][r] + own[p][r];   // top + bottom
-                s = s + a_up;
-                s = s + a_dn;
-                s = s + right;
-                s = s + left;
-                out[plane * p + (size_t)nx * r] = s * c1 - centre * c0;
+            const int j = j0 + r;
+            win[r] = x > 0 && x < nx - 1 && j > 0 && j < ny - 1;
+        }
+        float *out = Anext + (size_t)x + (size_t)nx * j0 + plane * k_first;
+#pragma unroll
+        for (int p = 0; p < Z; ++p) {
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                const float centre = own[p + 1][r];
+                float left = __shfl_up(centre, 1, 64);
+                float right = __shfl_down(centre, 1, 64);
+                const float edge_l = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge), r * Z + p));
+                const float edge_r = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge), 32 + r * Z + p));
+                if (lane == 0) left = edge_l;
+                if (lane == 63) right = edge_r;
+                const float a_up = (r + 1 < ROWS) ? own[p + 1][(r + 1 < ROWS) ? r + 1 : r] : up[p];
+                const float a_dn = (r > 0) ? own[p + 1][(r > 0) ? r - 1 : r] : dn[p];
+                if (win[r] && p < nplanes) {
+                    float s = own[p + 2][r] + own[p][r];   // top + bottom
+                    s = s + a_up;
+                    s = s + a_dn;
+                    s = s + right;
+                    s = s + left;
+                    out[plane * p + (size_t)nx * r] = s * c1 - centre * c0;
+                }
             }
         }
     }
+};
+
+template <int ROWS, int Z>
+__device__ __forceinline__ void stencil_wave_run(float c0, float c1, const float *__restrict__ A0,
+                                                 float *__restrict__ Anext, int nx, int ny,
+                                                 int k_first, int nplanes, int x0, int j0, int lane)
+{
+    StencilRun<ROWS, Z> run;
+    run.issue(A0, nx, ny, k_first, nplanes, x0, j0, lane);
+    run.finish(c0, c1, Anext, nx, ny, lane);
 }
 
 // GPTB form.  The unit of work of a wave is one reference block cut into runs of
@@ -120,15 +141,30 @@ __device__ __forceinline__ void stencil_role(float c0, float c1, const float *__
     const unsigned runs = (unsigned)(planes + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
     const unsigned tasks = (unsigned)(end - start) * runs;
     const unsigned stride = (unsigned)role_blocks * waves;
-    for (unsigned t = (unsigned)role_block * waves + wave; t < tasks; t += stride) {
+    // two runs in flight per wave: the loads of run n+1 are issued before run n is computed
+    StencilRun<STENCIL_TILE_Y, STENCIL_Z_RUN> ra, rb;
+    auto start_run = [&](StencilRun<STENCIL_TILE_Y, STENCIL_Z_RUN> &r, unsigned t) {
         const unsigned pos = (unsigned)start + t / runs;
         const int run = (int)(t % runs);
         const int bx = pos % grid_dimension_x;
         const int by = (pos / grid_dimension_x) % grid_dimension_y;
         const int k_first = 1 + run * STENCIL_Z_RUN;
-        const int nplanes = min(STENCIL_Z_RUN, nz - 1 - k_first);
-        stencil_wave_run<STENCIL_TILE_Y, STENCIL_Z_RUN>(c0, c1, A0, Anext, nx, ny, k_first, nplanes,
-                                                        bx * 2 * STENCIL_TILE_X, by * STENCIL_TILE_Y, lane);
+        r.issue(A0, nx, ny, k_first, min(STENCIL_Z_RUN, nz - 1 - k_first), bx * 2 * STENCIL_TILE_X,
+                by * STENCIL_TILE_Y, lane);
+    };
+    unsigned t = (unsigned)role_block * waves + wave;
+    if (t >= tasks) return;
+    start_run(ra, t);
+    for (;;) {
+        const bool more_b = t + stride < tasks;
+        if (more_b) start_run(rb, t + stride);
+        ra.finish(c0, c1, Anext, nx, ny, lane);
+        if (!more_b) break;
+        const bool more_a = t + 2 * stride < tasks;
+        if (more_a) start_run(ra, t + 2 * stride);
+        rb.finish(c0, c1, Anext, nx, ny, lane);
+        if (!more_a) break;
+        t += 2 * stride;
     }
 }
 

@@ -8,16 +8,28 @@
 // (tile_i = pos / (N/64), tile_j = pos % (N/64), :54-56), and exactly those tiles
 // are written.
 //
-// gfx950 design: a 256-thread role (4 wave64) owns a 128x128 macro tile = 2x2
+// gfx950 design.  A 256-thread role (4 wave64) owns a 128x128 macro tile = 2x2
 // reference tiles; wave (wr,wc) computes reference tile (2*mi+wr, 2*mj+wc) with
-// 4x4 v_mfma_f32_16x16x32_f16 accumulators (64 VGPRs).  A and B both have K
-// contiguous, which is the operand layout MFMA wants (lane l supplies 8
-// consecutive k of row l%16), so tiles are staged to LDS as-is, 16 B per lane,
-// rows skewed by 16 B, and read back with one ds_read_b128 per fragment.  Two
-// LDS stages: global loads of chunk k+1 are issued before the MFMAs of chunk k
-// and written to the other stage afterwards, one barrier per chunk.  The MFMA is
-// issued with the operands swapped (B fragment first) so each lane ends up with
-// 4 consecutive columns of one row of C and stores them as one 16-byte word.
+// 4x4 v_mfma_f32_16x16x32_f16 accumulators.  A and B both have K contiguous,
+// which is the operand layout MFMA wants (lane l supplies 8 consecutive k of row
+// l%16), so tiles go to LDS as they are.
+//
+// Two things keep the MFMA pipe fed with one GEMM wave per SIMD:
+//  * global latency -- the K loop is a ring of STAGES LDS stages (64 k each,
+//    32 KiB) filled by global_load_lds_dwordx4: the load writes LDS directly,
+//    costs no VGPRs, and STAGES-1 chunks are in flight while one is multiplied.
+//    A wave knows its loads of a chunk have landed from the vmcnt counter
+//    (s_waitcnt vmcnt(8*(STAGES-2))), then one role barrier publishes the chunk.
+//  * LDS latency -- fragments are double-buffered in registers: the 8
+//    ds_read_b128 of the next k-step are issued before the 16 MFMAs of the current
+//    one, so the wave never sits idle between its LDS reads and its MFMAs.
+// An LDS-direct load puts lane l's 16 bytes at base + 16*l, so tile rows are dense
+// (128 B); bank conflicts are avoided by a swizzle applied on the global side:
+// LDS slot (row, s) holds the row's 16-byte segment s ^ ((row >> 1) & 7), and the
+// fragment read undoes it.
+//
+// The MFMA is issued with the operands swapped (B fragment first) so each lane
+// ends up with 4 consecutive columns of one row of C and stores 16 bytes at once.
 // A wave stores its tile only if the tile's position is inside the range; macro
 // tiles with no position in range are skipped by the whole workgroup.
 #pragma once
@@ -26,30 +38,45 @@
 
 namespace tk {
 
-// Persistent-loop index -> macro tile.  With role_blocks a multiple of 8, loop
-// index t runs on XCD t % 8; giving each XCD a contiguous run of macro tiles
-// keeps the A row panels and B column panels it re-reads inside its own L2.
-__device__ __forceinline__ int tz_macro_tile_of(int t, int n_macro)
+// Persistent-loop index -> macro tile (row, column).  With role_blocks a multiple
+// of 8, loop index t runs on XCD t % 8.  Each XCD takes a contiguous run of the
+// tile sequence, and the sequence walks the tile grid in bands of 4 tile rows,
+// column by column, so the ~32 tiles an XCD works on at the same time form a
+// compact 4 x 8 block: they share 4 A row panels and 8 B column panels inside
+// that XCD's L2 instead of streaming a whole operand through it.
+__device__ __forceinline__ void tz_macro_tile_of(int t, int macro_rows, int macro_cols, int &mi, int &mj)
 {
-    if (n_macro % TK_XCD_NUM == 0)
-        return (t % TK_XCD_NUM) * (n_macro / TK_XCD_NUM) + t / TK_XCD_NUM;
-    return t;
+    const int n_macro = macro_rows * macro_cols;
+    int seq = t;
+    if (n_macro % TK_XCD_NUM == 0) seq = (t % TK_XCD_NUM) * (n_macro / TK_XCD_NUM) + t / TK_XCD_NUM;
+    const int band = (macro_rows % 4 == 0) ? 4 : ((macro_rows % 2 == 0) ? 2 : 1);
+    const int per_band = band * macro_cols;
+    const int in_band = seq % per_band;
+    mi = (seq / per_band) * band + in_band % band;
+    mj = in_band / band;
 }
 
-template <class Sync>
+// s_waitcnt immediate that waits for vmcnt <= n and leaves expcnt / lgkmcnt alone
+#define TK_VMCNT_IMM(n) (((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+// s_waitcnt immediate that waits for lgkmcnt == 0 (LDS reads landed) and nothing else
+#define TK_LGKMCNT0_IMM 0xC07F
+
+template <int STAGES, class Sync>
 __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
                                             const _Float16 *__restrict__ B, float *__restrict__ C,
                                             int M, int N, int K, int role_block, int role_blocks,
                                             int tile_start, int tile_end, int tid, char *lds,
                                             Sync &sync)
 {
+    typedef __attribute__((address_space(1))) const void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int BK = TZ_BLOCK_K;
-    constexpr int ROWB = TZ_LDS_ROW_BYTES;
-    constexpr int SEGS_PER_ROW = BK / 8;                          // 16-byte segments per tile row
-    constexpr int SEGS_PER_THREAD = TZ_MACRO_TILE * SEGS_PER_ROW / TZ_THREADS;
-    constexpr int OPERAND_BYTES = TZ_MACRO_TILE * ROWB;
-    constexpr int STAGE_BYTES = 2 * OPERAND_BYTES;
-    constexpr int KSTEPS = BK / TZ_MFMA_K;
+    constexpr int ROWB = BK * 2;                         // dense 128-byte tile rows
+    constexpr int OPERAND_BYTES = TZ_MACRO_TILE * ROWB;  // 16 KiB
+    constexpr int STAGE_BYTES = TZ_STAGE_BYTES;
+    constexpr int LOADS = 4;                             // LDS-direct loads per wave, operand and chunk
+    constexpr int LOADS_PER_CHUNK = 2 * LOADS;
+    static_assert(STAGES >= 3 && LOADS_PER_CHUNK * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
 
     const int lane = tid & 63;
     const int wave = tid >> 6;
@@ -60,14 +87,25 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
     const int n_macro = (M / TZ_MACRO_TILE) * macro_cols;
     const int kchunks = K / BK;
 
-    // fragment read offsets (bytes inside an operand's stage area)
-    const int frag_a = (wr * 64 + (lane & 15)) * ROWB + (lane >> 4) * 16;
-    const int frag_b = (wc * 64 + (lane & 15)) * ROWB + (lane >> 4) * 16;
+    // LDS-direct load map.  Load j (0..3) of this wave fills rows (4*wave+j)*8 ..+7 of an
+    // operand's stage area; lane l lands in row +l/8, slot l%8, and therefore fetches the
+    // row's segment slot ^ ((row>>1)&7).  Rows of consecutive loads are 8 apart, which flips
+    // bit 2 of the key: odd loads fetch segment (seg ^ 4).
+    const int dma_row = 4 * wave * 8 + (lane >> 3);
+    const int dma_seg = (lane & 7) ^ ((dma_row >> 1) & 7);
+    const size_t src_off = (size_t)dma_row * K;                 // + j*8*K + segment per load
+    const int dst_off = 4 * wave * 1024;                        // + j*1024 per load
+    // fragment reads: row r = lane%16 of a 16-row group (its swizzle key (r>>1)&7 is the
+    // same in every group), k segment 4*kstep + lane/16 of the 8 in a row
+    const int frag_key = ((lane & 15) >> 1) & 7;
+    const int frag_seg0 = ((lane >> 4) ^ frag_key) * 16;
+    const int frag_seg1 = ((4 + (lane >> 4)) ^ frag_key) * 16;
+    const int frag_a = (wr * 64 + (lane & 15)) * ROWB;
+    const int frag_b = OPERAND_BYTES + (wc * 64 + (lane & 15)) * ROWB;
 
     for (int t = role_block; t < n_macro; t += role_blocks) {
-        const int mt = tz_macro_tile_of(t, n_macro);
-        const int mi = mt / macro_cols;
-        const int mj = mt % macro_cols;
+        int mi, mj;
+        tz_macro_tile_of(t, M / TZ_MACRO_TILE, macro_cols, mi, mj);
         const int pos00 = (2 * mi) * ref_cols + 2 * mj;
         const int pos10 = pos00 + ref_cols;
         const bool in00 = pos00 >= tile_start && pos00 < tile_end;
@@ -77,8 +115,28 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
         if (!(in00 || in01 || in10 || in11)) continue;   // uniform over the workgroup
         const bool store = wr ? (wc ? in11 : in10) : (wc ? in01 : in00);
 
-        const _Float16 *a_tile = A + (size_t)(mi * TZ_MACRO_TILE) * K;
-        const _Float16 *b_tile = B + (size_t)(mj * TZ_MACRO_TILE) * K;
+        const _Float16 *a_tile = A + (size_t)(mi * TZ_MACRO_TILE) * K + src_off;
+        const _Float16 *b_tile = B + (size_t)(mj * TZ_MACRO_TILE) * K + src_off;
+
+#define TZ_ISSUE_CHUNK(chunk_, stage_)                                                            \
+    _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                             \
+    {                                                                                             \
+        char *dst_ = lds + (stage_) * STAGE_BYTES + dst_off + j * 1024;                           \
+        const size_t src_ = (size_t)(j * 8) * K + (size_t)(chunk_) * BK + (dma_seg ^ ((j & 1) * 4)) * 8; \
+        __builtin_amdgcn_global_load_lds((gptr_t)(a_tile + src_), (lptr_t)dst_, 16, 0, 0);        \
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_tile + src_), (lptr_t)(dst_ + OPERAND_BYTES), \
+                                         16, 0, 0);                                               \
+    }
+#define TZ_READ_FRAGS(fa_, fb_, stage_, seg_)                                                     \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                 \
+    {                                                                                             \
+        const char *s_ = lds + (stage_) * STAGE_BYTES + i * 16 * ROWB + (seg_);                   \
+        fa_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_a);                                 \
+        fb_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_b);                                 \
+    }
+#define TZ_MFMAS(fa_, fb_)                                                                        \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)   \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[j], fa_[i], acc[i][j], 0, 0, 0);
 
         float4_t acc[4][4];
 #pragma unroll
@@ -86,55 +144,59 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-        // This thread stages 16-byte segment s = tid + p*256 of each operand tile:
-        // row s / SEGS_PER_ROW, 16-byte column s % SEGS_PER_ROW.
-        uint4_t ga[SEGS_PER_THREAD], gb[SEGS_PER_THREAD];
-#define TZ_LOAD_GLOBAL(kc_)                                                                   \
-    _Pragma("unroll") for (int p = 0; p < SEGS_PER_THREAD; ++p)                               \
-    {                                                                                         \
-        const int s_ = tid + p * TZ_THREADS;                                                  \
-        const size_t off_ = (size_t)(s_ / SEGS_PER_ROW) * K + (size_t)(kc_) * BK +            \
-                            (s_ % SEGS_PER_ROW) * 8;                                          \
-        ga[p] = *reinterpret_cast<const uint4_t *>(a_tile + off_);                            \
-        gb[p] = *reinterpret_cast<const uint4_t *>(b_tile + off_);                            \
-    }
-#define TZ_STORE_LDS(stage_)                                                                  \
-    _Pragma("unroll") for (int p = 0; p < SEGS_PER_THREAD; ++p)                               \
-    {                                                                                         \
-        const int s_ = tid + p * TZ_THREADS;                                                  \
-        char *dst_ = lds + (stage_) * STAGE_BYTES + (s_ / SEGS_PER_ROW) * ROWB +              \
-                     (s_ % SEGS_PER_ROW) * 16;                                                \
-        *reinterpret_cast<uint4_t *>(dst_) = ga[p];                                           \
-        *reinterpret_cast<uint4_t *>(dst_ + OPERAND_BYTES) = gb[p];                           \
-    }
-
-        TZ_LOAD_GLOBAL(0)
-        TZ_STORE_LDS(0)
+        // fill the ring, publish chunk 0, fetch its first k-step
+        const int prologue = kchunks < STAGES ? kchunks : STAGES;
+        for (int c = 0; c < prologue; ++c) { TZ_ISSUE_CHUNK(c, c) }
+        if (STAGES - 1 < kchunks) __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(LOADS_PER_CHUNK * (STAGES - 1)));
+        else __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
         sync.sync();
-        for (int kc = 0; kc < kchunks; ++kc) {
-            const int cur = kc & 1;
-            const bool more = kc + 1 < kchunks;
-            if (more) { TZ_LOAD_GLOBAL(kc + 1) }
-            const char *sa = lds + cur * STAGE_BYTES;
-            const char *sb = sa + OPERAND_BYTES;
-#pragma unroll
-            for (int ks = 0; ks < KSTEPS; ++ks) {
-                half8_t fa[4], fb[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    fa[i] = *reinterpret_cast<const half8_t *>(sa + frag_a + i * 16 * ROWB + ks * 64);
-                    fb[i] = *reinterpret_cast<const half8_t *>(sb + frag_b + i * 16 * ROWB + ks * 64);
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int j = 0; j < 4; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j], fa[i], acc[i][j],
-                                                                           0, 0, 0);
-            }
-            if (more) { TZ_STORE_LDS(cur ^ 1) }
-            sync.sync();
+        half8_t fa0[4], fb0[4], fa1[4], fb1[4];
+        TZ_READ_FRAGS(fa0, fb0, 0, frag_seg0)
+        __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
+
+        int stage = 0;   // stage of chunk kc (and of chunk kc+STAGES, refilled once kc is consumed)
+        int kc = 0;
+        // steady state: chunk kc+STAGES exists, so exactly STAGES-2 chunks of this wave's
+        // loads may stay in flight when chunk kc+1 is needed.  Branch-free body.
+        for (; kc + STAGES < kchunks; ++kc) {
+            const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+            TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)     // second k-step of chunk kc, in flight ...
+            __builtin_amdgcn_sched_barrier(0);            // (keep the reads ahead of the MFMAs)
+            TZ_MFMAS(fa0, fb0)                            // ... while the first one is multiplied
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);  // those reads landed during the MFMA issue
+            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(LOADS_PER_CHUNK * (STAGES - 2)));
+            sync.sync();   // chunk kc+1 is complete in LDS; every wave has read all of chunk kc
+            TZ_ISSUE_CHUNK(kc + STAGES, stage)
+            TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
+            __builtin_amdgcn_sched_barrier(0);
+            TZ_MFMAS(fa1, fb1)
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
+            stage = next_stage;
         }
+        // drain: nothing left to issue, fewer loads in flight -- wait for all of them
+        for (; kc + 1 < kchunks; ++kc) {
+            const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+            TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)
+            __builtin_amdgcn_sched_barrier(0);
+            TZ_MFMAS(fa0, fb0)
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
+            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+            sync.sync();
+            TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
+            __builtin_amdgcn_sched_barrier(0);
+            TZ_MFMAS(fa1, fb1)
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
+            stage = next_stage;
+        }
+        // last chunk: nothing left to fetch
+        TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)
+        TZ_MFMAS(fa0, fb0)
+        TZ_MFMAS(fa1, fb1)
+        sync.sync();   // all waves are done reading before the next tile refills the ring
 
         if (store) {
             // lane holds C[row0 + i*16 + lane%16][col0 + j*16 + 4*(lane/16) .. +3]
@@ -148,9 +210,13 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
                     *reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16) = v;
                 }
         }
+        // stores and LDS-direct loads share the vmcnt counter: drain it so that the
+        // counts of the next tile's ring are exact
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+#undef TZ_ISSUE_CHUNK
+#undef TZ_READ_FRAGS
+#undef TZ_MFMAS
     }
-#undef TZ_LOAD_GLOBAL
-#undef TZ_STORE_LDS
 }
 
 }  // namespace tk

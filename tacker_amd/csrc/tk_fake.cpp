@@ -177,7 +177,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("pack_fc_input", {P, 8, P, I, I, P});
         const std::pair<const char *, const std::vector<int> *> bes[] = {
             {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}};
-        static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1", "@wave_256", "@wave_512"};
+        static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};
         for (auto &be : bes)
             for (auto v : variants)
                 add((std::string("tzgemm_") + be.first + v).c_str(),

@@ -43,7 +43,7 @@ REFERENCE_KERNEL_INFO = {
 # launch, ori_blks = blocks of the reference-shaped natural grid at the
 # benchmark's problem size.
 KERNEL_INFO = {
-    "tzgemm": {"register": 128, "shared_memory": 20480, "blocksize": 256, "solo_ptb_blks": 2},
+    "tzgemm": {"register": 160, "shared_memory": 131072, "blocksize": 256, "solo_ptb_blks": 1},
     "stencil": {"register": 48, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
                 "ori_blks": 1024},
     "lbm": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,

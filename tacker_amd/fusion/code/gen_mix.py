@@ -40,7 +40,7 @@ def generate_wg_split(be, tz_wgs, be_wgs, threads=256):
     p_be, sig_be = signature(be, 0)
     p_tz, sig_tz = signature("tzgemm", 1)
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="sp.role_block", blocks="sp.role_blocks",
-                                             tid="(int)threadIdx.x")
+                                             tid="(int)threadIdx.x", stages="TZ_STAGES_WG")
     be_call = ROLES[be]["call"].format(p=p_be, block="sp.role_block", blocks="sp.role_blocks",
                                        tid="(int)threadIdx.x", threads=threads)
     name = mix_kernel_name(be, variant)
@@ -48,7 +48,7 @@ def generate_wg_split(be, tz_wgs, be_wgs, threads=256):
 extern "C" __global__ __launch_bounds__({threads}) void {name}(
     {_params_text(sig_be, sig_tz)})
 {{
-{_void_unused(sig_be + sig_tz, tz_call + be_call)}    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
+{_void_unused(sig_be + sig_tz, tz_call + be_call)}    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES_WG];
     const tk::WgSplit sp = tk::wg_split((int)blockIdx.x, (int)gridDim.x, {tz_wgs}, {be_wgs});
     if (sp.role == 0) {{
         tk::WorkgroupSync sync;
@@ -76,7 +76,7 @@ def generate_wave_split(be, be_threads, tz_first=True):
         be_lo, tz_lo = 0, be_threads
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="(int)blockIdx.x",
                                              blocks=f"{p_tz}ptb_iter_block_step",
-                                             tid=f"(int)threadIdx.x - {tz_lo}")
+                                             tid=f"(int)threadIdx.x - {tz_lo}", stages="TZ_STAGES")
     be_call = ROLES[be]["call"].format(p=p_be, block="(int)blockIdx.x",
                                        blocks=f"{p_be}ptb_iter_block_step",
                                        tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads)

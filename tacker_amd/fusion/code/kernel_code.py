@@ -26,7 +26,7 @@ ROLES = {
                    ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K")],
         "needs_sync": True,
         "lds_bytes": "TZ_LDS_BYTES",
-        "call": ("tk::tzgemm_role({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, "
+        "call": ("tk::tzgemm_role<{stages}>({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, "
                  "{block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "tz_lds, sync);"),
     },

@@ -68,7 +68,7 @@ def test_cdna4_candidates_fit_one_compute_unit():
             assert threads <= data.CDNA4_CU.thread_slots
         for v in gen_run.pair_candidates(be):
             if v[0] == "wave":
-                assert (256 + v[1]) % 64 == 0 and 256 + v[1] <= 1024
+                assert (256 + v[1]) % 64 == 0 and 256 + v[1] <= 768
 
 
 def test_committed_generated_sources_are_fresh():

@@ -228,7 +228,7 @@ def test_cp_fewer_atoms():
 
 
 # ------------------------------------------------------------------ fused
-VARIANTS = [None, "wg_1_1", "wg_2_1", "wg_1_2"]
+VARIANTS = [None, "wave_256", "wave_512", "wg_1_1", "wg_1_2"]
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
@@ -249,6 +249,7 @@ def test_mix_tzgemm_stencil(variant):
     assert np.array_equal(host(mix_s), oracle.stencil(C0, C1, A0, A0))
     ok, fro, _ = gemm_tolerance_ok(host(mix_c), oracle.tzgemm(A, B, f64=True), K)
     assert ok and fro <= 1e-5
+    assert ta.spin_fail_flag() == 0          # no role-local barrier gave up waiting
 
 
 def test_mix_tzgemm_stencil_partial_ranges():

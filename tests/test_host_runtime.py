@@ -83,7 +83,7 @@ def test_tzgemm_grid_dim_known_answers(fake):
 
 
 def test_kinfo_lookups_and_missing_keys(fake):
-    assert fake.tacker_get_kernel_info(b"tzgemm_stencil", b"blocksize") in (256, 512, 768, 1024)
+    assert fake.tacker_get_kernel_info(b"tzgemm_stencil", b"blocksize") in (512, 768, 1024)
     assert fake.tacker_get_kernel_info(b"tzgemm_stencil", b"no_such_key") == ta.JSON_NOT_FOUND
     assert fake.tacker_get_kernel_info(b"no_such_kernel", b"blocksize") == ta.JSON_NOT_FOUND
     assert fake.tacker_fget_kernel_info(b"tzgemm_stencil", b"4096") > 0
