@@ -93,7 +93,10 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
     // bit 2 of the key: odd loads fetch segment (seg ^ 4).
     const int dma_row = 4 * wave * 8 + (lane >> 3);
     const int dma_seg = (lane & 7) ^ ((dma_row >> 1) & 7);
-    const size_t src_off = (size_t)dma_row * K;                 // + j*8*K + segment per load
+    // per-lane byte offsets below a wave-uniform row-block address (even / odd loads); kept as
+    // 32-bit offsets so a load is "scalar base + vector offset" and holds no 64-bit pointers
+    const unsigned src_even = (unsigned)(dma_row * K + dma_seg * 8) * 2u;
+    const unsigned src_odd = (unsigned)(dma_row * K + (dma_seg ^ 4) * 8) * 2u;
     const int dst_off = 4 * wave * 1024;                        // + j*1024 per load
     // fragment reads: row r = lane%16 of a 16-row group (its swizzle key (r>>1)&7 is the
     // same in every group), k segment 4*kstep + lane/16 of the 8 in a row
@@ -115,17 +118,19 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
         if (!(in00 || in01 || in10 || in11)) continue;   // uniform over the workgroup
         const bool store = wr ? (wc ? in11 : in10) : (wc ? in01 : in00);
 
-        const _Float16 *a_tile = A + (size_t)(mi * TZ_MACRO_TILE) * K + src_off;
-        const _Float16 *b_tile = B + (size_t)(mj * TZ_MACRO_TILE) * K + src_off;
+        const char *a_tile = reinterpret_cast<const char *>(A + (size_t)(mi * TZ_MACRO_TILE) * K);
+        const char *b_tile = reinterpret_cast<const char *>(B + (size_t)(mj * TZ_MACRO_TILE) * K);
 
 #define TZ_ISSUE_CHUNK(chunk_, stage_)                                                            \
     _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                             \
     {                                                                                             \
         char *dst_ = lds + (stage_) * STAGE_BYTES + dst_off + j * 1024;                           \
-        const size_t src_ = (size_t)(j * 8) * K + (size_t)(chunk_) * BK + (dma_seg ^ ((j & 1) * 4)) * 8; \
-        __builtin_amdgcn_global_load_lds((gptr_t)(a_tile + src_), (lptr_t)dst_, 16, 0, 0);        \
-        __builtin_amdgcn_global_load_lds((gptr_t)(b_tile + src_), (lptr_t)(dst_ + OPERAND_BYTES), \
-                                         16, 0, 0);                                               \
+        const size_t uni_ = ((size_t)(j * 8) * K + (size_t)(chunk_) * BK) * 2;                    \
+        unsigned lane_ = (j & 1) ? src_odd : src_even;                                            \
+        asm volatile("" : "+v"(lane_));   /* keep base + offset apart: scalar base, vector offset */ \
+        __builtin_amdgcn_global_load_lds((gptr_t)(a_tile + uni_ + lane_), (lptr_t)dst_, 16, 0, 0); \
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_tile + uni_ + lane_),                         \
+                                         (lptr_t)(dst_ + OPERAND_BYTES), 16, 0, 0);               \
     }
 #define TZ_READ_FRAGS(fa_, fb_, stage_, seg_)                                                     \
     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                 \
@@ -134,9 +139,31 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
         fa_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_a);                                 \
         fb_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_b);                                 \
     }
-#define TZ_MFMAS(fa_, fb_)                                                                        \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)   \
+#define TZ_MFMAS_ROWS(fa_, fb_, i0_, i1_)                                                         \
+    _Pragma("unroll") for (int i = i0_; i < i1_; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[j], fa_[i], acc[i][j], 0, 0, 0);
+#define TZ_MFMAS(fa_, fb_) TZ_MFMAS_ROWS(fa_, fb_, 0, 4)
+// First k-step of a chunk multiplied while the chunk barrier completes.  With a split
+// barrier the wave announces itself half way through the 16 MFMAs (its reads of the stage
+// have landed by then) and the other half hides the round trip of the arrival counter.
+#define TZ_MFMAS_ACROSS_BARRIER(fa_, fb_, vmcnt_)                                                 \
+    if constexpr (Sync::kSplit) {                                                                 \
+        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
+        sync.arrive();                                                                            \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        TZ_MFMAS_ROWS(fa_, fb_, 2, 4)                                                             \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        sync.wait();                                                                              \
+    } else {                                                                                      \
+        TZ_MFMAS(fa_, fb_)                                                                        \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
+        sync.wait();                                                                              \
+    }
 
         float4_t acc[4][4];
 #pragma unroll
@@ -162,11 +189,9 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
             const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
             TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)     // second k-step of chunk kc, in flight ...
             __builtin_amdgcn_sched_barrier(0);            // (keep the reads ahead of the MFMAs)
-            TZ_MFMAS(fa0, fb0)                            // ... while the first one is multiplied
-            __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);  // those reads landed during the MFMA issue
-            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(LOADS_PER_CHUNK * (STAGES - 2)));
-            sync.sync();   // chunk kc+1 is complete in LDS; every wave has read all of chunk kc
+            // ... while the first one is multiplied.  Past the barrier chunk kc+1 is complete
+            // in LDS and every wave has read all of chunk kc.
+            TZ_MFMAS_ACROSS_BARRIER(fa0, fb0, LOADS_PER_CHUNK * (STAGES - 2))
             TZ_ISSUE_CHUNK(kc + STAGES, stage)
             TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
             __builtin_amdgcn_sched_barrier(0);
@@ -180,11 +205,7 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
             const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
             TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)
             __builtin_amdgcn_sched_barrier(0);
-            TZ_MFMAS(fa0, fb0)
-            __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
-            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
-            sync.sync();
+            TZ_MFMAS_ACROSS_BARRIER(fa0, fb0, 0)
             TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
             __builtin_amdgcn_sched_barrier(0);
             TZ_MFMAS(fa1, fb1)
@@ -216,7 +237,10 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
 #undef TZ_ISSUE_CHUNK
 #undef TZ_READ_FRAGS
 #undef TZ_MFMAS
+#undef TZ_MFMAS_ROWS
+#undef TZ_MFMAS_ACROSS_BARRIER
     }
+    sync.finish();
 }
 
 }  // namespace tk

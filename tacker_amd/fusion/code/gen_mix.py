@@ -87,12 +87,18 @@ def generate_wave_split(be, be_threads, tz_first=True):
 extern "C" __global__ __launch_bounds__({total}) void {name}(
     {_params_text(sig_be, sig_tz)})
 {{
-{unused}    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
-    __shared__ unsigned tz_arrivals;
-    if (threadIdx.x == 0) tz_arrivals = 0u;
+{unused}    // One LDS object on purpose (ring + the arrival counter behind it): with two, the
+    // compiler tags LDS accesses per object and then waits for every LDS-direct load in
+    // flight before each read of the ring.
+    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES + 16];
+    unsigned *tz_arrivals = reinterpret_cast<unsigned *>(tz_lds + TZ_LDS_BYTES);
+    if (threadIdx.x == 0) *tz_arrivals = 0u;
     __syncthreads();   // the only workgroup-wide barrier: before the roles part ways
     if ({tz_cond}) {{
-        tk::RoleSpinSync sync(&tz_arrivals, {tz_threads // 64}, &tk_spin_fail);
+        // One tzgemm wave per SIMD shares it with {be} waves: let the MFMA stream issue
+        // whenever it is ready and the {be} waves fill the slots it leaves.
+        __builtin_amdgcn_s_setprio(2);
+        tk::RoleSpinSync sync(tz_arrivals, {tz_threads // 64}, &tk_spin_fail);
         {tz_call}
     }} else {{
         {be_call}
