@@ -91,24 +91,32 @@ struct RoleSpinSync {
     // Block until every wave of the role has arrived.  Work placed between arrive() and
     // wait() hides the LDS round trip of the counter; the poll has no sleep in it because
     // the other waves are at most a few hundred cycles behind.  The poll is bounded.
+    // seen: a value of the counter read after arrive() (the caller overlaps that read with
+    // its own work and hands the result in); a value from before the last arrival just polls.
+    __device__ __forceinline__ void wait(unsigned seen)
+    {
+        if ((int)(seen - expected) < 0) wait();
+    }
     __device__ __forceinline__ void wait()
     {
-        unsigned seen, left;
-        asm volatile("s_mov_b32 %1, %4\n"
-                     "1:\n\t"
-                     "ds_read_b32 %0, %2\n\t"
-                     "s_waitcnt lgkmcnt(0)\n\t"
-                     "v_sub_u32 %0, %0, %3\n\t"
-                     "v_cmp_gt_i32 vcc, 0, %0\n\t"
-                     "s_cbranch_vccz 2f\n\t"
-                     "s_sub_u32 %1, %1, 1\n\t"
-                     "s_cmp_lg_u32 %1, 0\n\t"
-                     "s_cbranch_scc1 1b\n"
-                     "2:"
-                     : "=&v"(seen), "=&s"(left)
-                     : "v"(counter_addr), "v"(expected), "s"(spin_limit)
-                     : "vcc", "scc", "memory");
-        gave_up |= (left == 0u);
+        {
+            unsigned now, left;
+            asm volatile("s_mov_b32 %1, %4\n"
+                         "1:\n\t"
+                         "ds_read_b32 %0, %2\n\t"
+                         "s_waitcnt lgkmcnt(0)\n\t"
+                         "v_sub_u32 %0, %0, %3\n\t"
+                         "v_cmp_gt_i32 vcc, 0, %0\n\t"
+                         "s_cbranch_vccz 2f\n\t"
+                         "s_sub_u32 %1, %1, 1\n\t"
+                         "s_cmp_lg_u32 %1, 0\n\t"
+                         "s_cbranch_scc1 1b\n"
+                         "2:"
+                         : "=&v"(now), "=&s"(left)
+                         : "v"(counter_addr), "v"(expected), "s"(spin_limit)
+                         : "vcc", "scc", "memory");
+            gave_up |= (left == 0u);
+        }
     }
     __device__ __forceinline__ void sync()
     {

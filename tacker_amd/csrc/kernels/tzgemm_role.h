@@ -143,26 +143,80 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
     _Pragma("unroll") for (int i = i0_; i < i1_; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[j], fa_[i], acc[i][j], 0, 0, 0);
 #define TZ_MFMAS(fa_, fb_) TZ_MFMAS_ROWS(fa_, fb_, 0, 4)
-// First k-step of a chunk multiplied while the chunk barrier completes.  With a split
-// barrier the wave announces itself half way through the 16 MFMAs (its reads of the stage
-// have landed by then) and the other half hides the round trip of the arrival counter.
-#define TZ_MFMAS_ACROSS_BARRIER(fa_, fb_, vmcnt_)                                                 \
+// Issue order inside one scheduling region: after each MFMA one LDS read (count_ of them),
+// then after each MFMA one LDS-direct load (count2_).  An MFMA occupies the matrix pipe for
+// 16 cycles but the wave for 4, so the memory instructions slot into its shadow instead
+// of queuing up in front of the next MFMA group.
+#define TZ_PAIR_MFMA_WITH(mask_, count_)                                                          \
+    _Pragma("unroll") for (int q = 0; q < count_; ++q)                                            \
+    {                                                                                             \
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                        \
+        __builtin_amdgcn_sched_group_barrier(mask_, 1, 0);                                        \
+    }
+#define TZ_SCHED_DS_READ 0x100
+#define TZ_SCHED_VMEM 0x010
+// First k-step of a chunk multiplied while the chunk barrier completes; the reads of the
+// second k-step (into fn_, fbn_) ride in the shadow of the first 8 MFMAs.  With a split
+// barrier the wave announces itself after 12 of the 16 MFMAs (its reads of the stage have
+// landed by then); the last 4 and the first 8 MFMAs of the second k-step, which need
+// nothing from behind the barrier, hide the round trip of the arrival counter.
+#define TZ_FIRST_STEP_ACROSS_BARRIER(fa_, fb_, fn_, fbn_, vmcnt_)                                 \
     if constexpr (Sync::kSplit) {                                                                 \
-        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
+        TZ_MFMAS_ROWS(fa_, fb_, 0, 3)                                                             \
+        TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                        \
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
         sync.arrive();                                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                        \
-        TZ_MFMAS_ROWS(fa_, fb_, 2, 4)                                                             \
+        TZ_MFMAS_ROWS(fa_, fb_, 3, 4)                                                             \
+        TZ_MFMAS_ROWS(fn_, fbn_, 0, 1)                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                        \
-        sync.wait();                                                                              \
+        {   /* counter read + 4 MFMAs + wait for the read, as one block: the compiler must */     \
+            /* not touch the destination register of the read while it is in flight       */     \
+            unsigned seen_;                                                                       \
+            asm volatile("ds_read_b32 %0, %5\n\t"                                                 \
+                         "v_mfma_f32_16x16x32_f16 %1, %6, %10, %1\n\t"                            \
+                         "v_mfma_f32_16x16x32_f16 %2, %7, %10, %2\n\t"                            \
+                         "v_mfma_f32_16x16x32_f16 %3, %8, %10, %3\n\t"                            \
+                         "v_mfma_f32_16x16x32_f16 %4, %9, %10, %4\n\t"                            \
+                         "s_waitcnt lgkmcnt(0)"                                                   \
+                         : "=&v"(seen_), "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]),       \
+                           "+v"(acc[1][3])                                                        \
+                         : "v"(sync.counter_addr), "v"(fbn_[0]), "v"(fbn_[1]), "v"(fbn_[2]),      \
+                           "v"(fbn_[3]), "v"(fn_[1])                                              \
+                         : "memory");                                                             \
+            sync.wait(seen_);                                                                     \
+        }                                                                                         \
     } else {                                                                                      \
         TZ_MFMAS(fa_, fb_)                                                                        \
+        TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                        \
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
         sync.wait();                                                                              \
+    }
+// Second k-step (what is left of it), with the 8 reads of the next chunk's first k-step and,
+// if loads_ is nonzero, the 8 LDS-direct loads of a new chunk slotted between its MFMAs.
+#define TZ_SECOND_STEP(fa_, fb_, loads_)                                                          \
+    if constexpr (Sync::kSplit) {                                                                 \
+        TZ_MFMAS_ROWS(fa_, fb_, 2, 4)                                                             \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
+        {                                                                                         \
+            __builtin_amdgcn_sched_group_barrier(TZ_SCHED_DS_READ, 2, 0);                         \
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                    \
+        }                                                                                         \
+        if (loads_) {                                                                             \
+            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                         \
+            {                                                                                     \
+                __builtin_amdgcn_sched_group_barrier(TZ_SCHED_VMEM, 2, 0);                        \
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                \
+            }                                                                                     \
+        }                                                                                         \
+    } else {                                                                                      \
+        TZ_MFMAS(fa_, fb_)                                                                        \
+        TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
+        if (loads_) { TZ_PAIR_MFMA_WITH(TZ_SCHED_VMEM, 8) }                                       \
     }
 
         float4_t acc[4][4];
@@ -188,14 +242,12 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
         for (; kc + STAGES < kchunks; ++kc) {
             const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
             TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)     // second k-step of chunk kc, in flight ...
-            __builtin_amdgcn_sched_barrier(0);            // (keep the reads ahead of the MFMAs)
             // ... while the first one is multiplied.  Past the barrier chunk kc+1 is complete
             // in LDS and every wave has read all of chunk kc.
-            TZ_MFMAS_ACROSS_BARRIER(fa0, fb0, LOADS_PER_CHUNK * (STAGES - 2))
-            TZ_ISSUE_CHUNK(kc + STAGES, stage)
+            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, LOADS_PER_CHUNK * (STAGES - 2))
             TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
-            __builtin_amdgcn_sched_barrier(0);
-            TZ_MFMAS(fa1, fb1)
+            TZ_ISSUE_CHUNK(kc + STAGES, stage)
+            TZ_SECOND_STEP(fa1, fb1, 1)
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
             stage = next_stage;
@@ -204,11 +256,9 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
         for (; kc + 1 < kchunks; ++kc) {
             const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
             TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)
-            __builtin_amdgcn_sched_barrier(0);
-            TZ_MFMAS_ACROSS_BARRIER(fa0, fb0, 0)
+            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, 0)
             TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
-            __builtin_amdgcn_sched_barrier(0);
-            TZ_MFMAS(fa1, fb1)
+            TZ_SECOND_STEP(fa1, fb1, 0)
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
             stage = next_stage;
@@ -238,7 +288,11 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
 #undef TZ_READ_FRAGS
 #undef TZ_MFMAS
 #undef TZ_MFMAS_ROWS
-#undef TZ_MFMAS_ACROSS_BARRIER
+#undef TZ_PAIR_MFMA_WITH
+#undef TZ_SCHED_DS_READ
+#undef TZ_SCHED_VMEM
+#undef TZ_FIRST_STEP_ACROSS_BARRIER
+#undef TZ_SECOND_STEP
     }
     sync.finish();
 }
