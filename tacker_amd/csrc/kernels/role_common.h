@@ -79,13 +79,12 @@ struct RoleSpinSync {
     {
         expected += waves;
         unsigned long long saved_exec;
-        const unsigned one = 1u;
         asm volatile("s_mov_b64 %0, exec\n\t"
                      "s_mov_b64 exec, 1\n\t"
                      "ds_add_u32 %1, %2\n\t"
                      "s_mov_b64 exec, %0"
                      : "=&s"(saved_exec)
-                     : "v"(counter_addr), "v"(one)
+                     : "v"(counter_addr), "v"(1u)
                      : "memory");
     }
     // Block until every wave of the role has arrived.  Work placed between arrive() and

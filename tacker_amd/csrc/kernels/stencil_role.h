@@ -119,28 +119,160 @@ __device__ __forceinline__ void stencil_wave_run(float c0, float c1, const float
     run.finish(c0, c1, Anext, nx, ny, lane);
 }
 
-// GPTB form.  The unit of work of a wave is one reference block cut into runs of
-// STENCIL_Z_RUN centre planes: a 512x512x64 grid has only 1024 blocks, far fewer
-// than the waves a 256-CU part needs in flight to pull HBM bandwidth, so the z
-// march of a block is shared out.  The waves of one workgroup take consecutive
-// runs of the same block (their overlap planes hit in the CU's own cache).
-// Task t of the range: block = start + t / runs, run = t % runs; the role's waves
-// enumerate t = role_block*waves + wave, stepping by role_blocks*waves.
+// ---------------------------------------------------------------------------------------
+// Wide form, used when nx is a multiple of 4 (rows are then 16-byte aligned).
+//
+// Per CU the vector-memory front end (address unit + data return) handles one wave
+// instruction every ~11 cycles for a dword access and every ~22 for a dwordx4 one, so a
+// kernel that moves its bytes with dword accesses is bound by that unit at less than half
+// of what the same bytes cost as dwordx4 -- and in a fused launch that unit is shared with
+// the GEMM's LDS-direct loads.  The wide form therefore gives a wave a "quad" of 4
+// horizontally adjacent reference blocks (256 columns x 4 rows): lane l owns columns
+// 256*q + 4*l .. +3 and every access is one float4 per lane, a 1 KiB contiguous row piece
+// per wave.  Along z the wave marches: planes k-1, k, k+1 live in registers while the
+// loads of planes k+2 and k+3 are in flight (a ring of 4 planes), so about 14 KiB per wave
+// are outstanding at any time.  y neighbours are the lane's own registers (rows above and
+// below the quad are two more float4 loads per plane), x neighbours inside a lane are its
+// own components, across lanes one wave shuffle per side, and the two columns outside the
+// quad come from one 8-lane gathered load per plane.
+//
+// The per-point expression and its order are those of StencilRun::finish.
+template <int Z>
+struct StencilQuadMarch {
+    static constexpr int ROWS = STENCIL_TILE_Y;
+    static constexpr int RING = 4;
+
+    const float *__restrict__ A0;
+    float *__restrict__ Anext;
+    int nx, ny, lane;
+    size_t plane;
+
+    float4_t own[RING][ROWS];   // plane ring, slot = plane index % RING
+    float4_t dn[3], up[3];      // rows j0-1 and j0+ROWS of centre planes, slot = centre % 3
+    float edge[3];              // lanes 0..3: column x0-1 of rows 0..3, lanes 4..7: column x0+256
+
+    // loads of plane p of the run (p = 0 is k_first-1): own rows always, halo rows and the
+    // outside columns only when p is a centre plane (1 <= p <= nplanes)
+    template <int P>
+    __device__ __forceinline__ void issue(int k_first, int nplanes, int x0, int j0)
+    {
+        const int x = x0 + 4 * lane;
+        const bool xin = x < nx;
+        const float *col = A0 + (size_t)x + (size_t)nx * j0 + plane * (size_t)(k_first - 1 + P);
+        const bool have = P <= nplanes + 1;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            float4_t v = {0.f, 0.f, 0.f, 0.f};
+            if (have && xin && (j0 + r) < ny) v = *reinterpret_cast<const float4_t *>(col + (size_t)nx * r);
+            own[P % RING][r] = v;
+        }
+        if (P >= 1 && P <= Z) {
+            const bool centre = P <= nplanes;
+            float4_t d = {0.f, 0.f, 0.f, 0.f}, u = {0.f, 0.f, 0.f, 0.f};
+            if (centre && xin && j0 > 0) d = *reinterpret_cast<const float4_t *>(col - (size_t)nx);
+            if (centre && xin && (j0 + ROWS) < ny) u = *reinterpret_cast<const float4_t *>(col + (size_t)nx * ROWS);
+            dn[P % 3] = d;
+            up[P % 3] = u;
+            float e = 0.f;
+            const int er = lane & 3;
+            const int ex = (lane & 4) ? x0 + 256 : x0 - 1;
+            if (centre && lane < 8 && ex >= 0 && ex < nx && (j0 + er) < ny)
+                e = A0[(size_t)ex + (size_t)nx * (j0 + er) + plane * (size_t)(k_first - 1 + P)];
+            edge[P % 3] = e;
+        }
+    }
+
+    // centre plane C of the run (1 <= C <= Z): needs planes C-1, C, C+1
+    template <int C>
+    __device__ __forceinline__ void finish(float c0, float c1, int k_first, int nplanes, int x0, int j0,
+                                           unsigned block_ok)
+    {
+        if (C > nplanes) return;
+        const int x = x0 + 4 * lane;
+        float *out = Anext + (size_t)x + (size_t)nx * j0 + plane * (size_t)(k_first - 1 + C);
+        const bool mine = (block_ok >> (lane >> 4)) & 1u;
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const float4_t centre = own[C % RING][r];
+            const float4_t top = own[(C + 1) % RING][r];
+            const float4_t bottom = own[(C + RING - 1) % RING][r];
+            const float4_t a_up = (r + 1 < ROWS) ? own[C % RING][(r + 1 < ROWS) ? r + 1 : r] : up[C % 3];
+            const float4_t a_dn = (r > 0) ? own[C % RING][(r > 0) ? r - 1 : r] : dn[C % 3];
+            float from_left = __shfl_up(centre.w, 1, 64);
+            float from_right = __shfl_down(centre.x, 1, 64);
+            const float edge_l = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge[C % 3]), r));
+            const float edge_r = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(edge[C % 3]), 4 + r));
+            if (lane == 0) from_left = edge_l;
+            if (lane == 63) from_right = edge_r;
+            const float4_t left = {from_left, centre.x, centre.y, centre.z};
+            const float4_t right = {centre.y, centre.z, centre.w, from_right};
+            float4_t s = top + bottom;
+            s = s + a_up;
+            s = s + a_dn;
+            s = s + right;
+            s = s + left;
+            const float4_t v = s * c1 - centre * c0;
+            const int j = j0 + r;
+            const bool row_ok = mine && j > 0 && j < ny - 1 && x < nx;
+            if (row_ok) {
+                float *o = out + (size_t)nx * r;
+                if (x > 0 && x + 3 < nx - 1) {
+                    *reinterpret_cast<float4_t *>(o) = v;
+                } else {   // the quad touches the first or the last column of the grid
+                    if (x > 0) o[0] = v.x;
+                    o[1] = v.y;
+                    o[2] = v.z;
+                    if (x + 3 < nx - 1) o[3] = v.w;
+                }
+            }
+        }
+    }
+
+    template <int C>
+    __device__ __forceinline__ void steps(float c0, float c1, int k_first, int nplanes, int x0, int j0,
+                                          unsigned block_ok)
+    {
+        if constexpr (C <= Z) {
+            if constexpr (C + 2 <= Z + 1) issue<C + 2>(k_first, nplanes, x0, j0);
+            __builtin_amdgcn_sched_barrier(0);   // loads of plane C+2 go out before plane C is computed
+            finish<C>(c0, c1, k_first, nplanes, x0, j0, block_ok);
+            __builtin_amdgcn_sched_barrier(0);
+            steps<C + 1>(c0, c1, k_first, nplanes, x0, j0, block_ok);
+        }
+    }
+
+    __device__ __forceinline__ void run(float c0, float c1, int k_first, int nplanes, int x0, int j0,
+                                        unsigned block_ok)
+    {
+        issue<0>(k_first, nplanes, x0, j0);
+        issue<1>(k_first, nplanes, x0, j0);
+        issue<2>(k_first, nplanes, x0, j0);
+        steps<1>(c0, c1, k_first, nplanes, x0, j0, block_ok);
+    }
+};
+
+// GPTB form.  The unit of work of a wave is a run of STENCIL_Z_RUN centre planes of one
+// reference block (narrow form) or of one quad of blocks (wide form): a 512x512x64 grid has
+// only 1024 blocks, far fewer than the waves a 256-CU part needs in flight to pull HBM
+// bandwidth, so the z march is shared out.  The waves of one workgroup take consecutive
+// runs of the same block or quad (their overlap planes hit in the CU's own cache).
+// The role's waves enumerate tasks t = role_block*waves + wave, stepping by
+// role_blocks*waves.
 #define STENCIL_Z_RUN 8
-__device__ __forceinline__ void stencil_role(float c0, float c1, const float *__restrict__ A0,
-                                             float *__restrict__ Anext, int nx, int ny, int nz,
-                                             int grid_dimension_x, int grid_dimension_y,
-                                             int role_block, int role_blocks, int start, int end,
-                                             int tid, int role_threads)
+__device__ __forceinline__ void stencil_role_narrow(float c0, float c1, const float *__restrict__ A0,
+                                                    float *__restrict__ Anext, int nx, int ny, int nz,
+                                                    int grid_dimension_x, int grid_dimension_y,
+                                                    int role_block, int role_blocks, int start, int end,
+                                                    int tid, int role_threads)
 {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int waves = role_threads >> 6;
     const int planes = nz - 2;
-    if (planes < 1 || end <= start) return;
     const unsigned runs = (unsigned)(planes + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
     const unsigned tasks = (unsigned)(end - start) * runs;
     const unsigned stride = (unsigned)role_blocks * waves;
+    // task t: block = start + t / runs, run = t % runs.
     // two runs in flight per wave: the loads of run n+1 are issued before run n is computed
     StencilRun<STENCIL_TILE_Y, STENCIL_Z_RUN> ra, rb;
     auto start_run = [&](StencilRun<STENCIL_TILE_Y, STENCIL_Z_RUN> &r, unsigned t) {
@@ -166,6 +298,67 @@ __device__ __forceinline__ void stencil_role(float c0, float c1, const float *__
         if (!more_a) break;
         t += 2 * stride;
     }
+}
+
+__device__ __forceinline__ void stencil_role_wide(float c0, float c1, const float *__restrict__ A0,
+                                                  float *__restrict__ Anext, int nx, int ny, int nz,
+                                                  int grid_dimension_x, int grid_dimension_y,
+                                                  int role_block, int role_blocks, int start, int end,
+                                                  int tid, int role_threads)
+{
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int waves = role_threads >> 6;
+    const int planes = nz - 2;
+    const unsigned runs = (unsigned)(planes + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
+    // Quads are cut on the block grid (columns 4*qx .. 4*qx+3 of a block row); the range
+    // [start, end) of block positions touches block rows first_row .. last_row, a position
+    // being row * grid_dimension_x + bx with the row wrapping modulo grid_dimension_y.
+    const unsigned gdx = (unsigned)grid_dimension_x;
+    const unsigned quads_per_row = (gdx + 3) / 4;
+    const unsigned first_row = (unsigned)start / gdx;
+    const unsigned last_row = (unsigned)(end - 1) / gdx;
+    const unsigned tasks = (last_row - first_row + 1) * quads_per_row * runs;
+    const unsigned stride = (unsigned)role_blocks * waves;
+    StencilQuadMarch<STENCIL_Z_RUN> m;
+    m.A0 = A0;
+    m.Anext = Anext;
+    m.nx = nx;
+    m.ny = ny;
+    m.lane = lane;
+    m.plane = (size_t)nx * (size_t)ny;
+    for (unsigned t = (unsigned)role_block * waves + wave; t < tasks; t += stride) {
+        const unsigned quad = t / runs;
+        const int run = (int)(t % runs);
+        const unsigned row = first_row + quad / quads_per_row;
+        const unsigned qx = quad % quads_per_row;
+        unsigned block_ok = 0;   // bit b: block 4*qx + b exists and its position is in range
+#pragma unroll
+        for (unsigned b = 0; b < 4; ++b) {
+            const unsigned bx = 4 * qx + b;
+            const unsigned pos = row * gdx + bx;
+            if (bx < gdx && pos >= (unsigned)start && pos < (unsigned)end) block_ok |= 1u << b;
+        }
+        if (block_ok == 0) continue;
+        const int k_first = 1 + run * STENCIL_Z_RUN;
+        m.run(c0, c1, k_first, min(STENCIL_Z_RUN, nz - 1 - k_first), (int)(qx * 4 * 2 * STENCIL_TILE_X),
+              (int)(row % (unsigned)grid_dimension_y) * STENCIL_TILE_Y, block_ok);
+    }
+}
+
+__device__ __forceinline__ void stencil_role(float c0, float c1, const float *__restrict__ A0,
+                                             float *__restrict__ Anext, int nx, int ny, int nz,
+                                             int grid_dimension_x, int grid_dimension_y,
+                                             int role_block, int role_blocks, int start, int end,
+                                             int tid, int role_threads)
+{
+    if (nz - 2 < 1 || end <= start) return;
+    if ((nx & 3) == 0)
+        stencil_role_wide(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, role_block,
+                          role_blocks, start, end, tid, role_threads);
+    else
+        stencil_role_narrow(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, role_block,
+                            role_blocks, start, end, tid, role_threads);
 }
 
 }  // namespace tk

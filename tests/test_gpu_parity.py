@@ -66,7 +66,10 @@ def test_tzgemm_tile_range_writes_only_its_tiles(start, end, grid):
 
 
 # ------------------------------------------------------------------ stencil
-@pytest.mark.parametrize("shape", [(8, 8, 64), (6, 10, 70), (5, 7, 130), (4, 9, 33), (64, 64, 128)])
+# widths that are multiples of 4 take the float4 (quad of blocks) form of the GPTB role, the
+# others the one-block-per-wave form; 3 planes is the smallest grid with an interior
+@pytest.mark.parametrize("shape", [(8, 8, 64), (6, 10, 70), (5, 7, 130), (4, 9, 33), (64, 64, 128),
+                                   (12, 9, 260), (3, 5, 4), (11, 6, 516), (20, 13, 1028), (10, 4, 200)])
 def test_stencil_ori_and_gptb_bit_exact(shape):
     A0 = stencil_inputs(*shape)
     want = oracle.stencil(C0, C1, A0, A0)
@@ -96,6 +99,28 @@ def test_stencil_gptb_ranges_and_wrap():
     assert np.array_equal(host(acc), want)
     ta.gptb_stencil(C0, C1, a0, acc, start=4, end=4)                # empty range
     assert np.array_equal(host(acc), want)
+
+
+@pytest.mark.parametrize("nx", [520, 200])
+def test_stencil_wide_form_ranges_and_wrap(nx):
+    # block rows are 9 (520) or 4 (200) blocks wide: quads of 4 blocks are ragged at the row
+    # end, ranges start and end inside quads, and positions past the grid wrap onto it
+    A0 = stencil_inputs(13, 10, nx)
+    nblk = ta.stencil_blocks(nx, 10)
+    a0 = dev(A0)
+    acc = torch.full_like(a0, -3.0)
+    want = np.full_like(A0, -3.0)
+    cuts = [0, 1, 3, 6, 11, 13, nblk - 2, nblk]
+    for s, e in zip(cuts[:-1], cuts[1:]):
+        if e <= s:
+            continue
+        ta.gptb_stencil(C0, C1, a0, acc, start=s, end=e, launch_grid=3, launch_block=128)
+        want = oracle.stencil_gptb(C0, C1, A0, want, s, e)
+        assert np.array_equal(host(acc), want), (s, e)
+    assert np.array_equal(want, oracle.stencil(C0, C1, A0, np.full_like(A0, -3.0)))
+    acc2 = torch.full_like(a0, -3.0)
+    ta.gptb_stencil(C0, C1, a0, acc2, start=nblk + 2, end=2 * nblk - 1)   # wraps onto blocks 2 .. nblk-2
+    assert np.array_equal(host(acc2), oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), 2, nblk - 1))
 
 
 def test_stencil_iterations_ping_pong():
