@@ -318,7 +318,8 @@ __device__ __forceinline__ void stencil_role_wide(float c0, float c1, const floa
     const unsigned quads_per_row = (gdx + 3) / 4;
     const unsigned first_row = (unsigned)start / gdx;
     const unsigned last_row = (unsigned)(end - 1) / gdx;
-    const unsigned tasks = (last_row - first_row + 1) * quads_per_row * runs;
+    const unsigned rows = last_row - first_row + 1;
+    const unsigned tasks = rows * quads_per_row * runs;
     const unsigned stride = (unsigned)role_blocks * waves;
     StencilQuadMarch<STENCIL_Z_RUN> m;
     m.A0 = A0;
@@ -328,10 +329,13 @@ __device__ __forceinline__ void stencil_role_wide(float c0, float c1, const floa
     m.lane = lane;
     m.plane = (size_t)nx * (size_t)ny;
     for (unsigned t = (unsigned)role_block * waves + wave; t < tasks; t += stride) {
-        const unsigned quad = t / runs;
-        const int run = (int)(t % runs);
-        const unsigned row = first_row + quad / quads_per_row;
-        const unsigned qx = quad % quads_per_row;
+        // consecutive tasks (the waves of one workgroup) are vertically adjacent quads of the
+        // same run: the row above one quad is the last own row of the next wave's quad, so
+        // those halo loads hit in the CU's cache instead of costing a second L2 request
+        const unsigned row = first_row + t % rows;
+        const unsigned rest = t / rows;
+        const int run = (int)(rest % runs);
+        const unsigned qx = rest / runs;
         unsigned block_ok = 0;   // bit b: block 4*qx + b exists and its position is in range
 #pragma unroll
         for (unsigned b = 0; b < 4; ++b) {
