@@ -23,6 +23,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK = 8.0e12          # B/s, MI355X HBM3E
 MFMA_F16_PEAK = 2.5e15     # flop/s, dense fp16 MFMA
 
+# HBM-side bytes one fused launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
+# file scaled by what the same counters read for a 64 MiB copy (x1.9988 and x1.0000); the summary with
+# the commands is profiles/pmc_hbm_traffic_bench_tzgemm2048_stencil512x512x64.txt
+FUSED_HBM_TRAFFIC_BYTES = 2.192e8
+
 GEMM_MNK = (2048, 2048, 2048)
 STENCIL_DIMS = (64, 512, 512)      # nz, ny, nx
 ITERATIONS = 100
@@ -137,7 +142,9 @@ def main():
     ms = {k: trimmed_mean(v) for k, v in samples.items()}
 
     gemm_flop = 2.0 * M * N * K
-    stencil_bytes = 2.0 * nx * ny * nz * 4
+    stencil_bytes = 2.0 * nx * ny * nz * 4                    # every cell read once, written once
+    gemm_bytes = 2.0 * (M * K + N * K) + 4.0 * M * N          # A, B read once, C written once
+    fused_bytes = stencil_bytes + gemm_bytes                  # algorithmic bytes of one fused launch
     fused_launch_s = ms["fused"] / ITERATIONS * 1e-3
     speedup = ms["serial"] / ms["fused"]
     info = mix.info()
@@ -154,11 +161,12 @@ def main():
         "serial_ms_per_step": round(ms["serial"], 4),
         "gemm_alone_ms_per_100": round(ms["gemm"], 4), "stencil_alone_ms_per_100": round(ms["stencil"], 4),
         "overlap_efficiency": round(max(ms["gemm"], ms["stencil"]) / ms["fused"], 4),
-        "roofline": {"bound": "hbm", "achieved": round(stencil_bytes / fused_launch_s / 1e9, 1),
+        "roofline": {"bound": "hbm", "achieved": round(fused_bytes / fused_launch_s / 1e9, 1),
                      "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(stencil_bytes / fused_launch_s / HBM_PEAK, 4), "traffic": None,
+                     "frac": round(fused_bytes / fused_launch_s / HBM_PEAK, 4),
+                     "traffic": FUSED_HBM_TRAFFIC_BYTES,
                      "kernel": "stencil_tzgemm_mix (one fused launch: 1 GEMM + 1 sweep)",
-                     "algorithmic_bytes_per_launch": stencil_bytes,
+                     "algorithmic_bytes_per_launch": fused_bytes,
                      "avg_launch_us": round(fused_launch_s * 1e6, 2)},
         "roofline_mfma": {"bound": "mfma", "achieved": round(gemm_flop / fused_launch_s / 1e12, 1),
                           "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s",

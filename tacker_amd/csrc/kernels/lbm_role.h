@@ -13,9 +13,10 @@
 // race is always resolved in favour of the in-range writer, so results are
 // reproducible.
 //
-// gfx950 design: a block is one x-row (y,z); lane = x, so each of the 20 loads
-// and 19 stores of a wave is one contiguous row segment.  No LDS, no barrier.
-// A role of T threads processes T / roundup64(sx) rows at once.
+// gfx950 design: a block is one x-row (y,z); a lane takes two x-adjacent cells (one
+// if the row length is odd), so each of the 20 loads and 19 stores of a wave is one
+// contiguous row segment of 8 bytes per lane.  No LDS, no barrier.
+// A role of T threads processes T / roundup64(lanes per row) rows at once.
 #pragma once
 #include "role_common.h"
 #include "../header/lbm_header.h"
@@ -23,30 +24,11 @@
 namespace tk {
 
 // All indices are 32-bit: the host refuses grids with 20*cells >= 2^31.
-__device__ __forceinline__ void lbm_cell(const float *__restrict__ src, float *__restrict__ dst,
-                                         int cells, int c, int sx, int sxy)
-{
-    float tempC = src[cells * LBM_C + c];
-    float tempN = src[cells * LBM_N + c];
-    float tempS = src[cells * LBM_S + c];
-    float tempE = src[cells * LBM_E + c];
-    float tempW = src[cells * LBM_W + c];
-    float tempT = src[cells * LBM_T + c];
-    float tempB = src[cells * LBM_B + c];
-    float tempNE = src[cells * LBM_NE + c];
-    float tempNW = src[cells * LBM_NW + c];
-    float tempSE = src[cells * LBM_SE + c];
-    float tempSW = src[cells * LBM_SW + c];
-    float tempNT = src[cells * LBM_NT + c];
-    float tempNB = src[cells * LBM_NB + c];
-    float tempST = src[cells * LBM_ST + c];
-    float tempSB = src[cells * LBM_SB + c];
-    float tempET = src[cells * LBM_ET + c];
-    float tempEB = src[cells * LBM_EB + c];
-    float tempWT = src[cells * LBM_WT + c];
-    float tempWB = src[cells * LBM_WB + c];
-    const unsigned flags = __float_as_uint(src[cells * LBM_FLAGS + c]);
 
+// Collision of one cell, in place (src/ori_kernel/lbm_kernel.cu:49-131): obstacle cells
+// swap opposite directions, the others relax towards equilibrium.
+__device__ __forceinline__ void lbm_collide(unsigned flags, float &tempC, float &tempN, float &tempS, float &tempE, float &tempW, float &tempT, float &tempB, float &tempNE, float &tempNW, float &tempSE, float &tempSW, float &tempNT, float &tempNB, float &tempST, float &tempSB, float &tempET, float &tempEB, float &tempWT, float &tempWB)
+{
     if (flags & LBM_OBSTACLE) {
         float t;
         t = tempN; tempN = tempS; tempS = t;
@@ -99,32 +81,96 @@ __device__ __forceinline__ void lbm_cell(const float *__restrict__ src, float *_
         tempWT = temp2 * tempWT + temp1 * ((-ux + uz) * (4.5f * (-ux + uz) + 3.0f) - u2);
         tempWB = temp2 * tempWB + temp1 * ((-ux - uz) * (4.5f * (-ux - uz) + 3.0f) - u2);
     }
+}
 
+#define TK_LBM_DIRECTIONS(X)                                                                       \
+    X(LBM_C, 0, 0, 0, tempC) \
+    X(LBM_N, 0, +1, 0, tempN) \
+    X(LBM_S, 0, -1, 0, tempS) \
+    X(LBM_E, +1, 0, 0, tempE) \
+    X(LBM_W, -1, 0, 0, tempW) \
+    X(LBM_T, 0, 0, +1, tempT) \
+    X(LBM_B, 0, 0, -1, tempB) \
+    X(LBM_NE, +1, +1, 0, tempNE) \
+    X(LBM_NW, -1, +1, 0, tempNW) \
+    X(LBM_SE, +1, -1, 0, tempSE) \
+    X(LBM_SW, -1, -1, 0, tempSW) \
+    X(LBM_NT, 0, +1, +1, tempNT) \
+    X(LBM_NB, 0, +1, -1, tempNB) \
+    X(LBM_ST, 0, -1, +1, tempST) \
+    X(LBM_SB, 0, -1, -1, tempSB) \
+    X(LBM_ET, +1, 0, +1, tempET) \
+    X(LBM_EB, +1, 0, -1, tempEB) \
+    X(LBM_WT, -1, 0, +1, tempWT) \
+    X(LBM_WB, -1, 0, -1, tempWB)
+
+__device__ __forceinline__ void lbm_cell(const float *__restrict__ src, float *__restrict__ dst,
+                                         int cells, int c, int sx, int sxy)
+{
+    float tempC = src[cells * LBM_C + c];
+    float tempN = src[cells * LBM_N + c];
+    float tempS = src[cells * LBM_S + c];
+    float tempE = src[cells * LBM_E + c];
+    float tempW = src[cells * LBM_W + c];
+    float tempT = src[cells * LBM_T + c];
+    float tempB = src[cells * LBM_B + c];
+    float tempNE = src[cells * LBM_NE + c];
+    float tempNW = src[cells * LBM_NW + c];
+    float tempSE = src[cells * LBM_SE + c];
+    float tempSW = src[cells * LBM_SW + c];
+    float tempNT = src[cells * LBM_NT + c];
+    float tempNB = src[cells * LBM_NB + c];
+    float tempST = src[cells * LBM_ST + c];
+    float tempSB = src[cells * LBM_SB + c];
+    float tempET = src[cells * LBM_ET + c];
+    float tempEB = src[cells * LBM_EB + c];
+    float tempWT = src[cells * LBM_WT + c];
+    float tempWB = src[cells * LBM_WB + c];
+    const unsigned flags = __float_as_uint(src[cells * LBM_FLAGS + c]);
+    lbm_collide(flags, tempC, tempN, tempS, tempE, tempW, tempT, tempB, tempNE, tempNW, tempSE, tempSW, tempNT, tempNB, tempST, tempSB, tempET, tempEB, tempWT, tempWB);
 #define TK_LBM_SCATTER(entry, dx, dy, dz, value)                          \
     do {                                                                  \
         const int t_ = c + (dx) + (dy) * sx + (dz) * sxy;                 \
         if (t_ >= 0 && t_ < cells) dst[cells * (entry) + t_] = (value);   \
-    } while (0)
-    TK_LBM_SCATTER(LBM_C, 0, 0, 0, tempC);
-    TK_LBM_SCATTER(LBM_N, 0, +1, 0, tempN);
-    TK_LBM_SCATTER(LBM_S, 0, -1, 0, tempS);
-    TK_LBM_SCATTER(LBM_E, +1, 0, 0, tempE);
-    TK_LBM_SCATTER(LBM_W, -1, 0, 0, tempW);
-    TK_LBM_SCATTER(LBM_T, 0, 0, +1, tempT);
-    TK_LBM_SCATTER(LBM_B, 0, 0, -1, tempB);
-    TK_LBM_SCATTER(LBM_NE, +1, +1, 0, tempNE);
-    TK_LBM_SCATTER(LBM_NW, -1, +1, 0, tempNW);
-    TK_LBM_SCATTER(LBM_SE, +1, -1, 0, tempSE);
-    TK_LBM_SCATTER(LBM_SW, -1, -1, 0, tempSW);
-    TK_LBM_SCATTER(LBM_NT, 0, +1, +1, tempNT);
-    TK_LBM_SCATTER(LBM_NB, 0, +1, -1, tempNB);
-    TK_LBM_SCATTER(LBM_ST, 0, -1, +1, tempST);
-    TK_LBM_SCATTER(LBM_SB, 0, -1, -1, tempSB);
-    TK_LBM_SCATTER(LBM_ET, +1, 0, +1, tempET);
-    TK_LBM_SCATTER(LBM_EB, +1, 0, -1, tempEB);
-    TK_LBM_SCATTER(LBM_WT, -1, 0, +1, tempWT);
-    TK_LBM_SCATTER(LBM_WB, -1, 0, -1, tempWB);
+    } while (0);
+    TK_LBM_DIRECTIONS(TK_LBM_SCATTER)
 #undef TK_LBM_SCATTER
+}
+
+// Two x-adjacent cells per lane (c even, c + 1 in the same row): every access is 8 bytes
+// per lane, which halves the number of vector-memory instructions per byte moved -- the
+// per-CU address/data-return unit is what a dword-per-lane streaming kernel saturates first,
+// and in a fused launch that unit is shared with the GEMM's loads.  Scatter targets are
+// shifted by +-1 cell for 10 of the 19 directions, so the 8-byte accesses are only 4-byte
+// aligned; the vector type says so.
+typedef float lbm_pair_t __attribute__((ext_vector_type(2), aligned(4)));
+
+__device__ __forceinline__ void lbm_cell_pair(const float *__restrict__ src, float *__restrict__ dst,
+                                              int cells, int c, int sx, int sxy)
+{
+#define TK_LBM_LOAD(entry, dx, dy, dz, name) \
+    const lbm_pair_t name##_in = *reinterpret_cast<const lbm_pair_t *>(src + cells * (entry) + c);
+    TK_LBM_DIRECTIONS(TK_LBM_LOAD)
+#undef TK_LBM_LOAD
+    const lbm_pair_t flags_in = *reinterpret_cast<const lbm_pair_t *>(src + cells * LBM_FLAGS + c);
+#define TK_LBM_SPLIT(entry, dx, dy, dz, name) float name##0 = name##_in.x, name##1 = name##_in.y;
+    TK_LBM_DIRECTIONS(TK_LBM_SPLIT)
+#undef TK_LBM_SPLIT
+    lbm_collide(__float_as_uint(flags_in.x), tempC0, tempN0, tempS0, tempE0, tempW0, tempT0, tempB0, tempNE0, tempNW0, tempSE0, tempSW0, tempNT0, tempNB0, tempST0, tempSB0, tempET0, tempEB0, tempWT0, tempWB0);
+    lbm_collide(__float_as_uint(flags_in.y), tempC1, tempN1, tempS1, tempE1, tempW1, tempT1, tempB1, tempNE1, tempNW1, tempSE1, tempSW1, tempNT1, tempNB1, tempST1, tempSB1, tempET1, tempEB1, tempWT1, tempWB1);
+#define TK_LBM_SCATTER2(entry, dx, dy, dz, name)                                           \
+    do {                                                                                   \
+        const int t_ = c + (dx) + (dy) * sx + (dz) * sxy;                                  \
+        float *o_ = dst + cells * (entry) + t_;                                            \
+        if (t_ >= 0 && t_ + 1 < cells) {                                                   \
+            *reinterpret_cast<lbm_pair_t *>(o_) = lbm_pair_t{name##0, name##1};            \
+        } else {                                                                           \
+            if (t_ >= 0 && t_ < cells) o_[0] = name##0;                                    \
+            if (t_ + 1 >= 0 && t_ + 1 < cells) o_[1] = name##1;                            \
+        }                                                                                  \
+    } while (0);
+    TK_LBM_DIRECTIONS(TK_LBM_SCATTER2)
+#undef TK_LBM_SCATTER2
 }
 
 // grid_dimension_x = sy, grid_dimension_y = sz, block_dimension_x = sx
@@ -137,27 +183,35 @@ __device__ __forceinline__ void lbm_role(const float *__restrict__ src, float *_
     const int sx = block_dimension_x, sy = grid_dimension_x, sz = grid_dimension_y;
     const int sxy = sx * sy;
     const int cells = sxy * sz;
-    const int lanes_per_row = ((sx + TK_WAVE_SIZE - 1) / TK_WAVE_SIZE) * TK_WAVE_SIZE;
+    // even row length: a lane takes two cells, odd: one
+    const int per_lane = (sx & 1) ? 1 : 2;
+    const int row_lanes = (sx + per_lane - 1) / per_lane;
+    const int lanes_per_row = ((row_lanes + TK_WAVE_SIZE - 1) / TK_WAVE_SIZE) * TK_WAVE_SIZE;
     int rows_at_once = role_threads / lanes_per_row;
     int row_slot, x_first, x_step;
     if (rows_at_once >= 1) {
         row_slot = tid / lanes_per_row;
-        x_first = tid % lanes_per_row;
-        x_step = lanes_per_row;
+        x_first = (tid % lanes_per_row) * per_lane;
+        x_step = lanes_per_row * per_lane;
         if (row_slot >= rows_at_once) return;
     } else {   // row longer than the role: the role's threads sweep it
         rows_at_once = 1;
         row_slot = 0;
-        x_first = tid;
-        x_step = role_threads;
+        x_first = tid * per_lane;
+        x_step = role_threads * per_lane;
     }
     const unsigned stride = (unsigned)role_blocks * rows_at_once;
     for (unsigned pos = (unsigned)start + role_block * rows_at_once + row_slot; pos < (unsigned)end;
          pos += stride) {
         const int y = pos % sy;
         const int z = (pos / sy) % sz;
-        for (int x = x_first; x < sx; x += x_step)
-            lbm_cell(src, dst, cells, x + y * sx + z * sxy, sx, sxy);
+        if (per_lane == 2) {
+            for (int x = x_first; x < sx; x += x_step)
+                lbm_cell_pair(src, dst, cells, x + y * sx + z * sxy, sx, sxy);
+        } else {
+            for (int x = x_first; x < sx; x += x_step)
+                lbm_cell(src, dst, cells, x + y * sx + z * sxy, sx, sxy);
+        }
     }
 }
 

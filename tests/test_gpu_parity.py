@@ -136,7 +136,9 @@ def test_stencil_iterations_ping_pong():
 
 
 # ------------------------------------------------------------------ lbm
-@pytest.mark.parametrize("dims", [(4, 4, 4), (12, 5, 6), (64, 3, 5), (120, 6, 4), (128, 4, 4), (200, 3, 3)])
+# even row lengths take the two-cells-per-lane form, odd ones one cell per lane; 300 is longer than one wave of pairs
+@pytest.mark.parametrize("dims", [(4, 4, 4), (12, 5, 6), (64, 3, 5), (120, 6, 4), (128, 4, 4), (200, 3, 3),
+                                  (7, 5, 4), (121, 4, 3), (2, 3, 5), (300, 3, 3), (1, 4, 4)])
 def test_lbm_ori_and_gptb_bit_exact(dims):
     sx, sy, sz = dims
     src = lbm_inputs(sx, sy, sz, obstacle_p=0.2, accel_p=0.1)
