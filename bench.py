@@ -61,6 +61,126 @@ def cpu_baseline(A, B, A0, c0, c1):
                       "512x512x64 (%.4f s each), scaled to 100 + 100" % (t_gemm, t_sweep)}
 
 
+def pair_leg(ta, torch, np, name, stream):
+    """One of the other fused pairs (BASELINE configs 3 and 4): each kernel alone, serial, and the
+    fused launch over the full ranges, 200 launches each, median of 3 rounds."""
+    import statistics
+    rng = np.random.default_rng(1337)
+
+    def gemm(M, N, K):
+        A = torch.from_numpy(rng.uniform(-1, 1, (M, K)).astype(np.float16)).cuda()
+        B = torch.from_numpy(rng.uniform(-1, 1, (N, K)).astype(np.float16)).cuda()
+        Cm = torch.zeros((M, N), device="cuda:0")
+        tiles = (M // 64) * (N // 64)
+        return ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, tiles), tiles, 2.0 * M * N * K
+
+    if name == "lbm":       # D3Q19, 120x120x150, rest equilibrium + noise, 5 % obstacle cells
+        sx, sy, sz = 120, 120, 150
+        cells = sx * sy * sz
+        w = np.array([1 / 3] + [1 / 18] * 6 + [1 / 36] * 12, np.float32)
+        g = np.zeros((20, cells), np.float32)
+        g[:19] = w[:, None] + rng.uniform(0, 1e-3, (19, cells)).astype(np.float32)
+        g[19] = (rng.uniform(0, 1, cells) < 0.05).astype(np.uint32).view(np.float32)
+        src = torch.from_numpy(g.reshape(-1)).cuda()
+        dst = src.clone()
+        be_ori = ta.ori_lbm_create(src, dst, sx, sy, sz)
+        nblk = sy * sz
+        tz, tiles, flop = gemm(4096, 4096, 1024)
+        work = {"bound": "hbm", "algorithmic_bytes": 156.0 * cells}
+        label = "configs[2]: tzgemm 4096x4096x1024 + lbm 120x120x150 (one step per launch)"
+    else:                   # mri-q, numK 2048, numX 262144
+        numK, numX = 2048, 262144
+        k = rng.uniform(-0.5, 0.5, (numK, 3)).astype(np.float32)
+        phi = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+        kv = np.concatenate([k, (phi[0] * phi[0] + phi[1] * phi[1])[:, None]], 1).astype(np.float32)
+        ta.mriq_set_kvalues(kv)
+        xyz = [torch.from_numpy(rng.uniform(-0.5, 0.5, numX).astype(np.float32)).cuda() for _ in range(3)]
+        Qr, Qi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+        be_ori = ta.ori_mriq_create(numK, xyz[0], xyz[1], xyz[2], Qr, Qi)
+        nblk = numX // 256
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "valu", "pairs": float(numK) * numX}
+        label = "configs[3]: tzgemm 2048^3 + mri-q numK 2048, numX 262144"
+    be = ta.gptb_create(be_ori, 0, 0, 0, nblk)
+    mix = ta.mix_create(be, tz, 0, nblk, 0, tiles)
+    # the slice TaskManager would co-locate with this GEMM: tiles x block_ratio(K) best-effort blocks
+    gemm_k = 1024 if name == "lbm" else 2048
+    ratio = ta.lib().tacker_qos_block_ratio(name.encode(), gemm_k)
+    slice_blocks = min(int(tiles * ratio), nblk)
+    be_slice = ta.gptb_create(be_ori, 0, 0, 0, max(slice_blocks, 1))
+    mix_slice = ta.mix_create(be, tz, 0, slice_blocks, 0, tiles)
+    e0, e1 = ta.Event(), ta.Event()
+    n = 200
+
+    def timed(fn):
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(n):
+            fn()
+        e1.record(stream)
+        e1.synchronize()
+        return e0.elapsed_ms(e1) / n * 1e3
+
+    def serial():
+        tz.execute(stream)
+        be.execute(stream)
+
+    def serial_slice():
+        tz.execute(stream)
+        be_slice.execute(stream)
+
+    cases = {"gemm_us": lambda: tz.execute(stream), "be_us": lambda: be.execute(stream), "serial_us": serial,
+             "fused_us": lambda: mix.execute(stream)}
+    if slice_blocks > 0:
+        cases["slice_serial_us"] = serial_slice
+        cases["slice_fused_us"] = lambda: mix_slice.execute(stream)
+    rounds = {key: [] for key in cases}
+    for _ in range(3):
+        for key, fn in cases.items():
+            rounds[key].append(timed(fn))
+    out = {key: round(statistics.median(v), 2) for key, v in rounds.items()}
+    out["workload"] = label
+    out["speedup"] = round(out["serial_us"] / out["fused_us"], 4)
+    out["slice_blocks"] = slice_blocks
+    out["be_blocks"] = nblk
+    if slice_blocks > 0:
+        out["slice_speedup"] = round(out["slice_serial_us"] / out["slice_fused_us"], 4)
+    out["gemm_tflops_alone"] = round(flop / out["gemm_us"] / 1e6, 1)
+    if work["bound"] == "hbm":
+        out["be_gbps_alone"] = round(work["algorithmic_bytes"] / out["be_us"] / 1e3, 1)
+        out["be_frac_of_hbm_peak"] = round(work["algorithmic_bytes"] / (out["be_us"] * 1e-6) / HBM_PEAK, 4)
+    else:
+        out["be_gpairs_per_s_alone"] = round(work["pairs"] / out["be_us"] / 1e3, 1)
+    return out
+
+
+def lc_leg(ta, torch, np, queries):
+    """BASELINE config 5: VGG16 batch 1 (224x224) as the latency-critical task, stencil 512x512x64 as
+    the best-effort stream, driven by TaskManager; query latency alone and co-located."""
+    task = ta.LcTask("vgg16")
+    tm = ta.TaskManager(task, "stencil", "lbm")
+    tm.configure(qos_budget_ms=50.0, guard_ms=4.0, warmup=5, profile=100, queries=queries, verbose=0)
+    rep = tm.run("aker", second_stage=True)
+    torch.cuda.synchronize()
+    co = np.array(tm.latencies())
+    solo = np.array(tm.latencies(solo=True))
+    out = {"workload": "configs[4]: VGG16 batch 1 224x224 (convs and FCs on tzgemm) + stencil 512x512x64 "
+                       "blocks co-located by TaskManager (Aker mode)",
+           "queries": int(len(co)), "solo_queries": int(len(solo)),
+           "solo_p50_ms": round(float(np.percentile(solo, 50)), 4),
+           "solo_p99_ms": round(float(np.percentile(solo, 99)), 4),
+           "colocated_p50_ms": round(float(np.percentile(co, 50)), 4),
+           "colocated_p99_ms": round(float(np.percentile(co, 99)), 4),
+           "qos_bound_ms": round(1.2 * float(np.percentile(solo, 99)), 4),
+           "qos_budget_ms": 50.0,
+           "mixed_launches_per_query": rep["mix_times"], "mixable_launches_per_query": rep["mixable_times"],
+           "be_blocks_per_query": rep["be_blocks_executed"], "time_earned_ms_per_query": round(rep["time_earned_ms"], 4)}
+    out["p99_within_bound"] = bool(out["colocated_p99_ms"] <= out["qos_bound_ms"])
+    tm.close()
+    task.close()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -69,6 +189,9 @@ def main():
     ap.add_argument("--variant", default=None, help="fused kernel variant (default: kinfo)")
     ap.add_argument("--grid", type=int, default=0, help="fused launch grid (default: kinfo gridsize x CUs)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the other pairs (configs 3, 4) and the co-location latency leg (config 5)")
+    ap.add_argument("--queries", type=int, default=1000, help="latency-critical queries of the co-location leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1",
@@ -182,6 +305,9 @@ def main():
         "wall_s_timed_region": round(t_wall, 3),
     }
     out["config"]["fused_kernel"] = "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)")
+    if not args.no_extras:
+        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq")}
+        out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(A, B, A0, c0, c1)
     print(json.dumps(out))

@@ -1,0 +1,128 @@
+#!/usr/bin/env python3
+"""Measure the load ratio of every fused pair on the GPU and write it into the kernel-info
+defaults: for a tzgemm of reduction length K, how many best-effort blocks per GEMM tile
+should ride along in one fused launch.
+
+Stands for the reference's load-ratio experiments (fusion/expr_load_ratio/*.py: sweep the
+best-effort block count of a fused kernel, keep the count at which both halves finish
+together) and the table they feed (`block_ratio` and the per-K entries TaskManager looks up,
+src/TaskManager.cu:593-600).  Instead of recompiling one .cu per point, the fused kernels of
+this build take their ranges as launch parameters, so a sweep is a loop of launches.
+
+Two steps, because the GPU box and the build tree are different places:
+    python profile_ratio.py --measure out.json          # on the GPU
+    python profile_ratio.py --apply out.json            # rewrites defaults.json; then gen_run.py
+Method per (pair, K): GEMM 2048 x 2048 x K (1024 tiles, one 128x128 macro tile per CU).
+t0 = fused launch with no best-effort block, t_be = the best-effort kernel alone (all N
+blocks).  For nb on a ladder of block counts, earned(nb) = t0 + t_be * nb / N - t_fused(nb)
+is the time one fused launch saves over the two serial launches (the quantity TaskManager
+credits, src/TaskManager.cu:626-640).  The ratio is nb / 1024 for the nb with the largest
+earned time among those whose launch stays within (1 + stretch) * t0, i.e. the
+latency-critical GEMM is never stretched by more than that factor; 0 if nothing earns.
+"""
+import argparse
+import json
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.abspath(os.path.join(HERE, "..", "..", ".."))
+DEFAULTS = os.path.join(HERE, "defaults.json")
+# reduction lengths of the VGG16 batch-1 layers after padding to 128, plus the benchmark's
+K_LADDER = (128, 640, 1152, 2048, 2304, 4096, 4608)
+PAIRS = ("stencil", "lbm", "mriq", "cp")
+TILES = 1024
+LADDER = 16          # best-effort block counts tried: N/16, 2N/16, ..., N
+
+
+def measure(out_path, stretch, launches):
+    sys.path.insert(0, ROOT)
+    import torch
+    import tacker_amd as ta
+
+    ta.init(0)
+    e0, e1 = ta.Event(), ta.Event()
+
+    def timed(kernel):
+        for _ in range(10):
+            kernel.execute()
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(launches):
+            kernel.execute()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_ms(e1) / launches * 1e3
+
+    result = {"stretch": stretch, "tiles": TILES, "device": ta.device_name(), "pairs": {}}
+    for be_name in PAIRS:
+        be = ta.create_kernel(be_name)
+        be_total = be.info()["ptb_end"]
+        be_us = timed(be)
+        table = {}
+        for K in K_LADDER:
+            A = (torch.rand((2048, K), device="cuda") * 2 - 1).half()
+            B = (torch.rand((2048, K), device="cuda") * 2 - 1).half()
+            Cm = torch.zeros((2048, 2048), device="cuda")
+            tz = ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, TILES)
+            mix = ta.mix_create(be, tz, 0, 0, 0, TILES)
+            t0 = timed(mix)
+            best = {"blocks": 0, "earned_us": 0.0, "fused_us": t0}
+            for step in range(1, LADDER + 1):
+                nb = be_total * step // LADDER
+                mix.set_range(0, nb, 0, TILES)
+                t = timed(mix)
+                earned = t0 + be_us * nb / be_total - t
+                if t <= (1 + stretch) * t0 and earned > best["earned_us"]:
+                    best = {"blocks": nb, "earned_us": earned, "fused_us": t}
+            table[str(K)] = {"blocks": best["blocks"], "ratio": round(best["blocks"] / TILES, 4),
+                             "gemm_in_fused_us": round(t0, 2), "fused_us": round(best["fused_us"], 2),
+                             "earned_us": round(best["earned_us"], 2)}
+            print(f"tzgemm_{be_name} K={K}: t0 {t0:.1f} us, best {best['blocks']} of {be_total} blocks "
+                  f"(fused {best['fused_us']:.1f} us, earns {best['earned_us']:.1f} us) "
+                  f"-> ratio {best['blocks'] / TILES:.4f}", flush=True)
+        result["pairs"]["tzgemm_" + be_name] = {"be_total_blocks": be_total, "be_solo_us": round(be_us, 2),
+                                                "by_k": table}
+    with open(out_path, "w") as f:
+        json.dump(result, f, indent=1)
+    print("wrote", out_path)
+
+
+def apply(in_path):
+    with open(in_path) as f:
+        meas = json.load(f)
+    with open(DEFAULTS) as f:
+        dflt = json.load(f)
+    for key, m in meas["pairs"].items():
+        entry = dflt[key]
+        entry["ratio_by_k"] = {k: v["ratio"] for k, v in m["by_k"].items()}
+        entry["block_ratio"] = m["by_k"]["4096"]["ratio"]
+    dflt["ratio_provenance"] = {"stretch": meas["stretch"], "device": meas["device"],
+                                "method": "profile_ratio.py: GEMM 2048x2048xK; best-effort block count with "
+                                          "the largest time earned over serial launches whose fused launch "
+                                          "stays within (1+stretch) of the launch without best-effort "
+                                          "blocks, divided by 1024 tiles"}
+    with open(DEFAULTS, "w") as f:
+        json.dump(dflt, f, indent=4)
+        f.write("\n")
+    print("updated", DEFAULTS, "- now run gen_run.py and rebuild")
+
+
+def main():
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--measure", metavar="OUT.json")
+    ap.add_argument("--apply", metavar="IN.json")
+    ap.add_argument("--stretch", type=float, default=1.0,
+                    help="largest tolerated stretch of the GEMM's launch (1.0 = at most twice as long)")
+    ap.add_argument("--launches", type=int, default=100)
+    args = ap.parse_args()
+    if args.measure:
+        measure(args.measure, args.stretch, args.launches)
+    elif args.apply:
+        apply(args.apply)
+    else:
+        ap.error("one of --measure / --apply")
+
+
+if __name__ == "__main__":
+    main()

@@ -96,7 +96,8 @@ def test_block_ratio_table_and_k_extrapolation(fake):
     assert fake.tacker_qos_block_ratio(b"stencil", 1152) == pytest.approx(
         fake.tacker_fget_kernel_info(b"tzgemm_stencil", b"1152"))
     # K absent from the table: the K=4096 entry scaled by K/4096 (src/TaskManager.cu:593-598)
-    assert fake.tacker_qos_block_ratio(b"stencil", 2048) == pytest.approx(r4096 * 2048 / 4096)
+    assert fake.tacker_fget_kernel_info(b"tzgemm_stencil", b"3072") == float(ta.JSON_NOT_FOUND)
+    assert fake.tacker_qos_block_ratio(b"stencil", 3072) == pytest.approx(r4096 * 3072 / 4096)
     assert fake.tacker_qos_block_ratio(b"stencil", 8192) == pytest.approx(r4096 * 2)
 
 
