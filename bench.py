@@ -2,7 +2,7 @@
 """Benchmark of the hot path on one MI355X: the fused tzgemm + stencil launch
 against serial launches of the same two kernels.
 
-Workload (BASELINE config 2): tzgemm fp16 2048x2048x2048 (uniform[-1,1], fp32
+Workload (benchmark configuration 2): tzgemm fp16 2048x2048x2048 (uniform[-1,1], fp32
 accumulate, alpha 1.1) + Parboil 7-point Jacobi stencil on an fp32 512x512x64 grid
 (uniform[0,1], c0=1/6, c1=1/36), 100 iterations with pointer swap.  One "step" is
 the whole 100-iteration job: serial = 100 x (1 GEMM launch + 1 sweep launch) on one
@@ -62,7 +62,7 @@ def cpu_baseline(A, B, A0, c0, c1):
 
 
 def pair_leg(ta, torch, np, name, stream):
-    """One of the other fused pairs (BASELINE configs 3 and 4): each kernel alone, serial, and the
+    """One of the other fused pairs (benchmark configurations 3 and 4): each kernel alone, serial, and the
     fused launch over the full ranges, 200 launches each, median of 3 rounds."""
     import statistics
     rng = np.random.default_rng(1337)
@@ -155,7 +155,7 @@ def pair_leg(ta, torch, np, name, stream):
 
 
 def lc_leg(ta, torch, np, queries):
-    """BASELINE config 5: VGG16 batch 1 (224x224) as the latency-critical task, stencil 512x512x64 as
+    """benchmark configuration 5: VGG16 batch 1 (224x224) as the latency-critical task, stencil 512x512x64 as
     the best-effort stream, driven by TaskManager; query latency alone and co-located."""
     task = ta.LcTask("vgg16")
     tm = ta.TaskManager(task, "stencil", "lbm")

@@ -13,7 +13,7 @@ def test_dims_known_answers_from_reference_files():
         assert oracle.tzgemm_dims(128, 128, k_in)[2] == k_out
     # src/Creator.cu:255-261: OriTZGEMMKernel(12800, 512, 4096)
     assert oracle.tzgemm_dims(12800, 512, 4096) == [12800, 512, 4096, 200 * 8]
-    # BASELINE config 1: 1024^3 -> 256 CTA tiles of 64x64
+    # benchmark configuration 1: 1024^3 -> 256 CTA tiles of 64x64
     assert oracle.tzgemm_dims(1024, 1024, 1024) == [1024, 1024, 1024, 256]
     # floor, not round; minimum 128 (src/tzgemm_kernel.h:31-33)
     assert oracle.tzgemm_dims(3136, 64, 255) == [3072, 128, 128, 48 * 2]
