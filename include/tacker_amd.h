@@ -255,6 +255,16 @@ TK_API tacker_kernel_t tacker_mix_create(tacker_kernel_t be_gptb, tacker_kernel_
                                          const char *variant, int launch_grid, int launch_block);
 TK_API int tacker_mix_set_range(tacker_kernel_t mix, int be_start, int be_end, int tile_start,
                                 int tile_end);
+/* new MixKernel(id, "<first>_<second>", first, second, grid, block, start1, end1, start2, end2)
+ * for two best-effort kernels, first < second alphabetically, with grid and block from
+ * kinfo (the constructor calls inside createMixKernel, src/Creator.cu:346-356).
+ * tacker_mix_set_range applies to the result: (start1, end1, start2, end2). */
+TK_API tacker_kernel_t tacker_be_pair_create(tacker_kernel_t first_gptb, tacker_kernel_t second_gptb,
+                                             int start1, int end1, int start2, int end2,
+                                             const char *variant, int launch_grid);
+/* createMixKernel(name) (src/Creator.cu:341-816): the memoised fused pair "<a>_<b>" of the
+ * memoised kernels createKernel(a), createKernel(b) over their full ranges. Never destroy. */
+TK_API tacker_kernel_t tacker_create_mix_kernel(const char *name);
 /* Kernel::execute(stream) */
 TK_API int tacker_kernel_execute(tacker_kernel_t kernel, tkStream_t stream);
 /* exchange the input and output grid of a stencil / lbm ori object (the
@@ -317,6 +327,9 @@ TK_API int tacker_task_manager_run(tacker_task_manager_t tm, int mode, tkStream_
  * mixable_times, time_earned_ms, qos_headroom_left_ms, stage1_be_ms, stage2_be_ms,
  * be_task_finish_num, n co-located latencies, n solo latencies} */
 TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
+/* "[Mix] BE task1 + task2 took ..." (src/TaskManager.cu:693): average time of the fused launch of
+ * the two best-effort kernels measured by the last run with a second stage; 0 if none ran. */
+TK_API float tacker_task_manager_be_mix_ms(tacker_task_manager_t tm);
 /* which = 0: per-query latency of the co-located queries, 1: of the solo profiling queries */
 TK_API int tacker_task_manager_latencies(tacker_task_manager_t tm, int which, float *out, int cap);
 

@@ -61,7 +61,8 @@ def _declare(lib):
     lib.tacker_fget_kernel_info.restype = f
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
                  "tacker_ori_mriq_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
-                 "tacker_gptb_create", "tacker_mix_create"):
+                 "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
+                 "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
     lib.tacker_create_kernel.argtypes = [cp]
     lib.tacker_ori_stencil_create.argtypes = [f, f, vp, vp, i, i, i]
@@ -73,6 +74,8 @@ def _declare(lib):
     lib.tacker_gptb_set_range.argtypes = [vp, i, i]
     lib.tacker_mix_create.argtypes = [vp, vp, i, i, i, i, cp, i, i]
     lib.tacker_mix_set_range.argtypes = [vp, i, i, i, i]
+    lib.tacker_be_pair_create.argtypes = [vp, vp, i, i, i, i, cp, i]
+    lib.tacker_create_mix_kernel.argtypes = [cp]
     lib.tacker_kernel_execute.argtypes = [vp, vp]
     lib.tacker_kernel_swap_buffers.argtypes = [vp]
     lib.tacker_kernel_info.argtypes = [vp, C.POINTER(i)]
@@ -99,6 +102,8 @@ def _declare(lib):
     lib.tacker_task_manager_run.argtypes = [vp, i, vp, i]
     lib.tacker_task_manager_report.argtypes = [vp, C.POINTER(f)]
     lib.tacker_task_manager_latencies.argtypes = [vp, i, C.POINTER(f), i]
+    lib.tacker_task_manager_be_mix_ms.argtypes = [vp]
+    lib.tacker_task_manager_be_mix_ms.restype = f
     lib.tacker_qos_block_ratio.argtypes = [cp, i]
     lib.tacker_qos_block_ratio.restype = f
     lib.tacker_qos_colocated_blocks.argtypes = [i, cp, i, i, i]
@@ -435,6 +440,17 @@ def mix_create(be_gptb, tz_gptb, be_start, be_end, tile_start, tile_end, variant
                                                 launch_block), "MixKernel", keep=(be_gptb, tz_gptb))
 
 
+def be_pair_create(first_gptb, second_gptb, start1, end1, start2, end2, variant=None, launch_grid=0):
+    """Fused launch of two best-effort GPTB kernels (first < second alphabetically)."""
+    return KernelHandle(lib().tacker_be_pair_create(first_gptb.handle, second_gptb.handle, start1, end1,
+                                                    start2, end2, _v(variant), launch_grid),
+                        "MixKernel", keep=(first_gptb, second_gptb))
+
+
+def create_mix_kernel(name):
+    return KernelHandle(lib().tacker_create_mix_kernel(name.encode()), f"createMixKernel({name})", owned=False)
+
+
 # ----------------------------------------------------------------------------- events
 class Event:
     """tkEvent (hipEvent) recorded on the stream the kernels are launched on."""
@@ -574,6 +590,9 @@ class TaskManager:
         out = (C.c_float * 13)()
         self.l.tacker_task_manager_report(self.h, out)
         return dict(zip(REPORT_KEYS, out))
+
+    def be_mix_ms(self):
+        return self.l.tacker_task_manager_be_mix_ms(self.h)
 
     def latencies(self, solo=False):
         cap = 1 << 20

@@ -86,10 +86,37 @@ MixKernel *createTzgemmMix(GPTBKernel *be, GPTBKernel *tz, int be_start, int be_
     return new MixKernel(1, key, be, tz, dim3(grid, 1, 1), dim3(bs, 1, 1), be_start, be_end, tile_start, tile_end);
 }
 
-// Best-effort x best-effort pairs are not part of the tzgemm path.
+MixKernel *createBePairMix(GPTBKernel *first, GPTBKernel *second, int start1, int end1, int start2, int end2,
+                           const std::string &variant, int launch_grid)
+{
+    const std::string base = first->kernelName + "_" + second->kernelName;
+    const std::string key = variant.empty() ? base : base + "@" + variant;
+    const int per_cu = get_kernel_info(key, "gridsize");
+    const int bs = get_kernel_info(key, "blocksize");
+    int group = get_kernel_info(key, "group");
+    if (per_cu == JSON_NOT_FOUND || bs == JSON_NOT_FOUND) logger.ERROR("kinfo has no entry for {" + key + "}");
+    if (group == JSON_NOT_FOUND || group < 1) group = 1;
+    int grid = launch_grid > 0 ? launch_grid : cuCount() * per_cu;
+    const int quantum = 8 * group;   // whole groups on every XCD
+    if (grid % quantum) grid = (grid / quantum + 1) * quantum;
+    return new MixKernel(2, key, first, second, dim3(grid, 1, 1), dim3(bs, 1, 1), start1, end1, start2, end2);
+}
+
+// "<a>_<b>" with a < b alphabetically (src/Creator.cu:341-816 lists its pairs one by one;
+// here every pair of the four best-effort kernels exists): both kernels over their full
+// ranges, memoised.
 MixKernel *createMixKernel(const std::string &name)
 {
     auto hit = mixKernelMap.find(name);
     if (hit != mixKernelMap.end()) return hit->second;
-    logger.ERROR("Creator: Mix kernel not found: " + name);
+    const size_t cut = name.find('_');
+    if (cut == std::string::npos || get_kernel_info(name, "blocksize") == JSON_NOT_FOUND)
+        logger.ERROR("Creator: Mix kernel not found: " + name);
+    GPTBKernel *first = createKernel(name.substr(0, cut));
+    GPTBKernel *second = createKernel(name.substr(cut + 1));
+    MixKernel *mix = createBePairMix(first, second, first->gptbParams.ptb_start_block_pos,
+                                     first->gptbParams.ptb_end_block_pos, second->gptbParams.ptb_start_block_pos,
+                                     second->gptbParams.ptb_end_block_pos, "", 0);
+    mixKernelMap[name] = mix;
+    return mix;
 }

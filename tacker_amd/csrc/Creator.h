@@ -23,5 +23,10 @@ MixKernel *createMixKernel(const std::string &name);
 MixKernel *createTzgemmMix(GPTBKernel *be, GPTBKernel *tz, int be_start, int be_end, int tile_start,
                            int tile_end, const std::string &variant, int launch_grid, int launch_block);
 
+// Fused launch of two best-effort kernels (first < second alphabetically), kinfo key
+// "<first>_<second>[@variant]".
+MixKernel *createBePairMix(GPTBKernel *first, GPTBKernel *second, int start1, int end1, int start2, int end2,
+                           const std::string &variant, int launch_grid);
+
 // compute units of the current device (cached tkGetCuCount)
 int cuCount();

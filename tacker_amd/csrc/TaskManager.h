@@ -61,6 +61,7 @@ struct TaskManagerReport {
     float time_earned_ms = 0.0f;
     float qos_headroom_left_ms = 0.0f;
     float stage1_be_ms = 0.0f, stage2_be_ms = 0.0f;
+    float be_mix_ms = 0.0f;             // fused launch of the two BE kernels (0 if the pair has no kernel)
     std::vector<float> query_latency_ms;   // one entry per co-located LC query
     std::vector<float> solo_latency_ms;    // one entry per solo LC query (profiling passes)
 };

@@ -515,6 +515,37 @@ tacker_kernel_t tacker_mix_create(tacker_kernel_t be_h, tacker_kernel_t tz_h, in
            createTzgemmMix(be, tz, be_start, be_end, tile_start, tile_end, v, launch_grid, launch_block));
 }
 
+tacker_kernel_t tacker_be_pair_create(tacker_kernel_t first_h, tacker_kernel_t second_h, int start1, int end1,
+                                      int start2, int end2, const char *variant, int launch_grid)
+{
+    GPTBKernel *a = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(first_h));
+    GPTBKernel *b = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(second_h));
+    if (!a || !b || a->kernelName == "tzgemm" || b->kernelName == "tzgemm" || !(a->kernelName < b->kernelName)) {
+        fail(TK_ERROR_INVALID_VALUE,
+             "tacker_be_pair_create: need two different best-effort GPTB kernels, first < second alphabetically");
+        return nullptr;
+    }
+    const std::string v = variant ? variant : "";
+    const std::string key = a->kernelName + "_" + b->kernelName + (v.empty() ? "" : "@" + v);
+    if (!has_key(key) || get_kernel_info(key, "blocksize") == JSON_NOT_FOUND) {
+        fail(TK_ERROR_NOT_FOUND, "no fused kernel {" + key + "}");
+        return nullptr;
+    }
+    CREATE(check_range(a->kernel_, start1, end1) || check_range(b->kernel_, start2, end2),
+           createBePairMix(a, b, start1, end1, start2, end2, v, launch_grid));
+}
+
+tacker_kernel_t tacker_create_mix_kernel(const char *name)
+{
+    const std::string n = name ? name : "";
+    if (n.find('_') == std::string::npos || !has_key(n) || get_kernel_info(n, "blocksize") == JSON_NOT_FOUND ||
+        n.rfind("tzgemm_", 0) == 0) {
+        fail(TK_ERROR_NOT_FOUND, "createMixKernel: no best-effort pair {" + n + "}");
+        return nullptr;
+    }
+    CREATE(TK_SUCCESS, createMixKernel(n));
+}
+
 int tacker_mix_set_range(tacker_kernel_t h, int be_start, int be_end, int tile_start, int tile_end)
 {
     MixKernel *m = dynamic_cast<MixKernel *>(static_cast<Kernel *>(h));
@@ -764,6 +795,12 @@ int tacker_task_manager_report(tacker_task_manager_t h, float out[13])
                          (float)r.query_latency_ms.size(), (float)r.solo_latency_ms.size()};
     memcpy(out, v, sizeof(v));
     return TK_SUCCESS;
+}
+
+float tacker_task_manager_be_mix_ms(tacker_task_manager_t h)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    return tm ? tm->report.be_mix_ms : -1.0f;
 }
 
 int tacker_task_manager_latencies(tacker_task_manager_t h, int which, float *out, int cap)

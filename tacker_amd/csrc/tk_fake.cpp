@@ -182,6 +182,14 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
             for (auto v : variants)
                 add((std::string("tzgemm_") + be.first + v).c_str(),
                     cat(cat(*be.second, trailer(false)), cat(TZ, trailer(false))));
+        // best-effort pairs, first < second alphabetically
+        static const char *pair_variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1"};
+        for (auto &a : bes)
+            for (auto &b : bes)
+                if (std::string(a.first) < std::string(b.first))
+                    for (auto v : pair_variants)
+                        add((std::string(a.first) + "_" + b.first + v).c_str(),
+                            cat(cat(*a.second, trailer(false)), cat(*b.second, trailer(false))));
     }
     for (auto *k : kernels()) insert(k->key.c_str(), k, ctx);
     return TK_SUCCESS;

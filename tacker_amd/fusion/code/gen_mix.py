@@ -110,6 +110,44 @@ extern "C" __global__ __launch_bounds__({total}) void {name}(
     return text, meta
 
 
+def be_pair_kernel_name(be1, be2, variant):
+    return f"{be1}_{be2}_mix_{variant}"
+
+
+def generate_be_pair(be1, be2, wgs1, wgs2, threads=256):
+    """Fused kernel of two vector kernels (no tzgemm): workgroup split wgs1 : wgs2.
+
+    Neither role uses LDS or a barrier, so workgroups of both kinds share a CU freely; the
+    split only fixes the proportion in which the launch's persistent workgroups serve the
+    two kernels (``createMixKernel`` pairs of the reference, src/Creator.cu:341-816).
+    Parameter order: be1's GPTB list, then be2's; be1 < be2 alphabetically, as the
+    reference names its pairs.
+    """
+    variant = f"wg_{wgs1}_{wgs2}"
+    p1, sig1 = signature(be1, 0)
+    p2, sig2 = signature(be2, 1)
+    call1 = ROLES[be1]["call"].format(p=p1, block="sp.role_block", blocks="sp.role_blocks",
+                                      tid="(int)threadIdx.x", threads=threads)
+    call2 = ROLES[be2]["call"].format(p=p2, block="sp.role_block", blocks="sp.role_blocks",
+                                      tid="(int)threadIdx.x", threads=threads)
+    name = be_pair_kernel_name(be1, be2, variant)
+    text = f"""// {be1}-{be2}  workgroup split  {wgs1} {be1} : {wgs2} {be2} workgroups per group
+extern "C" __global__ __launch_bounds__({threads}) void {name}(
+    {_params_text(sig1, sig2)})
+{{
+{_void_unused(sig1 + sig2, call1 + call2)}    const tk::WgSplit sp = tk::wg_split((int)blockIdx.x, (int)gridDim.x, {wgs1}, {wgs2});
+    if (sp.role == 0) {{
+        {call1}
+    }} else {{
+        {call2}
+    }}
+}}
+"""
+    meta = {"variant": variant, "symbol": name, "blocksize": threads, "group": wgs1 + wgs2,
+            "share1": wgs1, "share2": wgs2, "kind": "wg"}
+    return text, meta
+
+
 def generate_pair(be, candidates):
     """All fused kernels of one (be, tzgemm) pair: yields (text, meta)."""
     for cand in candidates:

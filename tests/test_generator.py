@@ -101,3 +101,24 @@ def test_kinfo_emitted_for_every_variant():
         assert f"tzgemm_{be}@{base['variant']}" in kinfo
         assert {"register", "shared_memory", "blocksize", "solo_ptb_blks", "ori_blks"} <= set(kinfo[be])
     assert set(kinfo["throughput_test"]) == {"a", "b"}
+
+
+def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
+    files = gen_run.generate()
+    kinfo = json.loads(files["../config/kinfo-gfx950.json"])
+    pairs = gen_run.be_pairs()
+    assert pairs == [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"), ("lbm", "stencil"),
+                     ("mriq", "stencil")]
+    assert ("lbm", "mriq") in pairs                       # the pair src/Creator.cu:341-816 also has
+    for a, b in pairs:
+        text = files[f"mix_kernel/{a}_{b}.hip"]
+        for w1, w2 in gen_run.BE_PAIR_SPLITS:
+            sym = f"{a}_{b}_mix_wg_{w1}_{w2}"
+            assert f"void {sym}(" in text
+            entry = kinfo[f"{a}_{b}@wg_{w1}_{w2}"]
+            assert entry["group"] == w1 + w2 and entry["blocksize"] == 256
+        assert kinfo[f"{a}_{b}"]["variant"] in ("wg_1_1", "wg_1_2", "wg_2_1")
+        assert f'insert("{a}_{b}", ' in files["mix_kernel/mix_kernels.inc"]
+        # parameter order: the first kernel's list, then the second's
+        assert text.index(f"{a}0_grid_dimension_x") < text.index(f"{b}1_grid_dimension_x")
+    assert "__shared__" not in files["mix_kernel/lbm_mriq.hip"]        # no role of a pair uses LDS

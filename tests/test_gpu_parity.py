@@ -349,3 +349,48 @@ def test_mix_tzgemm_cp(variant):
     ta.mix_tzgemm_cp(64, 0.1, g, dev(A), dev(B), mix_c, variant=variant)
     assert np.array_equal(host(mix_c), host(solo_c))
     assert np.array_equal(host(g).view(np.uint32), oracle.cp(info, np.zeros((32, 512), np.float32)).view(np.uint32))
+
+
+# ------------------------------------------------------------------ best-effort x best-effort pairs
+def _small_be(name):
+    """(ori kernel, blocks, output tensors, snapshot of the outputs before any launch)"""
+    if name == "stencil":
+        A0 = stencil_inputs(6, 20, 200, seed=31)
+        a0 = dev(A0)
+        out = a0.clone()
+        return ta.ori_stencil_create(C0, C1, a0, out), ta.stencil_blocks(200, 20), [out]
+    if name == "lbm":
+        src = dev(lbm_inputs(120, 6, 5, seed=32))
+        dst = torch.zeros_like(src)
+        return ta.ori_lbm_create(src, dst, 120, 6, 5), 30, [dst]
+    if name == "mriq":
+        k, phiR, phiI, xyz = mriq_inputs(256, 2048, seed=33)
+        kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+        ta.mriq_set_kvalues(kv)
+        Qr, Qi = torch.zeros(2048, device="cuda:0"), torch.zeros(2048, device="cuda:0")
+        return ta.ori_mriq_create(256, dev(xyz[0]), dev(xyz[1]), dev(xyz[2]), Qr, Qi), 8, [Qr, Qi]
+    ta.cp_set_atoms(cp_atoms(), 0.0)
+    g = torch.zeros((32, 512), device="cuda:0")
+    return ta.ori_cp_create(64, 0.1, g), (512 // 128) * (32 // 8), [g]
+
+
+@pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),
+                                          ("lbm", "stencil"), ("mriq", "stencil")])
+@pytest.mark.parametrize("variant", [None, "wg_1_2", "wg_2_1"])
+def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
+    ori1, n1, outs1 = _small_be(first)
+    ori2, n2, outs2 = _small_be(second)
+    outs = outs1 + outs2
+    before = [o.clone() for o in outs]
+    r1 = (1, n1 - 1) if n1 > 2 else (0, n1)          # a partial range of the first kernel
+    g1 = ta.gptb_create(ori1, 0, 0, r1[0], r1[1])
+    g2 = ta.gptb_create(ori2, 0, 0, 0, n2)
+    g1.execute()
+    g2.execute()
+    want = [host(o).copy() for o in outs]
+    for o, b in zip(outs, before):
+        o.copy_(b)
+    mix = ta.be_pair_create(ta.gptb_create(ori1, 0, 0, 0, n1), g2, r1[0], r1[1], 0, n2, variant=variant, launch_grid=48)
+    mix.execute()
+    for o, w in zip(outs, want):
+        assert np.array_equal(host(o).view(np.uint32), w.view(np.uint32))

@@ -244,6 +244,48 @@ def test_mix_follows_ori_buffer_swap_but_not_gptb_range_edits(fake):
     assert [as_int(launches(fake)[-1]["args"][13]), as_int(launches(fake)[-1]["args"][15])] == [1, 2]
 
 
+def test_best_effort_pair_parameter_vector_and_geometry(fake):
+    # [first's params + 6 dims][start1, step, end1][second's params + 6 dims][start2, step, end2]
+    fake.tk_fake_reset()
+    fake.tk_fake_set_cu_count(256)
+    a0 = np.zeros((6, 10, 70), np.float32)
+    grid = np.zeros(20 * 16 * 4 * 3 + 4096, np.float32)
+    st_ori = fake.tacker_ori_stencil_create(0.5, 0.25, a0.ctypes.data, a0.ctypes.data, 70, 10, 6)
+    st = fake.tacker_gptb_create(st_ori, 0, 0, 0, 6)
+    lb_ori = fake.tacker_ori_lbm_create(grid.ctypes.data, grid.ctypes.data, 16, 4, 3)
+    lb = fake.tacker_gptb_create(lb_ori, 0, 0, 0, 12)
+    assert not fake.tacker_be_pair_create(st, lb, 0, 6, 0, 12, None, 0)          # stencil > lbm: wrong order
+    assert b"alphabetically" in fake.tacker_last_error()
+    assert not fake.tacker_be_pair_create(lb, st, 5, 4, 0, 6, None, 0)           # end before start
+    assert not fake.tacker_be_pair_create(lb, st, 0, 12, 0, 6, b"wg_9_9", 0)
+    mix = fake.tacker_be_pair_create(lb, st, 2, 12, 1, 6, b"wg_1_2", 0)
+    assert mix, fake.tacker_last_error()
+    assert fake.tacker_kernel_execute(mix, None) == 0
+    l = launches(fake)[-1]
+    assert l["key"] == "lbm_stencil@wg_1_2" and len(l["args"]) == (2 + 6 + 3) + (7 + 6 + 3)
+    per_cu = fake.tacker_get_kernel_info(b"lbm_stencil@wg_1_2", b"gridsize")
+    want_grid = 256 * per_cu
+    want_grid += (-want_grid) % (8 * 3)                                          # whole 1:2 groups on every XCD
+    assert l["grid"][0] == want_grid and l["block"][0] == 256
+    assert [as_int(l["args"][i]) for i in (8, 9, 10)] == [2, want_grid, 12]      # lbm start, step, end
+    assert [as_int(l["args"][i]) for i in (24, 25, 26)] == [1, want_grid, 6]     # stencil start, step, end
+    assert [as_ptr(x) for x in l["args"][13:15]] == [a0.ctypes.data, a0.ctypes.data]
+
+
+def test_create_mix_kernel_is_memoised_and_uses_the_creator_kernels(fake):
+    fake.tk_fake_set_cu_count(256)
+    m1 = fake.tacker_create_mix_kernel(b"lbm_mriq")
+    assert m1 and m1 == fake.tacker_create_mix_kernel(b"lbm_mriq")
+    fake.tk_fake_reset()
+    assert fake.tacker_kernel_execute(m1, None) == 0
+    l = launches(fake)[-1]
+    assert l["key"] == "lbm_mriq" and len(l["args"]) == (2 + 6 + 3) + (7 + 6 + 3)
+    assert (as_int(l["args"][8]), as_int(l["args"][10])) == (0, 18000)           # lbm rows of 120x120x150
+    assert (as_int(l["args"][24]), as_int(l["args"][26])) == (0, 1024)           # mri-q blocks
+    for bad in (b"mriq_lbm", b"lbm", b"tzgemm_stencil", b"fft_lbm"):
+        assert not fake.tacker_create_mix_kernel(bad)
+
+
 def test_argument_validation_returns_codes_instead_of_exiting(fake):
     buf = np.zeros(1024, np.float32)
     p = buf.ctypes.data
@@ -362,6 +404,22 @@ def test_task_manager_fuses_when_budget_allows(fake, small_vgg):
     assert len(lat) == 2 and lat[0] == pytest.approx(0.01 * n, rel=1e-4)
     assert rep["qos_headroom_left_ms"] == pytest.approx(50.0 - 0.01 * n, rel=1e-3)
     assert rep["mix_times"] > 0 and rep["be_blocks_executed"] > 0
+
+
+def test_task_manager_second_stage_credits_the_fused_best_effort_pair(fake, small_vgg):
+    # every timed region takes 10 us, so the fused pair (10 us) beats the two solo launches
+    # (10 + 10 us): the budget left is worth twice as much best-effort time (src/TaskManager.cu:696-697)
+    fake.tk_fake_set_event_ms(0.01)
+    tm = ta.TaskManager(small_vgg, "stencil", "lbm", library=fake)
+    tm.configure(warmup=1, profile=2, verbose=0, qos_budget_ms=50.0, guard_ms=4.0, queries=1)
+    fake.tk_fake_reset()
+    rep = tm.run("aker", raw_stream=None, second_stage=True)
+    assert "lbm_stencil" in [l["key"] for l in launches(fake)]
+    assert tm.be_mix_ms() == pytest.approx(0.01, rel=1e-4)
+    assert rep["stage2_be_ms"] == pytest.approx(2.0 * rep["qos_headroom_left_ms"], rel=1e-4)
+    rep = tm.run("tacker", raw_stream=None, second_stage=True)                   # Tacker mode takes no credit
+    assert rep["stage2_be_ms"] == pytest.approx(rep["qos_headroom_left_ms"], rel=1e-4)
+    tm.close()
 
 
 def test_task_manager_falls_back_to_solo_when_headroom_is_short(fake, small_vgg):
