@@ -17,8 +17,13 @@
 #define TZ_BLOCK_K 64             // K extent of one LDS stage (128-byte tile rows)
 #define TZ_STAGE_BYTES (2 * TZ_MACRO_TILE * TZ_BLOCK_K * 2)   // A rows then B rows: 32 KiB
 #define TZ_STAGES 4               // LDS ring depth where the GEMM has the CU's LDS to itself
-#define TZ_STAGES_WG 3            // ring depth of workgroup-split fused kernels
+#define TZ_STAGES_WG 4            // ring depth of workgroup-split fused kernels
 #define TZ_LDS_BYTES (TZ_STAGES * TZ_STAGE_BYTES)
 #define TZ_LDS_BYTES_WG (TZ_STAGES_WG * TZ_STAGE_BYTES)
+
+// shapes that take the K-split form of the kernel (one reference tile per workgroup, K cut
+// over its 4 waves): few macro tiles for the CUs there are, and a reduction worth cutting
+#define TZ_KSPLIT_MAX_MACRO_TILES 64
+#define TZ_KSPLIT_MIN_K 512
 
 #define TZ_ALPHA 1.1f             // alpha_g, src/header/tzgemm_header.h:64

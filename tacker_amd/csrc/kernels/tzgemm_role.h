@@ -62,7 +62,7 @@ __device__ __forceinline__ void tz_macro_tile_of(int t, int macro_rows, int macr
 #define TK_LGKMCNT0_IMM 0xC07F
 
 template <int STAGES, class Sync>
-__device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
+__device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A,
                                             const _Float16 *__restrict__ B, float *__restrict__ C,
                                             int M, int N, int K, int role_block, int role_blocks,
                                             int tile_start, int tile_end, int tid, char *lds,
@@ -295,6 +295,154 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A,
 #undef TZ_SECOND_STEP
     }
     sync.finish();
+}
+
+// ---------------------------------------------------------------------------------------
+// K-split form for shapes with few output tiles and a long reduction (the batch-1 layers
+// of a network: 8 to 50 macro tiles for 256 CUs, K up to 25088).  The macro-tile form
+// would leave most CUs idle and walk K serially on the rest.  Here a workgroup owns ONE
+// reference 64x64 tile and its 4 waves each reduce a quarter of K into a private 4x4
+// accumulator set, then the four partial tiles are added in LDS in a fixed order
+// (((w0 + w1) + w2) + w3), so the result does not depend on timing.  Four times as many
+// workgroups, each with a K loop a quarter as long.  The waves share no operands, so each
+// has a private two-stage ring (2 x 16 KiB) and the K loop needs no barrier at all.
+// Which form runs depends on (M, N, K) only -- never on the launch geometry -- so a fused
+// launch and the plain kernel always add in the same order.
+__device__ __forceinline__ bool tz_use_ksplit(int M, int N, int K)
+{
+    const int n_macro = (M / TZ_MACRO_TILE) * (N / TZ_MACRO_TILE);
+    return n_macro <= TZ_KSPLIT_MAX_MACRO_TILES && K >= TZ_KSPLIT_MIN_K;
+}
+
+template <class Sync>
+__device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ A,
+                                                   const _Float16 *__restrict__ B, float *__restrict__ C,
+                                                   int M, int N, int K, int role_block, int role_blocks,
+                                                   int tile_start, int tile_end, int tid, char *lds,
+                                                   Sync &sync)
+{
+    typedef __attribute__((address_space(1))) const void *gptr_t;
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    constexpr int BK = TZ_BLOCK_K;
+    constexpr int ROWB = BK * 2;                      // 128-byte tile rows
+    constexpr int OPERAND_BYTES = TZ_REF_TILE * ROWB; // 8 KiB: 64 rows of one operand
+    constexpr int STAGE = 2 * OPERAND_BYTES;          // A rows then B rows
+    constexpr int LOADS = 8;                          // LDS-direct loads per operand and chunk
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int ref_cols = N / TZ_REF_TILE;
+    const int n_ref = (M / TZ_REF_TILE) * ref_cols;
+    const int kchunks = K / BK;
+    const int c_first = (wave * kchunks) / 4;
+    const int c_last = ((wave + 1) * kchunks) / 4;
+    char *mine = lds + wave * (2 * STAGE);            // this wave's two stages
+    // load j of an operand fills rows 8j .. 8j+7: lane lands in row 8j + lane/8, slot lane%8,
+    // and fetches the row's segment slot ^ ((row>>1)&7) = slot ^ (lane>>4) ^ (4*(j&1))
+    const unsigned seg_even = (unsigned)((lane & 7) ^ (lane >> 4));
+    const unsigned src_even = (unsigned)((lane >> 3) * K + (int)seg_even * 8) * 2u;
+    const unsigned src_odd = (unsigned)((lane >> 3) * K + (int)(seg_even ^ 4u) * 8) * 2u;
+    const int frag_key = ((lane & 15) >> 1) & 7;
+    const int frag_seg0 = ((lane >> 4) ^ frag_key) * 16;
+    const int frag_seg1 = ((4 + (lane >> 4)) ^ frag_key) * 16;
+    const int frag_row = (lane & 15) * ROWB;
+    if (tile_end > n_ref) tile_end = n_ref;
+
+    for (int pos = tile_start + role_block; pos < tile_end; pos += role_blocks) {
+        const int ti = pos / ref_cols;
+        const int tj = pos % ref_cols;
+        const char *a_tile = reinterpret_cast<const char *>(A + (size_t)(ti * TZ_REF_TILE) * K);
+        const char *b_tile = reinterpret_cast<const char *>(B + (size_t)(tj * TZ_REF_TILE) * K);
+#define TZK_ISSUE(chunk_, stage_)                                                                  \
+    _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                              \
+    {                                                                                              \
+        char *dst_ = mine + (stage_) * STAGE + j * 1024;                                           \
+        const size_t uni_ = ((size_t)(j * 8) * K + (size_t)(chunk_) * BK) * 2;                     \
+        unsigned lane_ = (j & 1) ? src_odd : src_even;                                             \
+        asm volatile("" : "+v"(lane_));                                                            \
+        __builtin_amdgcn_global_load_lds((gptr_t)(a_tile + uni_ + lane_), (lptr_t)dst_, 16, 0, 0); \
+        __builtin_amdgcn_global_load_lds((gptr_t)(b_tile + uni_ + lane_),                          \
+                                         (lptr_t)(dst_ + OPERAND_BYTES), 16, 0, 0);                \
+    }
+        float4_t acc[4][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+        if (c_first < c_last) { TZK_ISSUE(c_first, 0) }
+        for (int c = c_first; c < c_last; ++c) {
+            const int stage = (c - c_first) & 1;
+            if (c + 1 < c_last) {
+                TZK_ISSUE(c + 1, stage ^ 1)
+                __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(2 * LOADS));   // chunk c has landed
+            } else {
+                __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+            }
+            half8_t fa[2][4], fb[2][4];
+            const char *st = mine + stage * STAGE + frag_row;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                fa[0][i] = *reinterpret_cast<const half8_t *>(st + i * 16 * ROWB + frag_seg0);
+                fb[0][i] = *reinterpret_cast<const half8_t *>(st + OPERAND_BYTES + i * 16 * ROWB + frag_seg0);
+                fa[1][i] = *reinterpret_cast<const half8_t *>(st + i * 16 * ROWB + frag_seg1);
+                fb[1][i] = *reinterpret_cast<const half8_t *>(st + OPERAND_BYTES + i * 16 * ROWB + frag_seg1);
+            }
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[h][j], fa[h][i], acc[i][j], 0, 0, 0);
+            // the reads above have returned (the MFMAs consumed them) before the next
+            // iteration's loads overwrite this stage
+            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
+        }
+#undef TZK_ISSUE
+        // partial tiles of waves 1..3 go to LDS (each into its own region), wave 0 adds them
+        if (wave != 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    *reinterpret_cast<float4_t *>(mine + ((i * 4 + j) * 64 + lane) * 16) = acc[i][j];
+        }
+        sync.sync();
+        if (wave == 0) {
+#pragma unroll
+            for (int w = 1; w < 4; ++w)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        acc[i][j] += *reinterpret_cast<const float4_t *>(lds + w * (2 * STAGE) +
+                                                                         ((i * 4 + j) * 64 + lane) * 16);
+            float *c_lane = C + (size_t)(ti * TZ_REF_TILE + (lane & 15)) * N + tj * TZ_REF_TILE + (lane >> 4) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    float4_t v = acc[i][j] * TZ_ALPHA;
+                    *reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16) = v;
+                }
+        }
+        sync.sync();   // wave 0 has read the partial tiles before the next tile's loads land on them
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+    }
+    sync.finish();
+}
+
+template <int STAGES, class Sync>
+__device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
+                                            float *__restrict__ C, int M, int N, int K, int role_block,
+                                            int role_blocks, int tile_start, int tile_end, int tid, char *lds,
+                                            Sync &sync)
+{
+    static_assert(STAGES * TZ_STAGE_BYTES >= 4 * 2 * 2 * TZ_REF_TILE * TZ_BLOCK_K * 2,
+                  "the K-split form needs two 16 KiB stages per wave");
+    if (tz_use_ksplit(M, N, K))
+        tzgemm_role_ksplit(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds, sync);
+    else
+        tzgemm_role_tiles<STAGES>(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds, sync);
 }
 
 }  // namespace tk

@@ -24,7 +24,10 @@ def _init():
 
 
 # ------------------------------------------------------------------ tzgemm
-@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 128), (1024, 1024, 1024), (384, 128, 640)])
+# shapes with at most 64 macro tiles and K >= 512 take the K-split form of the kernel (one
+# reference tile per workgroup, K cut over its waves), the others the macro-tile form
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (256, 384, 128), (1024, 1024, 1024), (384, 128, 640),
+                                   (128, 512, 4608), (128, 256, 25088), (1152, 1024, 512), (256, 128, 576 + 64)])
 def test_gptb_tzgemm_matches_fp64_oracle(M, N, K):
     A, B = gemm_inputs(M, N, K)
     Cd = torch.full((M, N), -7.0, device="cuda:0")
@@ -49,9 +52,10 @@ def test_tzgemm_closed_forms():
     assert np.all(host(Cd2) == np.float32(K) * np.float32(1.1))
 
 
+@pytest.mark.parametrize("K", [128, 768])          # macro-tile form, K-split form
 @pytest.mark.parametrize("start,end,grid", [(0, 5, 0), (3, 9, 8), (7, 8, 16), (0, 0, 0), (0, 24, 3)])
-def test_tzgemm_tile_range_writes_only_its_tiles(start, end, grid):
-    M, N, K = 256, 384, 128
+def test_tzgemm_tile_range_writes_only_its_tiles(start, end, grid, K):
+    M, N = 256, 384
     A, B = gemm_inputs(M, N, K, seed=5)
     full = torch.zeros((M, N), device="cuda:0")
     ta.gptb_tzgemm(dev(A), dev(B), full)
@@ -394,3 +398,27 @@ def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
     mix.execute()
     for o, w in zip(outs, want):
         assert np.array_equal(host(o).view(np.uint32), w.view(np.uint32))
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_mix_with_a_k_split_gemm_shape(variant):
+    # 256 x 384 x 1024: 6 macro tiles, K >= 512 -> the GEMM role takes its K-split form,
+    # whose workgroup-level reduction runs on the role barrier of the fused kernel
+    M, N, K = 256, 384, 1024
+    A, B = gemm_inputs(M, N, K, seed=17)
+    A0 = stencil_inputs(6, 20, 200, seed=5)
+    a0 = dev(A0)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dev(A), dev(B), solo_c)
+    mix_c = torch.full((M, N), -7.0, device="cuda:0")
+    mix_s = a0.clone()
+    ta.mix_tzgemm_stencil(C0, C1, a0, mix_s, dev(A), dev(B), mix_c, variant=variant, tile_start=2, tile_end=19)
+    got = host(mix_c)
+    full = host(solo_c)
+    want = oracle.tzgemm(A, B, C_init=np.full((M, N), -7.0, np.float32), start=2, end=19)
+    mask = want != -7.0
+    assert np.array_equal(got[~mask], want[~mask]) and np.array_equal(got[mask], full[mask])
+    ok, fro, dmax = gemm_tolerance_ok(full, oracle.tzgemm(A, B, f64=True), K)
+    assert ok and fro <= 1e-5, (fro, dmax)
+    assert np.array_equal(host(mix_s), oracle.stencil(C0, C1, A0, A0))
+    assert ta.spin_fail_flag() == 0
