@@ -16,13 +16,43 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
                                            int KH, int KW, int pad, int stride, int Ho, int Wo,
                                            _Float16 *A, int K_pad)
 {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const int k_real = KH * KW * C;
+    if ((C & 7) == 0 && (c_stride & 3) == 0 && (K_pad & 7) == 0) {
+        // 8 consecutive k share one tap (C is a multiple of 8): two 16-byte loads of the
+        // activation, one 16-byte store of A, 32-bit index arithmetic
+        const unsigned groups_per_row = (unsigned)K_pad >> 3;
+        const unsigned total = (unsigned)(Ho * Wo) * groups_per_row;
+        for (unsigned g = blockIdx.x * blockDim.x + threadIdx.x; g < total; g += blockDim.x * gridDim.x) {
+            const unsigned m = g / groups_per_row;
+            const int k = (int)(g - m * groups_per_row) << 3;
+            h8 out = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (k < k_real) {
+                const int tap = k / C;
+                const int c = k - tap * C;
+                const int kh = tap / KW, kw = tap - kh * KW;
+                const int ho = (int)(m / (unsigned)Wo), wo = (int)(m - (unsigned)ho * (unsigned)Wo);
+                const int h = ho * stride - pad + kh, w = wo * stride - pad + kw;
+                if (h >= 0 && h < H && w >= 0 && w < W) {
+                    const float *src = act + ((size_t)h * W + w) * c_stride + c;
+                    const f4 lo = *reinterpret_cast<const f4 *>(src);
+                    const f4 hi = *reinterpret_cast<const f4 *>(src + 4);
+                    out = h8{(_Float16)lo.x, (_Float16)lo.y, (_Float16)lo.z, (_Float16)lo.w,
+                             (_Float16)hi.x, (_Float16)hi.y, (_Float16)hi.z, (_Float16)hi.w};
+                }
+            }
+            *reinterpret_cast<h8 *>(A + (size_t)g * 8) = out;
+        }
+        return;
+    }
     const long total = (long)Ho * Wo * K_pad;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (long)blockDim.x * gridDim.x) {
         const int k = (int)(i % K_pad);
         const long m = i / K_pad;
         float v = 0.0f;
-        if (k < KH * KW * C) {
+        if (k < k_real) {
             const int c = k % C;
             const int tap = k / C;
             const int kw = tap % KW, kh = tap / KW;
