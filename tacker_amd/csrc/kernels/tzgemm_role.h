@@ -61,6 +61,19 @@ __device__ __forceinline__ void tz_macro_tile_of(int t, int macro_rows, int macr
 // s_waitcnt immediate that waits for lgkmcnt == 0 (LDS reads landed) and nothing else
 #define TK_LGKMCNT0_IMM 0xC07F
 
+// One LDS-direct load of 16 bytes per lane: global address = scalar base + 32-bit lane
+// offset (an addressing mode of the instruction, so no 64-bit vector address is formed and
+// no VALU work is spent on it), LDS address = scalar (M0).  Written as asm because the
+// builtin only selects the vector-address form.  The compiler does not count these loads
+// in vmcnt; the role waits for them with explicit s_waitcnt.
+__device__ __forceinline__ void tz_load_to_lds(const char *uniform_base, unsigned lane_offset, unsigned lds_address)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_address), "v"(lane_offset), "s"(uniform_base)
+                 : "memory");
+}
+
 template <int STAGES, class Sync>
 __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A,
                                             const _Float16 *__restrict__ B, float *__restrict__ C,
@@ -79,7 +92,9 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
     static_assert(STAGES >= 3 && LOADS_PER_CHUNK * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
 
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    // wave-uniform by construction: everything derived from it (the LDS address an
+    // LDS-direct load goes to, i.e. M0) then stays in scalar registers
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wr = wave >> 1;
     const int wc = wave & 1;
     const int ref_cols = N / TZ_REF_TILE;
@@ -98,6 +113,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
     const unsigned src_even = (unsigned)(dma_row * K + dma_seg * 8) * 2u;
     const unsigned src_odd = (unsigned)(dma_row * K + (dma_seg ^ 4) * 8) * 2u;
     const int dst_off = 4 * wave * 1024;                        // + j*1024 per load
+    const unsigned lds_base = (unsigned)(size_t)(lptr_t)lds;
     // fragment reads: row r = lane%16 of a 16-row group (its swizzle key (r>>1)&7 is the
     // same in every group), k segment 4*kstep + lane/16 of the 8 in a row
     const int frag_key = ((lane & 15) >> 1) & 7;
@@ -121,17 +137,17 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         const char *a_tile = reinterpret_cast<const char *>(A + (size_t)(mi * TZ_MACRO_TILE) * K);
         const char *b_tile = reinterpret_cast<const char *>(B + (size_t)(mj * TZ_MACRO_TILE) * K);
 
-#define TZ_ISSUE_CHUNK(chunk_, stage_)                                                            \
-    _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                             \
+// load q (0..7) of a chunk: operand q&1 (A, B), row block j = q>>1
+#define TZ_ISSUE_ONE(chunk_, stage_, q_)                                                          \
     {                                                                                             \
-        char *dst_ = lds + (stage_) * STAGE_BYTES + dst_off + j * 1024;                           \
-        const size_t uni_ = ((size_t)(j * 8) * K + (size_t)(chunk_) * BK) * 2;                    \
-        unsigned lane_ = (j & 1) ? src_odd : src_even;                                            \
-        asm volatile("" : "+v"(lane_));   /* keep base + offset apart: scalar base, vector offset */ \
-        __builtin_amdgcn_global_load_lds((gptr_t)(a_tile + uni_ + lane_), (lptr_t)dst_, 16, 0, 0); \
-        __builtin_amdgcn_global_load_lds((gptr_t)(b_tile + uni_ + lane_),                         \
-                                         (lptr_t)(dst_ + OPERAND_BYTES), 16, 0, 0);               \
+        const int j_ = (q_) >> 1;                                                                 \
+        const size_t uni_ = ((size_t)(j_ * 8) * K + (size_t)(chunk_) * BK) * 2;                   \
+        const unsigned dst_ = lds_base + (stage_) * STAGE_BYTES + dst_off + j_ * 1024 +           \
+                              (((q_) & 1) ? OPERAND_BYTES : 0);                                   \
+        tz_load_to_lds((((q_) & 1) ? b_tile : a_tile) + uni_, (j_ & 1) ? src_odd : src_even, dst_); \
     }
+#define TZ_ISSUE_CHUNK(chunk_, stage_)                                                            \
+    _Pragma("unroll") for (int q = 0; q < LOADS_PER_CHUNK; ++q) TZ_ISSUE_ONE(chunk_, stage_, q)
 #define TZ_READ_FRAGS(fa_, fb_, stage_, seg_)                                                     \
     _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                 \
     {                                                                                             \
@@ -155,16 +171,30 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
     }
 #define TZ_SCHED_DS_READ 0x100
 #define TZ_SCHED_VMEM 0x010
+#define TZ_MFMA_AT(fa_, fb_, n_)                                                                  \
+    acc[(n_) >> 2][(n_) & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[(n_) & 3], fa_[(n_) >> 2], \
+                                                                      acc[(n_) >> 2][(n_) & 3], 0, 0, 0);
 // First k-step of a chunk multiplied while the chunk barrier completes; the reads of the
-// second k-step (into fn_, fbn_) ride in the shadow of the first 8 MFMAs.  With a split
-// barrier the wave announces itself after 12 of the 16 MFMAs (its reads of the stage have
-// landed by then); the last 4 and the first 8 MFMAs of the second k-step, which need
-// nothing from behind the barrier, hide the round trip of the arrival counter.
-#define TZ_FIRST_STEP_ACROSS_BARRIER(fa_, fb_, fn_, fbn_, vmcnt_)                                 \
+// second k-step (into fn_, fbn_) ride in the shadow of the first 8 MFMAs, and loads 4..7 of
+// chunk tail_chunk_ (the half of a chunk the previous second k-step did not issue) follow one
+// per MFMA.  The 8 loads of a chunk are spread over a whole chunk's worth of MFMAs on purpose:
+// the CU's vector-memory unit takes about 10 ns per load, a wave blocks at issue while the
+// unit's queue is full, and 32 loads issued right behind the barrier by the four waves at
+// once would stall the MFMAs queued behind them.
+// With a split barrier the wave announces itself after 12 of the 16 MFMAs (its reads of the
+// stage have landed by then); the last 4 and the first 8 MFMAs of the second k-step, which
+// need nothing from behind the barrier, hide the round trip of the arrival counter.
+#define TZ_FIRST_STEP_ACROSS_BARRIER(fa_, fb_, fn_, fbn_, vmcnt_, tail_chunk_, tail_stage_)       \
     if constexpr (Sync::kSplit) {                                                                 \
-        TZ_MFMAS_ROWS(fa_, fb_, 0, 3)                                                             \
+        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
         TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                        \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
+        {                                                                                         \
+            TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
+            if ((tail_chunk_) >= 0) TZ_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q)                 \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
         sync.arrive();                                                                            \
@@ -189,34 +219,47 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
             sync.wait(seen_);                                                                     \
         }                                                                                         \
     } else {                                                                                      \
-        TZ_MFMAS(fa_, fb_)                                                                        \
+        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
         TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
         __builtin_amdgcn_sched_barrier(0);                                                        \
+        _Pragma("unroll") for (int q = 0; q < 8; ++q)                                             \
+        {                                                                                         \
+            TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
+            if ((q & 1) == 0 && (tail_chunk_) >= 0) TZ_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q / 2) \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
         sync.wait();                                                                              \
     }
-// Second k-step (what is left of it), with the 8 reads of the next chunk's first k-step and,
-// if loads_ is nonzero, the 8 LDS-direct loads of a new chunk slotted between its MFMAs.
-#define TZ_SECOND_STEP(fa_, fb_, loads_)                                                          \
+// Second k-step (what is left of it): the 8 reads of the next chunk's first k-step ride
+// between its first MFMAs and, if chunk_ >= 0, loads 0..3 of a new chunk follow; its loads
+// 4..7 go out with the next first k-step.
+#define TZ_SECOND_STEP(fa_, fb_, chunk_, stage_)                                                  \
     if constexpr (Sync::kSplit) {                                                                 \
-        TZ_MFMAS_ROWS(fa_, fb_, 2, 4)                                                             \
+        TZ_MFMAS_ROWS(fa_, fb_, 2, 3)                                                             \
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
         {                                                                                         \
             __builtin_amdgcn_sched_group_barrier(TZ_SCHED_DS_READ, 2, 0);                         \
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                    \
         }                                                                                         \
-        if (loads_) {                                                                             \
-            _Pragma("unroll") for (int q = 0; q < 4; ++q)                                         \
-            {                                                                                     \
-                __builtin_amdgcn_sched_group_barrier(TZ_SCHED_VMEM, 2, 0);                        \
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                \
-            }                                                                                     \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
+        {                                                                                         \
+            TZ_MFMA_AT(fa_, fb_, 12 + q)                                                          \
+            if ((chunk_) >= 0) TZ_ISSUE_ONE(chunk_, stage_, q)                                    \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
     } else {                                                                                      \
-        TZ_MFMAS(fa_, fb_)                                                                        \
+        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
         TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
-        if (loads_) { TZ_PAIR_MFMA_WITH(TZ_SCHED_VMEM, 8) }                                       \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        _Pragma("unroll") for (int q = 0; q < 8; ++q)                                             \
+        {                                                                                         \
+            TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
+            if ((q & 1) == 0 && (chunk_) >= 0) TZ_ISSUE_ONE(chunk_, stage_, q / 2)                \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
     }
 
         float4_t acc[4][4];
@@ -225,11 +268,21 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
 #pragma unroll
             for (int j = 0; j < 4; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-        // fill the ring, publish chunk 0, fetch its first k-step
-        const int prologue = kchunks < STAGES ? kchunks : STAGES;
+        // fill the ring, publish chunk 0, fetch its first k-step.  When the K loop is longer
+        // than the ring, the last chunk of the prologue goes out only half (loads 0..3): its
+        // other half is the "tail" the first k-step of chunk 0 issues, which puts the loop into
+        // its steady rhythm (half a chunk of loads per k-step) without a special first pass.
+        const bool ring_runs = kchunks > STAGES;
+        const int prologue = ring_runs ? STAGES - 1 : kchunks;
         for (int c = 0; c < prologue; ++c) { TZ_ISSUE_CHUNK(c, c) }
-        if (STAGES - 1 < kchunks) __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(LOADS_PER_CHUNK * (STAGES - 1)));
-        else __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+        if (ring_runs) {
+            _Pragma("unroll") for (int q = 0; q < 4; ++q) TZ_ISSUE_ONE(STAGES - 1, STAGES - 1, q)
+            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(LOADS_PER_CHUNK * (STAGES - 2) + 4));
+        } else if (kchunks == STAGES) {
+            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(LOADS_PER_CHUNK * (STAGES - 1)));
+        } else {
+            __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+        }
         sync.sync();
         half8_t fa0[4], fb0[4], fa1[4], fb1[4];
         TZ_READ_FRAGS(fa0, fb0, 0, frag_seg0)
@@ -237,28 +290,44 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
 
         int stage = 0;   // stage of chunk kc (and of chunk kc+STAGES, refilled once kc is consumed)
         int kc = 0;
-        // steady state: chunk kc+STAGES exists, so exactly STAGES-2 chunks of this wave's
-        // loads may stay in flight when chunk kc+1 is needed.  Branch-free body.
+        // steady state: chunk kc+STAGES exists.  The first k-step completes chunk kc+STAGES-1
+        // (into the stage chunk kc-1 left), after which exactly STAGES-2 chunks of this wave's
+        // loads may stay in flight when chunk kc+1 is needed; the second k-step starts chunk
+        // kc+STAGES in the stage chunk kc has just left.  Branch-free body.
         for (; kc + STAGES < kchunks; ++kc) {
             const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+            const int prev_stage = stage == 0 ? STAGES - 1 : stage - 1;
             TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)     // second k-step of chunk kc, in flight ...
             // ... while the first one is multiplied.  Past the barrier chunk kc+1 is complete
             // in LDS and every wave has read all of chunk kc.
-            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, LOADS_PER_CHUNK * (STAGES - 2))
+            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, LOADS_PER_CHUNK * (STAGES - 2), kc + STAGES - 1,
+                                         prev_stage)
             TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
-            TZ_ISSUE_CHUNK(kc + STAGES, stage)
-            TZ_SECOND_STEP(fa1, fb1, 1)
+            TZ_SECOND_STEP(fa1, fb1, kc + STAGES, stage)
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
             stage = next_stage;
+        }
+        // one more first k-step has a tail to issue: the last chunk's second half
+        if (ring_runs) {
+            const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
+            const int prev_stage = stage == 0 ? STAGES - 1 : stage - 1;
+            TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)
+            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, LOADS_PER_CHUNK * (STAGES - 2), kchunks - 1, prev_stage)
+            TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
+            TZ_SECOND_STEP(fa1, fb1, -1, 0)
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
+            stage = next_stage;
+            ++kc;
         }
         // drain: nothing left to issue, fewer loads in flight -- wait for all of them
         for (; kc + 1 < kchunks; ++kc) {
             const int next_stage = stage + 1 == STAGES ? 0 : stage + 1;
             TZ_READ_FRAGS(fa1, fb1, stage, frag_seg1)
-            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, 0)
+            TZ_FIRST_STEP_ACROSS_BARRIER(fa0, fb0, fa1, fb1, 0, -1, 0)
             TZ_READ_FRAGS(fa0, fb0, next_stage, frag_seg0)
-            TZ_SECOND_STEP(fa1, fb1, 0)
+            TZ_SECOND_STEP(fa1, fb1, -1, 0)
             __builtin_amdgcn_sched_barrier(0);
             __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
             stage = next_stage;
@@ -285,6 +354,8 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         // counts of the next tile's ring are exact
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
 #undef TZ_ISSUE_CHUNK
+#undef TZ_ISSUE_ONE
+#undef TZ_MFMA_AT
 #undef TZ_READ_FRAGS
 #undef TZ_MFMAS
 #undef TZ_MFMAS_ROWS
