@@ -14,15 +14,19 @@
 // which is the operand layout MFMA wants (lane l supplies 8 consecutive k of row
 // l%16), so tiles go to LDS as they are.
 //
-// Two things keep the MFMA pipe fed with one GEMM wave per SIMD:
+// Three things keep the MFMA pipe fed with one GEMM wave per SIMD:
 //  * global latency -- the K loop is a ring of STAGES LDS stages (64 k each,
 //    32 KiB) filled by global_load_lds_dwordx4: the load writes LDS directly,
-//    costs no VGPRs, and STAGES-1 chunks are in flight while one is multiplied.
-//    A wave knows its loads of a chunk have landed from the vmcnt counter
-//    (s_waitcnt vmcnt(8*(STAGES-2))), then one role barrier publishes the chunk.
+//    costs no VGPRs, and almost STAGES-1 chunks are in flight while one is
+//    multiplied.  A wave knows its loads of a chunk have landed from the vmcnt
+//    counter (s_waitcnt vmcnt(8*(STAGES-2))), then one role barrier publishes
+//    the chunk.
 //  * LDS latency -- fragments are double-buffered in registers: the 8
-//    ds_read_b128 of the next k-step are issued before the 16 MFMAs of the current
-//    one, so the wave never sits idle between its LDS reads and its MFMAs.
+//    ds_read_b128 of the next k-step are issued between the first MFMAs of the
+//    current one, so the wave never sits idle between its LDS reads and its MFMAs.
+//  * issue slots -- a wave issues in order and blocks at a load while the CU's
+//    vector-memory queue is full, so the 8 loads of a chunk go out one at a time
+//    behind individual MFMAs, 4 in each k-step, with scalar address arithmetic only.
 // An LDS-direct load puts lane l's 16 bytes at base + 16*l, so tile rows are dense
 // (128 B); bank conflicts are avoided by a swizzle applied on the global side:
 // LDS slot (row, s) holds the row's 16-byte segment s ^ ((row >> 1) & 7), and the
@@ -32,6 +36,9 @@
 // ends up with 4 consecutive columns of one row of C and stores 16 bytes at once.
 // A wave stores its tile only if the tile's position is inside the range; macro
 // tiles with no position in range are skipped by the whole workgroup.
+//
+// Shapes with few tiles and a long reduction take a second form (tzgemm_role_ksplit,
+// below): one reference tile per workgroup, K cut over its 4 waves.
 #pragma once
 #include "role_common.h"
 #include "../header/tzgemm_header.h"
@@ -81,7 +88,6 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
                                             int tile_start, int tile_end, int tid, char *lds,
                                             Sync &sync)
 {
-    typedef __attribute__((address_space(1))) const void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int BK = TZ_BLOCK_K;
     constexpr int ROWB = BK * 2;                         // dense 128-byte tile rows
@@ -170,7 +176,6 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         __builtin_amdgcn_sched_group_barrier(mask_, 1, 0);                                        \
     }
 #define TZ_SCHED_DS_READ 0x100
-#define TZ_SCHED_VMEM 0x010
 #define TZ_MFMA_AT(fa_, fb_, n_)                                                                  \
     acc[(n_) >> 2][(n_) & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[(n_) & 3], fa_[(n_) >> 2], \
                                                                       acc[(n_) >> 2][(n_) & 3], 0, 0, 0);
@@ -361,7 +366,6 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
 #undef TZ_MFMAS_ROWS
 #undef TZ_PAIR_MFMA_WITH
 #undef TZ_SCHED_DS_READ
-#undef TZ_SCHED_VMEM
 #undef TZ_FIRST_STEP_ACROSS_BARRIER
 #undef TZ_SECOND_STEP
     }
@@ -392,7 +396,6 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
                                                    int tile_start, int tile_end, int tid, char *lds,
                                                    Sync &sync)
 {
-    typedef __attribute__((address_space(1))) const void *gptr_t;
     typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int BK = TZ_BLOCK_K;
     constexpr int ROWB = BK * 2;                      // 128-byte tile rows
@@ -400,13 +403,14 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
     constexpr int STAGE = 2 * OPERAND_BYTES;          // A rows then B rows
     constexpr int LOADS = 8;                          // LDS-direct loads per operand and chunk
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int ref_cols = N / TZ_REF_TILE;
     const int n_ref = (M / TZ_REF_TILE) * ref_cols;
     const int kchunks = K / BK;
     const int c_first = (wave * kchunks) / 4;
     const int c_last = ((wave + 1) * kchunks) / 4;
     char *mine = lds + wave * (2 * STAGE);            // this wave's two stages
+    const unsigned mine_lds = (unsigned)(size_t)(lptr_t)mine;
     // load j of an operand fills rows 8j .. 8j+7: lane lands in row 8j + lane/8, slot lane%8,
     // and fetches the row's segment slot ^ ((row>>1)&7) = slot ^ (lane>>4) ^ (4*(j&1))
     const unsigned seg_even = (unsigned)((lane & 7) ^ (lane >> 4));
@@ -426,13 +430,11 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
 #define TZK_ISSUE(chunk_, stage_)                                                                  \
     _Pragma("unroll") for (int j = 0; j < LOADS; ++j)                                              \
     {                                                                                              \
-        char *dst_ = mine + (stage_) * STAGE + j * 1024;                                           \
+        const unsigned dst_ = mine_lds + (stage_) * STAGE + j * 1024;                              \
         const size_t uni_ = ((size_t)(j * 8) * K + (size_t)(chunk_) * BK) * 2;                     \
-        unsigned lane_ = (j & 1) ? src_odd : src_even;                                             \
-        asm volatile("" : "+v"(lane_));                                                            \
-        __builtin_amdgcn_global_load_lds((gptr_t)(a_tile + uni_ + lane_), (lptr_t)dst_, 16, 0, 0); \
-        __builtin_amdgcn_global_load_lds((gptr_t)(b_tile + uni_ + lane_),                          \
-                                         (lptr_t)(dst_ + OPERAND_BYTES), 16, 0, 0);                \
+        const unsigned lane_ = (j & 1) ? src_odd : src_even;                                       \
+        tz_load_to_lds(a_tile + uni_, lane_, dst_);                                                \
+        tz_load_to_lds(b_tile + uni_, lane_, dst_ + OPERAND_BYTES);                                \
     }
         float4_t acc[4][4];
 #pragma unroll
