@@ -146,6 +146,11 @@ struct StencilQuadMarch {
     float *__restrict__ Anext;
     int nx, ny, lane;
     size_t plane;
+    // z index of step 0 of the march and its direction (+1 up, -1 down): step L of a run is
+    // plane z0 + dz*L.  Runs that are neighbours in z march in opposite directions, so the
+    // two planes they share are read by both at the same moment (both at their start or
+    // both at their end) and the second read hits in L2 instead of going to memory again.
+    int z0, dz;
 
     float4_t own[RING][ROWS];   // plane ring, slot = plane index % RING
     float4_t dn[3], up[3];      // rows j0-1 and j0+ROWS of centre planes, slot = centre % 3
@@ -158,7 +163,8 @@ struct StencilQuadMarch {
     {
         const int x = x0 + 4 * lane;
         const bool xin = x < nx;
-        const float *col = A0 + (size_t)x + (size_t)nx * j0 + plane * (size_t)(k_first - 1 + P);
+        const size_t z = (size_t)(z0 + dz * P);
+        const float *col = A0 + (size_t)x + (size_t)nx * j0 + plane * z;
         const bool have = P <= nplanes + 1;
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
@@ -177,7 +183,7 @@ struct StencilQuadMarch {
             const int er = lane & 3;
             const int ex = (lane & 4) ? x0 + 256 : x0 - 1;
             if (centre && lane < 8 && ex >= 0 && ex < nx && (j0 + er) < ny)
-                e = A0[(size_t)ex + (size_t)nx * (j0 + er) + plane * (size_t)(k_first - 1 + P)];
+                e = A0[(size_t)ex + (size_t)nx * (j0 + er) + plane * z];
             edge[P % 3] = e;
         }
     }
@@ -189,7 +195,7 @@ struct StencilQuadMarch {
     {
         if (C > nplanes) return;
         const int x = x0 + 4 * lane;
-        float *out = Anext + (size_t)x + (size_t)nx * j0 + plane * (size_t)(k_first - 1 + C);
+        float *out = Anext + (size_t)x + (size_t)nx * j0 + plane * (size_t)(z0 + dz * C);
         const bool mine = (block_ok >> (lane >> 4)) & 1u;
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
@@ -242,8 +248,10 @@ struct StencilQuadMarch {
     }
 
     __device__ __forceinline__ void run(float c0, float c1, int k_first, int nplanes, int x0, int j0,
-                                        unsigned block_ok)
+                                        unsigned block_ok, bool upward)
     {
+        z0 = upward ? k_first - 1 : k_first + nplanes;
+        dz = upward ? 1 : -1;
         issue<0>(k_first, nplanes, x0, j0);
         issue<1>(k_first, nplanes, x0, j0);
         issue<2>(k_first, nplanes, x0, j0);
@@ -346,7 +354,7 @@ __device__ __forceinline__ void stencil_role_wide(float c0, float c1, const floa
         if (block_ok == 0) continue;
         const int k_first = 1 + run * STENCIL_Z_RUN;
         m.run(c0, c1, k_first, min(STENCIL_Z_RUN, nz - 1 - k_first), (int)(qx * 4 * 2 * STENCIL_TILE_X),
-              (int)(row % (unsigned)grid_dimension_y) * STENCIL_TILE_Y, block_ok);
+              (int)(row % (unsigned)grid_dimension_y) * STENCIL_TILE_Y, block_ok, (run & 1) == 0);
     }
 }
 
