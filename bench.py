@@ -174,7 +174,9 @@ def lc_leg(ta, torch, np, queries):
            "qos_bound_ms": round(1.2 * float(np.percentile(solo, 99)), 4),
            "qos_budget_ms": 50.0,
            "mixed_launches_per_query": rep["mix_times"], "mixable_launches_per_query": rep["mixable_times"],
-           "be_blocks_per_query": rep["be_blocks_executed"], "time_earned_ms_per_query": round(rep["time_earned_ms"], 4)}
+           "be_blocks_per_query": rep["be_blocks_executed"], "time_earned_ms_per_query": round(rep["time_earned_ms"], 4),
+           "be_kernel_passes_completed": rep["be_task_finish_num"],
+           "lc_kernels_barred_from_fusion_at_end": tm.fusion_disabled()}
     out["p99_within_bound"] = bool(out["colocated_p99_ms"] <= out["qos_bound_ms"])
     tm.close()
     task.close()

@@ -327,6 +327,13 @@ TK_API int tacker_task_manager_run(tacker_task_manager_t tm, int mode, tkStream_
  * mixable_times, time_earned_ms, qos_headroom_left_ms, stage1_be_ms, stage2_be_ms,
  * be_task_finish_num, n co-located latencies, n solo latencies} */
 TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
+/* No counterpart in the reference (its hot loop, src/TaskManager.cu:586-640, fuses every mixable
+ * kernel of every query): an LC kernel whose fused launch lost against "LC alone, then the BE
+ * share alone" `limit` times in a row is launched alone for the rest of the run (Aker mode only).
+ * Default 3; 0 restores the reference's behaviour. */
+TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int limit);
+/* LC kernels barred from fusion at the end of the last run */
+TK_API int tacker_task_manager_fusion_disabled(tacker_task_manager_t tm);
 /* "[Mix] BE task1 + task2 took ..." (src/TaskManager.cu:693): average time of the fused launch of
  * the two best-effort kernels measured by the last run with a second stage; 0 if none ran. */
 TK_API float tacker_task_manager_be_mix_ms(tacker_task_manager_t tm);

@@ -102,6 +102,8 @@ def _declare(lib):
     lib.tacker_task_manager_run.argtypes = [vp, i, vp, i]
     lib.tacker_task_manager_report.argtypes = [vp, C.POINTER(f)]
     lib.tacker_task_manager_latencies.argtypes = [vp, i, C.POINTER(f), i]
+    lib.tacker_task_manager_set_fusion_strikes.argtypes = [vp, i]
+    lib.tacker_task_manager_fusion_disabled.argtypes = [vp]
     lib.tacker_task_manager_be_mix_ms.argtypes = [vp]
     lib.tacker_task_manager_be_mix_ms.restype = f
     lib.tacker_qos_block_ratio.argtypes = [cp, i]
@@ -590,6 +592,12 @@ class TaskManager:
         out = (C.c_float * 13)()
         self.l.tacker_task_manager_report(self.h, out)
         return dict(zip(REPORT_KEYS, out))
+
+    def set_fusion_strikes(self, limit):
+        check(self.l.tacker_task_manager_set_fusion_strikes(self.h, limit), "set_fusion_strikes")
+
+    def fusion_disabled(self):
+        return self.l.tacker_task_manager_fusion_disabled(self.h)
 
     def be_mix_ms(self):
         return self.l.tacker_task_manager_be_mix_ms(self.h)

@@ -221,9 +221,13 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     // co-located queries: a cursor walks the BE kernel's blocks across launches
     int be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;
     float qos_headroom = policy.qos_budget_ms;
+    std::vector<int> strikes(nk, 0);   // consecutive fused launches of kernel i that did not pay
     for (int q = 0; q < queries; ++q) {
         lc_task->initExecution();
         qos_headroom = policy.qos_budget_ms;
+        // a barred kernel gets one more chance every fusion_retry_period queries
+        if (fusion_retry_period > 0 && q > 0 && q % fusion_retry_period == 0)
+            for (int &v : strikes) v = std::min(v, std::max(fusion_strikes_limit - 1, 0));
         long long cd_block_num_executed = 0;
         report.mix_times = 0;
         report.time_earned_ms = 0.0f;
@@ -232,7 +236,9 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             Kernel *lc_kernel = lc_task->kernels[idx];
             int cd_block_num = 0;
             watch.start(stream);
-            if (policy.mustRunSolo(qos_headroom, lc_headroom_vec[idx]) || lc_kernel->mixable == 0) {
+            const bool barred = mode == ExecutionMode::Aker && fusion_strikes_limit > 0 &&
+                                strikes[idx] >= fusion_strikes_limit;
+            if (policy.mustRunSolo(qos_headroom, lc_headroom_vec[idx]) || lc_kernel->mixable == 0 || barred) {
                 lc_kernel->execute(stream);
             } else {
                 std::vector<int> args = lc_kernel->getArgs();
@@ -258,6 +264,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             const QosPolicy::Outcome o = QosPolicy::account(mixed, duration, lc_kernel_time_vec[idx],
                                                             report.be1_solo_ms, cd_block_num, be_total);
             qos_headroom -= o.charged_ms;
+            if (mixed) strikes[idx] = o.counted_as_mixed ? 0 : strikes[idx] + 1;
             if (o.counted_as_mixed) {
                 cd_block_num_executed += cd_block_num;
                 report.mix_times++;
@@ -268,6 +275,9 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         report.query_latency_ms.push_back(query_ms);
     }
     report.qos_headroom_left_ms = qos_headroom;
+    report.fusion_disabled = 0;
+    if (fusion_strikes_limit > 0)
+        for (int v : strikes) report.fusion_disabled += v >= fusion_strikes_limit;
     report.stage1_be_ms = report.be_blocks_executed * report.be1_solo_ms / std::max(be_total, 1);
     if (verbose) {
         printf("execed be blks: %lld, mix times: %d/%d, time earned: %f\n", report.be_blocks_executed,

@@ -58,6 +58,7 @@ struct TaskManagerReport {
     float be1_solo_ms = 0.0f, be2_solo_ms = 0.0f;
     long long be_blocks_executed = 0;   // BE blocks carried by fused launches in the last query
     int mix_times = 0, mixable_times = 0;
+    int fusion_disabled = 0;            // LC kernels that ended the run barred from fusion
     float time_earned_ms = 0.0f;
     float qos_headroom_left_ms = 0.0f;
     float stage1_be_ms = 0.0f, stage2_be_ms = 0.0f;
@@ -84,6 +85,13 @@ public:
     int profile_queries = 10;
     int queries = 5;
     bool verbose = true;
+    // Not in the reference: an LC kernel whose fused launch lost against "LC alone, then the
+    // BE share alone" this many times in a row is launched alone from then on (Aker mode).
+    // The static load ratios are measured on GEMMs that fill the GPU; layers with few tiles
+    // can still lose, and every lost fusion stretches the LC query for nothing.  0 = never
+    // stop (the reference's behaviour).
+    int fusion_strikes_limit = 3;
+    int fusion_retry_period = 64;   // queries between two chances for a barred kernel (0 = never again)
     TaskManagerReport report;
 
 private:

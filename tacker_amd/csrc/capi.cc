@@ -797,6 +797,20 @@ int tacker_task_manager_report(tacker_task_manager_t h, float out[13])
     return TK_SUCCESS;
 }
 
+int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t h, int limit)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || limit < 0) return fail(TK_ERROR_INVALID_VALUE, "bad task manager or limit");
+    tm->fusion_strikes_limit = limit;
+    return TK_SUCCESS;
+}
+
+int tacker_task_manager_fusion_disabled(tacker_task_manager_t h)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    return tm ? tm->report.fusion_disabled : -1;
+}
+
 float tacker_task_manager_be_mix_ms(tacker_task_manager_t h)
 {
     TaskManager *tm = static_cast<TaskManager *>(h);

@@ -422,6 +422,31 @@ def test_task_manager_second_stage_credits_the_fused_best_effort_pair(fake, smal
     tm.close()
 
 
+def test_task_manager_stops_fusing_kernels_whose_fusion_keeps_losing(fake, small_vgg):
+    # profiling passes see 10 us per kernel; from the co-located queries on every timed region
+    # takes 1 ms, so every fused launch loses against "LC alone + BE share alone": after 3 lost
+    # launches per kernel the manager launches that kernel alone (the reference never stops)
+    n = len(small_vgg.kernels())
+    tm = ta.TaskManager(small_vgg, "stencil", None, library=fake)
+    tm.configure(warmup=1, profile=2, verbose=0, qos_budget_ms=1e6, guard_ms=0.0, queries=6)
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(1.0)
+    cheap = [0.01] * (n * 2 + 1)            # the profiled LC kernels (2 queries) and the BE kernel alone
+    arr = (C.c_float * len(cheap))(*cheap)
+    fake.tk_fake_push_event_ms(arr, len(cheap))
+    rep = tm.run("aker", raw_stream=None, second_stage=False)
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
+    barred = tm.fusion_disabled()                     # mixable kernels with a nonzero load ratio
+    assert barred in (15, 16) and len(fused) == 3 * barred and rep["mix_times"] == 0
+    tm.set_fusion_strikes(0)                          # the reference's behaviour: keep fusing
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(1.0)
+    fake.tk_fake_push_event_ms(arr, len(cheap))
+    tm.run("aker", raw_stream=None, second_stage=False)
+    assert len([l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]) == 6 * barred
+    tm.close()
+
+
 def test_task_manager_falls_back_to_solo_when_headroom_is_short(fake, small_vgg):
     fake.tk_fake_set_event_ms(0.01)
     n = len(small_vgg.kernels())
