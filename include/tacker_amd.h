@@ -157,8 +157,15 @@ TK_API int tacker_mriq_phimag(const float *phiR, const float *phiI, float *phiMa
 #define TACKER_MRIQ_MAX_K 4096
 TK_API int tacker_mriq_set_kvalues(const float *kvals_host, int numK);
 /* ori_mriq / g_general_ptb_mriq (src/ori_kernel/mriq_kernel.cu:56-105,
- * src/gptb_kernel/mriq_kernel.cu:3-70): Q += sum over all numK samples for voxel
- * blocks (256 voxels each) [block_start, block_end). numX multiple of 256. */
+ * src/gptb_kernel/mriq_kernel.cu:3-70). numX multiple of 256. ori_mriq adds all numK
+ * samples to every voxel. The GPTB form works on block positions [block_start, block_end)
+ * of a grid of (numX / 256) voxel blocks by ceil(numK / TACKER_MRIQ_K_CHUNK) chunks of the
+ * k table: position p adds chunk p / (numX / 256) to voxel block p % (numX / 256) -- the
+ * reference's host loop over k chunks (mriq_kernel.cu:258-283) as the y index of the GPTB
+ * grid. [0, tacker_mriq_blocks(numK, numX)) equals ori_mriq bit for bit, and so does any
+ * sequence of launches whose ranges tile it in ascending order. */
+#define TACKER_MRIQ_K_CHUNK 128
+TK_API int tacker_mriq_blocks(int numK, int numX);
 TK_API int tacker_ori_mriq(int numK, const float *x, const float *y, const float *z, float *Qr,
                            float *Qi, int numX, tkStream_t stream);
 TK_API int tacker_gptb_mriq(int numK, const float *x, const float *y, const float *z, float *Qr,

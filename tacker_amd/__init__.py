@@ -42,6 +42,7 @@ def _declare(lib):
     lib.tacker_gptb_lbm.argtypes = [vp, vp, i, i, i, i, i, i, i, vp]
     lib.tacker_mriq_phimag.argtypes = [vp, vp, vp, i, vp]
     lib.tacker_mriq_set_kvalues.argtypes = [vp, i]
+    lib.tacker_mriq_blocks.argtypes = [i, i]
     lib.tacker_ori_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, vp]
     lib.tacker_gptb_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     lib.tacker_cp_set_atoms.argtypes = [vp, i, f]
@@ -239,6 +240,11 @@ def mriq_set_kvalues(kvals_np):
     check(lib().tacker_mriq_set_kvalues(kv.ctypes.data, kv.shape[0]), "tacker_mriq_set_kvalues")
 
 
+def mriq_blocks(numK, numX):
+    """block positions of the GPTB form: voxel blocks x chunks of the k table"""
+    return lib().tacker_mriq_blocks(numK, numX)
+
+
 def ori_mriq(numK, x, y, z, Qr, Qi, stream=None):
     check(lib().tacker_ori_mriq(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi), x.numel(),
                                 _stream(stream)), "tacker_ori_mriq")
@@ -246,7 +252,7 @@ def ori_mriq(numK, x, y, z, Qr, Qi, stream=None):
 
 def gptb_mriq(numK, x, y, z, Qr, Qi, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
     if end is None:
-        end = x.numel() // 256
+        end = mriq_blocks(numK, x.numel())
     check(lib().tacker_gptb_mriq(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi), x.numel(), start,
                                  end, launch_grid, launch_block, _stream(stream)), "tacker_gptb_mriq")
 
@@ -312,7 +318,7 @@ def mix_tzgemm_lbm(src, dst, sx, sy, sz, A, B, Cm, be_start=0, be_end=None, tile
 def mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, A, B, Cm, be_start=0, be_end=None, tile_start=0,
                     tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
     if be_end is None:
-        be_end = x.numel() // 256
+        be_end = mriq_blocks(numK, x.numel())
     check(lib().tacker_mix_tzgemm_mriq(
         numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi), x.numel(), be_start, be_end,
         *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),

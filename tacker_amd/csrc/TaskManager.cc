@@ -225,9 +225,13 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     for (int q = 0; q < queries; ++q) {
         lc_task->initExecution();
         qos_headroom = policy.qos_budget_ms;
-        // a barred kernel gets one more chance every fusion_retry_period queries
-        if (fusion_retry_period > 0 && q > 0 && q % fusion_retry_period == 0)
-            for (int &v : strikes) v = std::min(v, std::max(fusion_strikes_limit - 1, 0));
+        // a barred kernel gets one more chance every fusion_retry_period queries; kernel i takes
+        // its chance in the queries congruent to i, so that the retries (each a launch expected
+        // to lose) are spread over queries instead of piling up in one slow query
+        if (fusion_retry_period > 0 && q >= fusion_retry_period)
+            for (size_t idx = 0; idx < nk; ++idx)
+                if (q % fusion_retry_period == (int)(idx % (size_t)fusion_retry_period))
+                    strikes[idx] = std::min(strikes[idx], std::max(fusion_strikes_limit - 1, 0));
         long long cd_block_num_executed = 0;
         report.mix_times = 0;
         report.time_earned_ms = 0.0f;

@@ -263,6 +263,14 @@ int tacker_mriq_set_kvalues(const float *kvals_host, int numK)
     return rc ? fail(rc, tkGetErrorString(rc)) : rc;
 }
 
+int tacker_mriq_blocks(int numK, int numX)
+{
+    static_assert(TACKER_MRIQ_K_CHUNK == MRIQ_K_CHUNK, "public and device chunk sizes must agree");
+    if (numK < 0 || numX < 0) return 0;
+    const int chunks = numK > 0 ? (numK + MRIQ_K_CHUNK - 1) / MRIQ_K_CHUNK : 1;
+    return (numX / KERNEL_Q_THREADS_PER_BLOCK) * chunks;
+}
+
 int tacker_ori_mriq(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi, int numX, tkStream_t stream)
 {
     REQUIRE_INIT();

@@ -6,6 +6,8 @@
 #define KERNEL_Q_THREADS_PER_BLOCK 256
 #define KERNEL_Q_K_ELEMS_PER_GRID 1024
 #define MRIQ_MAX_K 4096          // capacity of the constant k table (64 KiB)
+// k records one block position of the GPTB form adds to its 256 voxels
+#define MRIQ_K_CHUNK 128
 struct mriq_kValues {
     float Kx;
     float Ky;

@@ -18,6 +18,10 @@
 #define TZ_STAGE_BYTES (2 * TZ_MACRO_TILE * TZ_BLOCK_K * 2)   // A rows then B rows: 32 KiB
 #define TZ_STAGES 4               // LDS ring depth where the GEMM has the CU's LDS to itself
 #define TZ_STAGES_WG 4            // ring depth of workgroup-split fused kernels
+// issue priority of the tzgemm waves of a wave-split fused kernel (s_setprio, 0..3)
+#ifndef TK_GEMM_WAVE_PRIORITY
+#define TK_GEMM_WAVE_PRIORITY 3
+#endif
 #define TZ_LDS_BYTES (TZ_STAGES * TZ_STAGE_BYTES)
 #define TZ_LDS_BYTES_WG (TZ_STAGES_WG * TZ_STAGE_BYTES)
 

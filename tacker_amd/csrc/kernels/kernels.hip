@@ -103,7 +103,7 @@ extern "C" __global__ void g_general_ptb_mriq(int numK, int kGlobalIndex, float 
                                               float *z, float *Qr, float *Qi, GPTB_TRAILER)
 {
     (void)kGlobalIndex;
-    tk::mriq_role(numK, x, y, z, Qr, Qi, grid_dimension_x, (int)blockIdx.x, ptb_iter_block_step,
+    tk::mriq_role(numK, x, y, z, Qr, Qi, grid_dimension_x, grid_dimension_y, (int)blockIdx.x, ptb_iter_block_step,
                   ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base,
                   (int)blockDim.x);
 }

@@ -8,7 +8,7 @@
 // array of {Kx,Ky,Kz,PhiMag} in constant memory, fp32 order
 //   arg = 2pi * ((Kx*x + Ky*y) + Kz*z); Qr += PhiMag*cos(arg); Qi += PhiMag*sin(arg)
 // with k ascending.  The reference's loop "for QGrid < 1" handles only the first
-// 1024-sample chunk; here the loop runs over all numK samples held in the table.
+// 1024-sample chunk; here all numK samples held in the table are used.
 //
 // gfx950: the table index is wave-uniform, so the compiler fetches each record
 // with one scalar 16-byte load; the work is VALU/transcendental bound.  The
@@ -47,20 +47,21 @@ __device__ __forceinline__ void mriq_voxel(int numK, const float *__restrict__ x
     Qi[xIndex] = sQi;
 }
 
-// V voxels per thread at once.  The k loop is a chain of dependent operations per voxel
-// (dot product, fract, sin/cos, accumulate) and a fused launch leaves the role at most two
-// waves per SIMD, so the independent work that hides instruction latency has to come
-// from inside the thread; V voxels also share each scalar load of a k record.
+// V voxels per thread at once, k records [k_begin, k_end).  The k loop is a chain of
+// dependent operations per voxel (dot product, fract, sin/cos, accumulate) and a fused
+// launch leaves the role at most two waves per SIMD, so the independent work that hides
+// instruction latency has to come from inside the thread; V voxels also share each
+// scalar load of a k record.
 template <int V>
-__device__ __forceinline__ void mriq_voxels(int numK, const float *__restrict__ x,
+__device__ __forceinline__ void mriq_voxels(int k_begin, int k_end, const float *__restrict__ x,
                                             const float *__restrict__ y, const float *__restrict__ z,
                                             float *__restrict__ Qr, float *__restrict__ Qi,
-                                            const int (&xIndex)[V], int count)
+                                            const int (&xIndex)[V])
 {
     float sX[V], sY[V], sZ[V], sQr[V], sQi[V];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-        const int i = xIndex[v < count ? v : 0];
+        const int i = xIndex[v];
         sX[v] = x[i];
         sY[v] = y[i];
         sZ[v] = z[i];
@@ -70,7 +71,7 @@ __device__ __forceinline__ void mriq_voxels(int numK, const float *__restrict__ 
     // unrolled so the scalar loads of 8 records are issued together: one record per
     // iteration would put a scalar-cache round trip on every step of the chain
 #pragma unroll 8
-    for (int kIndex = 0; kIndex < numK; ++kIndex) {
+    for (int kIndex = k_begin; kIndex < k_end; ++kIndex) {
         const mriq_kValues k = ck[kIndex];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
@@ -81,47 +82,105 @@ __device__ __forceinline__ void mriq_voxels(int numK, const float *__restrict__ 
         }
     }
 #pragma unroll
-    for (int v = 0; v < V; ++v)
-        if (v < count) {
-            Qr[xIndex[v]] = sQr[v];
-            Qi[xIndex[v]] = sQi[v];
-        }
+    for (int v = 0; v < V; ++v) {
+        Qr[xIndex[v]] = sQr[v];
+        Qi[xIndex[v]] = sQi[v];
+    }
 }
 
+// One phase of a launch: voxel blocks [block_lo, block_hi) each take records
+// [k_begin, k_end).  A thread serves the blocks it owns -- first_owned, first_owned +
+// stride, ... -- up to MRIQ_VOXELS_PER_THREAD at a time.
 #define MRIQ_VOXELS_PER_THREAD 4
-__device__ __forceinline__ void mriq_role(int numK, const float *__restrict__ x,
-                                          const float *__restrict__ y, const float *__restrict__ z,
-                                          float *__restrict__ Qr, float *__restrict__ Qi,
-                                          int grid_dimension_x, int role_block, int role_blocks,
-                                          int start, int end, int tid, int role_threads)
+__device__ __forceinline__ void mriq_phase(int block_lo, int block_hi, int k_begin, int k_end,
+                                           const float *__restrict__ x, const float *__restrict__ y,
+                                           const float *__restrict__ z, float *__restrict__ Qr,
+                                           float *__restrict__ Qi, int first_owned, int stride, int t)
 {
     constexpr int V = MRIQ_VOXELS_PER_THREAD;
-    const int blocks_at_once = role_threads / KERNEL_Q_THREADS_PER_BLOCK;
-    const int slot = tid / KERNEL_Q_THREADS_PER_BLOCK;
-    const int t = tid % KERNEL_Q_THREADS_PER_BLOCK;
-    if (slot >= blocks_at_once) return;
-    // block slots go round the role's workgroups first (slot-major), so a short range
-    // still spreads over all CUs; a thread takes V blocks that are one stride apart
-    const unsigned stride = (unsigned)role_blocks * blocks_at_once;
-    for (unsigned pos = (unsigned)start + slot * role_blocks + role_block; pos < (unsigned)end;
-         pos += stride * V) {
+    if (block_lo >= block_hi || k_begin >= k_end) return;
+    int b = first_owned;
+    if (b < block_lo) b += (block_lo - b + stride - 1) / stride * stride;
+    for (; b < block_hi; b += V * stride) {
         int idx[V];
         int count = 0;
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            const unsigned p = pos + v * stride;
-            idx[v] = (int)(p % grid_dimension_x) * KERNEL_Q_THREADS_PER_BLOCK + t;
-            if (p < (unsigned)end) count = v + 1;
+            const int bv = b + v * stride;
+            if (bv < block_hi) count = v + 1;
+            idx[v] = (bv < block_hi ? bv : b) * KERNEL_Q_THREADS_PER_BLOCK + t;
         }
-        if (count > 2) {
-            mriq_voxels<V>(numK, x, y, z, Qr, Qi, idx, count);
-        } else if (count == 2) {
-            const int two[2] = {idx[0], idx[1]};
-            mriq_voxels<2>(numK, x, y, z, Qr, Qi, two, 2);
+        if (count == V) {
+            mriq_voxels<V>(k_begin, k_end, x, y, z, Qr, Qi, idx);
         } else {
-            mriq_voxel(numK, x, y, z, Qr, Qi, idx[0]);
+            if (count >= 2) {
+                const int two[2] = {idx[0], idx[1]};
+                mriq_voxels<2>(k_begin, k_end, x, y, z, Qr, Qi, two);
+            }
+            if (count & 1) {
+                const int one[1] = {idx[count - 1]};
+                mriq_voxels<1>(k_begin, k_end, x, y, z, Qr, Qi, one);
+            }
         }
     }
+}
+
+// Block positions of the GPTB form are a grid of grid_dimension_x voxel blocks (256 voxels
+// each) by grid_dimension_y chunks of MRIQ_K_CHUNK k records: position p adds chunk
+// (p / grid_dimension_x) % grid_dimension_y to voxel block p % grid_dimension_x -- the
+// reference's host loop over k chunks (one launch per chunk with kGlobalIndex,
+// src/ori_kernel/mriq_kernel.cu:258-283) folded into the y index of the GPTB grid, so that
+// a short range of positions is a short piece of work.  Q is carried through memory
+// between chunks exactly as the reference carries it between launches, and a float stored
+// and reloaded is unchanged, so any split of [0, x*y) into ranges gives the bits of the
+// one k loop.
+//
+// A range [start, end) is a partial first row of the position grid, whole rows, and a
+// partial last row.  Every voxel block has one owner thread group for the whole launch
+// (slot-major over the role's workgroups, so a short range still spreads over all CUs),
+// and the owner walks the three parts in order: the chunks of a voxel are added in
+// ascending position order without any synchronisation between threads.  Whole rows that
+// follow each other are one run of the k loop.
+__device__ __forceinline__ void mriq_role(int numK, const float *__restrict__ x,
+                                          const float *__restrict__ y, const float *__restrict__ z,
+                                          float *__restrict__ Qr, float *__restrict__ Qi,
+                                          int grid_dimension_x, int grid_dimension_y, int role_block,
+                                          int role_blocks, int start, int end, int tid, int role_threads)
+{
+    const int blocks_at_once = role_threads / KERNEL_Q_THREADS_PER_BLOCK;
+    const int slot = tid / KERNEL_Q_THREADS_PER_BLOCK;
+    const int t = tid % KERNEL_Q_THREADS_PER_BLOCK;
+    if (slot >= blocks_at_once || start >= end) return;
+    const int gx = grid_dimension_x;
+    const int gy = grid_dimension_y;
+    const int stride = role_blocks * blocks_at_once;
+    const int first_owned = slot * role_blocks + role_block;
+    const auto chunk_begin = [&](int row) { return min((row % gy) * MRIQ_K_CHUNK, numK); };
+    const auto chunk_end = [&](int row) { return min((row % gy + 1) * MRIQ_K_CHUNK, numK); };
+
+    const int first_row = start / gx;
+    const int last_row = (end - 1) / gx;   // row of the last position
+    if (first_row == last_row) {
+        mriq_phase(start - first_row * gx, end - first_row * gx, chunk_begin(first_row), chunk_end(first_row),
+                   x, y, z, Qr, Qi, first_owned, stride, t);
+        return;
+    }
+    int row = first_row;
+    if (start != first_row * gx) {   // partial first row
+        mriq_phase(start - first_row * gx, gx, chunk_begin(row), chunk_end(row), x, y, z, Qr, Qi,
+                   first_owned, stride, t);
+        ++row;
+    }
+    const int whole_end = (end == (last_row + 1) * gx) ? last_row + 1 : last_row;   // whole rows [row, whole_end)
+    while (row < whole_end) {
+        // rows up to the next multiple of grid_dimension_y are consecutive chunks
+        const int run_end = min(whole_end, (row / gy + 1) * gy);
+        mriq_phase(0, gx, chunk_begin(row), chunk_end(run_end - 1), x, y, z, Qr, Qi, first_owned, stride, t);
+        row = run_end;
+    }
+    if (whole_end == last_row)       // partial last row
+        mriq_phase(0, end - last_row * gx, chunk_begin(last_row), chunk_end(last_row), x, y, z, Qr, Qi,
+                   first_owned, stride, t);
 }
 
 }  // namespace tk

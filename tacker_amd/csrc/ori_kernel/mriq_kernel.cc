@@ -97,9 +97,14 @@ void OriMRIQKernel::bind()
 {
     if (numX_ % KERNEL_Q_THREADS_PER_BLOCK != 0)
         logger.ERROR("mriq: numX must be a multiple of 256");
-    launchGridDim = dim3(numX_ / KERNEL_Q_THREADS_PER_BLOCK, 1, 1);
-    launchBlockDim = dim3(KERNEL_Q_THREADS_PER_BLOCK, 1, 1);
     OriMRIQParamsStruct *p = MRIQKernelParams;
+    // Block positions: x = blocks of 256 voxels, y = chunks of MRIQ_K_CHUNK k records (the
+    // reference's host loop over k chunks, mriq_kernel.cu:258-283, as a grid dimension).
+    // GPTBKernel takes its six dimension ints from here; the natural launch below runs one
+    // workgroup per voxel block, which walks all chunks itself.
+    const int chunks = p->numK > 0 ? (p->numK + MRIQ_K_CHUNK - 1) / MRIQ_K_CHUNK : 1;
+    launchGridDim = dim3(numX_ / KERNEL_Q_THREADS_PER_BLOCK, chunks, 1);
+    launchBlockDim = dim3(KERNEL_Q_THREADS_PER_BLOCK, 1, 1);
     kernelParams = {&p->numK, &p->kGlobalIndex, &p->x, &p->y, &p->z, &p->Qr, &p->Qi};
     this->smem = 0;
     auto it = fmap.find("ori_mriq");
@@ -110,6 +115,7 @@ void OriMRIQKernel::bind()
 void OriMRIQKernel::executeImpl(cudaStream_t stream)
 {
     if (!kernelFunc) logger.ERROR("load kernel {ori_mriq} failed!");
-    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
+    const dim3 voxel_blocks(launchGridDim.x, 1, 1);
+    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, voxel_blocks.raw(), launchBlockDim.raw(),
                                 (void **)this->kernelParams.data(), 0, stream));
 }

@@ -48,8 +48,9 @@ KERNEL_INFO = {
                 "ori_blks": 1024},
     "lbm": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
             "ori_blks": 18000},
+    # 1024 blocks of 256 voxels x 16 chunks of 128 k records
     "mriq": {"register": 40, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
-             "ori_blks": 1024},
+             "ori_blks": 16384},
     "cp": {"register": 40, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
            "ori_blks": 16384},
 }

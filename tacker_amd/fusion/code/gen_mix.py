@@ -97,7 +97,7 @@ extern "C" __global__ __launch_bounds__({total}) void {name}(
     if ({tz_cond}) {{
         // One tzgemm wave per SIMD shares it with {be} waves: let the MFMA stream issue
         // whenever it is ready and the {be} waves fill the slots it leaves.
-        __builtin_amdgcn_s_setprio(3);
+        __builtin_amdgcn_s_setprio(TK_GEMM_WAVE_PRIORITY);
         tk::RoleSpinSync sync(tz_arrivals, {tz_threads // 64}, &tk_spin_fail);
         {tz_call}
     }} else {{

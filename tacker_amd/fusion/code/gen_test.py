@@ -64,7 +64,7 @@ def make_inputs(np, torch, ta, be, small):
         ta.mriq_set_kvalues(kv)
         xyz = [torch.from_numpy(rng.uniform(-0.5, 0.5, numX).astype(np.float32)).cuda() for _ in range(3)]
         Qr, Qi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
-        return ta.ori_mriq_create(numK, xyz[0], xyz[1], xyz[2], Qr, Qi), numX // 256, [Qr, Qi]
+        return ta.ori_mriq_create(numK, xyz[0], xyz[1], xyz[2], Qr, Qi), ta.mriq_blocks(numK, numX), [Qr, Qi]
     if be == "cp":
         ta.cp_set_atoms(ta.cp_initatoms(4000)[1:65], 0.0)
         shape = (32, 512) if small else (4096, 4096)

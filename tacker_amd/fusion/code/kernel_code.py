@@ -50,7 +50,7 @@ ROLES = {
                    ("float*", "z"), ("float*", "Qr"), ("float*", "Qi")],
         "needs_sync": False,
         "call": ("tk::mriq_role({p}numK, {p}x, {p}y, {p}z, {p}Qr, {p}Qi, {p}grid_dimension_x, "
-                 "{block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "{p}grid_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "{threads});"),
     },
     "cp": {

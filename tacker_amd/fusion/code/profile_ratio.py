@@ -32,7 +32,7 @@ DEFAULTS = os.path.join(HERE, "defaults.json")
 K_LADDER = (128, 640, 1152, 2048, 2304, 4096, 4608)
 PAIRS = ("stencil", "lbm", "mriq", "cp")
 TILES = 1024
-LADDER = 16          # best-effort block counts tried: N/16, 2N/16, ..., N
+LADDER = 32          # best-effort block counts tried: N/32, 2N/32, ..., N
 
 
 def measure(out_path, stretch, launches):

@@ -148,3 +148,31 @@ def test_config4_tzgemm_2048_and_mriq_2048x262144():
     ok, dmax = gemm_sample_ok(host(mix_c), A, B, np.arange(0, M, 97))
     assert ok, dmax
     assert ta.spin_fail_flag() == 0
+
+
+def test_config4_mriq_spread_over_nine_fused_launches_equals_one_launch():
+    # the co-location pattern of benchmark configuration 4: the k-chunk x voxel-block grid of mri-q is cut
+    # into 9 consecutive slices, each riding with one GEMM launch; Q must come out bit-identical to the kernel
+    # run alone (a float carried through memory between chunks is the float the one k loop keeps in a register)
+    M = N = K = 2048
+    A, B = gemm_inputs(M, N, K, seed=23)
+    numK, numX = 2048, 262144
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX, seed=4)
+    kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+    ta.mriq_set_kvalues(kv)
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    dA, dB = dev(A), dev(B)
+    solo_r, solo_i = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    ta.ori_mriq(numK, x, y, z, solo_r, solo_i)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, solo_c)
+    Qr, Qi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    mix_c = torch.zeros((M, N), device="cuda:0")
+    total = ta.mriq_blocks(numK, numX)
+    assert total == 1024 * 16
+    n = 9
+    for i in range(n):
+        ta.mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, dA, dB, mix_c, be_start=total * i // n, be_end=total * (i + 1) // n)
+    assert np.array_equal(host(Qr), host(solo_r)) and np.array_equal(host(Qi), host(solo_i))
+    assert np.array_equal(host(mix_c), host(solo_c))
+    assert ta.spin_fail_flag() == 0

@@ -218,6 +218,52 @@ def test_mriq_closed_forms_and_ranges():
     assert np.array_equal(pr[256:768], fr[256:768]) and np.all(pr[:256] == 0) and np.all(pr[768:] == 0)
 
 
+def test_mriq_block_positions_are_voxel_blocks_by_k_chunks():
+    # numK 300 -> chunks of 128, 128 and 44 records; 4 voxel blocks -> 12 block positions
+    numK, numX = 300, 1024
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX, seed=5)
+    kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+    ta.mriq_set_kvalues(kv)
+    assert ta.mriq_blocks(numK, numX) == 12 and ta.mriq_blocks(0, numX) == 4 and ta.mriq_blocks(128, numX) == 4
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    q0 = np.linspace(-1, 1, numX).astype(np.float32)
+
+    def run(ranges, **kw):
+        Qr, Qi = dev(q0), dev(q0)
+        for a, b in ranges:
+            ta.gptb_mriq(numK, x, y, z, Qr, Qi, start=a, end=b, **kw)
+        return host(Qr), host(Qi)
+
+    Qr, Qi = dev(q0), dev(q0)
+    ta.ori_mriq(numK, x, y, z, Qr, Qi)
+    ori = host(Qr), host(Qi)
+    # the whole grid in one launch, for several launch shapes (3 workgroups: owners hold two
+    # voxel blocks; 7: more workgroups than voxel blocks), equals the natural kernel bit for bit
+    for kw in ({}, {"launch_grid": 3}, {"launch_grid": 7}, {"launch_grid": 1}):
+        got = run([(0, 12)], **kw)
+        assert np.array_equal(got[0], ori[0]) and np.array_equal(got[1], ori[1]), kw
+    # so does any tiling of it by ascending ranges: inside a row, across a row end, whole rows
+    for tiling in ([(0, 3), (3, 5), (5, 11), (11, 12)], [(0, 4), (4, 8), (8, 12)], [(0, 1), (1, 12)],
+                   [(0, 6), (6, 12)], [(i, i + 1) for i in range(12)]):
+        got = run(tiling, launch_grid=3)
+        assert np.array_equal(got[0], ori[0]) and np.array_equal(got[1], ori[1]), tiling
+    # positions 5 and 6 alone: chunk 1 (records 128..255) onto voxel blocks 1 and 2
+    got = run([(5, 7)])
+    sel = slice(256, 768)
+    tr, ti = oracle.mriq(kv[128:256], xyz[0][sel], xyz[1][sel], xyz[2][sel], q0[sel], q0[sel], f64=True)
+    assert mriq_close(got[0][sel], tr.astype(np.float64)) and mriq_close(got[1][sel], ti.astype(np.float64))
+    assert np.array_equal(got[0][:256], q0[:256]) and np.array_equal(got[0][768:], q0[768:])
+    assert np.array_equal(got[1][:256], q0[:256]) and np.array_equal(got[1][768:], q0[768:])
+    # positions past the grid wrap as the reference's index arithmetic does (block p % x, chunk
+    # (p / x) % y): [0, 24) adds every chunk twice, [10, 14) = last chunk of blocks 2,3 then first of 0,1
+    twice = run([(0, 24)], launch_grid=3)
+    again = run([(0, 12), (0, 12)], launch_grid=5)
+    assert np.array_equal(twice[0], again[0]) and np.array_equal(twice[1], again[1])
+    wrap = run([(10, 14)])
+    split = run([(10, 12), (0, 2)])
+    assert np.array_equal(wrap[0], split[0]) and np.array_equal(wrap[1], split[1])
+
+
 # ------------------------------------------------------------------ cp
 def cp_atoms():
     atoms = ta.cp_initatoms(4000)
@@ -372,7 +418,8 @@ def _small_be(name):
         kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
         ta.mriq_set_kvalues(kv)
         Qr, Qi = torch.zeros(2048, device="cuda:0"), torch.zeros(2048, device="cuda:0")
-        return ta.ori_mriq_create(256, dev(xyz[0]), dev(xyz[1]), dev(xyz[2]), Qr, Qi), 8, [Qr, Qi]
+        return (ta.ori_mriq_create(256, dev(xyz[0]), dev(xyz[1]), dev(xyz[2]), Qr, Qi), ta.mriq_blocks(256, 2048),
+                [Qr, Qi])
     ta.cp_set_atoms(cp_atoms(), 0.0)
     g = torch.zeros((32, 512), device="cuda:0")
     return ta.ori_cp_create(64, 0.1, g), (512 // 128) * (32 // 8), [g]
