@@ -180,8 +180,15 @@ TK_API int tacker_cp_initatoms(float *atoms_host, int count, unsigned volx, unsi
                                unsigned volz, float gridspacing);
 /* ori_cp / g_general_ptb_cp (src/ori_kernel/cp_kernel.cu:26-79,
  * src/gptb_kernel/cp_kernel.cu:8-96): energygrid[voly][volx] += potential of the
- * atoms set by tacker_cp_set_atoms; volx multiple of 128, voly multiple of 8;
- * blocks [block_start, block_end) of the (volx/128, voly/8) grid. */
+ * atoms set by tacker_cp_set_atoms; volx multiple of 128, voly multiple of 8.
+ * ori_cp runs the (volx/128, voly/8) blocks of 128 x 8 points. The GPTB form works on
+ * block positions [block_start, block_end) of a (volx/128, voly/8, TACKER_CP_X_PARTS)
+ * grid: position p computes part p / blocks of block p % blocks, a part being 2 of the 8
+ * x points each thread of the block owns (the reference's 3-D index reconstruction over a
+ * grid whose z splits the unrolled points). [0, tacker_cp_blocks(volx, voly)) equals
+ * ori_cp bit for bit, and so does any set of ranges that tiles it. */
+#define TACKER_CP_X_PARTS 4
+TK_API int tacker_cp_blocks(int volx, int voly);
 TK_API int tacker_ori_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly,
                          tkStream_t stream);
 TK_API int tacker_gptb_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly,

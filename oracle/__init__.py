@@ -51,10 +51,10 @@ def _declare(l):
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
     l.orc_mriq_gptb.argtypes = [C.c_int, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, C.c_int,
-                                C.c_int, C.c_int, C.c_int]
+                                C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_cp_initatoms.argtypes = [_f32p, C.c_int, C.c_uint, C.c_uint, C.c_uint, C.c_float]
     l.orc_cp_atoms_to_const.argtypes = [_f32p, C.c_int, C.c_float, _f32p]
-    l.orc_cp_gptb.argtypes = [C.c_int, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+    l.orc_cp_gptb.argtypes = [C.c_int, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_mnk_from_conv_args.argtypes = [_i32p, _i32p]
     l.orc_im2col.argtypes = [C.c_int, _f32p] + [C.c_int] * 12 + [_f32p]
 
@@ -147,20 +147,28 @@ def mriq_phimag(phiR, phiI):
     return out
 
 
-def mriq(kvals, x, y, z, Qr, Qi, start=0, end=None, gdx=None, f64=False):
-    """kvals is [numK][4] float32 {Kx,Ky,Kz,PhiMag}. Returns (Qr, Qi)."""
+def mriq(kvals, x, y, z, Qr, Qi, start=0, end=None, gdx=None, f64=False, kchunk=None):
+    """kvals is [numK][4] float32 {Kx,Ky,Kz,PhiMag}. Returns (Qr, Qi).
+
+    Block positions [start, end).  kchunk=None: one position per block of 256 voxels, each adding
+    the whole table.  kchunk=n: positions form a grid of gdx voxel blocks by ceil(numK / n) chunks of
+    the table; position p adds chunk (p // gdx) % chunks to voxel block p % gdx."""
     kvals = np.ascontiguousarray(kvals, np.float32)
     numK = kvals.shape[0]
     numX = x.size
     if gdx is None:
         gdx = numX // 256
+    if kchunk is None:
+        gdy, kchunk = 1, max(numK, 1)
+    else:
+        gdy = max(1, -(-numK // kchunk))
     if end is None:
-        end = gdx
+        end = gdx * gdy
     qr = np.array(Qr, np.float32, order="C")
     qi = np.array(Qi, np.float32, order="C")
     lib().orc_mriq_gptb(numK, kvals.reshape(-1), np.ascontiguousarray(x, np.float32),
                         np.ascontiguousarray(y, np.float32), np.ascontiguousarray(z, np.float32),
-                        qr, qi, gdx, start, end, 1 if f64 else 0)
+                        qr, qi, gdx, gdy, kchunk, start, end, 1 if f64 else 0)
     return qr, qi
 
 
@@ -178,15 +186,19 @@ def cp_atoms_to_const(atoms, zplane=0.0):
     return out.reshape(-1, 4)
 
 
-def cp(atominfo, energygrid, gridspacing=0.1, start=0, end=None):
-    """energygrid is [voly][volx] float32 (volx multiple of 128, voly multiple of 8)."""
+def cp(atominfo, energygrid, gridspacing=0.1, start=0, end=None, parts=1):
+    """energygrid is [voly][volx] float32 (volx multiple of 128, voly multiple of 8).
+
+    Block positions [start, end) of the (volx/128, voly/8, parts) grid: parts=1, a position is a block of
+    128 x 8 points; parts=4, position p is part p // blocks (2 of the 8 x-points of each thread) of block
+    p % blocks."""
     voly, volx = energygrid.shape
     gdx, gdy = volx // 128, voly // 8
     if end is None:
-        end = gdx * gdy
+        end = gdx * gdy * parts
     atominfo = np.ascontiguousarray(atominfo, np.float32).reshape(-1)
     out = np.array(energygrid, np.float32, order="C")
-    lib().orc_cp_gptb(atominfo.size // 4, gridspacing, out.reshape(-1), atominfo, gdx, gdy, start, end)
+    lib().orc_cp_gptb(atominfo.size // 4, gridspacing, out.reshape(-1), atominfo, gdx, gdy, parts, start, end)
     return out
 
 

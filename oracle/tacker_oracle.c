@@ -22,7 +22,9 @@
  *                         conservation, rest-equilibrium fixed point,
  *                         independent numpy formulation.
  *   orc_mriq*             x=0 closed form, single-k closed form, numpy
- *                         float64 brute force.
+ *                         float64 brute force; block-by-chunk positions: any
+ *                         ascending tiling = the one k loop bit for bit, one
+ *                         position = numpy float64 over its record range.
  *   orc_cp*               single atom closed form, numpy float64 brute force,
  *                         ori_blks = 16384 held by fusion/code/kinfo.json.
  *   orc_im2col            direct convolution brute force.
@@ -401,49 +403,66 @@ ORC_API void orc_mriq_phimag(const float *phiR, const float *phiI, float *phiMag
  * samples (the reference's "QGrid < 1" loop stops after the first 1024-sample
  * chunk, :58-59; the intended Parboil semantics is every chunk in order, which
  * for one voxel is simply k = 0..numK-1 in sequence).  kvals is the AoS table
- * {Kx,Ky,Kz,PhiMag} (src/header/mriq_header.h:12-17).  GPTB form: voxel blocks
- * of 256 (KERNEL_Q_THREADS_PER_BLOCK) in [start,end), block_id_x wraps modulo
- * grid_dimension_x (src/gptb_kernel/mriq_kernel.cu:17-33).  Read-modify-write
- * on Qr/Qi.  f64 = 1: double arithmetic throughout (truth), written back as
- * float. */
-ORC_API void orc_mriq_gptb(int numK, const float *kvals, const float *x, const float *y,
-                           const float *z, float *Qr, float *Qi, int gdx, int start, int end, int f64)
+ * {Kx,Ky,Kz,PhiMag} (src/header/mriq_header.h:12-17).
+ *
+ * GPTB form (src/gptb_kernel/mriq_kernel.cu:17-33 index reconstruction, with the
+ * host's loop over k chunks, src/ori_kernel/mriq_kernel.cu:258-283, as the y index
+ * of the grid): block positions [start,end) of a gdx x gdy grid; position p adds
+ * the records [c*kchunk, min(numK,(c+1)*kchunk)) of chunk c = (p / gdx) % gdy to
+ * the 256 voxels (KERNEL_Q_THREADS_PER_BLOCK) of block p % gdx, positions in
+ * ascending order.  gdy = 1 and kchunk >= numK is the plain form: every position
+ * adds the whole table.  Read-modify-write on Qr/Qi.  f64 = 1: double arithmetic
+ * throughout (truth), written back as float once per position. */
+static void orc_mriq_voxel(int k0, int k1, const float *kvals, const float *x, const float *y,
+                           const float *z, float *Qr, float *Qi, int xi, int f64)
 {
     const float PIx2 = 6.2831853071795864769252867665590058f;
+    if (f64) {
+        double sx = x[xi], sy = y[xi], sz = z[xi];
+        double qr = Qr[xi], qi = Qi[xi];
+        for (int k = k0; k < k1; k++) {
+            const float *kv = kvals + 4 * (size_t)k;
+            double arg = 6.2831853071795864769252867665590058 *
+                         ((double)kv[0] * sx + (double)kv[1] * sy + (double)kv[2] * sz);
+            qr += (double)kv[3] * cos(arg);
+            qi += (double)kv[3] * sin(arg);
+        }
+        Qr[xi] = (float)qr;
+        Qi[xi] = (float)qi;
+    } else {
+        float sx = x[xi], sy = y[xi], sz = z[xi];
+        float qr = Qr[xi], qi = Qi[xi];
+        for (int k = k0; k < k1; k++) {
+            const float *kv = kvals + 4 * (size_t)k;
+            float a = kv[0] * sx, b = kv[1] * sy, c = kv[2] * sz;
+            float d = a + b;
+            d = d + c;
+            float arg = PIx2 * d;
+            float pc = kv[3] * cosf(arg);
+            float ps = kv[3] * sinf(arg);
+            qr = qr + pc;
+            qi = qi + ps;
+        }
+        Qr[xi] = qr;
+        Qi[xi] = qi;
+    }
+}
+
+ORC_API void orc_mriq_gptb(int numK, const float *kvals, const float *x, const float *y,
+                           const float *z, float *Qr, float *Qi, int gdx, int gdy, int kchunk,
+                           int start, int end, int f64)
+{
+    /* one thread per voxel block; its positions are start-aligned p, p+gdx, ... in order */
 #pragma omp parallel for schedule(static)
-    for (int pos = start; pos < end; pos++) {
-        int bx = pos % gdx;
-        for (int t = 0; t < 256; t++) {
-            int xi = bx * 256 + t;
-            if (f64) {
-                double sx = x[xi], sy = y[xi], sz = z[xi];
-                double qr = Qr[xi], qi = Qi[xi];
-                for (int k = 0; k < numK; k++) {
-                    const float *kv = kvals + 4 * (size_t)k;
-                    double arg = 6.2831853071795864769252867665590058 *
-                                 ((double)kv[0] * sx + (double)kv[1] * sy + (double)kv[2] * sz);
-                    qr += (double)kv[3] * cos(arg);
-                    qi += (double)kv[3] * sin(arg);
-                }
-                Qr[xi] = (float)qr;
-                Qi[xi] = (float)qi;
-            } else {
-                float sx = x[xi], sy = y[xi], sz = z[xi];
-                float qr = Qr[xi], qi = Qi[xi];
-                for (int k = 0; k < numK; k++) {
-                    const float *kv = kvals + 4 * (size_t)k;
-                    float a = kv[0] * sx, b = kv[1] * sy, c = kv[2] * sz;
-                    float d = a + b;
-                    d = d + c;
-                    float arg = PIx2 * d;
-                    float pc = kv[3] * cosf(arg);
-                    float ps = kv[3] * sinf(arg);
-                    qr = qr + pc;
-                    qi = qi + ps;
-                }
-                Qr[xi] = qr;
-                Qi[xi] = qi;
-            }
+    for (int bx = 0; bx < gdx; bx++) {
+        int first = start + ((bx - start % gdx) + gdx) % gdx;
+        for (int pos = first; pos < end; pos += gdx) {
+            int chunk = (pos / gdx) % gdy;
+            long k0 = (long)chunk * kchunk, k1 = k0 + kchunk;
+            if (k0 > numK) k0 = numK;
+            if (k1 > numK) k1 = numK;
+            for (int t = 0; t < 256; t++)
+                orc_mriq_voxel((int)k0, (int)k1, kvals, x, y, z, Qr, Qi, bx * 256 + t, f64);
         }
     }
 }
@@ -486,42 +505,58 @@ ORC_API void orc_cp_atoms_to_const(const float *atoms, int count, float zplane, 
 
 /* src/gptb_kernel/cp_kernel.cu:8-96 (= ori_cp, src/ori_kernel/cp_kernel.cu:26-79,
  * with blockIdx reconstructed): grid (gdx,gdy) of (16,8) blocks, each thread 8
- * x-points 16 apart.  energygrid has row pitch gdx*16*8.  Blocks [start,end). */
+ * x-points 16 apart.  energygrid has row pitch gdx*16*8.
+ *
+ * Block positions [start,end) of a (gdx,gdy,gdz) grid, index reconstruction as in
+ * the reference's 3-D kernels (block_id_z = pos / (x*y) % z): position p computes,
+ * for block p % (gdx*gdy), the x-points n in [part*8/gdz, (part+1)*8/gdz) of every
+ * thread, part = (p / (gdx*gdy)) % gdz; dx of point n is reached by the chain of
+ * additions of the 8-point loop.  gdz = 1: a position is a whole block.  Positions
+ * of one block are applied in ascending order. */
 ORC_API void orc_cp_gptb(int numatoms, float gridspacing, float *energygrid, const float *atominfo,
-                         int gdx, int gdy, int start, int end)
+                         int gdx, int gdy, int gdz, int start, int end)
 {
     const int BX = 16, BY = 8, UNROLLX = 8;
+    const int blocks = gdx * gdy;
+    const int per_part = UNROLLX / gdz;
 #pragma omp parallel for schedule(static)
-    for (int pos = start; pos < end; pos++) {
-        unsigned bx = (unsigned)pos % (unsigned)gdx;
-        unsigned by = ((unsigned)pos / (unsigned)gdx) % (unsigned)gdy;
-        for (unsigned ty = 0; ty < (unsigned)BY; ty++) {
-            for (unsigned tx = 0; tx < (unsigned)BX; tx++) {
-                unsigned xindex = bx * BX * UNROLLX + tx;
-                unsigned yindex = by * BY + ty;
-                unsigned outaddr = ((unsigned)gdx * BX * UNROLLX) * yindex + xindex;
-                float coory = gridspacing * yindex;
-                float coorx = gridspacing * xindex;
-                float e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-                float gridspacing_u = gridspacing * BX;
-                for (int a = 0; a < numatoms; a++) {
-                    const float *at = atominfo + 4 * a;
-                    float dy = coory - at[1];
-                    float dy2 = dy * dy;
-                    float dyz2 = dy2 + at[2];
-                    float dx = coorx - at[0];
-                    for (int n = 0; n < 8; n++) {
-                        float dx2 = dx * dx;
-                        float r2 = dx2 + dyz2;
-                        float inv = 1.0f / sqrtf(r2);
-                        float contrib = at[3] * inv;
-                        e[n] = e[n] + contrib;
-                        dx = dx + gridspacing_u;
+    for (int blk = 0; blk < blocks; blk++) {
+        int first = start + ((blk - start % blocks) + blocks) % blocks;
+        for (int pos = first; pos < end; pos += blocks) {
+            unsigned bx = (unsigned)pos % (unsigned)gdx;
+            unsigned by = ((unsigned)pos / (unsigned)gdx) % (unsigned)gdy;
+            int part = (pos / blocks) % gdz;
+            int n0 = part * per_part, n1 = n0 + per_part;
+            for (unsigned ty = 0; ty < (unsigned)BY; ty++) {
+                for (unsigned tx = 0; tx < (unsigned)BX; tx++) {
+                    unsigned xindex = bx * BX * UNROLLX + tx;
+                    unsigned yindex = by * BY + ty;
+                    unsigned outaddr = ((unsigned)gdx * BX * UNROLLX) * yindex + xindex;
+                    float coory = gridspacing * yindex;
+                    float coorx = gridspacing * xindex;
+                    float e[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+                    float gridspacing_u = gridspacing * BX;
+                    for (int a = 0; a < numatoms; a++) {
+                        const float *at = atominfo + 4 * a;
+                        float dy = coory - at[1];
+                        float dy2 = dy * dy;
+                        float dyz2 = dy2 + at[2];
+                        float dx = coorx - at[0];
+                        for (int n = 0; n < n1; n++) {
+                            if (n >= n0) {
+                                float dx2 = dx * dx;
+                                float r2 = dx2 + dyz2;
+                                float inv = 1.0f / sqrtf(r2);
+                                float contrib = at[3] * inv;
+                                e[n] = e[n] + contrib;
+                            }
+                            dx = dx + gridspacing_u;
+                        }
                     }
-                }
-                for (int n = 0; n < 8; n++) {
-                    float *p = &energygrid[outaddr + (unsigned)n * BX];
-                    *p = *p + e[n];
+                    for (int n = n0; n < n1; n++) {
+                        float *p = &energygrid[outaddr + (unsigned)n * BX];
+                        *p = *p + e[n];
+                    }
                 }
             }
         }

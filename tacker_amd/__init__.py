@@ -43,6 +43,7 @@ def _declare(lib):
     lib.tacker_mriq_phimag.argtypes = [vp, vp, vp, i, vp]
     lib.tacker_mriq_set_kvalues.argtypes = [vp, i]
     lib.tacker_mriq_blocks.argtypes = [i, i]
+    lib.tacker_cp_blocks.argtypes = [i, i]
     lib.tacker_ori_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, vp]
     lib.tacker_gptb_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     lib.tacker_cp_set_atoms.argtypes = [vp, i, f]
@@ -271,6 +272,11 @@ def cp_set_atoms(atoms_np, zplane=0.0):
     check(lib().tacker_cp_set_atoms(a.ctypes.data, a.shape[0], zplane), "tacker_cp_set_atoms")
 
 
+def cp_blocks(volx, voly):
+    """block positions of the GPTB form: blocks of 128 x 8 points x parts of the unrolled x points"""
+    return lib().tacker_cp_blocks(volx, voly)
+
+
 def ori_cp(numatoms, gridspacing, grid, stream=None):
     voly, volx = grid.shape
     check(lib().tacker_ori_cp(numatoms, gridspacing, _ptr(grid), volx, voly, _stream(stream)),
@@ -280,7 +286,7 @@ def ori_cp(numatoms, gridspacing, grid, stream=None):
 def gptb_cp(numatoms, gridspacing, grid, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
     voly, volx = grid.shape
     if end is None:
-        end = (volx // 128) * (voly // 8)
+        end = cp_blocks(volx, voly)
     check(lib().tacker_gptb_cp(numatoms, gridspacing, _ptr(grid), volx, voly, start, end, launch_grid,
                                launch_block, _stream(stream)), "tacker_gptb_cp")
 
@@ -329,7 +335,7 @@ def mix_tzgemm_cp(numatoms, gridspacing, grid, A, B, Cm, be_start=0, be_end=None
                   tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
     voly, volx = grid.shape
     if be_end is None:
-        be_end = (volx // 128) * (voly // 8)
+        be_end = cp_blocks(volx, voly)
     check(lib().tacker_mix_tzgemm_cp(
         numatoms, gridspacing, _ptr(grid), volx, voly, be_start, be_end,
         *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),

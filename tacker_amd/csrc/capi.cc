@@ -306,6 +306,13 @@ int tacker_cp_initatoms(float *atoms_host, int count, unsigned volx, unsigned vo
     return TK_SUCCESS;
 }
 
+int tacker_cp_blocks(int volx, int voly)
+{
+    static_assert(TACKER_CP_X_PARTS == CP_X_PARTS, "public and device part counts must agree");
+    if (volx < 0 || voly < 0) return 0;
+    return (volx / (BLOCKSIZEX * UNROLLX)) * (voly / BLOCKSIZEY) * CP_X_PARTS;
+}
+
 int tacker_ori_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, tkStream_t stream)
 {
     REQUIRE_INIT();

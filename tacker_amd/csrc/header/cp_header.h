@@ -8,3 +8,7 @@
 #define VOLSIZEX 4096
 #define VOLSIZEY 4096
 #define ATOMCOUNT 4000
+// x points of a thread that one block position of the GPTB form computes, and the
+// positions a block is made of (the switch in cp_role lists the parts: keep it at 4)
+#define CP_POINTS_PER_POSITION 2
+#define CP_X_PARTS (UNROLLX / CP_POINTS_PER_POSITION)

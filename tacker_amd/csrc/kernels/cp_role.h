@@ -91,40 +91,155 @@ __device__ __forceinline__ void cp_block_pair(int numatoms, float gridspacing,
         for (int n = 0; n < UNROLLX; ++n) energygrid[outaddr[b] + n * BLOCKSIZEX] += energyval[b][n];
 }
 
+// U positions of one x part per thread at once: U blocks, CP_POINTS_PER_POSITION points of
+// each.  PART selects the points n in [PART * P, (PART + 1) * P) of the UNROLLX a block's
+// thread owns; their dx is reached by the same chain of additions cp_block runs through
+// (dx_{n+1} = dx_n + 16 * spacing), so every value equals the one cp_block stores.
+template <int U, int PART>
+__device__ __forceinline__ void cp_positions(int numatoms, float gridspacing, float *__restrict__ energygrid,
+                                             const unsigned (&block)[U], unsigned grid_dimension_x,
+                                             unsigned thread_id_x, unsigned thread_id_y)
+{
+    constexpr int P = CP_POINTS_PER_POSITION;
+    unsigned outaddr[U];
+    float coory[U], coorx[U];
+    float energyval[U][P];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const unsigned xindex = (block[u] % grid_dimension_x) * BLOCKSIZEX * UNROLLX + thread_id_x;
+        const unsigned yindex = (block[u] / grid_dimension_x) * BLOCKSIZEY + thread_id_y;
+        outaddr[u] = (grid_dimension_x * BLOCKSIZEX * UNROLLX) * yindex + xindex + PART * P * BLOCKSIZEX;
+        coory[u] = gridspacing * yindex;
+        coorx[u] = gridspacing * xindex;
+#pragma unroll
+        for (int n = 0; n < P; ++n) energyval[u][n] = 0.0f;
+    }
+    const float gridspacing_u = gridspacing * BLOCKSIZEX;
+    for (int atomid = 0; atomid < numatoms; ++atomid) {
+        const float4 a = atominfo[atomid];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const float dy = coory[u] - a.y;
+            const float dyz2 = (dy * dy) + a.z;
+            float dx = coorx[u] - a.x;
+#pragma unroll
+            for (int n = 0; n < PART * P; ++n) dx = dx + gridspacing_u;
+#pragma unroll
+            for (int n = 0; n < P; ++n) {
+                energyval[u][n] += a.w * (1.0f / sqrtf(dx * dx + dyz2));
+                dx = dx + gridspacing_u;
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int n = 0; n < P; ++n) energygrid[outaddr[u] + n * BLOCKSIZEX] += energyval[u][n];
+}
+
+template <int PART>
+__device__ __forceinline__ void cp_part_phase(int numatoms, float gridspacing, float *__restrict__ energygrid,
+                                              int block_lo, int block_hi, unsigned grid_dimension_x,
+                                              int first_owned, int stride, unsigned tx, unsigned ty)
+{
+    int b = first_owned;
+    if (b < block_lo) b += (block_lo - b + stride - 1) / stride * stride;
+    // 4, 2 or 1 of the thread's blocks at a time: 8, 4 or 2 independent sqrt/divide chains
+    for (; b + 3 * stride < block_hi; b += 4 * stride) {
+        const unsigned four[4] = {(unsigned)b, (unsigned)(b + stride), (unsigned)(b + 2 * stride),
+                                  (unsigned)(b + 3 * stride)};
+        cp_positions<4, PART>(numatoms, gridspacing, energygrid, four, grid_dimension_x, tx, ty);
+    }
+    if (b + stride < block_hi) {
+        const unsigned two[2] = {(unsigned)b, (unsigned)(b + stride)};
+        cp_positions<2, PART>(numatoms, gridspacing, energygrid, two, grid_dimension_x, tx, ty);
+        b += 2 * stride;
+    }
+    if (b < block_hi) {
+        const unsigned one[1] = {(unsigned)b};
+        cp_positions<1, PART>(numatoms, gridspacing, energygrid, one, grid_dimension_x, tx, ty);
+    }
+}
+
+// Block positions of the GPTB form are a grid of grid_dimension_x * grid_dimension_y
+// blocks (the reference's (16,8)-thread blocks of 128 x 8 points) by grid_dimension_z =
+// CP_X_PARTS parts: position p does part (p / blocks) % parts of block p % blocks, a part
+// being CP_POINTS_PER_POSITION of the UNROLLX points each thread of the block owns -- the
+// reference's 3-D index reconstruction (block_id_z = pos / (x * y) % z) over a grid whose z
+// splits the unrolled x points, so that a short range of positions is a short piece of
+// work.  Every output point is computed whole by one thread, so any split of the grid into
+// ranges stores the bits cp_block stores.
+//
+// A range [start, end) is a partial first row of that grid (one part of some blocks), whole
+// rows, and a partial last row.  Every block has one owner thread group for the whole launch
+// (slot-major over the role's workgroups), and the owner walks the rows in order: a range
+// that runs past the grid and comes round to a point again adds to it a second time, after
+// the first.  CP_X_PARTS whole rows that make up all parts of every block are served by the
+// whole-block code, two blocks at a time.
 __device__ __forceinline__ void cp_role(int numatoms, float gridspacing,
                                         float *__restrict__ energygrid, int grid_dimension_x,
-                                        int grid_dimension_y, int role_block, int role_blocks,
-                                        int start, int end, int tid, int role_threads)
+                                        int grid_dimension_y, int grid_dimension_z, int role_block,
+                                        int role_blocks, int start, int end, int tid, int role_threads)
 {
     constexpr int BLOCK_THREADS = BLOCKSIZEX * BLOCKSIZEY;
     const int blocks_at_once = role_threads / BLOCK_THREADS;
     const int slot = tid / BLOCK_THREADS;
     const int t = tid % BLOCK_THREADS;
-    if (slot >= blocks_at_once) return;
-    const unsigned stride = (unsigned)role_blocks * blocks_at_once;
-    // blocks go round the role's workgroups first; a thread takes two that are one stride apart
-    // (two positions of one launch never name the same block unless the range wraps, and a
-    // wrapped range is served one block at a time so that its += land one after the other)
-    const bool wraps = (unsigned)(end - start) > (unsigned)(grid_dimension_x * grid_dimension_y);
-    for (unsigned pos = (unsigned)start + slot * role_blocks + role_block; pos < (unsigned)end;
-         pos += 2 * stride) {
-        const unsigned second = pos + stride;
-        if (second < (unsigned)end && !wraps) {
-            const unsigned bx[2] = {pos % grid_dimension_x, second % grid_dimension_x};
-            const unsigned by[2] = {(pos / grid_dimension_x) % grid_dimension_y,
-                                    (second / grid_dimension_x) % grid_dimension_y};
-            cp_block_pair(numatoms, gridspacing, energygrid, bx, by, grid_dimension_x, t % BLOCKSIZEX,
-                          t / BLOCKSIZEX);
+    if (slot >= blocks_at_once || start >= end) return;
+    const unsigned tx = t % BLOCKSIZEX, ty = t / BLOCKSIZEX;
+    const unsigned gx = grid_dimension_x;
+    const int blocks = grid_dimension_x * grid_dimension_y;
+    const int parts = grid_dimension_z;   // CP_X_PARTS from the host; 1 = whole blocks only
+    const int stride = role_blocks * blocks_at_once;
+    const int first_owned = slot * role_blocks + role_block;
+
+    const auto part_phase = [&](int lo, int hi, int row) {
+        if (parts == 1) {   // a position is a whole block
+            int b = first_owned;
+            if (b < lo) b += (lo - b + stride - 1) / stride * stride;
+            for (; b < hi; b += stride)
+                cp_block(numatoms, gridspacing, energygrid, b % gx, b / gx, gx, tx, ty);
+            return;
+        }
+        switch (row % parts) {
+        case 0: cp_part_phase<0>(numatoms, gridspacing, energygrid, lo, hi, gx, first_owned, stride, tx, ty); break;
+        case 1: cp_part_phase<1>(numatoms, gridspacing, energygrid, lo, hi, gx, first_owned, stride, tx, ty); break;
+        case 2: cp_part_phase<2>(numatoms, gridspacing, energygrid, lo, hi, gx, first_owned, stride, tx, ty); break;
+        default: cp_part_phase<3>(numatoms, gridspacing, energygrid, lo, hi, gx, first_owned, stride, tx, ty); break;
+        }
+    };
+    const auto whole_blocks = [&]() {   // all parts of every block
+        int b = first_owned;
+        for (; b + stride < blocks; b += 2 * stride) {
+            const unsigned bx[2] = {b % gx, (b + stride) % gx};
+            const unsigned by[2] = {b / gx, (b + stride) / gx};
+            cp_block_pair(numatoms, gridspacing, energygrid, bx, by, gx, tx, ty);
+        }
+        if (b < blocks) cp_block(numatoms, gridspacing, energygrid, b % gx, b / gx, gx, tx, ty);
+    };
+
+    const int first_row = start / blocks;
+    const int last_row = (end - 1) / blocks;
+    if (first_row == last_row) {
+        part_phase(start - first_row * blocks, end - first_row * blocks, first_row);
+        return;
+    }
+    int row = first_row;
+    if (start != first_row * blocks) {
+        part_phase(start - first_row * blocks, blocks, row);
+        ++row;
+    }
+    const int whole_end = (end == (last_row + 1) * blocks) ? last_row + 1 : last_row;
+    while (row < whole_end) {
+        if (parts > 1 && row % parts == 0 && row + parts <= whole_end) {
+            whole_blocks();
+            row += parts;
         } else {
-            cp_block(numatoms, gridspacing, energygrid, pos % grid_dimension_x,
-                     (pos / grid_dimension_x) % grid_dimension_y, grid_dimension_x, t % BLOCKSIZEX,
-                     t / BLOCKSIZEX);
-            if (second < (unsigned)end)
-                cp_block(numatoms, gridspacing, energygrid, second % grid_dimension_x,
-                         (second / grid_dimension_x) % grid_dimension_y, grid_dimension_x,
-                         t % BLOCKSIZEX, t / BLOCKSIZEX);
+            part_phase(0, blocks, row);
+            ++row;
         }
     }
+    if (whole_end == last_row) part_phase(0, end - last_row * blocks, last_row);
 }
 
 }  // namespace tk

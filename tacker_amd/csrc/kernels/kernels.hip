@@ -111,7 +111,7 @@ extern "C" __global__ void g_general_ptb_mriq(int numK, int kGlobalIndex, float 
 extern "C" __global__ void g_general_ptb_cp(int numatoms, float gridspacing, float *energygrid,
                                             GPTB_TRAILER)
 {
-    tk::cp_role(numatoms, gridspacing, energygrid, grid_dimension_x, grid_dimension_y,
+    tk::cp_role(numatoms, gridspacing, energygrid, grid_dimension_x, grid_dimension_y, grid_dimension_z,
                 (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
                 (int)threadIdx.x - thread_base, (int)blockDim.x);
 }

@@ -67,7 +67,9 @@ OriCPKernel::OriCPKernel(int id, int numatoms, float gridspacing, float *energyg
     moduleName = "ori_cp";
     CPKernelParams = new OriCPParamsStruct<float>{numatoms, gridspacing, energygrid};
     launchBlockDim = dim3(BLOCKSIZEX, BLOCKSIZEY, 1);
-    launchGridDim = dim3(volx / (BLOCKSIZEX * UNROLLX), voly / BLOCKSIZEY, 1);
+    // z: the parts a block's unrolled x points are split into for the GPTB form's block
+    // positions; the natural launch below runs the (x, y) blocks, each whole
+    launchGridDim = dim3(volx / (BLOCKSIZEX * UNROLLX), voly / BLOCKSIZEY, CP_X_PARTS);
     kernelParams = {&CPKernelParams->numatoms, &CPKernelParams->gridspacing, &CPKernelParams->energygrid};
     auto it = fmap.find("ori_cp");
     kernelFunc = it == fmap.end() ? nullptr : it->second;
@@ -106,7 +108,7 @@ void OriCPKernel::initParams()
     if (!this->initialized) {
         CPKernelParams = new OriCPParamsStruct<float>{runatoms, 0.1f, output};
         launchBlockDim = dim3(BLOCKSIZEX, BLOCKSIZEY, 1);
-        launchGridDim = dim3(volsize.x / (BLOCKSIZEX * UNROLLX), volsize.y / BLOCKSIZEY, 1);
+        launchGridDim = dim3(volsize.x / (BLOCKSIZEX * UNROLLX), volsize.y / BLOCKSIZEY, CP_X_PARTS);
         kernelParams = {&CPKernelParams->numatoms, &CPKernelParams->gridspacing, &CPKernelParams->energygrid};
         auto it = fmap.find("ori_cp");
         kernelFunc = it == fmap.end() ? nullptr : it->second;
@@ -118,7 +120,8 @@ void OriCPKernel::initParams()
 void OriCPKernel::executeImpl(cudaStream_t stream)
 {
     if (!kernelFunc) logger.ERROR("load kernel {ori_cp} failed!");
-    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
+    const dim3 whole_blocks(launchGridDim.x, launchGridDim.y, 1);
+    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, whole_blocks.raw(), launchBlockDim.raw(),
                                 (void **)this->kernelParams.data(), 0, stream));
 }
 

@@ -69,7 +69,7 @@ def make_inputs(np, torch, ta, be, small):
         ta.cp_set_atoms(ta.cp_initatoms(4000)[1:65], 0.0)
         shape = (32, 512) if small else (4096, 4096)
         grid = torch.zeros(shape, device="cuda:0")
-        return ta.ori_cp_create(64, 0.1, grid), (shape[1] // 128) * (shape[0] // 8), [grid]
+        return ta.ori_cp_create(64, 0.1, grid), ta.cp_blocks(shape[1], shape[0]), [grid]
     raise SystemExit(f"unknown kernel {be}")
 
 

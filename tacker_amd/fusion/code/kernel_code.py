@@ -57,7 +57,7 @@ ROLES = {
         "params": [("int", "numatoms"), ("float", "gridspacing"), ("float*", "energygrid")],
         "needs_sync": False,
         "call": ("tk::cp_role({p}numatoms, {p}gridspacing, {p}energygrid, {p}grid_dimension_x, "
-                 "{p}grid_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, "
+                 "{p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, {p}ptb_start_block_pos, "
                  "{p}ptb_end_block_pos, {tid}, {threads});"),
     },
 }

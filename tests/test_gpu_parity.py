@@ -247,6 +247,13 @@ def test_mriq_block_positions_are_voxel_blocks_by_k_chunks():
                    [(0, 6), (6, 12)], [(i, i + 1) for i in range(12)]):
         got = run(tiling, launch_grid=3)
         assert np.array_equal(got[0], ori[0]) and np.array_equal(got[1], ori[1]), tiling
+    # partial ranges against the oracle's restatement of the position grid (float64 truth)
+    for a, b in ((5, 7), (2, 11), (11, 12), (3, 4), (7, 17)):
+        got = run([(a, b)], launch_grid=3)
+        tr, ti = oracle.mriq(kv, xyz[0], xyz[1], xyz[2], q0, q0, start=a, end=b, kchunk=128, f64=True)
+        assert mriq_close(got[0], tr.astype(np.float64)) and mriq_close(got[1], ti.astype(np.float64)), (a, b)
+        same = tr == q0                                     # voxels the range does not touch
+        assert np.array_equal(got[0][same], q0[same]) and np.array_equal(got[1][same], q0[same]), (a, b)
     # positions 5 and 6 alone: chunk 1 (records 128..255) onto voxel blocks 1 and 2
     got = run([(5, 7)])
     sel = slice(256, 768)
@@ -286,13 +293,44 @@ def test_cp_bit_exact(shape):
     ta.gptb_cp(64, 0.1, g2, launch_grid=5)
     assert np.array_equal(host(g2).view(np.uint32), want.view(np.uint32))
     g3 = dev(g0)
-    nblk = (shape[1] // 128) * (shape[0] // 8)
+    nblk = ta.cp_blocks(shape[1], shape[0])
+    assert nblk == (shape[1] // 128) * (shape[0] // 8) * 4
     want3 = g0
     for s, e in [(0, 1), (1, nblk)]:
         ta.gptb_cp(64, 0.1, g3, start=s, end=e, launch_block=256)
-        want3 = oracle.cp(info, want3, start=s, end=e)
+        want3 = oracle.cp(info, want3, start=s, end=e, parts=4)
     assert np.array_equal(host(g3).view(np.uint32), want3.view(np.uint32))
     assert np.array_equal(want3, want)
+
+
+def test_cp_block_positions_are_blocks_by_x_parts():
+    atoms = cp_atoms()
+    ta.cp_set_atoms(atoms, 0.0)
+    info = oracle.cp_atoms_to_const(atoms, 0.0)
+    H, Wd = 24, 384                                    # 3 x 3 blocks x 4 parts = 36 positions
+    g0 = np.random.default_rng(9).uniform(-1, 1, (H, Wd)).astype(np.float32)
+    whole = oracle.cp(info, g0)
+    assert ta.cp_blocks(Wd, H) == 36
+
+    def run(ranges, **kw):
+        g = dev(g0)
+        for a, b in ranges:
+            ta.gptb_cp(64, 0.1, g, start=a, end=b, **kw)
+        return host(g)
+
+    same = lambda a, b: np.array_equal(a.view(np.uint32), b.view(np.uint32))
+    for kw in ({}, {"launch_grid": 1}, {"launch_grid": 2, "launch_block": 256}, {"launch_grid": 5}, {"launch_grid": 40}):
+        assert same(run([(0, 36)], **kw), whole), kw
+    for tiling in ([(0, 5), (5, 11), (11, 30), (30, 36)], [(0, 9), (9, 18), (18, 27), (27, 36)],
+                   [(i, i + 1) for i in range(36)], [(20, 36), (0, 20)], [(0, 10), (10, 36)]):
+        assert same(run(tiling, launch_grid=2), whole), tiling
+    # partial ranges against the oracle's restatement of the position grid, bit for bit
+    for a, b in ((5, 7), (3, 31), (35, 36), (9, 18), (8, 28), (17, 19)):
+        for kw in ({"launch_grid": 2}, {}):
+            assert same(run([(a, b)], **kw), oracle.cp(info, g0, start=a, end=b, parts=4)), (a, b, kw)
+    # past the grid the positions come round again: every point gets its sum a second time, after the first
+    assert same(run([(0, 72)], launch_grid=2), oracle.cp(info, whole))
+    assert same(run([(30, 42)], launch_grid=3), oracle.cp(info, g0, start=30, end=42, parts=4))
 
 
 def test_cp_fewer_atoms():
@@ -422,7 +460,7 @@ def _small_be(name):
                 [Qr, Qi])
     ta.cp_set_atoms(cp_atoms(), 0.0)
     g = torch.zeros((32, 512), device="cuda:0")
-    return ta.ori_cp_create(64, 0.1, g), (512 // 128) * (32 // 8), [g]
+    return ta.ori_cp_create(64, 0.1, g), ta.cp_blocks(512, 32), [g]
 
 
 @pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),

@@ -104,7 +104,8 @@ def test_task_manager_colocation_keeps_lc_results_and_reports():
 def test_create_kernel_objects_run_and_match_oracle_for_cp():
     k = ta.create_kernel("cp")
     info = k.info()
-    assert (info["ptb_start"], info["ptb_end"]) == (0, 16384) and info["ori_grid_x"] == 32 and info["ori_grid_y"] == 512
+    # 32 x 512 blocks of 128 x 8 points, each in 4 parts of its x points
+    assert (info["ptb_start"], info["ptb_end"]) == (0, 65536) and info["ori_grid_x"] == 32 and info["ori_grid_y"] == 512
     k.execute()
     torch.cuda.synchronize()
     for name in ("stencil", "lbm", "mriq"):

@@ -72,6 +72,43 @@ def test_mriq_block_range():
     assert (2097152 // 10) // 256 == 819
 
 
+def test_mriq_positions_of_the_block_by_chunk_grid():
+    # 300 records in chunks of 128 (128, 128, 44) over 4 voxel blocks: 12 positions
+    numK, numX = 300, 1024
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX)
+    kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+    q0 = np.linspace(-1, 1, numX).astype(np.float32)
+    whole = oracle.mriq(kv, *xyz, q0, q0)
+    # all positions = the one k loop, bit for bit (a float carried through memory is unchanged)
+    grid = oracle.mriq(kv, *xyz, q0, q0, kchunk=128)
+    assert np.array_equal(grid[0], whole[0]) and np.array_equal(grid[1], whole[1])
+    # and so is any ascending tiling of the positions
+    for tiling in ([(0, 3), (3, 5), (5, 11), (11, 12)], [(0, 4), (4, 8), (8, 12)], [(i, i + 1) for i in range(12)]):
+        qr, qi = q0, q0
+        for a, b in tiling:
+            qr, qi = oracle.mriq(kv, *xyz, qr, qi, start=a, end=b, kchunk=128)
+        assert np.array_equal(qr, whole[0]) and np.array_equal(qi, whole[1]), tiling
+    # position 6 = chunk 1 onto voxel block 2: records 128..255 only, voxels 512..767 only (numpy, float64)
+    qr, qi = oracle.mriq(kv, *xyz, q0, q0, start=6, end=7, kchunk=128, f64=True)
+    sel = slice(512, 768)
+    phase = 2 * np.pi * (kv[128:256, 0:1].astype(np.float64) * xyz[0][sel] + kv[128:256, 1:2].astype(np.float64) * xyz[1][sel]
+                         + kv[128:256, 2:3].astype(np.float64) * xyz[2][sel])
+    want_r = q0[sel] + (kv[128:256, 3:4].astype(np.float64) * np.cos(phase)).sum(axis=0)
+    want_i = q0[sel] + (kv[128:256, 3:4].astype(np.float64) * np.sin(phase)).sum(axis=0)
+    np.testing.assert_allclose(qr[sel], want_r, rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(qi[sel], want_i, rtol=1e-6, atol=1e-6)
+    rest = np.r_[0:512, 768:1024]
+    assert np.array_equal(qr[rest], q0[rest]) and np.array_equal(qi[rest], q0[rest])
+    # the last chunk is the short one: position 11 adds records 256..299 to voxel block 3
+    qr, _ = oracle.mriq(kv, *xyz, q0, q0, start=11, end=12, kchunk=128, f64=True)
+    only_tail, _ = oracle.mriq(kv[256:], *xyz, q0, q0, start=3, end=4, f64=True)
+    assert np.array_equal(qr, only_tail)
+    # positions past the grid wrap: chunk (p // 4) % 3, block p % 4
+    twice = oracle.mriq(kv, *xyz, q0, q0, start=0, end=24, kchunk=128)
+    again = oracle.mriq(kv, *xyz, *whole, kchunk=128)
+    assert np.array_equal(twice[0], again[0]) and np.array_equal(twice[1], again[1])
+
+
 # ------------------------------------------------------------------ cp
 def test_initatoms_matches_glibc_stream_and_box():
     atoms = oracle.cp_initatoms(count=100)
@@ -121,6 +158,39 @@ def test_cp_matches_float64_brute_force_and_ranges():
     assert np.array_equal(acc, got)
     # fusion/code/kinfo.json "cp.ori_blks" = 16384 = (4096/128)*(4096/8)
     assert (4096 // 128) * (4096 // 8) == 16384
+
+
+def test_cp_positions_of_the_block_by_x_part_grid():
+    atoms = oracle.cp_initatoms(count=70)
+    atominfo = oracle.cp_atoms_to_const(atoms[1:65], 0.0)
+    atominfo[:, 2] += np.float32(0.01)
+    H, Wd = 16, 384                                                    # 3 x 2 blocks, 4 parts: 24 positions
+    g0 = np.random.default_rng(8).uniform(-1, 1, (H, Wd)).astype(np.float32)
+    whole = oracle.cp(atominfo, g0)
+    # all positions, and any tiling of them, store the bits of the whole-block form
+    assert np.array_equal(oracle.cp(atominfo, g0, parts=4), whole)
+    for tiling in ([(0, 5), (5, 7), (7, 19), (19, 24)], [(0, 6), (6, 12), (12, 18), (18, 24)],
+                   [(i, i + 1) for i in range(24)], [(13, 24), (0, 13)]):
+        acc = g0
+        for a, b in tiling:
+            acc = oracle.cp(atominfo, acc, start=a, end=b, parts=4)
+        assert np.array_equal(acc, whole), tiling
+    # position 6 + 2 = part 1 of block 2 (bx 2, by 0): columns 256 + {32..63} of rows 0..7, nothing else
+    one = oracle.cp(atominfo, g0, start=8, end=9, parts=4)
+    touched = np.zeros((H, Wd), bool)
+    touched[0:8, 256 + 32:256 + 64] = True
+    assert np.array_equal(one[touched], whole[touched]) and np.array_equal(one[~touched], g0[~touched])
+    # points of part 3 against float64 directly (their dx comes out of six chained additions)
+    last = oracle.cp(atominfo, np.zeros((H, Wd), np.float32), start=18, end=24, parts=4)
+    yy, xx = np.meshgrid(np.arange(H), np.arange(Wd), indexing="ij")
+    a = atominfo.astype(np.float64)
+    want = sum(a[n, 3] / np.sqrt((0.1 * xx - a[n, 0]) ** 2 + (0.1 * yy - a[n, 1]) ** 2 + a[n, 2]) for n in range(64))
+    part3 = (xx % 128) >= 96
+    np.testing.assert_allclose(last[part3], want[part3], rtol=1e-4, atol=1e-5)
+    assert np.all(last[~part3] == 0)
+    # past the grid the positions come round again and add a second time
+    twice = oracle.cp(atominfo, g0, start=0, end=48, parts=4)
+    assert np.array_equal(twice, oracle.cp(atominfo, whole, parts=4))
 
 
 # ------------------------------------------------------------------ conv helpers
