@@ -346,6 +346,14 @@ TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
  * share alone" `limit` times in a row is launched alone for the rest of the run (Aker mode only).
  * Default 3; 0 restores the reference's behaviour. */
 TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int limit);
+/* No counterpart in the reference (it takes tiles x block_ratio(K) from kinfo,
+ * src/TaskManager.cu:593-600): with on != 0 an Aker-mode run first times, for every mixable LC
+ * kernel, its fused launch with be_total / 64, / 32, ... best-effort blocks and then co-locates
+ * the count that earned most among those that kept the fused launch within (1 + max_stretch) of
+ * the kernel alone (none: the kernel runs alone).  For layers that leave most CUs without a tile.
+ * tacker_task_manager_calibrated_blocks copies the counts of the last run (one per LC kernel). */
+TK_API int tacker_task_manager_set_calibration(tacker_task_manager_t tm, int on, float max_stretch);
+TK_API int tacker_task_manager_calibrated_blocks(tacker_task_manager_t tm, int *out, int cap);
 /* LC kernels barred from fusion at the end of the last run */
 TK_API int tacker_task_manager_fusion_disabled(tacker_task_manager_t tm);
 /* "[Mix] BE task1 + task2 took ..." (src/TaskManager.cu:693): average time of the fused launch of

@@ -106,6 +106,8 @@ def _declare(lib):
     lib.tacker_task_manager_latencies.argtypes = [vp, i, C.POINTER(f), i]
     lib.tacker_task_manager_set_fusion_strikes.argtypes = [vp, i]
     lib.tacker_task_manager_fusion_disabled.argtypes = [vp]
+    lib.tacker_task_manager_set_calibration.argtypes = [vp, i, f]
+    lib.tacker_task_manager_calibrated_blocks.argtypes = [vp, vp, i]
     lib.tacker_task_manager_be_mix_ms.argtypes = [vp]
     lib.tacker_task_manager_be_mix_ms.restype = f
     lib.tacker_qos_block_ratio.argtypes = [cp, i]
@@ -607,6 +609,14 @@ class TaskManager:
 
     def set_fusion_strikes(self, limit):
         check(self.l.tacker_task_manager_set_fusion_strikes(self.h, limit), "set_fusion_strikes")
+
+    def set_calibration(self, on=True, max_stretch=0.10):
+        check(self.l.tacker_task_manager_set_calibration(self.h, 1 if on else 0, max_stretch), "set_calibration")
+
+    def calibrated_blocks(self):
+        buf = (C.c_int * 4096)()
+        n = self.l.tacker_task_manager_calibrated_blocks(self.h, buf, 4096)
+        return list(buf[:max(n, 0)])
 
     def fusion_disabled(self):
         return self.l.tacker_task_manager_fusion_disabled(self.h)

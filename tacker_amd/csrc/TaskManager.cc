@@ -218,6 +218,62 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         report.be2_solo_ms = watch.stop(stream);
     }
 
+    // launch of LC kernel idx fused with BE blocks [from, to) of be_kernel1
+    auto launch_mixed = [&](Kernel *lc_kernel, int from, int to) {
+        std::vector<int> args = lc_kernel->getArgs();
+        std::vector<int> mnk = lc_kernel->mixable == 1 ? args : get_mnk_from_cudnn_args(args);
+        if (auto *layer = dynamic_cast<LcGemmKernel *>(lc_kernel))
+            layer->executeMixed(be_kernel1, from, to, stream);   // the layer's own operands
+        else if (lc_kernel->mixable == 1) mixcublasSgemm(mnk, be_kernel1, from, to, stream);
+        else mixcudnnConvolutionForward(args, be_kernel1, from, to, stream);
+    };
+
+    // optional: measured block count per LC kernel instead of the kinfo table
+    calibrated_blocks.clear();
+    if (calibrate_blocks && mode == ExecutionMode::Aker && be_total > 0) {
+        calibrated_blocks.assign(nk, 0);
+        std::vector<float> best_earned(nk, 0.0f);
+        std::vector<bool> over(nk, false);   // a smaller count already stretched this kernel too far
+        const int first = be_kernel1->gptbParams.ptb_start_block_pos;
+        for (int divisor = 64; divisor >= 1; divisor /= 2) {
+            const int n = std::max(1, be_total / divisor);
+            std::vector<float> fused_ms(nk, 0.0f);
+            const int timed = 3;
+            for (int pass = -1; pass < timed; ++pass) {   // pass -1 warms up
+                lc_task->initExecution();
+                for (size_t idx = 0; idx < nk; ++idx) {
+                    Kernel *lc_kernel = lc_task->kernels[idx];
+                    if (lc_kernel->mixable == 0 || over[idx]) {
+                        lc_kernel->execute(stream);
+                        continue;
+                    }
+                    watch.start(stream);
+                    launch_mixed(lc_kernel, first, std::min(first + n, be_total));
+                    const float ms = watch.stop(stream);
+                    if (pass >= 0) fused_ms[idx] += ms / timed;
+                }
+            }
+            for (size_t idx = 0; idx < nk; ++idx) {
+                if (lc_task->kernels[idx]->mixable == 0 || over[idx]) continue;
+                const float alone = lc_kernel_time_vec[idx];
+                if (fused_ms[idx] > (1.0f + calibrate_max_stretch) * alone) {
+                    over[idx] = true;
+                    continue;
+                }
+                const float earned = alone + report.be1_solo_ms * n / be_total - fused_ms[idx];
+                if (earned > best_earned[idx]) {
+                    best_earned[idx] = earned;
+                    calibrated_blocks[idx] = n;
+                }
+            }
+        }
+        if (verbose)
+            for (size_t idx = 0; idx < nk; ++idx)
+                if (lc_task->kernels[idx]->mixable != 0)
+                    printf("[CAL] %s: %d blocks, earns %f ms\n", lc_task->kernels[idx]->kernelName.c_str(),
+                           calibrated_blocks[idx], best_earned[idx]);
+    }
+
     // co-located queries: a cursor walks the BE kernel's blocks across launches
     int be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;
     float qos_headroom = policy.qos_budget_ms;
@@ -242,20 +298,23 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             watch.start(stream);
             const bool barred = mode == ExecutionMode::Aker && fusion_strikes_limit > 0 &&
                                 strikes[idx] >= fusion_strikes_limit;
-            if (policy.mustRunSolo(qos_headroom, lc_headroom_vec[idx]) || lc_kernel->mixable == 0 || barred) {
+            const bool calibrated = !calibrated_blocks.empty();
+            if (policy.mustRunSolo(qos_headroom, lc_headroom_vec[idx]) || lc_kernel->mixable == 0 || barred ||
+                (calibrated && calibrated_blocks[idx] == 0)) {
                 lc_kernel->execute(stream);
             } else {
-                std::vector<int> args = lc_kernel->getArgs();
-                std::vector<int> mnk = lc_kernel->mixable == 1 ? args : get_mnk_from_cudnn_args(args);
-                if (auto *layer = dynamic_cast<LcGemmKernel *>(lc_kernel)) mnk = layer->gemmDims();
-                const std::vector<int> MNKD = getTZGEMMGridDim(mnk[0], mnk[1], mnk[2]);
-                cd_block_num = QosPolicy::coLocatedBlocks(mode, be_task1_name, MNKD[3], MNKD[2], be_total);
+                if (calibrated) {
+                    cd_block_num = calibrated_blocks[idx];
+                } else {
+                    std::vector<int> args = lc_kernel->getArgs();
+                    std::vector<int> mnk = lc_kernel->mixable == 1 ? args : get_mnk_from_cudnn_args(args);
+                    if (auto *layer = dynamic_cast<LcGemmKernel *>(lc_kernel)) mnk = layer->gemmDims();
+                    const std::vector<int> MNKD = getTZGEMMGridDim(mnk[0], mnk[1], mnk[2]);
+                    cd_block_num = QosPolicy::coLocatedBlocks(mode, be_task1_name, MNKD[3], MNKD[2], be_total);
+                }
                 const int end = std::min(be_cursor + cd_block_num, be_total);
                 cd_block_num = end - be_cursor;
-                if (auto *layer = dynamic_cast<LcGemmKernel *>(lc_kernel))
-                    layer->executeMixed(be_kernel1, be_cursor, end, stream);   // the layer's own operands
-                else if (lc_kernel->mixable == 1) mixcublasSgemm(mnk, be_kernel1, be_cursor, end, stream);
-                else mixcudnnConvolutionForward(args, be_kernel1, be_cursor, end, stream);
+                launch_mixed(lc_kernel, be_cursor, end);
                 be_cursor = end;
                 if (be_cursor >= be_total) {   // one pass over the BE kernel done
                     be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;

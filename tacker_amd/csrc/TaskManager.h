@@ -92,6 +92,17 @@ public:
     // stop (the reference's behaviour).
     int fusion_strikes_limit = 3;
     int fusion_retry_period = 64;   // queries between two chances for a barred kernel (0 = never again)
+    // Not in the reference: before the co-located queries, measure for every mixable LC kernel
+    // how many best-effort blocks its fused launch should carry (Aker mode), instead of taking
+    // tiles x block_ratio(K) from kinfo.  That table is measured on GEMMs that fill the GPU; a
+    // batch-1 layer with a few dozen tiles leaves most CUs free, and what those CUs can take
+    // depends on the layer and on the best-effort kernel.  The fused launch is timed with
+    // be_total / 64, / 32, ... blocks and the count with the largest earned time
+    // (lc alone + share of be alone - fused) is kept among those whose fused launch stays
+    // within (1 + calibrate_max_stretch) of the LC kernel alone; none -> the kernel runs alone.
+    bool calibrate_blocks = false;
+    float calibrate_max_stretch = 0.10f;
+    std::vector<int> calibrated_blocks;   // per LC kernel, filled by the last calibrated run
     TaskManagerReport report;
 
 private:

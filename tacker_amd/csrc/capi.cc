@@ -820,6 +820,24 @@ int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t h, int limit)
     return TK_SUCCESS;
 }
 
+int tacker_task_manager_set_calibration(tacker_task_manager_t h, int on, float max_stretch)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || max_stretch < 0.0f) return fail(TK_ERROR_INVALID_VALUE, "bad task manager or stretch");
+    tm->calibrate_blocks = on != 0;
+    tm->calibrate_max_stretch = max_stretch;
+    return TK_SUCCESS;
+}
+
+int tacker_task_manager_calibrated_blocks(tacker_task_manager_t h, int *out, int cap)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || !out) return -1;
+    const int n = std::min((int)tm->calibrated_blocks.size(), cap);
+    memcpy(out, tm->calibrated_blocks.data(), (size_t)n * sizeof(int));
+    return n;
+}
+
 int tacker_task_manager_fusion_disabled(tacker_task_manager_t h)
 {
     TaskManager *tm = static_cast<TaskManager *>(h);

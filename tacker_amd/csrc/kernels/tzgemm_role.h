@@ -518,4 +518,16 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A, cons
         tzgemm_role_tiles<STAGES>(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds, sync);
 }
 
+// Workgroups of a launch of role_blocks that can hold a tile of this GEMM (the first ones, in
+// both forms).  A fused kernel uses it to keep best-effort blocks off those workgroups when the
+// GEMM leaves most of the chip without a tile.
+__device__ __forceinline__ int tz_busy_workgroups(int M, int N, int K, int role_blocks, int tile_start,
+                                                  int tile_end)
+{
+    if (tile_start >= tile_end) return 0;
+    const int units = tz_use_ksplit(M, N, K) ? tile_end - tile_start
+                                             : (M / TZ_MACRO_TILE) * (N / TZ_MACRO_TILE);
+    return min(units, role_blocks);
+}
+
 }  // namespace tk

@@ -77,12 +77,11 @@ def generate_wave_split(be, be_threads, tz_first=True):
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="(int)blockIdx.x",
                                              blocks=f"{p_tz}ptb_iter_block_step",
                                              tid=f"(int)threadIdx.x - {tz_lo}", stages="TZ_STAGES")
-    be_call = ROLES[be]["call"].format(p=p_be, block="(int)blockIdx.x",
-                                       blocks=f"{p_be}ptb_iter_block_step",
+    be_call = ROLES[be]["call"].format(p=p_be, block="be_block", blocks="be_blocks",
                                        tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads)
     tz_cond = (f"threadIdx.x < {tz_threads}" if tz_first else f"threadIdx.x >= {be_threads}")
     name = mix_kernel_name(be, variant)
-    unused = _void_unused(sig_be + sig_tz, tz_call + be_call)
+    unused = _void_unused(sig_be + sig_tz, tz_call + be_call + f"{p_be}ptb_iter_block_step")
     text = f"""// {be}-tzgemm  wave split  {tz_threads} tzgemm threads + {be_threads} {be} threads per workgroup
 extern "C" __global__ __launch_bounds__({total}) void {name}(
     {_params_text(sig_be, sig_tz)})
@@ -101,7 +100,18 @@ extern "C" __global__ __launch_bounds__({total}) void {name}(
         tk::RoleSpinSync sync(tz_arrivals, {tz_threads // 64}, &tk_spin_fail);
         {tz_call}
     }} else {{
-        {be_call}
+        // A GEMM that leaves at least half of the workgroups without a tile: the {be} blocks go
+        // to those workgroups only, where nothing competes with them, and the workgroups that
+        // hold the latency-critical tiles run them undisturbed.
+        const int launched = {p_be}ptb_iter_block_step;
+        const int tz_busy = tk::tz_busy_workgroups({p_tz}NORMAL_M, {p_tz}NORMAL_N, {p_tz}NORMAL_K, launched,
+                                                   {p_tz}ptb_start_block_pos, {p_tz}ptb_end_block_pos);
+        const bool apart = 2 * tz_busy <= launched;
+        const int be_block = apart ? (int)blockIdx.x - tz_busy : (int)blockIdx.x;
+        const int be_blocks = apart ? launched - tz_busy : launched;
+        if (be_block >= 0) {{
+            {be_call}
+        }}
     }}
 }}
 """

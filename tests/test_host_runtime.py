@@ -448,6 +448,50 @@ def test_task_manager_stops_fusing_kernels_whose_fusion_keeps_losing(fake, small
     tm.close()
 
 
+def test_task_manager_calibrates_block_counts_per_kernel(fake, small_vgg):
+    n = len(small_vgg.kernels())
+    tm = ta.TaskManager(small_vgg, "stencil", None, library=fake)
+    tm.configure(warmup=1, profile=2, verbose=0, qos_budget_ms=1e6, guard_ms=0.0, queries=2)
+    tm.set_calibration(True, 0.10)
+    # every timed region takes 10 us, fused or not: a fused launch never stretches its kernel, and what it
+    # earns (share of the best-effort kernel's 10 us) grows with the block count -> the whole kernel each time
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.01)
+    rep = tm.run("aker", raw_stream=None, second_stage=False)
+    blocks = tm.calibrated_blocks()
+    mixable = [i for i, k in enumerate(small_vgg.kernels()) if k["mixable"]]
+    assert len(blocks) == n and len(mixable) == 16
+    assert all(blocks[i] == 1024 for i in mixable) and all(blocks[i] == 0 for i in range(n) if i not in mixable)
+    assert rep["mix_times"] == 16 and rep["be_blocks_executed"] == 16 * 1024
+    # 7 block counts (1/64 ... 1) x (1 warm-up + 3 timed) passes of 16 fused launches, then 2 queries
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
+    assert len(fused) == 7 * 4 * 16 + 2 * 16
+    ends = sorted({as_int(l["args"][15]) for l in fused[:7 * 4 * 16]})           # stencil ptb_end of the sweeps
+    assert ends == [16, 32, 64, 128, 256, 512, 1024]
+    # LC kernels alone take 10 us, every fused launch 12 us: 20 % over a 10 % allowance -> nothing is co-located
+    cheap = [0.01] * (n * 2 + 1)
+    arr = (C.c_float * len(cheap))(*cheap)
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.012)
+    fake.tk_fake_push_event_ms(arr, len(cheap))
+    rep = tm.run("aker", raw_stream=None, second_stage=False)
+    assert tm.calibrated_blocks() == [0] * n and rep["mix_times"] == 0 and rep["be_blocks_executed"] == 0
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
+    assert len(fused) == 4 * 16                                                  # only the first sweep (1/64)
+    # 5 % over: allowed, and it pays from 1/16 of the kernel up (10 us * n/N > 0.5 us) -> again the whole kernel
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.0105)
+    fake.tk_fake_push_event_ms(arr, len(cheap))
+    tm.run("aker", raw_stream=None, second_stage=False)
+    assert all(tm.calibrated_blocks()[i] == 1024 for i in mixable)
+    tm.set_calibration(False, 0.10)                                              # back to the kinfo table
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.01)
+    tm.run("aker", raw_stream=None, second_stage=False)
+    assert tm.calibrated_blocks() == []
+    tm.close()
+
+
 def test_task_manager_falls_back_to_solo_when_headroom_is_short(fake, small_vgg):
     fake.tk_fake_set_event_ms(0.01)
     n = len(small_vgg.kernels())
