@@ -99,10 +99,12 @@ protected:
 
 class ConvKernel : public GemmLayer {
 public:
-    ConvKernel(int id, const std::string &name, const float *act, int H, int W, int C, int c_stride,
-               int Cout, void *A, const void *Wt, float *out)
-        : GemmLayer(id, name, pad128(H * W), pad128(Cout), pad128(9 * C), A, Wt, out), act_(act), H_(H),
-          W_(W), C_(C), cs_(c_stride), Cout_(Cout), A_(A)
+    // act_bias != nullptr: act is the raw output of the previous convolution; its bias and
+    // ReLU are applied while the operand is gathered
+    ConvKernel(int id, const std::string &name, const float *act, const float *act_bias, int H, int W, int C,
+               int c_stride, int Cout, void *A, const void *Wt, float *out)
+        : GemmLayer(id, name, pad128(H * W), pad128(Cout), pad128(9 * C), A, Wt, out), act_(act),
+          act_bias_(act_bias), H_(H), W_(W), C_(C), cs_(c_stride), Cout_(Cout), A_(A)
     {
         this->mixable = 2;
     }
@@ -113,12 +115,14 @@ protected:
     void before(cudaStream_t stream) override
     {
         int KH = 3, KW = 3, pad = 1, stride = 1, Ho = H_, Wo = W_, Kp = K_;
-        void *args[] = {&act_, &H_, &W_, &C_, &cs_, &KH, &KW, &pad, &stride, &Ho, &Wo, &A_, &Kp};
+        int relu = 1;
+        void *args[] = {&act_, &H_, &W_, &C_, &cs_, &KH, &KW, &pad, &stride, &Ho, &Wo, &A_, &Kp, &act_bias_, &relu};
         launch1d("im2col_nhwc_f16", (long)Ho * Wo * Kp, args, stream);
     }
 
 private:
     const float *act_;
+    const float *act_bias_;
     int H_, W_, C_, cs_, Cout_;
     void *A_;
 };
@@ -169,32 +173,22 @@ protected:
     long work_;
 };
 
-class BiasReluKernel : public SimpleKernel {
-public:
-    BiasReluKernel(int id, const std::string &name, float *y, const float *bias, int M, int ld)
-        : SimpleKernel(id, name, "bias_relu_rows", (long)M * ld), y_(y), b_(bias), M_(M), ld_(ld)
-    {
-        argStore = {&y_, &b_, &M_, &ld_, &relu_};
-    }
-
-private:
-    float *y_;
-    const float *b_;
-    int M_, ld_, relu_ = 1;
-};
-
 class PoolKernel : public SimpleKernel {
 public:
-    PoolKernel(int id, const std::string &name, const float *in, int H, int W, int ld, float *out)
-        : SimpleKernel(id, name, "maxpool2x2_nhwc", (long)(H / 2) * (W / 2) * ld), in_(in), H_(H), W_(W),
-          ld_(ld), out_(out)
+    // in_bias != nullptr: in is the raw output of the previous convolution; its bias and ReLU
+    // are applied to the pooled value
+    PoolKernel(int id, const std::string &name, const float *in, const float *in_bias, int H, int W, int ld,
+               float *out)
+        : SimpleKernel(id, name, "maxpool2x2_nhwc", (long)(H / 2) * (W / 2) * ld), in_(in), bias_(in_bias),
+          H_(H), W_(W), ld_(ld), out_(out)
     {
-        argStore = {&in_, &H_, &W_, &ld_, &out_};
+        argStore = {&in_, &H_, &W_, &ld_, &out_, &bias_, &relu_};
     }
 
 private:
     const float *in_;
-    int H_, W_, ld_;
+    const float *bias_;
+    int H_, W_, ld_, relu_ = 1;
     float *out_;
 };
 
@@ -240,15 +234,19 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
     TK_SAFE_CALL(tkMemset(Abuf, 0, maxA * 2));
     fl.push_back(Abuf);
 
+    // A convolution leaves 1.1 * A * B^T in its output buffer; bias and ReLU are applied by
+    // whatever reads that buffer next (the next layer's operand gather, or the pooling).
     const float *act = impl->input;
+    const float *act_bias = nullptr;   // bias the reader of act still has to apply
     int id = 100;
     const int plan[] = {64, 64, -1, 128, 128, -1, 256, 256, 256, -1, 512, 512, 512, -1, 512, 512, 512, -1};
     int block = 1, layer = 1;
     for (int p : plan) {
         if (p < 0) {
             float *out = devAlloc(fl, (size_t)(H / 2) * (W / 2) * ld);
-            addKernel(new PoolKernel(id++, "MaxPool_" + std::to_string(block), act, H, W, ld, out));
+            addKernel(new PoolKernel(id++, "MaxPool_" + std::to_string(block), act, act_bias, H, W, ld, out));
             act = out;
+            act_bias = nullptr;
             H /= 2;
             W /= 2;
             block++;
@@ -260,10 +258,10 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
         void *Wt = randomHalfMatrix(fl, rng, Cout, 9 * C, Np, Kp, std::sqrt(2.0f / (9 * C)));
         float *bias = randomBias(fl, rng, Cout, Np);
         float *out = devAlloc(fl, (size_t)pad128(H * W) * Np);
-        addKernel(new ConvKernel(id++, "Convolution_" + name, act, H, W, C, ld, Cout, Abuf, Wt, out));
-        addKernel(new BiasReluKernel(id++, "BiasRelu_" + name, out, bias, H * W, Np));
+        addKernel(new ConvKernel(id++, "Convolution_" + name, act, act_bias, H, W, C, ld, Cout, Abuf, Wt, out));
         impl->convOut.push_back(Act{out, H, W, Cout, Np, Wt, bias, Np, Kp});
         act = out;
+        act_bias = bias;
         C = Cout;
         ld = Np;
     }

@@ -12,9 +12,12 @@
 // A[m][k] for m = (h*W + w), k = (kh*KW + kw)*C + c; zero for padding taps and for
 // k in [KH*KW*C, K_pad).  Rows m >= H*W of A are never written (they stay zero).
 // act is [H][W][c_stride] with c < C used.  3x3/stride-1 style parameters general.
+// bias != nullptr: act is the raw output of the previous GEMM and its epilogue is applied
+// on the way in, v = act + bias[c], then max(v, 0) if relu -- the values a separate
+// bias/ReLU pass over act would have left there, without that pass.
 extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C, int c_stride,
                                            int KH, int KW, int pad, int stride, int Ho, int Wo,
-                                           _Float16 *A, int K_pad)
+                                           _Float16 *A, int K_pad, const float *bias, int relu)
 {
     typedef float f4 __attribute__((ext_vector_type(4)));
     typedef _Float16 h8 __attribute__((ext_vector_type(8)));
@@ -36,8 +39,19 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
                 const int h = ho * stride - pad + kh, w = wo * stride - pad + kw;
                 if (h >= 0 && h < H && w >= 0 && w < W) {
                     const float *src = act + ((size_t)h * W + w) * c_stride + c;
-                    const f4 lo = *reinterpret_cast<const f4 *>(src);
-                    const f4 hi = *reinterpret_cast<const f4 *>(src + 4);
+                    f4 lo = *reinterpret_cast<const f4 *>(src);
+                    f4 hi = *reinterpret_cast<const f4 *>(src + 4);
+                    if (bias) {
+                        lo += *reinterpret_cast<const f4 *>(bias + c);
+                        hi += *reinterpret_cast<const f4 *>(bias + c + 4);
+                        if (relu) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                lo[e] = lo[e] < 0.0f ? 0.0f : lo[e];
+                                hi[e] = hi[e] < 0.0f ? 0.0f : hi[e];
+                            }
+                        }
+                    }
                     out = h8{(_Float16)lo.x, (_Float16)lo.y, (_Float16)lo.z, (_Float16)lo.w,
                              (_Float16)hi.x, (_Float16)hi.y, (_Float16)hi.z, (_Float16)hi.w};
                 }
@@ -58,7 +72,13 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
             const int kw = tap % KW, kh = tap / KW;
             const int wo = (int)(m % Wo), ho = (int)(m / Wo);
             const int h = ho * stride - pad + kh, w = wo * stride - pad + kw;
-            if (h >= 0 && h < H && w >= 0 && w < W) v = act[((long)h * W + w) * c_stride + c];
+            if (h >= 0 && h < H && w >= 0 && w < W) {
+                v = act[((long)h * W + w) * c_stride + c];
+                if (bias) {
+                    v += bias[c];
+                    if (relu && v < 0.0f) v = 0.0f;
+                }
+            }
         }
         A[i] = (_Float16)v;
     }
@@ -75,8 +95,11 @@ extern "C" __global__ void bias_relu_rows(float *y, const float *bias, int M, in
     }
 }
 
-// 2x2 / stride 2 max pooling, NHWC with channel stride ld
-extern "C" __global__ void maxpool2x2_nhwc(const float *in, int H, int W, int ld, float *out)
+// 2x2 / stride 2 max pooling, NHWC with channel stride ld.  bias != nullptr: in is the raw
+// output of the previous GEMM; out = max(in) + bias[c], then max(., 0) if relu, which is what
+// pooling the biased, rectified values gives (x -> fl(x + b) and ReLU are non-decreasing).
+extern "C" __global__ void maxpool2x2_nhwc(const float *in, int H, int W, int ld, float *out,
+                                           const float *bias, int relu)
 {
     const int Ho = H / 2, Wo = W / 2;
     const long total = (long)Ho * Wo * ld;
@@ -87,7 +110,12 @@ extern "C" __global__ void maxpool2x2_nhwc(const float *in, int H, int W, int ld
         const int wo = (int)(p % Wo), ho = (int)(p / Wo);
         const float *src = in + ((long)(2 * ho) * W + 2 * wo) * ld + c;
         const float a = src[0], b = src[ld], d = src[(long)W * ld], e = src[(long)W * ld + ld];
-        out[i] = fmaxf(fmaxf(a, b), fmaxf(d, e));
+        float v = fmaxf(fmaxf(a, b), fmaxf(d, e));
+        if (bias) {
+            v += bias[c];
+            if (relu && v < 0.0f) v = 0.0f;
+        }
+        out[i] = v;
     }
 }
 

@@ -61,6 +61,8 @@ def test_vgg16_layers_match_direct_convolution():
     for idx in range(4):                      # conv1_1, conv1_2, [pool], conv2_1, conv2_2
         w, b = task.conv_params(idx)
         got, Cout = read_act(task, idx)
+        # the buffer holds the raw GEMM output; the layer that reads it adds the bias and rectifies
+        got = np.maximum(got + b[None, None, :got.shape[2]], np.float32(0))
         if idx == 2:                          # a 2x2 max pool sits between conv1_2 and conv2_1
             H, W = prev.shape[:2]
             prev = prev.reshape(H // 2, 2, W // 2, 2, -1).max(axis=(1, 3))

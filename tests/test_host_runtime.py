@@ -379,7 +379,16 @@ def test_vgg16_solo_pass_launches_every_layer(fake, small_vgg):
     small_vgg.execute(raw_stream=None)
     keys = [l["key"] for l in launches(fake)]
     assert keys.count("gptb_tzgemm") == 16 and keys.count("im2col_nhwc_f16") == 13
-    assert keys.count("maxpool2x2_nhwc") == 5 and keys.count("bias_relu_rows") == 13 and keys.count("pack_fc_input") == 3
+    assert keys.count("maxpool2x2_nhwc") == 5 and keys.count("pack_fc_input") == 3
+    # no separate bias/ReLU pass: each convolution's bias travels to whatever reads its output next
+    assert keys.count("bias_relu_rows") == 0
+    gathers = [l for l in launches(fake) if l["key"] == "im2col_nhwc_f16"]
+    pools = [l for l in launches(fake) if l["key"] == "maxpool2x2_nhwc"]
+    assert as_ptr(gathers[0]["args"][13]) == 0                       # conv1_1 reads the image
+    has_bias = [as_ptr(g["args"][13]) != 0 for g in gathers]
+    # conv after conv carries the bias; conv after a pool does not (the pool applied it)
+    assert has_bias == [False, True, False, True, False, True, True, False, True, True, False, True, True]
+    assert all(as_ptr(p["args"][5]) != 0 and as_int(p["args"][6]) == 1 for p in pools)
 
 
 def run_manager(fake, task, durations=None, **cfg):
