@@ -25,28 +25,6 @@ __constant__ mriq_kValues ck[MRIQ_MAX_K];
 
 namespace tk {
 
-__device__ __forceinline__ void mriq_voxel(int numK, const float *__restrict__ x,
-                                           const float *__restrict__ y, const float *__restrict__ z,
-                                           float *__restrict__ Qr, float *__restrict__ Qi, int xIndex)
-{
-    const float sX = x[xIndex];
-    const float sY = y[xIndex];
-    const float sZ = z[xIndex];
-    float sQr = Qr[xIndex];
-    float sQi = Qi[xIndex];
-#pragma unroll 8
-    for (int kIndex = 0; kIndex < numK; ++kIndex) {
-        const float phase = ck[kIndex].Kx * sX + ck[kIndex].Ky * sY + ck[kIndex].Kz * sZ;   // revolutions
-        const float turn = __builtin_amdgcn_fractf(phase);
-        const float s = __builtin_amdgcn_sinf(turn);
-        const float c = __builtin_amdgcn_cosf(turn);
-        sQr += ck[kIndex].PhiMag * c;
-        sQi += ck[kIndex].PhiMag * s;
-    }
-    Qr[xIndex] = sQr;
-    Qi[xIndex] = sQi;
-}
-
 // V voxels per thread at once, k records [k_begin, k_end).  The k loop is a chain of
 // dependent operations per voxel (dot product, fract, sin/cos, accumulate) and a fused
 // launch leaves the role at most two waves per SIMD, so the independent work that hides
@@ -68,15 +46,47 @@ __device__ __forceinline__ void mriq_voxels(int k_begin, int k_end, const float 
         sQr[v] = Qr[i];
         sQi[v] = Qi[i];
     }
-    // unrolled so the scalar loads of 8 records are issued together: one record per
-    // iteration would put a scalar-cache round trip on every step of the chain
-#pragma unroll 8
-    for (int kIndex = k_begin; kIndex < k_end; ++kIndex) {
+    // U records at a time, written stage by stage (all phases, then all sines and cosines,
+    // then the accumulation in ascending k): the U * V chains are independent until the last
+    // stage, and the order of the source is already the interleaved one -- the compiler's
+    // scheduler does not have to find it (for one of the instances in a fused kernel it did
+    // not, and that loop ran one dependent chain at a time).  The scalar loads of the U
+    // records are issued together: one record per iteration would put a scalar-cache round
+    // trip on every step.
+    constexpr int U = V >= 4 ? 4 : 8;
+    int kIndex = k_begin;
+    for (; kIndex + U <= k_end; kIndex += U) {
+        mriq_kValues k[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) k[u] = ck[kIndex + u];
+        float c[U][V], s[U][V];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                const float phase = k[u].Kx * sX[v] + k[u].Ky * sY[v] + k[u].Kz * sZ[v];   // revolutions
+                c[u][v] = __builtin_amdgcn_fractf(phase);
+            }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                s[u][v] = __builtin_amdgcn_sinf(c[u][v]);
+                c[u][v] = __builtin_amdgcn_cosf(c[u][v]);
+            }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int v = 0; v < V; ++v) {
+                sQr[v] += k[u].PhiMag * c[u][v];
+                sQi[v] += k[u].PhiMag * s[u][v];
+            }
+    }
+    for (; kIndex < k_end; ++kIndex) {
         const mriq_kValues k = ck[kIndex];
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-            const float phase = k.Kx * sX[v] + k.Ky * sY[v] + k.Kz * sZ[v];   // revolutions
-            const float turn = __builtin_amdgcn_fractf(phase);
+            const float turn = __builtin_amdgcn_fractf(k.Kx * sX[v] + k.Ky * sY[v] + k.Kz * sZ[v]);
             sQr[v] += k.PhiMag * __builtin_amdgcn_cosf(turn);
             sQi[v] += k.PhiMag * __builtin_amdgcn_sinf(turn);
         }
@@ -86,6 +96,15 @@ __device__ __forceinline__ void mriq_voxels(int k_begin, int k_end, const float 
         Qr[xIndex[v]] = sQr[v];
         Qi[xIndex[v]] = sQi[v];
     }
+}
+
+// the natural kernel's thread: one voxel, every record
+__device__ __forceinline__ void mriq_voxel(int numK, const float *__restrict__ x,
+                                           const float *__restrict__ y, const float *__restrict__ z,
+                                           float *__restrict__ Qr, float *__restrict__ Qi, int xIndex)
+{
+    const int one[1] = {xIndex};
+    mriq_voxels<1>(0, numK, x, y, z, Qr, Qi, one);
 }
 
 // One phase of a launch: voxel blocks [block_lo, block_hi) each take records
