@@ -1,28 +1,30 @@
 #include "Recorder.h"
 
-#include <fstream>
-#include <iostream>
+#include <cstdio>
+#include <sstream>
 
 void Recorder::text(const std::string &filename)
 {
-    std::ofstream file(filename);
-    if (!file.is_open()) {
-        std::cerr << "cannot open file: " << filename << std::endl;
+    // numbers print the way the reference's stream insertion prints a float (%g, 6 digits)
+    std::ostringstream table;
+    for (const auto &entry : tasks_) {
+        const TaskTimes &task = entry.second;
+        std::ostringstream header;
+        header << "taskID: " << entry.first << ", taskName: " << task.name << "\n";
+        std::fputs(header.str().c_str(), stdout);
+        table << header.str();
+        float total = 0.0f;
+        for (const KernelTime &k : task.kernels) {
+            table << "    kernelID: " << k.id << ", kernelName: " << k.name << ", execTime: " << k.ms << "ms\n";
+            total += k.ms;
+        }
+        table << "    task running time: " << total << "ms\n\n";
+    }
+    FILE *file = std::fopen(filename.c_str(), "w");
+    if (!file) {
+        std::fprintf(stderr, "cannot open file: %s\n", filename.c_str());
         return;
     }
-    for (auto &task_pair : task_time_map) {
-        const int taskId = task_pair.first;
-        auto &times = task_pair.second;
-        auto &kernelIds = task_kernel_map[taskId];
-        auto &taskName = task_name_map[taskId];
-        std::cout << "taskID: " << taskId << ", taskName: " << taskName << "\n";
-        file << "taskID: " << taskId << ", taskName: " << taskName << "\n";
-        float totalTaskTime = 0.0f;
-        for (size_t i = 0; i < times.size(); ++i) {
-            totalTaskTime += times[i];
-            file << "    kernelID: " << kernelIds[i] << ", kernelName: " << task_kernel_name_vec[taskId][i]
-                 << ", execTime: " << times[i] << "ms\n";
-        }
-        file << "    task running time: " << totalTaskTime << "ms\n\n";
-    }
+    std::fputs(table.str().c_str(), file);
+    std::fclose(file);
 }

@@ -209,13 +209,16 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         if (be_task2) be_task2->execute(stream);
     }
     TK_SAFE_CALL(tkDeviceSynchronize());
+    // mean of a few back-to-back launches: one launch alone right after a synchronisation is
+    // timed with the start-up of the queue in it, and this figure prices every co-located block
+    const int be_samples = 10;
     watch.start(stream);
-    be_task1->execute(stream);
-    report.be1_solo_ms = watch.stop(stream);
+    for (int i = 0; i < be_samples; ++i) be_task1->execute(stream);
+    report.be1_solo_ms = watch.stop(stream) / be_samples;
     if (be_task2) {
         watch.start(stream);
-        be_task2->execute(stream);
-        report.be2_solo_ms = watch.stop(stream);
+        for (int i = 0; i < be_samples; ++i) be_task2->execute(stream);
+        report.be2_solo_ms = watch.stop(stream) / be_samples;
     }
 
     // launch of LC kernel idx fused with BE blocks [from, to) of be_kernel1
@@ -362,13 +365,9 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             MixKernel *be_mix = createMixKernel(mix_be_name);
             for (int i = 0; i < 5; ++i) be_mix->execute(stream);
             TK_SAFE_CALL(tkDeviceSynchronize());
-            float mix_be_time = 0.0f;
-            for (int i = 0; i < 10; ++i) {
-                watch.start(stream);
-                be_mix->execute(stream);
-                mix_be_time += watch.stop(stream);
-            }
-            mix_be_time /= 10;
+            watch.start(stream);   // timed the way the two kernels alone were
+            for (int i = 0; i < be_samples; ++i) be_mix->execute(stream);
+            const float mix_be_time = watch.stop(stream) / be_samples;
             report.be_mix_ms = mix_be_time;
             if (verbose) printf("[Mix] BE task1 + task2 took %f ms to execute.\n", mix_be_time);
             const float solo_sum = report.be1_solo_ms + report.be2_solo_ms;
