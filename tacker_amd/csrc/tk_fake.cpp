@@ -183,7 +183,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
                 add((std::string("tzgemm_") + be.first + v).c_str(),
                     cat(cat(*be.second, trailer(false)), cat(TZ, trailer(false))));
         // best-effort pairs, first < second alphabetically
-        static const char *pair_variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1"};
+        static const char *pair_variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1", "@ord_1_1", "@ord_1_2", "@ord_2_1"};
         for (auto &a : bes)
             for (auto &b : bes)
                 if (std::string(a.first) < std::string(b.first))

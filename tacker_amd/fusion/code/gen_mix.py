@@ -124,33 +124,52 @@ def be_pair_kernel_name(be1, be2, variant):
     return f"{be1}_{be2}_mix_{variant}"
 
 
-def generate_be_pair(be1, be2, wgs1, wgs2, threads=256):
+def generate_be_pair(be1, be2, wgs1, wgs2, threads=256, order=False):
     """Fused kernel of two vector kernels (no tzgemm): workgroup split wgs1 : wgs2.
 
-    Neither role uses LDS or a barrier, so workgroups of both kinds share a CU freely; the
-    split only fixes the proportion in which the launch's persistent workgroups serve the
-    two kernels (``createMixKernel`` pairs of the reference, src/Creator.cu:341-816).
-    Parameter order: be1's GPTB list, then be2's; be1 < be2 alphabetically, as the
-    reference names its pairs.
+    Neither role uses LDS or a barrier, so workgroups of both kinds share a CU freely
+    (``createMixKernel`` pairs of the reference, src/Creator.cu:341-816).  Parameter order:
+    be1's GPTB list, then be2's; be1 < be2 alphabetically, as the reference names its pairs.
+
+    ``wg_<a>_<b>``: the split fixes which kernel a workgroup serves -- a of every a + b
+    workgroups run be1's blocks, the others be2's.  When the shorter kernel ends, its
+    workgroups idle.
+
+    ``ord_<a>_<b>`` (order=True): every workgroup serves both kernels, each kernel's blocks
+    spread over all workgroups; the split only fixes the order -- a of every a + b workgroups
+    start with be1 and go on to be2, the others the other way round.  While both kinds are at
+    work a CU holds both kernels at once, and no workgroup ends before its share of both is
+    done.
     """
-    variant = f"wg_{wgs1}_{wgs2}"
+    variant = f"{'ord' if order else 'wg'}_{wgs1}_{wgs2}"
     p1, sig1 = signature(be1, 0)
     p2, sig2 = signature(be2, 1)
-    call1 = ROLES[be1]["call"].format(p=p1, block="sp.role_block", blocks="sp.role_blocks",
-                                      tid="(int)threadIdx.x", threads=threads)
-    call2 = ROLES[be2]["call"].format(p=p2, block="sp.role_block", blocks="sp.role_blocks",
-                                      tid="(int)threadIdx.x", threads=threads)
+    block, blocks = ("(int)blockIdx.x", "(int)gridDim.x") if order else ("sp.role_block", "sp.role_blocks")
+    call1 = ROLES[be1]["call"].format(p=p1, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads)
+    call2 = ROLES[be2]["call"].format(p=p2, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads)
     name = be_pair_kernel_name(be1, be2, variant)
-    text = f"""// {be1}-{be2}  workgroup split  {wgs1} {be1} : {wgs2} {be2} workgroups per group
+    if order:
+        title = f"order split  {wgs1} of {wgs1 + wgs2} workgroups start with {be1}, the others with {be2}"
+        body = f"""    for (int phase = 0; phase < 2; ++phase) {{
+        if ((sp.role ^ phase) == 0) {{
+            {call1}
+        }} else {{
+            {call2}
+        }}
+    }}"""
+    else:
+        title = f"workgroup split  {wgs1} {be1} : {wgs2} {be2} workgroups per group"
+        body = f"""    if (sp.role == 0) {{
+        {call1}
+    }} else {{
+        {call2}
+    }}"""
+    text = f"""// {be1}-{be2}  {title}
 extern "C" __global__ __launch_bounds__({threads}) void {name}(
     {_params_text(sig1, sig2)})
 {{
 {_void_unused(sig1 + sig2, call1 + call2)}    const tk::WgSplit sp = tk::wg_split((int)blockIdx.x, (int)gridDim.x, {wgs1}, {wgs2});
-    if (sp.role == 0) {{
-        {call1}
-    }} else {{
-        {call2}
-    }}
+{body}
 }}
 """
     meta = {"variant": variant, "symbol": name, "blocksize": threads, "group": wgs1 + wgs2,

@@ -117,7 +117,7 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
             assert f"void {sym}(" in text
             entry = kinfo[f"{a}_{b}@wg_{w1}_{w2}"]
             assert entry["group"] == w1 + w2 and entry["blocksize"] == 256
-        assert kinfo[f"{a}_{b}"]["variant"] in ("wg_1_1", "wg_1_2", "wg_2_1")
+        assert kinfo[f"{a}_{b}"]["variant"] in ("wg_1_1", "wg_1_2", "wg_2_1", "ord_1_1", "ord_1_2", "ord_2_1")
         assert f'insert("{a}_{b}", ' in files["mix_kernel/mix_kernels.inc"]
         # parameter order: the first kernel's list, then the second's
         assert text.index(f"{a}0_grid_dimension_x") < text.index(f"{b}1_grid_dimension_x")

@@ -465,7 +465,7 @@ def _small_be(name):
 
 @pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),
                                           ("lbm", "stencil"), ("mriq", "stencil")])
-@pytest.mark.parametrize("variant", [None, "wg_1_2", "wg_2_1"])
+@pytest.mark.parametrize("variant", [None, "wg_1_2", "wg_2_1", "ord_1_1", "ord_1_2"])
 def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
     ori1, n1, outs1 = _small_be(first)
     ori2, n2, outs2 = _small_be(second)
