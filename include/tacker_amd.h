@@ -189,6 +189,12 @@ TK_API int tacker_cp_initatoms(float *atoms_host, int count, unsigned volx, unsi
  * ori_cp bit for bit, and so does any set of ranges that tiles it. */
 #define TACKER_CP_X_PARTS 4
 TK_API int tacker_cp_blocks(int volx, int voly);
+/* No counterpart in the reference. The cp kernels evaluate 1.0f / sqrtf(r2) with a short
+ * instruction sequence where r2 is in [2^-20, 2^20) and with the general IEEE expansions
+ * elsewhere; this runs the short sequence on the GPU for every float with bit pattern in
+ * [lo_bits, hi_bits) and writes to *mismatches how many results differ from
+ * 1.0f / sqrtf(x) in any bit (0 for the whole range [0x35800000, 0x49800000)). */
+TK_API int tacker_cp_inv_sqrt_selftest(unsigned lo_bits, unsigned hi_bits, unsigned long long *mismatches);
 TK_API int tacker_ori_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly,
                          tkStream_t stream);
 TK_API int tacker_gptb_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly,

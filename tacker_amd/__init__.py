@@ -44,6 +44,7 @@ def _declare(lib):
     lib.tacker_mriq_set_kvalues.argtypes = [vp, i]
     lib.tacker_mriq_blocks.argtypes = [i, i]
     lib.tacker_cp_blocks.argtypes = [i, i]
+    lib.tacker_cp_inv_sqrt_selftest.argtypes = [C.c_uint, C.c_uint, C.POINTER(C.c_ulonglong)]
     lib.tacker_ori_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, vp]
     lib.tacker_gptb_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     lib.tacker_cp_set_atoms.argtypes = [vp, i, f]
@@ -272,6 +273,13 @@ def cp_set_atoms(atoms_np, zplane=0.0):
     import numpy as np
     a = np.ascontiguousarray(atoms_np, np.float32)
     check(lib().tacker_cp_set_atoms(a.ctypes.data, a.shape[0], zplane), "tacker_cp_set_atoms")
+
+
+def cp_inv_sqrt_selftest(lo_bits=0x35800000, hi_bits=0x49800000):
+    """floats in [lo_bits, hi_bits) for which the cp kernels' short 1/sqrt differs from 1.0f / sqrtf(x)"""
+    n = C.c_ulonglong(0)
+    check(lib().tacker_cp_inv_sqrt_selftest(lo_bits, hi_bits, C.byref(n)), "tacker_cp_inv_sqrt_selftest")
+    return n.value
 
 
 def cp_blocks(volx, voly):

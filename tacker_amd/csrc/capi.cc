@@ -313,6 +313,28 @@ int tacker_cp_blocks(int volx, int voly)
     return (volx / (BLOCKSIZEX * UNROLLX)) * (voly / BLOCKSIZEY) * CP_X_PARTS;
 }
 
+int tacker_cp_inv_sqrt_selftest(unsigned lo_bits, unsigned hi_bits, unsigned long long *mismatches)
+{
+    REQUIRE_INIT();
+    if (!mismatches || hi_bits < lo_bits) return fail(TK_ERROR_INVALID_VALUE, "cp_inv_sqrt_selftest: bad arguments");
+    auto it = fmap.find("cp_inv_sqrt_selftest");
+    if (it == fmap.end()) return fail(TK_ERROR_NOT_FOUND, "no kernel {cp_inv_sqrt_selftest}");
+    return guarded([&]() -> int {
+        unsigned long long *count = nullptr;
+        TK_SAFE_CALL(tkMalloc((void **)&count, sizeof(*count)));
+        TK_SAFE_CALL(tkMemset(count, 0, sizeof(*count)));
+        void *args[] = {&lo_bits, &hi_bits, &count};
+        const int rc = tkLaunchKernel(it->second, dim3(cuCount() * 8, 1, 1).raw(), dim3(256, 1, 1).raw(), args, 0,
+                                      nullptr);
+        if (rc == TK_SUCCESS) {
+            TK_SAFE_CALL(tkDeviceSynchronize());
+            TK_SAFE_CALL(tkMemcpy(mismatches, count, sizeof(*count), TK_MEMCPY_D2H));
+        }
+        tkErrCheck(tkFree(count));
+        return rc;
+    });
+}
+
 int tacker_ori_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, tkStream_t stream)
 {
     REQUIRE_INIT();

@@ -10,6 +10,17 @@
 //
 // gfx950: 16 lanes write 64 contiguous bytes and the 8 unrolled points of a row
 // tile a contiguous 512-byte span; atoms are read with scalar loads.
+//
+// 1.0f / sqrtf(r2) is two correctly rounded operations, and the general expansions of an IEEE
+// square root and an IEEE divide (scaling for denormals, fix-up of special values) are what the
+// kernel's time goes into: about 35 instructions per atom-point pair.  For r2 in
+// [2^-20, 2^20) a shorter sequence gives the same two roundings, bit for bit --
+//   s0 = v_sqrt(r2); h = 0.5 * v_rcp(s0);            s  = s0 corrected twice by its residual
+//   y0 = 2h;                                         y  = y0 after two Newton steps on s
+// -- which was checked against sqrtf / divide for every one of the 335 544 320 floats of that
+// range (cp_inv_sqrt_selftest below repeats the check on demand).  A wave uses it for an atom
+// when all its lanes' r2 are sure to be in the range, and the general expansion otherwise
+// (a point within 2^-10 of an atom in y and z, about one atom-row pair in fifty).
 #pragma once
 #include "role_common.h"
 #include "../header/cp_header.h"
@@ -17,6 +28,36 @@
 __constant__ float4 atominfo[MAXATOMS];
 
 namespace tk {
+
+#define CP_SHORT_LO 9.5367431640625e-07f   // 2^-20
+#define CP_SHORT_HI 1048576.0f             // 2^20
+
+// fl(1 / fl(sqrt(r2))) for r2 in [CP_SHORT_LO, CP_SHORT_HI)
+__device__ __forceinline__ float cp_inv_sqrt_short(float r2)
+{
+    const float s0 = __builtin_amdgcn_sqrtf(r2);
+    const float h = 0.5f * __builtin_amdgcn_rcpf(s0);
+    const float s1 = __builtin_fmaf(__builtin_fmaf(-s0, s0, r2), h, s0);
+    const float s = __builtin_fmaf(__builtin_fmaf(-s1, s1, r2), h, s1);
+    const float y0 = h + h;
+    const float y1 = __builtin_fmaf(__builtin_fmaf(-s, y0, 1.0f), y0, y0);
+    return __builtin_fmaf(__builtin_fmaf(-s, y1, 1.0f), y1, y1);
+}
+
+template <bool SHORT>
+__device__ __forceinline__ float cp_inv_sqrt(float r2)
+{
+    return SHORT ? cp_inv_sqrt_short(r2) : 1.0f / sqrtf(r2);
+}
+
+// true when every lane of the wave may take the short form for this atom: r2 = dx^2 + dyz2 of
+// all `points` points of the lane lies in [CP_SHORT_LO, CP_SHORT_HI)
+__device__ __forceinline__ bool cp_wave_in_short_range(float dx_first, float dyz2, float reach)
+{
+    const float far = __builtin_fabsf(dx_first) + reach;
+    const bool ok = dyz2 >= CP_SHORT_LO && dyz2 < 0.5f * CP_SHORT_HI && far * far < 0.5f * CP_SHORT_HI;
+    return __builtin_amdgcn_ballot_w64(!ok) == 0;
+}
 
 __device__ __forceinline__ void cp_block(int numatoms, float gridspacing,
                                          float *__restrict__ energygrid, unsigned block_id_x,
@@ -34,14 +75,23 @@ __device__ __forceinline__ void cp_block(int numatoms, float gridspacing,
     for (int n = 0; n < UNROLLX; ++n) energyval[n] = 0.0f;
     const float gridspacing_u = gridspacing * BLOCKSIZEX;
 
+    const float reach = UNROLLX * gridspacing_u;
     for (int atomid = 0; atomid < numatoms; ++atomid) {
         const float dy = coory - atominfo[atomid].y;
         const float dyz2 = (dy * dy) + atominfo[atomid].z;
         float dx = coorx - atominfo[atomid].x;
+        if (cp_wave_in_short_range(dx, dyz2, reach)) {
 #pragma unroll
-        for (int n = 0; n < UNROLLX; ++n) {
-            energyval[n] += atominfo[atomid].w * (1.0f / sqrtf(dx * dx + dyz2));
-            dx = dx + gridspacing_u;
+            for (int n = 0; n < UNROLLX; ++n) {
+                energyval[n] += atominfo[atomid].w * cp_inv_sqrt<true>(dx * dx + dyz2);
+                dx = dx + gridspacing_u;
+            }
+        } else {
+#pragma unroll
+            for (int n = 0; n < UNROLLX; ++n) {
+                energyval[n] += atominfo[atomid].w * cp_inv_sqrt<false>(dx * dx + dyz2);
+                dx = dx + gridspacing_u;
+            }
         }
     }
 #pragma unroll
@@ -71,18 +121,34 @@ __device__ __forceinline__ void cp_block_pair(int numatoms, float gridspacing,
         for (int n = 0; n < UNROLLX; ++n) energyval[b][n] = 0.0f;
     }
     const float gridspacing_u = gridspacing * BLOCKSIZEX;
+    const float reach = UNROLLX * gridspacing_u;
     for (int atomid = 0; atomid < numatoms; ++atomid) {
         const float4 a = atominfo[atomid];
+        float dyz2[2], dx[2];
 #pragma unroll
         for (int b = 0; b < 2; ++b) {
             const float dy = coory[b] - a.y;
-            const float dyz2 = (dy * dy) + a.z;
-            float dx = coorx[b] - a.x;
+            dyz2[b] = (dy * dy) + a.z;
+            dx[b] = coorx[b] - a.x;
+        }
+        const bool fast = cp_wave_in_short_range(dx[0], dyz2[0], reach) &&
+                          cp_wave_in_short_range(dx[1], dyz2[1], reach);
+        if (fast) {
 #pragma unroll
-            for (int n = 0; n < UNROLLX; ++n) {
-                energyval[b][n] += a.w * (1.0f / sqrtf(dx * dx + dyz2));
-                dx = dx + gridspacing_u;
-            }
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int n = 0; n < UNROLLX; ++n) {
+                    energyval[b][n] += a.w * cp_inv_sqrt<true>(dx[b] * dx[b] + dyz2[b]);
+                    dx[b] = dx[b] + gridspacing_u;
+                }
+        } else {
+#pragma unroll
+            for (int b = 0; b < 2; ++b)
+#pragma unroll
+                for (int n = 0; n < UNROLLX; ++n) {
+                    energyval[b][n] += a.w * cp_inv_sqrt<false>(dx[b] * dx[b] + dyz2[b]);
+                    dx[b] = dx[b] + gridspacing_u;
+                }
         }
     }
 #pragma unroll
@@ -115,20 +181,36 @@ __device__ __forceinline__ void cp_positions(int numatoms, float gridspacing, fl
         for (int n = 0; n < P; ++n) energyval[u][n] = 0.0f;
     }
     const float gridspacing_u = gridspacing * BLOCKSIZEX;
+    const float reach = P * gridspacing_u;
     for (int atomid = 0; atomid < numatoms; ++atomid) {
         const float4 a = atominfo[atomid];
+        float dyz2[U], dx[U];
+        bool fast = true;
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const float dy = coory[u] - a.y;
-            const float dyz2 = (dy * dy) + a.z;
-            float dx = coorx[u] - a.x;
+            dyz2[u] = (dy * dy) + a.z;
+            dx[u] = coorx[u] - a.x;
 #pragma unroll
-            for (int n = 0; n < PART * P; ++n) dx = dx + gridspacing_u;
+            for (int n = 0; n < PART * P; ++n) dx[u] = dx[u] + gridspacing_u;
+            fast = cp_wave_in_short_range(dx[u], dyz2[u], reach) && fast;
+        }
+        if (fast) {
 #pragma unroll
-            for (int n = 0; n < P; ++n) {
-                energyval[u][n] += a.w * (1.0f / sqrtf(dx * dx + dyz2));
-                dx = dx + gridspacing_u;
-            }
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int n = 0; n < P; ++n) {
+                    energyval[u][n] += a.w * cp_inv_sqrt<true>(dx[u] * dx[u] + dyz2[u]);
+                    dx[u] = dx[u] + gridspacing_u;
+                }
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int n = 0; n < P; ++n) {
+                    energyval[u][n] += a.w * cp_inv_sqrt<false>(dx[u] * dx[u] + dyz2[u]);
+                    dx[u] = dx[u] + gridspacing_u;
+                }
         }
     }
 #pragma unroll

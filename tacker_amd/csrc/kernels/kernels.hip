@@ -116,6 +116,20 @@ extern "C" __global__ void g_general_ptb_cp(int numatoms, float gridspacing, flo
                 (int)threadIdx.x - thread_base, (int)blockDim.x);
 }
 
+// Counts the floats with bit patterns in [lo_bits, hi_bits) for which the short form of
+// 1 / sqrt (tk::cp_inv_sqrt_short) differs from 1.0f / sqrtf(x) in any bit.
+extern "C" __global__ void cp_inv_sqrt_selftest(unsigned lo_bits, unsigned hi_bits,
+                                                unsigned long long *mismatches)
+{
+    unsigned long long bad = 0;
+    for (unsigned long long b = (unsigned long long)lo_bits + blockIdx.x * (unsigned long long)blockDim.x + threadIdx.x;
+         b < hi_bits; b += (unsigned long long)gridDim.x * blockDim.x) {
+        const float x = __uint_as_float((unsigned)b);
+        bad += __float_as_uint(tk::cp_inv_sqrt_short(x)) != __float_as_uint(1.0f / sqrtf(x));
+    }
+    if (bad) atomicAdd(mismatches, bad);
+}
+
 // ------------------------------------------------------------------ conv -> GEMM helpers
 
 // Caffe im2col, NCHW (src/TaskManager.cu:48-82): grid-stride over
@@ -175,6 +189,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("gptb_lbm", (const void *)general_ptb_lbm, ctx);
     insert("gptb_mriq", (const void *)g_general_ptb_mriq, ctx);
     insert("gptb_cp", (const void *)g_general_ptb_cp, ctx);
+    insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);
     insert("im2col", (const void *)im2col_gpu_kernel_, ctx);
     insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);
     insert("im2col_nhwc_f16", (const void *)im2col_nhwc_f16, ctx);

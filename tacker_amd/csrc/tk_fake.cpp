@@ -169,6 +169,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("gptb_lbm", cat(LBM, trailer(true)));
         add("gptb_mriq", cat(MRIQ, trailer(true)));
         add("gptb_cp", cat(CP, trailer(true)));
+        add("cp_inv_sqrt_selftest", {I, I, P});
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
         add("im2col_nhwc_f16", {P, I, I, I, I, I, I, I, I, I, I, P, I, P, I});

@@ -31,10 +31,10 @@ def check_session(p, cwd):
     assert len(re.findall(r"\[Ori\] BE task1 \+ task2 took [\d.]+ \+ [\d.]+ = [\d.]+ ms to execute\.", out)) == 2
     m = re.search(r"\[Result\] Aker BE task took ([\d.]+) \+ ([\d.]+)\(([\d.]+)\) = ([\d.]+) ms to execute\.", out)
     stage1, stage2, headroom, total = map(float, m.groups())
-    assert total == pytest.approx(stage1 + stage2, abs=2e-6) and stage2 >= headroom - 2e-6
+    assert total == pytest.approx(stage1 + stage2, abs=1e-4) and stage2 >= headroom - 1e-4
     m = re.search(r"\[Result\] Tacker BE task took ([\d.]+) \+ ([\d.]+)\(([\d.]+)\) = ([\d.]+) ms", out)
     stage1, stage2, headroom, total = map(float, m.groups())
-    assert stage2 == headroom and total == pytest.approx(stage1 + stage2, abs=2e-6)
+    assert stage2 == headroom and total == pytest.approx(stage1 + stage2, abs=1e-4)
     assert len(re.findall(r"\n\[PRE\]lc kernel took \d+\.\d+ ms to execute\.\n", out)) == 2
     # the recorder's table, written at exit
     text = open(os.path.join(cwd, "recorder_output.txt")).read().split("\n")

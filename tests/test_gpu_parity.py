@@ -333,6 +333,38 @@ def test_cp_block_positions_are_blocks_by_x_parts():
     assert same(run([(30, 42)], launch_grid=3), oracle.cp(info, g0, start=30, end=42, parts=4))
 
 
+def test_cp_short_inverse_square_root_is_the_ieee_one_on_its_whole_range():
+    # every float in [2^-20, 2^20): 335 544 320 values, each compared bitwise with 1.0f / sqrtf(x)
+    assert ta.cp_inv_sqrt_selftest() == 0
+    # the check itself can fail: just below the range the short form is not exact everywhere
+    assert ta.cp_inv_sqrt_selftest(0x00800000, 0x35800000) > 0
+
+
+def test_cp_points_on_and_next_to_atoms_take_the_general_path():
+    # atoms exactly on grid points (r2 = 0 -> inf, as IEEE says), within 2^-10 of a grid row, and far away:
+    # the wave-level range guard must send the close ones through sqrtf / divide
+    atoms = np.array([[1.6, 0.8, 0.0, 1.0],        # on the point (16, 8)
+                      [3.2005, 1.6003, 0.0, -0.5], # dy = 0.0003 from row 16: dyz2 below 2^-20
+                      [7.3, 2.29, 0.0, 0.25],
+                      [0.0, 0.0, 0.0, 2.0]], np.float32)
+    ta.cp_set_atoms(atoms, 0.0)
+    info = oracle.cp_atoms_to_const(atoms, 0.0)
+    g0 = np.zeros((32, 256), np.float32)
+    want = oracle.cp(info, g0)
+    assert np.isinf(want).sum() >= 1
+    for kw in ({}, {"launch_grid": 3}):
+        g = dev(g0)
+        ta.gptb_cp(4, 0.1, g, **kw)
+        assert np.array_equal(host(g).view(np.uint32), want.view(np.uint32))
+    g = dev(g0)
+    ta.ori_cp(4, 0.1, g)
+    assert np.array_equal(host(g).view(np.uint32), want.view(np.uint32))
+    g = dev(g0)
+    for a, b in ((0, 5), (5, 23), (23, ta.cp_blocks(256, 32))):
+        ta.gptb_cp(4, 0.1, g, start=a, end=b)
+    assert np.array_equal(host(g).view(np.uint32), want.view(np.uint32))
+
+
 def test_cp_fewer_atoms():
     atoms = cp_atoms()[:7]
     ta.cp_set_atoms(atoms, 0.5)
