@@ -471,6 +471,57 @@ def test_mix_tzgemm_cp(variant):
     assert np.array_equal(host(g).view(np.uint32), oracle.cp(info, np.zeros((32, 512), np.float32)).view(np.uint32))
 
 
+# ------------------------------------------------------------------ randomised ranges of the position grids
+@pytest.mark.parametrize("seed", range(12))
+def test_mriq_random_position_ranges_and_launch_shapes(seed):
+    rng = np.random.default_rng(1000 + seed)
+    numK = int(rng.integers(1, 420))
+    numX = int(rng.choice([256, 512, 1024, 1536]))
+    k, phiR, phiI, xyz = mriq_inputs(numK, numX, seed=seed)
+    kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+    ta.mriq_set_kvalues(kv)
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    total = ta.mriq_blocks(numK, numX)
+    q0 = rng.uniform(-1, 1, numX).astype(np.float32)
+    a = int(rng.integers(0, total + 1))
+    b = int(rng.integers(a, 2 * total + 1))                       # may run past the grid and wrap
+    mid = int(rng.integers(a, b + 1))
+    grid = int(rng.choice([1, 2, 3, 5, 8, 40, 0]))
+    Qr, Qi = dev(q0), dev(q0)
+    ta.gptb_mriq(numK, x, y, z, Qr, Qi, start=a, end=b, launch_grid=grid)
+    tr, ti = oracle.mriq(kv, xyz[0], xyz[1], xyz[2], q0, q0, start=a, end=b, kchunk=128, f64=True)
+    tol = lambda got, want: np.all(np.abs(got.astype(np.float64) - want) <= 2e-3 + 2e-4 * np.abs(want))
+    assert tol(host(Qr), tr.astype(np.float64)) and tol(host(Qi), ti.astype(np.float64)), (numK, numX, a, b, grid)
+    # the same range cut in two, with another launch shape: the same bits
+    Pr, Pi = dev(q0), dev(q0)
+    other = int(rng.choice([1, 3, 7, 16, 0]))
+    ta.gptb_mriq(numK, x, y, z, Pr, Pi, start=a, end=mid, launch_grid=other)
+    ta.gptb_mriq(numK, x, y, z, Pr, Pi, start=mid, end=b, launch_grid=grid)
+    assert np.array_equal(host(Pr), host(Qr)) and np.array_equal(host(Pi), host(Qi)), (numK, numX, a, mid, b, grid, other)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_cp_random_position_ranges_and_launch_shapes(seed):
+    rng = np.random.default_rng(2000 + seed)
+    H, Wd = [(8, 128), (16, 256), (24, 384), (40, 128), (8, 640)][int(rng.integers(0, 5))]
+    natoms = int(rng.integers(1, 65))
+    atoms = cp_atoms()[:natoms].copy()
+    atoms[:, :2] *= np.float32(0.1)                               # bring some atoms into the small volume
+    zplane = float(rng.choice([0.0, 0.3]))
+    ta.cp_set_atoms(atoms, zplane)
+    info = oracle.cp_atoms_to_const(atoms, zplane)
+    g0 = rng.uniform(-1, 1, (H, Wd)).astype(np.float32)
+    total = ta.cp_blocks(Wd, H)
+    a = int(rng.integers(0, total + 1))
+    b = int(rng.integers(a, 2 * total + 1))
+    grid = int(rng.choice([1, 2, 3, 5, 8, 40, 0]))
+    block = int(rng.choice([128, 256]))
+    g = dev(g0)
+    ta.gptb_cp(natoms, 0.1, g, start=a, end=b, launch_grid=grid, launch_block=block)
+    want = oracle.cp(info, g0, start=a, end=b, parts=4)
+    assert np.array_equal(host(g).view(np.uint32), want.view(np.uint32)), (H, Wd, natoms, a, b, grid, block)
+
+
 # ------------------------------------------------------------------ best-effort x best-effort pairs
 def _small_be(name):
     """(ori kernel, blocks, output tensors, snapshot of the outputs before any launch)"""
@@ -538,4 +589,39 @@ def test_mix_with_a_k_split_gemm_shape(variant):
     ok, fro, dmax = gemm_tolerance_ok(full, oracle.tzgemm(A, B, f64=True), K)
     assert ok and fro <= 1e-5, (fro, dmax)
     assert np.array_equal(host(mix_s), oracle.stencil(C0, C1, A0, A0))
+    assert ta.spin_fail_flag() == 0
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_fused_launches_equal_the_two_kernels_alone(seed):
+    # random GEMM shape (both forms of the role), tile range, best-effort kernel, block range (may wrap),
+    # variant and launch grid: the fused launch must leave exactly what the two GPTB kernels leave
+    rng = np.random.default_rng(3000 + seed)
+    name = ["stencil", "lbm", "mriq", "cp"][seed % 4]
+    M, N, K = [(256, 384, 256), (256, 384, 1024), (128, 128, 640), (384, 256, 128), (512, 128, 2048)][int(rng.integers(0, 5))]
+    A, B = gemm_inputs(M, N, K, seed=seed)
+    dA, dB = dev(A), dev(B)
+    tiles = (M // 64) * (N // 64)
+    t0 = int(rng.integers(0, tiles))
+    t1 = int(rng.integers(t0, tiles + 1))
+    ori, nblk, outs = _small_be(name)
+    wrap_ok = name in ("mriq", "cp")                     # accumulating kernels: a second pass adds again, in order
+    b0 = int(rng.integers(0, nblk))
+    b1 = int(rng.integers(b0, (2 * nblk if wrap_ok else nblk) + 1))
+    variant = [None, "wave_256", "wave_512", "wg_1_1", "wg_1_2"][int(rng.integers(0, 5))]
+    before = [o.clone() for o in outs]
+    solo_c = torch.full((M, N), -3.0, device="cuda:0")
+    tz_ori = ta.ori_tzgemm_create(dA, dB, solo_c)
+    ta.gptb_create(ori, 0, 0, b0, b1).execute()
+    ta.gptb_create(tz_ori, 0, 0, t0, t1).execute()
+    want = [host(o).copy() for o in outs] + [host(solo_c).copy()]
+    for o, keep in zip(outs, before):
+        o.copy_(keep)
+    solo_c.fill_(-3.0)
+    be_full = ta.gptb_create(ori, 0, 0, 0, nblk)
+    tz_full = ta.gptb_create(tz_ori, 0, 0, 0, tiles)
+    ta.mix_create(be_full, tz_full, b0, b1, t0, t1, variant=variant).execute()
+    got = [host(o) for o in outs] + [host(solo_c)]
+    for g, w in zip(got, want):
+        assert np.array_equal(g.view(np.uint32), w.view(np.uint32)), (name, (M, N, K), (t0, t1), (b0, b1), variant)
     assert ta.spin_fail_flag() == 0
