@@ -121,6 +121,20 @@ TK_API const char *tacker_last_error(void);
  * units of the reference's 64x64 CTA tile. */
 TK_API int tacker_tzgemm_grid_dim(int m, int n, int k, int out[4]);
 
+/* No counterpart in the reference (its tzgemm is one CTA per tile whatever the shape). Shapes
+ * with few tiles and a long reduction (the batch-1 layers of src/dnn/: 32-128 tiles, K up to
+ * 25088) cut the reduction of a tile over `parts` workgroups; the partial tiles and one arrival
+ * counter per tile live in a workspace the library binds to the output buffer C on the first
+ * GEMM that writes it (general_ptb_tzgemm's seventh parameter; NULL when parts == 1).
+ * tacker_tzgemm_parts: the number of parts for (m, n, k) rounded as tacker_tzgemm_grid_dim
+ * rounds them -- a function of the shape only, so fused and unfused launches add in the same
+ * order. tacker_tzgemm_workspace_bytes: size of that workspace, 0 when parts == 1.
+ * tacker_tzgemm_release_workspaces: synchronises the device and frees them all; only when no
+ * kernel object built on caller-owned operands is left. */
+TK_API int tacker_tzgemm_parts(int m, int n, int k);
+TK_API long long tacker_tzgemm_workspace_bytes(int m, int n, int k);
+TK_API int tacker_tzgemm_release_workspaces(void);
+
 /* general_ptb_tzgemm through GPTBKernel (src/gptb_kernel/tzgemm_kernel.cu:430-449,
  * src/GPTBKernel.h:99-119, src/TaskManager.cu:238-248): C[M][N] f32 =
  * 1.1 * A[M][K] f16 * (B[N][K] f16)^T for the 64x64 tiles [tile_start, tile_end).

@@ -86,6 +86,7 @@ def _declare(lib):
     lib.tacker_spin_fail_flag.argtypes = [C.POINTER(i)]
     lib.tacker_float_to_half_bits.argtypes = [f]
     lib.tacker_float_to_half_bits.restype = C.c_uint16
+    lib.tacker_tzgemm_workspace_bytes.restype = C.c_longlong
     lib.tacker_rng_uniform.argtypes = [C.c_uint64, f, f, vp, C.c_size_t]
     lib.tacker_task_create.restype = vp
     lib.tacker_task_create.argtypes = [cp, i, i]
@@ -163,6 +164,19 @@ def tzgemm_grid_dim(m, n, k):
     out = (C.c_int * 4)()
     lib().tacker_tzgemm_grid_dim(m, n, k, out)
     return list(out)
+
+
+def tzgemm_parts(m, n, k):
+    """Workgroups that share the reduction of one tile of this shape (1 for most shapes)."""
+    return int(lib().tacker_tzgemm_parts(m, n, k))
+
+
+def tzgemm_workspace_bytes(m, n, k):
+    return int(lib().tacker_tzgemm_workspace_bytes(m, n, k))
+
+
+def tzgemm_release_workspaces():
+    check(lib().tacker_tzgemm_release_workspaces(), "tzgemm_release_workspaces")
 
 
 def get_kernel_info(kernel, key):

@@ -197,6 +197,27 @@ int tacker_tzgemm_grid_dim(int m, int n, int k, int out[4])
     return TK_SUCCESS;
 }
 
+int tacker_tzgemm_parts(int m, int n, int k)
+{
+    const std::vector<int> d = getTZGEMMGridDim(m, n, k);
+    return tz_ksplit_parts(d[0], d[1], d[2]);
+}
+
+long long tacker_tzgemm_workspace_bytes(int m, int n, int k)
+{
+    const std::vector<int> d = getTZGEMMGridDim(m, n, k);
+    return tz_workspace_bytes(d[0], d[1], d[2]);
+}
+
+int tacker_tzgemm_release_workspaces(void)
+{
+    REQUIRE_INIT();
+    return guarded([&]() -> int {
+        tzgemmReleaseWorkspaces();
+        return TK_SUCCESS;
+    });
+}
+
 int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
                        int tile_end, int launch_grid, tkStream_t stream)
 {

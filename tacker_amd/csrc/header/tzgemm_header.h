@@ -29,5 +29,53 @@
 // over its 4 waves): few macro tiles for the CUs there are, and a reduction worth cutting
 #define TZ_KSPLIT_MAX_MACRO_TILES 64
 #define TZ_KSPLIT_MIN_K 512
+#define TZ_KSPLIT_LDS_BYTES (4 * 2 * 2 * TZ_REF_TILE * TZ_BLOCK_K * 2)   // two 16 KiB stages per wave
+// ... and, when the tiles are fewer still, the reduction of one tile is also cut over several
+// workgroups ("parts"): each adds its share of K into a partial tile in the workspace, and the
+// last one to finish adds the partial tiles in part order and stores C.
+#define TZ_KSPLIT_TARGET_WORKGROUPS 256   // parts are chosen to give about this many workgroups a share
+#define TZ_KSPLIT_MAX_PARTS 8
+#define TZ_KSPLIT_MIN_CHUNKS_PER_PART 8   // TZ_BLOCK_K chunks: two per wave
+#define TZ_PARTIAL_TILE_BYTES (TZ_REF_TILE * TZ_REF_TILE * 4)
+#define TZ_WORKSPACE_ALIGN 1024
+
+#ifdef __HIPCC__
+#define TZ_HOST_DEVICE __host__ __device__
+#else
+#define TZ_HOST_DEVICE
+#endif
+
+// Both depend on (M, N, K) only -- never on the launch -- so a fused launch and the plain kernel
+// always add in the same order.
+TZ_HOST_DEVICE inline bool tz_use_ksplit(int M, int N, int K)
+{
+    const int n_macro = (M / TZ_MACRO_TILE) * (N / TZ_MACRO_TILE);
+    return n_macro <= TZ_KSPLIT_MAX_MACRO_TILES && K >= TZ_KSPLIT_MIN_K;
+}
+// workgroups that share the reduction of one reference tile (1: no workspace needed)
+TZ_HOST_DEVICE inline int tz_ksplit_parts(int M, int N, int K)
+{
+    if (!tz_use_ksplit(M, N, K)) return 1;
+    const int n_ref = (M / TZ_REF_TILE) * (N / TZ_REF_TILE);
+    int parts = TZ_KSPLIT_TARGET_WORKGROUPS / n_ref;
+    const int by_k = (K / TZ_BLOCK_K) / TZ_KSPLIT_MIN_CHUNKS_PER_PART;
+    if (parts > by_k) parts = by_k;
+    if (parts > TZ_KSPLIT_MAX_PARTS) parts = TZ_KSPLIT_MAX_PARTS;
+    return parts < 1 ? 1 : parts;
+}
+// Workspace of one GEMM: a zeroed arrival counter per reference tile (the kernel leaves them
+// zero again), then parts partial tiles per reference tile.  0 when the shape needs none.
+TZ_HOST_DEVICE inline long long tz_workspace_counter_bytes(int M, int N)
+{
+    const long long n_ref = (long long)(M / TZ_REF_TILE) * (N / TZ_REF_TILE);
+    return (n_ref * 4 + TZ_WORKSPACE_ALIGN - 1) / TZ_WORKSPACE_ALIGN * TZ_WORKSPACE_ALIGN;
+}
+TZ_HOST_DEVICE inline long long tz_workspace_bytes(int M, int N, int K)
+{
+    const int parts = tz_ksplit_parts(M, N, K);
+    if (parts == 1) return 0;
+    const long long n_ref = (long long)(M / TZ_REF_TILE) * (N / TZ_REF_TILE);
+    return tz_workspace_counter_bytes(M, N) + n_ref * parts * TZ_PARTIAL_TILE_BYTES;
+}
 
 #define TZ_ALPHA 1.1f             // alpha_g, src/header/tzgemm_header.h:64

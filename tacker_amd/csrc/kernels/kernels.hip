@@ -75,11 +75,11 @@ extern "C" __global__ __launch_bounds__(128) void ori_cp(int numatoms, float gri
 // ------------------------------------------------------------------ GPTB kernels
 
 extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void general_ptb_tzgemm(
-    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, GPTB_TRAILER)
+    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, unsigned *workspace, GPTB_TRAILER)
 {
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
     tk::WorkgroupSync sync;
-    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x, ptb_iter_block_step,
+    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, workspace, (int)blockIdx.x, ptb_iter_block_step,
                     ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base, tz_lds,
                     sync);
 }

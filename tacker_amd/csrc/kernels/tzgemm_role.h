@@ -381,20 +381,58 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
 // (((w0 + w1) + w2) + w3), so the result does not depend on timing.  Four times as many
 // workgroups, each with a K loop a quarter as long.  The waves share no operands, so each
 // has a private two-stage ring (2 x 16 KiB) and the K loop needs no barrier at all.
-// Which form runs depends on (M, N, K) only -- never on the launch geometry -- so a fused
-// launch and the plain kernel always add in the same order.
-__device__ __forceinline__ bool tz_use_ksplit(int M, int N, int K)
+//
+// When even that leaves CUs without work (32 to 128 tiles), the reduction of a tile is
+// also cut over tz_ksplit_parts workgroups.  A unit of work is (part, tile); a workgroup
+// adds its part of K as above, stores the partial tile to the workspace, and takes a
+// ticket from the tile's arrival counter.  The workgroup that draws the last ticket adds
+// the partial tiles in part order (((p0 + p1) + p2) ...), scales, stores C and puts the
+// counter back to zero: nobody ever waits for another workgroup, and the sum does not
+// depend on who came last.
+//
+// Which form runs, and how many parts, depends on (M, N, K) only -- never on the launch
+// geometry -- so a fused launch and the plain kernel always add in the same order.
+
+// Unit of the K-split form a workgroup takes in one round of the persistent loop, -1 for
+// none.  count units (at most role_blocks) are handed out; when both are multiples of 8,
+// workgroup b runs on XCD b % 8 and each XCD gets a contiguous run of units -- units that
+// follow each other share operand panels (same part of K, neighbouring tiles), which then
+// meet in that XCD's L2.  Either way the first count workgroups are the ones with a unit.
+__device__ __forceinline__ int tz_ksplit_unit_of(int role_block, int role_blocks, int count)
 {
-    const int n_macro = (M / TZ_MACRO_TILE) * (N / TZ_MACRO_TILE);
-    return n_macro <= TZ_KSPLIT_MAX_MACRO_TILES && K >= TZ_KSPLIT_MIN_K;
+    if (role_block >= count) return -1;
+    if (role_blocks % TK_XCD_NUM == 0 && count % TK_XCD_NUM == 0)
+        return (role_block % TK_XCD_NUM) * (count / TK_XCD_NUM) + role_block / TK_XCD_NUM;
+    return role_block;
+}
+
+// Partial tiles travel between workgroups on other XCDs, whose L2s do not see each other's
+// lines.  Every access to them is an agent-scope access of its own (it goes through to the
+// memory side both XCDs share), so no cache has to be written back or dropped as a whole.
+// A partial tile is 16 blocks of 64 x float4 (block = i * 4 + j of the accumulator set),
+// stored as two 8-byte halves per lane: [block][half][lane].
+typedef unsigned long long tz_u64;
+__device__ __forceinline__ void tz_partial_store(tz_u64 *tile, int block, int lane, float4_t v)
+{
+    union { float4_t f; tz_u64 q[2]; } u;
+    u.f = v;
+    __hip_atomic_store(tile + (block * 2 + 0) * 64 + lane, u.q[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(tile + (block * 2 + 1) * 64 + lane, u.q[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float4_t tz_partial_load(const tz_u64 *tile, int block, int lane)
+{
+    union { float4_t f; tz_u64 q[2]; } u;
+    u.q[0] = __hip_atomic_load(tile + (block * 2 + 0) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    u.q[1] = __hip_atomic_load(tile + (block * 2 + 1) * 64 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return u.f;
 }
 
 template <class Sync>
 __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ A,
                                                    const _Float16 *__restrict__ B, float *__restrict__ C,
-                                                   int M, int N, int K, int role_block, int role_blocks,
-                                                   int tile_start, int tile_end, int tid, char *lds,
-                                                   Sync &sync)
+                                                   int M, int N, int K, unsigned *workspace,
+                                                   int role_block, int role_blocks, int tile_start,
+                                                   int tile_end, int tid, char *lds, Sync &sync)
 {
     typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int BK = TZ_BLOCK_K;
@@ -407,8 +445,9 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
     const int ref_cols = N / TZ_REF_TILE;
     const int n_ref = (M / TZ_REF_TILE) * ref_cols;
     const int kchunks = K / BK;
-    const int c_first = (wave * kchunks) / 4;
-    const int c_last = ((wave + 1) * kchunks) / 4;
+    const int parts = tz_ksplit_parts(M, N, K);
+    tz_u64 *partial_tiles =
+        reinterpret_cast<tz_u64 *>(reinterpret_cast<char *>(workspace) + tz_workspace_counter_bytes(M, N));
     char *mine = lds + wave * (2 * STAGE);            // this wave's two stages
     const unsigned mine_lds = (unsigned)(size_t)(lptr_t)mine;
     // load j of an operand fills rows 8j .. 8j+7: lane lands in row 8j + lane/8, slot lane%8,
@@ -421,10 +460,22 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
     const int frag_seg1 = ((4 + (lane >> 4)) ^ frag_key) * 16;
     const int frag_row = (lane & 15) * ROWB;
     if (tile_end > n_ref) tile_end = n_ref;
+    if (parts > 1 && workspace == nullptr) tile_end = tile_start;   // the host always binds one; never fault
+    const int tiles = tile_end - tile_start;
+    const int units = tiles > 0 ? tiles * parts : 0;
 
-    for (int pos = tile_start + role_block; pos < tile_end; pos += role_blocks) {
+    for (int round_base = 0; round_base < units; round_base += role_blocks) {
+        const int in_round = tz_ksplit_unit_of(role_block, role_blocks, min(units - round_base, role_blocks));
+        if (in_round < 0) break;
+        const int unit = round_base + in_round;
+        const int part = unit / tiles;
+        const int pos = tile_start + unit % tiles;
         const int ti = pos / ref_cols;
         const int tj = pos % ref_cols;
+        const int part_first = (part * kchunks) / parts;
+        const int part_chunks = ((part + 1) * kchunks) / parts - part_first;
+        const int c_first = part_first + (wave * part_chunks) / 4;
+        const int c_last = part_first + ((wave + 1) * part_chunks) / 4;
         const char *a_tile = reinterpret_cast<const char *>(A + (size_t)(ti * TZ_REF_TILE) * K);
         const char *b_tile = reinterpret_cast<const char *>(B + (size_t)(tj * TZ_REF_TILE) * K);
 #define TZK_ISSUE(chunk_, stage_)                                                                  \
@@ -489,16 +540,66 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
                     for (int j = 0; j < 4; ++j)
                         acc[i][j] += *reinterpret_cast<const float4_t *>(lds + w * (2 * STAGE) +
                                                                          ((i * 4 + j) * 64 + lane) * 16);
-            float *c_lane = C + (size_t)(ti * TZ_REF_TILE + (lane & 15)) * N + tj * TZ_REF_TILE + (lane >> 4) * 4;
+            if (parts == 1) {
+                float *c_lane = C + (size_t)(ti * TZ_REF_TILE + (lane & 15)) * N + tj * TZ_REF_TILE + (lane >> 4) * 4;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+                for (int i = 0; i < 4; ++i)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    float4_t v = acc[i][j] * TZ_ALPHA;
-                    *reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16) = v;
-                }
+                    for (int j = 0; j < 4; ++j) {
+                        float4_t v = acc[i][j] * TZ_ALPHA;
+                        *reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16) = v;
+                    }
+            } else {
+                tz_u64 *my_partial = partial_tiles + ((size_t)pos * parts + part) * (TZ_PARTIAL_TILE_BYTES / 8);
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) tz_partial_store(my_partial, i * 4 + j, lane, acc[i][j]);
+                // the partial tile has arrived where the other XCDs read it before the ticket is drawn
+                __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
+                asm volatile("" ::: "memory");
+                unsigned ticket = 0;
+                if (lane == 0)
+                    ticket = __hip_atomic_fetch_add(workspace + pos, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                ticket = __builtin_amdgcn_readfirstlane(ticket);
+                // tell every wave whether this workgroup drew the last ticket: one word at the head of
+                // each wave's own LDS region (wave 0 is done with the partial tiles that were there)
+                if (lane < 4)
+                    *reinterpret_cast<unsigned *>(lds + lane * (2 * STAGE)) = (ticket == (unsigned)(parts - 1)) ? 1u : 0u;
+            }
         }
         sync.sync();   // wave 0 has read the partial tiles before the next tile's loads land on them
+        if (parts > 1 &&
+            __builtin_amdgcn_readfirstlane(*(const __attribute__((address_space(3))) unsigned *)(lptr_t)mine) != 0u) {
+            // last to arrive: add the partial tiles in part order.  Wave w takes rows 16w .. 16w+15 of
+            // the tile; loads go out four parts at a time so that a batch is one trip to memory.
+            const tz_u64 *tile_parts = partial_tiles + (size_t)pos * parts * (TZ_PARTIAL_TILE_BYTES / 8);
+            float4_t sum[4];
+            for (int p0 = 0; p0 < parts; p0 += 4) {
+                float4_t got[4][4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (p0 + q < parts) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j)
+                            got[q][j] = tz_partial_load(tile_parts + (p0 + q) * (TZ_PARTIAL_TILE_BYTES / 8),
+                                                        wave * 4 + j, lane);
+                    }
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    if (p0 + q < parts) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) sum[j] = (p0 + q == 0) ? got[q][j] : sum[j] + got[q][j];
+                    }
+            }
+            float *c_lane = C + (size_t)(ti * TZ_REF_TILE + wave * 16 + (lane & 15)) * N + tj * TZ_REF_TILE + (lane >> 4) * 4;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                float4_t v = sum[j] * TZ_ALPHA;
+                *reinterpret_cast<float4_t *>(c_lane + j * 16) = v;
+            }
+            if (tid == 0) __hip_atomic_store(workspace + pos, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
     }
     sync.finish();
@@ -506,14 +607,15 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
 
 template <int STAGES, class Sync>
 __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
-                                            float *__restrict__ C, int M, int N, int K, int role_block,
-                                            int role_blocks, int tile_start, int tile_end, int tid, char *lds,
-                                            Sync &sync)
+                                            float *__restrict__ C, int M, int N, int K, unsigned *workspace,
+                                            int role_block, int role_blocks, int tile_start, int tile_end,
+                                            int tid, char *lds, Sync &sync)
 {
-    static_assert(STAGES * TZ_STAGE_BYTES >= 4 * 2 * 2 * TZ_REF_TILE * TZ_BLOCK_K * 2,
+    static_assert(STAGES * TZ_STAGE_BYTES >= TZ_KSPLIT_LDS_BYTES,
                   "the K-split form needs two 16 KiB stages per wave");
     if (tz_use_ksplit(M, N, K))
-        tzgemm_role_ksplit(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds, sync);
+        tzgemm_role_ksplit(A, B, C, M, N, K, workspace, role_block, role_blocks, tile_start, tile_end, tid, lds,
+                           sync);
     else
         tzgemm_role_tiles<STAGES>(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds, sync);
 }
@@ -525,7 +627,7 @@ __device__ __forceinline__ int tz_busy_workgroups(int M, int N, int K, int role_
                                                   int tile_end)
 {
     if (tile_start >= tile_end) return 0;
-    const int units = tz_use_ksplit(M, N, K) ? tile_end - tile_start
+    const int units = tz_use_ksplit(M, N, K) ? (tile_end - tile_start) * tz_ksplit_parts(M, N, K)
                                              : (M / TZ_MACRO_TILE) * (N / TZ_MACRO_TILE);
     return min(units, role_blocks);
 }

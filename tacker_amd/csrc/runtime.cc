@@ -1,6 +1,7 @@
 // runtime.cc -- process-wide state of the host runtime: the objects the
 // reference defines in src/main.cu (logger, recorder, moduleCenter, fmap) and in
 // src/TaskManager.cu:19-46 (global GEMM buffers), and the one-time set-up.
+#include <mutex>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -25,6 +26,8 @@ bool gemm_malloced = false;
 void *ori_wmma_A = nullptr;
 void *ori_wmma_B = nullptr;
 float *ori_wmma_C = nullptr;
+long long MAX_ORI_WMMA_WS = 0;
+void *ori_wmma_workspace = nullptr;
 
 static void grow(void **ptr, long long *have, long long need, bool seed_halves)
 {
@@ -54,7 +57,50 @@ void ensureGlobalGemmBuffers(int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
     grow(&ori_wmma_A, &MAX_ORI_WMMA_A, a, true);
     grow(&ori_wmma_B, &MAX_ORI_WMMA_B, b, true);
     grow((void **)&ori_wmma_C, &MAX_ORI_WMMA_C, c, false);
+    grow(&ori_wmma_workspace, &MAX_ORI_WMMA_WS, tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL), false);
     gemm_malloced = true;
+}
+
+namespace {
+struct BoundWorkspace {
+    void *ptr;
+    long long bytes;
+};
+std::mutex g_workspace_mutex;
+std::unordered_map<const void *, BoundWorkspace> g_workspaces;   // by output buffer
+std::vector<void *> g_outgrown_workspaces;   // replaced by a larger one; older kernel objects may still hold them
+constexpr size_t kMaxBoundWorkspaces = 1024;
+}  // namespace
+
+void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
+{
+    const long long need = tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL);
+    if (need == 0 || C == nullptr) return nullptr;
+    std::lock_guard<std::mutex> lock(g_workspace_mutex);
+    auto it = g_workspaces.find(C);
+    if (it != g_workspaces.end() && it->second.bytes >= need) return it->second.ptr;
+    if (it == g_workspaces.end() && g_workspaces.size() >= kMaxBoundWorkspaces)
+        logger.ERROR("tzgemm: " + std::to_string(kMaxBoundWorkspaces) +
+                     " output buffers hold a workspace; call tzgemmReleaseWorkspaces() once the kernels "
+                     "that use them are gone");
+    // a new binding is rare (first GEMM on this C, or a larger shape), so it may wait for the device
+    void *ptr = nullptr;
+    TK_SAFE_CALL(tkMalloc(&ptr, (size_t)need));
+    TK_SAFE_CALL(tkMemset(ptr, 0, (size_t)need));
+    TK_SAFE_CALL(tkDeviceSynchronize());   // zero before any stream's kernel reads the counters
+    if (it != g_workspaces.end()) g_outgrown_workspaces.push_back(it->second.ptr);
+    g_workspaces[C] = BoundWorkspace{ptr, need};
+    return ptr;
+}
+
+void tzgemmReleaseWorkspaces()
+{
+    std::lock_guard<std::mutex> lock(g_workspace_mutex);
+    TK_SAFE_CALL(tkDeviceSynchronize());
+    for (auto &w : g_workspaces) TK_SAFE_CALL(tkFree(w.second.ptr));
+    for (void *p : g_outgrown_workspaces) TK_SAFE_CALL(tkFree(p));
+    g_workspaces.clear();
+    g_outgrown_workspaces.clear();
 }
 
 static void fmap_insert(const char *key, const void *func, void *)

@@ -50,7 +50,7 @@ const std::vector<int> STENCIL = {F, F, P, P, I, I, I};
 const std::vector<int> LBM = {P, P};
 const std::vector<int> MRIQ = {I, I, P, P, P, P, P};
 const std::vector<int> CP = {I, F, P};
-const std::vector<int> TZ = {P, P, P, I, I, I};
+const std::vector<int> TZ = {P, P, P, I, I, I, P};
 }  // namespace
 
 extern "C" {

@@ -69,6 +69,61 @@ def test_tzgemm_tile_range_writes_only_its_tiles(start, end, grid, K):
     assert np.array_equal(got[mask], full[mask])         # same values as the full launch
 
 
+# Shapes whose tiles are so few that the reduction of one tile is shared by several workgroups (the
+# batch-1 layers of VGG16: conv5, conv4, fc2, fc3 with 8, 2, 2, 8 parts).  Who stores C is decided by
+# arrival order, what is stored is not: every launch -- whatever its grid, however its range is cut --
+# must give the same bits, and the arrival counters must be back at zero for the next one.
+@pytest.mark.parametrize("M,N,K", [(256, 512, 4608), (896, 512, 4608), (4096, 128, 4096), (1024, 128, 4096)])
+def test_tzgemm_reduction_shared_by_workgroups(M, N, K):
+    parts = ta.tzgemm_parts(M, N, K)
+    assert parts > 1 and ta.tzgemm_workspace_bytes(M, N, K) >= (M // 64) * (N // 64) * parts * 64 * 64 * 4
+    A, B = gemm_inputs(M, N, K, seed=M + K)
+    dA, dB = dev(A), dev(B)
+    Cd = torch.full((M, N), -7.0, device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, Cd)
+    first = host(Cd).copy()
+    ok, fro, dmax = gemm_tolerance_ok(first, oracle.tzgemm(A, B, f64=True), K)
+    assert ok and fro <= 1e-5, (fro, dmax)
+    tiles = (M // 64) * (N // 64)
+    for grid in (0, 8, 17, 64, 256, 300):
+        Cd.fill_(-7.0)
+        ta.gptb_tzgemm(dA, dB, Cd, launch_grid=grid)
+        assert np.array_equal(host(Cd).view(np.uint32), first.view(np.uint32)), grid
+    # the range cut into three launches, the middle one first
+    cuts = [0, tiles // 3 + 1, tiles - 5, tiles]
+    Cd.fill_(-7.0)
+    for i in (1, 0, 2):
+        ta.gptb_tzgemm(dA, dB, Cd, tile_start=cuts[i], tile_end=cuts[i + 1], launch_grid=(0, 40, 256)[i])
+    assert np.array_equal(host(Cd).view(np.uint32), first.view(np.uint32))
+    # a range of one tile leaves the others alone
+    Cd.fill_(-7.0)
+    ta.gptb_tzgemm(dA, dB, Cd, tile_start=3, tile_end=4)
+    got = host(Cd)
+    want = oracle.tzgemm(A, B, C_init=np.full((M, N), -7.0, np.float32), start=3, end=4)
+    mask = want != -7.0
+    assert np.array_equal(got[~mask], want[~mask]) and np.array_equal(got[mask], first[mask])
+
+
+def test_tzgemm_shared_reduction_fused_equals_unfused():
+    # conv5's shape with a best-effort kernel in the same launch: same bits as the GEMM alone
+    M, N, K = 256, 512, 4608
+    A, B = gemm_inputs(M, N, K, seed=41)
+    dA, dB = dev(A), dev(B)
+    solo = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, solo)
+    A0 = stencil_inputs(16, 64, 256, seed=9)
+    a0 = dev(A0)
+    want_s = oracle.stencil(C0, C1, A0, A0)
+    for variant in ("wave_512", "wave_256", "wg_1_1"):
+        for _ in range(2):
+            mix_c = torch.full((M, N), -7.0, device="cuda:0")
+            mix_s = a0.clone()
+            ta.mix_tzgemm_stencil(C0, C1, a0, mix_s, dA, dB, mix_c, variant=variant)
+            assert np.array_equal(host(mix_c).view(np.uint32), host(solo).view(np.uint32)), variant
+            assert np.array_equal(host(mix_s), want_s)
+    assert ta.spin_fail_flag() == 0
+
+
 # ------------------------------------------------------------------ stencil
 # widths that are multiples of 4 take the float4 (quad of blocks) form of the GPTB role, the
 # others the one-block-per-wave form; 3 planes is the smallest grid with an interior

@@ -129,6 +129,36 @@ def test_qos_guard(fake):
     assert fake.tacker_qos_must_run_solo(50.0, 0.0, 6.5, 6.5) == 0
 
 
+def test_tzgemm_parts_rule(fake):
+    # a function of the shape only: 1 unless the K-split form applies and leaves workgroups idle
+    fake.tacker_tzgemm_workspace_bytes.restype = C.c_longlong
+    want = {(2048, 2048, 2048): 1, (3200, 256, 2304): 1, (896, 512, 4608): 2, (256, 512, 4608): 8,
+            (4096, 128, 25088): 2, (4096, 128, 4096): 2, (1024, 128, 4096): 8, (128, 128, 512): 1,
+            (128, 128, 1024): 2, (128, 128, 128): 1, (196, 512, 4608): 8}
+    for (m, n, k), parts in want.items():
+        assert fake.tacker_tzgemm_parts(m, n, k) == parts, (m, n, k)
+        mg, ng = max(128, m // 128 * 128), max(128, n // 128 * 128)
+        tiles = (mg // 64) * (ng // 64)
+        size = fake.tacker_tzgemm_workspace_bytes(m, n, k)
+        assert size == (0 if parts == 1 else (tiles * 4 + 1023) // 1024 * 1024 + tiles * parts * 16384)
+
+
+def test_tzgemm_workspace_is_bound_to_the_output_buffer(fake):
+    fake.tk_fake_reset()
+    A = np.zeros((256, 1024), np.float16)
+    C1 = np.zeros((256, 256), np.float32)
+    C2 = np.zeros((256, 256), np.float32)
+    seen = []
+    for Cm in (C1, C1, C2):
+        assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 256, 256, 1024, 0, 16, 0, None) == 0
+        seen.append(as_ptr(launches(fake)[-1]["args"][6]))
+    assert seen[0] != 0 and seen[0] == seen[1] and seen[2] not in (0, seen[0])
+    # a shape without shared reductions gets none
+    assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, C1.ctypes.data, 256, 256, 128, 0, 16, 0, None) == 0
+    assert as_ptr(launches(fake)[-1]["args"][6]) == 0
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+
+
 # ------------------------------------------------------------------ marshalling
 def test_gptb_stencil_parameter_vector(fake):
     fake.tk_fake_reset()
@@ -162,8 +192,9 @@ def test_mix_parameter_vector_matches_reference_signature(fake):
     assert rc == 0, fake.tacker_last_error()
     (l,) = launches(fake)
     # stencil_tzgemm_mix has 16 + 15 = 31 parameters (src/mix_kernel/tzgemm_stencil.cu:281-283):
-    # [stencil 7 + 6 dims + start,step,end][A,B,C,M,N,K + 6 dims + start,step,end]
-    assert l["key"] == "tzgemm_stencil@wg_1_1" and len(l["args"]) == 31
+    # [stencil 7 + 6 dims + start,step,end][A,B,C,M,N,K + 6 dims + start,step,end]; here the GEMM's
+    # workspace pointer follows K (null for a shape whose reduction stays inside a workgroup)
+    assert l["key"] == "tzgemm_stencil@wg_1_1" and len(l["args"]) == 32
     a = l["args"]
     grid = l["grid"][0]
     assert grid % 16 == 0 and l["block"] == (256, 1, 1)
@@ -171,8 +202,9 @@ def test_mix_parameter_vector_matches_reference_signature(fake):
     assert [as_int(x) for x in a[13:16]] == [1, grid, 4]            # start1, step = fused grid, end1
     assert [as_ptr(x) for x in a[16:19]] == [A.ctypes.data, B.ctypes.data, Cm.ctypes.data]
     assert [as_int(x) for x in a[19:22]] == [256, 384, 128]
-    assert [as_int(x) for x in a[22:28]] == [24, 1, 1, 256, 1, 1]   # tzgemm ori grid = tile count, block 256
-    assert [as_int(x) for x in a[28:31]] == [3, grid, 20]
+    assert as_ptr(a[22]) == 0
+    assert [as_int(x) for x in a[23:29]] == [24, 1, 1, 256, 1, 1]   # tzgemm ori grid = tile count, block 256
+    assert [as_int(x) for x in a[29:32]] == [3, grid, 20]
 
 
 @pytest.mark.parametrize("be,n_be", [("lbm", 2), ("mriq", 7), ("cp", 3)])
@@ -192,8 +224,8 @@ def test_other_mix_vectors_have_reference_lengths(fake, be, n_be):
     assert rc == 0, fake.tacker_last_error()
     (l,) = launches(fake)
     # lbm_tzgemm_mix 11+15, mriq_tzgemm_mix 16+15, cp_tzgemm_mix 12+15
-    # (src/mix_kernel/tzgemm_{lbm,mriq,cp}.cu dispatcher signatures)
-    assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 15
+    # (src/mix_kernel/tzgemm_{lbm,mriq,cp}.cu dispatcher signatures), plus the GEMM's workspace pointer
+    assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 16
 
 
 def test_gptb_vector_is_restored_after_launch_and_after_failure(fake):
