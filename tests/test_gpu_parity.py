@@ -104,6 +104,29 @@ def test_tzgemm_reduction_shared_by_workgroups(M, N, K):
     assert np.array_equal(got[~mask], want[~mask]) and np.array_equal(got[mask], first[mask])
 
 
+def test_tzgemm_shared_reductions_on_two_streams_do_not_meet():
+    # each output buffer has a workspace of its own, so GEMMs of the same shape that run at the same
+    # time on different streams cannot draw each other's tickets
+    M, N, K = 256, 512, 4608
+    inputs = [gemm_inputs(M, N, K, seed=70 + i) for i in range(2)]
+    dev_in = [(dev(A), dev(B)) for A, B in inputs]
+    want = []
+    for dA, dB in dev_in:
+        Cd = torch.zeros((M, N), device="cuda:0")
+        ta.gptb_tzgemm(dA, dB, Cd)
+        want.append(host(Cd).copy())
+    assert not np.array_equal(want[0], want[1])
+    streams = [torch.cuda.Stream(device="cuda:0") for _ in range(2)]
+    outs = [torch.zeros((M, N), device="cuda:0") for _ in range(2)]
+    torch.cuda.synchronize()
+    for _ in range(20):
+        for (dA, dB), Cd, st in zip(dev_in, outs, streams):
+            ta.gptb_tzgemm(dA, dB, Cd, launch_grid=96, stream=st)
+    torch.cuda.synchronize()
+    for Cd, w in zip(outs, want):
+        assert np.array_equal(host(Cd).view(np.uint32), w.view(np.uint32))
+
+
 def test_tzgemm_shared_reduction_fused_equals_unfused():
     # conv5's shape with a best-effort kernel in the same launch: same bits as the GEMM alone
     M, N, K = 256, 512, 4608
