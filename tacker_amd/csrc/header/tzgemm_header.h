@@ -37,6 +37,7 @@
 #define TZ_KSPLIT_MAX_PARTS 8
 #define TZ_KSPLIT_MIN_CHUNKS_PER_PART 8   // TZ_BLOCK_K chunks: two per wave
 #define TZ_PARTIAL_TILE_BYTES (TZ_REF_TILE * TZ_REF_TILE * 4)
+#define TZ_KSPLIT_PARTS_IN_FLIGHT 2      // partial tiles the last workgroup loads at a time (registers)
 #define TZ_WORKSPACE_ALIGN 1024
 
 #ifdef __HIPCC__

@@ -173,8 +173,63 @@ __device__ __forceinline__ void lbm_cell_pair(const float *__restrict__ src, flo
 #undef TK_LBM_SCATTER2
 }
 
+// Two rows at once, for a role that has few waves on its CU (inside a fused kernel): all 40
+// loads of both rows are issued before the first collision, so a wave has twice the bytes in
+// flight.  Each destination word has one writer whichever rows are paired, so the result is
+// the same as row by row.
+__device__ __forceinline__ void lbm_cell_pair_x2(const float *__restrict__ src, float *__restrict__ dst,
+                                                 int cells, int ca, int cb, int sx, int sxy)
+{
+#define TK_LBM_LOAD(entry, dx, dy, dz, name)                                                          \
+    const lbm_pair_t name##_a = *reinterpret_cast<const lbm_pair_t *>(src + cells * (entry) + ca);      \
+    const lbm_pair_t name##_b = *reinterpret_cast<const lbm_pair_t *>(src + cells * (entry) + cb);
+    TK_LBM_DIRECTIONS(TK_LBM_LOAD)
+#undef TK_LBM_LOAD
+    const lbm_pair_t flags_a = *reinterpret_cast<const lbm_pair_t *>(src + cells * LBM_FLAGS + ca);
+    const lbm_pair_t flags_b = *reinterpret_cast<const lbm_pair_t *>(src + cells * LBM_FLAGS + cb);
+#define TK_LBM_SCATTER_ROW(c_, entry, dx, dy, dz, v0_, v1_)                                \
+    do {                                                                                   \
+        const int t_ = (c_) + (dx) + (dy) * sx + (dz) * sxy;                               \
+        float *o_ = dst + cells * (entry) + t_;                                            \
+        if (t_ >= 0 && t_ + 1 < cells) {                                                   \
+            *reinterpret_cast<lbm_pair_t *>(o_) = lbm_pair_t{v0_, v1_};                    \
+        } else {                                                                           \
+            if (t_ >= 0 && t_ < cells) o_[0] = v0_;                                        \
+            if (t_ + 1 >= 0 && t_ + 1 < cells) o_[1] = v1_;                                \
+        }                                                                                  \
+    } while (0);
+    // row a is collided and scattered while row b's loads are still on their way; the scheduling
+    // fences keep the two rows' arithmetic apart (interleaved it needs more registers than a fused
+    // kernel has)
+    __builtin_amdgcn_sched_barrier(0);
+    {
+#define TK_LBM_SPLIT(entry, dx, dy, dz, name) float name##0 = name##_a.x, name##1 = name##_a.y;
+        TK_LBM_DIRECTIONS(TK_LBM_SPLIT)
+#undef TK_LBM_SPLIT
+        lbm_collide(__float_as_uint(flags_a.x), tempC0, tempN0, tempS0, tempE0, tempW0, tempT0, tempB0, tempNE0, tempNW0, tempSE0, tempSW0, tempNT0, tempNB0, tempST0, tempSB0, tempET0, tempEB0, tempWT0, tempWB0);
+        lbm_collide(__float_as_uint(flags_a.y), tempC1, tempN1, tempS1, tempE1, tempW1, tempT1, tempB1, tempNE1, tempNW1, tempSE1, tempSW1, tempNT1, tempNB1, tempST1, tempSB1, tempET1, tempEB1, tempWT1, tempWB1);
+#define TK_LBM_SCATTER_A(entry, dx, dy, dz, name) TK_LBM_SCATTER_ROW(ca, entry, dx, dy, dz, name##0, name##1)
+        TK_LBM_DIRECTIONS(TK_LBM_SCATTER_A)
+#undef TK_LBM_SCATTER_A
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    {
+#define TK_LBM_SPLIT(entry, dx, dy, dz, name) float name##0 = name##_b.x, name##1 = name##_b.y;
+        TK_LBM_DIRECTIONS(TK_LBM_SPLIT)
+#undef TK_LBM_SPLIT
+        lbm_collide(__float_as_uint(flags_b.x), tempC0, tempN0, tempS0, tempE0, tempW0, tempT0, tempB0, tempNE0, tempNW0, tempSE0, tempSW0, tempNT0, tempNB0, tempST0, tempSB0, tempET0, tempEB0, tempWT0, tempWB0);
+        lbm_collide(__float_as_uint(flags_b.y), tempC1, tempN1, tempS1, tempE1, tempW1, tempT1, tempB1, tempNE1, tempNW1, tempSE1, tempSW1, tempNT1, tempNB1, tempST1, tempSB1, tempET1, tempEB1, tempWT1, tempWB1);
+#define TK_LBM_SCATTER_B(entry, dx, dy, dz, name) TK_LBM_SCATTER_ROW(cb, entry, dx, dy, dz, name##0, name##1)
+        TK_LBM_DIRECTIONS(TK_LBM_SCATTER_B)
+#undef TK_LBM_SCATTER_B
+    }
+#undef TK_LBM_SCATTER_ROW
+}
+
 // grid_dimension_x = sy, grid_dimension_y = sz, block_dimension_x = sx
-// (src/ori_kernel/lbm_kernel.cu:218-222).
+// (src/ori_kernel/lbm_kernel.cu:218-222).  ROWS_PER_WAVE = 2: a wave takes two of its rows at a
+// time (see lbm_cell_pair_x2); which rows a wave owns is the same either way.
+template <int ROWS_PER_WAVE = 1>
 __device__ __forceinline__ void lbm_role(const float *__restrict__ src, float *__restrict__ dst,
                                          int grid_dimension_x, int grid_dimension_y,
                                          int block_dimension_x, int role_block, int role_blocks,
@@ -201,8 +256,17 @@ __device__ __forceinline__ void lbm_role(const float *__restrict__ src, float *_
         x_step = role_threads * per_lane;
     }
     const unsigned stride = (unsigned)role_blocks * rows_at_once;
-    for (unsigned pos = (unsigned)start + role_block * rows_at_once + row_slot; pos < (unsigned)end;
-         pos += stride) {
+    unsigned pos = (unsigned)start + role_block * rows_at_once + row_slot;
+    if (ROWS_PER_WAVE == 2 && per_lane == 2) {
+        for (; pos + stride < (unsigned)end && pos + stride > pos; pos += 2 * stride) {
+            const unsigned pos_b = pos + stride;
+            const int row_a = (int)(pos % sy) * sx + (int)((pos / sy) % sz) * sxy;
+            const int row_b = (int)(pos_b % sy) * sx + (int)((pos_b / sy) % sz) * sxy;
+            for (int x = x_first; x < sx; x += x_step)
+                lbm_cell_pair_x2(src, dst, cells, x + row_a, x + row_b, sx, sxy);
+        }
+    }
+    for (; pos < (unsigned)end; pos += stride) {
         const int y = pos % sy;
         const int z = (pos / sy) % sz;
         if (per_lane == 2) {

@@ -412,6 +412,15 @@ __device__ __forceinline__ int tz_ksplit_unit_of(int role_block, int role_blocks
 // A partial tile is 16 blocks of 64 x float4 (block = i * 4 + j of the accumulator set),
 // stored as two 8-byte halves per lane: [block][half][lane].
 typedef unsigned long long tz_u64;
+// The same value, but one the compiler has to take as computed here: addresses derived from it
+// are formed where they are used instead of being kept in registers across the K loop (the
+// sixteen block offsets of a partial tile, hoisted out of the tile loop, do not fit beside the
+// accumulators in a fused kernel's 168 registers).
+__device__ __forceinline__ int tz_opaque(int v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
 __device__ __forceinline__ void tz_partial_store(tz_u64 *tile, int block, int lane, float4_t v)
 {
     union { float4_t f; tz_u64 q[2]; } u;
@@ -551,10 +560,11 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
                     }
             } else {
                 tz_u64 *my_partial = partial_tiles + ((size_t)pos * parts + part) * (TZ_PARTIAL_TILE_BYTES / 8);
+                const int lane_here = tz_opaque(lane);
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) tz_partial_store(my_partial, i * 4 + j, lane, acc[i][j]);
+                    for (int j = 0; j < 4; ++j) tz_partial_store(my_partial, i * 4 + j, lane_here, acc[i][j]);
                 // the partial tile has arrived where the other XCDs read it before the ticket is drawn
                 __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
                 asm volatile("" ::: "memory");
@@ -572,21 +582,22 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
         if (parts > 1 &&
             __builtin_amdgcn_readfirstlane(*(const __attribute__((address_space(3))) unsigned *)(lptr_t)mine) != 0u) {
             // last to arrive: add the partial tiles in part order.  Wave w takes rows 16w .. 16w+15 of
-            // the tile; loads go out four parts at a time so that a batch is one trip to memory.
+            // the tile; loads go out two parts at a time so that a batch is one trip to memory.
             const tz_u64 *tile_parts = partial_tiles + (size_t)pos * parts * (TZ_PARTIAL_TILE_BYTES / 8);
+            const int lane_here = tz_opaque(lane);
             float4_t sum[4];
-            for (int p0 = 0; p0 < parts; p0 += 4) {
-                float4_t got[4][4];
+            for (int p0 = 0; p0 < parts; p0 += TZ_KSPLIT_PARTS_IN_FLIGHT) {
+                float4_t got[TZ_KSPLIT_PARTS_IN_FLIGHT][4];
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
+                for (int q = 0; q < TZ_KSPLIT_PARTS_IN_FLIGHT; ++q)
                     if (p0 + q < parts) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
                             got[q][j] = tz_partial_load(tile_parts + (p0 + q) * (TZ_PARTIAL_TILE_BYTES / 8),
-                                                        wave * 4 + j, lane);
+                                                        wave * 4 + j, lane_here);
                     }
 #pragma unroll
-                for (int q = 0; q < 4; ++q)
+                for (int q = 0; q < TZ_KSPLIT_PARTS_IN_FLIGHT; ++q)
                     if (p0 + q < parts) {
 #pragma unroll
                         for (int j = 0; j < 4; ++j) sum[j] = (p0 + q == 0) ? got[q][j] : sum[j] + got[q][j];

@@ -42,7 +42,7 @@ def generate_wg_split(be, tz_wgs, be_wgs, threads=256):
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="sp.role_block", blocks="sp.role_blocks",
                                              tid="(int)threadIdx.x", stages="TZ_STAGES_WG")
     be_call = ROLES[be]["call"].format(p=p_be, block="sp.role_block", blocks="sp.role_blocks",
-                                       tid="(int)threadIdx.x", threads=threads)
+                                       tid="(int)threadIdx.x", threads=threads, extra="")
     name = mix_kernel_name(be, variant)
     text = f"""// {be}-tzgemm  workgroup split  {tz_wgs} tzgemm : {be_wgs} {be} workgroups per group
 extern "C" __global__ __launch_bounds__({threads}) void {name}(
@@ -77,8 +77,11 @@ def generate_wave_split(be, be_threads, tz_first=True):
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="(int)blockIdx.x",
                                              blocks=f"{p_tz}ptb_iter_block_step",
                                              tid=f"(int)threadIdx.x - {tz_lo}", stages="TZ_STAGES")
+    # few best-effort waves share the CU with the GEMM: lbm takes two rows per wave to keep
+    # enough loads in flight
     be_call = ROLES[be]["call"].format(p=p_be, block="be_block", blocks="be_blocks",
-                                       tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads)
+                                       tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads,
+                                       extra="<2>" if be == "lbm" else "")
     tz_cond = (f"threadIdx.x < {tz_threads}" if tz_first else f"threadIdx.x >= {be_threads}")
     name = mix_kernel_name(be, variant)
     unused = _void_unused(sig_be + sig_tz, tz_call + be_call + f"{p_be}ptb_iter_block_step")
@@ -145,8 +148,9 @@ def generate_be_pair(be1, be2, wgs1, wgs2, threads=256, order=False):
     p1, sig1 = signature(be1, 0)
     p2, sig2 = signature(be2, 1)
     block, blocks = ("(int)blockIdx.x", "(int)gridDim.x") if order else ("sp.role_block", "sp.role_blocks")
-    call1 = ROLES[be1]["call"].format(p=p1, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads)
-    call2 = ROLES[be2]["call"].format(p=p2, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads)
+    call1 = ROLES[be1]["call"].format(p=p1, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads, extra="")
+    call2 = ROLES[be2]["call"].format(p=p2, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads,
+                                      extra="")
     name = be_pair_kernel_name(be1, be2, variant)
     if order:
         title = f"order split  {wgs1} of {wgs1 + wgs2} workgroups start with {be1}, the others with {be2}"

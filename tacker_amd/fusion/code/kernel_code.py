@@ -42,7 +42,7 @@ ROLES = {
     "lbm": {
         "params": [("float*", "srcGrid"), ("float*", "dstGrid")],
         "needs_sync": False,
-        "call": ("tk::lbm_role({p}srcGrid, {p}dstGrid, {p}grid_dimension_x, {p}grid_dimension_y, "
+        "call": ("tk::lbm_role{extra}({p}srcGrid, {p}dstGrid, {p}grid_dimension_x, {p}grid_dimension_y, "
                  "{p}block_dimension_x, {block}, {blocks}, {p}ptb_start_block_pos, "
                  "{p}ptb_end_block_pos, {tid}, {threads});"),
     },
