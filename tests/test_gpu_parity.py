@@ -69,6 +69,34 @@ def test_tzgemm_tile_range_writes_only_its_tiles(start, end, grid, K):
     assert np.array_equal(got[mask], full[mask])         # same values as the full launch
 
 
+# A workgroup with several macro tiles refills its LDS ring for each of them.  Few workgroups, K just
+# above and well above the ring depth (4 chunks of 64), ranges with holes: same bits as one tile per
+# workgroup.
+@pytest.mark.parametrize("M,N,K", [(256, 384, 384), (1152, 1024, 512), (1280, 1024, 640), (1152, 1024, 1280)])
+def test_tzgemm_several_tiles_per_workgroup_equal_one_tile_per_workgroup(M, N, K):
+    assert (M // 128) * (N // 128) > 64 or K < 512          # shapes of the macro-tile form
+    A, B = gemm_inputs(M, N, K, seed=M + N + K)
+    dA, dB = dev(A), dev(B)
+    tiles = (M // 64) * (N // 64)
+    ref = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, ref, launch_grid=256)             # at most one macro tile per workgroup
+    ref = host(ref)
+    ok, fro, dmax = gemm_tolerance_ok(ref, oracle.tzgemm(A, B, f64=True), K)
+    assert ok and fro <= 1e-5, (fro, dmax)
+    for grid in (1, 2, 3, 5, 8):
+        Cd = torch.full((M, N), -7.0, device="cuda:0")
+        ta.gptb_tzgemm(dA, dB, Cd, launch_grid=grid)
+        assert np.array_equal(host(Cd).view(np.uint32), ref.view(np.uint32)), grid
+    # ranges that skip macro tiles between the ones a workgroup takes
+    for start, end, grid in ((0, tiles // 2, 2), (tiles // 3, tiles, 1), (5, tiles - 7, 3)):
+        Cd = torch.full((M, N), -7.0, device="cuda:0")
+        ta.gptb_tzgemm(dA, dB, Cd, tile_start=start, tile_end=end, launch_grid=grid)
+        want = oracle.tzgemm(A, B, C_init=np.full((M, N), -7.0, np.float32), start=start, end=end)
+        mask = want != -7.0
+        got = host(Cd)
+        assert np.array_equal(got[~mask], want[~mask]) and np.array_equal(got[mask], ref[mask]), (start, end, grid)
+
+
 # Shapes whose tiles are so few that the reduction of one tile is shared by several workgroups (the
 # batch-1 layers of VGG16: conv5, conv4, fc2, fc3 with 8, 2, 2, 8 parts).  Who stores C is decided by
 # arrival order, what is stored is not: every launch -- whatever its grid, however its range is cut --
