@@ -60,6 +60,48 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
         }
         return;
     }
+    if ((K_pad & 7) == 0 && (long)Ho * Wo * K_pad < (1L << 31)) {
+        // any channel count (the first layer has 3): still one 16-byte store of A per thread and
+        // 32-bit index arithmetic, the 8 values gathered one by one; groups past the real K
+        // (most of the row when C is small) are just zeros
+        const unsigned groups_per_row = (unsigned)K_pad >> 3;
+        const unsigned total = (unsigned)(Ho * Wo) * groups_per_row;
+        for (unsigned g = blockIdx.x * blockDim.x + threadIdx.x; g < total; g += blockDim.x * gridDim.x) {
+            const unsigned m = g / groups_per_row;
+            const int k0 = (int)(g - m * groups_per_row) << 3;
+            h8 out = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (k0 < k_real) {
+                const int ho = (int)(m / (unsigned)Wo), wo = (int)(m - (unsigned)ho * (unsigned)Wo);
+                // (kh, kw, c) of k0 by division, of the 7 that follow by counting up
+                int tap = (int)((unsigned)k0 / (unsigned)C);
+                int c = k0 - tap * C;
+                int kh = (int)((unsigned)tap / (unsigned)KW), kw = tap - kh * KW;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    if (k0 + e < k_real) {
+                        const int h = ho * stride - pad + kh, w = wo * stride - pad + kw;
+                        if (h >= 0 && h < H && w >= 0 && w < W) {
+                            float v = act[((size_t)h * W + w) * c_stride + c];
+                            if (bias) {
+                                v += bias[c];
+                                if (relu && v < 0.0f) v = 0.0f;
+                            }
+                            out[e] = (_Float16)v;
+                        }
+                    }
+                    if (++c == C) {
+                        c = 0;
+                        if (++kw == KW) {
+                            kw = 0;
+                            ++kh;
+                        }
+                    }
+                }
+            }
+            *reinterpret_cast<h8 *>(A + (size_t)g * 8) = out;
+        }
+        return;
+    }
     const long total = (long)Ho * Wo * K_pad;
     for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (long)blockDim.x * gridDim.x) {
