@@ -224,8 +224,13 @@ int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int
     REQUIRE_INIT();
     const int rc = check_gemm(A, B, C, M, N, K);
     if (rc) return rc;
-    return run_gptb_once(new OriTZGEMMKernel(0, M, N, K, A, B, C), tile_start, tile_end, launch_grid,
-                         TZ_THREADS, stream);
+    Kernel *ori = nullptr;   // binding a workspace to C can fail (allocation): not outside guarded()
+    const int made = guarded([&]() -> int {
+        ori = new OriTZGEMMKernel(0, M, N, K, A, B, C);
+        return TK_SUCCESS;
+    });
+    if (made) return made;
+    return run_gptb_once(ori, tile_start, tile_end, launch_grid, TZ_THREADS, stream);
 }
 
 int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz, tkStream_t stream)

@@ -2,6 +2,7 @@
 // reference defines in src/main.cu (logger, recorder, moduleCenter, fmap) and in
 // src/TaskManager.cu:19-46 (global GEMM buffers), and the one-time set-up.
 #include <mutex>
+#include <stdexcept>
 #include <string>
 #include <unordered_map>
 #include <vector>
@@ -80,9 +81,9 @@ void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBA
     auto it = g_workspaces.find(C);
     if (it != g_workspaces.end() && it->second.bytes >= need) return it->second.ptr;
     if (it == g_workspaces.end() && g_workspaces.size() >= kMaxBoundWorkspaces)
-        logger.ERROR("tzgemm: " + std::to_string(kMaxBoundWorkspaces) +
-                     " output buffers hold a workspace; call tzgemmReleaseWorkspaces() once the kernels "
-                     "that use them are gone");
+        throw std::runtime_error("tzgemm: " + std::to_string(kMaxBoundWorkspaces) +
+                                 " output buffers hold a workspace; call tzgemmReleaseWorkspaces() once the "
+                                 "kernels that use them are gone");
     // a new binding is rare (first GEMM on this C, or a larger shape), so it may wait for the device
     void *ptr = nullptr;
     TK_SAFE_CALL(tkMalloc(&ptr, (size_t)need));
