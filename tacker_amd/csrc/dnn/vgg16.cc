@@ -100,13 +100,16 @@ protected:
 class ConvKernel : public GemmLayer {
 public:
     // act_bias != nullptr: act is the raw output of the previous convolution; its bias and
-    // ReLU are applied while the operand is gathered
-    ConvKernel(int id, const std::string &name, const float *act, const float *act_bias, int H, int W, int C,
-               int c_stride, int Cout, void *A, const void *Wt, float *out)
+    // ReLU are applied while the operand is gathered.  pooled: act is that output at twice the
+    // height and width, and the 2x2 max pooling between the two layers happens on the way in too.
+    ConvKernel(int id, const std::string &name, const float *act, const float *act_bias, bool pooled, int H,
+               int W, int C, int c_stride, int Cout, void *A, const void *Wt, float *out)
         : GemmLayer(id, name, pad128(H * W), pad128(Cout), pad128(9 * C), A, Wt, out), act_(act),
-          act_bias_(act_bias), H_(H), W_(W), C_(C), cs_(c_stride), Cout_(Cout), A_(A)
+          act_bias_(act_bias), pool_(pooled ? 1 : 0), H_(H), W_(W), C_(C), cs_(c_stride), Cout_(Cout), A_(A)
     {
         this->mixable = 2;
+        if (pooled && !(C % 8 == 0 && c_stride % 4 == 0))
+            logger.ERROR("vgg16: a pooled input needs a channel count that is a multiple of 8");
     }
     // {n,c,h,w, k,c,kh,kw, pad,pad, stride,stride, dil,dil}
     std::vector<int> getArgs() override { return {1, C_, H_, W_, Cout_, C_, 3, 3, 1, 1, 1, 1, 1, 1}; }
@@ -116,6 +119,11 @@ protected:
     {
         int KH = 3, KW = 3, pad = 1, stride = 1, Ho = H_, Wo = W_, Kp = K_;
         int relu = 1;
+        if (C_ % 8 == 0 && cs_ % 4 == 0) {   // every layer but the first: each activation read once
+            void *args[] = {&act_, &H_, &W_, &C_, &cs_, &A_, &Kp, &act_bias_, &relu, &pool_};
+            launch1d("im2col3x3_scatter_nhwc_f16", (long)H_ * W_ * (C_ / 8), args, stream);
+            return;
+        }
         void *args[] = {&act_, &H_, &W_, &C_, &cs_, &KH, &KW, &pad, &stride, &Ho, &Wo, &A_, &Kp, &act_bias_, &relu};
         launch1d("im2col_nhwc_f16", (long)Ho * Wo * Kp, args, stream);
     }
@@ -123,6 +131,7 @@ protected:
 private:
     const float *act_;
     const float *act_bias_;
+    int pool_;
     int H_, W_, C_, cs_, Cout_;
     void *A_;
 };
@@ -240,13 +249,22 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
     const float *act_bias = nullptr;   // bias the reader of act still has to apply
     int id = 100;
     const int plan[] = {64, 64, -1, 128, 128, -1, 256, 256, 256, -1, 512, 512, 512, -1, 512, 512, 512, -1};
+    // A pooling layer between two convolutions is not a kernel either: the next convolution's
+    // operand is built from the 2x2 maxima.  Only the last one, which feeds the classifier, is.
+    bool pooled = false;
     int block = 1, layer = 1;
-    for (int p : plan) {
+    const int n_plan = (int)(sizeof(plan) / sizeof(plan[0]));
+    for (int step = 0; step < n_plan; ++step) {
+        const int p = plan[step];
         if (p < 0) {
-            float *out = devAlloc(fl, (size_t)(H / 2) * (W / 2) * ld);
-            addKernel(new PoolKernel(id++, "MaxPool_" + std::to_string(block), act, act_bias, H, W, ld, out));
-            act = out;
-            act_bias = nullptr;
+            if (step + 1 < n_plan) {
+                pooled = true;
+            } else {
+                float *out = devAlloc(fl, (size_t)(H / 2) * (W / 2) * ld);
+                addKernel(new PoolKernel(id++, "MaxPool_" + std::to_string(block), act, act_bias, H, W, ld, out));
+                act = out;
+                act_bias = nullptr;
+            }
             H /= 2;
             W /= 2;
             block++;
@@ -258,7 +276,9 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
         void *Wt = randomHalfMatrix(fl, rng, Cout, 9 * C, Np, Kp, std::sqrt(2.0f / (9 * C)));
         float *bias = randomBias(fl, rng, Cout, Np);
         float *out = devAlloc(fl, (size_t)pad128(H * W) * Np);
-        addKernel(new ConvKernel(id++, "Convolution_" + name, act, act_bias, H, W, C, ld, Cout, Abuf, Wt, out));
+        addKernel(new ConvKernel(id++, "Convolution_" + name, act, act_bias, pooled, H, W, C, ld, Cout, Abuf, Wt,
+                                 out));
+        pooled = false;
         impl->convOut.push_back(Act{out, H, W, Cout, Np, Wt, bias, Np, Kp});
         act = out;
         act_bias = bias;

@@ -126,6 +126,82 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
     }
 }
 
+// The same operand for a 3x3 / pad 1 / stride 1 convolution with C a multiple of 8, built the other
+// way round: a thread takes 8 channels of one input pixel, reads them once (bias and ReLU applied as
+// above) and stores them to the up to 9 rows of A whose window covers the pixel -- A[(ho*W + wo)][tap*C
+// + c] with ho = h + 1 - kh, wo = w + 1 - kw.  The gather form reads every activation 9 times (18 bytes
+// read per byte of A written); this one reads it once.  What no pixel writes is zero and is written by
+// the thread of the row's own pixel: the taps of its window that fall outside the image, and the
+// columns from 9*C up to K_pad.  Every element of rows < H*W is written exactly once.
+// pool != 0: act is [2H][2W][c_stride] and the pixel is the maximum of its 2x2 cell, taken before the
+// bias and the ReLU exactly as maxpool2x2_nhwc takes it -- the pooling layer between two
+// convolutions without a launch and without its round trip through memory.
+extern "C" __global__ void im2col3x3_scatter_nhwc_f16(const float *act, int H, int W, int C, int c_stride,
+                                                      _Float16 *A, int K_pad, const float *bias, int relu,
+                                                      int pool)
+{
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+    const unsigned groups = (unsigned)C >> 3;                 // 8-channel groups of a pixel
+    const unsigned total = (unsigned)(H * W) * groups;
+    const unsigned row_groups = (unsigned)K_pad >> 3;
+    const h8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (unsigned id = blockIdx.x * blockDim.x + threadIdx.x; id < total; id += blockDim.x * gridDim.x) {
+        const unsigned p = id / groups;
+        const int c = (int)(id - p * groups) << 3;
+        const int h = (int)(p / (unsigned)W), w = (int)(p - (unsigned)h * (unsigned)W);
+        f4 lo, hi;
+        if (pool) {
+            const size_t right = (size_t)c_stride, below = (size_t)(2 * W) * c_stride;
+            const float *src = act + ((size_t)(2 * h) * (2 * W) + 2 * w) * c_stride + c;
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                const float *s4 = src + 4 * half;
+                const f4 a = *reinterpret_cast<const f4 *>(s4);
+                const f4 b = *reinterpret_cast<const f4 *>(s4 + right);
+                const f4 d = *reinterpret_cast<const f4 *>(s4 + below);
+                const f4 e = *reinterpret_cast<const f4 *>(s4 + below + right);
+                f4 m;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) m[i] = fmaxf(fmaxf(a[i], b[i]), fmaxf(d[i], e[i]));
+                if (half == 0) lo = m;
+                else hi = m;
+            }
+        } else {
+            const float *src = act + (size_t)p * c_stride + c;
+            lo = *reinterpret_cast<const f4 *>(src);
+            hi = *reinterpret_cast<const f4 *>(src + 4);
+        }
+        if (bias) {
+            lo += *reinterpret_cast<const f4 *>(bias + c);
+            hi += *reinterpret_cast<const f4 *>(bias + c + 4);
+            if (relu) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    lo[e] = lo[e] < 0.0f ? 0.0f : lo[e];
+                    hi[e] = hi[e] < 0.0f ? 0.0f : hi[e];
+                }
+            }
+        }
+        const h8 v = {(_Float16)lo.x, (_Float16)lo.y, (_Float16)lo.z, (_Float16)lo.w,
+                      (_Float16)hi.x, (_Float16)hi.y, (_Float16)hi.z, (_Float16)hi.w};
+        _Float16 *own = A + (size_t)p * K_pad + c;             // this pixel's row, this channel group
+#pragma unroll
+        for (int kh = 0; kh < 3; ++kh)
+#pragma unroll
+            for (int kw = 0; kw < 3; ++kw) {
+                const int tap = (kh * 3 + kw) * C;
+                const int ho = h + 1 - kh, wo = w + 1 - kw;    // row whose tap (kh, kw) is this pixel
+                if (ho >= 0 && ho < H && wo >= 0 && wo < W)
+                    *reinterpret_cast<h8 *>(A + (size_t)(ho * W + wo) * K_pad + tap + c) = v;
+                const int hs = h - 1 + kh, ws = w - 1 + kw;    // pixel under tap (kh, kw) of the own row
+                if (hs < 0 || hs >= H || ws < 0 || ws >= W) *reinterpret_cast<h8 *>(own + tap) = zero;
+            }
+        for (unsigned g = 9 * groups + ((unsigned)c >> 3); g < row_groups; g += groups)
+            *reinterpret_cast<h8 *>(A + (size_t)p * K_pad + (size_t)g * 8) = zero;
+    }
+}
+
 // y[m][n] = max(0, y[m][n] + bias[n]) over rows < M of a [M][ld] matrix
 extern "C" __global__ void bias_relu_rows(float *y, const float *bias, int M, int ld, int relu)
 {

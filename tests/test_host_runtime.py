@@ -399,7 +399,7 @@ def test_vgg16_task_structure(small_vgg):
     ks = small_vgg.kernels()
     convs = [k for k in ks if k["mixable"] == 2]
     fcs = [k for k in ks if k["mixable"] == 1]
-    assert len(convs) == 13 and len(fcs) == 3 and len([k for k in ks if "MaxPool" in k["name"]]) == 5
+    assert len(convs) == 13 and len(fcs) == 3 and len([k for k in ks if "MaxPool" in k["name"]]) == 1
     assert convs[0]["args"] == [1, 3, 32, 32, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1]
     assert convs[-1]["args"] == [1, 512, 2, 2, 512, 512, 3, 3, 1, 1, 1, 1, 1, 1]
     assert [k["args"] for k in fcs] == [[4096, 128, 512], [4096, 128, 4096], [1024, 128, 4096]]
@@ -410,16 +410,22 @@ def test_vgg16_solo_pass_launches_every_layer(fake, small_vgg):
     fake.tk_fake_reset()
     small_vgg.execute(raw_stream=None)
     keys = [l["key"] for l in launches(fake)]
-    assert keys.count("gptb_tzgemm") == 16 and keys.count("im2col_nhwc_f16") == 13
-    assert keys.count("maxpool2x2_nhwc") == 5 and keys.count("pack_fc_input") == 3
+    # the first layer (3 channels) gathers its operand, the others scatter it (activations read once)
+    assert keys.count("gptb_tzgemm") == 16 and keys.count("im2col_nhwc_f16") == 1
+    assert keys.count("im2col3x3_scatter_nhwc_f16") == 12
+    # pooling between two convolutions happens while the next operand is built; only the pool
+    # in front of the classifier is a launch
+    assert keys.count("maxpool2x2_nhwc") == 1 and keys.count("pack_fc_input") == 3
     # no separate bias/ReLU pass: each convolution's bias travels to whatever reads its output next
     assert keys.count("bias_relu_rows") == 0
-    gathers = [l for l in launches(fake) if l["key"] == "im2col_nhwc_f16"]
+    gathers = [l for l in launches(fake) if l["key"] in ("im2col_nhwc_f16", "im2col3x3_scatter_nhwc_f16")]
     pools = [l for l in launches(fake) if l["key"] == "maxpool2x2_nhwc"]
-    assert as_ptr(gathers[0]["args"][13]) == 0                       # conv1_1 reads the image
-    has_bias = [as_ptr(g["args"][13]) != 0 for g in gathers]
-    # conv after conv carries the bias; conv after a pool does not (the pool applied it)
-    assert has_bias == [False, True, False, True, False, True, True, False, True, True, False, True, True]
+    assert gathers[0]["key"] == "im2col_nhwc_f16" and as_ptr(gathers[0]["args"][13]) == 0   # conv1_1 reads the image
+    has_bias = [as_ptr(g["args"][13 if g["key"] == "im2col_nhwc_f16" else 7]) != 0 for g in gathers]
+    # every convolution but the first applies its predecessor's bias, through the pooling or not
+    assert has_bias == [False] + [True] * 12
+    pooled = [as_int(g["args"][9]) for g in gathers[1:]]
+    assert pooled == [0, 1, 0, 1, 0, 0, 1, 0, 0, 1, 0, 0]
     assert all(as_ptr(p["args"][5]) != 0 and as_int(p["args"][6]) == 1 for p in pools)
 
 
