@@ -71,3 +71,35 @@ def mriq_inputs(numK, numX, seed=1337):
 
 C0 = float(np.float32(1.0 / 6.0))
 C1 = float(np.float32(1.0 / 6.0 / 6.0))
+
+
+# ---- launching a kernel of the registry by key (the device layer of include/tacker_amd.h) ----
+import ctypes as _C
+
+_registry = {}
+
+
+class _Dim3(_C.Structure):
+    _fields_ = [("x", _C.c_uint), ("y", _C.c_uint), ("z", _C.c_uint)]
+
+
+def registry():
+    """key -> device function handle, as tk_register_kernels hands them out."""
+    if not _registry:
+        lib = ta.lib()
+        cb_t = _C.CFUNCTYPE(None, _C.c_char_p, _C.c_void_p, _C.c_void_p)
+        cb = cb_t(lambda key, func, ctx: _registry.__setitem__(key.decode(), func))
+        lib.tk_register_kernels.argtypes = [cb_t, _C.c_void_p]
+        assert lib.tk_register_kernels(cb, None) == 0
+        lib.tkLaunchKernel.argtypes = [_C.c_void_p, _Dim3, _Dim3, _C.POINTER(_C.c_void_p), _C.c_size_t, _C.c_void_p]
+    return _registry
+
+
+def launch(key, grid, block, args):
+    """args: ctypes values (c_int, c_float, c_void_p ...), in the kernel's parameter order."""
+    func = registry()[key]
+    holders = list(args)
+    ptrs = (_C.c_void_p * len(holders))(*[_C.cast(_C.pointer(a), _C.c_void_p) for a in holders])
+    rc = ta.lib().tkLaunchKernel(func, _Dim3(grid, 1, 1), _Dim3(block, 1, 1), ptrs, 0,
+                                 torch.cuda.current_stream().cuda_stream)
+    assert rc == 0, rc

@@ -76,6 +76,44 @@ def test_vgg16_layers_match_direct_convolution():
     task.close()
 
 
+@pytest.mark.parametrize("H,W,C,cs,pool", [(5, 7, 8, 8, 0), (8, 8, 64, 128, 0), (14, 14, 24, 32, 0), (3, 3, 16, 16, 0),
+                                           (1, 1, 8, 8, 0), (2, 9, 40, 44, 0), (4, 6, 16, 128, 1), (7, 7, 64, 64, 1),
+                                           (1, 2, 8, 12, 1)])
+def test_scattered_conv_operand_equals_the_gathered_one(H, W, C, cs, pool):
+    # A[m][(kh*3+kw)*C + c] built by scattering each pixel to the rows whose window covers it must be,
+    # bit for bit, what the gather form builds -- including the zeros of border taps and of the columns
+    # past 9*C, in a buffer that held something else before; with pool, what pooling first and gathering
+    # from the pooled activations gives
+    import ctypes as C_
+    from gpu_util import launch
+    rng = np.random.default_rng(H * 100 + W * 10 + C + pool)
+    Hin, Win = (2 * H, 2 * W) if pool else (H, W)
+    act = rng.uniform(-1, 1, (Hin, Win, cs)).astype(np.float32)
+    bias = rng.uniform(-0.5, 0.5, cs).astype(np.float32)
+    Kp = -(-9 * C // 128) * 128
+    rows = H * W
+    d_act, d_bias = dev(act), dev(bias)
+    ptr = lambda t: C_.c_void_p(t.data_ptr())
+    i = C_.c_int
+    gathered = torch.zeros((rows, Kp), dtype=torch.float16, device="cuda:0")
+    if pool:
+        pooled = torch.zeros((H, W, cs), dtype=torch.float32, device="cuda:0")
+        launch("maxpool2x2_nhwc", 64, 256, [ptr(d_act), i(Hin), i(Win), i(cs), ptr(pooled), ptr(d_bias), i(1)])
+        launch("im2col_nhwc_f16", 64, 256, [ptr(pooled), i(H), i(W), i(C), i(cs), i(3), i(3), i(1), i(1), i(H), i(W),
+                                            ptr(gathered), i(Kp), C_.c_void_p(0), i(1)])
+    else:
+        launch("im2col_nhwc_f16", 64, 256, [ptr(d_act), i(H), i(W), i(C), i(cs), i(3), i(3), i(1), i(1), i(H), i(W),
+                                            ptr(gathered), i(Kp), ptr(d_bias), i(1)])
+    scattered = torch.full((rows, Kp), 777.0, dtype=torch.float16, device="cuda:0")
+    launch("im2col3x3_scatter_nhwc_f16", 64, 256, [ptr(d_act), i(H), i(W), i(C), i(cs), ptr(scattered), i(Kp),
+                                                   ptr(d_bias), i(1), i(pool)])
+    torch.cuda.synchronize()
+    g = gathered.cpu().numpy().view(np.uint16)
+    s_ = scattered.cpu().numpy().view(np.uint16)
+    assert np.array_equal(g, s_)
+    assert np.any(g[:, :9 * C] != 0) and np.all(g[:, 9 * C:] == 0)
+
+
 def test_task_manager_colocation_keeps_lc_results_and_reports():
     task = ta.LcTask("vgg16", 64, 64)
     task.execute()
