@@ -1,4 +1,4 @@
-"""GPU parity at the benchmark's full sizes (configs 2, 3 and 4), through the C-ABI.
+"""GPU parity at the benchmark's full sizes (configs 2 to 5), through the C-ABI.
 
 The oracle runs where it finishes in seconds (stencil sweeps, one lbm step, row samples of
 the GEMM, voxel samples of mri-q); what it cannot cover is checked through properties that
@@ -176,3 +176,46 @@ def test_config4_mriq_spread_over_nine_fused_launches_equals_one_launch():
     assert np.array_equal(host(Qr), host(solo_r)) and np.array_equal(host(Qi), host(solo_i))
     assert np.array_equal(host(mix_c), host(solo_c))
     assert ta.spin_fail_flag() == 0
+
+
+def test_config5_vgg16_224_colocated_queries_equal_the_solo_query():
+    # VGG16 batch 1 at 224x224 under TaskManager, once with the reference's always-fuse policy and the
+    # kinfo block counts (every mixable layer carries stencil blocks), once with calibrated counts and
+    # mri-q: whatever rides along, the logits are the solo query's bit for bit, no role barrier was
+    # abandoned, and the latencies are inside the budget.  The deep layers take the shared-reduction
+    # form of the GEMM here (conv4, conv5, fc: 2 to 8 workgroups per tile).
+    task = ta.LcTask("vgg16")
+    shapes = [k["args"] for k in task.kernels() if k["mixable"]]
+    assert len(shapes) == 16
+    assert ta.tzgemm_parts(14 * 14, 512, 9 * 512) == 8 and ta.tzgemm_parts(4096, 128, 25088) == 2
+    task.execute()
+    torch.cuda.synchronize()
+    p, stride, n = task.logits()
+    solo = ta.device_to_host(p, (n, stride), np.float32)[:, 0].copy()
+    assert np.isfinite(solo).all() and np.abs(solo).max() > 0
+    for _ in range(3):                                   # the query is reproducible
+        task.execute()
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo)
+
+    tm = ta.TaskManager(task, "stencil", "lbm")
+    tm.configure(qos_budget_ms=50.0, guard_ms=4.0, warmup=2, profile=5, queries=20, verbose=0)
+    tm.set_fusion_strikes(0)                             # the reference's loop: fuse whenever the budget allows
+    rep = tm.run("aker", second_stage=False)
+    torch.cuda.synchronize()
+    assert rep["mix_times"] > 0 and rep["be_blocks_executed"] > 0
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo)
+    assert all(0 < v < 50.0 for v in tm.latencies())
+    tm.close()
+
+    tm = ta.TaskManager(task, "mriq", "lbm")
+    tm.configure(qos_budget_ms=50.0, guard_ms=4.0, warmup=2, profile=5, queries=20, verbose=0)
+    tm.set_calibration(True, 0.10)
+    rep = tm.run("aker", second_stage=False)
+    torch.cuda.synchronize()
+    assert len(tm.calibrated_blocks()) >= 16
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo)
+    assert all(0 < v < 50.0 for v in tm.latencies())
+    assert ta.spin_fail_flag() == 0
+    tm.close()
+    task.close()
