@@ -59,13 +59,15 @@ float *randomBias(std::vector<void *> &freeList, tk::Rng &rng, int n, int n_pad)
 // Shared GEMM machinery of conv and FC layers: persistent objects built once.
 class GemmLayer : public LcGemmKernel {
 public:
-    GemmLayer(int id, const std::string &name, int M, int N, int K, const void *A, const void *B, float *C)
+    // tile_end > 0: only the reference tiles [0, tile_end) are computed (the others would be padding)
+    GemmLayer(int id, const std::string &name, int M, int N, int K, const void *A, const void *B, float *C,
+              int tile_end = 0)
         : M_(M), N_(N), K_(K)
     {
         this->Id = id;
         this->kernelName = name;
         ori_.reset(new OriTZGEMMKernel(id, M, N, K, A, B, C));
-        tiles_ = getTZGEMMGridDim(M, N, K)[3];
+        tiles_ = tile_end > 0 ? tile_end : getTZGEMMGridDim(M, N, K)[3];
         gptb_.reset(new GPTBKernel(id, "tzgemm", "gptb_tzgemm", ori_.get(), dim3(cuCount(), 1, 1),
                                    dim3(TZ_THREADS, 1, 1), 0, tiles_));
     }
@@ -138,11 +140,17 @@ private:
 
 class FcKernel : public GemmLayer {
 public:
-    // C[out_pad][128] = W[out_pad][K] * X[128][K]^T; x comes from src (stride src_stride)
+    // C[128][out_pad] = X[128][K] * W[out_pad][K]^T with the batch-1 activation in row 0 of X, taken
+    // from src with stride src_stride.  The activation is the M side so that the reference tiles that
+    // hold the result, row 0 .. 63 of C, are the first out_pad / 64 of the tile order: only those are
+    // launched, every one of them streams weights nobody else reads, and rows 64 .. 127 of C (all
+    // padding) stay as allocated.
     FcKernel(int id, const std::string &name, const float *src, long src_stride, const float *src_bias,
              int src_relu, int in_features, int out_features, const void *Wt, void *X, float *out)
-        : GemmLayer(id, name, pad128(out_features), 128, pad128(in_features), Wt, X, out), src_(src),
-          stride_(src_stride), bias_(src_bias), relu_(src_relu), in_(in_features), out_(out_features), X_(X)
+        : GemmLayer(id, name, 128, pad128(out_features), pad128(in_features), X, Wt, out,
+                    pad128(out_features) / TZ_REF_TILE),
+          src_(src), stride_(src_stride), bias_(src_bias), relu_(src_relu), in_(in_features), out_(out_features),
+          X_(X)
     {
         this->mixable = 1;
     }
@@ -286,7 +294,7 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
         ld = Np;
     }
     // classifier: 512*(H/32)*(W/32) -> 4096 -> 4096 -> classes; activations travel as
-    // column 0 of the previous FC output, bias+ReLU applied while packing the next input
+    // row 0 of the previous FC output, bias+ReLU applied while packing the next input
     const int feat = H * W * C;   // NHWC flatten (ld == C == 512 here)
     void *X1 = nullptr, *X2 = nullptr, *X3 = nullptr;
     auto halfBuf = [&](void **p, size_t n) {
@@ -301,13 +309,13 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
     void *W2 = randomHalfMatrix(fl, rng, 4096, 4096, 4096, 4096, std::sqrt(2.0f / 4096));
     void *W3 = randomHalfMatrix(fl, rng, opt.classes, 4096, pad128(opt.classes), 4096, std::sqrt(2.0f / 4096));
     float *b1 = randomBias(fl, rng, 4096, 4096), *b2 = randomBias(fl, rng, 4096, 4096);
-    float *o1 = devAlloc(fl, (size_t)4096 * 128), *o2 = devAlloc(fl, (size_t)4096 * 128);
-    float *o3 = devAlloc(fl, (size_t)pad128(opt.classes) * 128);
+    float *o1 = devAlloc(fl, (size_t)128 * 4096), *o2 = devAlloc(fl, (size_t)128 * 4096);
+    float *o3 = devAlloc(fl, (size_t)128 * pad128(opt.classes));
     addKernel(new FcKernel(id++, "Dot_fc1", act, 1, nullptr, 0, feat, 4096, W1, X1, o1));
-    addKernel(new FcKernel(id++, "Dot_fc2", o1, 128, b1, 1, 4096, 4096, W2, X2, o2));
-    addKernel(new FcKernel(id++, "Dot_fc3", o2, 128, b2, 1, 4096, opt.classes, W3, X3, o3));
+    addKernel(new FcKernel(id++, "Dot_fc2", o1, 1, b1, 1, 4096, 4096, W2, X2, o2));
+    addKernel(new FcKernel(id++, "Dot_fc3", o2, 1, b2, 1, 4096, opt.classes, W3, X3, o3));
     impl->logits = o3;
-    impl->logitsStride = 128;
+    impl->logitsStride = 1;
 }
 
 VGG16::~VGG16()

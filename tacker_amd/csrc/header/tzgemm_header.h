@@ -58,7 +58,11 @@ TZ_HOST_DEVICE inline int tz_ksplit_parts(int M, int N, int K)
 {
     if (!tz_use_ksplit(M, N, K)) return 1;
     const int n_ref = (M / TZ_REF_TILE) * (N / TZ_REF_TILE);
-    int parts = TZ_KSPLIT_TARGET_WORKGROUPS / n_ref;
+    // M at its minimum of 128 is a batch padded up (a fully-connected layer at batch 1 .. 64): the
+    // caller launches the tile row that holds its batch, half of the tiles, and the parts are sized
+    // for that half
+    const int launched = M == TZ_MACRO_TILE ? n_ref / 2 : n_ref;
+    int parts = TZ_KSPLIT_TARGET_WORKGROUPS / launched;
     const int by_k = (K / TZ_BLOCK_K) / TZ_KSPLIT_MIN_CHUNKS_PER_PART;
     if (parts > by_k) parts = by_k;
     if (parts > TZ_KSPLIT_MAX_PARTS) parts = TZ_KSPLIT_MAX_PARTS;

@@ -101,7 +101,8 @@ def test_tzgemm_several_tiles_per_workgroup_equal_one_tile_per_workgroup(M, N, K
 # batch-1 layers of VGG16: conv5, conv4, fc2, fc3 with 8, 2, 2, 8 parts).  Who stores C is decided by
 # arrival order, what is stored is not: every launch -- whatever its grid, however its range is cut --
 # must give the same bits, and the arrival counters must be back at zero for the next one.
-@pytest.mark.parametrize("M,N,K", [(256, 512, 4608), (896, 512, 4608), (4096, 128, 4096), (1024, 128, 4096)])
+@pytest.mark.parametrize("M,N,K", [(256, 512, 4608), (896, 512, 4608), (4096, 128, 4096), (1024, 128, 4096),
+                                   (128, 4096, 4096), (128, 1024, 4096)])
 def test_tzgemm_reduction_shared_by_workgroups(M, N, K):
     parts = ta.tzgemm_parts(M, N, K)
     assert parts > 1 and ta.tzgemm_workspace_bytes(M, N, K) >= (M // 64) * (N // 64) * parts * 64 * 64 * 4

@@ -134,6 +134,7 @@ def test_tzgemm_parts_rule(fake):
     fake.tacker_tzgemm_workspace_bytes.restype = C.c_longlong
     want = {(2048, 2048, 2048): 1, (3200, 256, 2304): 1, (896, 512, 4608): 2, (256, 512, 4608): 8,
             (4096, 128, 25088): 2, (4096, 128, 4096): 2, (1024, 128, 4096): 8, (128, 128, 512): 1,
+            (128, 4096, 25088): 4, (128, 4096, 4096): 4, (128, 1024, 4096): 8,   # M = 128: half the tiles are launched
             (128, 128, 1024): 2, (128, 128, 128): 1, (196, 512, 4608): 8}
     for (m, n, k), parts in want.items():
         assert fake.tacker_tzgemm_parts(m, n, k) == parts, (m, n, k)
@@ -402,7 +403,7 @@ def test_vgg16_task_structure(small_vgg):
     assert len(convs) == 13 and len(fcs) == 3 and len([k for k in ks if "MaxPool" in k["name"]]) == 1
     assert convs[0]["args"] == [1, 3, 32, 32, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1]
     assert convs[-1]["args"] == [1, 512, 2, 2, 512, 512, 3, 3, 1, 1, 1, 1, 1, 1]
-    assert [k["args"] for k in fcs] == [[4096, 128, 512], [4096, 128, 4096], [1024, 128, 4096]]
+    assert [k["args"] for k in fcs] == [[128, 4096, 512], [128, 4096, 4096], [128, 1024, 4096]]
     assert ta.LcTask.__init__  # keep the class referenced
 
 
