@@ -406,12 +406,6 @@ __device__ __forceinline__ int tz_ksplit_unit_of(int role_block, int role_blocks
     return role_block;
 }
 
-// Partial tiles travel between workgroups on other XCDs, whose L2s do not see each other's
-// lines.  Every access to them is an agent-scope access of its own (it goes through to the
-// memory side both XCDs share), so no cache has to be written back or dropped as a whole.
-// A partial tile is 16 blocks of 64 x float4 (block = i * 4 + j of the accumulator set),
-// stored as two 8-byte halves per lane: [block][half][lane].
-typedef unsigned long long tz_u64;
 // The same value, but one the compiler has to take as computed here: addresses derived from it
 // are formed where they are used instead of being kept in registers across the K loop (the
 // sixteen block offsets of a partial tile, hoisted out of the tile loop, do not fit beside the
@@ -421,6 +415,13 @@ __device__ __forceinline__ int tz_opaque(int v)
     asm volatile("" : "+v"(v));
     return v;
 }
+
+// Partial tiles travel between workgroups on other XCDs, whose L2s do not see each other's
+// lines.  Every access to them is an agent-scope access of its own (it goes through to the
+// memory side both XCDs share), so no cache has to be written back or dropped as a whole.
+// A partial tile is 16 blocks of 64 x float4 (block = i * 4 + j of the accumulator set),
+// stored as two 8-byte halves per lane: [block][half][lane].
+typedef unsigned long long tz_u64;
 __device__ __forceinline__ void tz_partial_store(tz_u64 *tile, int block, int lane, float4_t v)
 {
     union { float4_t f; tz_u64 q[2]; } u;
