@@ -133,6 +133,27 @@ def test_tzgemm_reduction_shared_by_workgroups(M, N, K):
     assert np.array_equal(got[~mask], want[~mask]) and np.array_equal(got[mask], first[mask])
 
 
+def test_tzgemm_shared_reduction_never_reads_a_previous_launch():
+    # the workspace keeps the partial tiles of the last launch; a launch on other operands must not
+    # see any of them (they were written and are read across the XCDs' separate L2s).  The witnesses
+    # are first launches into output buffers of their own: their workspaces are new and zeroed.
+    M, N, K = 256, 512, 4608
+    ta.tzgemm_release_workspaces()
+    dev_pairs = [tuple(dev(x) for x in gemm_inputs(M, N, K, seed=900 + i)) for i in range(4)]
+    witnesses = []
+    for dA, dB in dev_pairs:
+        out = torch.zeros((M, N), device="cuda:0")      # kept alive: four different addresses
+        ta.gptb_tzgemm(dA, dB, out)
+        witnesses.append(out)
+    want = [host(w).view(np.uint32).copy() for w in witnesses]
+    assert not np.array_equal(want[0], want[1])
+    used = torch.zeros((M, N), device="cuda:0")
+    for rounds in range(3):
+        for i, (dA, dB) in enumerate(dev_pairs):
+            ta.gptb_tzgemm(dA, dB, used, launch_grid=(0, 64, 256)[rounds])
+            assert np.array_equal(host(used).view(np.uint32), want[i]), (rounds, i)
+
+
 def test_tzgemm_shared_reductions_on_two_streams_do_not_meet():
     # each output buffer has a workspace of its own, so GEMMs of the same shape that run at the same
     # time on different streams cannot draw each other's tickets
