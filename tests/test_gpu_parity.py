@@ -154,6 +154,46 @@ def test_tzgemm_shared_reduction_never_reads_a_previous_launch():
             assert np.array_equal(host(used).view(np.uint32), want[i]), (rounds, i)
 
 
+@pytest.mark.parametrize("M,N,K", [(256, 512, 4608), (128, 4096, 4096)])
+def test_tzgemm_shared_reduction_under_traffic(M, N, K):
+    # changing operands, launch grids, ranges cut in three, fused launches, and a sweep of the stencil on
+    # another stream keeping HBM and the L2s busy: every result equals the witness of its operands
+    rng = np.random.default_rng(M + N)
+    ta.tzgemm_release_workspaces()
+    pairs = [tuple(dev(x) for x in gemm_inputs(M, N, K, seed=50 + i)) for i in range(3)]
+    witnesses = []
+    for dA, dB in pairs:
+        out = torch.zeros((M, N), device="cuda:0")
+        ta.gptb_tzgemm(dA, dB, out)
+        witnesses.append(out)
+    torch.cuda.synchronize()
+    A0 = dev(stencil_inputs(64, 256, 512, seed=2))
+    A1 = A0.clone()
+    side = torch.cuda.Stream(device="cuda:0")
+    used = torch.zeros((M, N), device="cuda:0")
+    tiles = (M // 64) * (N // 64)
+    for it in range(48):
+        i = int(rng.integers(0, 3))
+        grid = int(rng.choice([0, 8, 40, 96, 256, 304]))
+        dA, dB = pairs[i]
+        if it % 3 == 0:
+            ta.gptb_stencil(C0, C1, A0, A1, stream=side)
+        if it % 4 == 1:
+            t0 = int(rng.integers(0, tiles))
+            t1 = int(rng.integers(t0, tiles + 1))
+            used.fill_(0)
+            ta.gptb_tzgemm(dA, dB, used, tile_start=0, tile_end=t0, launch_grid=grid)
+            ta.gptb_tzgemm(dA, dB, used, tile_start=t1, tile_end=tiles, launch_grid=grid)
+            ta.gptb_tzgemm(dA, dB, used, tile_start=t0, tile_end=t1, launch_grid=grid)
+        elif it % 4 == 2:
+            ta.mix_tzgemm_stencil(C0, C1, A0, A1, dA, dB, used, be_start=0, be_end=int(rng.integers(0, 256)))
+        else:
+            ta.gptb_tzgemm(dA, dB, used, launch_grid=grid)
+        assert torch.equal(used.view(torch.int32), witnesses[i].view(torch.int32)), (it, i, grid)
+    torch.cuda.synchronize()
+    assert ta.spin_fail_flag() == 0
+
+
 def test_tzgemm_shared_reductions_on_two_streams_do_not_meet():
     # each output buffer has a workspace of its own, so GEMMs of the same shape that run at the same
     # time on different streams cannot draw each other's tickets
