@@ -145,12 +145,15 @@ public:
     // hold the result, row 0 .. 63 of C, are the first out_pad / 64 of the tile order: only those are
     // launched, every one of them streams weights nobody else reads, and rows 64 .. 127 of C (all
     // padding) stay as allocated.
+    // pool_W > 0: src is the raw output of the last convolution, [.][pool_W][pool_ld] with pool_C
+    // channels, and the 2x2 max pooling in front of the classifier happens while the row is packed
     FcKernel(int id, const std::string &name, const float *src, long src_stride, const float *src_bias,
-             int src_relu, int in_features, int out_features, const void *Wt, void *X, float *out)
+             int src_relu, int in_features, int out_features, const void *Wt, void *X, float *out,
+             int pool_W = 0, int pool_ld = 0, int pool_C = 0)
         : GemmLayer(id, name, 128, pad128(out_features), pad128(in_features), X, Wt, out,
                     pad128(out_features) / TZ_REF_TILE),
           src_(src), stride_(src_stride), bias_(src_bias), relu_(src_relu), in_(in_features), out_(out_features),
-          X_(X)
+          X_(X), poolW_(pool_W), poolLd_(pool_ld), poolC_(pool_C)
     {
         this->mixable = 1;
     }
@@ -159,6 +162,11 @@ public:
 protected:
     void before(cudaStream_t stream) override
     {
+        if (poolW_ > 0) {
+            void *args[] = {&src_, &poolW_, &poolLd_, &poolC_, &bias_, &relu_, &in_, &X_};
+            launch1d("pack_fc_input_pooled", in_, args, stream);
+            return;
+        }
         void *args[] = {&src_, &stride_, &bias_, &relu_, &in_, &X_};
         launch1d("pack_fc_input", in_, args, stream);
     }
@@ -169,44 +177,7 @@ private:
     const float *bias_;
     int relu_, in_, out_;
     void *X_;
-};
-
-class SimpleKernel : public Kernel {
-public:
-    SimpleKernel(int id, const std::string &name, const char *key, long work) : key_(key), work_(work)
-    {
-        this->Id = id;
-        this->kernelName = name;
-        this->mixable = 0;
-    }
-    void initParams() override {}
-    void loadKernel() override {}
-    std::vector<int> getArgs() override { return {}; }
-    std::vector<void *> argStore;   // owns nothing; points at the members below
-
-protected:
-    void executeImpl(cudaStream_t stream) override { launch1d(key_, work_, argStore.data(), stream); }
-    const char *key_;
-    long work_;
-};
-
-class PoolKernel : public SimpleKernel {
-public:
-    // in_bias != nullptr: in is the raw output of the previous convolution; its bias and ReLU
-    // are applied to the pooled value
-    PoolKernel(int id, const std::string &name, const float *in, const float *in_bias, int H, int W, int ld,
-               float *out)
-        : SimpleKernel(id, name, "maxpool2x2_nhwc", (long)(H / 2) * (W / 2) * ld), in_(in), bias_(in_bias),
-          H_(H), W_(W), ld_(ld), out_(out)
-    {
-        argStore = {&in_, &H_, &W_, &ld_, &out_, &bias_, &relu_};
-    }
-
-private:
-    const float *in_;
-    const float *bias_;
-    int H_, W_, ld_, relu_ = 1;
-    float *out_;
+    int poolW_, poolLd_, poolC_;
 };
 
 }  // namespace
@@ -257,22 +228,17 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
     const float *act_bias = nullptr;   // bias the reader of act still has to apply
     int id = 100;
     const int plan[] = {64, 64, -1, 128, 128, -1, 256, 256, 256, -1, 512, 512, 512, -1, 512, 512, 512, -1};
-    // A pooling layer between two convolutions is not a kernel either: the next convolution's
-    // operand is built from the 2x2 maxima.  Only the last one, which feeds the classifier, is.
+    // A pooling layer is not a kernel either: the next convolution's operand, or the classifier's
+    // input row, is built from the 2x2 maxima.
     bool pooled = false;
+    int unpooled_W = 0;   // width of the raw convolution output a pending pooling reads
     int block = 1, layer = 1;
     const int n_plan = (int)(sizeof(plan) / sizeof(plan[0]));
     for (int step = 0; step < n_plan; ++step) {
         const int p = plan[step];
         if (p < 0) {
-            if (step + 1 < n_plan) {
-                pooled = true;
-            } else {
-                float *out = devAlloc(fl, (size_t)(H / 2) * (W / 2) * ld);
-                addKernel(new PoolKernel(id++, "MaxPool_" + std::to_string(block), act, act_bias, H, W, ld, out));
-                act = out;
-                act_bias = nullptr;
-            }
+            pooled = true;
+            unpooled_W = W;
             H /= 2;
             W /= 2;
             block++;
@@ -311,7 +277,8 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
     float *b1 = randomBias(fl, rng, 4096, 4096), *b2 = randomBias(fl, rng, 4096, 4096);
     float *o1 = devAlloc(fl, (size_t)128 * 4096), *o2 = devAlloc(fl, (size_t)128 * 4096);
     float *o3 = devAlloc(fl, (size_t)128 * pad128(opt.classes));
-    addKernel(new FcKernel(id++, "Dot_fc1", act, 1, nullptr, 0, feat, 4096, W1, X1, o1));
+    // act is conv5_3's raw output; its pooling, bias and ReLU happen while fc1's input is packed
+    addKernel(new FcKernel(id++, "Dot_fc1", act, 1, act_bias, 1, feat, 4096, W1, X1, o1, pooled ? unpooled_W : 0, ld, C));
     addKernel(new FcKernel(id++, "Dot_fc2", o1, 1, b1, 1, 4096, 4096, W2, X2, o2));
     addKernel(new FcKernel(id++, "Dot_fc3", o2, 1, b2, 1, 4096, opt.classes, W3, X3, o3));
     impl->logits = o3;

@@ -252,3 +252,27 @@ extern "C" __global__ void pack_fc_input(const float *src, long src_stride, cons
         x_row[i] = (_Float16)v;
     }
 }
+
+// The same row from the raw output of the last convolution, [2*Ho][W][ld] with C channels used, through
+// the 2x2 max pooling that precedes the classifier: element i = (ho*Wo + wo)*C + c of the NHWC
+// flattening is the maximum of its 2x2 cell, then + bias[c], then ReLU -- the operations of
+// maxpool2x2_nhwc followed by pack_fc_input, in their order.
+extern "C" __global__ void pack_fc_input_pooled(const float *in, int W, int ld, int C, const float *bias,
+                                                int relu, int n, _Float16 *x_row)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int c = i % C;
+        const int p = i / C;
+        const int Wo = W / 2;
+        const int wo = p % Wo, ho = p / Wo;
+        const float *src = in + ((long)(2 * ho) * W + 2 * wo) * ld + c;
+        const float a = src[0], b = src[ld], d = src[(long)W * ld], e = src[(long)W * ld + ld];
+        float v = fmaxf(fmaxf(a, b), fmaxf(d, e));
+        if (bias) {
+            v += bias[c];
+            if (relu && v < 0.0f) v = 0.0f;
+        }
+        x_row[i] = (_Float16)v;
+    }
+}

@@ -197,6 +197,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("bias_relu_rows", (const void *)bias_relu_rows, ctx);
     insert("maxpool2x2_nhwc", (const void *)maxpool2x2_nhwc, ctx);
     insert("pack_fc_input", (const void *)pack_fc_input, ctx);
+    insert("pack_fc_input_pooled", (const void *)pack_fc_input_pooled, ctx);
     tk_register_mix_kernels(insert, ctx);
     return TK_SUCCESS;
 }

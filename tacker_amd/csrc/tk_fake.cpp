@@ -177,6 +177,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("bias_relu_rows", {P, P, I, I, I});
         add("maxpool2x2_nhwc", {P, I, I, I, P, P, I});
         add("pack_fc_input", {P, 8, P, I, I, P});
+        add("pack_fc_input_pooled", {P, I, I, I, P, I, I, P});
         const std::pair<const char *, const std::vector<int> *> bes[] = {
             {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}};
         static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};

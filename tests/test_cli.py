@@ -40,7 +40,7 @@ def check_session(p, cwd):
     text = open(os.path.join(cwd, "recorder_output.txt")).read().split("\n")
     assert text[0] == "taskID: 1, taskName: vgg16"
     rows = [l for l in text if l.startswith("    kernelID: ")]
-    assert len(rows) == 17                                                       # 13 conv + the last pool + 3 fc
+    assert len(rows) == 16                                                       # 13 conv + 3 fc (pooling rides with their inputs)
     for l in rows:
         assert re.fullmatch(r"    kernelID: \d+, kernelName: \w+, execTime: [-+.e\d]+ms", l), l
     assert rows[0].startswith("    kernelID: 100, kernelName: Convolution_conv1_1, execTime: ")

@@ -114,6 +114,31 @@ def test_scattered_conv_operand_equals_the_gathered_one(H, W, C, cs, pool):
     assert np.any(g[:, :9 * C] != 0) and np.all(g[:, 9 * C:] == 0)
 
 
+@pytest.mark.parametrize("H,W,C,ld", [(14, 14, 512, 512), (4, 6, 24, 32), (2, 2, 8, 8)])
+def test_pooled_classifier_input_equals_pooling_then_packing(H, W, C, ld):
+    import ctypes as C_
+    from gpu_util import launch
+    rng = np.random.default_rng(H + W + C)
+    raw = dev(rng.uniform(-1, 1, (H, W, ld)).astype(np.float32))
+    bias = dev(rng.uniform(-0.5, 0.5, ld).astype(np.float32))
+    n = (H // 2) * (W // 2) * C
+    ptr = lambda t: C_.c_void_p(t.data_ptr())
+    i = C_.c_int
+    pooled = torch.zeros((H // 2, W // 2, ld), dtype=torch.float32, device="cuda:0")
+    launch("maxpool2x2_nhwc", 64, 256, [ptr(raw), i(H), i(W), i(ld), ptr(pooled), ptr(bias), i(1)])
+    want = torch.zeros(n, dtype=torch.float16, device="cuda:0")
+    if ld == C:      # the packing kernel walks a dense vector: the pooled map flattens to one when ld == C
+        launch("pack_fc_input", (n + 255) // 256, 256, [ptr(pooled), C_.c_long(1), C_.c_void_p(0), i(0), i(n), ptr(want)])
+        want_bits = want.cpu().numpy().view(np.uint16)
+    else:
+        want_bits = pooled.cpu().numpy()[:, :, :C].reshape(-1).astype(np.float16).view(np.uint16)
+    got = torch.full((n,), 777.0, dtype=torch.float16, device="cuda:0")
+    launch("pack_fc_input_pooled", (n + 255) // 256, 256, [ptr(raw), i(W), i(ld), i(C), ptr(bias), i(1), i(n), ptr(got)])
+    torch.cuda.synchronize()
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), want_bits)
+    assert np.any(want_bits != 0)
+
+
 def test_task_manager_colocation_keeps_lc_results_and_reports():
     task = ta.LcTask("vgg16", 64, 64)
     task.execute()

@@ -400,7 +400,7 @@ def test_vgg16_task_structure(small_vgg):
     ks = small_vgg.kernels()
     convs = [k for k in ks if k["mixable"] == 2]
     fcs = [k for k in ks if k["mixable"] == 1]
-    assert len(convs) == 13 and len(fcs) == 3 and len([k for k in ks if "MaxPool" in k["name"]]) == 1
+    assert len(convs) == 13 and len(fcs) == 3 and len([k for k in ks if "MaxPool" in k["name"]]) == 0
     assert convs[0]["args"] == [1, 3, 32, 32, 64, 3, 3, 3, 1, 1, 1, 1, 1, 1]
     assert convs[-1]["args"] == [1, 512, 2, 2, 512, 512, 3, 3, 1, 1, 1, 1, 1, 1]
     assert [k["args"] for k in fcs] == [[128, 4096, 512], [128, 4096, 4096], [128, 1024, 4096]]
@@ -414,20 +414,20 @@ def test_vgg16_solo_pass_launches_every_layer(fake, small_vgg):
     # the first layer (3 channels) gathers its operand, the others scatter it (activations read once)
     assert keys.count("gptb_tzgemm") == 16 and keys.count("im2col_nhwc_f16") == 1
     assert keys.count("im2col3x3_scatter_nhwc_f16") == 12
-    # pooling between two convolutions happens while the next operand is built; only the pool
-    # in front of the classifier is a launch
-    assert keys.count("maxpool2x2_nhwc") == 1 and keys.count("pack_fc_input") == 3
+    # pooling happens while the next operand (or the classifier's input row) is built
+    assert keys.count("maxpool2x2_nhwc") == 0
+    assert keys.count("pack_fc_input_pooled") == 1 and keys.count("pack_fc_input") == 2
     # no separate bias/ReLU pass: each convolution's bias travels to whatever reads its output next
     assert keys.count("bias_relu_rows") == 0
     gathers = [l for l in launches(fake) if l["key"] in ("im2col_nhwc_f16", "im2col3x3_scatter_nhwc_f16")]
-    pools = [l for l in launches(fake) if l["key"] == "maxpool2x2_nhwc"]
     assert gathers[0]["key"] == "im2col_nhwc_f16" and as_ptr(gathers[0]["args"][13]) == 0   # conv1_1 reads the image
     has_bias = [as_ptr(g["args"][13 if g["key"] == "im2col_nhwc_f16" else 7]) != 0 for g in gathers]
     # every convolution but the first applies its predecessor's bias, through the pooling or not
     assert has_bias == [False] + [True] * 12
     pooled = [as_int(g["args"][9]) for g in gathers[1:]]
     assert pooled == [0, 1, 0, 1, 0, 0, 1, 0, 0, 1, 0, 0]
-    assert all(as_ptr(p["args"][5]) != 0 and as_int(p["args"][6]) == 1 for p in pools)
+    (packed,) = [l for l in launches(fake) if l["key"] == "pack_fc_input_pooled"]
+    assert as_ptr(packed["args"][4]) != 0 and as_int(packed["args"][5]) == 1     # conv5_3's bias, ReLU
 
 
 def run_manager(fake, task, durations=None, **cfg):
