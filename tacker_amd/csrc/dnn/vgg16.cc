@@ -126,8 +126,11 @@ protected:
             launch1d("im2col3x3_scatter_nhwc_f16", (long)H_ * W_ * (C_ / 8), args, stream);
             return;
         }
-        void *args[] = {&act_, &H_, &W_, &C_, &cs_, &KH, &KW, &pad, &stride, &Ho, &Wo, &A_, &Kp, &act_bias_, &relu};
-        launch1d("im2col_nhwc_f16", (long)Ho * Wo * Kp, args, stream);
+        // the first layer (3 channels): an operand buffer of its own, zeroed once, of which only the
+        // columns that hold data are rewritten
+        int Kw = (9 * C_ + 7) / 8 * 8;
+        void *args[] = {&act_, &H_, &W_, &C_, &cs_, &KH, &KW, &pad, &stride, &Ho, &Wo, &A_, &Kp, &act_bias_, &relu, &Kw};
+        launch1d("im2col_nhwc_f16", (long)Ho * Wo * Kw, args, stream);
     }
 
 private:
@@ -250,7 +253,13 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
         void *Wt = randomHalfMatrix(fl, rng, Cout, 9 * C, Np, Kp, std::sqrt(2.0f / (9 * C)));
         float *bias = randomBias(fl, rng, Cout, Np);
         float *out = devAlloc(fl, (size_t)pad128(H * W) * Np);
-        addKernel(new ConvKernel(id++, "Convolution_" + name, act, act_bias, pooled, H, W, C, ld, Cout, Abuf, Wt,
+        void *operand = Abuf;
+        if (C % 8 != 0) {   // gathered, and only its data columns rewritten: needs zeros nobody else disturbs
+            TK_SAFE_CALL(tkMalloc(&operand, (size_t)pad128(H * W) * Kp * 2));
+            TK_SAFE_CALL(tkMemset(operand, 0, (size_t)pad128(H * W) * Kp * 2));
+            fl.push_back(operand);
+        }
+        addKernel(new ConvKernel(id++, "Convolution_" + name, act, act_bias, pooled, H, W, C, ld, Cout, operand, Wt,
                                  out));
         pooled = false;
         impl->convOut.push_back(Act{out, H, W, Cout, Np, Wt, bias, Np, Kp});

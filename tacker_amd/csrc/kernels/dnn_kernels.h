@@ -15,14 +15,16 @@
 // bias != nullptr: act is the raw output of the previous GEMM and its epilogue is applied
 // on the way in, v = act + bias[c], then max(v, 0) if relu -- the values a separate
 // bias/ReLU pass over act would have left there, without that pass.
+// K_write (a multiple of 8, 0 = K_pad): only columns [0, K_write) of each row are written -- for an
+// operand buffer of its own whose columns from K_write on were zeroed once and stay zero.
 extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C, int c_stride,
                                            int KH, int KW, int pad, int stride, int Ho, int Wo,
-                                           _Float16 *A, int K_pad, const float *bias, int relu)
+                                           _Float16 *A, int K_pad, const float *bias, int relu, int K_write)
 {
     typedef float f4 __attribute__((ext_vector_type(4)));
     typedef _Float16 h8 __attribute__((ext_vector_type(8)));
     const int k_real = KH * KW * C;
-    if ((C & 7) == 0 && (c_stride & 3) == 0 && (K_pad & 7) == 0) {
+    if ((C & 7) == 0 && (c_stride & 3) == 0 && (K_pad & 7) == 0 && K_write == 0) {
         // 8 consecutive k share one tap (C is a multiple of 8): two 16-byte loads of the
         // activation, one 16-byte store of A, 32-bit index arithmetic
         const unsigned groups_per_row = (unsigned)K_pad >> 3;
@@ -60,11 +62,11 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
         }
         return;
     }
-    if ((K_pad & 7) == 0 && (long)Ho * Wo * K_pad < (1L << 31)) {
+    if ((K_pad & 7) == 0 && (K_write & 7) == 0 && (long)Ho * Wo * K_pad < (1L << 31)) {
         // any channel count (the first layer has 3): still one 16-byte store of A per thread and
         // 32-bit index arithmetic, the 8 values gathered one by one; groups past the real K
         // (most of the row when C is small) are just zeros
-        const unsigned groups_per_row = (unsigned)K_pad >> 3;
+        const unsigned groups_per_row = (unsigned)(K_write > 0 ? K_write : K_pad) >> 3;
         const unsigned total = (unsigned)(Ho * Wo) * groups_per_row;
         for (unsigned g = blockIdx.x * blockDim.x + threadIdx.x; g < total; g += blockDim.x * gridDim.x) {
             const unsigned m = g / groups_per_row;
@@ -98,7 +100,7 @@ extern "C" __global__ void im2col_nhwc_f16(const float *act, int H, int W, int C
                     }
                 }
             }
-            *reinterpret_cast<h8 *>(A + (size_t)g * 8) = out;
+            *reinterpret_cast<h8 *>(A + (size_t)m * K_pad + k0) = out;
         }
         return;
     }

@@ -100,10 +100,10 @@ def test_scattered_conv_operand_equals_the_gathered_one(H, W, C, cs, pool):
         pooled = torch.zeros((H, W, cs), dtype=torch.float32, device="cuda:0")
         launch("maxpool2x2_nhwc", 64, 256, [ptr(d_act), i(Hin), i(Win), i(cs), ptr(pooled), ptr(d_bias), i(1)])
         launch("im2col_nhwc_f16", 64, 256, [ptr(pooled), i(H), i(W), i(C), i(cs), i(3), i(3), i(1), i(1), i(H), i(W),
-                                            ptr(gathered), i(Kp), C_.c_void_p(0), i(1)])
+                                            ptr(gathered), i(Kp), C_.c_void_p(0), i(1), i(0)])
     else:
         launch("im2col_nhwc_f16", 64, 256, [ptr(d_act), i(H), i(W), i(C), i(cs), i(3), i(3), i(1), i(1), i(H), i(W),
-                                            ptr(gathered), i(Kp), ptr(d_bias), i(1)])
+                                            ptr(gathered), i(Kp), ptr(d_bias), i(1), i(0)])
     scattered = torch.full((rows, Kp), 777.0, dtype=torch.float16, device="cuda:0")
     launch("im2col3x3_scatter_nhwc_f16", 64, 256, [ptr(d_act), i(H), i(W), i(C), i(cs), ptr(scattered), i(Kp),
                                                    ptr(d_bias), i(1), i(pool)])
@@ -112,6 +112,36 @@ def test_scattered_conv_operand_equals_the_gathered_one(H, W, C, cs, pool):
     s_ = scattered.cpu().numpy().view(np.uint16)
     assert np.array_equal(g, s_)
     assert np.any(g[:, :9 * C] != 0) and np.all(g[:, 9 * C:] == 0)
+
+
+@pytest.mark.parametrize("H,W,C,cs", [(9, 11, 3, 3), (6, 5, 3, 4), (4, 4, 5, 8)])
+def test_gathered_operand_with_only_its_data_columns_rewritten(H, W, C, cs):
+    # the first layer's operand: a buffer of its own whose columns past the data were zeroed once; a
+    # gather that rewrites only columns [0, roundup8(9*C)) leaves what a gather of every column leaves,
+    # which for every element is the plain definition A[m][(kh*3+kw)*C + c] = act[h+kh-1][w+kw-1][c]
+    import ctypes as C_
+    from gpu_util import launch
+    rng = np.random.default_rng(H * W + C)
+    act = rng.uniform(-1, 1, (H, W, cs)).astype(np.float32)
+    d_act = dev(act)
+    Kp, Kw = 128, (9 * C + 7) // 8 * 8
+    ptr = lambda t: C_.c_void_p(t.data_ptr())
+    i = C_.c_int
+    outs = []
+    for kw_arg, fill in ((0, 777.0), (Kw, 0.0)):
+        A = torch.full((H * W, Kp), fill, dtype=torch.float16, device="cuda:0")
+        launch("im2col_nhwc_f16", 64, 256, [ptr(d_act), i(H), i(W), i(C), i(cs), i(3), i(3), i(1), i(1), i(H), i(W),
+                                            ptr(A), i(Kp), C_.c_void_p(0), i(0), i(kw_arg)])
+        torch.cuda.synchronize()
+        outs.append(A.cpu().numpy())
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))
+    padded = np.zeros((H + 2, W + 2, C), np.float32)
+    padded[1:-1, 1:-1] = act[:, :, :C]
+    want = np.zeros((H * W, Kp), np.float16)
+    for kh in range(3):
+        for kw in range(3):
+            want[:, (kh * 3 + kw) * C:(kh * 3 + kw + 1) * C] = padded[kh:kh + H, kw:kw + W].reshape(H * W, C).astype(np.float16)
+    assert np.array_equal(outs[0].view(np.uint16), want.view(np.uint16))
 
 
 @pytest.mark.parametrize("H,W,C,ld", [(14, 14, 512, 512), (4, 6, 24, 32), (2, 2, 8, 8)])
