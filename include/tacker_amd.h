@@ -276,6 +276,10 @@ TK_API tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, flo
  * by getTZGEMMGridDim's rule. A == NULL selects the global ori_wmma_* buffers. */
 TK_API tacker_kernel_t tacker_ori_tzgemm_create(const void *A, const void *B, float *C, int m, int n,
                                                 int k);
+/* The global operand buffers ori_wmma_A / _B / _C (src/TaskManager.cu:19-46) as they are now:
+ * device pointers and the bytes allocated for each (they grow when a larger shape is created, so
+ * ask after creating the kernel). A and B hold seeded halves, C is where such kernels write. */
+TK_API int tacker_global_gemm_buffers(const void **A, const void **B, float **C, long long bytes[3]);
 /* new GPTBKernel(id, name, "gptb_<name>", ori, dim3(launch_grid), dim3(launch_block),
  * start, end) (src/GPTBKernel.h:14-70). launch_grid / launch_block 0 = the
  * Creator geometry for this GPU. */

@@ -466,6 +466,14 @@ def ori_tzgemm_create(A, B, Cm, m=None, n=None, k=None):
                         "OriTZGEMMKernel", keep=(A, B, Cm))
 
 
+def global_gemm_buffers():
+    """(A, B, C device addresses, (bytes of A, B, C)) of the global operand buffers."""
+    a, b, c = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    sizes = (C.c_longlong * 3)()
+    check(lib().tacker_global_gemm_buffers(C.byref(a), C.byref(b), C.byref(c), sizes), "global_gemm_buffers")
+    return a.value, b.value, c.value, tuple(sizes)
+
+
 def gptb_create(ori, launch_grid=0, launch_block=0, start=0, end=0):
     return KernelHandle(lib().tacker_gptb_create(ori.handle, launch_grid, launch_block, start, end),
                         "GPTBKernel", keep=(ori,))

@@ -218,6 +218,18 @@ int tacker_tzgemm_release_workspaces(void)
     });
 }
 
+int tacker_global_gemm_buffers(const void **A, const void **B, float **C, long long bytes[3])
+{
+    if (!A || !B || !C || !bytes) return fail(TK_ERROR_INVALID_VALUE, "null output");
+    *A = ori_wmma_A;
+    *B = ori_wmma_B;
+    *C = ori_wmma_C;
+    bytes[0] = MAX_ORI_WMMA_A;
+    bytes[1] = MAX_ORI_WMMA_B;
+    bytes[2] = MAX_ORI_WMMA_C;
+    return TK_SUCCESS;
+}
+
 int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
                        int tile_end, int launch_grid, tkStream_t stream)
 {

@@ -217,6 +217,29 @@ def test_tzgemm_shared_reductions_on_two_streams_do_not_meet():
         assert np.array_equal(host(Cd).view(np.uint32), w.view(np.uint32))
 
 
+def test_tzgemm_on_the_global_operand_buffers():
+    # OriTZGEMMKernel(id, m, n, k) of the reference works on process-wide buffers; here they grow with
+    # the largest shape seen, and the workspace of the shared reductions is a fourth one beside A, B, C.
+    # A shape without a workspace first, then two that need one (the second one larger): each result is
+    # the GEMM of what the buffers hold, and equals the launch on caller-owned copies bit for bit.
+    for (m, n, k) in [(256, 256, 128), (256, 512, 4608), (128, 4096, 4096)]:
+        ori = ta.ori_tzgemm_create(None, None, None, m, n, k)
+        g = ta.gptb_create(ori, 0, 0, 0, (m // 64) * (n // 64))
+        for _ in range(2):
+            g.execute()
+        torch.cuda.synchronize()
+        pa, pb, pc, sizes = ta.global_gemm_buffers()
+        assert sizes[0] >= 2 * m * k and sizes[1] >= 2 * n * k and sizes[2] >= 4 * m * n
+        A = ta.device_to_host(pa, (m, k), np.float16)
+        B = ta.device_to_host(pb, (n, k), np.float16)
+        got = ta.device_to_host(pc, (m, n), np.float32)
+        ok, fro, dmax = gemm_tolerance_ok(got, oracle.tzgemm(A, B, f64=True), k)
+        assert ok and fro <= 1e-5, (m, n, k, fro, dmax)
+        own = torch.zeros((m, n), device="cuda:0")
+        ta.gptb_tzgemm(dev(A), dev(B), own)
+        assert np.array_equal(host(own).view(np.uint32), got.view(np.uint32))
+
+
 def test_tzgemm_shared_reduction_fused_equals_unfused():
     # conv5's shape with a best-effort kernel in the same launch: same bits as the GEMM alone
     M, N, K = 256, 512, 4608
