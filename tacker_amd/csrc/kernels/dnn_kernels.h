@@ -204,18 +204,9 @@ extern "C" __global__ void im2col3x3_scatter_nhwc_f16(const float *act, int H, i
     }
 }
 
-// y[m][n] = max(0, y[m][n] + bias[n]) over rows < M of a [M][ld] matrix
-extern "C" __global__ void bias_relu_rows(float *y, const float *bias, int M, int ld, int relu)
-{
-    const long total = (long)M * ld;
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-         i += (long)blockDim.x * gridDim.x) {
-        float v = y[i] + bias[i % ld];
-        y[i] = (relu && v < 0.0f) ? 0.0f : v;
-    }
-}
-
-// 2x2 / stride 2 max pooling, NHWC with channel stride ld.  bias != nullptr: in is the raw
+// 2x2 / stride 2 max pooling, NHWC with channel stride ld.  The network itself pools while it builds
+// the next operand (im2col3x3_scatter_nhwc_f16, pack_fc_input_pooled); this kernel is the plain
+// statement of what they compute, and what the tests hold them against.  bias != nullptr: in is the raw
 // output of the previous GEMM; out = max(in) + bias[c], then max(., 0) if relu, which is what
 // pooling the biased, rectified values gives (x -> fl(x + b) and ReLU are non-decreasing).
 extern "C" __global__ void maxpool2x2_nhwc(const float *in, int H, int W, int ld, float *out,

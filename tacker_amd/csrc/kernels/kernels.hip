@@ -194,7 +194,6 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);
     insert("im2col_nhwc_f16", (const void *)im2col_nhwc_f16, ctx);
     insert("im2col3x3_scatter_nhwc_f16", (const void *)im2col3x3_scatter_nhwc_f16, ctx);
-    insert("bias_relu_rows", (const void *)bias_relu_rows, ctx);
     insert("maxpool2x2_nhwc", (const void *)maxpool2x2_nhwc, ctx);
     insert("pack_fc_input", (const void *)pack_fc_input, ctx);
     insert("pack_fc_input_pooled", (const void *)pack_fc_input_pooled, ctx);

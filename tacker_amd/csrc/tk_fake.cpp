@@ -174,7 +174,6 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("convert_fp32_to_fp16", {P, P, I});
         add("im2col_nhwc_f16", {P, I, I, I, I, I, I, I, I, I, I, P, I, P, I, I});
         add("im2col3x3_scatter_nhwc_f16", {P, I, I, I, I, P, I, P, I, I});
-        add("bias_relu_rows", {P, P, I, I, I});
         add("maxpool2x2_nhwc", {P, I, I, I, P, P, I});
         add("pack_fc_input", {P, 8, P, I, I, P});
         add("pack_fc_input_pooled", {P, I, I, I, P, I, I, P});

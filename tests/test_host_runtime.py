@@ -418,7 +418,8 @@ def test_vgg16_solo_pass_launches_every_layer(fake, small_vgg):
     assert keys.count("maxpool2x2_nhwc") == 0
     assert keys.count("pack_fc_input_pooled") == 1 and keys.count("pack_fc_input") == 2
     # no separate bias/ReLU pass: each convolution's bias travels to whatever reads its output next
-    assert keys.count("bias_relu_rows") == 0
+    assert set(keys) == {"gptb_tzgemm", "im2col_nhwc_f16", "im2col3x3_scatter_nhwc_f16", "pack_fc_input",
+                         "pack_fc_input_pooled"}
     gathers = [l for l in launches(fake) if l["key"] in ("im2col_nhwc_f16", "im2col3x3_scatter_nhwc_f16")]
     assert gathers[0]["key"] == "im2col_nhwc_f16" and as_ptr(gathers[0]["args"][13]) == 0   # conv1_1 reads the image
     has_bias = [as_ptr(g["args"][13 if g["key"] == "im2col_nhwc_f16" else 7]) != 0 for g in gathers]
