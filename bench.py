@@ -227,6 +227,7 @@ def main():
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the other pairs (configs 3, 4) and the co-location latency leg (config 5)")
     ap.add_argument("--queries", type=int, default=1000, help="latency-critical queries of the co-location leg")
+    ap.add_argument("--no-lc", action="store_true", help="skip the co-location latency legs (config 5)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1",
@@ -342,8 +343,9 @@ def main():
     out["config"]["fused_kernel"] = "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)")
     if not args.no_extras:
         out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq")}
-        out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
-        out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")
+        if not args.no_lc:
+            out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
+            out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(A, B, A0, c0, c1)
     print(json.dumps(out))
