@@ -81,7 +81,7 @@ __device__ __forceinline__ void tz_load_to_lds(const char *uniform_base, unsigne
                  : "memory");
 }
 
-template <int STAGES, class Sync>
+template <int STAGES, bool STREAM_C, class Sync>
 __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A,
                                             const _Float16 *__restrict__ B, float *__restrict__ C,
                                             int M, int N, int K, int role_block, int role_blocks,
@@ -352,7 +352,12 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     float4_t v = acc[i][j] * TZ_ALPHA;
-                    *reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16) = v;
+                    // C is written once and not read again by this kernel: as a streaming store it
+                    // does not push the operand panels the next tiles need out of the L2 (STREAM_C;
+                    // off where the other role of a fused kernel measures better without it)
+                    float4_t *c_at = reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16);
+                    if constexpr (STREAM_C) __builtin_nontemporal_store(v, c_at);
+                    else *c_at = v;
                 }
         }
         // stores and LDS-direct loads share the vmcnt counter: drain it so that the
@@ -617,7 +622,7 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
     sync.finish();
 }
 
-template <int STAGES, class Sync>
+template <int STAGES, bool STREAM_C = true, class Sync>
 __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
                                             float *__restrict__ C, int M, int N, int K, unsigned *workspace,
                                             int role_block, int role_blocks, int tile_start, int tile_end,
@@ -629,7 +634,8 @@ __device__ __forceinline__ void tzgemm_role(const _Float16 *__restrict__ A, cons
         tzgemm_role_ksplit(A, B, C, M, N, K, workspace, role_block, role_blocks, tile_start, tile_end, tid, lds,
                            sync);
     else
-        tzgemm_role_tiles<STAGES>(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds, sync);
+        tzgemm_role_tiles<STAGES, STREAM_C>(A, B, C, M, N, K, role_block, role_blocks, tile_start, tile_end, tid, lds,
+                                            sync);
 }
 
 // Workgroups of a launch of role_blocks that can hold a tile of this GEMM (the first ones, in

@@ -34,13 +34,20 @@ def mix_kernel_name(be, variant):
     return f"{be}_tzgemm_mix_{variant}"
 
 
+def _stream_c(be):
+    """Whether the GEMM role stores C with streaming stores in a kernel fused with ``be``: measured per
+    pair (config 2 with the stencil 34.3 us without, 35.3 us with; the lbm pair 124 us without, 117 us
+    with; no difference for mri-q and cp)."""
+    return "false" if be == "stencil" else "true"
+
+
 def generate_wg_split(be, tz_wgs, be_wgs, threads=256):
     """Workgroup-split fused kernel of ``be`` with tzgemm; tz_wgs : be_wgs per group."""
     variant = f"wg_{tz_wgs}_{be_wgs}"
     p_be, sig_be = signature(be, 0)
     p_tz, sig_tz = signature("tzgemm", 1)
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="sp.role_block", blocks="sp.role_blocks",
-                                             tid="(int)threadIdx.x", stages="TZ_STAGES_WG")
+                                             tid="(int)threadIdx.x", stages="TZ_STAGES_WG", stream_c=_stream_c(be))
     be_call = ROLES[be]["call"].format(p=p_be, block="sp.role_block", blocks="sp.role_blocks",
                                        tid="(int)threadIdx.x", threads=threads, extra="")
     name = mix_kernel_name(be, variant)
@@ -76,7 +83,7 @@ def generate_wave_split(be, be_threads, tz_first=True):
         be_lo, tz_lo = 0, be_threads
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="(int)blockIdx.x",
                                              blocks=f"{p_tz}ptb_iter_block_step",
-                                             tid=f"(int)threadIdx.x - {tz_lo}", stages="TZ_STAGES")
+                                             tid=f"(int)threadIdx.x - {tz_lo}", stages="TZ_STAGES", stream_c=_stream_c(be))
     # few best-effort waves share the CU with the GEMM: lbm takes two rows per wave to keep
     # enough loads in flight
     be_call = ROLES[be]["call"].format(p=p_be, block="be_block", blocks="be_blocks",

@@ -27,7 +27,7 @@ ROLES = {
                    ("unsigned*", "workspace")],
         "needs_sync": True,
         "lds_bytes": "TZ_LDS_BYTES",
-        "call": ("tk::tzgemm_role<{stages}>({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, "
+        "call": ("tk::tzgemm_role<{stages}, {stream_c}>({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, "
                  "{p}workspace, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "tz_lds, sync);"),
     },
