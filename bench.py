@@ -90,6 +90,22 @@ def pair_leg(ta, torch, np, name, stream):
         tz, tiles, flop = gemm(4096, 4096, 1024)
         work = {"bound": "hbm", "algorithmic_bytes": 156.0 * cells}
         label = "configs[2]: tzgemm 4096x4096x1024 + lbm 120x120x150 (one step per launch)"
+    elif name == "mrif":    # mri-fhd, numK 2048, numX 262144 (the reference's tzgemm_mrif mix; no benchmark configuration of its own)
+        numK, numX = 2048, 262144
+        k = rng.uniform(-0.5, 0.5, (numK, 3)).astype(np.float32)
+        phi = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+        d = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+        rho = [torch.zeros(numK, device="cuda:0") for _ in range(2)]
+        ta.mrif_rhophi(*[torch.from_numpy(a).cuda() for a in (phi[0], phi[1], d[0], d[1])], rho[0], rho[1])
+        kv = np.concatenate([k, rho[0].cpu().numpy()[:, None], rho[1].cpu().numpy()[:, None]], 1).astype(np.float32)
+        ta.mrif_set_kvalues(kv)
+        xyz = [torch.from_numpy(rng.uniform(-0.5, 0.5, numX).astype(np.float32)).cuda() for _ in range(3)]
+        outR, outI = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+        be_ori = ta.ori_mrif_create(numK, xyz[0], xyz[1], xyz[2], outR, outI)
+        nblk = ta.mrif_blocks(numK, numX)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "valu", "pairs": float(numK) * numX}
+        label = "tzgemm 2048^3 + mri-fhd numK 2048, numX 262144 (reference mix tzgemm_mrif)"
     else:                   # mri-q, numK 2048, numX 262144
         numK, numX = 2048, 262144
         k = rng.uniform(-0.5, 0.5, (numK, 3)).astype(np.float32)
@@ -148,7 +164,7 @@ def pair_leg(ta, torch, np, name, stream):
     out["be_blocks"] = nblk
     if slice_blocks > 0:
         out["slice_speedup"] = round(out["slice_serial_us"] / out["slice_fused_us"], 4)
-    if name == "mriq":
+    if name in ("mriq", "mrif"):
         # the long best-effort kernel spread over the GEMMs it rides with: n = T_be / T_gemm fused launches,
         # each carrying the next 1/n of the block positions, against n GEMM launches plus the kernel alone
         n_cur = max(1, int(round(out["be_us"] / out["gemm_us"])))
@@ -342,7 +358,7 @@ def main():
     }
     out["config"]["fused_kernel"] = "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)")
     if not args.no_extras:
-        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq")}
+        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq", "mrif")}
         if not args.no_lc:
             out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")

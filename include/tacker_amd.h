@@ -101,8 +101,8 @@ TK_API int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void 
 /* Fills the string-keyed device-function registry (the global `fmap` of
  * src/main.cu:108-159) without the host translation unit including device
  * sources: insert(key, function, ctx) is called once per kernel. Keys on the
- * hot path: ori_{stencil,lbm,mriq,cp}, gptb_{tzgemm,stencil,lbm,mriq,cp},
- * tzgemm_{stencil,lbm,mriq,cp}, plus variant keys "<key>@<variant>". */
+ * hot path: ori_{stencil,lbm,mriq,mrif,cp}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp},
+ * tzgemm_{stencil,lbm,mriq,mrif,cp}, plus variant keys "<key>@<variant>". */
 typedef void (*tk_kernel_insert_fn)(const char *key, const void *func, void *ctx);
 TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx);
 
@@ -186,6 +186,30 @@ TK_API int tacker_gptb_mriq(int numK, const float *x, const float *y, const floa
                             float *Qi, int numX, int block_start, int block_end, int launch_grid,
                             int launch_block, tkStream_t stream);
 
+/* ComputeRhoPhiGPU (src/ori_kernel/mrif_kernel.cu:62-75): RhoPhi = conj(phi) * d per k sample. */
+TK_API int tacker_mrif_rhophi(int numK, const float *phiR, const float *phiI, const float *dR,
+                              const float *dI, float *realRhoPhi, float *imagRhoPhi,
+                              tkStream_t stream);
+/* cudaMemcpyToSymbol(c, ...) (src/ori_kernel/mrif_kernel.cu:304): host table of numK
+ * {Kx,Ky,Kz,RhoPhiR,RhoPhiI} records, numK <= TACKER_MRIF_MAX_K. */
+#define TACKER_MRIF_MAX_K 4096
+TK_API int tacker_mrif_set_kvalues(const float *kvals_host, int numK);
+/* ori_mrif / general_ptb_mrif (src/ori_kernel/mrif_kernel.cu:77-152,
+ * src/gptb_kernel/mrif_kernel.cu:96-170). numX multiple of 256. ori_mrif adds all numK
+ * samples to every voxel (the reference stops after the first grid of 256). Block positions
+ * of the GPTB form are laid out as MRI-Q's: (numX / 256) voxel blocks by
+ * ceil(numK / TACKER_MRIF_K_CHUNK) chunks of the k table, the reference's loop over grids of
+ * the table (mrif_kernel.cu:84-85) as the y index. [0, tacker_mrif_blocks(numK, numX))
+ * equals ori_mrif bit for bit, and so does any sequence of launches whose ranges tile it in
+ * ascending order. */
+#define TACKER_MRIF_K_CHUNK 128
+TK_API int tacker_mrif_blocks(int numK, int numX);
+TK_API int tacker_ori_mrif(int numK, const float *x, const float *y, const float *z, float *outR,
+                           float *outI, int numX, tkStream_t stream);
+TK_API int tacker_gptb_mrif(int numK, const float *x, const float *y, const float *z, float *outR,
+                            float *outI, int numX, int block_start, int block_end, int launch_grid,
+                            int launch_block, tkStream_t stream);
+
 /* copyatomstoconstbuf (src/ori_kernel/cp_kernel.cu:159-179): host array of
  * count (<= 64) {x,y,z,q}; z is replaced by (zplane - z)^2 on the way. */
 TK_API int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane);
@@ -236,6 +260,12 @@ TK_API int tacker_mix_tzgemm_mriq(int numK, const float *x, const float *y, cons
                                   const void *A, const void *B, float *C, int M, int N, int K,
                                   int tile_start, int tile_end, const char *variant,
                                   int launch_grid, int launch_block, tkStream_t stream);
+/* src/mix_kernel/tzgemm_mrif.cu */
+TK_API int tacker_mix_tzgemm_mrif(int numK, const float *x, const float *y, const float *z,
+                                  float *outR, float *outI, int numX, int be_start, int be_end,
+                                  const void *A, const void *B, float *C, int M, int N, int K,
+                                  int tile_start, int tile_end, const char *variant,
+                                  int launch_grid, int launch_block, tkStream_t stream);
 TK_API int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx,
                                 int voly, int be_start, int be_end, const void *A, const void *B,
                                 float *C, int M, int N, int K, int tile_start, int tile_end,
@@ -258,7 +288,7 @@ TK_API float tacker_fget_kernel_info(const char *kernel, const char *key);
 /* ---- object API: the class layer itself, one handle per C++ object ---------- */
 typedef void *tacker_kernel_t;
 
-/* createKernel (src/Creator.cu:21-337) for the names cp, lbm, mriq, stencil,
+/* createKernel (src/Creator.cu:21-337) for the names cp, lbm, mrif, mriq, stencil,
  * tzgemm: the memoised GPTBKernel that owns seeded device buffers exactly as the
  * reference's Ori*Kernel::initParams builds them. Never destroy these. */
 TK_API tacker_kernel_t tacker_create_kernel(const char *name);
@@ -270,6 +300,8 @@ TK_API tacker_kernel_t tacker_ori_stencil_create(float c0, float c1, const float
 TK_API tacker_kernel_t tacker_ori_lbm_create(const float *src, float *dst, int sx, int sy, int sz);
 TK_API tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y,
                                               const float *z, float *Qr, float *Qi, int numX);
+TK_API tacker_kernel_t tacker_ori_mrif_create(int numK, const float *x, const float *y,
+                                              const float *z, float *outR, float *outI, int numX);
 TK_API tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid,
                                             int volx, int voly);
 /* OriTZGEMMKernel(id, m, n, k) (src/tzgemm_kernel.h:56-147); m, n, k are rounded

@@ -50,6 +50,9 @@ def _declare(l):
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
+    l.orc_mrif_rhophi.argtypes = [C.c_int, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p]
+    l.orc_mrif_gptb.argtypes = [C.c_int, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, C.c_int,
+                                C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_gptb.argtypes = [C.c_int, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, C.c_int,
                                 C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_cp_initatoms.argtypes = [_f32p, C.c_int, C.c_uint, C.c_uint, C.c_uint, C.c_float]
@@ -170,6 +173,36 @@ def mriq(kvals, x, y, z, Qr, Qi, start=0, end=None, gdx=None, f64=False, kchunk=
                         np.ascontiguousarray(y, np.float32), np.ascontiguousarray(z, np.float32),
                         qr, qi, gdx, gdy, kchunk, start, end, 1 if f64 else 0)
     return qr, qi
+
+
+# --------------------------------------------------------------------------- mri-fhd
+def mrif_rhophi(phiR, phiI, dR, dI):
+    f = lambda a: np.ascontiguousarray(a, np.float32)
+    re, im = np.zeros(phiR.size, np.float32), np.zeros(phiR.size, np.float32)
+    lib().orc_mrif_rhophi(phiR.size, f(phiR), f(phiI), f(dR), f(dI), re, im)
+    return re, im
+
+
+def mrif(kvals, x, y, z, outR, outI, start=0, end=None, gdx=None, f64=False, kchunk=None):
+    """kvals is [numK][5] float32 {Kx,Ky,Kz,RhoPhiR,RhoPhiI}. Returns (outR, outI).
+    Block positions as in mriq()."""
+    kvals = np.ascontiguousarray(kvals, np.float32)
+    numK = kvals.shape[0]
+    numX = x.size
+    if gdx is None:
+        gdx = numX // 256
+    if kchunk is None:
+        gdy, kchunk = 1, max(numK, 1)
+    else:
+        gdy = max(1, -(-numK // kchunk))
+    if end is None:
+        end = gdx * gdy
+    r = np.array(outR, np.float32, order="C")
+    i = np.array(outI, np.float32, order="C")
+    lib().orc_mrif_gptb(numK, kvals.reshape(-1), np.ascontiguousarray(x, np.float32),
+                        np.ascontiguousarray(y, np.float32), np.ascontiguousarray(z, np.float32),
+                        r, i, gdx, gdy, kchunk, start, end, 1 if f64 else 0)
+    return r, i
 
 
 # --------------------------------------------------------------------------- cp

@@ -25,6 +25,9 @@
  *                         float64 brute force; block-by-chunk positions: any
  *                         ascending tiling = the one k loop bit for bit, one
  *                         position = numpy float64 over its record range.
+ *   orc_mrif*             x=0 closed form, single-k closed form, numpy complex128
+ *                         sum conj(phi) d e^{i 2 pi k.x}; block-by-chunk
+ *                         positions as orc_mriq.
  *   orc_cp*               single atom closed form, numpy float64 brute force,
  *                         ori_blks = 16384 held by fusion/code/kinfo.json.
  *   orc_im2col            direct convolution brute force.
@@ -463,6 +466,83 @@ ORC_API void orc_mriq_gptb(int numK, const float *kvals, const float *x, const f
             if (k1 > numK) k1 = numK;
             for (int t = 0; t < 256; t++)
                 orc_mriq_voxel((int)k0, (int)k1, kvals, x, y, z, Qr, Qi, bx * 256 + t, f64);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------------ */
+/* mri-fhd                                                                  */
+/* ------------------------------------------------------------------------ */
+
+/* src/ori_kernel/mrif_kernel.cu:62-75: RhoPhi = conj(phi) * d */
+ORC_API void orc_mrif_rhophi(int numK, const float *phiR, const float *phiI, const float *dR,
+                             const float *dI, float *realRhoPhi, float *imagRhoPhi)
+{
+    for (int k = 0; k < numK; k++) {
+        float a = phiR[k] * dR[k], b = phiI[k] * dI[k];
+        float c = phiR[k] * dI[k], d = phiI[k] * dR[k];
+        realRhoPhi[k] = a + b;
+        imagRhoPhi[k] = c - d;
+    }
+}
+
+/* src/ori_kernel/mrif_kernel.cu:77-152 with the k loop running over all numK
+ * samples (the reference's "FHGrid < 1" loop stops after the first grid of 256,
+ * :84-85).  kvals is the AoS table {Kx,Ky,Kz,RhoPhiR,RhoPhiI}
+ * (src/header/mrif_header.h:23-29).  Block positions as orc_mriq_gptb
+ * (src/gptb_kernel/mrif_kernel.cu:113-125 index reconstruction). */
+static void orc_mrif_voxel(int k0, int k1, const float *kvals, const float *x, const float *y,
+                           const float *z, float *outR, float *outI, int xi, int f64)
+{
+    const float PIx2 = 6.2831853071795864769252867665590058f;
+    if (f64) {
+        double sx = x[xi], sy = y[xi], sz = z[xi];
+        double r = outR[xi], i = outI[xi];
+        for (int k = k0; k < k1; k++) {
+            const float *kv = kvals + 5 * (size_t)k;
+            double arg = 6.2831853071795864769252867665590058 *
+                         ((double)kv[0] * sx + (double)kv[1] * sy + (double)kv[2] * sz);
+            double c = cos(arg), sn = sin(arg);
+            r += (double)kv[3] * c - (double)kv[4] * sn;
+            i += (double)kv[4] * c + (double)kv[3] * sn;
+        }
+        outR[xi] = (float)r;
+        outI[xi] = (float)i;
+    } else {
+        float sx = x[xi], sy = y[xi], sz = z[xi];
+        float r = outR[xi], i = outI[xi];
+        for (int k = k0; k < k1; k++) {
+            const float *kv = kvals + 5 * (size_t)k;
+            float a = kv[0] * sx, b = kv[1] * sy, c = kv[2] * sz;
+            float d = a + b;
+            d = d + c;
+            float arg = PIx2 * d;
+            float cs = cosf(arg), sn = sinf(arg);
+            float rc = kv[3] * cs, is = kv[4] * sn;
+            float ic = kv[4] * cs, rs = kv[3] * sn;
+            float re = rc - is, im = ic + rs;
+            r = r + re;
+            i = i + im;
+        }
+        outR[xi] = r;
+        outI[xi] = i;
+    }
+}
+
+ORC_API void orc_mrif_gptb(int numK, const float *kvals, const float *x, const float *y,
+                           const float *z, float *outR, float *outI, int gdx, int gdy, int kchunk,
+                           int start, int end, int f64)
+{
+#pragma omp parallel for schedule(static)
+    for (int bx = 0; bx < gdx; bx++) {
+        int first = start + ((bx - start % gdx) + gdx) % gdx;
+        for (int pos = first; pos < end; pos += gdx) {
+            int chunk = (pos / gdx) % gdy;
+            long k0 = (long)chunk * kchunk, k1 = k0 + kchunk;
+            if (k0 > numK) k0 = numK;
+            if (k1 > numK) k1 = numK;
+            for (int t = 0; t < 256; t++)
+                orc_mrif_voxel((int)k0, (int)k1, kvals, x, y, z, outR, outI, bx * 256 + t, f64);
         }
     }
 }

@@ -55,6 +55,12 @@ def _declare(lib):
     lib.tacker_mix_tzgemm_stencil.argtypes = [f, f, vp, vp, i, i, i, i, i] + gemm
     lib.tacker_mix_tzgemm_lbm.argtypes = [vp, vp, i, i, i, i, i] + gemm
     lib.tacker_mix_tzgemm_mriq.argtypes = [i, vp, vp, vp, vp, vp, i, i, i] + gemm
+    lib.tacker_mrif_rhophi.argtypes = [i, vp, vp, vp, vp, vp, vp, vp]
+    lib.tacker_mrif_set_kvalues.argtypes = [vp, i]
+    lib.tacker_mrif_blocks.argtypes = [i, i]
+    lib.tacker_ori_mrif.argtypes = [i, vp, vp, vp, vp, vp, i, vp]
+    lib.tacker_gptb_mrif.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_mrif.argtypes = [i, vp, vp, vp, vp, vp, i, i, i] + gemm
     lib.tacker_mix_tzgemm_cp.argtypes = [i, f, vp, i, i, i, i] + gemm
     lib.tacker_im2col.argtypes = [vp] + [i] * 11 + [vp, vp]
     lib.tacker_convert_fp32_to_fp16.argtypes = [vp, vp, i, vp]
@@ -63,7 +69,7 @@ def _declare(lib):
     lib.tacker_fget_kernel_info.argtypes = [cp, cp]
     lib.tacker_fget_kernel_info.restype = f
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
-                 "tacker_ori_mriq_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
+                 "tacker_ori_mriq_create", "tacker_ori_mrif_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
                  "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
                  "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
@@ -71,6 +77,7 @@ def _declare(lib):
     lib.tacker_ori_stencil_create.argtypes = [f, f, vp, vp, i, i, i]
     lib.tacker_ori_lbm_create.argtypes = [vp, vp, i, i, i]
     lib.tacker_ori_mriq_create.argtypes = [i, vp, vp, vp, vp, vp, i]
+    lib.tacker_ori_mrif_create.argtypes = [i, vp, vp, vp, vp, vp, i]
     lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
     lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_gptb_create.argtypes = [vp, i, i, i, i]
@@ -343,6 +350,43 @@ def mix_tzgemm_lbm(src, dst, sx, sy, sz, A, B, Cm, be_start=0, be_end=None, tile
         _ptr(src), _ptr(dst), sx, sy, sz, be_start, be_end,
         *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
         "tacker_mix_tzgemm_lbm")
+def mrif_rhophi(phiR, phiI, dR, dI, realRhoPhi, imagRhoPhi, stream=None):
+    check(lib().tacker_mrif_rhophi(phiR.numel(), _ptr(phiR), _ptr(phiI), _ptr(dR), _ptr(dI), _ptr(realRhoPhi),
+                                   _ptr(imagRhoPhi), _stream(stream)), "tacker_mrif_rhophi")
+
+
+def mrif_set_kvalues(kvals_np):
+    """kvals_np: host numpy float32 [numK][5] = {Kx,Ky,Kz,RhoPhiR,RhoPhiI}."""
+    import numpy as np
+    kv = np.ascontiguousarray(kvals_np, np.float32)
+    check(lib().tacker_mrif_set_kvalues(kv.ctypes.data, kv.shape[0]), "tacker_mrif_set_kvalues")
+
+
+def mrif_blocks(numK, numX):
+    """block positions of the GPTB form: voxel blocks x chunks of the k table"""
+    return lib().tacker_mrif_blocks(numK, numX)
+
+
+def ori_mrif(numK, x, y, z, outR, outI, stream=None):
+    check(lib().tacker_ori_mrif(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(outR), _ptr(outI), x.numel(),
+                                _stream(stream)), "tacker_ori_mrif")
+
+
+def gptb_mrif(numK, x, y, z, outR, outI, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    if end is None:
+        end = mrif_blocks(numK, x.numel())
+    check(lib().tacker_gptb_mrif(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(outR), _ptr(outI), x.numel(), start,
+                                 end, launch_grid, launch_block, _stream(stream)), "tacker_gptb_mrif")
+
+
+def mix_tzgemm_mrif(numK, x, y, z, outR, outI, A, B, Cm, be_start=0, be_end=None, tile_start=0,
+                    tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    if be_end is None:
+        be_end = mrif_blocks(numK, x.numel())
+    check(lib().tacker_mix_tzgemm_mrif(
+        numK, _ptr(x), _ptr(y), _ptr(z), _ptr(outR), _ptr(outI), x.numel(), be_start, be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_mrif")
 
 
 def mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, A, B, Cm, be_start=0, be_end=None, tile_start=0,
@@ -450,6 +494,11 @@ def ori_lbm_create(src, dst, sx, sy, sz):
 def ori_mriq_create(numK, x, y, z, Qr, Qi):
     return KernelHandle(lib().tacker_ori_mriq_create(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(Qr), _ptr(Qi),
                                                      x.numel()), "OriMRIQKernel", keep=(x, y, z, Qr, Qi))
+
+
+def ori_mrif_create(numK, x, y, z, outR, outI):
+    return KernelHandle(lib().tacker_ori_mrif_create(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(outR), _ptr(outI),
+                                                     x.numel()), "OriMRIFKernel", keep=(x, y, z, outR, outI))
 
 
 def ori_cp_create(numatoms, gridspacing, grid):

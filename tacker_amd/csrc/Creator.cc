@@ -52,6 +52,9 @@ GPTBKernel *createKernel(const std::string &name)
     } else if (name == "mriq") {
         auto *ori = new OriMRIQKernel(18);
         k = new GPTBKernel(18, "mriq", "gptb_mriq", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
+    } else if (name == "mrif") {
+        auto *ori = new OriMRIFKernel(17);
+        k = new GPTBKernel(17, "mrif", "gptb_mrif", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
     } else if (name == "stencil") {
         auto *ori = new OriSTENCILKernel(19);
         k = new GPTBKernel(19, "stencil", "gptb_stencil", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));

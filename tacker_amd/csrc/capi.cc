@@ -65,8 +65,8 @@ int check_block(const std::string &name, int block)
         return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 64 in [64,256]");
     if (name == "tzgemm" && block != TZ_THREADS)
         return fail(TK_ERROR_INVALID_VALUE, "tzgemm: launch_block must be 256");
-    if (name == "mriq" && block % 256)
-        return fail(TK_ERROR_INVALID_VALUE, "mriq: launch_block must be a multiple of 256");
+    if ((name == "mriq" || name == "mrif") && block % 256)
+        return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 256");
     if (name == "cp" && block % 128)
         return fail(TK_ERROR_INVALID_VALUE, "cp: launch_block must be a multiple of 128");
     return TK_SUCCESS;
@@ -110,6 +110,13 @@ int check_mriq(int numK, const float *x, const float *y, const float *z, float *
     if (!x || !y || !z || !Qr || !Qi || numK < 0 || numK > MRIQ_MAX_K || numX < 0)
         return fail(TK_ERROR_INVALID_VALUE, "mriq: bad arguments");
     if (numX % KERNEL_Q_THREADS_PER_BLOCK) return fail(TK_ERROR_UNSUPPORTED, "mriq: numX must be a multiple of 256");
+    return TK_SUCCESS;
+}
+int check_mrif(int numK, const float *x, const float *y, const float *z, float *outR, float *outI, int numX)
+{
+    if (!x || !y || !z || !outR || !outI || numK < 0 || numK > MRIF_MAX_K || numX < 0)
+        return fail(TK_ERROR_INVALID_VALUE, "mrif: bad arguments");
+    if (numX % KERNEL_FH_THREADS_PER_BLOCK) return fail(TK_ERROR_UNSUPPORTED, "mrif: numX must be a multiple of 256");
     return TK_SUCCESS;
 }
 int check_cp(int numatoms, float *grid, int volx, int voly)
@@ -329,6 +336,55 @@ int tacker_gptb_mriq(int numK, const float *x, const float *y, const float *z, f
                          launch_block, stream);
 }
 
+int tacker_mrif_rhophi(int numK, const float *phiR, const float *phiI, const float *dR, const float *dI,
+                       float *realRhoPhi, float *imagRhoPhi, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    if (!phiR || !phiI || !dR || !dI || !realRhoPhi || !imagRhoPhi || numK < 0)
+        return fail(TK_ERROR_INVALID_VALUE, "mrif_rhophi: bad arguments");
+    if (numK == 0) return TK_SUCCESS;
+    void *args[] = {&numK, &phiR, &phiI, &dR, &dI, &realRhoPhi, &imagRhoPhi};
+    const dim3 grid((numK + KERNEL_RHO_PHI_THREADS_PER_BLOCK - 1) / KERNEL_RHO_PHI_THREADS_PER_BLOCK);
+    const int rc = tkLaunchKernel(fmap["ComputeRhoPhiGPU"], grid.raw(), dim3(KERNEL_RHO_PHI_THREADS_PER_BLOCK).raw(), args, 0, stream);
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+int tacker_mrif_set_kvalues(const float *kvals_host, int numK)
+{
+    REQUIRE_INIT();
+    if (!kvals_host || numK < 0 || numK > MRIF_MAX_K) return fail(TK_ERROR_INVALID_VALUE, "mrif: numK out of range");
+    const int rc = OriMRIFKernel::setKValues(reinterpret_cast<const mrif_kValues *>(kvals_host), numK);
+    return rc ? fail(rc, tkGetErrorString(rc)) : rc;
+}
+
+int tacker_mrif_blocks(int numK, int numX)
+{
+    static_assert(TACKER_MRIF_K_CHUNK == MRIF_K_CHUNK, "public and device chunk sizes must agree");
+    if (numK < 0 || numX < 0) return 0;
+    const int chunks = numK > 0 ? (numK + MRIF_K_CHUNK - 1) / MRIF_K_CHUNK : 1;
+    return (numX / KERNEL_FH_THREADS_PER_BLOCK) * chunks;
+}
+
+int tacker_ori_mrif(int numK, const float *x, const float *y, const float *z, float *outR, float *outI, int numX, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_mrif(numK, x, y, z, outR, outI, numX);
+    if (rc) return rc;
+    if (numX == 0) return TK_SUCCESS;
+    return run_once(new OriMRIFKernel(0, numK, x, y, z, outR, outI, numX), stream);
+}
+
+int tacker_gptb_mrif(int numK, const float *x, const float *y, const float *z, float *outR, float *outI, int numX,
+                     int block_start, int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_mrif(numK, x, y, z, outR, outI, numX);
+    if (rc) return rc;
+    if (numX == 0) return TK_SUCCESS;
+    return run_gptb_once(new OriMRIFKernel(0, numK, x, y, z, outR, outI, numX), block_start, block_end, launch_grid,
+                         launch_block, stream);
+}
+
 int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane)
 {
     REQUIRE_INIT();
@@ -426,6 +482,18 @@ int tacker_mix_tzgemm_mriq(int numK, const float *x, const float *y, const float
                         tile_start, tile_end, variant, launch_grid, launch_block, stream);
 }
 
+int tacker_mix_tzgemm_mrif(int numK, const float *x, const float *y, const float *z, float *outR, float *outI,
+                           int numX, int be_start, int be_end, const void *A, const void *B, float *C, int M,
+                           int N, int K, int tile_start, int tile_end, const char *variant, int launch_grid,
+                           int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_mrif(numK, x, y, z, outR, outI, numX);
+    if (rc) return rc;
+    return run_mix_once(new OriMRIFKernel(0, numK, x, y, z, outR, outI, numX), be_start, be_end, A, B, C, M, N, K,
+                        tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
 int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, int be_start,
                          int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
                          int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
@@ -489,7 +557,7 @@ tacker_kernel_t tacker_create_kernel(const char *name)
         fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
         return nullptr;
     }
-    static const char *known[] = {"cp", "lbm", "mriq", "stencil", "tzgemm"};
+    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "stencil", "tzgemm"};
     bool ok = false;
     for (auto k : known) ok |= (strcmp(k, name) == 0);
     if (!ok) {
@@ -530,6 +598,10 @@ tacker_kernel_t tacker_ori_lbm_create(const float *src, float *dst, int sx, int 
 tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y, const float *z, float *Qr, float *Qi, int numX)
 {
     CREATE(check_mriq(numK, x, y, z, Qr, Qi, numX), new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX));
+}
+tacker_kernel_t tacker_ori_mrif_create(int numK, const float *x, const float *y, const float *z, float *outR, float *outI, int numX)
+{
+    CREATE(check_mrif(numK, x, y, z, outR, outI, numX), new OriMRIFKernel(0, numK, x, y, z, outR, outI, numX));
 }
 tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid, int volx, int voly)
 {
@@ -812,7 +884,7 @@ tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const ch
         fail(TK_ERROR_INVALID_VALUE, "tacker_task_manager_create: bad arguments");
         return nullptr;
     }
-    static const char *known[] = {"cp", "lbm", "mriq", "stencil"};
+    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "stencil"};
     bool ok1 = false, ok2 = !be2 || !*be2;
     for (auto k : known) {
         ok1 |= strcmp(k, be1) == 0;

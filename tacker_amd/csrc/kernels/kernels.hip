@@ -15,6 +15,7 @@
 #include "dnn_kernels.h"
 #include "lbm_role.h"
 #include "mriq_role.h"
+#include "mrif_role.h"
 #include "stencil_role.h"
 #include "tzgemm_role.h"
 
@@ -64,6 +65,29 @@ extern "C" __global__ __launch_bounds__(256) void ori_mriq(int numK, int kGlobal
     tk::mriq_voxel(numK, x, y, z, Qr, Qi, blockIdx.x * KERNEL_Q_THREADS_PER_BLOCK + threadIdx.x);
 }
 
+extern "C" __global__ void ComputeRhoPhiGPU(int numK, float *phiR, float *phiI, float *dR, float *dI,
+                                            float *realRhoPhi, float *imagRhoPhi)
+{
+    const int indexK = blockIdx.x * KERNEL_RHO_PHI_THREADS_PER_BLOCK + threadIdx.x;
+    if (indexK < numK) {
+        const float rPhiR = phiR[indexK];
+        const float rPhiI = phiI[indexK];
+        const float rDR = dR[indexK];
+        const float rDI = dI[indexK];
+        // the product on the left folded into the sum / difference, as nvcc contracts the source
+        realRhoPhi[indexK] = __builtin_fmaf(rPhiR, rDR, rPhiI * rDI);
+        imagRhoPhi[indexK] = __builtin_fmaf(rPhiR, rDI, -(rPhiI * rDR));
+    }
+}
+
+// grid numX/256, block 256
+extern "C" __global__ __launch_bounds__(256) void ori_mrif(int numK, int kGlobalIndex, float *x,
+                                                           float *y, float *z, float *outR, float *outI)
+{
+    (void)kGlobalIndex;
+    tk::mrif_voxel(numK, x, y, z, outR, outI, blockIdx.x * KERNEL_FH_THREADS_PER_BLOCK + threadIdx.x);
+}
+
 // grid (volx/128, voly/8), block (16,8)
 extern "C" __global__ __launch_bounds__(128) void ori_cp(int numatoms, float gridspacing,
                                                          float *energygrid)
@@ -104,6 +128,15 @@ extern "C" __global__ void g_general_ptb_mriq(int numK, int kGlobalIndex, float 
 {
     (void)kGlobalIndex;
     tk::mriq_role(numK, x, y, z, Qr, Qi, grid_dimension_x, grid_dimension_y, (int)blockIdx.x, ptb_iter_block_step,
+                  ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base,
+                  (int)blockDim.x);
+}
+
+extern "C" __global__ void general_ptb_mrif(int numK, int kGlobalIndex, float *x, float *y,
+                                            float *z, float *outR, float *outI, GPTB_TRAILER)
+{
+    (void)kGlobalIndex;
+    tk::mrif_role(numK, x, y, z, outR, outI, grid_dimension_x, grid_dimension_y, (int)blockIdx.x, ptb_iter_block_step,
                   ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base,
                   (int)blockDim.x);
 }
@@ -184,11 +217,14 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ori_ComputePhiMag", (const void *)ori_ComputePhiMag, ctx);
     insert("ori_mriq", (const void *)ori_mriq, ctx);
     insert("ori_cp", (const void *)ori_cp, ctx);
+    insert("ComputeRhoPhiGPU", (const void *)ComputeRhoPhiGPU, ctx);
+    insert("ori_mrif", (const void *)ori_mrif, ctx);
     insert("gptb_tzgemm", (const void *)general_ptb_tzgemm, ctx);
     insert("gptb_stencil", (const void *)general_ptb_stencil, ctx);
     insert("gptb_lbm", (const void *)general_ptb_lbm, ctx);
     insert("gptb_mriq", (const void *)g_general_ptb_mriq, ctx);
     insert("gptb_cp", (const void *)g_general_ptb_cp, ctx);
+    insert("gptb_mrif", (const void *)general_ptb_mrif, ctx);
     insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);
     insert("im2col", (const void *)im2col_gpu_kernel_, ctx);
     insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);
@@ -208,6 +244,11 @@ extern "C" int tk_device_symbol(const char *name, const void **symbol, size_t *b
     if (__builtin_strcmp(name, "ck") == 0) {
         *symbol = (const void *)&ck;
         *bytes = sizeof(ck);
+        return TK_SUCCESS;
+    }
+    if (__builtin_strcmp(name, "c_mrif") == 0) {
+        *symbol = (const void *)&c_mrif;
+        *bytes = sizeof(c_mrif);
         return TK_SUCCESS;
     }
     if (__builtin_strcmp(name, "atominfo") == 0) {

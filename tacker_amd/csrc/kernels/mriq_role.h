@@ -111,10 +111,26 @@ __device__ __forceinline__ void mriq_voxel(int numK, const float *__restrict__ x
     mriq_voxels<1>(0, numK, x, y, z, Qr, Qi, one);
 }
 
+// What a thread does for V voxels and a run of k records: the part of the kernel that the
+// walk over block positions below does not know about.  MRI-FHD (mrif_role.h) walks the
+// same position grid with another body.
+struct MriqBody {
+    static __device__ __forceinline__ int chunk() { return MRIQ_K_CHUNK; }
+    template <int V>
+    static __device__ __forceinline__ void voxels(int k_begin, int k_end, const float *__restrict__ x,
+                                                  const float *__restrict__ y, const float *__restrict__ z,
+                                                  float *__restrict__ Qr, float *__restrict__ Qi,
+                                                  const int (&xIndex)[V])
+    {
+        mriq_voxels<V>(k_begin, k_end, x, y, z, Qr, Qi, xIndex);
+    }
+};
+
 // One phase of a launch: voxel blocks [block_lo, block_hi) each take records
 // [k_begin, k_end).  A thread serves the blocks it owns -- first_owned, first_owned +
 // stride, ... -- up to MRIQ_VOXELS_PER_THREAD at a time.
 #define MRIQ_VOXELS_PER_THREAD 4
+template <class Body>
 __device__ __forceinline__ void mriq_phase(int block_lo, int block_hi, int k_begin, int k_end,
                                            const float *__restrict__ x, const float *__restrict__ y,
                                            const float *__restrict__ z, float *__restrict__ Qr,
@@ -134,15 +150,15 @@ __device__ __forceinline__ void mriq_phase(int block_lo, int block_hi, int k_beg
             idx[v] = (bv < block_hi ? bv : b) * KERNEL_Q_THREADS_PER_BLOCK + t;
         }
         if (count == V) {
-            mriq_voxels<V>(k_begin, k_end, x, y, z, Qr, Qi, idx);
+            Body::template voxels<V>(k_begin, k_end, x, y, z, Qr, Qi, idx);
         } else {
             if (count >= 2) {
                 const int two[2] = {idx[0], idx[1]};
-                mriq_voxels<2>(k_begin, k_end, x, y, z, Qr, Qi, two);
+                Body::template voxels<2>(k_begin, k_end, x, y, z, Qr, Qi, two);
             }
             if (count & 1) {
                 const int one[1] = {idx[count - 1]};
-                mriq_voxels<1>(k_begin, k_end, x, y, z, Qr, Qi, one);
+                Body::template voxels<1>(k_begin, k_end, x, y, z, Qr, Qi, one);
             }
         }
     }
@@ -164,6 +180,7 @@ __device__ __forceinline__ void mriq_phase(int block_lo, int block_hi, int k_beg
 // and the owner walks the three parts in order: the chunks of a voxel are added in
 // ascending position order without any synchronisation between threads.  Whole rows that
 // follow each other are one run of the k loop.
+template <class Body = MriqBody>
 __device__ __forceinline__ void mriq_role(int numK, const float *__restrict__ x,
                                           const float *__restrict__ y, const float *__restrict__ z,
                                           float *__restrict__ Qr, float *__restrict__ Qi,
@@ -178,19 +195,19 @@ __device__ __forceinline__ void mriq_role(int numK, const float *__restrict__ x,
     const int gy = grid_dimension_y;
     const int stride = role_blocks * blocks_at_once;
     const int first_owned = slot * role_blocks + role_block;
-    const auto chunk_begin = [&](int row) { return min((row % gy) * MRIQ_K_CHUNK, numK); };
-    const auto chunk_end = [&](int row) { return min((row % gy + 1) * MRIQ_K_CHUNK, numK); };
+    const auto chunk_begin = [&](int row) { return min((row % gy) * Body::chunk(), numK); };
+    const auto chunk_end = [&](int row) { return min((row % gy + 1) * Body::chunk(), numK); };
 
     const int first_row = start / gx;
     const int last_row = (end - 1) / gx;   // row of the last position
     if (first_row == last_row) {
-        mriq_phase(start - first_row * gx, end - first_row * gx, chunk_begin(first_row), chunk_end(first_row),
+        mriq_phase<Body>(start - first_row * gx, end - first_row * gx, chunk_begin(first_row), chunk_end(first_row),
                    x, y, z, Qr, Qi, first_owned, stride, t);
         return;
     }
     int row = first_row;
     if (start != first_row * gx) {   // partial first row
-        mriq_phase(start - first_row * gx, gx, chunk_begin(row), chunk_end(row), x, y, z, Qr, Qi,
+        mriq_phase<Body>(start - first_row * gx, gx, chunk_begin(row), chunk_end(row), x, y, z, Qr, Qi,
                    first_owned, stride, t);
         ++row;
     }
@@ -198,11 +215,11 @@ __device__ __forceinline__ void mriq_role(int numK, const float *__restrict__ x,
     while (row < whole_end) {
         // rows up to the next multiple of grid_dimension_y are consecutive chunks
         const int run_end = min(whole_end, (row / gy + 1) * gy);
-        mriq_phase(0, gx, chunk_begin(row), chunk_end(run_end - 1), x, y, z, Qr, Qi, first_owned, stride, t);
+        mriq_phase<Body>(0, gx, chunk_begin(row), chunk_end(run_end - 1), x, y, z, Qr, Qi, first_owned, stride, t);
         row = run_end;
     }
     if (whole_end == last_row)       // partial last row
-        mriq_phase(0, end - last_row * gx, chunk_begin(last_row), chunk_end(last_row), x, y, z, Qr, Qi,
+        mriq_phase<Body>(0, end - last_row * gx, chunk_begin(last_row), chunk_end(last_row), x, y, z, Qr, Qi,
                    first_owned, stride, t);
 }
 

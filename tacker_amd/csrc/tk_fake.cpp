@@ -49,6 +49,7 @@ std::vector<int> cat(std::vector<int> a, const std::vector<int> &b)
 const std::vector<int> STENCIL = {F, F, P, P, I, I, I};
 const std::vector<int> LBM = {P, P};
 const std::vector<int> MRIQ = {I, I, P, P, P, P, P};
+const std::vector<int> MRIF = {I, I, P, P, P, P, P};
 const std::vector<int> CP = {I, F, P};
 const std::vector<int> TZ = {P, P, P, I, I, I, P};
 }  // namespace
@@ -76,7 +77,7 @@ int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int, tkStream_t) { m
 int tkMemset(void *ptr, int value, size_t bytes) { memset(ptr, value, bytes); return TK_SUCCESS; }
 int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset)
 {
-    if (strcmp(symbol, "ck") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail"))
+    if (strcmp(symbol, "ck") && strcmp(symbol, "c_mrif") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail"))
         return TK_ERROR_NOT_FOUND;
     auto &buf = g_symbols[symbol];
     if (buf.size() < offset + bytes) buf.resize(offset + bytes);
@@ -164,11 +165,14 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ori_ComputePhiMag", {P, P, P, I});
         add("ori_mriq", MRIQ);
         add("ori_cp", CP);
+        add("ComputeRhoPhiGPU", {I, P, P, P, P, P, P});
+        add("ori_mrif", MRIF);
         add("gptb_tzgemm", cat(TZ, trailer(true)));
         add("gptb_stencil", cat(STENCIL, trailer(true)));
         add("gptb_lbm", cat(LBM, trailer(true)));
         add("gptb_mriq", cat(MRIQ, trailer(true)));
         add("gptb_cp", cat(CP, trailer(true)));
+        add("gptb_mrif", cat(MRIF, trailer(true)));
         add("cp_inv_sqrt_selftest", {I, I, P});
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
@@ -178,7 +182,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("pack_fc_input", {P, 8, P, I, I, P});
         add("pack_fc_input_pooled", {P, I, I, I, P, I, I, P});
         const std::pair<const char *, const std::vector<int> *> bes[] = {
-            {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}};
+            {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}, {"mrif", &MRIF}};
         static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};
         for (auto &be : bes)
             for (auto v : variants)

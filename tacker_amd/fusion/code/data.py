@@ -51,6 +51,9 @@ KERNEL_INFO = {
     # 1024 blocks of 256 voxels x 16 chunks of 128 k records
     "mriq": {"register": 40, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
              "ori_blks": 16384},
+    # 1024 blocks of 256 voxels x 16 chunks of 128 k records
+    "mrif": {"register": 44, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
+             "ori_blks": 16384},
     # 16384 blocks of 128 x 8 points x 4 parts of the unrolled x points
     "cp": {"register": 40, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
            "ori_blks": 65536},

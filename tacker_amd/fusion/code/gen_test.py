@@ -65,6 +65,16 @@ def make_inputs(np, torch, ta, be, small):
         xyz = [torch.from_numpy(rng.uniform(-0.5, 0.5, numX).astype(np.float32)).cuda() for _ in range(3)]
         Qr, Qi = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
         return ta.ori_mriq_create(numK, xyz[0], xyz[1], xyz[2], Qr, Qi), ta.mriq_blocks(numK, numX), [Qr, Qi]
+    if be == "mrif":
+        numK, numX = (256, 2048) if small else (2048, 262144)
+        k = rng.uniform(-0.5, 0.5, (numK, 3)).astype(np.float32)
+        phi = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+        d = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+        rho = np.stack([phi[0] * d[0] + phi[1] * d[1], phi[0] * d[1] - phi[1] * d[0]], 1)
+        ta.mrif_set_kvalues(np.concatenate([k, rho], 1).astype(np.float32))
+        xyz = [torch.from_numpy(rng.uniform(-0.5, 0.5, numX).astype(np.float32)).cuda() for _ in range(3)]
+        outR, outI = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+        return ta.ori_mrif_create(numK, xyz[0], xyz[1], xyz[2], outR, outI), ta.mrif_blocks(numK, numX), [outR, outI]
     if be == "cp":
         ta.cp_set_atoms(ta.cp_initatoms(4000)[1:65], 0.0)
         shape = (32, 512) if small else (4096, 4096)

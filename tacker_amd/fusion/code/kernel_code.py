@@ -1,7 +1,7 @@
 """Role descriptions the generator stitches together.
 
 Each entry plays the part of one ``<kernel>_code.py`` of the reference
-(fusion/code/cp_code.py, lbm_code.py, mriq_code.py, stencil_code.py and the
+(fusion/code/cp_code.py, lbm_code.py, mriq_code.py, mrif_code.py, stencil_code.py and the
 truncated tzgemm_code.py): the kernel's parameter list in reference order and
 how to call its device-side role.  The role bodies themselves live in
 ``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
@@ -51,6 +51,14 @@ ROLES = {
                    ("float*", "z"), ("float*", "Qr"), ("float*", "Qi")],
         "needs_sync": False,
         "call": ("tk::mriq_role({p}numK, {p}x, {p}y, {p}z, {p}Qr, {p}Qi, {p}grid_dimension_x, "
+                 "{p}grid_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "{threads});"),
+    },
+    "mrif": {
+        "params": [("int", "numK"), ("int", "kGlobalIndex"), ("float*", "x"), ("float*", "y"),
+                   ("float*", "z"), ("float*", "outR"), ("float*", "outI")],
+        "needs_sync": False,
+        "call": ("tk::mrif_role({p}numK, {p}x, {p}y, {p}z, {p}outR, {p}outI, {p}grid_dimension_x, "
                  "{p}grid_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "{threads});"),
     },

@@ -30,12 +30,12 @@ ROOT = os.path.abspath(os.path.join(HERE, "..", "..", ".."))
 DEFAULTS = os.path.join(HERE, "defaults.json")
 # reduction lengths of the VGG16 batch-1 layers after padding to 128, plus the benchmark's
 K_LADDER = (128, 640, 1152, 2048, 2304, 4096, 4608)
-PAIRS = ("stencil", "lbm", "mriq", "cp")
+PAIRS = ("stencil", "lbm", "mriq", "cp", "mrif")
 TILES = 1024
 LADDER = 32          # best-effort block counts tried: N/32, 2N/32, ..., N
 
 
-def measure(out_path, stretch, launches):
+def measure(out_path, stretch, launches, pairs=PAIRS):
     sys.path.insert(0, ROOT)
     import torch
     import tacker_amd as ta
@@ -55,7 +55,7 @@ def measure(out_path, stretch, launches):
         return e0.elapsed_ms(e1) / launches * 1e3
 
     result = {"stretch": stretch, "tiles": TILES, "device": ta.device_name(), "pairs": {}}
-    for be_name in PAIRS:
+    for be_name in pairs:
         be = ta.create_kernel(be_name)
         be_total = be.info()["ptb_end"]
         be_us = timed(be)
@@ -115,9 +115,11 @@ def main():
     ap.add_argument("--stretch", type=float, default=1.0,
                     help="largest tolerated stretch of the GEMM's launch (1.0 = at most twice as long)")
     ap.add_argument("--launches", type=int, default=100)
+    ap.add_argument("--pairs", default=",".join(PAIRS),
+                    help="best-effort kernels to measure (comma separated); --apply only touches those measured")
     args = ap.parse_args()
     if args.measure:
-        measure(args.measure, args.stretch, args.launches)
+        measure(args.measure, args.stretch, args.launches, tuple(args.pairs.split(",")))
     elif args.apply:
         apply(args.apply)
     else:

@@ -103,3 +103,20 @@ def launch(key, grid, block, args):
     rc = ta.lib().tkLaunchKernel(func, _Dim3(grid, 1, 1), _Dim3(block, 1, 1), ptrs, 0,
                                  torch.cuda.current_stream().cuda_stream)
     assert rc == 0, rc
+
+
+def mrif_inputs(numK, numX, seed=1337):
+    """k samples, phi (2, numK), d (2, numK), voxel coordinates (3, numX)"""
+    rng = np.random.default_rng(seed)
+    k = rng.uniform(-0.5, 0.5, (numK, 3)).astype(np.float32)
+    phi = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+    d = rng.uniform(0, 1, (2, numK)).astype(np.float32)
+    xyz = rng.uniform(-0.5, 0.5, (3, numX)).astype(np.float32)
+    return k, phi, d, xyz
+
+
+def mrif_table(k, phi, d):
+    """AoS table {Kx,Ky,Kz,RhoPhiR,RhoPhiI} with RhoPhi from the oracle"""
+    import oracle
+    re, im = oracle.mrif_rhophi(phi[0], phi[1], d[0], d[1])
+    return np.concatenate([k, re[:, None], im[:, None]], 1).astype(np.float32)

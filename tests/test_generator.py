@@ -108,8 +108,10 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
     files = gen_run.generate()
     kinfo = json.loads(files["../config/kinfo-gfx950.json"])
     pairs = gen_run.be_pairs()
-    assert pairs == [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"), ("lbm", "stencil"),
+    assert pairs == [("cp", "lbm"), ("cp", "mrif"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mrif"),
+                     ("lbm", "mriq"), ("lbm", "stencil"), ("mrif", "mriq"), ("mrif", "stencil"),
                      ("mriq", "stencil")]
+    assert ("lbm", "mrif") in pairs and ("mrif", "stencil") in pairs   # src/mix_kernel/lbm_mrif_1_3.cu, mrif_stencil_3_2.cu
     assert ("lbm", "mriq") in pairs                       # the pair src/Creator.cu:341-816 also has
     for a, b in pairs:
         text = files[f"mix_kernel/{a}_{b}.hip"]

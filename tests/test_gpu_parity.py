@@ -12,8 +12,8 @@ import torch
 
 import oracle
 import tacker_amd as ta
-from gpu_util import (C0, C1, dev, gemm_inputs, gemm_tolerance_ok, host, lbm_inputs, mriq_inputs, setup,
-                      stencil_inputs)
+from gpu_util import (C0, C1, dev, gemm_inputs, gemm_tolerance_ok, host, lbm_inputs, mrif_inputs, mrif_table,
+                      mriq_inputs, setup, stencil_inputs)
 
 pytestmark = pytest.mark.gpu
 
@@ -732,13 +732,20 @@ def _small_be(name):
         Qr, Qi = torch.zeros(2048, device="cuda:0"), torch.zeros(2048, device="cuda:0")
         return (ta.ori_mriq_create(256, dev(xyz[0]), dev(xyz[1]), dev(xyz[2]), Qr, Qi), ta.mriq_blocks(256, 2048),
                 [Qr, Qi])
+    if name == "mrif":
+        k, phi, d, xyz = mrif_inputs(256, 2048, seed=34)
+        ta.mrif_set_kvalues(mrif_table(k, phi, d))
+        outR, outI = torch.zeros(2048, device="cuda:0"), torch.zeros(2048, device="cuda:0")
+        return (ta.ori_mrif_create(256, dev(xyz[0]), dev(xyz[1]), dev(xyz[2]), outR, outI), ta.mrif_blocks(256, 2048),
+                [outR, outI])
     ta.cp_set_atoms(cp_atoms(), 0.0)
     g = torch.zeros((32, 512), device="cuda:0")
     return ta.ori_cp_create(64, 0.1, g), ta.cp_blocks(512, 32), [g]
 
 
 @pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),
-                                          ("lbm", "stencil"), ("mriq", "stencil")])
+                                          ("lbm", "stencil"), ("mriq", "stencil"), ("cp", "mrif"), ("lbm", "mrif"),
+                                          ("mrif", "mriq"), ("mrif", "stencil")])
 @pytest.mark.parametrize("variant", [None, "wg_1_2", "wg_2_1", "ord_1_1", "ord_1_2"])
 def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
     ori1, n1, outs1 = _small_be(first)

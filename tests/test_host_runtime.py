@@ -208,7 +208,7 @@ def test_mix_parameter_vector_matches_reference_signature(fake):
     assert [as_int(x) for x in a[29:32]] == [3, grid, 20]
 
 
-@pytest.mark.parametrize("be,n_be", [("lbm", 2), ("mriq", 7), ("cp", 3)])
+@pytest.mark.parametrize("be,n_be", [("lbm", 2), ("mriq", 7), ("mrif", 7), ("cp", 3)])
 def test_other_mix_vectors_have_reference_lengths(fake, be, n_be):
     fake.tk_fake_reset()
     buf = np.zeros(1 << 16, np.float32)
@@ -220,12 +220,14 @@ def test_other_mix_vectors_have_reference_lengths(fake, be, n_be):
         rc = fake.tacker_mix_tzgemm_lbm(p, p, 8, 4, 4, 0, 16, *g)
     elif be == "mriq":
         rc = fake.tacker_mix_tzgemm_mriq(16, p, p, p, p, p, 512, 0, 2, *g)
+    elif be == "mrif":
+        rc = fake.tacker_mix_tzgemm_mrif(16, p, p, p, p, p, 512, 0, 2, *g)
     else:
         rc = fake.tacker_mix_tzgemm_cp(64, 0.1, p, 256, 16, 0, 4, *g)
     assert rc == 0, fake.tacker_last_error()
     (l,) = launches(fake)
-    # lbm_tzgemm_mix 11+15, mriq_tzgemm_mix 16+15, cp_tzgemm_mix 12+15
-    # (src/mix_kernel/tzgemm_{lbm,mriq,cp}.cu dispatcher signatures), plus the GEMM's workspace pointer
+    # lbm_tzgemm_mix 11+15, mriq_tzgemm_mix and mrif_tzgemm_mix 16+15, cp_tzgemm_mix 12+15
+    # (src/mix_kernel/tzgemm_{lbm,mriq,mrif,cp}.cu dispatcher signatures), plus the GEMM's workspace pointer
     assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 16
 
 
@@ -327,6 +329,8 @@ def test_argument_validation_returns_codes_instead_of_exiting(fake):
     assert fake.tacker_gptb_tzgemm(p, p, p, 128, 128, 128, 0, 5, 0, None) == 1        # range beyond the 4 tiles
     assert fake.tacker_gptb_stencil(0.1, 0.1, p, p, 8, 8, 8, 0, 1, 4, 100, None) == 1  # block not a multiple of 64
     assert fake.tacker_ori_mriq(8, p, p, p, p, p, 100, None) == 3
+    assert fake.tacker_ori_mrif(8, p, p, p, p, p, 100, None) == 3
+    assert fake.tacker_gptb_mrif(5000, p, p, p, p, p, 256, 0, 1, 0, 0, None) == 1     # more samples than the table holds
     assert fake.tacker_ori_cp(65, 0.1, p, 128, 8, None) == 1
     assert fake.tacker_mix_tzgemm_stencil(0.1, 0.1, p, p, 8, 8, 8, 0, 1, p, p, p, 128, 128, 128, 0, 4,
                                           b"no_such_variant", 0, 0, None) == 2
@@ -347,6 +351,13 @@ def test_constant_tables_reach_the_device_layer(fake):
     fake.tk_fake_symbol(b"atominfo", out.ctypes.data, 32)
     assert np.array_equal(out.reshape(2, 4), np.array([[1, 2, 4, 0.5], [4, 5, 4, -0.25]], np.float32))
     assert fake.tacker_mriq_set_kvalues(kv.ctypes.data, 5000) == 1
+    kf = np.arange(15, dtype=np.float32).reshape(3, 5)
+    assert fake.tacker_mrif_set_kvalues(kf.ctypes.data, 3) == 0
+    out = np.zeros(15, np.float32)
+    assert fake.tk_fake_symbol(b"c_mrif", out.ctypes.data, 60) >= 60
+    assert np.array_equal(out, kf.reshape(-1))
+    assert fake.tacker_mrif_set_kvalues(kf.ctypes.data, 5000) == 1
+    assert fake.tacker_mrif_blocks(2048, 262144) == 16384
 
 
 def test_create_kernel_geometry_and_memoisation(fake):
