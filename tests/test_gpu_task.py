@@ -196,6 +196,31 @@ def test_task_manager_colocation_keeps_lc_results_and_reports():
     task.close()
 
 
+def test_task_manager_colocates_mrif_and_pairs_it_with_lbm():
+    # the fifth best-effort kernel through the same scheduler: tzgemm_mrif launches in stage 1,
+    # the lbm_mrif pair (src/mix_kernel/lbm_mrif_1_3.cu) in stage 2
+    task = ta.LcTask("vgg16", 64, 64)
+    task.execute()
+    torch.cuda.synchronize()
+    p, stride, n = task.logits()
+    solo_logits = ta.device_to_host(p, (n, stride), np.float32)[:, 0].copy()
+    tm = ta.TaskManager(task, "lbm", "mrif")
+    tm.configure(qos_budget_ms=50.0, guard_ms=0.5, warmup=1, profile=3, queries=3, verbose=0)
+    rep = tm.run("aker", second_stage=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
+    assert rep["mixable_times"] == 16 and rep["be1_solo_ms"] > 0 and rep["n_colocated"] == 3
+    tm.close()
+    tm = ta.TaskManager(task, "mrif", None)
+    tm.configure(qos_budget_ms=50.0, guard_ms=0.5, warmup=1, profile=3, queries=3, verbose=0)
+    rep = tm.run("aker", second_stage=False)
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
+    assert rep["n_colocated"] == 3 and ta.spin_fail_flag() == 0
+    tm.close()
+    task.close()
+
+
 def test_create_kernel_objects_run_and_match_oracle_for_cp():
     k = ta.create_kernel("cp")
     info = k.info()
@@ -203,7 +228,7 @@ def test_create_kernel_objects_run_and_match_oracle_for_cp():
     assert (info["ptb_start"], info["ptb_end"]) == (0, 65536) and info["ori_grid_x"] == 32 and info["ori_grid_y"] == 512
     k.execute()
     torch.cuda.synchronize()
-    for name in ("stencil", "lbm", "mriq"):
+    for name in ("stencil", "lbm", "mriq", "mrif"):
         ta.create_kernel(name).execute()
     torch.cuda.synchronize()
     assert ta.spin_fail_flag() == 0
