@@ -62,6 +62,14 @@ def main():
     # im2col 3 x 6 x 7, 3x3, pad 1
     im = rng.uniform(-1, 1, (3, 6, 7)).astype(np.float32)
     out.update(im2col_im=im, im2col_col=oracle.im2col(im, (3, 3), (1, 1), (1, 1)))
+    # mri-fhd 96 samples x 512 voxels (drawn last: the entries above keep their values)
+    fk = rng.uniform(-0.5, 0.5, (96, 3)).astype(np.float32)
+    fphi, fd = rng.uniform(0, 1, (2, 96)).astype(np.float32), rng.uniform(0, 1, (2, 96)).astype(np.float32)
+    fxyz = rng.uniform(-0.5, 0.5, (3, 512)).astype(np.float32)
+    re, im_ = oracle.mrif_rhophi(fphi[0], fphi[1], fd[0], fd[1])
+    fkv = np.concatenate([fk, re[:, None], im_[:, None]], 1).astype(np.float32)
+    fr, fi = oracle.mrif(fkv, *fxyz, z, z, f64=True)
+    out.update(mrif_phi=fphi, mrif_d=fd, mrif_kvals=fkv, mrif_xyz=fxyz, mrif_outR=fr, mrif_outI=fi)
     path = os.path.join(HERE, "kernels_small.npz")
     np.savez_compressed(path, **out)
     print("wrote", path, os.path.getsize(path), "bytes")

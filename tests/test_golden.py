@@ -30,6 +30,10 @@ def test_oracle_reproduces_golden_vectors():
     assert np.array_equal(oracle.cp(oracle.cp_atoms_to_const(G["cp_atoms"], 0.0), np.zeros((16, 256), np.float32)),
                           G["cp_grid"])
     assert np.array_equal(oracle.im2col(G["im2col_im"], (3, 3), (1, 1), (1, 1)), G["im2col_col"])
+    re, im = oracle.mrif_rhophi(G["mrif_phi"][0], G["mrif_phi"][1], G["mrif_d"][0], G["mrif_d"][1])
+    assert np.array_equal(re, G["mrif_kvals"][:, 3]) and np.array_equal(im, G["mrif_kvals"][:, 4])
+    fr, fi = oracle.mrif(G["mrif_kvals"], *G["mrif_xyz"], z, z, f64=True)
+    assert np.array_equal(fr, G["mrif_outR"]) and np.array_equal(fi, G["mrif_outI"])
 
 
 @pytest.mark.gpu
@@ -69,3 +73,9 @@ def test_hip_path_matches_golden_vectors():
     col = torch.zeros(G["im2col_col"].shape, device="cuda:0")
     ta.im2col(dev(G["im2col_im"]), (3, 3), (1, 1), (1, 1), (1, 1), col)
     assert np.array_equal(host(col), G["im2col_col"])
+    ta.mrif_set_kvalues(G["mrif_kvals"])
+    outR, outI = torch.zeros(512, device="cuda:0"), torch.zeros(512, device="cuda:0")
+    x, y, z = (dev(v) for v in G["mrif_xyz"])
+    ta.gptb_mrif(96, x, y, z, outR, outI)
+    for got, want in ((host(outR), G["mrif_outR"]), (host(outI), G["mrif_outI"])):
+        assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-3 + 1e-4 * np.abs(want))

@@ -178,6 +178,41 @@ def test_config4_mriq_spread_over_nine_fused_launches_equals_one_launch():
     assert ta.spin_fail_flag() == 0
 
 
+def test_mrif_2048x262144_spread_over_ten_fused_launches_equals_one_launch():
+    # mri-fhd at mri-q's benchmark size (the reference's tzgemm_mrif mix): the position grid cut into 10
+    # consecutive slices, each riding with one 2048^3 GEMM launch, gives the bits of the natural launch; a
+    # sample of voxels is checked against a complex128 matrix product in numpy
+    from gpu_util import mrif_inputs, mrif_table
+    M = N = K = 2048
+    A, B = gemm_inputs(M, N, K, seed=24)
+    numK, numX = 2048, 262144
+    k, phi, d, xyz = mrif_inputs(numK, numX, seed=6)
+    kv = mrif_table(k, phi, d)
+    ta.mrif_set_kvalues(kv)
+    x, y, z = dev(xyz[0]), dev(xyz[1]), dev(xyz[2])
+    dA, dB = dev(A), dev(B)
+    solo_r, solo_i = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    ta.ori_mrif(numK, x, y, z, solo_r, solo_i)
+    solo_c = torch.zeros((M, N), device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, solo_c)
+    outR, outI = torch.zeros(numX, device="cuda:0"), torch.zeros(numX, device="cuda:0")
+    mix_c = torch.zeros((M, N), device="cuda:0")
+    total = ta.mrif_blocks(numK, numX)
+    assert total == 1024 * 16
+    n = 10
+    for i in range(n):
+        ta.mix_tzgemm_mrif(numK, x, y, z, outR, outI, dA, dB, mix_c, be_start=total * i // n, be_end=total * (i + 1) // n)
+    got_r, got_i = host(outR), host(outI)
+    assert np.array_equal(got_r, host(solo_r)) and np.array_equal(got_i, host(solo_i))
+    assert np.array_equal(host(mix_c), host(solo_c))
+    pick = np.random.default_rng(3).choice(numX, 512, replace=False)
+    X = np.stack([xyz[0][pick], xyz[1][pick], xyz[2][pick]], 1).astype(np.float64)
+    want = np.exp(2j * np.pi * (X @ kv[:, :3].astype(np.float64).T)) @ (kv[:, 3].astype(np.float64) + 1j * kv[:, 4])
+    assert np.all(np.abs(got_r[pick] - want.real) <= 1e-3 + 1e-4 * np.abs(want.real))
+    assert np.all(np.abs(got_i[pick] - want.imag) <= 1e-3 + 1e-4 * np.abs(want.imag))
+    assert ta.spin_fail_flag() == 0
+
+
 def test_config5_vgg16_224_colocated_queries_equal_the_solo_query():
     # VGG16 batch 1 at 224x224 under TaskManager, with the reference's always-fuse policy and the kinfo
     # block counts (mri-q, then the stencil), then with calibrated counts and mri-q: whatever rides along, the logits are the solo query's bit for bit, no role barrier was
