@@ -164,8 +164,8 @@ def pair_leg(ta, torch, np, name, stream):
     out["be_blocks"] = nblk
     if slice_blocks > 0:
         out["slice_speedup"] = round(out["slice_serial_us"] / out["slice_fused_us"], 4)
-    if name in ("mriq", "mrif"):
-        # the long best-effort kernel spread over the GEMMs it rides with: n = T_be / T_gemm fused launches,
+    if out["be_us"] > 1.3 * out["gemm_us"]:
+        # the longer best-effort kernel spread over the GEMMs it rides with: n = T_be / T_gemm fused launches,
         # each carrying the next 1/n of the block positions, against n GEMM launches plus the kernel alone
         n_cur = max(1, int(round(out["be_us"] / out["gemm_us"])))
         bounds = [nblk * i // n_cur for i in range(n_cur + 1)]
