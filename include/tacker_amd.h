@@ -125,7 +125,8 @@ TK_API int tacker_tzgemm_grid_dim(int m, int n, int k, int out[4]);
  * with few tiles and a long reduction (the batch-1 layers of src/dnn/: 32-128 tiles, K up to
  * 25088) cut the reduction of a tile over `parts` workgroups; the partial tiles and one arrival
  * counter per tile live in a workspace the library binds to the output buffer C on the first
- * GEMM that writes it (general_ptb_tzgemm's seventh parameter; NULL when parts == 1).
+ * GEMM that writes it; the kernels, whose parameter lists are the reference's, find it by looking
+ * C up in a device-resident table the binding fills (nothing is bound when parts == 1).
  * tacker_tzgemm_parts: the number of parts for (m, n, k) rounded as tacker_tzgemm_grid_dim
  * rounds them -- a function of the shape only, so fused and unfused launches add in the same
  * order. tacker_tzgemm_workspace_bytes: size of that workspace, 0 when parts == 1.
@@ -345,8 +346,11 @@ TK_API int tacker_kernel_swap_buffers(tacker_kernel_t ori);
  * parameters, smem, ori grid x, ori grid y} (start/end are 0 for non-GPTB objects) */
 TK_API int tacker_kernel_info(tacker_kernel_t kernel, int out[8]);
 TK_API int tacker_kernel_destroy(tacker_kernel_t kernel);
-/* value of the device flag a role-local barrier raises when it gives up waiting
- * (wave-split fused kernels); reading clears it. 0 = no barrier ever timed out */
+/* value of the device word kernels raise when they have to give up; reading clears it.
+ * Bit 0: a role-local barrier of a wave-split fused kernel stopped waiting (its poll is
+ * bounded). Bit 1: a GEMM whose reduction is shared by workgroups found no workspace bound to
+ * its C (a hand-made launch on a buffer the library never saw) and left C untouched.
+ * 0 = neither ever happened */
 TK_API int tacker_spin_fail_flag(int *flag);
 /* host half conversion used for the synthetic GEMM operands (round to nearest even) */
 TK_API uint16_t tacker_float_to_half_bits(float f);

@@ -83,4 +83,23 @@ TZ_HOST_DEVICE inline long long tz_workspace_bytes(int M, int N, int K)
     return tz_workspace_counter_bytes(M, N) + n_ref * parts * TZ_PARTIAL_TILE_BYTES;
 }
 
+// Where a kernel finds the workspace of the output buffer it writes: a device-resident hash
+// table from C to workspace that the host fills when it binds one (open addressing, linear
+// probing, an entry is never moved or removed while kernels may run; key 0 = empty).  The
+// reference's tzgemm has no such buffer and its parameter list (A, B, C, M, N, K) has no slot for
+// one, so the kernels look it up by the pointer they are given anyway.
+#define TZ_WS_TABLE_SLOTS 1024
+#define TZ_WS_TABLE_MAX_PROBES 16
+struct tz_ws_entry {
+    unsigned long long c;           // output buffer (device address), 0 = empty slot
+    unsigned long long workspace;   // its workspace
+};
+TZ_HOST_DEVICE inline unsigned tz_ws_hash(unsigned long long c)
+{
+    return (unsigned)(((c >> 8) * 0x9E3779B97F4A7C15ull) >> 54) & (TZ_WS_TABLE_SLOTS - 1);
+}
+// bits of the device word tk_spin_fail
+#define TK_FAIL_SPIN 1u        // a role-local barrier gave up waiting
+#define TK_FAIL_WORKSPACE 2u   // a GEMM whose reduction is shared by workgroups found no workspace for its C
+
 #define TZ_ALPHA 1.1f             // alpha_g, src/header/tzgemm_header.h:64

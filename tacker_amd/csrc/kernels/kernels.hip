@@ -99,13 +99,13 @@ extern "C" __global__ __launch_bounds__(128) void ori_cp(int numatoms, float gri
 // ------------------------------------------------------------------ GPTB kernels
 
 extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void general_ptb_tzgemm(
-    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, unsigned *workspace, GPTB_TRAILER)
+    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, GPTB_TRAILER)
 {
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
     tk::WorkgroupSync sync;
-    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, workspace, (int)blockIdx.x, ptb_iter_block_step,
-                    ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base, tz_lds,
-                    sync);
+    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, tk::tz_workspace_of(C, M_GLOBAL, N_GLOBAL, K_GLOBAL),
+                    (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
+                    (int)threadIdx.x - thread_base, tz_lds, sync);
 }
 
 extern "C" __global__ __launch_bounds__(256) void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
@@ -254,6 +254,11 @@ extern "C" int tk_device_symbol(const char *name, const void **symbol, size_t *b
     if (__builtin_strcmp(name, "atominfo") == 0) {
         *symbol = (const void *)&atominfo;
         *bytes = sizeof(atominfo);
+        return TK_SUCCESS;
+    }
+    if (__builtin_strcmp(name, "tz_ws_table") == 0) {
+        *symbol = (const void *)&tz_ws_table;
+        *bytes = sizeof(tz_ws_table);
         return TK_SUCCESS;
     }
     if (__builtin_strcmp(name, "tk_spin_fail") == 0) {

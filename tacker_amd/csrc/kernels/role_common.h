@@ -15,6 +15,9 @@
 #include <hip/hip_runtime.h>
 #include "../header/pets_common.h"
 
+// Raised by device code that has to give up (bits TK_FAIL_*), read and cleared by the host.
+__device__ unsigned tk_spin_fail = 0u;
+
 namespace tk {
 
 typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
@@ -126,7 +129,7 @@ struct RoleSpinSync {
     // once, when the role is over: tell the host if any barrier was abandoned
     __device__ __forceinline__ void finish()
     {
-        if (gave_up && fail) *fail = 1u;
+        if (gave_up && fail) __hip_atomic_fetch_or(fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 };
 

@@ -43,7 +43,32 @@
 #include "role_common.h"
 #include "../header/tzgemm_header.h"
 
+// Output buffer -> workspace, filled by the host when it binds a workspace to a C
+// (tzgemmWorkspaceFor); see tz_ws_entry.
+__device__ tz_ws_entry tz_ws_table[TZ_WS_TABLE_SLOTS];
+
 namespace tk {
+
+// The workspace bound to output buffer C, nullptr if there is none.  C is a kernel argument, so
+// the probes are scalar loads; the host never lets a key sit more than TZ_WS_TABLE_MAX_PROBES
+// slots from its hash.
+__device__ __forceinline__ unsigned *tz_find_workspace(const float *C)
+{
+    const unsigned long long key = (unsigned long long)(size_t)C;
+    unsigned slot = tz_ws_hash(key);
+    for (int probe = 0; probe < TZ_WS_TABLE_MAX_PROBES; ++probe) {
+        const unsigned long long c = tz_ws_table[slot].c;
+        if (c == key) return reinterpret_cast<unsigned *>((size_t)tz_ws_table[slot].workspace);
+        if (c == 0ull) return nullptr;
+        slot = (slot + 1) & (TZ_WS_TABLE_SLOTS - 1);
+    }
+    return nullptr;
+}
+// ... for a GEMM of this shape: only the shapes whose reduction is shared by workgroups look.
+__device__ __forceinline__ unsigned *tz_workspace_of(const float *C, int M, int N, int K)
+{
+    return tz_ksplit_parts(M, N, K) > 1 ? tz_find_workspace(C) : nullptr;
+}
 
 // Persistent-loop index -> macro tile (row, column).  With role_blocks a multiple
 // of 8, loop index t runs on XCD t % 8.  Each XCD takes a contiguous run of the
@@ -475,7 +500,13 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
     const int frag_seg1 = ((4 + (lane >> 4)) ^ frag_key) * 16;
     const int frag_row = (lane & 15) * ROWB;
     if (tile_end > n_ref) tile_end = n_ref;
-    if (parts > 1 && workspace == nullptr) tile_end = tile_start;   // the host always binds one; never fault
+    if (parts > 1 && workspace == nullptr) {
+        // the host binds one to every C it builds a kernel object on; a launch that reaches this
+        // point without one computes nothing and says so (TK_FAIL_WORKSPACE), it never faults
+        if (tid == 0 && role_block == 0)
+            __hip_atomic_fetch_or(&tk_spin_fail, TK_FAIL_WORKSPACE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        tile_end = tile_start;
+    }
     const int tiles = tile_end - tile_start;
     const int units = tiles > 0 ? tiles * parts : 0;
 

@@ -27,8 +27,6 @@ bool gemm_malloced = false;
 void *ori_wmma_A = nullptr;
 void *ori_wmma_B = nullptr;
 float *ori_wmma_C = nullptr;
-long long MAX_ORI_WMMA_WS = 0;
-void *ori_wmma_workspace = nullptr;
 
 static void grow(void **ptr, long long *have, long long need, bool seed_halves)
 {
@@ -44,6 +42,7 @@ static void grow(void **ptr, long long *have, long long need, bool seed_halves)
         TK_SAFE_CALL(tkMemcpy(*ptr, host.data(), (size_t)need, TK_MEMCPY_H2D));
     } else {
         TK_SAFE_CALL(tkMemset(*ptr, 0, (size_t)need));
+        TK_SAFE_CALL(tkDeviceSynchronize());   // zero before a kernel on any stream touches it
     }
 }
 
@@ -58,7 +57,6 @@ void ensureGlobalGemmBuffers(int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
     grow(&ori_wmma_A, &MAX_ORI_WMMA_A, a, true);
     grow(&ori_wmma_B, &MAX_ORI_WMMA_B, b, true);
     grow((void **)&ori_wmma_C, &MAX_ORI_WMMA_C, c, false);
-    grow(&ori_wmma_workspace, &MAX_ORI_WMMA_WS, tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL), false);
     gemm_malloced = true;
 }
 
@@ -69,8 +67,27 @@ struct BoundWorkspace {
 };
 std::mutex g_workspace_mutex;
 std::unordered_map<const void *, BoundWorkspace> g_workspaces;   // by output buffer
-std::vector<void *> g_outgrown_workspaces;   // replaced by a larger one; older kernel objects may still hold them
-constexpr size_t kMaxBoundWorkspaces = 1024;
+std::vector<void *> g_outgrown_workspaces;   // replaced by a larger one; launches in flight may still use them
+constexpr size_t kMaxBoundWorkspaces = TZ_WS_TABLE_SLOTS / 2;   // load factor of the device table
+std::vector<tz_ws_entry> g_table_mirror(TZ_WS_TABLE_SLOTS, tz_ws_entry{0, 0});   // host copy of tz_ws_table
+
+// Enters (C, workspace) into the device table, or updates C's entry.  A slot is written with one
+// 16-byte copy and never moves, so a kernel that runs meanwhile and probes past it for another key
+// sees it either empty or whole.
+void publish_workspace(const void *C, void *workspace)
+{
+    const unsigned long long key = (unsigned long long)(size_t)C;
+    unsigned slot = tz_ws_hash(key);
+    for (int probe = 0; probe < TZ_WS_TABLE_MAX_PROBES; ++probe, slot = (slot + 1) & (TZ_WS_TABLE_SLOTS - 1)) {
+        if (g_table_mirror[slot].c != key && g_table_mirror[slot].c != 0) continue;
+        g_table_mirror[slot] = tz_ws_entry{key, (unsigned long long)(size_t)workspace};
+        TK_SAFE_CALL(tkMemcpyToSymbol("tz_ws_table", &g_table_mirror[slot], sizeof(tz_ws_entry),
+                                      slot * sizeof(tz_ws_entry)));
+        return;
+    }
+    throw std::runtime_error("tzgemm: the device table of workspaces has no free slot near this output "
+                             "buffer's hash; call tzgemmReleaseWorkspaces() once the kernels that use them are gone");
+}
 }  // namespace
 
 void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
@@ -89,6 +106,12 @@ void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBA
     TK_SAFE_CALL(tkMalloc(&ptr, (size_t)need));
     TK_SAFE_CALL(tkMemset(ptr, 0, (size_t)need));
     TK_SAFE_CALL(tkDeviceSynchronize());   // zero before any stream's kernel reads the counters
+    try {
+        publish_workspace(C, ptr);
+    } catch (...) {
+        tkErrCheck(tkFree(ptr));
+        throw;
+    }
     if (it != g_workspaces.end()) g_outgrown_workspaces.push_back(it->second.ptr);
     g_workspaces[C] = BoundWorkspace{ptr, need};
     return ptr;
@@ -102,6 +125,8 @@ void tzgemmReleaseWorkspaces()
     for (void *p : g_outgrown_workspaces) TK_SAFE_CALL(tkFree(p));
     g_workspaces.clear();
     g_outgrown_workspaces.clear();
+    std::fill(g_table_mirror.begin(), g_table_mirror.end(), tz_ws_entry{0, 0});
+    TK_SAFE_CALL(tkMemcpyToSymbol("tz_ws_table", g_table_mirror.data(), g_table_mirror.size() * sizeof(tz_ws_entry), 0));
 }
 
 static void fmap_insert(const char *key, const void *func, void *)

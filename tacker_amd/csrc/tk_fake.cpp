@@ -51,7 +51,7 @@ const std::vector<int> LBM = {P, P};
 const std::vector<int> MRIQ = {I, I, P, P, P, P, P};
 const std::vector<int> MRIF = {I, I, P, P, P, P, P};
 const std::vector<int> CP = {I, F, P};
-const std::vector<int> TZ = {P, P, P, I, I, I, P};
+const std::vector<int> TZ = {P, P, P, I, I, I};
 }  // namespace
 
 extern "C" {
@@ -77,7 +77,8 @@ int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int, tkStream_t) { m
 int tkMemset(void *ptr, int value, size_t bytes) { memset(ptr, value, bytes); return TK_SUCCESS; }
 int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset)
 {
-    if (strcmp(symbol, "ck") && strcmp(symbol, "c_mrif") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail"))
+    if (strcmp(symbol, "ck") && strcmp(symbol, "c_mrif") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail") &&
+        strcmp(symbol, "tz_ws_table"))
         return TK_ERROR_NOT_FOUND;
     auto &buf = g_symbols[symbol];
     if (buf.size() < offset + bytes) buf.resize(offset + bytes);

@@ -9,11 +9,11 @@
 //
 // Differences: the global buffers grow on demand (the reference sizes them once,
 // from the first shape it sees), and a second constructor binds caller-owned
-// buffers, which is what the C entry points use.  A seventh parameter carries the
-// kernel's workspace (partial tiles and arrival counters of the shapes whose
-// reduction is cut over several workgroups, nullptr for all others): a fourth
-// global buffer beside A, B and C, or, for caller-owned operands, a buffer the
-// library keeps for that C (tzgemmWorkspaceFor).
+// buffers, which is what the C entry points use.  The parameter list is the
+// reference's six.  The shapes whose reduction is cut over several workgroups
+// need a workspace (partial tiles and arrival counters); the library keeps one
+// per output buffer C (tzgemmWorkspaceFor) and publishes the pair in a
+// device-resident table in which the kernels look their C up.
 #pragma once
 
 #include <algorithm>
@@ -31,8 +31,6 @@ extern bool gemm_malloced;
 extern void *ori_wmma_A;           // f16 [M][K]
 extern void *ori_wmma_B;           // f16 [N][K]
 extern float *ori_wmma_C;          // f32 [M][N]
-extern long long MAX_ORI_WMMA_WS;
-extern void *ori_wmma_workspace;   // counters + partial tiles, zero between launches
 
 inline int tzgemmRoundDim(int x) { return (x < 128) ? 128 : (x / 128) * 128; }
 
@@ -51,10 +49,11 @@ inline std::vector<int> getTZGEMMGridDim(int m, int n, int k)
 // leaves them zero after cudaMemset; synthetic operands make the result checkable).
 void ensureGlobalGemmBuffers(int M_GLOBAL, int N_GLOBAL, int K_GLOBAL);
 
-// Workspace for GEMMs that write the caller-owned buffer C: nullptr when the shape needs none,
-// else a zeroed device buffer of at least tz_workspace_bytes(M, N, K) that stays bound to C until
-// the process ends (or until a larger one replaces it).  Launches that write the same C must not
-// overlap anyway, so they can share it; launches on different C never do.  Thread-safe.
+// Workspace for GEMMs that write the buffer C: nullptr when the shape needs none, else a zeroed
+// device buffer of at least tz_workspace_bytes(M, N, K) that stays bound to C until
+// tzgemmReleaseWorkspaces (or until a larger one replaces it), entered into the device table
+// tz_ws_table where the kernels find it.  Launches that write the same C must not overlap anyway,
+// so they can share it; launches on different C never do.  Thread-safe.
 void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL);
 // Frees every such workspace after a device synchronisation.  Only when no kernel object built on
 // caller-owned operands is left (they keep the pointer they were given).
@@ -88,7 +87,7 @@ public:
         K_GLOBAL = d[2];
         ori_blks = d[3];
         if (useGlobals) ensureGlobalGemmBuffers(M_GLOBAL, N_GLOBAL, K_GLOBAL);
-        else workspace_ = tzgemmWorkspaceFor(C_, M_GLOBAL, N_GLOBAL, K_GLOBAL);
+        tzgemmWorkspaceFor(useGlobals ? ori_wmma_C : C_, M_GLOBAL, N_GLOBAL, K_GLOBAL);
 
         launchGridDim = dim3(ori_blks, 1, 1);
         launchBlockDim = dim3(TZ_THREADS, 1, 1);
@@ -99,7 +98,6 @@ public:
         kernelParams.push_back(&M_GLOBAL);
         kernelParams.push_back(&N_GLOBAL);
         kernelParams.push_back(&K_GLOBAL);
-        kernelParams.push_back(useGlobals ? (void *)&ori_wmma_workspace : (void *)&workspace_);
         this->smem = TZ_LDS_BYTES;
     }
 
@@ -123,5 +121,4 @@ private:
     void *A_ = nullptr;
     void *B_ = nullptr;
     float *C_ = nullptr;
-    void *workspace_ = nullptr;
 };

@@ -23,12 +23,11 @@ GPTB_RANGE = ["ptb_start_block_pos", "ptb_iter_block_step", "ptb_end_block_pos"]
 ROLES = {
     "tzgemm": {
         "params": [("_Float16*", "A"), ("_Float16*", "B"), ("float*", "C"),
-                   ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K"),
-                   ("unsigned*", "workspace")],
+                   ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K")],
         "needs_sync": True,
         "lds_bytes": "TZ_LDS_BYTES",
         "call": ("tk::tzgemm_role<{stages}, {stream_c}>({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, "
-                 "{p}workspace, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "tk::tz_workspace_of({p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K), {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "tz_lds, sync);"),
     },
     "stencil": {

@@ -76,17 +76,19 @@ def test_committed_generated_sources_are_fresh():
     assert rc.returncode == 0, rc.stdout + rc.stderr
 
 
-@pytest.mark.parametrize("be,n_params", [("stencil", 32), ("lbm", 27), ("mriq", 32), ("cp", 28)])
+@pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27)])
 def test_emitted_dispatcher_signature(be, n_params):
-    # parameter count = the reference dispatcher's (src/mix_kernel/tzgemm_<be>.cu) plus the GEMM's
-    # workspace pointer, order: be first
+    # parameter count = the reference dispatcher's (src/mix_kernel/tzgemm_stencil.cu:281-283 31,
+    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27), order: be first
     text, meta = gen_mix.generate_wg_split(be, 1, 1)
     sig = re.search(r"void (\w+)\(\s*(.*?)\)\s*\{", text, re.S)
     params = [p.strip() for p in sig.group(2).split(",")]
     assert len(params) == n_params and sig.group(1) == f"{be}_tzgemm_mix_wg_1_1"
     names = [p.split()[-1] for p in params]
     assert names[0].startswith(f"{be}0_") and names[-1] == "tzgemm1_ptb_end_block_pos"
-    assert names[-16:-13] == ["tzgemm1_A", "tzgemm1_B", "tzgemm1_C"] and names[-10] == "tzgemm1_workspace"
+    assert names[-15:-9] == ["tzgemm1_A", "tzgemm1_B", "tzgemm1_C", "tzgemm1_NORMAL_M", "tzgemm1_NORMAL_N",
+                             "tzgemm1_NORMAL_K"]
+    assert names[-9] == "tzgemm1_grid_dimension_x"
     assert names[-3:] == ["tzgemm1_ptb_start_block_pos", "tzgemm1_ptb_iter_block_step", "tzgemm1_ptb_end_block_pos"]
     assert meta["blocksize"] == 256 and meta["group"] == 2
     wave, wmeta = gen_mix.generate_wave_split(be, 256)

@@ -149,14 +149,54 @@ def test_tzgemm_workspace_is_bound_to_the_output_buffer(fake):
     A = np.zeros((256, 1024), np.float16)
     C1 = np.zeros((256, 256), np.float32)
     C2 = np.zeros((256, 256), np.float32)
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+
+    def table():
+        # the device table the kernels look their output buffer up in: {C, workspace} per slot
+        raw = C.create_string_buffer(1024 * 16)
+        n = fake.tk_fake_symbol(b"tz_ws_table", raw, len(raw))
+        words = struct.unpack(f"<{n // 8}Q", raw.raw[:n])
+        return {words[i]: words[i + 1] for i in range(0, len(words), 2) if words[i]}
+
+    assert table() == {}
     seen = []
     for Cm in (C1, C1, C2):
         assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 256, 256, 1024, 0, 16, 0, None) == 0
-        seen.append(as_ptr(launches(fake)[-1]["args"][6]))
+        # general_ptb_tzgemm(A, B, C, M, N, K, 6 dims, start, step, end, thread_base)
+        # (src/gptb_kernel/tzgemm_kernel.cu:430-433): no workspace argument
+        assert len(launches(fake)[-1]["args"]) == 16
+        seen.append(table().get(Cm.ctypes.data, 0))
     assert seen[0] != 0 and seen[0] == seen[1] and seen[2] not in (0, seen[0])
-    # a shape without shared reductions gets none
-    assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, C1.ctypes.data, 256, 256, 128, 0, 16, 0, None) == 0
-    assert as_ptr(launches(fake)[-1]["args"][6]) == 0
+    assert set(table()) == {C1.ctypes.data, C2.ctypes.data}
+    # a shape without shared reductions binds none
+    C3 = np.zeros((256, 256), np.float32)
+    assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, C3.ctypes.data, 256, 256, 128, 0, 16, 0, None) == 0
+    assert C3.ctypes.data not in table()
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+    assert table() == {}
+
+
+def test_workspace_table_slots_follow_the_hash_the_kernels_probe(fake):
+    # slot = top 10 bits of (C >> 8) * 0x9E3779B97F4A7C15 mod 2^64, linear probing: the rule the
+    # device-side lookup applies (csrc/header/tzgemm_header.h tz_ws_hash)
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+    A = np.zeros((256, 1024), np.float16)
+    outs = [np.zeros((256, 256), np.float32) for _ in range(24)]
+    for Cm in outs:
+        assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 256, 256, 1024, 0, 16, 0, None) == 0
+    raw = C.create_string_buffer(1024 * 16)
+    n = fake.tk_fake_symbol(b"tz_ws_table", raw, len(raw))
+    words = struct.unpack(f"<{n // 8}Q", raw.raw[:n]) + (0,) * (2048 - n // 8)
+    for Cm in outs:
+        key = Cm.ctypes.data
+        slot = (((key >> 8) * 0x9E3779B97F4A7C15) % (1 << 64)) >> 54
+        for probe in range(16):
+            c = words[2 * ((slot + probe) % 1024)]
+            assert c != 0, "an empty slot before the key: the device lookup would stop here"
+            if c == key:
+                break
+        else:
+            raise AssertionError("key not within 16 probes of its hash")
     assert fake.tacker_tzgemm_release_workspaces() == 0
 
 
@@ -193,9 +233,8 @@ def test_mix_parameter_vector_matches_reference_signature(fake):
     assert rc == 0, fake.tacker_last_error()
     (l,) = launches(fake)
     # stencil_tzgemm_mix has 16 + 15 = 31 parameters (src/mix_kernel/tzgemm_stencil.cu:281-283):
-    # [stencil 7 + 6 dims + start,step,end][A,B,C,M,N,K + 6 dims + start,step,end]; here the GEMM's
-    # workspace pointer follows K (null for a shape whose reduction stays inside a workgroup)
-    assert l["key"] == "tzgemm_stencil@wg_1_1" and len(l["args"]) == 32
+    # [stencil 7 + 6 dims + start,step,end][A,B,C,M,N,K + 6 dims + start,step,end]
+    assert l["key"] == "tzgemm_stencil@wg_1_1" and len(l["args"]) == 31
     a = l["args"]
     grid = l["grid"][0]
     assert grid % 16 == 0 and l["block"] == (256, 1, 1)
@@ -203,9 +242,8 @@ def test_mix_parameter_vector_matches_reference_signature(fake):
     assert [as_int(x) for x in a[13:16]] == [1, grid, 4]            # start1, step = fused grid, end1
     assert [as_ptr(x) for x in a[16:19]] == [A.ctypes.data, B.ctypes.data, Cm.ctypes.data]
     assert [as_int(x) for x in a[19:22]] == [256, 384, 128]
-    assert as_ptr(a[22]) == 0
-    assert [as_int(x) for x in a[23:29]] == [24, 1, 1, 256, 1, 1]   # tzgemm ori grid = tile count, block 256
-    assert [as_int(x) for x in a[29:32]] == [3, grid, 20]
+    assert [as_int(x) for x in a[22:28]] == [24, 1, 1, 256, 1, 1]   # tzgemm ori grid = tile count, block 256
+    assert [as_int(x) for x in a[28:31]] == [3, grid, 20]
 
 
 @pytest.mark.parametrize("be,n_be", [("lbm", 2), ("mriq", 7), ("mrif", 7), ("cp", 3)])
@@ -227,8 +265,8 @@ def test_other_mix_vectors_have_reference_lengths(fake, be, n_be):
     assert rc == 0, fake.tacker_last_error()
     (l,) = launches(fake)
     # lbm_tzgemm_mix 11+15, mriq_tzgemm_mix and mrif_tzgemm_mix 16+15, cp_tzgemm_mix 12+15
-    # (src/mix_kernel/tzgemm_{lbm,mriq,mrif,cp}.cu dispatcher signatures), plus the GEMM's workspace pointer
-    assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 16
+    # (src/mix_kernel/tzgemm_{lbm,mriq,mrif,cp}.cu dispatcher signatures)
+    assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 15
 
 
 def test_gptb_vector_is_restored_after_launch_and_after_failure(fake):
