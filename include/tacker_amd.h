@@ -144,6 +144,22 @@ TK_API int tacker_tzgemm_release_workspaces(void);
 TK_API int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int K,
                               int tile_start, int tile_end, int launch_grid, tkStream_t stream);
 
+/* No counterpart in the reference. tacker_gptb_tzgemm for callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc):
+ * same arguments, same kernel code, same bits in C, but the workspace of the shapes whose
+ * reduction is shared by workgroups is a static device array of the library
+ * (TACKER_TZGEMM_STATIC_SCRATCH_BYTES, held by each GPU the library runs on until the process
+ * ends) instead of a buffer bound to C, and the call itself allocates nothing (no hipMalloc /
+ * hipFree, no kernel objects with device state; the counters are cleared by a small kernel, not a
+ * memset, so the call can be captured). A shape whose workspace
+ * (tacker_tzgemm_workspace_bytes) exceeds the array is refused with TK_ERROR_UNSUPPORTED.
+ * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (two
+ * streams, two threads) race on it -- serialise them. */
+#define TACKER_TZGEMM_STATIC_SCRATCH_BYTES ((8u << 20) + (64u << 10))
+TK_API int tacker_gptb_tzgemm_static_scratch(const void *A, const void *B, float *C, int M, int N,
+                                             int K, int tile_start, int tile_end, int launch_grid,
+                                             tkStream_t stream);
+
 /* ori_stencil through OriSTENCILKernel::executeImpl
  * (src/ori_kernel/stencil_kernel.cu:9-94,189-201): one Jacobi sweep A0 -> Anext. */
 TK_API int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny,

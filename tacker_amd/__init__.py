@@ -36,6 +36,7 @@ def _declare(lib):
     lib.tkGetDeviceName.argtypes = [C.c_char_p, C.c_size_t]
     lib.tacker_tzgemm_grid_dim.argtypes = [i, i, i, C.POINTER(i)]
     lib.tacker_gptb_tzgemm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp]
+    lib.tacker_gptb_tzgemm_static_scratch.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp]
     lib.tacker_ori_stencil.argtypes = [f, f, vp, vp, i, i, i, vp]
     lib.tacker_gptb_stencil.argtypes = [f, f, vp, vp, i, i, i, i, i, i, i, vp]
     lib.tacker_ori_lbm.argtypes = [vp, vp, i, i, i, vp]
@@ -222,6 +223,16 @@ def gptb_tzgemm(A, B, Cm, tile_start=0, tile_end=None, launch_grid=0, stream=Non
         tile_end = (M // 64) * (N // 64)
     check(lib().tacker_gptb_tzgemm(_ptr(A), _ptr(B), _ptr(Cm), M, N, K, tile_start, tile_end,
                                    launch_grid, _stream(stream)), "tacker_gptb_tzgemm")
+
+
+def gptb_tzgemm_static_scratch(A, B, Cm, tile_start=0, tile_end=None, launch_grid=0, stream=None):
+    """gptb_tzgemm that allocates nothing: its workspace is the library's static device array"""
+    M, K = A.shape
+    N = B.shape[0]
+    if tile_end is None:
+        tile_end = (M // 64) * (N // 64)
+    check(lib().tacker_gptb_tzgemm_static_scratch(_ptr(A), _ptr(B), _ptr(Cm), M, N, K, tile_start, tile_end,
+                                                  launch_grid, _stream(stream)), "tacker_gptb_tzgemm_static_scratch")
 
 
 def stencil_blocks(nx, ny):

@@ -17,6 +17,7 @@
 extern Logger logger;
 extern std::unordered_map<std::string, void *> fmap;
 int tacker_runtime_init(int device, const char *kinfo_json_path);
+extern "C" int tk_tzgemm_scratch(void **ptr, size_t *bytes);   // beside the array, in the device translation unit
 bool tacker_runtime_ready();
 
 namespace {
@@ -250,6 +251,45 @@ int tacker_gptb_tzgemm(const void *A, const void *B, float *C, int M, int N, int
     });
     if (made) return made;
     return run_gptb_once(ori, tile_start, tile_end, launch_grid, TZ_THREADS, stream);
+}
+
+int tacker_gptb_tzgemm_static_scratch(const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                                      int tile_end, int launch_grid, tkStream_t stream)
+{
+    static_assert(TACKER_TZGEMM_STATIC_SCRATCH_BYTES == TZ_SCRATCH_BYTES, "public and device array sizes must agree");
+    REQUIRE_INIT();
+    const int rc = check_gemm(A, B, C, M, N, K);
+    if (rc) return rc;
+    const int tiles = (M / TZ_REF_TILE) * (N / TZ_REF_TILE);
+    if (tile_start < 0 || tile_end < tile_start || tile_end > tiles)
+        return fail(TK_ERROR_INVALID_VALUE, "tzgemm: bad tile range");
+    void *scratch = nullptr;
+    size_t scratch_bytes = 0;
+    if (tk_tzgemm_scratch(&scratch, &scratch_bytes) != TK_SUCCESS)
+        return fail(TK_ERROR_INVALID_VALUE, "tzgemm: the current device's static scratch array was never set up (tacker_init)");
+    const long long need = tz_workspace_bytes(M, N, K);
+    if (need > (long long)scratch_bytes)
+        return fail(TK_ERROR_UNSUPPORTED, "tzgemm: this shape needs a workspace of " + std::to_string(need) +
+                                              " bytes, the static scratch array holds " + std::to_string(scratch_bytes));
+    auto clear = fmap.find("tz_clear_words");
+    auto gemm = fmap.find("gptb_tzgemm_scratch");
+    if (clear == fmap.end() || gemm == fmap.end()) return fail(TK_ERROR_NOT_FOUND, "no kernel {gptb_tzgemm_scratch}");
+    if (need > 0) {
+        // every call on this GPU shares the array and it keeps the last call's contents: the
+        // arrival counters of this shape must start at zero
+        int words = (int)(tz_workspace_counter_bytes(M, N) / 4);
+        void *clear_args[] = {&scratch, &words};
+        const int rc2 = tkLaunchKernel(clear->second, dim3((words + 255) / 256).raw(), dim3(256).raw(), clear_args, 0, stream);
+        if (rc2) return fail(rc2, tkGetErrorString(rc2));
+    }
+    int grid = launch_grid > 0 ? launch_grid : default_grid("tzgemm");
+    int dims[6] = {tiles, 1, 1, TZ_THREADS, 1, 1};
+    int thread_base = 0;
+    void *workspace = need > 0 ? scratch : nullptr;
+    void *args[] = {&A, &B, &C, &M, &N, &K, &workspace, &dims[0], &dims[1], &dims[2], &dims[3], &dims[4], &dims[5],
+                    &tile_start, &grid, &tile_end, &thread_base};
+    const int rc3 = tkLaunchKernel(gemm->second, dim3(grid).raw(), dim3(TZ_THREADS).raw(), args, 0, stream);
+    return rc3 ? fail(rc3, tkGetErrorString(rc3)) : rc3;
 }
 
 int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz, tkStream_t stream)

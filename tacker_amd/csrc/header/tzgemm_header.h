@@ -98,6 +98,10 @@ TZ_HOST_DEVICE inline unsigned tz_ws_hash(unsigned long long c)
 {
     return (unsigned)(((c >> 8) * 0x9E3779B97F4A7C15ull) >> 54) & (TZ_WS_TABLE_SLOTS - 1);
 }
+// the device array the no-allocation entry point uses as workspace: the largest one any shape
+// needs (a batch padded to M = 128 with N = 8192: 256 tiles x 2 parts) plus the counters
+#define TZ_SCRATCH_BYTES ((8u << 20) + (64u << 10))
+
 // bits of the device word tk_spin_fail
 #define TK_FAIL_SPIN 1u        // a role-local barrier gave up waiting
 #define TK_FAIL_WORKSPACE 2u   // a GEMM whose reduction is shared by workgroups found no workspace for its C

@@ -108,6 +108,61 @@ extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_
                     (int)threadIdx.x - thread_base, tz_lds, sync);
 }
 
+// ---- tzgemm for callers that cannot allocate device memory --------------------------------
+// The same role with its workspace handed in as an argument, and the workspace itself: a
+// file-scope array every GPU the library runs on holds until the process ends.  TZ_SCRATCH_BYTES
+// covers the largest workspace any shape needs (512 partial tiles of 16 KiB + the counters).
+// `scratch` is a host-side stand-in in host code, never a device address: host code uses the
+// address hipGetSymbolAddress gave for the current device (tk_scratch_setup / tk_tzgemm_scratch).
+static __device__ __align__(256) unsigned char scratch[TZ_SCRATCH_BYTES];
+
+extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void general_ptb_tzgemm_scratch(
+    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, unsigned *workspace, GPTB_TRAILER)
+{
+    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
+    tk::WorkgroupSync sync;
+    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, workspace, (int)blockIdx.x, ptb_iter_block_step,
+                    ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base, tz_lds,
+                    sync);
+}
+
+// zeroes n 32-bit words (the arrival counters at the head of the workspace); a kernel rather
+// than a memset so that the call can be recorded into a HIP graph
+extern "C" __global__ void tz_clear_words(unsigned *words, int n)
+{
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) words[i] = 0u;
+}
+
+namespace {
+constexpr int kMaxDevices = 64;
+void *g_scratch_address[kMaxDevices];   // address of `scratch` on each device that was set up
+}
+
+// Once per device, with that device current (tkInit calls it): the device address of the array.
+extern "C" int tk_scratch_setup(int device)
+{
+    if (device < 0 || device >= kMaxDevices) return TK_ERROR_INVALID_VALUE;
+    if (g_scratch_address[device]) return TK_SUCCESS;
+    void *ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) {
+        (void)hipGetLastError();
+        return TK_ERROR_DEVICE;
+    }
+    g_scratch_address[device] = ptr;
+    return TK_SUCCESS;
+}
+
+// The current device's copy of the array and its size; fails if the device was never set up.
+extern "C" int tk_tzgemm_scratch(void **ptr, size_t *bytes)
+{
+    int device = -1;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices || !g_scratch_address[device])
+        return TK_ERROR_INVALID_VALUE;
+    *ptr = g_scratch_address[device];
+    *bytes = sizeof(scratch);
+    return TK_SUCCESS;
+}
+
 extern "C" __global__ __launch_bounds__(256) void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
                                                int ny, int nz, GPTB_TRAILER)
 {
@@ -220,6 +275,8 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ComputeRhoPhiGPU", (const void *)ComputeRhoPhiGPU, ctx);
     insert("ori_mrif", (const void *)ori_mrif, ctx);
     insert("gptb_tzgemm", (const void *)general_ptb_tzgemm, ctx);
+    insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);
+    insert("tz_clear_words", (const void *)tz_clear_words, ctx);
     insert("gptb_stencil", (const void *)general_ptb_stencil, ctx);
     insert("gptb_lbm", (const void *)general_ptb_lbm, ctx);
     insert("gptb_mriq", (const void *)g_general_ptb_mriq, ctx);

@@ -93,6 +93,13 @@ int tkMemcpyFromSymbol(void *dst, const char *symbol, size_t bytes, size_t offse
     if (offset + bytes <= it->second.size()) memcpy(dst, it->second.data() + offset, bytes);
     return TK_SUCCESS;
 }
+int tk_tzgemm_scratch(void **ptr, size_t *bytes)
+{
+    static std::vector<unsigned char> scratch((8u << 20) + (64u << 10));
+    *ptr = scratch.data();
+    *bytes = scratch.size();
+    return TK_SUCCESS;
+}
 int tkStreamCreate(tkStream_t *s) { *s = malloc(1); return TK_SUCCESS; }
 int tkStreamDestroy(tkStream_t s) { free(s); return TK_SUCCESS; }
 int tkStreamSynchronize(tkStream_t) { return TK_SUCCESS; }
@@ -169,6 +176,8 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ComputeRhoPhiGPU", {I, P, P, P, P, P, P});
         add("ori_mrif", MRIF);
         add("gptb_tzgemm", cat(TZ, trailer(true)));
+        add("gptb_tzgemm_scratch", cat(cat(TZ, {P}), trailer(true)));
+        add("tz_clear_words", {P, I});
         add("gptb_stencil", cat(STENCIL, trailer(true)));
         add("gptb_lbm", cat(LBM, trailer(true)));
         add("gptb_mriq", cat(MRIQ, trailer(true)));

@@ -10,6 +10,7 @@
 #include "../../include/tacker_amd.h"
 
 extern "C" int tk_device_symbol(const char *name, const void **symbol, size_t *bytes);
+extern "C" int tk_scratch_setup(int device);
 
 namespace {
 thread_local std::string g_last_hip_error;
@@ -47,7 +48,11 @@ int tkInit(int device)
     }
     rc = FOLD(hipSetDevice(device));
     if (rc) return rc;
-    return FOLD(hipFree(0));   // force context creation, as initCUDA does
+    rc = FOLD(hipFree(0));   // force context creation, as initCUDA does
+    if (rc) return rc;
+    rc = tk_scratch_setup(device);   // device address of the library's static scratch array
+    if (rc) g_last_hip_error = "tkInit: hipGetSymbolAddress of the static scratch array failed";
+    return rc;
 }
 
 const char *tkGetErrorString(int code)
