@@ -76,7 +76,18 @@ def pair_leg(ta, torch, np, name, stream):
         tiles = (M // 64) * (N // 64)
         return ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, tiles), tiles, 2.0 * M * N * K
 
-    if name == "lbm":       # D3Q19, 120x120x150, rest equilibrium + noise, 5 % obstacle cells
+    swap = None             # exchanges the best-effort kernel's input and output grid after a launch
+    if name == "cp":        # Coulomb potential, 4096x4096 grid, 64 atoms (the Creator's instance, src/Creator.cu:23-37)
+        volx = voly = 4096
+        atoms = ta.cp_initatoms(4000, volx, voly, 1, 0.1)
+        ta.cp_set_atoms(atoms[1:65], 0.0)
+        grid = torch.zeros((voly, volx), device="cuda:0")
+        be_ori = ta.ori_cp_create(64, 0.1, grid)
+        nblk = ta.cp_blocks(volx, voly)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "valu", "pairs": 64.0 * volx * voly}
+        label = "tzgemm 2048^3 + cp 4096x4096, 64 atoms (reference mix tzgemm_cp; named by the north star)"
+    elif name == "lbm":     # D3Q19, 120x120x150, rest equilibrium + noise, 5 % obstacle cells
         sx, sy, sz = 120, 120, 150
         cells = sx * sy * sz
         w = np.array([1 / 3] + [1 / 18] * 6 + [1 / 36] * 12, np.float32)
@@ -86,10 +97,11 @@ def pair_leg(ta, torch, np, name, stream):
         src = torch.from_numpy(g.reshape(-1)).cuda()
         dst = src.clone()
         be_ori = ta.ori_lbm_create(src, dst, sx, sy, sz)
+        swap = be_ori.swap_buffers     # every launch is the next step of the simulation: src <-> dst
         nblk = sy * sz
         tz, tiles, flop = gemm(4096, 4096, 1024)
         work = {"bound": "hbm", "algorithmic_bytes": 156.0 * cells}
-        label = "configs[2]: tzgemm 4096x4096x1024 + lbm 120x120x150 (one step per launch)"
+        label = "configs[2]: tzgemm 4096x4096x1024 + lbm 120x120x150 (one step per launch, src and dst exchanged after each)"
     elif name == "mrif":    # mri-fhd, numK 2048, numX 262144 (the reference's tzgemm_mrif mix; no benchmark configuration of its own)
         numK, numX = 2048, 262144
         k = rng.uniform(-0.5, 0.5, (numK, 3)).astype(np.float32)
@@ -140,16 +152,25 @@ def pair_leg(ta, torch, np, name, stream):
         e1.synchronize()
         return e0.elapsed_ms(e1) / n * 1e3
 
+    def be_alone():
+        be.execute(stream)
+        if swap:
+            swap()
+
     def serial():
         tz.execute(stream)
-        be.execute(stream)
+        be_alone()
+
+    def fused():
+        mix.execute(stream)
+        if swap:
+            swap()
 
     def serial_slice():
         tz.execute(stream)
         be_slice.execute(stream)
 
-    cases = {"gemm_us": lambda: tz.execute(stream), "be_us": lambda: be.execute(stream), "serial_us": serial,
-             "fused_us": lambda: mix.execute(stream)}
+    cases = {"gemm_us": lambda: tz.execute(stream), "be_us": be_alone, "serial_us": serial, "fused_us": fused}
     if slice_blocks > 0:
         cases["slice_serial_us"] = serial_slice
         cases["slice_fused_us"] = lambda: mix_slice.execute(stream)
@@ -195,6 +216,43 @@ def pair_leg(ta, torch, np, name, stream):
         out["be_frac_of_hbm_peak"] = round(work["algorithmic_bytes"] / (out["be_us"] * 1e-6) / HBM_PEAK, 4)
     else:
         out["be_gpairs_per_s_alone"] = round(work["pairs"] / out["be_us"] / 1e3, 1)
+    return out
+
+
+def gemm_leg(ta, torch, np, stream):
+    """tzgemm alone at the shapes of the benchmark configurations and at 4096^3, with a yardstick from the same
+    GPU beside each: torch.matmul on the same fp16 operands (the vendor library's kernel; time only)."""
+    import statistics
+    rng = np.random.default_rng(1337)
+    out = {}
+    for M, N, K in ((1024, 1024, 1024), (2048, 2048, 2048), (4096, 4096, 1024), (4096, 4096, 4096)):
+        A = torch.from_numpy(rng.uniform(-1, 1, (M, K)).astype(np.float16)).cuda()
+        B = torch.from_numpy(rng.uniform(-1, 1, (N, K)).astype(np.float16)).cuda()
+        Cm = torch.zeros((M, N), device="cuda:0")
+        tz = ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, (M // 64) * (N // 64))
+        Bt = B.t()
+        e0, e1 = ta.Event(), ta.Event()
+        n = 50
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0.record(stream)
+            for _ in range(n):
+                fn()
+            e1.record(stream)
+            e1.synchronize()
+            return e0.elapsed_ms(e1) / n * 1e3
+
+        ours = statistics.median(timed(lambda: tz.execute(stream)) for _ in range(3))
+        lib = statistics.median(timed(lambda: torch.matmul(A, Bt)) for _ in range(3))
+        flop = 2.0 * M * N * K
+        out[f"{M}x{N}x{K}"] = {"us": round(ours, 2), "tflops": round(flop / ours / 1e6, 1),
+                               "frac_of_mfma_peak": round(flop / (ours * 1e-6) / MFMA_F16_PEAK, 4),
+                               "form": "256x256 tiles" if (M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) >= 256)
+                               else "128x128 tiles",
+                               "torch_matmul_us": round(lib, 2), "torch_matmul_tflops": round(flop / lib / 1e6, 1)}
     return out
 
 
@@ -331,7 +389,7 @@ def main():
         "data": "synthetic (numpy default_rng(1337): A,B uniform[-1,1] -> f16; grid uniform[0,1])",
         "config": {"workload": "configs[1]: fused tzgemm fp16 2048x2048x2048 + 7-point stencil fp32 "
                                "512x512x64, c0=1/6, c1=1/36, 100 iterations",
-                   "fused_kernel": "tzgemm_stencil@" + (args.variant or ta.lib().tacker_last_error() and "default" or "default"),
+                   "fused_kernel": "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)"),
                    "fused_grid": info["grid"], "fused_block": info["block"], "device": ta.device_name()},
         "serial_ms_per_step": round(ms["serial"], 4),
         "gemm_alone_ms_per_100": round(ms["gemm"], 4), "stencil_alone_ms_per_100": round(ms["stencil"], 4),
@@ -356,9 +414,9 @@ def main():
                         "frac_of_hbm_peak": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / HBM_PEAK, 4)}},
         "wall_s_timed_region": round(t_wall, 3),
     }
-    out["config"]["fused_kernel"] = "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)")
     if not args.no_extras:
-        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq", "mrif")}
+        out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
+        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq", "cp", "mrif")}
         if not args.no_lc:
             out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")

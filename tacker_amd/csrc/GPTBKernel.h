@@ -72,7 +72,8 @@ public:
 
     void loadKernel() override
     {
-        auto it = fmap.find(funcKey);
+        auto it = fmap.find(funcKey + kernel_->funcVariant());   // a build made for this problem, if any
+        if (it == fmap.end()) it = fmap.find(funcKey);
         if (it == fmap.end()) logger.ERROR("load kernel {" + funcKey + "} failed!");
         this->kernelFunc = it->second;
     }

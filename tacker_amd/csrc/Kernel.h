@@ -32,6 +32,11 @@ public:
     // (mixable == 1), the 14 convolution ints (mixable == 2), empty otherwise
     virtual std::vector<int> getArgs() = 0;
 
+    // No counterpart in the reference.  Suffix a wrapper appends to its function key when it looks
+    // the device function up ("" = the key as given): lets a kernel object pick among builds of
+    // the same device function by what it knows about its problem, without its callers naming one.
+    virtual const char *funcVariant() { return ""; }
+
     int getKernelId() { return Id; }
     std::string &getKernelName() { return kernelName; }
 

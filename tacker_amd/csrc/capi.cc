@@ -273,7 +273,9 @@ int tacker_gptb_tzgemm_static_scratch(const void *A, const void *B, float *C, in
                                               " bytes, the static scratch array holds " + std::to_string(scratch_bytes));
     auto clear = fmap.find("tz_clear_words");
     auto gemm = fmap.find("gptb_tzgemm_scratch");
-    if (clear == fmap.end() || gemm == fmap.end()) return fail(TK_ERROR_NOT_FOUND, "no kernel {gptb_tzgemm_scratch}");
+    auto large = fmap.find("gptb_tzgemm@large");
+    if (clear == fmap.end() || gemm == fmap.end() || large == fmap.end())
+        return fail(TK_ERROR_NOT_FOUND, "no kernel {gptb_tzgemm_scratch}");
     if (need > 0) {
         // every call on this GPU shares the array and it keeps the last call's contents: the
         // arrival counters of this shape must start at zero
@@ -288,7 +290,15 @@ int tacker_gptb_tzgemm_static_scratch(const void *A, const void *B, float *C, in
     void *workspace = need > 0 ? scratch : nullptr;
     void *args[] = {&A, &B, &C, &M, &N, &K, &workspace, &dims[0], &dims[1], &dims[2], &dims[3], &dims[4], &dims[5],
                     &tile_start, &grid, &tile_end, &thread_base};
-    const int rc3 = tkLaunchKernel(gemm->second, dim3(grid).raw(), dim3(TZ_THREADS).raw(), args, 0, stream);
+    int rc3;
+    if (tz_use_large(M, N, K)) {
+        // the large-tile build takes general_ptb_tzgemm's list (it never needs a workspace)
+        void *largs[] = {&A, &B, &C, &M, &N, &K, &dims[0], &dims[1], &dims[2], &dims[3], &dims[4], &dims[5],
+                         &tile_start, &grid, &tile_end, &thread_base};
+        rc3 = tkLaunchKernel(large->second, dim3(grid).raw(), dim3(TZ_THREADS).raw(), largs, 0, stream);
+    } else {
+        rc3 = tkLaunchKernel(gemm->second, dim3(grid).raw(), dim3(TZ_THREADS).raw(), args, 0, stream);
+    }
     return rc3 ? fail(rc3, tkGetErrorString(rc3)) : rc3;
 }
 

@@ -83,6 +83,17 @@ TZ_HOST_DEVICE inline long long tz_workspace_bytes(int M, int N, int K)
     return tz_workspace_counter_bytes(M, N) + n_ref * parts * TZ_PARTIAL_TILE_BYTES;
 }
 
+// Shapes the stand-alone kernel computes with 256 x 256 macro tiles (kernels/tzgemm_large.h):
+// whole 256 x 256 tiles and at least one of them for every CU.  Same bits as the other forms.
+#define TZ_LARGE_TILE 256
+#define TZ_LARGE_MIN_TILES TK_CU_NUM
+TZ_HOST_DEVICE inline bool tz_use_large(int M, int N, int K)
+{
+    (void)K;
+    return M % TZ_LARGE_TILE == 0 && N % TZ_LARGE_TILE == 0 &&
+           (long long)(M / TZ_LARGE_TILE) * (N / TZ_LARGE_TILE) >= TZ_LARGE_MIN_TILES;
+}
+
 // Where a kernel finds the workspace of the output buffer it writes: a device-resident hash
 // table from C to workspace that the host fills when it binds one (open addressing, linear
 // probing, an entry is never moved or removed while kernels may run; key 0 = empty).  The

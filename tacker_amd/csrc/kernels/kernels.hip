@@ -264,6 +264,8 @@ extern "C" __global__ void convertFp32ToFp16_(_Float16 *out, float *in, int n)
 #include "../mix_kernel/mix_kernels.inc"
 
 // ------------------------------------------------------------------ registry
+extern "C" void tk_register_large_kernels(tk_kernel_insert_fn insert, void *ctx);   // tzgemm_large.hip
+
 extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
 {
     if (!insert) return TK_ERROR_INVALID_VALUE;
@@ -291,6 +293,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("pack_fc_input", (const void *)pack_fc_input, ctx);
     insert("pack_fc_input_pooled", (const void *)pack_fc_input_pooled, ctx);
     tk_register_mix_kernels(insert, ctx);
+    tk_register_large_kernels(insert, ctx);
     return TK_SUCCESS;
 }
 

@@ -176,6 +176,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ComputeRhoPhiGPU", {I, P, P, P, P, P, P});
         add("ori_mrif", MRIF);
         add("gptb_tzgemm", cat(TZ, trailer(true)));
+        add("gptb_tzgemm@large", cat(TZ, trailer(true)));
         add("gptb_tzgemm_scratch", cat(cat(TZ, {P}), trailer(true)));
         add("tz_clear_words", {P, I});
         add("gptb_stencil", cat(STENCIL, trailer(true)));

@@ -102,6 +102,9 @@ public:
     }
 
     std::vector<int> getArgs() override { return std::vector<int>{m, n, k}; }
+    // shapes with a 256 x 256 tile for every CU run the large-tile build of general_ptb_tzgemm
+    // (same parameter list, same bits)
+    const char *funcVariant() override { return tz_use_large(M_GLOBAL, N_GLOBAL, K_GLOBAL) ? "@large" : ""; }
 
     int m, n, k;
     int M_GLOBAL, N_GLOBAL, K_GLOBAL;
