@@ -328,7 +328,7 @@ def main():
     stream = torch.cuda.current_stream()
 
     tiles = ta.tzgemm_grid_dim(M, N, K)[3]
-    blocks = ta.stencil_blocks(nx, ny)
+    blocks = ta.stencil_blocks(nx, ny, nz)
     st_ori = ta.ori_stencil_create(c0, c1, g0, g1)
     st = ta.gptb_create(st_ori, 0, 0, 0, blocks)
     tz_ori = ta.ori_tzgemm_create(dA, dB, dC)

@@ -165,9 +165,16 @@ TK_API int tacker_gptb_tzgemm_static_scratch(const void *A, const void *B, float
 TK_API int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny,
                               int nz, tkStream_t stream);
 /* general_ptb_stencil through GPTBKernel (src/gptb_kernel/stencil_kernel.cu:3-104,
- * src/Creator.cu:179-192): blocks [block_start, block_end) of the ori grid
- * (ceil(nx/64), ceil(ny/4)). launch_grid workgroups of launch_block threads
- * (0 = the Creator default for this GPU). */
+ * src/Creator.cu:179-192): block positions [block_start, block_end) of a grid of
+ * (ceil(nx/64), ceil(ny/4), runs) positions, runs = ceil((nz-2) / TACKER_STENCIL_Z_RUN): position
+ * p computes run p / blocks of block p % blocks (blocks = the ori grid's ceil(nx/64) *
+ * ceil(ny/4)), a run being TACKER_STENCIL_Z_RUN centre planes of the block's march along z --
+ * the reference's 3-D index reconstruction over a grid whose z cuts that march, so that a
+ * range can be as short as the GEMM it rides with.  [0, tacker_stencil_blocks(nx, ny, nz)) is
+ * one sweep (ori_stencil bit for bit), and so is any set of ranges that tiles it. launch_grid
+ * workgroups of launch_block threads (0 = the Creator default for this GPU). */
+#define TACKER_STENCIL_Z_RUN 8
+TK_API int tacker_stencil_blocks(int nx, int ny, int nz);
 TK_API int tacker_gptb_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny,
                                int nz, int block_start, int block_end, int launch_grid,
                                int launch_block, tkStream_t stream);
@@ -424,7 +431,7 @@ TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
 TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int limit);
 /* No counterpart in the reference (it takes tiles x block_ratio(K) from kinfo,
  * src/TaskManager.cu:593-600): with on != 0 an Aker-mode run first times, for every mixable LC
- * kernel, its fused launch with be_total / 64, / 32, ... best-effort blocks and then co-locates
+ * kernel, its fused launch with be_total / 256, / 128, ... best-effort blocks and then co-locates
  * the count that earned most among those that kept the fused launch within (1 + max_stretch) of
  * the kernel alone (none: the kernel runs alone).  For layers that leave most CUs without a tile.
  * tacker_task_manager_calibrated_blocks copies the counts of the last run (one per LC kernel). */

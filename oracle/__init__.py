@@ -45,7 +45,7 @@ def _declare(l):
                              C.c_int, C.c_int]
     l.orc_gptb_index.argtypes = [C.c_uint, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, _i32p]
     l.orc_stencil_gptb.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int,
-                                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
+                                   C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_stencil.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
@@ -117,13 +117,26 @@ def stencil(c0, c1, A0, Anext):
     return out
 
 
-def stencil_gptb(c0, c1, A0, Anext, start, end, gdx=None, gdy=None, bdx=32, bdy=4):
+STENCIL_Z_RUN = 8
+
+
+def stencil_positions(nx, ny, nz, zrun=STENCIL_Z_RUN):
+    """Block positions of the device objects' grid: blocks x runs of zrun centre planes."""
+    gdx, gdy = stencil_grid(nx, ny)
+    return gdx * gdy * max(1, -(-(nz - 2) // zrun))
+
+
+def stencil_gptb(c0, c1, A0, Anext, start, end, gdx=None, gdy=None, bdx=32, bdy=4, gdz=1, zrun=STENCIL_Z_RUN):
+    """Positions [start, end) of the (gdx, gdy, gdz) grid; gdz = 1 (default): whole block columns, the
+    reference's kernel; gdz = 'runs': one run of zrun centre planes per position."""
     nz, ny, nx = A0.shape
     if gdx is None:
         gdx, gdy = stencil_grid(nx, ny)
+    if gdz == "runs":
+        gdz = max(1, -(-(nz - 2) // zrun))
     out = np.array(Anext, np.float32, order="C")
-    lib().orc_stencil_gptb(c0, c1, np.ascontiguousarray(A0, np.float32), out, nx, ny, nz, gdx, gdy,
-                           bdx, bdy, start, end)
+    lib().orc_stencil_gptb(c0, c1, np.ascontiguousarray(A0, np.float32), out, nx, ny, nz, gdx, gdy, gdz,
+                           bdx, bdy, zrun, start, end)
     return out
 
 

@@ -183,10 +183,11 @@ ORC_API void orc_gptb_index(unsigned block_pos, int t, int grid_dimension_x, int
 /* One block of src/ori_kernel/stencil_kernel.cu:9-94 (= general_ptb_stencil
  * body, src/gptb_kernel/stencil_kernel.cu:26-102): block (bx,by) of
  * block_dimension (bdx,bdy) covers x in [2*bdx*bx, 2*bdx*bx + 2*bdx),
- * y in [bdy*by, bdy*by + bdy), marches k = 1..nz-2. */
+ * y in [bdy*by, bdy*by + bdy), marches k = k_lo .. k_hi-1 (the reference: 1 .. nz-2). */
 static void stencil_block(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz,
-                          int bx, int by, int bdx, int bdy)
+                          int bx, int by, int bdx, int bdy, int k_lo, int k_hi)
 {
+    (void)nz;
     for (int ty = 0; ty < bdy; ty++) {
         int j = by * bdy + ty;
         for (int half = 0; half < 2; half++) {
@@ -196,7 +197,7 @@ static void stencil_block(float c0, float c1, const float *A0, float *Anext, int
                 int w = (half == 0) ? (i > 0 && j > 0 && i < nx - 1 && j < ny - 1)
                                     : (j > 0 && i < nx - 1 && j < ny - 1);
                 if (!w) continue;
-                for (int k = 1; k < nz - 1; k++) {
+                for (int k = k_lo; k < k_hi; k++) {
                     float top = A0[IDX3(nx, ny, i, j, k + 1)];
                     float bottom = A0[IDX3(nx, ny, i, j, k - 1)];
                     float up = A0[IDX3(nx, ny, i, j + 1, k)];
@@ -219,16 +220,27 @@ static void stencil_block(float c0, float c1, const float *A0, float *Anext, int
     }
 }
 
-/* GPTB form: blocks block_pos in [start,end) of a (gdx,gdy) grid of (bdx,bdy)
- * blocks; by wraps modulo gdy (src/gptb_kernel/stencil_kernel.cu:22-24). */
+/* GPTB form: block positions [start,end) of a (gdx,gdy,gdz) grid of (bdx,bdy) blocks, index
+ * reconstruction as in the reference's kernels (block_id_x = pos % gdx, block_id_y =
+ * pos / gdx % gdy, src/gptb_kernel/stencil_kernel.cu:22-24; block_id_z = pos / (gdx*gdy) % gdz
+ * as in its 3-D kernels).  The z index cuts the march of a block column: with
+ * runs = ceil((nz-2) / zrun) runs of zrun centre planes, position p computes the runs
+ * [part*runs/gdz, (part+1)*runs/gdz) of block p % (gdx*gdy), part = p / (gdx*gdy) % gdz.
+ * gdz = 1: a position is a whole block column, the reference's kernel. */
 ORC_API void orc_stencil_gptb(float c0, float c1, const float *A0, float *Anext, int nx, int ny,
-                              int nz, int gdx, int gdy, int bdx, int bdy, int start, int end)
+                              int nz, int gdx, int gdy, int gdz, int bdx, int bdy, int zrun, int start, int end)
 {
+    if (nz < 3 || gdz < 1 || zrun < 1) return;
+    const int runs = (nz - 2 + zrun - 1) / zrun;
 #pragma omp parallel for schedule(static)
     for (int pos = start; pos < end; pos++) {
         int bx = pos % gdx;
         int by = (pos / gdx) % gdy;
-        stencil_block(c0, c1, A0, Anext, nx, ny, nz, bx, by, bdx, bdy);
+        int part = (pos / (gdx * gdy)) % gdz;
+        int k_lo = 1 + (part * runs / gdz) * zrun;
+        int k_hi = 1 + ((part + 1) * runs / gdz) * zrun;
+        if (k_hi > nz - 1) k_hi = nz - 1;
+        stencil_block(c0, c1, A0, Anext, nx, ny, nz, bx, by, bdx, bdy, k_lo, k_hi);
     }
 }
 
@@ -238,7 +250,7 @@ ORC_API void orc_stencil(float c0, float c1, const float *A0, float *Anext, int 
 {
     int gdx = (nx + 32 * 2 - 1) / (32 * 2);
     int gdy = (ny + 4 - 1) / 4;
-    orc_stencil_gptb(c0, c1, A0, Anext, nx, ny, nz, gdx, gdy, 32, 4, 0, gdx * gdy);
+    orc_stencil_gptb(c0, c1, A0, Anext, nx, ny, nz, gdx, gdy, 1, 32, 4, nz, 0, gdx * gdy);
 }
 
 /* ------------------------------------------------------------------------ */

@@ -38,6 +38,7 @@ def _declare(lib):
     lib.tacker_gptb_tzgemm.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp]
     lib.tacker_gptb_tzgemm_static_scratch.argtypes = [vp, vp, vp, i, i, i, i, i, i, vp]
     lib.tacker_ori_stencil.argtypes = [f, f, vp, vp, i, i, i, vp]
+    lib.tacker_stencil_blocks.argtypes = [i, i, i]
     lib.tacker_gptb_stencil.argtypes = [f, f, vp, vp, i, i, i, i, i, i, i, vp]
     lib.tacker_ori_lbm.argtypes = [vp, vp, i, i, i, vp]
     lib.tacker_gptb_lbm.argtypes = [vp, vp, i, i, i, i, i, i, i, vp]
@@ -235,8 +236,12 @@ def gptb_tzgemm_static_scratch(A, B, Cm, tile_start=0, tile_end=None, launch_gri
                                                   launch_grid, _stream(stream)), "tacker_gptb_tzgemm_static_scratch")
 
 
-def stencil_blocks(nx, ny):
-    return ((nx + 63) // 64) * ((ny + 3) // 4)
+def stencil_blocks(nx, ny, nz=None):
+    """block positions of the GPTB form: blocks of 64 x 4 columns, times (when nz is given) the runs of
+    8 centre planes a block column is cut into along z"""
+    if nz is None:
+        return ((nx + 63) // 64) * ((ny + 3) // 4)
+    return lib().tacker_stencil_blocks(nx, ny, nz)
 
 
 def ori_stencil(c0, c1, A0, Anext, stream=None):
@@ -248,7 +253,7 @@ def ori_stencil(c0, c1, A0, Anext, stream=None):
 def gptb_stencil(c0, c1, A0, Anext, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
     nz, ny, nx = A0.shape
     if end is None:
-        end = stencil_blocks(nx, ny)
+        end = stencil_blocks(nx, ny, nz)
     check(lib().tacker_gptb_stencil(c0, c1, _ptr(A0), _ptr(Anext), nx, ny, nz, start, end, launch_grid,
                                     launch_block, _stream(stream)), "tacker_gptb_stencil")
 
@@ -346,7 +351,7 @@ def mix_tzgemm_stencil(c0, c1, A0, Anext, A, B, Cm, be_start=0, be_end=None, til
                        tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
     nz, ny, nx = A0.shape
     if be_end is None:
-        be_end = stencil_blocks(nx, ny)
+        be_end = stencil_blocks(nx, ny, nz)
     check(lib().tacker_mix_tzgemm_stencil(
         c0, c1, _ptr(A0), _ptr(Anext), nx, ny, nz, be_start, be_end,
         *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),

@@ -238,7 +238,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         std::vector<float> best_earned(nk, 0.0f);
         std::vector<bool> over(nk, false);   // a smaller count already stretched this kernel too far
         const int first = be_kernel1->gptbParams.ptb_start_block_pos;
-        for (int divisor = 64; divisor >= 1; divisor /= 2) {
+        for (int divisor = 256; divisor >= 1; divisor /= 2) {
             const int n = std::max(1, be_total / divisor);
             std::vector<float> fused_ms(nk, 0.0f);
             const int timed = 3;

@@ -97,7 +97,7 @@ public:
     // tiles x block_ratio(K) from kinfo.  That table is measured on GEMMs that fill the GPU; a
     // batch-1 layer with a few dozen tiles leaves most CUs free, and what those CUs can take
     // depends on the layer and on the best-effort kernel.  The fused launch is timed with
-    // be_total / 64, / 32, ... blocks and the count with the largest earned time
+    // be_total / 256, / 128, ... blocks and the count with the largest earned time
     // (lc alone + share of be alone - fused) is kept among those whose fused launch stays
     // within (1 + calibrate_max_stretch) of the LC kernel alone; none -> the kernel runs alone.
     bool calibrate_blocks = false;

@@ -13,6 +13,7 @@
 #include "rng.h"
 #include "TaskManager.h"
 #include "dnn/vgg16.h"
+#include "header/stencil_header.h"
 
 extern Logger logger;
 extern std::unordered_map<std::string, void *> fmap;
@@ -308,6 +309,14 @@ int tacker_ori_stencil(float c0, float c1, const float *A0, float *Anext, int nx
     const int rc = check_stencil(A0, Anext, nx, ny, nz);
     if (rc) return rc;
     return run_once(new OriSTENCILKernel(0, c0, c1, A0, Anext, nx, ny, nz), stream);
+}
+
+int tacker_stencil_blocks(int nx, int ny, int nz)
+{
+    static_assert(TACKER_STENCIL_Z_RUN == STENCIL_Z_RUN, "public and device run lengths must agree");
+    if (nx < 1 || ny < 1 || nz < 1) return 0;
+    const int runs = nz > 2 ? (nz - 2 + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN : 1;
+    return ((nx + STENCIL_TILE_X * 2 - 1) / (STENCIL_TILE_X * 2)) * ((ny + STENCIL_TILE_Y - 1) / STENCIL_TILE_Y) * runs;
 }
 
 int tacker_gptb_stencil(float c0, float c1, const float *A0, float *Anext, int nx, int ny, int nz,

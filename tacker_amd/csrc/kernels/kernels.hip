@@ -166,7 +166,7 @@ extern "C" int tk_tzgemm_scratch(void **ptr, size_t *bytes)
 extern "C" __global__ __launch_bounds__(256) void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
                                                int ny, int nz, GPTB_TRAILER)
 {
-    tk::stencil_role(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y,
+    tk::stencil_role(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, grid_dimension_z,
                      (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
                      (int)threadIdx.x - thread_base, (int)blockDim.x);
 }

@@ -262,37 +262,102 @@ struct StencilQuadMarch {
 // GPTB form.  The unit of work of a wave is a run of STENCIL_Z_RUN centre planes of one
 // reference block (narrow form) or of one quad of blocks (wide form): a 512x512x64 grid has
 // only 1024 blocks, far fewer than the waves a 256-CU part needs in flight to pull HBM
-// bandwidth, so the z march is shared out.  The waves of one workgroup take consecutive
-// runs of the same block or quad (their overlap planes hit in the CU's own cache).
-// The role's waves enumerate tasks t = role_block*waves + wave, stepping by
-// role_blocks*waves.
-#define STENCIL_Z_RUN 8
+// bandwidth, so the z march is shared out.
+//
+// Block positions.  The position space is the reference's 3-D index reconstruction
+// (block_id_x = pos % gx, block_id_y = pos / gx % gy, block_id_z = pos / (gx * gy) % gz) over
+// the grid (gx, gy, gz): position p is part p / (gx * gy) % gz of block p % (gx * gy), a part
+// being the runs [part * runs / gz, (part + 1) * runs / gz) of the block's
+// runs = ceil((nz - 2) / STENCIL_Z_RUN) runs of centre planes.  gz = 1 is the reference's
+// grid (a position is a whole block column); the host objects use gz = runs, so that a
+// position is one run of one block -- short enough to ride along with a GEMM of a few
+// microseconds -- and any set of ranges that tiles [0, gx * gy * gz) is one sweep, bit for
+// bit (a point's value depends on A0 only).
+//
+// A range [start, end) is served part by part: the blocks [lo, hi) of the first part it
+// touches, every block of the parts in between, the blocks [0, hi) of the last one.
+
+#define STENCIL_SHORT_RANGE_TASKS 2048
+
+// The block positions [start, end) as segments (one per part touched) of tasks.
+struct StencilRange {
+    unsigned blocks;        // gx * gy
+    unsigned gz, runs;
+    unsigned first_part;    // unwrapped part index of the first segment
+    unsigned lo_first;      // first block of the first segment
+    unsigned cut_last;      // blocks the last segment stops short of a whole part
+    unsigned parts;         // segments
+
+    __device__ __forceinline__ StencilRange(int gx, int gy, int gz_, int nz, int start, int end)
+    {
+        blocks = (unsigned)gx * (unsigned)gy;
+        gz = gz_ > 0 ? (unsigned)gz_ : 1u;
+        runs = (unsigned)(nz - 2 + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
+        first_part = (unsigned)start / blocks;
+        const unsigned last_part = (unsigned)(end - 1) / blocks;
+        parts = last_part - first_part + 1;
+        lo_first = (unsigned)start - first_part * blocks;
+        cut_last = blocks - ((unsigned)end - last_part * blocks);
+    }
+    // block range [lo, hi) and runs [r0, r1) of segment s
+    struct Segment {
+        unsigned lo, hi, r0, r1;
+    };
+    __device__ __forceinline__ Segment segment(unsigned s) const
+    {
+        Segment g;
+        // masks, not selects between members: a select of member addresses would keep the struct
+        // in memory (the compiler then parks it in LDS) instead of in scalar registers
+        g.lo = lo_first & (0u - (unsigned)(s == 0));
+        g.hi = blocks - (cut_last & (0u - (unsigned)(s + 1 == parts)));
+        const unsigned part = (first_part + s) % gz;
+        g.r0 = part * runs / gz;
+        g.r1 = (part + 1) * runs / gz;
+        return g;
+    }
+};
+
+// Narrow form: a task is (block, run); all loads of a run are issued at once and a wave keeps
+// two runs in flight, so a wave with one or two tasks is done after one trip to memory.
+// spread: hand consecutive tasks to different workgroups (a short range then uses every CU
+// the role has) instead of to the waves of one workgroup.
 __device__ __forceinline__ void stencil_role_narrow(float c0, float c1, const float *__restrict__ A0,
                                                     float *__restrict__ Anext, int nx, int ny, int nz,
                                                     int grid_dimension_x, int grid_dimension_y,
-                                                    int role_block, int role_blocks, int start, int end,
-                                                    int tid, int role_threads)
+                                                    const StencilRange rg, unsigned tasks, bool spread,
+                                                    int role_block, int role_blocks, int tid, int role_threads)
 {
     const int lane = tid & 63;
     const int wave = tid >> 6;
     const int waves = role_threads >> 6;
-    const int planes = nz - 2;
-    const unsigned runs = (unsigned)(planes + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
-    const unsigned tasks = (unsigned)(end - start) * runs;
     const unsigned stride = (unsigned)role_blocks * waves;
-    // task t: block = start + t / runs, run = t % runs.
-    // two runs in flight per wave: the loads of run n+1 are issued before run n is computed
+    // tasks of segment 0, of a whole part, of the last segment
+    const StencilRange::Segment g0 = rg.segment(0);
+    const unsigned n_first = (g0.hi - g0.lo) * (g0.r1 - g0.r0);
     StencilRun<STENCIL_TILE_Y, STENCIL_Z_RUN> ra, rb;
     auto start_run = [&](StencilRun<STENCIL_TILE_Y, STENCIL_Z_RUN> &r, unsigned t) {
-        const unsigned pos = (unsigned)start + t / runs;
-        const int run = (int)(t % runs);
-        const int bx = pos % grid_dimension_x;
-        const int by = (pos / grid_dimension_x) % grid_dimension_y;
+        // locate the segment of task t: the first one, or walk the following ones
+        StencilRange::Segment g = g0;
+        unsigned local = t;
+        if (t >= n_first) {
+            local = t - n_first;
+            for (unsigned s = 1; s < rg.parts; ++s) {
+                g = rg.segment(s);
+                const unsigned n = (g.hi - g.lo) * (g.r1 - g.r0);
+                if (local < n) break;
+                local -= n;
+            }
+        }
+        const unsigned nr = g.r1 - g.r0;
+        const unsigned block = g.lo + local / nr;
+        const int run = (int)(g.r0 + local % nr);
+        const int bx = block % (unsigned)grid_dimension_x;
+        const int by = (block / (unsigned)grid_dimension_x) % (unsigned)grid_dimension_y;
         const int k_first = 1 + run * STENCIL_Z_RUN;
         r.issue(A0, nx, ny, k_first, min(STENCIL_Z_RUN, nz - 1 - k_first), bx * 2 * STENCIL_TILE_X,
                 by * STENCIL_TILE_Y, lane);
     };
-    unsigned t = (unsigned)role_block * waves + wave;
+    unsigned t = spread ? (unsigned)wave * role_blocks + role_block : (unsigned)role_block * waves + wave;
     if (t >= tasks) return;
     start_run(ra, t);
     for (;;) {
@@ -308,27 +373,28 @@ __device__ __forceinline__ void stencil_role_narrow(float c0, float c1, const fl
     }
 }
 
+// Wide form: a task is (quad of blocks, run), marched plane by plane.  Quads are cut on the
+// block grid (columns 4*qx .. 4*qx+3 of a block row); blocks [lo, hi) touch block rows
+// lo / gx .. (hi - 1) / gx.  The range is served as at most three pieces: the part it starts
+// inside (if it does not start on a part boundary, or has only that one), all whole parts as
+// ONE piece -- consecutive parts are consecutive runs, so the tasks of the piece are (row,
+// run, quad) with the row index fastest: the waves of a workgroup take vertically adjacent
+// quads of the same run (the row above one quad is the last own row of the next wave's quad,
+// so those halo loads hit in the CU's cache), and neighbouring runs of the same rows go to
+// workgroups that are dispatched together -- and the part it ends inside.
 __device__ __forceinline__ void stencil_role_wide(float c0, float c1, const float *__restrict__ A0,
                                                   float *__restrict__ Anext, int nx, int ny, int nz,
                                                   int grid_dimension_x, int grid_dimension_y,
-                                                  int role_block, int role_blocks, int start, int end,
+                                                  const StencilRange rg, int role_block, int role_blocks,
                                                   int tid, int role_threads)
 {
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // task bookkeeping stays in scalar registers
     const int waves = role_threads >> 6;
-    const int planes = nz - 2;
-    const unsigned runs = (unsigned)(planes + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN;
-    // Quads are cut on the block grid (columns 4*qx .. 4*qx+3 of a block row); the range
-    // [start, end) of block positions touches block rows first_row .. last_row, a position
-    // being row * grid_dimension_x + bx with the row wrapping modulo grid_dimension_y.
     const unsigned gdx = (unsigned)grid_dimension_x;
     const unsigned quads_per_row = (gdx + 3) / 4;
-    const unsigned first_row = (unsigned)start / gdx;
-    const unsigned last_row = (unsigned)(end - 1) / gdx;
-    const unsigned rows = last_row - first_row + 1;
-    const unsigned tasks = rows * quads_per_row * runs;
     const unsigned stride = (unsigned)role_blocks * waves;
+    const unsigned me = (unsigned)role_block * waves + wave;
     StencilQuadMarch<STENCIL_Z_RUN> m;
     m.A0 = A0;
     m.Anext = Anext;
@@ -336,41 +402,89 @@ __device__ __forceinline__ void stencil_role_wide(float c0, float c1, const floa
     m.ny = ny;
     m.lane = lane;
     m.plane = (size_t)nx * (size_t)ny;
-    for (unsigned t = (unsigned)role_block * waves + wave; t < tasks; t += stride) {
-        // consecutive tasks (the waves of one workgroup) are vertically adjacent quads of the
-        // same run: the row above one quad is the last own row of the next wave's quad, so
-        // those halo loads hit in the CU's cache instead of costing a second L2 request
-        const unsigned row = first_row + t % rows;
-        const unsigned rest = t / rows;
-        const int run = (int)(rest % runs);
-        const unsigned qx = rest / runs;
-        unsigned block_ok = 0;   // bit b: block 4*qx + b exists and its position is in range
-#pragma unroll
-        for (unsigned b = 0; b < 4; ++b) {
-            const unsigned bx = 4 * qx + b;
-            const unsigned pos = row * gdx + bx;
-            if (bx < gdx && pos >= (unsigned)start && pos < (unsigned)end) block_ok |= 1u << b;
+    // runs of all parts before unwrapped part index q
+    auto runs_before = [&](unsigned q) { return (q / rg.gz) * rg.runs + (q % rg.gz) * rg.runs / rg.gz; };
+    const bool head = rg.lo_first != 0 || rg.parts == 1;           // a piece of its own for the first part
+    const bool tail = rg.parts > 1 && rg.cut_last != 0;            // ... and for the last one
+    const unsigned whole_first = rg.first_part + (head ? 1u : 0u);
+    const unsigned whole = rg.parts - (head ? 1u : 0u) - (tail ? 1u : 0u);
+    unsigned base = 0;   // tasks of the pieces before this one
+    for (int piece = 0; piece < 3; ++piece) {
+        unsigned lo, hi, q0, q1;   // blocks and unwrapped parts [q0, q1) of the piece
+        if (piece == 0) {
+            if (!head) continue;
+            lo = rg.lo_first;
+            hi = rg.parts == 1 ? rg.blocks - rg.cut_last : rg.blocks;
+            q0 = rg.first_part;
+            q1 = q0 + 1;
+        } else if (piece == 1) {
+            if (whole == 0) continue;
+            lo = 0;
+            hi = rg.blocks;
+            q0 = whole_first;
+            q1 = q0 + whole;
+        } else {
+            if (!tail) continue;
+            lo = 0;
+            hi = rg.blocks - rg.cut_last;
+            q0 = rg.first_part + rg.parts - 1;
+            q1 = q0 + 1;
         }
-        if (block_ok == 0) continue;
-        const int k_first = 1 + run * STENCIL_Z_RUN;
-        m.run(c0, c1, k_first, min(STENCIL_Z_RUN, nz - 1 - k_first), (int)(qx * 4 * 2 * STENCIL_TILE_X),
-              (int)(row % (unsigned)grid_dimension_y) * STENCIL_TILE_Y, block_ok, (run & 1) == 0);
+        const unsigned run_first = runs_before(q0);
+        const unsigned nr = runs_before(q1) - run_first;
+        const unsigned first_row = lo / gdx;
+        const unsigned rows = (hi - 1) / gdx - first_row + 1;
+        const unsigned tasks = rows * quads_per_row * nr;
+        // this wave's tasks of the piece: global task numbers base + local, = me modulo stride
+        unsigned local = (me + stride - base % stride) % stride;
+        for (; local < tasks; local += stride) {
+            const unsigned row = first_row + local % rows;
+            const unsigned rest = local / rows;
+            const int run = (int)((run_first + rest % nr) % rg.runs);
+            const unsigned qx = rest / nr;
+            unsigned block_ok = 0;   // bit b: block 4*qx + b exists and is one of the piece's
+#pragma unroll
+            for (unsigned b = 0; b < 4; ++b) {
+                const unsigned bx = 4 * qx + b;
+                const unsigned pos = row * gdx + bx;
+                if (bx < gdx && pos >= lo && pos < hi) block_ok |= 1u << b;
+            }
+            if (block_ok == 0) continue;
+            const int k_first = 1 + run * STENCIL_Z_RUN;
+            m.run(c0, c1, k_first, min(STENCIL_Z_RUN, nz - 1 - k_first), (int)(qx * 4 * 2 * STENCIL_TILE_X),
+                  (int)(row % (unsigned)grid_dimension_y) * STENCIL_TILE_Y, block_ok, (run & 1) == 0);
+        }
+        base += tasks;
     }
 }
 
 __device__ __forceinline__ void stencil_role(float c0, float c1, const float *__restrict__ A0,
                                              float *__restrict__ Anext, int nx, int ny, int nz,
-                                             int grid_dimension_x, int grid_dimension_y,
+                                             int grid_dimension_x, int grid_dimension_y, int grid_dimension_z,
                                              int role_block, int role_blocks, int start, int end,
                                              int tid, int role_threads)
 {
-    if (nz - 2 < 1 || end <= start) return;
-    if ((nx & 3) == 0)
-        stencil_role_wide(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, role_block,
-                          role_blocks, start, end, tid, role_threads);
+    if (nz - 2 < 1 || end <= start || start < 0) return;
+    const StencilRange rg(grid_dimension_x, grid_dimension_y, grid_dimension_z, nz, start, end);
+    // (block, run) tasks of the range
+    unsigned tasks = 0;
+    for (unsigned s = 0; s < rg.parts; ++s) {
+        const StencilRange::Segment g = rg.segment(s);
+        tasks += (g.hi - g.lo) * (g.r1 - g.r0);
+    }
+    const unsigned role_waves = (unsigned)role_blocks * (unsigned)(role_threads >> 6);
+    // Rows that are 16-byte aligned take the wide form -- unless the range is short: when every
+    // wave gets at most two runs, the narrow form's "all loads of a run at once" ends after one
+    // trip to memory where the march makes five, and latency is all that counts.  Its dword
+    // accesses move bytes at half the wide form's rate, so beyond STENCIL_SHORT_RANGE_TASKS runs
+    // (a quarter of the 512 x 512 x 64 sweep, where the two forms take the same time on 256 CUs)
+    // the march wins whatever the launch.
+    if ((nx & 3) == 0 && (tasks > 2 * role_waves || tasks > STENCIL_SHORT_RANGE_TASKS))
+        stencil_role_wide(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, rg, role_block,
+                          role_blocks, tid, role_threads);
     else
-        stencil_role_narrow(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, role_block,
-                            role_blocks, start, end, tid, role_threads);
+        stencil_role_narrow(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, rg, tasks,
+                            tasks <= role_waves, role_block, role_blocks, tid, role_threads);
 }
 
 }  // namespace tk

@@ -60,8 +60,14 @@ void OriSTENCILKernel::bind()
 {
     OriSTENCILParamsStruct *p = STENCILKernelParams;
     launchBlockDim = dim3(STENCIL_TILE_X, STENCIL_TILE_Y, 1);
+    // Block positions: (x, y) = the reference's blocks of 64 x 4 columns, z = runs of
+    // STENCIL_Z_RUN centre planes of a block column (the march along z of
+    // src/ori_kernel/stencil_kernel.cu:47-93 cut into pieces and made a grid dimension), so that a
+    // GPTB range can be as short as a few planes of a few blocks.  GPTBKernel takes its six
+    // dimension ints from here; the natural launch below runs the (x, y) grid, each block all of z.
+    const int runs = p->nz > 2 ? (p->nz - 2 + STENCIL_Z_RUN - 1) / STENCIL_Z_RUN : 1;
     launchGridDim = dim3((p->nx + STENCIL_TILE_X * 2 - 1) / (STENCIL_TILE_X * 2),
-                         (p->ny + STENCIL_TILE_Y - 1) / STENCIL_TILE_Y, 1);
+                         (p->ny + STENCIL_TILE_Y - 1) / STENCIL_TILE_Y, runs);
     kernelParams = {&p->c0, &p->c1, &p->A0, &p->Anext, &p->nx, &p->ny, &p->nz};
     this->smem = 0;
     auto it = fmap.find("ori_stencil");
@@ -79,6 +85,7 @@ void OriSTENCILKernel::swapGrids()
 void OriSTENCILKernel::executeImpl(cudaStream_t stream)
 {
     if (!kernelFunc) logger.ERROR("load kernel {ori_stencil} failed!");
-    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
+    const dim3 blocks(launchGridDim.x, launchGridDim.y, 1);
+    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, blocks.raw(), launchBlockDim.raw(),
                                 (void **)this->kernelParams.data(), 0, stream));
 }

@@ -44,8 +44,9 @@ REFERENCE_KERNEL_INFO = {
 # benchmark's problem size.
 KERNEL_INFO = {
     "tzgemm": {"register": 160, "shared_memory": 131072, "blocksize": 256, "solo_ptb_blks": 1},
+    # 1024 blocks of 64 x 4 columns x 8 runs of 8 centre planes
     "stencil": {"register": 48, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
-                "ori_blks": 1024},
+                "ori_blks": 8192},
     "lbm": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
             "ori_blks": 18000},
     # 1024 blocks of 256 voxels x 16 chunks of 128 k records

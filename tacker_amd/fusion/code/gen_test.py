@@ -45,7 +45,7 @@ def make_inputs(np, torch, ta, be, small):
         out = a0.clone()
         c0 = float(np.float32(1.0 / 6.0))
         c1 = float(np.float32(1.0 / 36.0))
-        return ta.ori_stencil_create(c0, c1, a0, out), ta.stencil_blocks(shape[2], shape[1]), [out]
+        return ta.ori_stencil_create(c0, c1, a0, out), ta.stencil_blocks(shape[2], shape[1], shape[0]), [out]
     if be == "lbm":
         sx, sy, sz = (120, 6, 5) if small else (120, 120, 150)
         cells = sx * sy * sz

@@ -35,7 +35,7 @@ ROLES = {
                    ("int", "nx"), ("int", "ny"), ("int", "nz")],
         "needs_sync": False,
         "call": ("tk::stencil_role({p}c0, {p}c1, {p}A0, {p}Anext, {p}nx, {p}ny, {p}nz, "
-                 "{p}grid_dimension_x, {p}grid_dimension_y, {block}, {blocks}, "
+                 "{p}grid_dimension_x, {p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, "
                  "{p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "lbm": {

@@ -299,23 +299,51 @@ def test_stencil_gptb_ranges_and_wrap():
 @pytest.mark.parametrize("nx", [520, 200])
 def test_stencil_wide_form_ranges_and_wrap(nx):
     # block rows are 9 (520) or 4 (200) blocks wide: quads of 4 blocks are ragged at the row
-    # end, ranges start and end inside quads, and positions past the grid wrap onto it
+    # end, ranges start and end inside quads and inside either of the two runs of 8 centre
+    # planes a block column of 13 planes has, and positions past the grid wrap onto it
     A0 = stencil_inputs(13, 10, nx)
     nblk = ta.stencil_blocks(nx, 10)
+    npos = ta.stencil_blocks(nx, 10, 13)
+    assert npos == 2 * nblk
     a0 = dev(A0)
     acc = torch.full_like(a0, -3.0)
     want = np.full_like(A0, -3.0)
-    cuts = [0, 1, 3, 6, 11, 13, nblk - 2, nblk]
+    cuts = [0, 1, 3, 6, 11, 13, nblk - 2, nblk + 5, npos - 3, npos]
     for s, e in zip(cuts[:-1], cuts[1:]):
         if e <= s:
             continue
-        ta.gptb_stencil(C0, C1, a0, acc, start=s, end=e, launch_grid=3, launch_block=128)
-        want = oracle.stencil_gptb(C0, C1, A0, want, s, e)
+        ta.gptb_stencil(C0, C1, a0, acc, start=s, end=e, launch_grid=1, launch_block=128)   # 2 waves: the march
+        want = oracle.stencil_gptb(C0, C1, A0, want, s, e, gdz="runs")
         assert np.array_equal(host(acc), want), (s, e)
     assert np.array_equal(want, oracle.stencil(C0, C1, A0, np.full_like(A0, -3.0)))
     acc2 = torch.full_like(a0, -3.0)
-    ta.gptb_stencil(C0, C1, a0, acc2, start=nblk + 2, end=2 * nblk - 1)   # wraps onto blocks 2 .. nblk-2
-    assert np.array_equal(host(acc2), oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), 2, nblk - 1))
+    ta.gptb_stencil(C0, C1, a0, acc2, start=npos + 2, end=2 * npos - 1, launch_grid=2)   # wraps onto 2 .. npos-2
+    assert np.array_equal(host(acc2), oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), 2, npos - 1, gdz="runs"))
+
+
+@pytest.mark.parametrize("shape", [(30, 20, 260), (27, 9, 130), (64, 24, 512)])
+@pytest.mark.parametrize("grid", [1, 7, 256])
+def test_stencil_any_tiling_of_the_position_grid_is_one_sweep(shape, grid):
+    # positions = blocks x runs of 8 centre planes; few workgroups march quads of blocks plane by
+    # plane, many (every wave at most two runs) issue all loads of a run at once: same bits
+    nz, ny, nx = shape
+    A0 = stencil_inputs(*shape, seed=nz + nx)
+    npos = ta.stencil_blocks(nx, ny, nz)
+    assert npos == ta.stencil_blocks(nx, ny) * -(-(nz - 2) // 8)
+    want = oracle.stencil(C0, C1, A0, np.full_like(A0, -3.0))
+    a0 = dev(A0)
+    rng = np.random.default_rng(grid + nz)
+    cuts = sorted(set([0, npos] + list(rng.integers(1, npos, 9))))
+    acc = torch.full_like(a0, -3.0)
+    ranges = list(zip(cuts[:-1], cuts[1:]))
+    for i in rng.permutation(len(ranges)):            # in any order
+        ta.gptb_stencil(C0, C1, a0, acc, start=int(ranges[i][0]), end=int(ranges[i][1]), launch_grid=grid)
+    assert np.array_equal(host(acc), want)
+    # one range alone writes exactly what the oracle's restatement of the position grid writes
+    s, e = int(cuts[1]), int(cuts[3])
+    one = torch.full_like(a0, -3.0)
+    ta.gptb_stencil(C0, C1, a0, one, start=s, end=e, launch_grid=grid)
+    assert np.array_equal(host(one), oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), s, e, gdz="runs"))
 
 
 def test_stencil_iterations_ping_pong():

@@ -407,10 +407,15 @@ def test_create_kernel_geometry_and_memoisation(fake):
     fake.tacker_kernel_info(k1, info)
     per_cu = fake.tacker_get_kernel_info(b"stencil", b"solo_ptb_blks")
     assert info[0] == 256 * per_cu and info[1] == fake.tacker_get_kernel_info(b"stencil", b"blocksize")
-    assert (info[2], info[3]) == (0, 1024) and (info[6], info[7]) == (8, 128)
+    # 512 x 512 x 64: 8 x 128 blocks of 64 x 4 columns (fusion/code/kinfo.json "stencil.ori_blks" = 1024)
+    # times 8 runs of 8 centre planes
+    assert (info[2], info[3]) == (0, 8192) and (info[6], info[7]) == (8, 128)
+    assert fake.tacker_stencil_blocks(512, 512, 64) == 8192 and fake.tacker_stencil_blocks(130, 12, 5) == 9
     fake.tk_fake_reset()
     assert fake.tacker_kernel_execute(k1, None) == 0
-    assert launches(fake)[0]["key"] == "gptb_stencil"
+    l = launches(fake)[0]
+    assert l["key"] == "gptb_stencil"
+    assert [as_int(x) for x in l["args"][7:13]] == [8, 128, 8, 32, 4, 1]     # grid (8, 128, 8 runs), block (32, 4)
 
 
 def test_host_half_conversion_matches_numpy():
@@ -560,13 +565,13 @@ def test_task_manager_calibrates_block_counts_per_kernel(fake, small_vgg):
     blocks = tm.calibrated_blocks()
     mixable = [i for i, k in enumerate(small_vgg.kernels()) if k["mixable"]]
     assert len(blocks) == n and len(mixable) == 16
-    assert all(blocks[i] == 1024 for i in mixable) and all(blocks[i] == 0 for i in range(n) if i not in mixable)
-    assert rep["mix_times"] == 16 and rep["be_blocks_executed"] == 16 * 1024
-    # 7 block counts (1/64 ... 1) x (1 warm-up + 3 timed) passes of 16 fused launches, then 2 queries
+    assert all(blocks[i] == 8192 for i in mixable) and all(blocks[i] == 0 for i in range(n) if i not in mixable)
+    assert rep["mix_times"] == 16 and rep["be_blocks_executed"] == 16 * 8192
+    # 9 block counts (1/256 ... 1) x (1 warm-up + 3 timed) passes of 16 fused launches, then 2 queries
     fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
-    assert len(fused) == 7 * 4 * 16 + 2 * 16
-    ends = sorted({as_int(l["args"][15]) for l in fused[:7 * 4 * 16]})           # stencil ptb_end of the sweeps
-    assert ends == [16, 32, 64, 128, 256, 512, 1024]
+    assert len(fused) == 9 * 4 * 16 + 2 * 16
+    ends = sorted({as_int(l["args"][15]) for l in fused[:9 * 4 * 16]})           # stencil ptb_end of the sweeps
+    assert ends == [32, 64, 128, 256, 512, 1024, 2048, 4096, 8192]
     # LC kernels alone take 10 us, every fused launch 12 us: 20 % over a 10 % allowance -> nothing is co-located
     cheap = [0.01] * (n * 2 + 1)
     arr = (C.c_float * len(cheap))(*cheap)
@@ -576,13 +581,13 @@ def test_task_manager_calibrates_block_counts_per_kernel(fake, small_vgg):
     rep = tm.run("aker", raw_stream=None, second_stage=False)
     assert tm.calibrated_blocks() == [0] * n and rep["mix_times"] == 0 and rep["be_blocks_executed"] == 0
     fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
-    assert len(fused) == 4 * 16                                                  # only the first sweep (1/64)
+    assert len(fused) == 4 * 16                                                  # only the first sweep (1/256)
     # 5 % over: allowed, and it pays from 1/16 of the kernel up (10 us * n/N > 0.5 us) -> again the whole kernel
     fake.tk_fake_reset()
     fake.tk_fake_set_event_ms(0.0105)
     fake.tk_fake_push_event_ms(arr, len(cheap))
     tm.run("aker", raw_stream=None, second_stage=False)
-    assert all(tm.calibrated_blocks()[i] == 1024 for i in mixable)
+    assert all(tm.calibrated_blocks()[i] == 8192 for i in mixable)
     tm.set_calibration(False, 0.10)                                              # back to the kinfo table
     fake.tk_fake_reset()
     fake.tk_fake_set_event_ms(0.01)
@@ -609,7 +614,7 @@ def test_task_manager_cursor_advances_and_wraps(fake, small_vgg):
     fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
     assert len(fused) == 3 * 16
     for l in fused:
-        assert (as_int(l["args"][13]), as_int(l["args"][15])) == (0, 1024)
+        assert (as_int(l["args"][13]), as_int(l["args"][15])) == (0, 8192)
     assert tm.report()["be_task_finish_num"] == 48
     tm.close()
     tm = ta.TaskManager(small_vgg, "stencil", None, library=fake)

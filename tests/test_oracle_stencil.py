@@ -88,6 +88,41 @@ def test_gptb_partition_equals_full_and_wraps():
     assert not touched[:, :, :64].any() and not touched[:, :, 128:].any()
 
 
+def test_z_parts_of_the_position_grid_tile_the_sweep():
+    # the position grid (gdx, gdy, gdz) with gdz runs of zrun centre planes: any tiling is one sweep,
+    # a position writes only its block's columns and its run's planes, gdz = 1 is the block grid
+    rng = np.random.default_rng(8)
+    A0 = rng.uniform(0, 1, (21, 12, 130)).astype(np.float32)
+    gdx, gdy = oracle.stencil_grid(130, 12)
+    blocks = gdx * gdy
+    full = oracle.stencil(C0, C1, A0, A0)
+    for zrun in (8, 5, 19, 40):
+        runs = -(-(21 - 2) // zrun)
+        npos = blocks * runs
+        assert oracle.stencil_positions(130, 12, 21, zrun) == npos
+        acc = A0.copy()
+        for s, e in [(5, npos), (0, 2), (2, 5)]:
+            acc = oracle.stencil_gptb(C0, C1, A0, acc, s, e, gdz=runs, zrun=zrun)
+        assert np.array_equal(acc, full), zrun
+        # position p = block p % blocks, run p // blocks: block (1, 1) = 4, its second run if there is one
+        r = min(1, runs - 1)
+        part = oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), r * blocks + 4, r * blocks + 5,
+                                   gdz=runs, zrun=zrun)
+        touched = part != -3.0
+        k_lo, k_hi = 1 + r * zrun, min(20, 1 + (r + 1) * zrun)
+        want = np.zeros(A0.shape, bool)
+        want[k_lo:k_hi, 4:8, 64:128] = True
+        assert np.array_equal(touched, want)
+        assert np.array_equal(part[want], full[want])
+    # fewer parts than runs: a part is a group of consecutive runs
+    acc = A0.copy()
+    for s, e in [(0, 7), (7, 2 * blocks)]:
+        acc = oracle.stencil_gptb(C0, C1, A0, acc, s, e, gdz=2, zrun=4)   # 5 runs in 2 parts: runs 0-1, 2-4
+    assert np.array_equal(acc, full)
+    half = oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), 0, blocks, gdz=2, zrun=4)
+    assert np.all(half[9:] == -3.0) and np.all(half[1:9, 1:-1, 1:-1] != -3.0)
+
+
 def test_reference_launch_shape_known_answer():
     # fusion/code/kinfo.json "stencil.ori_blks" = 1024 = ceil(512/64)*ceil(512/4)
     gdx, gdy = oracle.stencil_grid(512, 512)
