@@ -368,6 +368,10 @@ TK_API int tacker_kernel_swap_buffers(tacker_kernel_t ori);
 /* out = {launch grid x, launch block x, ptb_start, ptb_end, number of kernel
  * parameters, smem, ori grid x, ori grid y} (start/end are 0 for non-GPTB objects) */
 TK_API int tacker_kernel_info(tacker_kernel_t kernel, int out[8]);
+/* copies `bytes` (4 or 8) of kernel parameter `index` -- entry `index` of Kernel::kernelParams
+ * (src/Kernel.h:36), the void*-per-argument vector every launch passes to the driver -- into
+ * `out`.  How a caller reaches the buffers an Ori*Kernel(id) constructor allocated itself. */
+TK_API int tacker_kernel_param(tacker_kernel_t kernel, int index, void *out, int bytes);
 TK_API int tacker_kernel_destroy(tacker_kernel_t kernel);
 /* value of the device word kernels raise when they have to give up; reading clears it.
  * Bit 0: a role-local barrier of a wave-split fused kernel stopped waiting (its poll is
@@ -442,7 +446,15 @@ TK_API int tacker_task_manager_fusion_disabled(tacker_task_manager_t tm);
 /* "[Mix] BE task1 + task2 took ..." (src/TaskManager.cu:693): average time of the fused launch of
  * the two best-effort kernels measured by the last run with a second stage; 0 if none ran. */
 TK_API float tacker_task_manager_be_mix_ms(tacker_task_manager_t tm);
-/* which = 0: per-query latency of the co-located queries, 1: of the solo profiling queries */
+/* No counterpart in the reference (its query latency is a sum of per-kernel intervals with a
+ * synchronisation after each, src/TaskManager.cu:620-624): after the co-located queries, run
+ * `queries` more of each kind -- every kernel alone, and with the best-effort blocks the last
+ * co-located query carried -- with nothing between the launches of a query, each timed by one
+ * pair of events and by the host's steady clock.  0 (default) = off. */
+TK_API int tacker_task_manager_set_end_to_end(tacker_task_manager_t tm, int queries);
+/* which = 0: per-query latency of the co-located queries (sum of per-kernel intervals), 1: of the
+ * solo profiling queries; end-to-end queries (tacker_task_manager_set_end_to_end): 2 co-located and
+ * 3 solo by events, 4 co-located and 5 solo by the host clock */
 TK_API int tacker_task_manager_latencies(tacker_task_manager_t tm, int which, float *out, int cap);
 
 /* the scheduler's arithmetic on its own (src/TaskManager.cu:586-640) */

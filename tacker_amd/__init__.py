@@ -91,6 +91,7 @@ def _declare(lib):
     lib.tacker_kernel_execute.argtypes = [vp, vp]
     lib.tacker_kernel_swap_buffers.argtypes = [vp]
     lib.tacker_kernel_info.argtypes = [vp, C.POINTER(i)]
+    lib.tacker_kernel_param.argtypes = [vp, i, vp, i]
     lib.tacker_kernel_destroy.argtypes = [vp]
     lib.tacker_spin_fail_flag.argtypes = [C.POINTER(i)]
     lib.tacker_float_to_half_bits.argtypes = [f]
@@ -118,6 +119,7 @@ def _declare(lib):
     lib.tacker_task_manager_set_fusion_strikes.argtypes = [vp, i]
     lib.tacker_task_manager_fusion_disabled.argtypes = [vp]
     lib.tacker_task_manager_set_calibration.argtypes = [vp, i, f]
+    lib.tacker_task_manager_set_end_to_end.argtypes = [vp, i]
     lib.tacker_task_manager_calibrated_blocks.argtypes = [vp, vp, i]
     lib.tacker_task_manager_be_mix_ms.argtypes = [vp]
     lib.tacker_task_manager_be_mix_ms.restype = f
@@ -474,6 +476,13 @@ class KernelHandle:
         keys = ("grid", "block", "ptb_start", "ptb_end", "nparams", "smem", "ori_grid_x", "ori_grid_y")
         return dict(zip(keys, out))
 
+    def param(self, index, kind="ptr"):
+        """Kernel parameter ``index`` as the launch passes it: a device address (``ptr``), ``int`` or ``float``."""
+        ctype = {"ptr": C.c_void_p, "int": C.c_int, "float": C.c_float}[kind]
+        out = ctype()
+        check(lib().tacker_kernel_param(self.handle, index, C.byref(out), C.sizeof(ctype)), "tacker_kernel_param")
+        return out.value or 0
+
     def set_range(self, *r):
         if len(r) == 2:
             check(lib().tacker_gptb_set_range(self.handle, *r), "tacker_gptb_set_range")
@@ -719,11 +728,22 @@ class TaskManager:
     def be_mix_ms(self):
         return self.l.tacker_task_manager_be_mix_ms(self.h)
 
-    def latencies(self, solo=False):
-        cap = 1 << 20
+    def set_end_to_end(self, queries):
+        check(self.l.tacker_task_manager_set_end_to_end(self.h, queries), "set_end_to_end")
+
+    LATENCY_KINDS = {"colocated": 0, "solo": 1, "e2e_colocated": 2, "e2e_solo": 3,
+                     "e2e_colocated_wall": 4, "e2e_solo_wall": 5}
+
+    def latencies(self, solo=False, kind=None):
+        """Per-query latencies in ms.  ``kind`` picks one of LATENCY_KINDS: the sums of per-kernel
+        intervals (``colocated``, ``solo``) or whole queries timed end to end by events / by the
+        host clock (``e2e_*``, after ``set_end_to_end``).  Without it, ``solo`` picks between the
+        first two."""
+        which = self.LATENCY_KINDS[kind] if kind is not None else (1 if solo else 0)
+        cap = 1 << 16
         buf = (C.c_float * cap)()
-        n = self.l.tacker_task_manager_latencies(self.h, 1 if solo else 0, buf, cap)
-        return list(buf[:n])
+        n = self.l.tacker_task_manager_latencies(self.h, which, buf, cap)
+        return list(buf[:max(n, 0)])
 
     def close(self):
         if self.h:

@@ -281,6 +281,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     int be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;
     float qos_headroom = policy.qos_budget_ms;
     std::vector<int> strikes(nk, 0);   // consecutive fused launches of kernel i that did not pay
+    std::vector<int> carried(nk, 0);   // best-effort blocks kernel i's launch carried in the last query
     for (int q = 0; q < queries; ++q) {
         lc_task->initExecution();
         qos_headroom = policy.qos_budget_ms;
@@ -326,6 +327,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             }
             const float duration = watch.stop(stream);
             query_ms += duration;
+            carried[idx] = cd_block_num;
             const unsigned mixed = cd_block_num > 0 ? lc_kernel->mixable : 0u;
             const QosPolicy::Outcome o = QosPolicy::account(mixed, duration, lc_kernel_time_vec[idx],
                                                             report.be1_solo_ms, cd_block_num, be_total);
@@ -339,6 +341,34 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         }
         report.be_blocks_executed = cd_block_num_executed;
         report.query_latency_ms.push_back(query_ms);
+    }
+    // whole queries end to end, nothing between their launches: every kernel alone, then with what
+    // the last co-located query carried (the cursor keeps walking the best-effort kernel's blocks)
+    for (int kind = 0; kind < 2 && end_to_end_queries > 0; ++kind) {
+        std::vector<float> &by_event = kind ? report.e2e_colocated_ms : report.e2e_solo_ms;
+        std::vector<float> &by_clock = kind ? report.e2e_colocated_wall_ms : report.e2e_solo_wall_ms;
+        for (int q = -2; q < end_to_end_queries; ++q) {   // two untimed queries first
+            lc_task->initExecution();
+            TK_SAFE_CALL(tkStreamSynchronize(stream));
+            const auto t0 = std::chrono::steady_clock::now();
+            watch.start(stream);
+            for (size_t idx = 0; idx < nk; ++idx) {
+                Kernel *lc_kernel = lc_task->kernels[idx];
+                if (kind == 0 || carried[idx] <= 0 || lc_kernel->mixable == 0) {
+                    lc_kernel->execute(stream);
+                    continue;
+                }
+                const int end = std::min(be_cursor + carried[idx], be_total);
+                launch_mixed(lc_kernel, be_cursor, end);
+                be_cursor = end >= be_total ? be_kernel1->gptbParams.ptb_start_block_pos : end;
+            }
+            const float ms = watch.stop(stream);   // waits for the query's last kernel
+            const float wall = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+            if (q >= 0) {
+                by_event.push_back(ms);
+                by_clock.push_back(wall);
+            }
+        }
     }
     report.qos_headroom_left_ms = qos_headroom;
     report.fusion_disabled = 0;

@@ -65,6 +65,10 @@ struct TaskManagerReport {
     float be_mix_ms = 0.0f;             // fused launch of the two BE kernels (0 if the pair has no kernel)
     std::vector<float> query_latency_ms;   // one entry per co-located LC query
     std::vector<float> solo_latency_ms;    // one entry per solo LC query (profiling passes)
+    // whole queries timed end to end (end_to_end_queries > 0): all launches of a query between one
+    // pair of events, no synchronisation between kernels; and the same span on the host clock
+    std::vector<float> e2e_colocated_ms, e2e_solo_ms;
+    std::vector<float> e2e_colocated_wall_ms, e2e_solo_wall_ms;
 };
 
 class TaskManager {
@@ -103,6 +107,13 @@ public:
     bool calibrate_blocks = false;
     float calibrate_max_stretch = 0.10f;
     std::vector<int> calibrated_blocks;   // per LC kernel, filled by the last calibrated run
+    // Not in the reference (its latency of a query is the sum of per-kernel intervals, each
+    // followed by a synchronisation, src/TaskManager.cu:620-624): after the co-located queries,
+    // run this many more queries of each kind -- every kernel alone, and with the best-effort
+    // blocks the last co-located query carried -- with nothing between the launches of a query,
+    // timed by one pair of events and by the host's steady clock around the query.  What a
+    // client of the latency-critical service would see: launch gaps and host time included.
+    int end_to_end_queries = 0;
     TaskManagerReport report;
 
 private:

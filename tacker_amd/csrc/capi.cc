@@ -805,6 +805,16 @@ int tacker_kernel_info(tacker_kernel_t h, int out[8])
     return TK_SUCCESS;
 }
 
+int tacker_kernel_param(tacker_kernel_t h, int index, void *out, int bytes)
+{
+    Kernel *k = static_cast<Kernel *>(h);
+    if (!k || !out) return fail(TK_ERROR_INVALID_VALUE, "null kernel or output");
+    if (index < 0 || (size_t)index >= k->kernelParams.size() || (bytes != 4 && bytes != 8))
+        return fail(TK_ERROR_INVALID_VALUE, "parameter index out of range, or size not 4 or 8 bytes");
+    memcpy(out, k->kernelParams[index], (size_t)bytes);
+    return TK_SUCCESS;
+}
+
 int tacker_kernel_destroy(tacker_kernel_t h)
 {
     delete static_cast<Kernel *>(h);
@@ -1020,6 +1030,14 @@ int tacker_task_manager_set_calibration(tacker_task_manager_t h, int on, float m
     return TK_SUCCESS;
 }
 
+int tacker_task_manager_set_end_to_end(tacker_task_manager_t h, int queries)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || queries < 0) return fail(TK_ERROR_INVALID_VALUE, "bad task manager handle or query count");
+    tm->end_to_end_queries = queries;
+    return TK_SUCCESS;
+}
+
 int tacker_task_manager_calibrated_blocks(tacker_task_manager_t h, int *out, int cap)
 {
     TaskManager *tm = static_cast<TaskManager *>(h);
@@ -1045,7 +1063,11 @@ int tacker_task_manager_latencies(tacker_task_manager_t h, int which, float *out
 {
     TaskManager *tm = static_cast<TaskManager *>(h);
     if (!tm || !out) return -1;
-    const std::vector<float> &v = which ? tm->report.solo_latency_ms : tm->report.query_latency_ms;
+    const std::vector<float> *all[] = {&tm->report.query_latency_ms,      &tm->report.solo_latency_ms,
+                                       &tm->report.e2e_colocated_ms,      &tm->report.e2e_solo_ms,
+                                       &tm->report.e2e_colocated_wall_ms, &tm->report.e2e_solo_wall_ms};
+    if (which < 0 || which > 5) return -1;
+    const std::vector<float> &v = *all[which];
     const int n = std::min((int)v.size(), cap);
     memcpy(out, v.data(), (size_t)n * sizeof(float));
     return n;

@@ -188,6 +188,19 @@ def test_task_manager_colocation_keeps_lc_results_and_reports():
     lat = tm.latencies()
     assert len(lat) == 4 and all(0 < v < 50.0 for v in lat)
     assert rep["qos_headroom_left_ms"] > 0
+    assert tm.latencies(kind="e2e_solo") == []
+    # whole queries between one pair of events: same logits, and never longer than the sum of
+    # per-kernel intervals with a synchronisation after each kernel
+    tm.set_end_to_end(5)
+    tm.run("aker", second_stage=False)
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
+    for kind in ("e2e_solo", "e2e_colocated", "e2e_solo_wall", "e2e_colocated_wall"):
+        got = tm.latencies(kind=kind)
+        assert len(got) == 5 and all(0 < v < 50.0 for v in got), kind
+    assert min(tm.latencies(kind="e2e_solo")) < min(tm.latencies(solo=True))
+    assert all(w >= e - 1e-3 for w, e in zip(tm.latencies(kind="e2e_solo_wall"), tm.latencies(kind="e2e_solo")))
+    tm.set_end_to_end(0)
     rep2 = tm.run("tacker", second_stage=False)
     assert rep2["n_colocated"] == 4
     torch.cuda.synchronize()
@@ -226,8 +239,19 @@ def test_create_kernel_objects_run_and_match_oracle_for_cp():
     info = k.info()
     # 32 x 512 blocks of 128 x 8 points, each in 4 parts of its x points
     assert (info["ptb_start"], info["ptb_end"]) == (0, 65536) and info["ori_grid_x"] == 32 and info["ori_grid_y"] == 512
+    assert info["nparams"] == 3 + 6 and k.param(0, "int") == 64 and k.param(1, "float") == np.float32(0.1)
     k.execute()
     torch.cuda.synchronize()
+    # the object's own inputs (src/ori_kernel/cp_kernel.cu:66-100): atoms 1..64 of the seeded
+    # 4000, plane z = 0, a zeroed 4096 x 4096 grid; rows of blocks from the top, middle and bottom
+    grid = ta.device_to_host(k.param(2), (4096, 4096), np.float32)
+    consts = oracle.cp_atoms_to_const(oracle.cp_initatoms(4000)[1:65], 0.0)
+    for first_row in (0, 2048, 4088):
+        rows = slice(first_row, first_row + 8)
+        lo = (first_row // 8) * 32                    # the 32 blocks of this row of blocks
+        want = oracle.cp(consts, np.zeros((4096, 4096), np.float32), start=lo, end=lo + 32)[rows]
+        assert np.array_equal(grid[rows].view(np.uint32), want.view(np.uint32)), first_row
+    assert np.count_nonzero(grid) == grid.size
     for name in ("stencil", "lbm", "mriq", "mrif"):
         ta.create_kernel(name).execute()
     torch.cuda.synchronize()

@@ -596,6 +596,44 @@ def test_task_manager_calibrates_block_counts_per_kernel(fake, small_vgg):
     tm.close()
 
 
+def test_task_manager_times_whole_queries_with_one_interval_each(fake, small_vgg):
+    n = len(small_vgg.kernels())
+    tm = ta.TaskManager(small_vgg, "stencil", None, library=fake)
+    tm.configure(warmup=0, profile=1, queries=1, verbose=0, qos_budget_ms=50.0, guard_ms=0.0)
+    tm.set_end_to_end(3)
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.01)
+    tm.run("aker", raw_stream=None, second_stage=False)
+    all_launches = launches(fake)
+    fused = [i for i, l in enumerate(all_launches) if l["key"].startswith("tzgemm_stencil")]
+    per_query = len(fused) // 6                # 1 co-located query + (2 untimed + 3 timed) end to end
+    assert per_query > 0 and len(fused) == 6 * per_query
+    # the sums of per-kernel intervals see n intervals a query, the end-to-end figures one
+    assert tm.latencies()[0] == pytest.approx(0.01 * n, rel=1e-4)
+    for kind in ("e2e_solo", "e2e_colocated"):
+        assert tm.latencies(kind=kind) == pytest.approx([0.01] * 3, rel=1e-4)
+    for kind in ("e2e_solo_wall", "e2e_colocated_wall"):
+        wall = tm.latencies(kind=kind)
+        assert len(wall) == 3 and all(w >= 0.0 for w in wall)
+    # the solo queries come first and fuse nothing: between the co-located query's last fused launch
+    # and the next one lie the five solo queries' launches
+    first_e2e_fused = fused[per_query]
+    solo_span = all_launches[fused[per_query - 1] + 1:first_e2e_fused]
+    assert len([l for l in solo_span if l["key"] == "gptb_tzgemm"]) >= 5 * 16
+    # the cursor keeps walking: each slice starts where the last ended, or wrapped
+    ranges = [(as_int(all_launches[i]["args"][13]), as_int(all_launches[i]["args"][15])) for i in fused]
+    for (a0, b0), (a1, b1) in zip(ranges, ranges[1:]):
+        assert a1 == b0 or a1 == 0
+    # a kernel carries at most what it carried in the co-located query (less where the cursor wraps)
+    sizes = [b - a for a, b in ranges]
+    for q in range(1, 6):
+        assert all(s <= c for s, c in zip(sizes[q * per_query:(q + 1) * per_query], sizes[:per_query]))
+    tm.set_end_to_end(0)
+    tm.run("aker", raw_stream=None, second_stage=False)
+    assert tm.latencies(kind="e2e_solo") == [] and tm.latencies(kind="e2e_colocated_wall") == []
+    tm.close()
+
+
 def test_task_manager_falls_back_to_solo_when_headroom_is_short(fake, small_vgg):
     fake.tk_fake_set_event_ms(0.01)
     n = len(small_vgg.kernels())
