@@ -359,6 +359,19 @@ TK_API tacker_kernel_t tacker_be_pair_create(tacker_kernel_t first_gptb, tacker_
 /* createMixKernel(name) (src/Creator.cu:341-816): the memoised fused pair "<a>_<b>" of the
  * memoised kernels createKernel(a), createKernel(b) over their full ranges. Never destroy. */
 TK_API tacker_kernel_t tacker_create_mix_kernel(const char *name);
+/* mixcublasSgemm(gemm_args, gptb_cd_kernel, cd_start_blk, cd_end_blk) (src/TaskManager.cu:309-400):
+ * one fused launch of the GEMM {M, N, K} (rounded up to whole tiles, on the global operand buffers,
+ * see tacker_global_gemm_buffers) with block positions [cd_start_blk, cd_end_blk) of the best-effort
+ * GPTB kernel; an empty range launches the GEMM alone.  What TaskManager calls for a latency-critical
+ * kernel that declares mixable = 1 and brings no operands of its own. */
+TK_API int tacker_mix_cublas_sgemm(const int mnk[3], tacker_kernel_t be_gptb, int cd_start_blk,
+                                   int cd_end_blk, tkStream_t stream);
+/* mixcudnnConvolutionForward(cudnn_args, ...) (src/TaskManager.cu:125-306): the same for a
+ * convolution given by its 14 integers {n, c, h, w, k, c, r, s, pad_h, pad_w, stride_h, stride_w,
+ * dilation_h, dilation_w}: im2col of the library's scratch image on the stream, then the fused
+ * launch of the GEMM {n*ho*wo, k, r*s*c} (get_mnk_from_cudnn_args, src/TaskManager.cu:92-123). */
+TK_API int tacker_mix_cudnn_convolution_forward(const int cudnn_args[14], tacker_kernel_t be_gptb,
+                                                int cd_start_blk, int cd_end_blk, tkStream_t stream);
 /* Kernel::execute(stream) */
 TK_API int tacker_kernel_execute(tacker_kernel_t kernel, tkStream_t stream);
 /* exchange the input and output grid of a stencil / lbm ori object (the
@@ -400,12 +413,15 @@ TK_API int tacker_task_kernel_count(tacker_task_t task);
 /* name (up to name_cap bytes), mixable flag, getArgs() (up to 14 ints, count in *nargs) */
 TK_API int tacker_task_kernel_info(tacker_task_t task, int index, char *name, int name_cap,
                                    int *mixable, int args[14], int *nargs);
-/* VGG16 only: output of convolution conv_index after bias+ReLU: device pointer and
- * dims = {H, W, channels, channel stride}; logits = column 0 of the last GEMM */
+/* VGG16 only: the buffer layer conv_index writes (0..12 the convolutions, 13..15 the three fully
+ * connected layers, whose result is one row: H = W = 1): device pointer and dims = {H, W, channels,
+ * channel stride}.  It holds the raw GEMM output 1.1 * A * B^T; the layer that reads it adds the bias
+ * and rectifies.  logits = the first `count` floats of the last layer's buffer */
 TK_API int tacker_task_activation(tacker_task_t task, int conv_index, float **ptr, int dims[4]);
 TK_API int tacker_task_logits(tacker_task_t task, const float **ptr, long *stride, int *count);
 /* VGG16 only: weights (f16 [dims[0]][dims[1]] = [Cout padded][9*Cin padded], k =
- * (kh*3+kw)*Cin + c) and bias (f32 [dims[0]]) of convolution conv_index */
+ * (kh*3+kw)*Cin + c) and bias (f32 [dims[0]]) of convolution conv_index; 13..15: of the fully
+ * connected layers ([out padded][in padded]; the last one has no bias: NULL) */
 TK_API int tacker_task_conv_params(tacker_task_t task, int conv_index, void **weights, float **bias,
                                    int dims[2]);
 TK_API int tacker_task_input(tacker_task_t task, float **host_ptr, int *bytes);

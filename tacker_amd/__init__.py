@@ -92,6 +92,8 @@ def _declare(lib):
     lib.tacker_kernel_swap_buffers.argtypes = [vp]
     lib.tacker_kernel_info.argtypes = [vp, C.POINTER(i)]
     lib.tacker_kernel_param.argtypes = [vp, i, vp, i]
+    lib.tacker_mix_cublas_sgemm.argtypes = [C.POINTER(i), vp, i, i, vp]
+    lib.tacker_mix_cudnn_convolution_forward.argtypes = [C.POINTER(i), vp, i, i, vp]
     lib.tacker_kernel_destroy.argtypes = [vp]
     lib.tacker_spin_fail_flag.argtypes = [C.POINTER(i)]
     lib.tacker_float_to_half_bits.argtypes = [f]
@@ -567,6 +569,21 @@ def be_pair_create(first_gptb, second_gptb, start1, end1, start2, end2, variant=
                         "MixKernel", keep=(first_gptb, second_gptb))
 
 
+def mix_cublas_sgemm(mnk, be_gptb, start, end, stream=None, library=None):
+    """mixcublasSgemm of the reference (src/TaskManager.cu:309-400): GEMM {M, N, K} on the global operand
+    buffers fused with block positions [start, end) of a best-effort GPTB kernel."""
+    l = library or lib()
+    check(l.tacker_mix_cublas_sgemm((C.c_int * 3)(*mnk), be_gptb.handle, start, end,
+                                    None if library else _stream(stream)), "mixcublasSgemm")
+
+
+def mix_cudnn_convolution_forward(args14, be_gptb, start, end, stream=None, library=None):
+    """mixcudnnConvolutionForward of the reference (src/TaskManager.cu:125-306)."""
+    l = library or lib()
+    check(l.tacker_mix_cudnn_convolution_forward((C.c_int * 14)(*args14), be_gptb.handle, start, end,
+                                                 None if library else _stream(stream)), "mixcudnnConvolutionForward")
+
+
 def create_mix_kernel(name):
     return KernelHandle(lib().tacker_create_mix_kernel(name.encode()), f"createMixKernel({name})", owned=False)
 
@@ -654,7 +671,8 @@ class LcTask:
         return p.value, tuple(dims)
 
     def conv_params(self, conv_index):
-        """(weights f16 [Np][Kp], bias f32 [Np]) of a convolution, copied to the host."""
+        """(weights f16 [Np][Kp], bias f32 [Np]) of a convolution (0..12) or a fully connected layer
+        (13..15; the last has no bias: zeros), copied to the host."""
         import numpy as np
         w, b = C.c_void_p(), C.c_void_p()
         dims = (C.c_int * 2)()
@@ -662,7 +680,7 @@ class LcTask:
         if rc:
             raise TackerError(self.l.tacker_last_error().decode())
         return (device_to_host(w.value, (dims[0], dims[1]), np.float16, self.l),
-                device_to_host(b.value, (dims[0],), np.float32, self.l))
+                device_to_host(b.value, (dims[0],), np.float32, self.l) if b.value else np.zeros(dims[0], np.float32))
 
     def logits(self):
         p = C.c_void_p()

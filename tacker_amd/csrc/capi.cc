@@ -765,6 +765,52 @@ int tacker_mix_set_range(tacker_kernel_t h, int be_start, int be_end, int tile_s
     return TK_SUCCESS;
 }
 
+namespace {
+int check_mix_call(GPTBKernel *be, int start, int end)
+{
+    if (!be) return fail(TK_ERROR_INVALID_VALUE, "the best-effort kernel must be a GPTB kernel object");
+    if (dynamic_cast<OriTZGEMMKernel *>(be->kernel_))
+        return fail(TK_ERROR_INVALID_VALUE, "the best-effort kernel cannot be the GEMM itself");
+    if (start < 0 || end < start) return fail(TK_ERROR_INVALID_VALUE, "bad block range");
+    return TK_SUCCESS;
+}
+}  // namespace
+
+int tacker_mix_cublas_sgemm(const int mnk[3], tacker_kernel_t be_gptb, int cd_start_blk, int cd_end_blk,
+                            tkStream_t stream)
+{
+    REQUIRE_INIT();
+    GPTBKernel *be = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(be_gptb));
+    const int rc = check_mix_call(be, cd_start_blk, cd_end_blk);
+    if (rc) return rc;
+    if (!mnk || mnk[0] <= 0 || mnk[1] <= 0 || mnk[2] <= 0) return fail(TK_ERROR_INVALID_VALUE, "bad GEMM dimensions");
+    return guarded([&]() -> int {
+        std::vector<int> args(mnk, mnk + 3);
+        mixcublasSgemm(args, be, cd_start_blk, cd_end_blk, stream);
+        return TK_SUCCESS;
+    });
+}
+
+int tacker_mix_cudnn_convolution_forward(const int cudnn_args[14], tacker_kernel_t be_gptb, int cd_start_blk,
+                                         int cd_end_blk, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    GPTBKernel *be = dynamic_cast<GPTBKernel *>(static_cast<Kernel *>(be_gptb));
+    const int rc = check_mix_call(be, cd_start_blk, cd_end_blk);
+    if (rc) return rc;
+    if (!cudnn_args) return fail(TK_ERROR_INVALID_VALUE, "null convolution arguments");
+    for (int i = 0; i < 14; ++i)
+        if (cudnn_args[i] < (i == 8 || i == 9 ? 0 : 1)) return fail(TK_ERROR_INVALID_VALUE, "bad convolution arguments");
+    std::vector<int> args(cudnn_args, cudnn_args + 14);
+    const int *a = cudnn_args;   // the dilated filter must fit the padded image in both directions
+    if (a[2] + 2 * a[8] < a[12] * (a[6] - 1) + 1 || a[3] + 2 * a[9] < a[13] * (a[7] - 1) + 1)
+        return fail(TK_ERROR_INVALID_VALUE, "the filter does not fit the input");
+    return guarded([&]() -> int {
+        mixcudnnConvolutionForward(args, be, cd_start_blk, cd_end_blk, stream);
+        return TK_SUCCESS;
+    });
+}
+
 int tacker_kernel_execute(tacker_kernel_t h, tkStream_t stream)
 {
     Kernel *k = static_cast<Kernel *>(h);
@@ -910,7 +956,7 @@ int tacker_task_kernel_info(tacker_task_t h, int index, char *name, int name_cap
 int tacker_task_activation(tacker_task_t h, int conv_index, float **ptr, int dims[4])
 {
     VGG16 *v = dynamic_cast<VGG16 *>(static_cast<Task *>(h));
-    if (!v || conv_index < 0 || conv_index >= 13) return fail(TK_ERROR_INVALID_VALUE, "bad activation index");
+    if (!v || conv_index < 0 || conv_index >= 16) return fail(TK_ERROR_INVALID_VALUE, "bad activation index");
     const VGG16::Act a = v->activation(conv_index);
     *ptr = a.ptr;
     dims[0] = a.H; dims[1] = a.W; dims[2] = a.C; dims[3] = a.ld;
@@ -920,7 +966,7 @@ int tacker_task_activation(tacker_task_t h, int conv_index, float **ptr, int dim
 int tacker_task_conv_params(tacker_task_t h, int conv_index, void **weights, float **bias, int dims[2])
 {
     VGG16 *v = dynamic_cast<VGG16 *>(static_cast<Task *>(h));
-    if (!v || conv_index < 0 || conv_index >= 13) return fail(TK_ERROR_INVALID_VALUE, "bad convolution index");
+    if (!v || conv_index < 0 || conv_index >= 16) return fail(TK_ERROR_INVALID_VALUE, "bad layer index");
     const VGG16::Act a = v->activation(conv_index);
     *weights = a.weights;
     *bias = a.bias;

@@ -189,7 +189,7 @@ struct VGG16::Impl {
     std::vector<void *> freeList;
     std::vector<float> hostInput;
     float *input = nullptr;
-    std::vector<VGG16::Act> convOut;
+    std::vector<VGG16::Act> convOut;   // the 13 convolutions, then the 3 fully connected layers
     float *logits = nullptr;
     long logitsStride = 0;
 };
@@ -290,6 +290,9 @@ VGG16::VGG16(int taskId, const VGG16Options &o) : Task(taskId, "vgg16"), opt(o),
     addKernel(new FcKernel(id++, "Dot_fc1", act, 1, act_bias, 1, feat, 4096, W1, X1, o1, pooled ? unpooled_W : 0, ld, C));
     addKernel(new FcKernel(id++, "Dot_fc2", o1, 1, b1, 1, 4096, 4096, W2, X2, o2));
     addKernel(new FcKernel(id++, "Dot_fc3", o2, 1, b2, 1, 4096, opt.classes, W3, X3, o3));
+    impl->convOut.push_back(Act{o1, 1, 1, 4096, 4096, W1, b1, 4096, pad128(feat)});
+    impl->convOut.push_back(Act{o2, 1, 1, 4096, 4096, W2, b2, 4096, 4096});
+    impl->convOut.push_back(Act{o3, 1, 1, opt.classes, pad128(opt.classes), W3, nullptr, pad128(opt.classes), 4096});
     impl->logits = o3;
     impl->logitsStride = 1;
 }

@@ -45,8 +45,9 @@ public:
     void initExecution() override;       // host -> device copy of the input image
     // device pointer / length of the logits (column 0 of the last GEMM's output, stride ld)
     const float *logits(long *stride) const;
-    // output buffer of convolution `idx` (for tests): device pointer, rows, channel stride.  It
-    // holds 1.1 * A * B^T; bias (returned here) and ReLU are applied by the layer that reads it
+    // output buffer of layer `idx` (0..12 the convolutions, 13..15 the fully connected layers; for
+    // tests): device pointer, rows, channel stride.  It holds 1.1 * A * B^T; bias (returned here,
+    // none for the last layer) and ReLU are applied by the layer that reads it
     struct Act { float *ptr; int H, W, C, ld; void *weights; float *bias; int Np, Kp; };
     Act activation(int conv_index) const;
     VGG16Options opt;

@@ -237,8 +237,7 @@ extern "C" __global__ void maxpool2x2_nhwc(const float *in, int H, int W, int ld
 extern "C" __global__ void pack_fc_input(const float *src, long src_stride, const float *bias, int relu,
                                          int n, _Float16 *x_row)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         float v = src[(long)i * src_stride];
         if (bias) v += bias[i];
         if (relu && v < 0.0f) v = 0.0f;
@@ -253,8 +252,7 @@ extern "C" __global__ void pack_fc_input(const float *src, long src_stride, cons
 extern "C" __global__ void pack_fc_input_pooled(const float *in, int W, int ld, int C, const float *bias,
                                                 int relu, int n, _Float16 *x_row)
 {
-    const int i = blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
         const int c = i % C;
         const int p = i / C;
         const int Wo = W / 2;

@@ -118,6 +118,28 @@ def test_config3_tzgemm_4096x4096x1024_and_lbm_120x120x150():
     assert 0.5 * (2.0 / sz) / 6 <= loss <= 1.5 * (2.0 / sz) / 6, loss
 
 
+def test_config3_ten_lbm_steps_with_grid_swap_track_the_oracle_step_by_step():
+    # both grids start as the same lattice (obstacle and accelerated cells marked in both, as the
+    # benchmark's loader leaves them); after each step source and destination change places
+    sx, sy, sz = 120, 120, 150
+    src = lbm_inputs(sx, sy, sz, seed=77, accel_p=0.01)
+    a, b = dev(src), dev(src)
+    ha, hb = src.copy(), src.copy()
+    k = ta.ori_lbm_create(a, b, sx, sy, sz)
+    g = ta.gptb_create(k, 0, 0, 0, sy * sz)
+    for step in range(10):
+        g.execute()                                              # the object follows the swap below
+        hb = oracle.lbm(ha, hb, sx, sy, sz)
+        k.swap_buffers()
+        a, b = b, a
+        ha, hb = hb, ha
+        torch.cuda.synchronize()
+        assert np.array_equal(host(a).view(np.uint32), ha.view(np.uint32)), step
+    assert np.isfinite(ha.reshape(20, -1)[:19]).all()
+    g.close()
+    k.close()
+
+
 def test_config4_tzgemm_2048_and_mriq_2048x262144():
     M = N = K = 2048
     A, B = gemm_inputs(M, N, K, seed=22)

@@ -794,6 +794,43 @@ def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
         assert np.array_equal(host(o).view(np.uint32), w.view(np.uint32))
 
 
+def _small_be_matches_oracle(name, outs):
+    """the outputs of _small_be(name) after one full pass, against the oracle on the same seeded inputs:
+    bit-exact for stencil, lbm and cp, the float tolerance for the two MRI kernels"""
+    if name == "stencil":
+        A0 = stencil_inputs(6, 20, 200, seed=31)
+        return np.array_equal(host(outs[0]).view(np.uint32), oracle.stencil(C0, C1, A0, A0).view(np.uint32))
+    if name == "lbm":
+        src = lbm_inputs(120, 6, 5, seed=32)
+        want = oracle.lbm(src, np.zeros_like(src), 120, 6, 5)
+        return np.array_equal(host(outs[0]).view(np.uint32), want.view(np.uint32))
+    zq = np.zeros(2048, np.float32)
+    if name == "mriq":
+        k, phiR, phiI, xyz = mriq_inputs(256, 2048, seed=33)
+        kv = np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32)
+        tr, ti = oracle.mriq(kv, xyz[0], xyz[1], xyz[2], zq, zq, f64=True)
+        return mriq_close(host(outs[0]), tr.astype(np.float64)) and mriq_close(host(outs[1]), ti.astype(np.float64))
+    if name == "mrif":
+        k, phi, d, xyz = mrif_inputs(256, 2048, seed=34)
+        tr, ti = oracle.mrif(mrif_table(k, phi, d), xyz[0], xyz[1], xyz[2], zq, zq, f64=True)
+        return mriq_close(host(outs[0]), tr.astype(np.float64)) and mriq_close(host(outs[1]), ti.astype(np.float64))
+    want = oracle.cp(oracle.cp_atoms_to_const(cp_atoms(), 0.0), np.zeros((32, 512), np.float32))
+    return np.array_equal(host(outs[0]).view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),
+                                          ("lbm", "stencil"), ("mriq", "stencil"), ("cp", "mrif"), ("lbm", "mrif"),
+                                          ("mrif", "mriq"), ("mrif", "stencil")])
+def test_best_effort_pairs_full_ranges_match_the_oracle(first, second):
+    ori1, n1, outs1 = _small_be(first)
+    ori2, n2, outs2 = _small_be(second)
+    g1, g2 = ta.gptb_create(ori1, 0, 0, 0, n1), ta.gptb_create(ori2, 0, 0, 0, n2)
+    ta.be_pair_create(g1, g2, 0, n1, 0, n2, launch_grid=48).execute()
+    assert _small_be_matches_oracle(first, outs1), first
+    assert _small_be_matches_oracle(second, outs2), second
+    assert ta.spin_fail_flag() == 0
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_mix_with_a_k_split_gemm_shape(variant):
     # 256 x 384 x 1024: 6 macro tiles, K >= 512 -> the GEMM role takes its K-split form,

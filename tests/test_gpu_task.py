@@ -76,6 +76,53 @@ def test_vgg16_layers_match_direct_convolution():
     task.close()
 
 
+def test_vgg16_whole_forward_pass_matches_a_float64_model_of_it():
+    # the whole network from the image to the logits in float64, never looking at the device's
+    # intermediate results: operands rounded to f16 where the layers round them, 13 convolutions with
+    # bias + ReLU, the five 2x2 max poolings, NHWC flattening, three fully connected layers
+    task = ta.LcTask("vgg16", 32, 64)
+    task.execute()
+    torch.cuda.synchronize()
+    f16 = lambda a: a.astype(np.float16).astype(np.float64)
+    scale = float(np.float32(1.1))
+    x = task.host_input().reshape(32, 64, 3).astype(np.float64)
+    pool_before = {2, 4, 7, 10}               # convolutions whose input went through a pooling
+    C = 3
+    worst = 0.0
+    for idx in range(13):
+        w, b = task.conv_params(idx)
+        if idx in pool_before:
+            H, W = x.shape[:2]
+            x = x.reshape(H // 2, 2, W // 2, 2, -1).max(axis=(1, 3))
+        ptr, (H, W, Cout, ld) = task.activation(idx)
+        assert x.shape == (H, W, C)
+        want = conv_reference(x, w, b, C, Cout)
+        raw = ta.device_to_host(ptr, (H, W, ld), np.float32)
+        got = np.maximum(raw[:, :, :Cout] + b[None, None, :Cout], np.float32(0))
+        tol = 1e-3 * np.abs(want).max()
+        worst = max(worst, np.abs(got - want).max() / np.abs(want).max())
+        assert np.abs(got - want).max() <= tol, (idx, np.abs(got - want).max(), tol)
+        x, C = want, Cout
+    H, W = x.shape[:2]
+    v = x.reshape(H // 2, 2, W // 2, 2, -1).max(axis=(1, 3)).reshape(-1)      # pool5, NHWC flattening
+    for idx in (13, 14, 15):
+        w, b = task.conv_params(idx)
+        ptr, (_, _, n_out, ld) = task.activation(idx)
+        assert w.shape[1] >= v.size
+        raw = scale * (w[:n_out, :v.size].astype(np.float64) @ f16(v))
+        got_raw = ta.device_to_host(ptr, (ld,), np.float32)[:n_out]
+        tol = 1e-3 * np.abs(raw).max()
+        assert np.abs(got_raw - raw).max() <= tol, (idx, np.abs(got_raw - raw).max(), tol)
+        worst = max(worst, np.abs(got_raw - raw).max() / np.abs(raw).max())
+        v = np.maximum(raw + b[:n_out], 0.0)
+    p, stride, n = task.logits()
+    logits = ta.device_to_host(p, (n, stride), np.float32)[:, 0]
+    assert n == raw.size and np.abs(logits - raw).max() <= 1e-3 * np.abs(raw).max()
+    assert int(np.argmax(logits)) == int(np.argmax(raw)) or np.sort(raw)[-1] - np.sort(raw)[-2] < 2e-3 * np.abs(raw).max()
+    assert np.abs(raw).max() > 0 and worst < 1e-3
+    task.close()
+
+
 @pytest.mark.parametrize("H,W,C,cs,pool", [(5, 7, 8, 8, 0), (8, 8, 64, 128, 0), (14, 14, 24, 32, 0), (3, 3, 16, 16, 0),
                                            (1, 1, 8, 8, 0), (2, 9, 40, 44, 0), (4, 6, 16, 128, 1), (7, 7, 64, 64, 1),
                                            (1, 2, 8, 12, 1)])
@@ -167,6 +214,15 @@ def test_pooled_classifier_input_equals_pooling_then_packing(H, W, C, ld):
     torch.cuda.synchronize()
     assert np.array_equal(got.cpu().numpy().view(np.uint16), want_bits)
     assert np.any(want_bits != 0)
+    # a grid smaller than the vector (the launcher caps it at a multiple of the CU count): same result
+    for key, args in (("pack_fc_input_pooled", [ptr(raw), i(W), i(ld), i(C), ptr(bias), i(1), i(n)]),
+                      ("pack_fc_input", [ptr(pooled), C_.c_long(1), C_.c_void_p(0), i(0), i(n)] if ld == C else None)):
+        if args is None:
+            continue
+        few = torch.full((n,), 777.0, dtype=torch.float16, device="cuda:0")
+        launch(key, 1, 64, args + [ptr(few)])
+        torch.cuda.synchronize()
+        assert np.array_equal(few.cpu().numpy().view(np.uint16), want_bits), key
 
 
 def test_task_manager_colocation_keeps_lc_results_and_reports():
@@ -207,6 +263,41 @@ def test_task_manager_colocation_keeps_lc_results_and_reports():
     assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
     tm.close()
     task.close()
+
+
+def test_mix_entry_points_on_the_global_operands_match_the_oracle():
+    # mixcublasSgemm / mixcudnnConvolutionForward (src/TaskManager.cu:309-400, 125-306) for a latency-critical
+    # kernel that brings no operands: the GEMM reads the library's seeded operand buffers
+    from gpu_util import C0, C1, gemm_tolerance_ok, stencil_inputs
+    A0 = stencil_inputs(6, 20, 200, seed=41)
+    for call, dims in ((lambda g, a, b: ta.mix_cublas_sgemm([200, 100, 300], g, a, b), (200, 100, 300)),
+                       (lambda g, a, b: ta.mix_cudnn_convolution_forward([1, 8, 20, 20, 32, 8, 3, 3, 1, 1, 1, 1, 1, 1],
+                                                                         g, a, b), (400, 32, 72))):
+        M, N, K, tiles = ta.tzgemm_grid_dim(*dims)
+        a0 = dev(A0)
+        out = a0.clone()
+        ori = ta.ori_stencil_create(C0, C1, a0, out)
+        blocks = ta.stencil_blocks(200, 20, 6)
+        g = ta.gptb_create(ori, 0, 0, 0, blocks)
+        call(g, 0, blocks)
+        torch.cuda.synchronize()
+        pa, pb, pc, _ = ta.global_gemm_buffers()
+        A = ta.device_to_host(pa, (M, K), np.float16)
+        B = ta.device_to_host(pb, (N, K), np.float16)
+        got = ta.device_to_host(pc, (M, N), np.float32)
+        assert np.abs(A.astype(np.float32)).max() > 0
+        ok, fro, dmax = gemm_tolerance_ok(got, oracle.tzgemm(A, B, f64=True), K)
+        assert ok and fro <= 1e-5, (dims, fro, dmax)
+        assert np.array_equal(host(out).view(np.uint32), oracle.stencil(C0, C1, A0, A0).view(np.uint32)), dims
+        # a partial range leaves the other positions of the sweep untouched; an empty one runs the GEMM alone
+        out.copy_(a0)
+        call(g, 1, 3)
+        want = oracle.stencil_gptb(C0, C1, A0, A0, start=1, end=3, gdz="runs")
+        assert np.array_equal(host(out).view(np.uint32), want.view(np.uint32)), dims
+        out.copy_(a0)
+        call(g, 2, 2)
+        assert np.array_equal(host(out), A0)
+    assert ta.spin_fail_flag() == 0
 
 
 def test_task_manager_colocates_mrif_and_pairs_it_with_lbm():

@@ -317,6 +317,57 @@ def test_mix_follows_ori_buffer_swap_but_not_gptb_range_edits(fake):
     assert [as_int(launches(fake)[-1]["args"][13]), as_int(launches(fake)[-1]["args"][15])] == [1, 2]
 
 
+def test_mix_entry_points_for_kernels_that_bring_no_operands(fake):
+    # mixcublasSgemm / mixcudnnConvolutionForward (src/TaskManager.cu:309-400, 125-306): the GEMM on the
+    # global operand buffers, fused with a block range of a best-effort kernel; the convolution lowers first
+    fake.tk_fake_reset()
+    fake.tk_fake_set_cu_count(256)
+    a0 = np.zeros((6, 10, 70), np.float32)
+    st_ori = fake.tacker_ori_stencil_create(0.5, 0.25, a0.ctypes.data, a0.ctypes.data, 70, 10, 6)
+    st = fake.tacker_gptb_create(st_ori, 0, 0, 0, 6)
+    mnk = (C.c_int * 3)(200, 100, 300)
+    assert fake.tacker_mix_cublas_sgemm(mnk, st, 2, 5, None) == 0, fake.tacker_last_error()
+    (l,) = launches(fake)
+    assert l["key"].startswith("tzgemm_stencil") and len(l["args"]) == (7 + 6 + 3) + (6 + 6 + 3)
+    assert [as_int(l["args"][i]) for i in (13, 15)] == [2, 5]
+    dims = (C.c_int * 4)()
+    fake.tacker_tzgemm_grid_dim(200, 100, 300, dims)
+    assert [as_int(x) for x in l["args"][19:22]] == list(dims[:3])           # M, N, K rounded up to whole tiles
+    assert [as_int(l["args"][i]) for i in (28, 30)] == [0, dims[3]]
+    ga, gb, gc = C.c_void_p(), C.c_void_p(), C.c_void_p()
+    sizes = (C.c_longlong * 3)()
+    fake.tacker_global_gemm_buffers(C.byref(ga), C.byref(gb), C.byref(gc), sizes)
+    assert [as_ptr(x) for x in l["args"][16:19]] == [ga.value, gb.value, gc.value]
+    assert sizes[0] >= dims[0] * dims[2] * 2 and sizes[2] >= dims[0] * dims[1] * 4
+    # an empty range: the GEMM alone
+    fake.tk_fake_reset()
+    assert fake.tacker_mix_cublas_sgemm(mnk, st, 3, 3, None) == 0
+    assert [x["key"] for x in launches(fake)] == ["gptb_tzgemm"]
+    # convolution: im2col into the staging buffer, then the fused launch of {n*ho*wo, k, r*s*c}
+    fake.tk_fake_reset()
+    conv = (C.c_int * 14)(1, 8, 20, 20, 32, 8, 3, 3, 1, 1, 1, 1, 1, 1)
+    assert fake.tacker_mix_cudnn_convolution_forward(conv, st, 0, 6, None) == 0, fake.tacker_last_error()
+    first, second = launches(fake)
+    assert first["key"] == "im2col" and as_int(first["args"][0]) == 1 * 8 * 20 * 20
+    assert second["key"].startswith("tzgemm_stencil")
+    fake.tacker_tzgemm_grid_dim(400, 32, 72, dims)
+    assert [as_int(x) for x in second["args"][19:22]] == list(dims[:3])
+    # refusals: not a GPTB object, the GEMM as its own partner, bad ranges and shapes
+    assert fake.tacker_mix_cublas_sgemm(mnk, st_ori, 0, 6, None) == 1
+    A = np.zeros((128, 128), np.float16)
+    Cm = np.zeros((128, 128), np.float32)
+    tz = fake.tacker_gptb_create(fake.tacker_ori_tzgemm_create(A.ctypes.data, A.ctypes.data, Cm.ctypes.data,
+                                                               128, 128, 128), 0, 0, 0, 4)
+    assert fake.tacker_mix_cublas_sgemm(mnk, tz, 0, 4, None) == 1
+    assert fake.tacker_mix_cublas_sgemm(mnk, st, 4, 2, None) == 1
+    assert fake.tacker_mix_cublas_sgemm((C.c_int * 3)(0, 4, 4), st, 0, 6, None) == 1
+    bad = (C.c_int * 14)(1, 8, 2, 2, 32, 8, 7, 7, 0, 0, 1, 1, 1, 1)              # a 7x7 filter on a 2x2 image
+    assert fake.tacker_mix_cudnn_convolution_forward(bad, st, 0, 6, None) == 1
+    fake.tk_fake_reset()
+    fake.tk_fake_fail_next_launches(1)                                           # a failing launch reaches the caller
+    assert fake.tacker_mix_cublas_sgemm(mnk, st, 0, 6, None) != 0
+
+
 def test_best_effort_pair_parameter_vector_and_geometry(fake):
     # [first's params + 6 dims][start1, step, end1][second's params + 6 dims][start2, step, end2]
     fake.tk_fake_reset()
