@@ -372,6 +372,21 @@ TK_API int tacker_mix_cublas_sgemm(const int mnk[3], tacker_kernel_t be_gptb, in
  * launch of the GEMM {n*ho*wo, k, r*s*c} (get_mnk_from_cudnn_args, src/TaskManager.cu:92-123). */
 TK_API int tacker_mix_cudnn_convolution_forward(const int cudnn_args[14], tacker_kernel_t be_gptb,
                                                 int cd_start_blk, int cd_end_blk, tkStream_t stream);
+/* ModuleCenter::registerModule(moduleName, cubinPath) (src/ModuleCenter.cu:8-19): load a gfx950 code
+ * object (what `hipcc --genco` writes; the build leaves the library's own kernels as
+ * lib/tacker_kernels.hsaco and lib/tacker_kernels_large.hsaco) under a name.  The object's copies of
+ * the device symbols the host fills by name (mri-q / mri-fhd / cp constant tables, the GEMM's
+ * workspace table, the failure word) are filled from the library's at load and written along with
+ * them from then on, so kernels launched from it see what tacker_*_set_* and the runtime publish. */
+TK_API int tacker_register_module(const char *module_name, const char *code_object_path);
+/* ModuleCenter::getFunction(moduleName, functionName) != nullptr (src/ModuleCenter.cu:21-43) */
+TK_API int tacker_module_has_function(const char *module_name, const char *function_name);
+/* lmode DRIVER_LAUNCH (src/Kernel.h:7-10,39) for a GPTB or fused kernel object: take its device
+ * function from a registered code object by the function's name there (the loadKernel of
+ * src/ori_kernel/cp_kernel.cu:423-434; e.g. "general_ptb_stencil") and launch through
+ * tkModuleLaunchKernel from then on.  TK_ERROR_NOT_FOUND leaves the object as it was. */
+TK_API int tacker_kernel_use_module(tacker_kernel_t kernel, const char *module_name,
+                                    const char *function_name);
 /* Kernel::execute(stream) */
 TK_API int tacker_kernel_execute(tacker_kernel_t kernel, tkStream_t stream);
 /* exchange the input and output grid of a stencil / lbm ori object (the

@@ -15,6 +15,9 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libtacker_amd.so")
 FAKE_LIB_PATH = os.path.join(_HERE, "lib", "libtacker_host_fake.so")
+# the device code alone, as code objects for tacker_register_module
+CODE_OBJECT_PATH = os.path.join(_HERE, "lib", "tacker_kernels.hsaco")
+CODE_OBJECT_LARGE_PATH = os.path.join(_HERE, "lib", "tacker_kernels_large.hsaco")
 KINFO_PATH = os.path.join(_HERE, "config", "kinfo-gfx950.json")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "tacker_amd.h")
 
@@ -92,6 +95,9 @@ def _declare(lib):
     lib.tacker_kernel_swap_buffers.argtypes = [vp]
     lib.tacker_kernel_info.argtypes = [vp, C.POINTER(i)]
     lib.tacker_kernel_param.argtypes = [vp, i, vp, i]
+    lib.tacker_register_module.argtypes = [C.c_char_p, C.c_char_p]
+    lib.tacker_module_has_function.argtypes = [C.c_char_p, C.c_char_p]
+    lib.tacker_kernel_use_module.argtypes = [vp, C.c_char_p, C.c_char_p]
     lib.tacker_mix_cublas_sgemm.argtypes = [C.POINTER(i), vp, i, i, vp]
     lib.tacker_mix_cudnn_convolution_forward.argtypes = [C.POINTER(i), vp, i, i, vp]
     lib.tacker_kernel_destroy.argtypes = [vp]
@@ -485,6 +491,10 @@ class KernelHandle:
         check(lib().tacker_kernel_param(self.handle, index, C.byref(out), C.sizeof(ctype)), "tacker_kernel_param")
         return out.value or 0
 
+    def use_module(self, module, function):
+        """lmode DRIVER_LAUNCH: launch ``function`` of the registered code object ``module`` from now on."""
+        check(lib().tacker_kernel_use_module(self.handle, module.encode(), function.encode()), "tacker_kernel_use_module")
+
     def set_range(self, *r):
         if len(r) == 2:
             check(lib().tacker_gptb_set_range(self.handle, *r), "tacker_gptb_set_range")
@@ -501,6 +511,15 @@ class KernelHandle:
             self.close()
         except Exception:
             pass
+
+
+def register_module(name, path):
+    """ModuleCenter::registerModule of the reference (src/ModuleCenter.cu:8-19) for a gfx950 code object."""
+    check(lib().tacker_register_module(name.encode(), str(path).encode()), "tacker_register_module")
+
+
+def module_has_function(module, function):
+    return bool(lib().tacker_module_has_function(module.encode(), function.encode()))
 
 
 def create_kernel(name):

@@ -90,8 +90,7 @@ protected:
         kernelParams.push_back(&gptbParams.ptb_iter_block_step);
         kernelParams.push_back(&gptbParams.ptb_end_block_pos);
         kernelParams.push_back(&thread_base);
-        const int launch_status = tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
-                                                 (void **)kernelParams.data(), 0, stream);
+        const int launch_status = launchBy((void **)kernelParams.data(), stream);
         kernelParams.resize(base);   // also on failure: the vector must not keep &thread_base
         TK_SAFE_CALL(launch_status);
     }

@@ -40,6 +40,12 @@ public:
     int getKernelId() { return Id; }
     std::string &getKernelName() { return kernelName; }
 
+    // Switch this object to lmode DRIVER_LAUNCH: `function` is taken from the code object registered
+    // with the ModuleCenter under `module` (the loadKernel of src/ori_kernel/cp_kernel.cu:423-434)
+    // and launches go through tkModuleLaunchKernel (cuLaunchKernel) instead of the registry's
+    // function.  false, and the object unchanged, when the module or the function is not there.
+    bool useModule(const std::string &module, const std::string &function_name);
+
     int Id = 0;
     std::string kernelName;
     std::string moduleName;
@@ -57,6 +63,13 @@ public:
 
 protected:
     virtual void executeImpl(cudaStream_t stream) = 0;
+    // the launch of wrappers whose whole argument list is `params`: by the object's launch mode
+    int launchBy(void **params, cudaStream_t stream)
+    {
+        if (launchMode == DRIVER_LAUNCH)
+            return tkModuleLaunchKernel(function, launchGridDim.raw(), launchBlockDim.raw(), params, 0, stream);
+        return tkLaunchKernel(kernelFunc, launchGridDim.raw(), launchBlockDim.raw(), params, 0, stream);
+    }
 };
 
 // The uniform tail of every GPTB kernel's parameter list (thread_base follows

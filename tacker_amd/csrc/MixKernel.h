@@ -72,8 +72,7 @@ public:
 protected:
     void executeImpl(cudaStream_t stream) override
     {
-        TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
-                                    (void **)kernelParams.data(), 0, stream));
+        TK_SAFE_CALL(launchBy((void **)kernelParams.data(), stream));
     }
 
 private:

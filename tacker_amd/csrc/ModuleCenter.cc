@@ -2,6 +2,20 @@
 
 #include <iostream>
 
+#include "Kernel.h"
+
+extern ModuleCenter moduleCenter;
+
+bool Kernel::useModule(const std::string &module, const std::string &function_name)
+{
+    CUfunction f = moduleCenter.getFunction(module, function_name);
+    if (!f) return false;
+    function = f;
+    moduleName = module;
+    launchMode = DRIVER_LAUNCH;
+    return true;
+}
+
 ModuleCenter::~ModuleCenter()
 {
     for (auto &m : modules)

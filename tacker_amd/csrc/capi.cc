@@ -811,6 +811,32 @@ int tacker_mix_cudnn_convolution_forward(const int cudnn_args[14], tacker_kernel
     });
 }
 
+int tacker_register_module(const char *module_name, const char *code_object_path)
+{
+    REQUIRE_INIT();
+    if (!module_name || !*module_name || !code_object_path) return fail(TK_ERROR_INVALID_VALUE, "null module name or path");
+    if (!moduleCenter.registerModule(module_name, code_object_path))
+        return fail(TK_ERROR_DEVICE, std::string("cannot load code object ") + code_object_path);
+    return TK_SUCCESS;
+}
+
+int tacker_module_has_function(const char *module_name, const char *function_name)
+{
+    if (!module_name || !function_name) return 0;
+    return moduleCenter.getFunction(module_name, function_name) != nullptr;
+}
+
+int tacker_kernel_use_module(tacker_kernel_t h, const char *module_name, const char *function_name)
+{
+    Kernel *k = static_cast<Kernel *>(h);
+    if (!k || !module_name || !function_name) return fail(TK_ERROR_INVALID_VALUE, "null kernel, module or function name");
+    if (!dynamic_cast<GPTBKernel *>(k) && !dynamic_cast<MixKernel *>(k))
+        return fail(TK_ERROR_UNSUPPORTED, "only GPTB and fused kernel objects launch from a code object");
+    if (!k->useModule(module_name, function_name))
+        return fail(TK_ERROR_NOT_FOUND, std::string("no function ") + function_name + " in module " + module_name);
+    return TK_SUCCESS;
+}
+
 int tacker_kernel_execute(tacker_kernel_t h, tkStream_t stream)
 {
     Kernel *k = static_cast<Kernel *>(h);

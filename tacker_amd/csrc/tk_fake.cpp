@@ -21,6 +21,7 @@ struct Launch {
     tkDim3 grid, block;
     std::vector<std::vector<unsigned char>> args;
     void *stream;
+    bool by_driver = false;   // launched through tkModuleLaunchKernel
 };
 std::vector<FakeKernel *> &kernels()
 {
@@ -151,15 +152,25 @@ int tkModuleLoad(tkModule_t *m, const char *path)
     return TK_SUCCESS;
 }
 int tkModuleUnload(tkModule_t m) { free(m); return TK_SUCCESS; }
+// a fake code object holds every kernel of the registry, under the name its device function has in
+// the real one: general_ptb_<kernel> (g_general_ptb_<kernel> for mriq and cp) for gptb_<kernel>
 int tkModuleGetFunction(tkFunction_t *f, tkModule_t, const char *name)
 {
+    std::string key = name;
+    for (const char *prefix : {"g_general_ptb_", "general_ptb_"})
+        if (key.rfind(prefix, 0) == 0) {
+            key = "gptb_" + key.substr(strlen(prefix));
+            break;
+        }
     for (auto *k : kernels())
-        if (k->key == name) { *f = k; return TK_SUCCESS; }
+        if (k->key == key) { *f = k; return TK_SUCCESS; }
     return TK_ERROR_NOT_FOUND;
 }
 int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void **args, size_t shmem, tkStream_t s)
 {
-    return tkLaunchKernel(f, grid, block, args, shmem, s);
+    const int rc = tkLaunchKernel(f, grid, block, args, shmem, s);
+    if (rc == TK_SUCCESS) g_launches.back().by_driver = true;
+    return rc;
 }
 
 int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
@@ -221,6 +232,7 @@ TK_API void tk_fake_set_event_ms(float ms) { g_event_ms = ms; }
 TK_API void tk_fake_push_event_ms(const float *ms, int n) { g_event_queue.insert(g_event_queue.end(), ms, ms + n); }
 TK_API int tk_fake_event_queue_len(void) { return (int)g_event_queue.size(); }
 TK_API const char *tk_fake_launch_key(int i) { return g_launches[i].key.c_str(); }
+TK_API int tk_fake_launch_by_driver(int i) { return g_launches[i].by_driver ? 1 : 0; }
 TK_API int tk_fake_launch_nargs(int i) { return (int)g_launches[i].args.size(); }
 TK_API void tk_fake_launch_dims(int i, unsigned out[6])
 {

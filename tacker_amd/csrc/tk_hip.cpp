@@ -5,7 +5,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <mutex>
 #include <string>
+#include <vector>
 
 #include "../../include/tacker_amd.h"
 
@@ -14,6 +16,9 @@ extern "C" int tk_scratch_setup(int device);
 
 namespace {
 thread_local std::string g_last_hip_error;
+std::mutex g_modules_mutex;
+std::vector<hipModule_t> g_modules;   // code objects loaded through tkModuleLoad
+const char *const kMirroredSymbols[] = {"ck", "c_mrif", "atominfo", "tz_ws_table", "tk_spin_fail"};
 
 int fold(hipError_t e, const char *what)
 {
@@ -109,7 +114,21 @@ int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t o
         g_last_hip_error = "tkMemcpyToSymbol: range exceeds the symbol";
         return TK_ERROR_INVALID_VALUE;
     }
-    return FOLD(hipMemcpyToSymbol(sym, src, bytes, offset, hipMemcpyHostToDevice));
+    const int wrote = FOLD(hipMemcpyToSymbol(sym, src, bytes, offset, hipMemcpyHostToDevice));
+    if (wrote) return wrote;
+    std::lock_guard<std::mutex> lock(g_modules_mutex);
+    for (hipModule_t mod : g_modules) {   // the loaded code objects' copies follow
+        hipDeviceptr_t dst = nullptr;
+        size_t have = 0;
+        if (hipModuleGetGlobal(&dst, &have, mod, symbol) != hipSuccess) {
+            (void)hipGetLastError();
+            continue;
+        }
+        if (offset + bytes > have) continue;
+        const int e = FOLD(hipMemcpy((char *)dst + offset, src, bytes, hipMemcpyHostToDevice));
+        if (e) return e;
+    }
+    return TK_SUCCESS;
 }
 
 int tkMemcpyFromSymbol(void *dst, const char *symbol, size_t bytes, size_t offset)
@@ -122,7 +141,23 @@ int tkMemcpyFromSymbol(void *dst, const char *symbol, size_t bytes, size_t offse
         g_last_hip_error = "tkMemcpyFromSymbol: range exceeds the symbol";
         return TK_ERROR_INVALID_VALUE;
     }
-    return FOLD(hipMemcpyFromSymbol(dst, sym, bytes, offset, hipMemcpyDeviceToHost));
+    const int got = FOLD(hipMemcpyFromSymbol(dst, sym, bytes, offset, hipMemcpyDeviceToHost));
+    if (got || strcmp(symbol, "tk_spin_fail") != 0 || bytes != sizeof(unsigned) || offset != 0) return got;
+    // the failure word is a set of bits any kernel may raise: those of loaded code objects count too
+    std::lock_guard<std::mutex> lock(g_modules_mutex);
+    for (hipModule_t mod : g_modules) {
+        hipDeviceptr_t src = nullptr;
+        size_t have = 0;
+        unsigned bits = 0;
+        if (hipModuleGetGlobal(&src, &have, mod, symbol) != hipSuccess) {
+            (void)hipGetLastError();
+            continue;
+        }
+        const int e = FOLD(hipMemcpy(&bits, src, sizeof(bits), hipMemcpyDeviceToHost));
+        if (e) return e;
+        *(unsigned *)dst |= bits;
+    }
+    return TK_SUCCESS;
 }
 
 int tkStreamCreate(tkStream_t *s) { return FOLD(hipStreamCreate((hipStream_t *)s)); }
@@ -149,8 +184,49 @@ int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, siz
                                 args, shmem, (hipStream_t)stream));
 }
 
-int tkModuleLoad(tkModule_t *m, const char *path) { return FOLD(hipModuleLoad((hipModule_t *)m, path)); }
-int tkModuleUnload(tkModule_t m) { return FOLD(hipModuleUnload((hipModule_t)m)); }
+// A code object carries copies of its own of the device symbols the host fills by name (constant
+// tables, the workspace table, the failure word).  They follow the library's: filled from the
+// library's copies when the object is loaded, and written along with them from then on.
+int tkModuleLoad(tkModule_t *m, const char *path)
+{
+    hipModule_t mod = nullptr;
+    const int rc = FOLD(hipModuleLoad(&mod, path));
+    if (rc) return rc;
+    for (const char *name : kMirroredSymbols) {
+        hipDeviceptr_t dst = nullptr;
+        size_t bytes = 0;
+        if (hipModuleGetGlobal(&dst, &bytes, mod, name) != hipSuccess) {
+            (void)hipGetLastError();   // this object does not use the symbol
+            continue;
+        }
+        const void *sym = nullptr;
+        void *src = nullptr;
+        size_t cap = 0;
+        int e = tk_device_symbol(name, &sym, &cap);
+        if (!e) e = FOLD(hipGetSymbolAddress(&src, sym));
+        if (!e) e = FOLD(hipMemcpy(dst, src, bytes < cap ? bytes : cap, hipMemcpyDeviceToDevice));
+        if (e) {
+            (void)hipModuleUnload(mod);
+            return e;
+        }
+    }
+    std::lock_guard<std::mutex> lock(g_modules_mutex);
+    g_modules.push_back(mod);
+    *m = mod;
+    return TK_SUCCESS;
+}
+int tkModuleUnload(tkModule_t m)
+{
+    {
+        std::lock_guard<std::mutex> lock(g_modules_mutex);
+        for (size_t i = 0; i < g_modules.size(); ++i)
+            if (g_modules[i] == (hipModule_t)m) {
+                g_modules.erase(g_modules.begin() + (long)i);
+                break;
+            }
+    }
+    return FOLD(hipModuleUnload((hipModule_t)m));
+}
 int tkModuleGetFunction(tkFunction_t *f, tkModule_t m, const char *name)
 {
     return FOLD(hipModuleGetFunction((hipFunction_t *)f, (hipModule_t)m, name));

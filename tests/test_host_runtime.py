@@ -39,7 +39,7 @@ def launches(l):
             n = l.tk_fake_launch_arg(i, a, buf, 8)
             args.append(buf.raw[:n])
         out.append({"key": l.tk_fake_launch_key(i).decode(), "grid": tuple(dims[:3]), "block": tuple(dims[3:]),
-                    "args": args})
+                    "args": args, "by_driver": bool(l.tk_fake_launch_by_driver(i))})
     return out
 
 
@@ -366,6 +366,47 @@ def test_mix_entry_points_for_kernels_that_bring_no_operands(fake):
     fake.tk_fake_reset()
     fake.tk_fake_fail_next_launches(1)                                           # a failing launch reaches the caller
     assert fake.tacker_mix_cublas_sgemm(mnk, st, 0, 6, None) != 0
+
+
+def test_module_center_and_driver_launch_mode(fake, tmp_path):
+    # ModuleCenter::registerModule / getFunction (src/ModuleCenter.cu:8-43) and lmode DRIVER_LAUNCH
+    fake.tk_fake_reset()
+    assert fake.tacker_register_module(b"nowhere", str(tmp_path / "missing.hsaco").encode()) == 4
+    assert b"missing.hsaco" in fake.tacker_last_error()
+    assert fake.tacker_module_has_function(b"nowhere", b"general_ptb_stencil") == 0      # a module that never loaded
+    co = tmp_path / "kernels.hsaco"
+    co.write_bytes(b"stand-in for a code object")
+    assert fake.tacker_register_module(b"kernels", str(co).encode()) == 0, fake.tacker_last_error()
+    assert fake.tacker_register_module(b"kernels", str(co).encode()) == 0                # registering again is fine
+    assert fake.tacker_module_has_function(b"kernels", b"general_ptb_stencil") == 1
+    assert fake.tacker_module_has_function(b"kernels", b"no_such_function") == 0
+    a0 = np.zeros((6, 10, 70), np.float32)
+    st_ori = fake.tacker_ori_stencil_create(0.5, 0.25, a0.ctypes.data, a0.ctypes.data, 70, 10, 6)
+    st = fake.tacker_gptb_create(st_ori, 0, 0, 0, 6)
+    assert fake.tacker_kernel_execute(st, None) == 0
+    # refusals leave the object launching through the registry
+    assert fake.tacker_kernel_use_module(st, b"kernels", b"no_such_function") == 2
+    assert b"no_such_function" in fake.tacker_last_error()
+    assert fake.tacker_kernel_use_module(st, b"other_module", b"general_ptb_stencil") == 2
+    assert fake.tacker_kernel_use_module(st_ori, b"kernels", b"general_ptb_stencil") == 3
+    assert fake.tacker_kernel_execute(st, None) == 0
+    assert fake.tacker_kernel_use_module(st, b"kernels", b"general_ptb_stencil") == 0, fake.tacker_last_error()
+    assert fake.tacker_kernel_execute(st, None) == 0
+    first, second, third = launches(fake)
+    assert [l["by_driver"] for l in (first, second, third)] == [False, False, True]
+    for l in (second, third):                                        # same function, geometry and argument list
+        assert (l["key"], l["grid"], l["block"], l["args"]) == (first["key"], first["grid"], first["block"], first["args"])
+    # a fused object the same way, and a failing driver launch reaches the caller
+    A = np.zeros((128, 128), np.float16)
+    Cm = np.zeros((128, 128), np.float32)
+    tz = fake.tacker_gptb_create(fake.tacker_ori_tzgemm_create(A.ctypes.data, A.ctypes.data, Cm.ctypes.data,
+                                                               128, 128, 128), 0, 0, 0, 4)
+    mix = fake.tacker_mix_create(st, tz, 0, 6, 0, 4, None, 0, 0)
+    assert fake.tacker_kernel_use_module(mix, b"kernels", b"tzgemm_stencil@wg_1_1") == 0
+    assert fake.tacker_kernel_execute(mix, None) == 0
+    assert launches(fake)[-1]["by_driver"] and launches(fake)[-1]["key"] == "tzgemm_stencil@wg_1_1"
+    fake.tk_fake_fail_next_launches(1)
+    assert fake.tacker_kernel_execute(mix, None) != 0
 
 
 def test_best_effort_pair_parameter_vector_and_geometry(fake):
