@@ -115,6 +115,7 @@ def _declare(lib):
     lib.tacker_task_activation.argtypes = [vp, i, C.POINTER(vp), C.POINTER(i)]
     lib.tacker_task_conv_params.argtypes = [vp, i, C.POINTER(vp), C.POINTER(vp), C.POINTER(i)]
     lib.tkMemcpy.argtypes = [vp, vp, C.c_size_t, i]
+    lib.tkMemset.argtypes = [vp, i, C.c_size_t]
     lib.tacker_task_logits.argtypes = [vp, C.POINTER(vp), C.POINTER(C.c_long), C.POINTER(i)]
     lib.tacker_task_input.argtypes = [vp, C.POINTER(vp), C.POINTER(i)]
     lib.tacker_task_manager_create.restype = vp

@@ -16,31 +16,50 @@
 // tiles x 4), which only a kernel that has the CU to itself can pay: one wave per SIMD owns
 // all 512 registers, accumulators in the AGPR half.  Fused kernels keep the 128 x 128 form.
 //
-// K loop.  One LDS stage holds 32 k of the tile: rows of 64 bytes, A rows then B rows,
-// (32*FM + 32*FN) * 64 bytes = 32 KiB for 256 x 256; STAGES = 4 of them form a ring filled by
-// LDS-direct loads (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l, so one load
-// fills 16 rows).  In iteration c a wave multiplies the fragments of chunk c, which it already
-// holds in registers, and meanwhile (i) waits until its own loads of chunk c+1 have landed
-// (vmcnt) and meets the other waves at the barrier -- after which chunk c+1 is whole and nobody
-// reads chunk c's stage any more -- (ii) reads the fragments of chunk c+1 and (iii) starts
-// the loads of chunk c+STAGES into the stage chunk c left.  So three chunks are in flight
-// while one is multiplied, and the barrier sits behind the first MFMAs of an iteration.
-// The LDS reads follow every third MFMA behind the barrier (the LDS returns 1 KiB to a SIMD
-// in about 32 cycles, and the four waves read in step), the loads are spread evenly over the
-// iteration (the vector-memory unit takes about 25 cycles per load), and every MFMA is
-// fenced with sched_barrier so that the issue order is the source order.
+// K loop.  The tile's operands travel in pairs of 32-k chunks: one buffer of the LDS ring holds
+// 64 k of the tile as rows of 128 bytes, A rows then B rows, (32*FM + 32*FN) * 128 bytes = 64 KiB
+// for 256 x 256, and the ring is two buffers.  They are filled by LDS-direct loads
+// (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l, so one load fills 8 rows),
+// each of which takes whole 128-byte lines from 8 matrix rows: the same loads taking 64 bytes
+// from 16 rows each move 55 GB/s into a CU, these 86 (microbench/feed_rate.hip).
+// An iteration multiplies one chunk, whose fragments the wave already holds in registers, and
+// meanwhile reads the fragments of the next chunk.  In the first iteration of a pair those come
+// from the same buffer, which was published an iteration ago: no wait, no barrier.  In the second
+// the wave (i) waits until its own loads of the next pair have landed (vmcnt) and meets the other
+// waves at the barrier -- after which the next pair is whole and nobody reads this pair's buffer
+// any more -- (ii) reads the first fragments of the next pair and (iii) starts the loads of the
+// pair after that into the buffer this pair leaves.  So a pair is fetched while a pair is
+// multiplied, there is one barrier per 128 MFMAs of a wave, and it sits behind the first MFMAs of
+// its iteration.  The LDS reads follow every third MFMA (the LDS returns 1 KiB to a SIMD in
+// about 32 cycles, and the four waves read in step), the loads every third MFMA behind the
+// barrier, and every MFMA is fenced with sched_barrier so that the issue order is the source
+// order.
 //
 // The barrier is the hardware one: a counter in LDS with a split arrive / wait (what the
 // wave-split fused kernels use) was measured here too and lost 15 % -- its atomics and polls
-// queue behind 96 KiB of ring traffic per iteration.
+// queue behind the ring traffic.
 //
-// LDS layout.  Slot (row, s) of a stage holds the row's 16-byte k segment s ^ ((row >> 2) & 3).
-// The swizzle is applied on the global side of the LDS-direct load (a lane fetches the segment
-// that belongs in the slot it will write) and undone by the fragment read.  The hardware
-// counts 4 conflict cycles per fragment read for it (and for every other key tried); they hide
-// behind the 32 cycles a SIMD needs to take a read's data.
+// LDS layout.  Slot (row, s) of a buffer holds the row's 16-byte k segment s ^ ((row >> 1) & 7):
+// the 16 rows a fragment read touches with one k segment then cover all 64 banks once, and the
+// hardware counts no bank conflict.  The swizzle is applied on the global side of the
+// LDS-direct load (a lane fetches the segment that belongs in the slot it will write) and
+// undone by the fragment read.
 #pragma once
 #include "tzgemm_role.h"
+
+// Measurement builds only (microbench/tzgemm_large_probe.hip): each macro takes one ingredient out
+// of the steady K loop -- the results are wrong, the time says what the ingredient costs.
+#ifdef TZL_KNOCK_OUT_LOADS
+#define TZL_LOOP_LOAD(...)
+#else
+#define TZL_LOOP_LOAD(...) tz_load_to_lds(__VA_ARGS__)
+#endif
+#ifdef TZL_KNOCK_OUT_BARRIER
+#define TZL_LOOP_BARRIER()
+#else
+#define TZL_LOOP_BARRIER() __builtin_amdgcn_s_barrier()
+#endif
+#define TZL_LOOP_READ(dst_, src_) dst_ = src_
 
 namespace tk {
 
@@ -60,7 +79,7 @@ __device__ __forceinline__ void tz_large_tile_of(int t, int tile_rows, int tile_
 }
 
 // The role owns every wave of its workgroup (it synchronises with s_barrier).
-template <int FM, int FN, int STAGES, bool STREAM_C>
+template <int FM, int FN, bool STREAM_C>
 __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
                                                   float *__restrict__ C, int M, int N, int K, int role_block,
                                                   int role_blocks, int tile_start, int tile_end, int tid,
@@ -68,22 +87,22 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
 {
     typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int TM = 32 * FM, TN = 32 * FN;      // macro tile
-    constexpr int BK = 32;
-    constexpr int ROWB = BK * 2;                   // 64-byte tile rows
+    constexpr int BK = 32;                         // k of one MFMA step (a chunk)
+    constexpr int ROWB = 4 * BK;                   // 128-byte tile rows: a pair of chunks
     constexpr int A_BYTES = TM * ROWB;
-    constexpr int STAGE_BYTES = (TM + TN) * ROWB;
-    constexpr int LA = TM / 16 / 4;                // LDS-direct loads per wave and chunk: A ...
-    constexpr int LB = TN / 16 / 4;                // ... and B (one load = 16 rows)
+    constexpr int PAIR_BYTES = (TM + TN) * ROWB;   // one buffer of the ring: 64 KiB for 256 x 256
+    constexpr int LA = TM / 8 / 4;                 // LDS-direct loads per wave and pair: A ...
+    constexpr int LB = TN / 8 / 4;                 // ... and B (one load = 8 rows of 128 bytes)
     constexpr int L = LA + LB;
     constexpr int FIRST = 8;                       // MFMAs of an iteration in front of the barrier
-    constexpr int READ_GAP = 3;                    // one LDS read per READ_GAP MFMAs behind it
+    constexpr int READ_GAP = 3;                    // one LDS read per READ_GAP MFMAs
     constexpr int LOAD_GAP = (FM * FN - FIRST) / L;
     static_assert(FM % 4 == 0 && FN % 4 == 0, "a wave tile is whole reference tiles");
-    static_assert(LA <= 4 && LB <= 4, "four row blocks of 16 per wave and operand at most");
-    static_assert(L * (STAGES - 2) < 64, "vmcnt is a 6-bit counter");
+    static_assert(LA <= 8 && LB <= 8, "eight row blocks of 8 per wave and operand at most");
+    static_assert(L < 64, "vmcnt is a 6-bit counter");
     static_assert((FM + FN) * READ_GAP <= FM * FN - FIRST && LOAD_GAP >= 1,
                   "an iteration slots its LDS reads and loads between the MFMAs behind the barrier");
-    static_assert(STAGES == 4, "K is a multiple of 128 = 4 chunks; the tail of the K loop is written for 4 stages");
+    static_assert(2 * PAIR_BYTES <= TZ_LDS_BYTES, "the ring is two buffers");
 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -93,23 +112,26 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
     const int tile_rows = M / TM;
     const int tile_cols = N / TN;
     const int n_tiles = tile_rows * tile_cols;
-    const int kchunks = K / BK;                    // a multiple of 4
+    const int npairs = K / (2 * BK);               // K is a multiple of 128: an even number of pairs
 
-    // LDS-direct load map: load j of an operand fills rows 16 (4 j + wave) .. + 15 of its stage
-    // area; lane l lands in row + l / 4, slot l % 4 and therefore fetches k segment
-    // (l % 4) ^ ((row >> 2) & 3) = (l & 3) ^ ((l >> 4) & 3).  Per load a 32-bit lane offset below a
-    // wave-uniform pointer to the chunk: a load is "scalar base + vector offset" and costs no
-    // address arithmetic of its own.
-    const unsigned src_lane = (unsigned)((lane >> 2) * K + (((lane & 3) ^ ((lane >> 4) & 3)) * 8)) * 2u;
-    unsigned src_blk[4];
+    // LDS-direct load map: load j of an operand fills rows 8 (4 j + wave) .. + 7 of its area of the
+    // buffer; lane l lands in row + l / 8, slot l % 8 and therefore fetches the 16-byte k segment
+    // (l % 8) ^ ((row >> 1) & 7), and (row >> 1) & 7 = l / 16 + 4 (wave % 2) whatever j is.  Per load a
+    // 32-bit lane offset below a wave-uniform pointer to the pair of chunks: a load is "scalar base
+    // + vector offset" and costs no address arithmetic of its own.
+    const unsigned src_lane =
+        (unsigned)((lane >> 3) * K + (((lane & 7) ^ ((lane >> 4) | ((wave & 1) << 2))) * 8)) * 2u;
+    unsigned src_blk[LA > LB ? LA : LB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) src_blk[j] = src_lane + (unsigned)((4 * j + wave) * 16) * (unsigned)K * 2u;
-    const unsigned lds_dst = (unsigned)(size_t)(lptr_t)lds + wave * 1024;   // + stage, operand, 4096 j
-    // fragment reads: row r = lane % 16 of a 16-row group, k segment lane / 16, found in slot
-    // (lane / 16) ^ ((r >> 2) & 3)
-    const int frag_lane = (lane & 15) * ROWB + (((lane >> 4) ^ ((lane >> 2) & 3)) * 16);
-    const int frag_a = wr * (FM * 16) * ROWB + frag_lane;
-    const int frag_b = A_BYTES + wc * (FN * 16) * ROWB + frag_lane;
+    for (int j = 0; j < (LA > LB ? LA : LB); ++j) src_blk[j] = src_lane + (unsigned)((4 * j + wave) * 8) * (unsigned)K * 2u;
+    const unsigned lds_dst = (unsigned)(size_t)(lptr_t)lds + wave * 1024;   // + buffer, operand, 4096 j
+    // fragment reads: row r = lane % 16 of a 16-row group, k segment lane / 16 of chunk h of the
+    // pair, found in slot (4 h + lane / 16) ^ ((r >> 1) & 7)
+    const int frag_row = (lane & 15) * ROWB;
+    const int frag_h0 = frag_row + (((lane >> 4) ^ ((lane & 15) >> 1)) * 16);
+    const int frag_h1 = frag_row + (((4 + (lane >> 4)) ^ ((lane & 15) >> 1)) * 16);
+    const int off_a = wr * (FM * 16) * ROWB;
+    const int off_b = A_BYTES + wc * (FN * 16) * ROWB;
 
     for (int t = role_block; t < n_tiles; t += role_blocks) {
         int mi, mj;
@@ -131,60 +153,70 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
         const char *a_tile = reinterpret_cast<const char *>(A + (size_t)(mi * TM) * K);
         const char *b_tile = reinterpret_cast<const char *>(B + (size_t)(mj * TN) * K);
 
-// all loads of the chunk a_ptr_ / b_ptr_ point at, into stage slot_
-#define TZL_ISSUE_CHUNK(a_ptr_, b_ptr_, slot_)                                                    \
+// all loads of the pair of chunks a_ptr_ / b_ptr_ point at, into buffer buf_
+#define TZL_ISSUE_PAIR(a_ptr_, b_ptr_, buf_)                                                      \
     {                                                                                             \
         _Pragma("unroll") for (int q = 0; q < LA; ++q)                                            \
-            tz_load_to_lds(a_ptr_, src_blk[q], lds_dst + (slot_) * STAGE_BYTES + q * 4096);       \
+            tz_load_to_lds(a_ptr_, src_blk[q], lds_dst + (buf_) * PAIR_BYTES + q * 4096);         \
         _Pragma("unroll") for (int q = 0; q < LB; ++q)                                            \
-            tz_load_to_lds(b_ptr_, src_blk[q], lds_dst + (slot_) * STAGE_BYTES + A_BYTES + q * 4096); \
+            tz_load_to_lds(b_ptr_, src_blk[q], lds_dst + (buf_) * PAIR_BYTES + A_BYTES + q * 4096); \
     }
-#define TZL_READ_FRAGS(fa_, fb_, slot_)                                                           \
-    {                                                                                             \
-        const char *s_ = lds + (slot_) * STAGE_BYTES;                                             \
-        _Pragma("unroll") for (int i = 0; i < FM; ++i)                                            \
-            fa_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_a + i * 16 * ROWB);             \
-        _Pragma("unroll") for (int j = 0; j < FN; ++j)                                            \
-            fb_[j] = *reinterpret_cast<const half8_t *>(s_ + frag_b + j * 16 * ROWB);             \
-    }
+// fragment i of A / j of B of chunk h_ (its lane offset frag_) in buffer buf_
+#define TZL_FRAG_A(buf_, frag_, i_) \
+    *reinterpret_cast<const half8_t *>(lds + (buf_) * PAIR_BYTES + off_a + (frag_) + (i_) * 16 * ROWB)
+#define TZL_FRAG_B(buf_, frag_, j_) \
+    *reinterpret_cast<const half8_t *>(lds + (buf_) * PAIR_BYTES + off_b + (frag_) + (j_) * 16 * ROWB)
 // MFMA n of an iteration updates accumulator tile (n / FN, n % FN)
 #define TZL_MFMA_AT(fa_, fb_, n_)                                                                 \
     acc[(n_) / FN][(n_) % FN] = __builtin_amdgcn_mfma_f32_16x16x32_f16(                           \
         fb_[(n_) % FN], fa_[(n_) / FN], acc[(n_) / FN][(n_) % FN], 0, 0, 0);
-// One iteration: multiply chunk c (fragments fc_) and bring in the fragments of chunk c + 1
-// (into fn_) behind the barrier; do_issue_ (a literal) starts the loads of the chunk a_next /
-// b_next point at into the stage chunk c has left.  vmcnt_: loads of this wave that may still
-// be in flight once chunk c + 1 has landed.
-#define TZL_ITERATION(fc_a_, fc_b_, fn_a_, fn_b_, c_, vmcnt_, do_issue_)                          \
+// First iteration of a pair: multiply its first chunk (fragments fc_) and read the fragments of
+// its second chunk (into fn_) from the same buffer -- landed and published an iteration ago, so
+// no wait and no barrier.
+#define TZL_ITERATION_FIRST(fc_a_, fc_b_, fn_a_, fn_b_, buf_)                                     \
+    {                                                                                             \
+        _Pragma("unroll") for (int n = 0; n < FM * FN; ++n)                                       \
+        {                                                                                         \
+            TZL_MFMA_AT(fc_a_, fc_b_, n)                                                          \
+            if (n % READ_GAP == 0 && n / READ_GAP < FM)                                           \
+                TZL_LOOP_READ(fn_a_[n / READ_GAP], TZL_FRAG_A(buf_, frag_h1, n / READ_GAP));      \
+            else if (n % READ_GAP == 0 && n / READ_GAP < FM + FN)                                 \
+                TZL_LOOP_READ(fn_b_[n / READ_GAP - FM], TZL_FRAG_B(buf_, frag_h1, n / READ_GAP - FM)); \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
+        __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
+    }
+// Second iteration of a pair: multiply its second chunk; behind the first MFMAs wait for this
+// wave's loads of the next pair and meet the other waves -- from then on the next pair is whole
+// in buffer nbuf_ and nobody reads this pair's buffer buf_ any more -- then read the first
+// fragments of the next pair and, if do_issue_, start the loads of the pair a_next / b_next
+// point at into buf_.
+#define TZL_ITERATION_SECOND(fc_a_, fc_b_, fn_a_, fn_b_, buf_, nbuf_, do_issue_)                  \
     {                                                                                             \
         _Pragma("unroll") for (int n = 0; n < FIRST; ++n)                                         \
         {                                                                                         \
             TZL_MFMA_AT(fc_a_, fc_b_, n)                                                          \
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
-        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
-        __builtin_amdgcn_s_barrier();                                                             \
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));                                              \
+        TZL_LOOP_BARRIER();                                                                       \
         asm volatile("" ::: "memory");                                                            \
         __builtin_amdgcn_sched_barrier(0);                                                        \
-        const int slot_ = (c_) & (STAGES - 1);                                                    \
-        const char *next_ = lds + (((c_) + 1) & (STAGES - 1)) * STAGE_BYTES;                      \
         _Pragma("unroll") for (int n = FIRST; n < FM * FN; ++n)                                   \
         {                                                                                         \
             TZL_MFMA_AT(fc_a_, fc_b_, n)                                                          \
             const int r_ = n - FIRST;                                                             \
             if (r_ % READ_GAP == 0 && r_ / READ_GAP < FM)                                         \
-                fn_a_[r_ / READ_GAP] =                                                            \
-                    *reinterpret_cast<const half8_t *>(next_ + frag_a + (r_ / READ_GAP) * 16 * ROWB); \
+                TZL_LOOP_READ(fn_a_[r_ / READ_GAP], TZL_FRAG_A(nbuf_, frag_h0, r_ / READ_GAP));   \
             else if (r_ % READ_GAP == 0 && r_ / READ_GAP < FM + FN)                               \
-                fn_b_[r_ / READ_GAP - FM] =                                                       \
-                    *reinterpret_cast<const half8_t *>(next_ + frag_b + (r_ / READ_GAP - FM) * 16 * ROWB); \
+                TZL_LOOP_READ(fn_b_[r_ / READ_GAP - FM], TZL_FRAG_B(nbuf_, frag_h0, r_ / READ_GAP - FM)); \
             if (do_issue_ && r_ % LOAD_GAP == LOAD_GAP - 1 && r_ / LOAD_GAP < L) {                \
                 const int q_ = r_ / LOAD_GAP;                                                     \
                 if (q_ < LA)                                                                      \
-                    tz_load_to_lds(a_next, src_blk[q_], lds_dst + slot_ * STAGE_BYTES + q_ * 4096); \
+                    TZL_LOOP_LOAD(a_next, src_blk[q_], lds_dst + (buf_) * PAIR_BYTES + q_ * 4096); \
                 else                                                                              \
-                    tz_load_to_lds(b_next, src_blk[q_ - LA],                                      \
-                                   lds_dst + slot_ * STAGE_BYTES + A_BYTES + (q_ - LA) * 4096);   \
+                    TZL_LOOP_LOAD(b_next, src_blk[q_ - LA],                                       \
+                                  lds_dst + (buf_) * PAIR_BYTES + A_BYTES + (q_ - LA) * 4096);    \
             }                                                                                     \
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
@@ -201,29 +233,34 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
 #pragma unroll
             for (int j = 0; j < FN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
 
-        // fill the whole ring (kchunks >= STAGES always), publish chunk 0, fetch its fragments
-        const char *a_next = a_tile, *b_next = b_tile;   // chunk the next loads fetch
-        for (int c = 0; c < STAGES; ++c) {
-            TZL_ISSUE_CHUNK(a_next, b_next, c)
+        // fill both buffers (npairs >= 2 always), publish pair 0, fetch its first fragments
+        const char *a_next = a_tile, *b_next = b_tile;   // pair the next loads fetch
+        for (int b = 0; b < 2; ++b) {
+            TZL_ISSUE_PAIR(a_next, b_next, b)
             a_next += ROWB;
             b_next += ROWB;
         }
-        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(L * (STAGES - 1)));
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(L));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         half8_t fa0[FM], fb0[FN], fa1[FM], fb1[FN];
-        TZL_READ_FRAGS(fa0, fb0, 0)
+#pragma unroll
+        for (int i = 0; i < FM; ++i) fa0[i] = TZL_FRAG_A(0, frag_h0, i);
+#pragma unroll
+        for (int j = 0; j < FN; ++j) fb0[j] = TZL_FRAG_B(0, frag_h0, j);
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);
 
-        int c = 0;
-        for (; c + STAGES < kchunks; c += 2) {
-            TZL_ITERATION(fa0, fb0, fa1, fb1, c, L * (STAGES - 2), true)
-            TZL_ITERATION(fa1, fb1, fa0, fb0, c + 1, L * (STAGES - 2), true)
+        // pairs p, p + 1 live in buffers 0, 1; while they are multiplied pairs p + 2, p + 3 are fetched
+        for (int p = 0; p + 2 < npairs; p += 2) {
+            TZL_ITERATION_FIRST(fa0, fb0, fa1, fb1, 0)
+            TZL_ITERATION_SECOND(fa1, fb1, fa0, fb0, 0, 1, true)
+            TZL_ITERATION_FIRST(fa0, fb0, fa1, fb1, 1)
+            TZL_ITERATION_SECOND(fa1, fb1, fa0, fb0, 1, 0, true)
         }
-        // the last four chunks: nothing left to fetch, fewer loads in flight
-        TZL_ITERATION(fa0, fb0, fa1, fb1, c, L * 2, false)
-        TZL_ITERATION(fa1, fb1, fa0, fb0, c + 1, L * 1, false)
-        TZL_ITERATION(fa0, fb0, fa1, fb1, c + 2, 0, false)
+        // the last two pairs: nothing left to fetch
+        TZL_ITERATION_FIRST(fa0, fb0, fa1, fb1, 0)
+        TZL_ITERATION_SECOND(fa1, fb1, fa0, fb0, 0, 1, false)
+        TZL_ITERATION_FIRST(fa0, fb0, fa1, fb1, 1)
         _Pragma("unroll") for (int n = 0; n < FM * FN; ++n) { TZL_MFMA_AT(fa1, fb1, n) }
         __builtin_amdgcn_s_barrier();   // every wave is done reading before the next tile refills the ring
         asm volatile("" ::: "memory");
@@ -247,13 +284,15 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
                         else *c_at = v;
                     }
             }
-        // stores and LDS-direct loads share the vmcnt counter: drain it so that the counts of
-        // the next tile's ring are exact
-        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
-#undef TZL_ISSUE_CHUNK
-#undef TZL_READ_FRAGS
+        // The stores stay in flight while the next tile starts: they share the vmcnt counter with
+        // the LDS-direct loads, but loads complete in their own order, so "at most L operations
+        // outstanding" in the next tile's prologue still means that its first pair has landed.
+#undef TZL_ISSUE_PAIR
+#undef TZL_FRAG_A
+#undef TZL_FRAG_B
 #undef TZL_MFMA_AT
-#undef TZL_ITERATION
+#undef TZL_ITERATION_FIRST
+#undef TZL_ITERATION_SECOND
     }
 }
 

@@ -25,7 +25,7 @@ extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
     // a launch on a shape the form does not cover (the host never makes one) computes nothing
     if (M_GLOBAL % TZ_LARGE_TILE || N_GLOBAL % TZ_LARGE_TILE || K_GLOBAL % 128) return;
-    tk::tzgemm_role_large<8, 8, TZ_STAGES, true>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x,
+    tk::tzgemm_role_large<8, 8, true>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x,
                                                  ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
                                                  (int)threadIdx.x - thread_base, tz_lds);
 }

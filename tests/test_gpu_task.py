@@ -331,6 +331,8 @@ def test_create_kernel_objects_run_and_match_oracle_for_cp():
     # 32 x 512 blocks of 128 x 8 points, each in 4 parts of its x points
     assert (info["ptb_start"], info["ptb_end"]) == (0, 65536) and info["ori_grid_x"] == 32 and info["ori_grid_y"] == 512
     assert info["nparams"] == 3 + 6 and k.param(0, "int") == 64 and k.param(1, "float") == np.float32(0.1)
+    # the object is memoised and the kernel accumulates: start from the zeroed grid its constructor made
+    assert ta.lib().tkMemset(k.param(2), 0, 4096 * 4096 * 4) == 0
     k.execute()
     torch.cuda.synchronize()
     # the object's own inputs (src/ori_kernel/cp_kernel.cu:66-100): atoms 1..64 of the seeded
