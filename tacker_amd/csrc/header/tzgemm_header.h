@@ -87,6 +87,8 @@ TZ_HOST_DEVICE inline long long tz_workspace_bytes(int M, int N, int K)
 // whole 256 x 256 tiles and at least one of them for every CU.  Same bits as the other forms.
 #define TZ_LARGE_TILE 256
 #define TZ_LARGE_MIN_TILES TK_CU_NUM
+// the large-tile form writes a C above this size with nontemporal stores
+#define TZ_LARGE_STREAM_C_BYTES (128u << 20)
 TZ_HOST_DEVICE inline bool tz_use_large(int M, int N, int K)
 {
     (void)K;

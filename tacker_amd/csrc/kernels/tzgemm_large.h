@@ -79,11 +79,16 @@ __device__ __forceinline__ void tz_large_tile_of(int t, int tile_rows, int tile_
 }
 
 // The role owns every wave of its workgroup (it synchronises with s_barrier).
-template <int FM, int FN, bool STREAM_C>
+// stream_c: C leaves with nontemporal stores.  Pays when C is larger than the caches can hold
+// until the memory has taken it (256 MiB at 8192 x 8192: plain stores push the operand panels out
+// of the L2s); below that plain stores are the faster ones -- the L2s and the memory-side cache
+// take the tile at once and write it back while the next kernel already runs (4096 x 4096 x 1024:
+// 37 instead of 43 us).
+template <int FM, int FN>
 __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
                                                   float *__restrict__ C, int M, int N, int K, int role_block,
                                                   int role_blocks, int tile_start, int tile_end, int tid,
-                                                  char *lds)
+                                                  char *lds, bool stream_c)
 {
     typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int TM = 32 * FM, TN = 32 * FN;      // macro tile
@@ -280,7 +285,7 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
                     for (int j = 4 * rj; j < 4 * rj + 4; ++j) {
                         float4_t v = acc[i][j] * TZ_ALPHA;
                         float4_t *c_at = reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16);
-                        if constexpr (STREAM_C) __builtin_nontemporal_store(v, c_at);
+                        if (stream_c) __builtin_nontemporal_store(v, c_at);   // uniform
                         else *c_at = v;
                     }
             }

@@ -27,8 +27,8 @@ __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1
     _Float16 *A, _Float16 *B, float *C, int M, int N, int K)
 {
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
-    tk::tzgemm_role_large<8, 8, true>(A, B, C, M, N, K, (int)blockIdx.x, (int)gridDim.x, 0, (M / 64) * (N / 64),
-                                      (int)threadIdx.x, tz_lds);
+    tk::tzgemm_role_large<8, 8>(A, B, C, M, N, K, (int)blockIdx.x, (int)gridDim.x, 0, (M / 64) * (N / 64),
+                                (int)threadIdx.x, tz_lds, (size_t)M * (size_t)N * sizeof(float) > TZ_LARGE_STREAM_C_BYTES);
 }
 
 int main(int argc, char **argv)
