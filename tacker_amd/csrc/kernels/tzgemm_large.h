@@ -48,7 +48,8 @@
 #include "tzgemm_role.h"
 
 // Measurement builds only (microbench/tzgemm_large_probe.hip): each macro takes one ingredient out
-// of the steady K loop -- the results are wrong, the time says what the ingredient costs.
+// of the kernel (the loads or the barrier of the steady K loop, the C stores) -- the results are
+// wrong, the time says what the ingredient costs.
 #ifdef TZL_KNOCK_OUT_LOADS
 #define TZL_LOOP_LOAD(...)
 #else
@@ -60,6 +61,11 @@
 #define TZL_LOOP_BARRIER() __builtin_amdgcn_s_barrier()
 #endif
 #define TZL_LOOP_READ(dst_, src_) dst_ = src_
+#ifdef TZL_KNOCK_OUT_STORES
+#define TZL_STORE_IF(v_) if ((v_)[0] == 123.456f)   // never true for the probe's operands
+#else
+#define TZL_STORE_IF(v_)
+#endif
 
 namespace tk {
 
@@ -285,8 +291,11 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
                     for (int j = 4 * rj; j < 4 * rj + 4; ++j) {
                         float4_t v = acc[i][j] * TZ_ALPHA;
                         float4_t *c_at = reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16);
-                        if (stream_c) __builtin_nontemporal_store(v, c_at);   // uniform
-                        else *c_at = v;
+                        TZL_STORE_IF(v)
+                        {
+                            if (stream_c) __builtin_nontemporal_store(v, c_at);   // uniform
+                            else *c_at = v;
+                        }
                     }
             }
         // The stores stay in flight while the next tile starts: they share the vmcnt counter with

@@ -1,7 +1,8 @@
 // tzgemm_large_probe.hip -- the large-tile tzgemm kernel alone in a plain HIP program: its time
-// at a shape, on zero and on random operands, and -- built with TZL_KNOCK_OUT_LOADS or
-// TZL_KNOCK_OUT_BARRIER -- what the global->LDS loads and the workgroup barrier of the steady
-// K loop cost (those builds compute wrong results on purpose).
+// at a shape, on zero and on random operands, and -- built with TZL_KNOCK_OUT_LOADS,
+// TZL_KNOCK_OUT_BARRIER or TZL_KNOCK_OUT_STORES -- what the global->LDS loads and the workgroup
+// barrier of the steady K loop and the C stores cost (those builds compute wrong results on
+// purpose).
 //
 //   build: hipcc --offload-arch=gfx950 -O3 -std=c++17 -ffp-contract=off -Xclang -target-feature
 //          -Xclang -packed-fp32-ops [-DTZL_KNOCK_OUT_...] -o tzgemm_large_probe tzgemm_large_probe.hip
