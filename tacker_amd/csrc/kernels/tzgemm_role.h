@@ -177,6 +177,13 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
                               (((q_) & 1) ? OPERAND_BYTES : 0);                                   \
         tz_load_to_lds((((q_) & 1) ? b_tile : a_tile) + uni_, (j_ & 1) ? src_odd : src_even, dst_); \
     }
+// loads issued from inside the steady K loop; a measurement build (microbench/fused_probe.hip)
+// takes them out to see what they cost (results wrong on purpose)
+#ifdef TZ_KNOCK_OUT_LOADS
+#define TZ_LOOP_ISSUE_ONE(chunk_, stage_, q_) {}
+#else
+#define TZ_LOOP_ISSUE_ONE(chunk_, stage_, q_) TZ_ISSUE_ONE(chunk_, stage_, q_)
+#endif
 #define TZ_ISSUE_CHUNK(chunk_, stage_)                                                            \
     _Pragma("unroll") for (int q = 0; q < LOADS_PER_CHUNK; ++q) TZ_ISSUE_ONE(chunk_, stage_, q)
 #define TZ_READ_FRAGS(fa_, fb_, stage_, seg_)                                                     \
@@ -186,9 +193,13 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         fa_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_a);                                 \
         fb_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_b);                                 \
     }
+#ifdef TZ_KNOCK_OUT_MFMA   // measurement build: no MFMAs but the 4 of a split barrier's asm block
+#define TZ_MFMAS_ROWS(fa_, fb_, i0_, i1_)
+#else
 #define TZ_MFMAS_ROWS(fa_, fb_, i0_, i1_)                                                         \
     _Pragma("unroll") for (int i = i0_; i < i1_; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[j], fa_[i], acc[i][j], 0, 0, 0);
+#endif
 #define TZ_MFMAS(fa_, fb_) TZ_MFMAS_ROWS(fa_, fb_, 0, 4)
 // Issue order inside one scheduling region: after each MFMA one LDS read (count_ of them),
 // then after each MFMA one LDS-direct load (count2_).  An MFMA occupies the matrix pipe for
@@ -201,9 +212,13 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         __builtin_amdgcn_sched_group_barrier(mask_, 1, 0);                                        \
     }
 #define TZ_SCHED_DS_READ 0x100
+#ifdef TZ_KNOCK_OUT_MFMA
+#define TZ_MFMA_AT(fa_, fb_, n_)
+#else
 #define TZ_MFMA_AT(fa_, fb_, n_)                                                                  \
     acc[(n_) >> 2][(n_) & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[(n_) & 3], fa_[(n_) >> 2], \
                                                                       acc[(n_) >> 2][(n_) & 3], 0, 0, 0);
+#endif
 // First k-step of a chunk multiplied while the chunk barrier completes; the reads of the
 // second k-step (into fn_, fbn_) ride in the shadow of the first 8 MFMAs, and loads 4..7 of
 // chunk tail_chunk_ (the half of a chunk the previous second k-step did not issue) follow one
@@ -222,7 +237,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
         {                                                                                         \
             TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
-            if ((tail_chunk_) >= 0) TZ_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q)                 \
+            if ((tail_chunk_) >= 0) TZ_LOOP_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q)            \
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
@@ -255,7 +270,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         _Pragma("unroll") for (int q = 0; q < 8; ++q)                                             \
         {                                                                                         \
             TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
-            if ((q & 1) == 0 && (tail_chunk_) >= 0) TZ_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q / 2) \
+            if ((q & 1) == 0 && (tail_chunk_) >= 0) TZ_LOOP_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q / 2) \
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
         __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
@@ -277,7 +292,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
         {                                                                                         \
             TZ_MFMA_AT(fa_, fb_, 12 + q)                                                          \
-            if ((chunk_) >= 0) TZ_ISSUE_ONE(chunk_, stage_, q)                                    \
+            if ((chunk_) >= 0) TZ_LOOP_ISSUE_ONE(chunk_, stage_, q)                               \
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
     } else {                                                                                      \
@@ -287,7 +302,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         _Pragma("unroll") for (int q = 0; q < 8; ++q)                                             \
         {                                                                                         \
             TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
-            if ((q & 1) == 0 && (chunk_) >= 0) TZ_ISSUE_ONE(chunk_, stage_, q / 2)                \
+            if ((q & 1) == 0 && (chunk_) >= 0) TZ_LOOP_ISSUE_ONE(chunk_, stage_, q / 2)           \
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
     }
@@ -390,6 +405,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
 #undef TZ_ISSUE_CHUNK
 #undef TZ_ISSUE_ONE
+#undef TZ_LOOP_ISSUE_ONE
 #undef TZ_MFMA_AT
 #undef TZ_READ_FRAGS
 #undef TZ_MFMAS
