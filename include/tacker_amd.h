@@ -101,8 +101,8 @@ TK_API int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void 
 /* Fills the string-keyed device-function registry (the global `fmap` of
  * src/main.cu:108-159) without the host translation unit including device
  * sources: insert(key, function, ctx) is called once per kernel. Keys on the
- * hot path: ori_{stencil,lbm,mriq,mrif,cp}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp},
- * tzgemm_{stencil,lbm,mriq,mrif,cp}, plus variant keys "<key>@<variant>". */
+ * hot path: ori_{stencil,lbm,mriq,mrif,cp,sgemm}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp,sgemm},
+ * tzgemm_{stencil,lbm,mriq,mrif,cp,sgemm}, plus variant keys "<key>@<variant>". */
 typedef void (*tk_kernel_insert_fn)(const char *key, const void *func, void *ctx);
 TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx);
 
@@ -234,6 +234,23 @@ TK_API int tacker_gptb_mrif(int numK, const float *x, const float *y, const floa
                             float *outI, int numX, int block_start, int block_end, int launch_grid,
                             int launch_block, tkStream_t stream);
 
+/* ori_sgemm / general_ptb_sgemm (src/ori_kernel/sgemm_kernel.cu:9-44,
+ * src/gptb_kernel/sgemm_kernel.cu:3-77): C = 2 C + 2 A B in fp32; A is K rows of M floats (lda = M),
+ * B K rows of N floats (ldb = N), C N columns of M floats (ldc = M); M a multiple of 128, N of 16.
+ * k ascends per element of C, every step one fused multiply-add.  Block positions of the GPTB form:
+ * the reference's (M / 128) x (N / 16) blocks by ceil(K / TACKER_SGEMM_K_CHUNK) parts of the k loop as
+ * the z index; between parts a block's partial results rest in a workspace of M x N floats that the
+ * library binds to C when a kernel object is built on it (tacker_tzgemm_release_workspaces frees
+ * it).  [0, tacker_sgemm_blocks(M, N, K)) equals ori_sgemm bit for bit, and so does any sequence
+ * of launches whose ranges tile it in ascending order. */
+#define TACKER_SGEMM_K_CHUNK 256
+TK_API int tacker_sgemm_blocks(int M, int N, int K);
+TK_API int tacker_ori_sgemm(const float *A, const float *B, float *C, int M, int N, int K,
+                            tkStream_t stream);
+TK_API int tacker_gptb_sgemm(const float *A, const float *B, float *C, int M, int N, int K,
+                             int block_start, int block_end, int launch_grid, int launch_block,
+                             tkStream_t stream);
+
 /* copyatomstoconstbuf (src/ori_kernel/cp_kernel.cu:159-179): host array of
  * count (<= 64) {x,y,z,q}; z is replaced by (zplane - z)^2 on the way. */
 TK_API int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane);
@@ -290,6 +307,13 @@ TK_API int tacker_mix_tzgemm_mrif(int numK, const float *x, const float *y, cons
                                   const void *A, const void *B, float *C, int M, int N, int K,
                                   int tile_start, int tile_end, const char *variant,
                                   int launch_grid, int launch_block, tkStream_t stream);
+/* src/mix_kernel/tzgemm_sgemm.cu: the best-effort SGEMM (sA, sB, sC, sM, sN, sK) first, then the
+ * latency-critical GEMM, as MixKernel concatenates them */
+TK_API int tacker_mix_tzgemm_sgemm(const float *sA, const float *sB, float *sC, int sM, int sN, int sK,
+                                   int be_start, int be_end, const void *A, const void *B, float *C,
+                                   int M, int N, int K, int tile_start, int tile_end,
+                                   const char *variant, int launch_grid, int launch_block,
+                                   tkStream_t stream);
 TK_API int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx,
                                 int voly, int be_start, int be_end, const void *A, const void *B,
                                 float *C, int M, int N, int K, int tile_start, int tile_end,
@@ -312,7 +336,7 @@ TK_API float tacker_fget_kernel_info(const char *kernel, const char *key);
 /* ---- object API: the class layer itself, one handle per C++ object ---------- */
 typedef void *tacker_kernel_t;
 
-/* createKernel (src/Creator.cu:21-337) for the names cp, lbm, mrif, mriq, stencil,
+/* createKernel (src/Creator.cu:21-337) for the names cp, lbm, mrif, mriq, sgemm, stencil,
  * tzgemm: the memoised GPTBKernel that owns seeded device buffers exactly as the
  * reference's Ori*Kernel::initParams builds them. Never destroy these. */
 TK_API tacker_kernel_t tacker_create_kernel(const char *name);
@@ -324,6 +348,8 @@ TK_API tacker_kernel_t tacker_ori_stencil_create(float c0, float c1, const float
 TK_API tacker_kernel_t tacker_ori_lbm_create(const float *src, float *dst, int sx, int sy, int sz);
 TK_API tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y,
                                               const float *z, float *Qr, float *Qi, int numX);
+TK_API tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N,
+                                               int K);
 TK_API tacker_kernel_t tacker_ori_mrif_create(int numK, const float *x, const float *y,
                                               const float *z, float *outR, float *outI, int numX);
 TK_API tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid,

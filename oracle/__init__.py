@@ -47,6 +47,7 @@ def _declare(l):
     l.orc_stencil_gptb.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int,
                                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_stencil.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+    l.orc_sgemm_gptb.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 9
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
@@ -245,6 +246,40 @@ def cp(atominfo, energygrid, gridspacing=0.1, start=0, end=None, parts=1):
     atominfo = np.ascontiguousarray(atominfo, np.float32).reshape(-1)
     out = np.array(energygrid, np.float32, order="C")
     lib().orc_cp_gptb(atominfo.size // 4, gridspacing, out.reshape(-1), atominfo, gdx, gdy, parts, start, end)
+    return out
+
+
+# --------------------------------------------------------------------------- sgemm
+SGEMM_K_CHUNK = 256
+
+
+def sgemm_positions(M, N, K, chunk=SGEMM_K_CHUNK):
+    return (M // 128) * (N // 16) * -(-K // chunk)
+
+
+def sgemm(A, B, Cm, start=0, end=None, parts=1, W=None, chunk=SGEMM_K_CHUNK):
+    """C = 2 C + 2 A B with A [K][M], B [K][N], C [N][M] float32 (M multiple of 128, N of 16).
+
+    Block positions [start, end) of the (M/128, N/16, parts) grid: parts=1, a position is a block's whole
+    k loop (the reference's kernel); parts='chunks', position p adds k part p // blocks (chunk k steps) to
+    block p % blocks, partial results resting in W ([N][M], updated in place when given) between parts.
+    Returns the new C."""
+    A = np.ascontiguousarray(A, np.float32)
+    B = np.ascontiguousarray(B, np.float32)
+    K, M = A.shape
+    N = B.shape[1]
+    assert B.shape[0] == K and Cm.shape == (N, M) and M % 128 == 0 and N % 16 == 0
+    gdx, gdy = M // 128, N // 16
+    if parts == "chunks":
+        parts = -(-K // chunk)
+    if end is None:
+        end = gdx * gdy * parts
+    out = np.array(Cm, np.float32, order="C")
+    if W is None:
+        W = np.zeros((N, M), np.float32)
+    assert W.dtype == np.float32 and W.flags["C_CONTIGUOUS"] and W.shape == (N, M)
+    lib().orc_sgemm_gptb(A.reshape(-1), B.reshape(-1), out.reshape(-1), W.reshape(-1), M, N, K, gdx, gdy, parts,
+                         chunk, start, end)
     return out
 
 

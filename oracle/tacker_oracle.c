@@ -700,3 +700,52 @@ ORC_API void orc_im2col(int n, const float *data_im, int height, int width, int 
         }
     }
 }
+
+/* ------------------------------------------------------------------ sgemm
+ * src/ori_kernel/sgemm_kernel.cu:9-44 (general_ptb_sgemm: src/gptb_kernel/sgemm_kernel.cu:3-77):
+ * C[m + n ldc] = C[m + n ldc] * beta + alpha * sum_k A[m + k lda] * B[n + k ldb], lda = ldc = M,
+ * ldb = N, alpha = beta = 2, k ascending, each step c = fma(a, b, c) -- what nvcc's default
+ * -fmad=true makes of "c[kk] += a * b_s[j][kk]".  A block is 128 rows m by 16 columns n.
+ *
+ * Positions [start, end) of the (gdx, gdy, gdz) grid: position p adds, to block p % (gdx*gdy),
+ * k part (p / (gdx*gdy)) % gdz, i.e. k in [part*chunk, min((part+1)*chunk, K)) (the last part
+ * runs to K).  gdz = 1: a position is a block's whole k loop, the reference's kernel.  Part 0
+ * starts from zero, other parts from what the block's previous part left in W (M x N floats,
+ * laid out as C); the last part scales and updates C.  Positions of one block are applied in
+ * ascending order. */
+ORC_API void orc_sgemm_gptb(const float *A, const float *B, float *C, float *W, int M, int N, int K, int gdx,
+                            int gdy, int gdz, int chunk, int start, int end)
+{
+    const int TILE_M = 128, TILE_N = 16;
+    const float alpha = 2.0f, beta = 2.0f;
+    const int blocks = gdx * gdy;
+#pragma omp parallel for schedule(dynamic)
+    for (int blk = 0; blk < blocks; blk++) {
+        int first = start + ((blk - start % blocks) + blocks) % blocks;
+        for (int pos = first; pos < end; pos += blocks) {
+            const int bx = pos % gdx, by = (pos / gdx) % gdy, part = (pos / blocks) % gdz;
+            const int k0 = gdz > 1 ? (part * chunk < K ? part * chunk : K) : 0;
+            const int k1 = (gdz == 1 || part == gdz - 1) ? K : ((part + 1) * chunk < K ? (part + 1) * chunk : K);
+            for (int mid = 0; mid < TILE_M; mid++) {
+                const size_t m = (size_t)bx * TILE_M + mid;
+                const size_t t = (size_t)M * by * TILE_N + m;
+                float c[16];
+                for (int i = 0; i < TILE_N; i++) c[i] = k0 == 0 ? 0.0f : W[t + (size_t)i * M];
+                for (int k = k0; k < k1; k++) {
+                    const float a = A[m + (size_t)k * M];
+                    const float *b = B + (size_t)by * TILE_N + (size_t)k * N;
+                    for (int i = 0; i < TILE_N; i++) c[i] = fmaf(a, b[i], c[i]);
+                }
+                for (int i = 0; i < TILE_N; i++) {
+                    if (k1 == K) {
+                        const float scaled_old = C[t + (size_t)i * M] * beta;
+                        const float scaled_sum = alpha * c[i];
+                        C[t + (size_t)i * M] = scaled_old + scaled_sum;
+                    } else {
+                        W[t + (size_t)i * M] = c[i];
+                    }
+                }
+            }
+        }
+    }
+}

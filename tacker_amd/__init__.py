@@ -66,6 +66,10 @@ def _declare(lib):
     lib.tacker_ori_mrif.argtypes = [i, vp, vp, vp, vp, vp, i, vp]
     lib.tacker_gptb_mrif.argtypes = [i, vp, vp, vp, vp, vp, i, i, i, i, i, vp]
     lib.tacker_mix_tzgemm_mrif.argtypes = [i, vp, vp, vp, vp, vp, i, i, i] + gemm
+    lib.tacker_sgemm_blocks.argtypes = [i, i, i]
+    lib.tacker_ori_sgemm.argtypes = [vp, vp, vp, i, i, i, vp]
+    lib.tacker_gptb_sgemm.argtypes = [vp, vp, vp, i, i, i, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_sgemm.argtypes = [vp, vp, vp, i, i, i, i, i] + gemm
     lib.tacker_mix_tzgemm_cp.argtypes = [i, f, vp, i, i, i, i] + gemm
     lib.tacker_im2col.argtypes = [vp] + [i] * 11 + [vp, vp]
     lib.tacker_convert_fp32_to_fp16.argtypes = [vp, vp, i, vp]
@@ -75,6 +79,7 @@ def _declare(lib):
     lib.tacker_fget_kernel_info.restype = f
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
                  "tacker_ori_mriq_create", "tacker_ori_mrif_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
+                 "tacker_ori_sgemm_create",
                  "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
                  "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
@@ -83,6 +88,7 @@ def _declare(lib):
     lib.tacker_ori_lbm_create.argtypes = [vp, vp, i, i, i]
     lib.tacker_ori_mriq_create.argtypes = [i, vp, vp, vp, vp, vp, i]
     lib.tacker_ori_mrif_create.argtypes = [i, vp, vp, vp, vp, vp, i]
+    lib.tacker_ori_sgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
     lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_gptb_create.argtypes = [vp, i, i, i, i]
@@ -416,6 +422,43 @@ def mix_tzgemm_mrif(numK, x, y, z, outR, outI, A, B, Cm, be_start=0, be_end=None
         "tacker_mix_tzgemm_mrif")
 
 
+def _sgemm_dims(sA, sB, sC):
+    """A is [K][M], B [K][N], C [N][M] (the reference's lda = M, ldb = N, ldc = M)"""
+    K, M = sA.shape
+    N = sB.shape[1]
+    assert sB.shape[0] == K and tuple(sC.shape) == (N, M)
+    return M, N, K
+
+
+def sgemm_blocks(M, N, K):
+    """block positions of the GPTB form: blocks of 128 x 16 of C x parts of the k loop"""
+    return lib().tacker_sgemm_blocks(M, N, K)
+
+
+def ori_sgemm(sA, sB, sC, stream=None):
+    M, N, K = _sgemm_dims(sA, sB, sC)
+    check(lib().tacker_ori_sgemm(_ptr(sA), _ptr(sB), _ptr(sC), M, N, K, _stream(stream)), "tacker_ori_sgemm")
+
+
+def gptb_sgemm(sA, sB, sC, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    M, N, K = _sgemm_dims(sA, sB, sC)
+    if end is None:
+        end = sgemm_blocks(M, N, K)
+    check(lib().tacker_gptb_sgemm(_ptr(sA), _ptr(sB), _ptr(sC), M, N, K, start, end, launch_grid, launch_block,
+                                  _stream(stream)), "tacker_gptb_sgemm")
+
+
+def mix_tzgemm_sgemm(sA, sB, sC, A, B, Cm, be_start=0, be_end=None, tile_start=0, tile_end=None, variant=None,
+                     launch_grid=0, launch_block=0, stream=None):
+    M, N, K = _sgemm_dims(sA, sB, sC)
+    if be_end is None:
+        be_end = sgemm_blocks(M, N, K)
+    check(lib().tacker_mix_tzgemm_sgemm(
+        _ptr(sA), _ptr(sB), _ptr(sC), M, N, K, be_start, be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_sgemm")
+
+
 def mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, A, B, Cm, be_start=0, be_end=None, tile_start=0,
                     tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
     if be_end is None:
@@ -546,6 +589,12 @@ def ori_mriq_create(numK, x, y, z, Qr, Qi):
 def ori_mrif_create(numK, x, y, z, outR, outI):
     return KernelHandle(lib().tacker_ori_mrif_create(numK, _ptr(x), _ptr(y), _ptr(z), _ptr(outR), _ptr(outI),
                                                      x.numel()), "OriMRIFKernel", keep=(x, y, z, outR, outI))
+
+
+def ori_sgemm_create(sA, sB, sC):
+    M, N, K = _sgemm_dims(sA, sB, sC)
+    return KernelHandle(lib().tacker_ori_sgemm_create(_ptr(sA), _ptr(sB), _ptr(sC), M, N, K), "OriSGEMMKernel",
+                        keep=(sA, sB, sC))
 
 
 def ori_cp_create(numatoms, gridspacing, grid):

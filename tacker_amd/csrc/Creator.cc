@@ -55,6 +55,9 @@ GPTBKernel *createKernel(const std::string &name)
     } else if (name == "mrif") {
         auto *ori = new OriMRIFKernel(17);
         k = new GPTBKernel(17, "mrif", "gptb_mrif", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
+    } else if (name == "sgemm") {
+        auto *ori = new OriSGEMMKernel(21);
+        k = new GPTBKernel(21, "sgemm", "gptb_sgemm", ori, gptbGrid(name), gptbBlock(name, 128), 0, oriBlocks(name, ori));
     } else if (name == "stencil") {
         auto *ori = new OriSTENCILKernel(19);
         k = new GPTBKernel(19, "stencil", "gptb_stencil", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));

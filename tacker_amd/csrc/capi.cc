@@ -69,8 +69,8 @@ int check_block(const std::string &name, int block)
         return fail(TK_ERROR_INVALID_VALUE, "tzgemm: launch_block must be 256");
     if ((name == "mriq" || name == "mrif") && block % 256)
         return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 256");
-    if (name == "cp" && block % 128)
-        return fail(TK_ERROR_INVALID_VALUE, "cp: launch_block must be a multiple of 128");
+    if ((name == "cp" || name == "sgemm") && block % 128)
+        return fail(TK_ERROR_INVALID_VALUE, name + ": launch_block must be a multiple of 128");
     return TK_SUCCESS;
 }
 
@@ -444,6 +444,54 @@ int tacker_gptb_mrif(int numK, const float *x, const float *y, const float *z, f
                          launch_block, stream);
 }
 
+namespace {
+int check_sgemm(const float *A, const float *B, float *C, int M, int N, int K)
+{
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return fail(TK_ERROR_INVALID_VALUE, "sgemm: bad arguments");
+    if (M % SGEMM_TILE_M || N % SGEMM_TILE_N)
+        return fail(TK_ERROR_UNSUPPORTED, "sgemm: M must be a multiple of 128 and N of 16");
+    if ((long long)M * K >= (1ll << 31) || (long long)N * K >= (1ll << 31) || (long long)M * N >= (1ll << 31))
+        return fail(TK_ERROR_UNSUPPORTED, "sgemm: a matrix of 2^31 elements or more");
+    return TK_SUCCESS;
+}
+}  // namespace
+
+int tacker_sgemm_blocks(int M, int N, int K)
+{
+    static_assert(TACKER_SGEMM_K_CHUNK == SGEMM_K_CHUNK, "public and device chunk sizes must agree");
+    if (M < 0 || N < 0 || K <= 0) return 0;
+    return (M / SGEMM_TILE_M) * (N / SGEMM_TILE_N) * ((K + SGEMM_K_CHUNK - 1) / SGEMM_K_CHUNK);
+}
+
+int tacker_ori_sgemm(const float *A, const float *B, float *C, int M, int N, int K, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_sgemm(A, B, C, M, N, K);
+    if (rc) return rc;
+    Kernel *ori = nullptr;   // binding a workspace to C can fail (allocation): not outside guarded()
+    const int made = guarded([&]() -> int {
+        ori = new OriSGEMMKernel(0, A, B, C, M, N, K);
+        return TK_SUCCESS;
+    });
+    if (made) return made;
+    return run_once(ori, stream);
+}
+
+int tacker_gptb_sgemm(const float *A, const float *B, float *C, int M, int N, int K, int block_start, int block_end,
+                      int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_sgemm(A, B, C, M, N, K);
+    if (rc) return rc;
+    Kernel *ori = nullptr;
+    const int made = guarded([&]() -> int {
+        ori = new OriSGEMMKernel(0, A, B, C, M, N, K);
+        return TK_SUCCESS;
+    });
+    if (made) return made;
+    return run_gptb_once(ori, block_start, block_end, launch_grid, launch_block, stream);
+}
+
 int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane)
 {
     REQUIRE_INIT();
@@ -553,6 +601,23 @@ int tacker_mix_tzgemm_mrif(int numK, const float *x, const float *y, const float
                         tile_start, tile_end, variant, launch_grid, launch_block, stream);
 }
 
+int tacker_mix_tzgemm_sgemm(const float *sA, const float *sB, float *sC, int sM, int sN, int sK, int be_start,
+                            int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                            int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_sgemm(sA, sB, sC, sM, sN, sK);
+    if (rc) return rc;
+    Kernel *ori = nullptr;
+    const int made = guarded([&]() -> int {
+        ori = new OriSGEMMKernel(0, sA, sB, sC, sM, sN, sK);
+        return TK_SUCCESS;
+    });
+    if (made) return made;
+    return run_mix_once(ori, be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid,
+                        launch_block, stream);
+}
+
 int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, int be_start,
                          int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
                          int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
@@ -616,7 +681,7 @@ tacker_kernel_t tacker_create_kernel(const char *name)
         fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
         return nullptr;
     }
-    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "stencil", "tzgemm"};
+    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "sgemm", "stencil", "tzgemm"};
     bool ok = false;
     for (auto k : known) ok |= (strcmp(k, name) == 0);
     if (!ok) {
@@ -658,6 +723,11 @@ tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y,
 {
     CREATE(check_mriq(numK, x, y, z, Qr, Qi, numX), new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX));
 }
+tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N, int K)
+{
+    CREATE(check_sgemm(A, B, C, M, N, K), new OriSGEMMKernel(0, A, B, C, M, N, K));
+}
+
 tacker_kernel_t tacker_ori_mrif_create(int numK, const float *x, const float *y, const float *z, float *outR, float *outI, int numX)
 {
     CREATE(check_mrif(numK, x, y, z, outR, outI, numX), new OriMRIFKernel(0, numK, x, y, z, outR, outI, numX));
@@ -1025,7 +1095,7 @@ tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const ch
         fail(TK_ERROR_INVALID_VALUE, "tacker_task_manager_create: bad arguments");
         return nullptr;
     }
-    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "stencil"};
+    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "sgemm", "stencil"};
     bool ok1 = false, ok2 = !be2 || !*be2;
     for (auto k : known) {
         ok1 |= strcmp(k, be1) == 0;

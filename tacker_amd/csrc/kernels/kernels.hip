@@ -16,6 +16,7 @@
 #include "lbm_role.h"
 #include "mriq_role.h"
 #include "mrif_role.h"
+#include "sgemm_role.h"
 #include "stencil_role.h"
 #include "tzgemm_role.h"
 
@@ -86,6 +87,16 @@ extern "C" __global__ __launch_bounds__(256) void ori_mrif(int numK, int kGlobal
 {
     (void)kGlobalIndex;
     tk::mrif_voxel(numK, x, y, z, outR, outI, blockIdx.x * KERNEL_FH_THREADS_PER_BLOCK + threadIdx.x);
+}
+
+// grid (M/128, N/16), block (16,8): a thread's row of C is its flattened id in the block
+// (src/ori_kernel/sgemm_kernel.cu:9-44)
+extern "C" __global__ __launch_bounds__(128) void ori_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N,
+                                                            int NORMAL_K)
+{
+    const int mid = threadIdx.y * blockDim.x + threadIdx.x;
+    tk::sgemm_thread(A, B, C, nullptr, NORMAL_M, NORMAL_N, NORMAL_K, blockIdx.x * SGEMM_TILE_M + mid,
+                     blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K);
 }
 
 // grid (volx/128, voly/8), block (16,8)
@@ -196,6 +207,15 @@ extern "C" __global__ void general_ptb_mrif(int numK, int kGlobalIndex, float *x
                   (int)blockDim.x);
 }
 
+// src/gptb_kernel/sgemm_kernel.cu:3-6
+extern "C" __global__ void general_ptb_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N, int NORMAL_K,
+                                             GPTB_TRAILER)
+{
+    tk::sgemm_role(A, B, C, NORMAL_M, NORMAL_N, NORMAL_K, grid_dimension_x, grid_dimension_y, grid_dimension_z,
+                   (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
+                   (int)threadIdx.x - thread_base, (int)blockDim.x);
+}
+
 extern "C" __global__ void g_general_ptb_cp(int numatoms, float gridspacing, float *energygrid,
                                             GPTB_TRAILER)
 {
@@ -276,6 +296,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ori_cp", (const void *)ori_cp, ctx);
     insert("ComputeRhoPhiGPU", (const void *)ComputeRhoPhiGPU, ctx);
     insert("ori_mrif", (const void *)ori_mrif, ctx);
+    insert("ori_sgemm", (const void *)ori_sgemm, ctx);
     insert("gptb_tzgemm", (const void *)general_ptb_tzgemm, ctx);
     insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);
     insert("tz_clear_words", (const void *)tz_clear_words, ctx);
@@ -284,6 +305,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("gptb_mriq", (const void *)g_general_ptb_mriq, ctx);
     insert("gptb_cp", (const void *)g_general_ptb_cp, ctx);
     insert("gptb_mrif", (const void *)general_ptb_mrif, ctx);
+    insert("gptb_sgemm", (const void *)general_ptb_sgemm, ctx);
     insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);
     insert("im2col", (const void *)im2col_gpu_kernel_, ctx);
     insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);

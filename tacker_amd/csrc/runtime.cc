@@ -13,6 +13,7 @@
 #include "json.h"
 #include "rng.h"
 #include "tzgemm_kernel.h"
+#include "ori_kernel/sgemm_kernel.h"
 #include "mix_kernel/kinfo_builtin.inc"
 
 Logger logger("", getenv("TACKER_QUIET") == nullptr, false);
@@ -90,9 +91,9 @@ void publish_workspace(const void *C, void *workspace)
 }
 }  // namespace
 
-void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
+// a device buffer of at least `need` zeroed bytes bound to the output buffer C
+static void *workspaceFor(const void *C, long long need)
 {
-    const long long need = tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL);
     if (need == 0 || C == nullptr) return nullptr;
     std::lock_guard<std::mutex> lock(g_workspace_mutex);
     auto it = g_workspaces.find(C);
@@ -101,7 +102,7 @@ void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBA
         throw std::runtime_error("tzgemm: " + std::to_string(kMaxBoundWorkspaces) +
                                  " output buffers hold a workspace; call tzgemmReleaseWorkspaces() once the "
                                  "kernels that use them are gone");
-    // a new binding is rare (first GEMM on this C, or a larger shape), so it may wait for the device
+    // a new binding is rare (first kernel object on this C, or a larger shape), so it may wait for the device
     void *ptr = nullptr;
     TK_SAFE_CALL(tkMalloc(&ptr, (size_t)need));
     TK_SAFE_CALL(tkMemset(ptr, 0, (size_t)need));
@@ -115,6 +116,16 @@ void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBA
     if (it != g_workspaces.end()) g_outgrown_workspaces.push_back(it->second.ptr);
     g_workspaces[C] = BoundWorkspace{ptr, need};
     return ptr;
+}
+
+void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
+{
+    return workspaceFor(C, tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL));
+}
+
+void *sgemmWorkspaceFor(const float *C, int M, int N)
+{
+    return workspaceFor(C, (long long)M * N * (long long)sizeof(float));
 }
 
 void tzgemmReleaseWorkspaces()

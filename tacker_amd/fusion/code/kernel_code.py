@@ -1,7 +1,7 @@
 """Role descriptions the generator stitches together.
 
 Each entry plays the part of one ``<kernel>_code.py`` of the reference
-(fusion/code/cp_code.py, lbm_code.py, mriq_code.py, mrif_code.py, stencil_code.py and the
+(fusion/code/cp_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
 truncated tzgemm_code.py): the kernel's parameter list in reference order and
 how to call its device-side role.  The role bodies themselves live in
 ``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
@@ -60,6 +60,14 @@ ROLES = {
         "call": ("tk::mrif_role({p}numK, {p}x, {p}y, {p}z, {p}outR, {p}outI, {p}grid_dimension_x, "
                  "{p}grid_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "{threads});"),
+    },
+    "sgemm": {
+        "params": [("float*", "A"), ("float*", "B"), ("float*", "C"),
+                   ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K")],
+        "needs_sync": False,
+        "call": ("tk::sgemm_role({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, {p}grid_dimension_x, "
+                 "{p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, {p}ptb_start_block_pos, "
+                 "{p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "cp": {
         "params": [("int", "numatoms"), ("float", "gridspacing"), ("float*", "energygrid")],

@@ -76,10 +76,10 @@ def test_committed_generated_sources_are_fresh():
     assert rc.returncode == 0, rc.stdout + rc.stderr
 
 
-@pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27)])
+@pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27), ("sgemm", 30)])
 def test_emitted_dispatcher_signature(be, n_params):
     # parameter count = the reference dispatcher's (src/mix_kernel/tzgemm_stencil.cu:281-283 31,
-    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27), order: be first
+    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27, tzgemm_sgemm.cu:303 30), order: be first
     text, meta = gen_mix.generate_wg_split(be, 1, 1)
     sig = re.search(r"void (\w+)\(\s*(.*?)\)\s*\{", text, re.S)
     params = [p.strip() for p in sig.group(2).split(",")]
@@ -110,9 +110,15 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
     files = gen_run.generate()
     kinfo = json.loads(files["../config/kinfo-gfx950.json"])
     pairs = gen_run.be_pairs()
-    assert pairs == [("cp", "lbm"), ("cp", "mrif"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mrif"),
-                     ("lbm", "mriq"), ("lbm", "stencil"), ("mrif", "mriq"), ("mrif", "stencil"),
-                     ("mriq", "stencil")]
+    assert pairs == [("cp", "lbm"), ("cp", "mrif"), ("cp", "mriq"), ("cp", "sgemm"), ("cp", "stencil"), ("lbm", "mrif"),
+                     ("lbm", "mriq"), ("lbm", "sgemm"), ("lbm", "stencil"), ("mrif", "mriq"), ("mrif", "sgemm"),
+                     ("mrif", "stencil"), ("mriq", "sgemm"), ("mriq", "stencil"), ("sgemm", "stencil")]
+    # the four sgemm pairs the reference ships: src/mix_kernel/{cp_sgemm_1_1,lbm_sgemm_1_7,mrif_sgemm_1_4,mriq_sgemm_1_2}.cu
+    cp_sgemm = files["mix_kernel/cp_sgemm.hip"]
+    sig = re.search(r"void cp_sgemm_mix_wg_1_1\(\s*(.*?)\)\s*\{", cp_sgemm, re.S)
+    names = [q.split()[-1] for q in sig.group(1).split(",")]
+    assert len(names) == 27 and names[12:18] == ["sgemm1_A", "sgemm1_B", "sgemm1_C", "sgemm1_NORMAL_M", "sgemm1_NORMAL_N",
+                                                 "sgemm1_NORMAL_K"]          # cp_sgemm_1_1.cu:163
     assert ("lbm", "mrif") in pairs and ("mrif", "stencil") in pairs   # src/mix_kernel/lbm_mrif_1_3.cu, mrif_stencil_3_2.cu
     assert ("lbm", "mriq") in pairs                       # the pair src/Creator.cu:341-816 also has
     for a, b in pairs:

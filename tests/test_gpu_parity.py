@@ -766,14 +766,27 @@ def _small_be(name):
         outR, outI = torch.zeros(2048, device="cuda:0"), torch.zeros(2048, device="cuda:0")
         return (ta.ori_mrif_create(256, dev(xyz[0]), dev(xyz[1]), dev(xyz[2]), outR, outI), ta.mrif_blocks(256, 2048),
                 [outR, outI])
+    if name == "sgemm":
+        sA, sB, sC0 = sgemm_inputs()
+        sC = dev(sC0)
+        return ta.ori_sgemm_create(dev(sA), dev(sB), sC), ta.sgemm_blocks(256, 48, 700), [sC]
     ta.cp_set_atoms(cp_atoms(), 0.0)
     g = torch.zeros((32, 512), device="cuda:0")
     return ta.ori_cp_create(64, 0.1, g), ta.cp_blocks(512, 32), [g]
 
 
-@pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),
-                                          ("lbm", "stencil"), ("mriq", "stencil"), ("cp", "mrif"), ("lbm", "mrif"),
-                                          ("mrif", "mriq"), ("mrif", "stencil")])
+def sgemm_inputs():
+    rng = np.random.default_rng(35)
+    return (rng.uniform(0, 1, (700, 256)).astype(np.float32), rng.uniform(0, 1, (700, 48)).astype(np.float32),
+            rng.uniform(-1, 1, (48, 256)).astype(np.float32))
+
+
+BE_PAIRS = [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"), ("lbm", "stencil"), ("mriq", "stencil"),
+            ("cp", "mrif"), ("lbm", "mrif"), ("mrif", "mriq"), ("mrif", "stencil"), ("cp", "sgemm"), ("lbm", "sgemm"),
+            ("mrif", "sgemm"), ("mriq", "sgemm"), ("sgemm", "stencil")]
+
+
+@pytest.mark.parametrize("first,second", BE_PAIRS)
 @pytest.mark.parametrize("variant", [None, "wg_1_2", "wg_2_1", "ord_1_1", "ord_1_2"])
 def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
     ori1, n1, outs1 = _small_be(first)
@@ -781,6 +794,8 @@ def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
     outs = outs1 + outs2
     before = [o.clone() for o in outs]
     r1 = (1, n1 - 1) if n1 > 2 else (0, n1)          # a partial range of the first kernel
+    if first == "sgemm":
+        r1 = (0, n1 - 1)    # its later k parts continue from the workspace, which only part 0 resets: start there
     g1 = ta.gptb_create(ori1, 0, 0, r1[0], r1[1])
     g2 = ta.gptb_create(ori2, 0, 0, 0, n2)
     g1.execute()
@@ -814,13 +829,13 @@ def _small_be_matches_oracle(name, outs):
         k, phi, d, xyz = mrif_inputs(256, 2048, seed=34)
         tr, ti = oracle.mrif(mrif_table(k, phi, d), xyz[0], xyz[1], xyz[2], zq, zq, f64=True)
         return mriq_close(host(outs[0]), tr.astype(np.float64)) and mriq_close(host(outs[1]), ti.astype(np.float64))
+    if name == "sgemm":
+        return np.array_equal(host(outs[0]).view(np.uint32), oracle.sgemm(*sgemm_inputs()).view(np.uint32))
     want = oracle.cp(oracle.cp_atoms_to_const(cp_atoms(), 0.0), np.zeros((32, 512), np.float32))
     return np.array_equal(host(outs[0]).view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("first,second", [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"),
-                                          ("lbm", "stencil"), ("mriq", "stencil"), ("cp", "mrif"), ("lbm", "mrif"),
-                                          ("mrif", "mriq"), ("mrif", "stencil")])
+@pytest.mark.parametrize("first,second", BE_PAIRS)
 def test_best_effort_pairs_full_ranges_match_the_oracle(first, second):
     ori1, n1, outs1 = _small_be(first)
     ori2, n2, outs2 = _small_be(second)
