@@ -77,6 +77,8 @@ def pair_leg(ta, torch, np, name, stream):
         return ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, tiles), tiles, 2.0 * M * N * K
 
     swap = None             # exchanges the best-effort kernel's input and output grid after a launch
+    reset = None            # puts the best-effort kernel's output back to its start before a timed round
+    n = 200                 # launches per timed round
     if name == "cp":        # Coulomb potential, 4096x4096 grid, 64 atoms (the Creator's instance, src/Creator.cu:23-37)
         volx = voly = 4096
         atoms = ta.cp_initatoms(4000, volx, voly, 1, 0.1)
@@ -87,6 +89,18 @@ def pair_leg(ta, torch, np, name, stream):
         tz, tiles, flop = gemm(2048, 2048, 2048)
         work = {"bound": "valu", "pairs": 64.0 * volx * voly}
         label = "tzgemm 2048^3 + cp 4096x4096, 64 atoms (reference mix tzgemm_cp; named by the north star)"
+    elif name == "sgemm":   # Parboil SGEMM, 4096 x 4128 x 4064 (the Creator's instance, src/ori_kernel/sgemm_kernel.cu:86-88)
+        sM, sN, sK = 4096, 4128, 4064
+        sA = torch.rand((sK, sM), device="cuda:0")
+        sB = torch.rand((sK, sN), device="cuda:0")
+        sC = torch.zeros((sN, sM), device="cuda:0")
+        be_ori = ta.ori_sgemm_create(sA, sB, sC)
+        nblk = ta.sgemm_blocks(sM, sN, sK)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "valu", "pairs": float(sM) * sN * sK}
+        label = "tzgemm 2048^3 + sgemm 4096x4128x4064 fp32 (reference mix tzgemm_sgemm)"
+        reset = sC.zero_        # C = 2 C + 2 A B doubles with every pass: start every timed round from zero
+        n = 50
     elif name == "lbm":     # D3Q19, 120x120x150, rest equilibrium + noise, 5 % obstacle cells
         sx, sy, sz = 120, 120, 150
         cells = sx * sy * sz
@@ -140,10 +154,11 @@ def pair_leg(ta, torch, np, name, stream):
     be_slice = ta.gptb_create(be_ori, 0, 0, 0, max(slice_blocks, 1))
     mix_slice = ta.mix_create(be, tz, 0, slice_blocks, 0, tiles)
     e0, e1 = ta.Event(), ta.Event()
-    n = 200
 
     def timed(fn):
         nonlocal n
+        if reset:
+            reset()
         torch.cuda.synchronize()
         e0.record(stream)
         for _ in range(n):
@@ -202,7 +217,7 @@ def pair_leg(ta, torch, np, name, stream):
                 tz.execute(stream)
             be.execute(stream)
 
-        n = 40
+        n = 40 if n_cur <= 30 else 10
         cur = {"cursor_serial_us": [], "cursor_fused_us": []}
         for _ in range(3):
             cur["cursor_serial_us"].append(timed(cursor_serial))
@@ -429,7 +444,8 @@ def main():
     }
     if not args.no_extras:
         out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
-        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in ("lbm", "mriq", "cp", "mrif")}
+        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream)
+                              for name in ("lbm", "mriq", "cp", "mrif", "sgemm")}
         if not args.no_lc:
             out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")

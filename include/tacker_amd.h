@@ -516,6 +516,7 @@ TK_API int tacker_task_manager_latencies(tacker_task_manager_t tm, int which, fl
 
 /* the scheduler's arithmetic on its own (src/TaskManager.cu:586-640) */
 TK_API float tacker_qos_block_ratio(const char *be_name, int K_GLOBAL);
+/* mode: 0 = Aker, 1 = Tacker (enum ExecutionMode) */
 TK_API int tacker_qos_colocated_blocks(int mode, const char *be_name, int tiles, int K_GLOBAL,
                                        int be_total_blocks);
 TK_API int tacker_qos_must_run_solo(float budget_ms, float guard_ms, float qos_headroom,

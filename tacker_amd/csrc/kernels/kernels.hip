@@ -95,8 +95,9 @@ extern "C" __global__ __launch_bounds__(128) void ori_sgemm(float *A, float *B, 
                                                             int NORMAL_K)
 {
     const int mid = threadIdx.y * blockDim.x + threadIdx.x;
+    __shared__ __align__(16) float stage[2][64];
     tk::sgemm_thread(A, B, C, nullptr, NORMAL_M, NORMAL_N, NORMAL_K, blockIdx.x * SGEMM_TILE_M + mid,
-                     blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K);
+                     blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K, (tk::sgemm_lds_float *)&stage[mid >> 6][0]);
 }
 
 // grid (volx/128, voly/8), block (16,8)
@@ -208,7 +209,7 @@ extern "C" __global__ void general_ptb_mrif(int numK, int kGlobalIndex, float *x
 }
 
 // src/gptb_kernel/sgemm_kernel.cu:3-6
-extern "C" __global__ void general_ptb_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N, int NORMAL_K,
+extern "C" __global__ __launch_bounds__(256) void general_ptb_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N, int NORMAL_K,
                                              GPTB_TRAILER)
 {
     tk::sgemm_role(A, B, C, NORMAL_M, NORMAL_N, NORMAL_K, grid_dimension_x, grid_dimension_y, grid_dimension_z,

@@ -9,12 +9,15 @@
 // alpha = beta = 2 (both products exact, so every way of contracting that line gives one result).
 //
 // gfx950: the reference stages an 8 x 16 tile of B in shared memory behind two barriers per 8 k
-// steps.  Every thread of a block reads the same 16 values of B per k, so here they are
-// wave-uniform scalar loads (64 bytes per k row, 64-byte aligned because N is a multiple of 16)
-// and the multiply-adds take them as scalar operands: per k step a wave issues one coalesced
-// load of A and 16 v_fmac_f32 -- no LDS, no barrier, and the role drops into the wave-split fused
-// kernels like the other vector roles.  The work is bound by the vector ALUs (64 cycles per k
-// step and wave).
+// steps, shared by the block's 4 warps.  Here every wave stages its own copy -- 4 k rows x 16
+// columns = one float per lane, fetched with one vector load an iteration ahead, written to a
+// 256-byte slot of LDS and read back as 16 broadcast reads of 16 bytes -- so a wave is its own
+// synchronisation domain: no barrier, and the role drops into the wave-split fused kernels like
+// the other vector roles (it adds 4 KiB of LDS to a kernel).  Per 4 k steps a wave issues two
+// vector loads, one LDS write, 16 LDS reads and 64 v_fmac_f32; the work is bound by the vector
+// ALUs (64 cycles per k step and wave).  Fetching the rows of B with scalar loads instead (they
+// are wave-uniform) was measured first and ran 4.8 times slower: every k row is another 64-byte
+// line, and the scalar cache serves its misses one after the other.
 //
 // Block positions.  A block's whole k loop is long (K = 4064: 4064 x 64 cycles, 110 us), so the
 // GPTB position grid has a third dimension through the reference's own index reconstruction
@@ -34,10 +37,14 @@
 
 namespace tk {
 
-// thread's row m, columns n0 .. n0 + 15, k in [k_begin, k_end); n0, k_begin, k_end wave-uniform
+typedef __attribute__((address_space(3))) float sgemm_lds_float;
+typedef __attribute__((address_space(3))) float4_t sgemm_lds_float4;
+
+// thread's row m, columns n0 .. n0 + 15, k in [k_begin, k_end); n0, k_begin, k_end wave-uniform;
+// stage: this wave's 64 floats of LDS
 __device__ __forceinline__ void sgemm_thread(const float *__restrict__ A, const float *__restrict__ B,
                                              float *__restrict__ C, float *__restrict__ W, int M, int N, int K,
-                                             int m, int n0, int k_begin, int k_end)
+                                             int m, int n0, int k_begin, int k_end, sgemm_lds_float *stage)
 {
     float c[SGEMM_TILE_N];
     const size_t t = (size_t)M * n0 + m;   // of C and of the workspace: column n0, row m
@@ -48,38 +55,92 @@ __device__ __forceinline__ void sgemm_thread(const float *__restrict__ A, const 
 #pragma unroll
         for (int i = 0; i < SGEMM_TILE_N; ++i) c[i] = W[t + (size_t)i * M];
     }
-    const float *a_at = A + (size_t)k_begin * M + m;
-    const float *b_at = B + (size_t)k_begin * N + n0;   // the same address in every lane
+    const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));   // whatever the block shape
+    // 32-bit element indices (the host refuses matrices of 2^31 elements): fewer scalar registers
+    // for the strides than 64-bit byte offsets take, which matters inside a fused kernel
+    int a_at = k_begin * M + m;
+    // lane l fetches B[k + l / 16][n0 + l % 16]: the 4 x 16 values of four k steps
+    int b_at = (k_begin + (lane >> 4)) * N + n0 + (lane & 15);
     int k = k_begin;
-    // four k steps per iteration; the next iteration's values of A are on their way while this
-    // one's are used (the rows of B arrive by scalar loads at the top of the iteration)
-#define SGEMM_FOUR_STEPS(a_)                                                                      \
-    _Pragma("unroll") for (int j = 0; j < 4; ++j) _Pragma("unroll") for (int i = 0; i < SGEMM_TILE_N; ++i)  \
-        c[i] = __builtin_fmaf(a_[j], b_at[(size_t)j * N + i], c[i]);                              \
-    a_at += (size_t)4 * M;                                                                        \
-    b_at += (size_t)4 * N;
-    if (k + 4 <= k_end) {
-        float a[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) a[j] = a_at[(size_t)j * M];
-        for (; k + 8 <= k_end; k += 4) {
-            float a_next[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) a_next[j] = a_at[(size_t)(4 + j) * M];
-            SGEMM_FOUR_STEPS(a)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) a[j] = a_next[j];
-        }
-        SGEMM_FOUR_STEPS(a)
-        k += 4;
+    // four k steps per iteration; the next iteration's values of A and B are on their way while
+    // this one's are used
+#define SGEMM_FOUR_STEPS(a_, b_)                                                                  \
+    {                                                                                             \
+        /* the wave's previous reads of the slot are behind it: LDS serves a wave in order */     \
+        stage[lane] = b_;                                                                         \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                    \
+        __builtin_amdgcn_wave_barrier();                                                          \
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                    \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j)                                             \
+        {                                                                                         \
+            float4_t bv[SGEMM_TILE_N / 4];   /* row k + j of the tile */                          \
+            _Pragma("unroll") for (int q = 0; q < SGEMM_TILE_N / 4; ++q)                          \
+                bv[q] = *reinterpret_cast<const sgemm_lds_float4 *>(stage + SGEMM_TILE_N * j + 4 * q); \
+            _Pragma("unroll") for (int i = 0; i < SGEMM_TILE_N; ++i)                              \
+                c[i] = __builtin_fmaf(a_[j], bv[i / 4][i % 4], c[i]);                             \
+        }                                                                                         \
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                    \
+        __builtin_amdgcn_wave_barrier();                                                          \
     }
+// every register set walks its own index, 16 k steps at a time: the only strides are M, 2 M,
+// 3 M, 16 M and 16 N, which keeps the scalar registers of a fused kernel within reach
+#define SGEMM_FETCH(a_, b_, ia_, ib_)                                                             \
+    _Pragma("unroll") for (int j = 0; j < 4; ++j) a_[j] = A[(ia_) + j * M];                       \
+    b_ = B[ib_];                                                                                  \
+    ia_ += 16 * M;                                                                                \
+    ib_ += 16 * N;
+    if (k + 4 <= k_end) {
+        // Four register sets take turns: the values of an iteration are fetched four iterations
+        // (16 k steps, a thousand cycles of this wave's own arithmetic) before they are used, so
+        // that a wave with a SIMD to itself -- a short slice next to a GEMM -- is bound by the ALUs
+        // and not by the round trip to the L2.
+        float a0[4], a1[4], a2[4], a3[4], b0, b1, b2, b3;
+        int ia0 = a_at, ia1 = a_at + 4 * M, ia2 = a_at + 8 * M, ia3 = a_at + 12 * M;
+        int ib0 = b_at, ib1 = b_at + 4 * N, ib2 = b_at + 8 * N, ib3 = b_at + 12 * N;
+        const int n_iter = (k_end - k) >> 2;
+        SGEMM_FETCH(a0, b0, ia0, ib0)
+        if (n_iter > 1) { SGEMM_FETCH(a1, b1, ia1, ib1) }
+        if (n_iter > 2) { SGEMM_FETCH(a2, b2, ia2, ib2) }
+        if (n_iter > 3) { SGEMM_FETCH(a3, b3, ia3, ib3) }
+        int it = 0;
+        for (; it + 8 <= n_iter; it += 4) {
+            SGEMM_FOUR_STEPS(a0, b0)
+            SGEMM_FETCH(a0, b0, ia0, ib0)
+            SGEMM_FOUR_STEPS(a1, b1)
+            SGEMM_FETCH(a1, b1, ia1, ib1)
+            SGEMM_FOUR_STEPS(a2, b2)
+            SGEMM_FETCH(a2, b2, ia2, ib2)
+            SGEMM_FOUR_STEPS(a3, b3)
+            SGEMM_FETCH(a3, b3, ia3, ib3)
+        }
+        // at most seven iterations left: those in the sets, then those fetched meanwhile
+        const int left = n_iter - it;
+        SGEMM_FOUR_STEPS(a0, b0)
+        if (left > 4) { SGEMM_FETCH(a0, b0, ia0, ib0) }
+        if (left > 1) {
+            SGEMM_FOUR_STEPS(a1, b1)
+            if (left > 5) { SGEMM_FETCH(a1, b1, ia1, ib1) }
+        }
+        if (left > 2) {
+            SGEMM_FOUR_STEPS(a2, b2)
+            if (left > 6) { SGEMM_FETCH(a2, b2, ia2, ib2) }
+        }
+        if (left > 3) { SGEMM_FOUR_STEPS(a3, b3) }
+        if (left > 4) { SGEMM_FOUR_STEPS(a0, b0) }
+        if (left > 5) { SGEMM_FOUR_STEPS(a1, b1) }
+        if (left > 6) { SGEMM_FOUR_STEPS(a2, b2) }
+        k += 4 * n_iter;
+        a_at += 4 * n_iter * M;
+    }
+#undef SGEMM_FETCH
 #undef SGEMM_FOUR_STEPS
+    // what is left of a k range that is not a multiple of four: values of B by scalar loads
     for (; k < k_end; ++k) {
-        const float av = *a_at;
+        const float av = A[a_at];
+        const float *b_row = B + (size_t)k * N + n0;
 #pragma unroll
-        for (int i = 0; i < SGEMM_TILE_N; ++i) c[i] = __builtin_fmaf(av, b_at[i], c[i]);
+        for (int i = 0; i < SGEMM_TILE_N; ++i) c[i] = __builtin_fmaf(av, b_row[i], c[i]);
         a_at += M;
-        b_at += N;
     }
     if (k_end == K) {
 #pragma unroll
@@ -90,20 +151,28 @@ __device__ __forceinline__ void sgemm_thread(const float *__restrict__ A, const 
     }
 }
 
+// the LDS slot of the calling wave: 64 floats per wave of a workgroup of up to 1024 threads
+__device__ __forceinline__ sgemm_lds_float *sgemm_stage_of_wave()
+{
+    __shared__ __align__(16) float sgemm_stage[16][64];
+    return (sgemm_lds_float *)&sgemm_stage[threadIdx.x >> 6][0];
+}
+
 // One phase of a launch: blocks [block_lo, block_hi) (block = block_x + grid_x block_y) each take
 // k in [k_begin, k_end).  A thread group serves the blocks it owns: first_owned, first_owned +
 // stride, ...
 __device__ __forceinline__ void sgemm_phase(int block_lo, int block_hi, int k_begin, int k_end,
                                             const float *__restrict__ A, const float *__restrict__ B,
                                             float *__restrict__ C, float *__restrict__ W, int M, int N, int K,
-                                            int grid_x, int first_owned, int stride, int t)
+                                            int grid_x, int first_owned, int stride, int t, sgemm_lds_float *stage)
 {
     if (block_lo >= block_hi || k_begin >= k_end) return;
     int b = first_owned;
     if (b < block_lo) b += (block_lo - b + stride - 1) / stride * stride;
     for (; b < block_hi; b += stride) {
         const int bu = __builtin_amdgcn_readfirstlane(b);   // the 128 threads of a group are whole waves
-        sgemm_thread(A, B, C, W, M, N, K, (bu % grid_x) * SGEMM_TILE_M + t, (bu / grid_x) * SGEMM_TILE_N, k_begin, k_end);
+        sgemm_thread(A, B, C, W, M, N, K, (bu % grid_x) * SGEMM_TILE_M + t, (bu / grid_x) * SGEMM_TILE_N, k_begin, k_end,
+                     stage);
     }
 }
 
@@ -126,6 +195,7 @@ __device__ __forceinline__ void sgemm_role(const float *__restrict__ A, const fl
     const auto chunk_begin = [&](int row) { return min((row % gy) * chunk, K); };
     const auto chunk_end = [&](int row) { return (row % gy) == gy - 1 ? K : min((row % gy + 1) * chunk, K); };
 
+    sgemm_lds_float *stage = sgemm_stage_of_wave();
     float *W = nullptr;
     if (gy > 1) {
         // partial results rest in the workspace bound to C; without one nothing can be computed
@@ -141,13 +211,13 @@ __device__ __forceinline__ void sgemm_role(const float *__restrict__ A, const fl
     const int last_row = (end - 1) / gx;   // row of the last position
     if (first_row == last_row) {
         sgemm_phase(start - first_row * gx, end - first_row * gx, chunk_begin(first_row), chunk_end(first_row), A, B, C,
-                    W, M, N, K, grid_dimension_x, first_owned, stride, t);
+                    W, M, N, K, grid_dimension_x, first_owned, stride, t, stage);
         return;
     }
     int row = first_row;
     if (start != first_row * gx) {   // partial first row
         sgemm_phase(start - first_row * gx, gx, chunk_begin(row), chunk_end(row), A, B, C, W, M, N, K, grid_dimension_x,
-                    first_owned, stride, t);
+                    first_owned, stride, t, stage);
         ++row;
     }
     const int whole_end = (end == (last_row + 1) * gx) ? last_row + 1 : last_row;   // whole rows [row, whole_end)
@@ -155,12 +225,12 @@ __device__ __forceinline__ void sgemm_role(const float *__restrict__ A, const fl
         // rows up to the next multiple of the part count are consecutive k parts: one run of the k loop
         const int run_end = min(whole_end, (row / gy + 1) * gy);
         sgemm_phase(0, gx, chunk_begin(row), chunk_end(run_end - 1), A, B, C, W, M, N, K, grid_dimension_x, first_owned,
-                    stride, t);
+                    stride, t, stage);
         row = run_end;
     }
     if (whole_end == last_row)       // partial last row
         sgemm_phase(0, end - last_row * gx, chunk_begin(last_row), chunk_end(last_row), A, B, C, W, M, N, K,
-                    grid_dimension_x, first_owned, stride, t);
+                    grid_dimension_x, first_owned, stride, t, stage);
 }
 
 }  // namespace tk

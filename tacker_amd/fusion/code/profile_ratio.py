@@ -16,7 +16,8 @@ Method per (pair, K): GEMM 2048 x 2048 x K (1024 tiles, one 128x128 macro tile p
 t0 = fused launch with no best-effort block, t_be = the best-effort kernel alone (all N
 blocks).  For nb on a ladder of block counts, earned(nb) = t0 + t_be * nb / N - t_fused(nb)
 is the time one fused launch saves over the two serial launches (the quantity TaskManager
-credits, src/TaskManager.cu:626-640).  The ratio is nb / 1024 for the nb with the largest
+credits, src/TaskManager.cu:626-640); the ladder runs N/1024, N/512, ..., N/64, then N/32, 2N/32, ..., N
+and stops once a launch is twice as long as allowed.  The ratio is nb / 1024 for the nb with the largest
 earned time among those whose launch stays within (1 + stretch) * t0, i.e. the
 latency-critical GEMM is never stretched by more than that factor; 0 if nothing earns.
 """
@@ -30,9 +31,16 @@ ROOT = os.path.abspath(os.path.join(HERE, "..", "..", ".."))
 DEFAULTS = os.path.join(HERE, "defaults.json")
 # reduction lengths of the VGG16 batch-1 layers after padding to 128, plus the benchmark's
 K_LADDER = (128, 640, 1152, 2048, 2304, 4096, 4608)
-PAIRS = ("stencil", "lbm", "mriq", "cp", "mrif")
+PAIRS = ("stencil", "lbm", "mriq", "cp", "mrif", "sgemm")
 TILES = 1024
-LADDER = 32          # best-effort block counts tried: N/32, 2N/32, ..., N
+LADDER = 32          # best-effort block counts tried: N/1024, N/512, ..., N/64, then N/32, 2N/32, ..., N
+
+
+def ladder(be_total):
+    """ascending block counts: a geometric run-up for kernels whose 1/32 is already longer than a GEMM
+    (sgemm: 2 ms for 132096 positions), then the linear ladder"""
+    counts = {be_total >> j for j in range(6, 11)} | {be_total * step // LADDER for step in range(1, LADDER + 1)}
+    return sorted(c for c in counts if c > 0)
 
 
 def measure(out_path, stretch, launches, pairs=PAIRS):
@@ -68,13 +76,14 @@ def measure(out_path, stretch, launches, pairs=PAIRS):
             mix = ta.mix_create(be, tz, 0, 0, 0, TILES)
             t0 = timed(mix)
             best = {"blocks": 0, "earned_us": 0.0, "fused_us": t0}
-            for step in range(1, LADDER + 1):
-                nb = be_total * step // LADDER
+            for nb in ladder(be_total):
                 mix.set_range(0, nb, 0, TILES)
                 t = timed(mix)
                 earned = t0 + be_us * nb / be_total - t
                 if t <= (1 + stretch) * t0 and earned > best["earned_us"]:
                     best = {"blocks": nb, "earned_us": earned, "fused_us": t}
+                if t > 2 * (1 + stretch) * t0:      # more blocks only make the launch longer
+                    break
             table[str(K)] = {"blocks": best["blocks"], "ratio": round(best["blocks"] / TILES, 4),
                              "gemm_in_fused_us": round(t0, 2), "fused_us": round(best["fused_us"], 2),
                              "earned_us": round(best["earned_us"], 2)}
@@ -94,6 +103,8 @@ def apply(in_path):
     with open(DEFAULTS) as f:
         dflt = json.load(f)
     for key, m in meas["pairs"].items():
+        if key not in dflt:
+            raise SystemExit(f"{DEFAULTS} has no entry {key}: add the pair to the generator first")
         entry = dflt[key]
         entry["ratio_by_k"] = {k: v["ratio"] for k, v in m["by_k"].items()}
         entry["block_ratio"] = m["by_k"]["4096"]["ratio"]
@@ -103,7 +114,7 @@ def apply(in_path):
                                           "stays within (1+stretch) of the launch without best-effort "
                                           "blocks, divided by 1024 tiles"}
     with open(DEFAULTS, "w") as f:
-        json.dump(dflt, f, indent=4)
+        json.dump(dflt, f, indent=2)
         f.write("\n")
     print("updated", DEFAULTS, "- now run gen_run.py and rebuild")
 

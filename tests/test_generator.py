@@ -133,3 +133,51 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
         # parameter order: the first kernel's list, then the second's
         assert text.index(f"{a}0_grid_dimension_x") < text.index(f"{b}1_grid_dimension_x")
     assert "__shared__" not in files["mix_kernel/lbm_mriq.hip"]        # no role of a pair uses LDS
+
+
+def test_measured_load_ratios_travel_from_profile_ratio_to_the_schedulers_lookup(tmp_path, monkeypatch):
+    # profile_ratio.py --apply -> defaults.json -> gen_run.py -> kinfo json -> QosPolicy::blockRatio
+    # (src/TaskManager.cu:593-598), on copies of the files, the last step in a fresh process over the
+    # recording device layer
+    import shutil
+    import profile_ratio
+    dflt = tmp_path / "defaults.json"
+    shutil.copy(os.path.join(GEN, "defaults.json"), dflt)
+    monkeypatch.setattr(profile_ratio, "DEFAULTS", str(dflt))
+    monkeypatch.setattr(gen_run, "DEFAULTS_PATH", str(dflt))
+    ladder = profile_ratio.ladder(132096)
+    assert ladder[0] == 129 and ladder[-1] == 132096 and ladder == sorted(set(ladder)) and len(ladder) == 37
+    meas = {"stretch": 0.5, "tiles": 1024, "device": "test double",
+            "pairs": {"tzgemm_sgemm": {"be_total_blocks": 132096, "be_solo_us": 2000.0,
+                                       "by_k": {str(k): {"blocks": 1024 * i, "ratio": float(i) + 0.25}
+                                                for i, k in enumerate(profile_ratio.K_LADDER)}}}}
+    src = tmp_path / "measured.json"
+    src.write_text(json.dumps(meas))
+    before = json.loads(dflt.read_text())
+    profile_ratio.apply(str(src))
+    after = json.loads(dflt.read_text())
+    assert after["tzgemm_sgemm"]["ratio_by_k"] == {"128": 0.25, "640": 1.25, "1152": 2.25, "2048": 3.25, "2304": 4.25,
+                                                   "4096": 5.25, "4608": 6.25}
+    assert after["tzgemm_sgemm"]["block_ratio"] == 5.25 and after["ratio_provenance"]["stretch"] == 0.5
+    assert after["tzgemm_stencil"] == before["tzgemm_stencil"]          # pairs that were not measured keep theirs
+    with pytest.raises(SystemExit):                                    # a pair the generator does not know
+        bad = tmp_path / "bad.json"
+        bad.write_text(json.dumps({"stretch": 1.0, "device": "x", "pairs": {"tzgemm_fft": {"by_k": {}}}}))
+        profile_ratio.apply(str(bad))
+    kinfo_text = gen_run.generate()["../config/kinfo-gfx950.json"]
+    kinfo = json.loads(kinfo_text)
+    assert kinfo["tzgemm_sgemm"]["block_ratio"] == 5.25 and kinfo["tzgemm_sgemm"]["1152"] == 2.25
+    kinfo_path = tmp_path / "kinfo.json"
+    kinfo_path.write_text(kinfo_text)
+    code = ("import sys, ctypes as C; sys.path.insert(0, %r); import tacker_amd as ta; "
+            "l = ta.load_library(ta.FAKE_LIB_PATH); assert l.tacker_init(0, %r.encode()) == 0; "
+            "l.tacker_qos_block_ratio.restype = C.c_float; "
+            "print(l.tacker_qos_block_ratio(b'sgemm', 1152), l.tacker_qos_block_ratio(b'sgemm', 4096), "
+            "l.tacker_qos_block_ratio(b'sgemm', 8192), l.tacker_qos_colocated_blocks(0, b'sgemm', 1024, 2304, 132096))"
+            % (ROOT, str(kinfo_path)))
+    rc = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True)
+    assert rc.returncode == 0, rc.stdout + rc.stderr
+    got = rc.stdout.strip().splitlines()[-1].split()     # the library's log lines come first
+    # a K of the table, the base entry, linear extrapolation from 4096 beyond the table, and the block count
+    # Aker mode gives a 1024-tile GEMM of K = 2304: tiles x ratio
+    assert [float(v) for v in got[:3]] == [2.25, 5.25, 10.5] and int(got[3]) == int(1024 * 4.25)
