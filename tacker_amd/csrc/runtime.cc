@@ -65,6 +65,7 @@ namespace {
 struct BoundWorkspace {
     void *ptr;
     long long bytes;
+    bool zero_at_rest;   // only kernels that hand it back all zero (tzgemm's counters) have used it
 };
 std::mutex g_workspace_mutex;
 std::unordered_map<const void *, BoundWorkspace> g_workspaces;   // by output buffer
@@ -91,13 +92,25 @@ void publish_workspace(const void *C, void *workspace)
 }
 }  // namespace
 
-// a device buffer of at least `need` zeroed bytes bound to the output buffer C
-static void *workspaceFor(const void *C, long long need)
+// A device buffer of at least `need` bytes bound to the output buffer C.  keeps_zero: the asking
+// kernel needs it zero and leaves it zero (tzgemm's arrival counters); sgemm writes its partial sums
+// before it reads them and leaves them there, so a buffer it has used is cleared again before a
+// kernel of the first kind gets it (an output address the caller's allocator handed out twice).
+static void *workspaceFor(const void *C, long long need, bool keeps_zero)
 {
     if (need == 0 || C == nullptr) return nullptr;
     std::lock_guard<std::mutex> lock(g_workspace_mutex);
     auto it = g_workspaces.find(C);
-    if (it != g_workspaces.end() && it->second.bytes >= need) return it->second.ptr;
+    if (it != g_workspaces.end() && it->second.bytes >= need) {
+        if (keeps_zero && !it->second.zero_at_rest) {
+            TK_SAFE_CALL(tkDeviceSynchronize());   // the kernels that wrote it are done
+            TK_SAFE_CALL(tkMemset(it->second.ptr, 0, (size_t)it->second.bytes));
+            TK_SAFE_CALL(tkDeviceSynchronize());
+            it->second.zero_at_rest = true;
+        }
+        if (!keeps_zero) it->second.zero_at_rest = false;
+        return it->second.ptr;
+    }
     if (it == g_workspaces.end() && g_workspaces.size() >= kMaxBoundWorkspaces)
         throw std::runtime_error("tzgemm: " + std::to_string(kMaxBoundWorkspaces) +
                                  " output buffers hold a workspace; call tzgemmReleaseWorkspaces() once the "
@@ -114,18 +127,18 @@ static void *workspaceFor(const void *C, long long need)
         throw;
     }
     if (it != g_workspaces.end()) g_outgrown_workspaces.push_back(it->second.ptr);
-    g_workspaces[C] = BoundWorkspace{ptr, need};
+    g_workspaces[C] = BoundWorkspace{ptr, need, keeps_zero};
     return ptr;
 }
 
 void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL)
 {
-    return workspaceFor(C, tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL));
+    return workspaceFor(C, tz_workspace_bytes(M_GLOBAL, N_GLOBAL, K_GLOBAL), true);
 }
 
 void *sgemmWorkspaceFor(const float *C, int M, int N)
 {
-    return workspaceFor(C, (long long)M * N * (long long)sizeof(float));
+    return workspaceFor(C, (long long)M * N * (long long)sizeof(float), false);
 }
 
 void tzgemmReleaseWorkspaces()

@@ -139,3 +139,31 @@ def test_creator_object_at_the_reference_size_matches_the_oracle_on_sampled_bloc
         assert np.array_equal(got[cols, rows].view(np.uint32), want[cols, rows].view(np.uint32)), blk
     assert np.count_nonzero(got) == got.size
     assert ta.spin_fail_flag() == 0
+
+
+def test_an_output_address_sgemm_has_used_serves_a_shared_reduction_tzgemm_afterwards():
+    # sgemm leaves partial sums in the workspace bound to its C; tzgemm's shared reduction counts
+    # arrivals there and needs them zero: the binding is cleared when the kind of kernel changes
+    M, N, K = 256, 512, 4608
+    assert ta.tzgemm_parts(M, N, K) > 1
+    buf = torch.zeros(M * N, device="cuda:0")
+    A, B, C0 = inputs(256, 512, 600, seed=9)
+    c_s = buf.view(512, 256)
+    c_s.copy_(dev(C0))
+    ta.gptb_sgemm(dev(A), dev(B), c_s)
+    assert np.array_equal(bits(c_s), oracle.sgemm(A, B, C0).view(np.uint32))
+    gA, gB = gemm_inputs(M, N, K, 77)
+    dA, dB = dev(gA), dev(gB)
+    c_t = buf.view(M, N)
+    assert c_t.data_ptr() == c_s.data_ptr()
+    c_t.fill_(-7.0)
+    other = torch.full((M, N), -7.0, device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, other)
+    ta.gptb_tzgemm(dA, dB, c_t)
+    assert np.array_equal(host(c_t), host(other))
+    assert (host(c_t) != -7.0).all()
+    # and back: sgemm on the address tzgemm has used
+    c_s.copy_(dev(C0))
+    ta.gptb_sgemm(dev(A), dev(B), c_s)
+    assert np.array_equal(bits(c_s), oracle.sgemm(A, B, C0).view(np.uint32))
+    assert ta.spin_fail_flag() == 0
