@@ -110,15 +110,9 @@ extern "C" __global__ __launch_bounds__(128) void ori_cp(int numatoms, float gri
 
 // ------------------------------------------------------------------ GPTB kernels
 
-extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1))) void general_ptb_tzgemm(
-    _Float16 *A, _Float16 *B, float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL, GPTB_TRAILER)
-{
-    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
-    tk::WorkgroupSync sync;
-    tk::tzgemm_role<TZ_STAGES>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, tk::tz_workspace_of(C, M_GLOBAL, N_GLOBAL, K_GLOBAL),
-                    (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
-                    (int)threadIdx.x - thread_base, tz_lds, sync);
-}
+// general_ptb_<kernel> (g_general_ptb_ for mriq and cp): written by fusion/code/gen_run.py from the
+// same role descriptions as the fused kernels
+#include "../gptb_kernel/gptb_kernels.inc"
 
 // ---- tzgemm for callers that cannot allocate device memory --------------------------------
 // The same role with its workspace handed in as an argument, and the workspace itself: a
@@ -173,56 +167,6 @@ extern "C" int tk_tzgemm_scratch(void **ptr, size_t *bytes)
     *ptr = g_scratch_address[device];
     *bytes = sizeof(scratch);
     return TK_SUCCESS;
-}
-
-extern "C" __global__ __launch_bounds__(256) void general_ptb_stencil(float c0, float c1, float *A0, float *Anext, int nx,
-                                               int ny, int nz, GPTB_TRAILER)
-{
-    tk::stencil_role(c0, c1, A0, Anext, nx, ny, nz, grid_dimension_x, grid_dimension_y, grid_dimension_z,
-                     (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
-                     (int)threadIdx.x - thread_base, (int)blockDim.x);
-}
-
-extern "C" __global__ void general_ptb_lbm(float *srcGrid, float *dstGrid, GPTB_TRAILER)
-{
-    tk::lbm_role(srcGrid, dstGrid, grid_dimension_x, grid_dimension_y, block_dimension_x,
-                 (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
-                 (int)threadIdx.x - thread_base, (int)blockDim.x);
-}
-
-extern "C" __global__ void g_general_ptb_mriq(int numK, int kGlobalIndex, float *x, float *y,
-                                              float *z, float *Qr, float *Qi, GPTB_TRAILER)
-{
-    (void)kGlobalIndex;
-    tk::mriq_role(numK, x, y, z, Qr, Qi, grid_dimension_x, grid_dimension_y, (int)blockIdx.x, ptb_iter_block_step,
-                  ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base,
-                  (int)blockDim.x);
-}
-
-extern "C" __global__ void general_ptb_mrif(int numK, int kGlobalIndex, float *x, float *y,
-                                            float *z, float *outR, float *outI, GPTB_TRAILER)
-{
-    (void)kGlobalIndex;
-    tk::mrif_role(numK, x, y, z, outR, outI, grid_dimension_x, grid_dimension_y, (int)blockIdx.x, ptb_iter_block_step,
-                  ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base,
-                  (int)blockDim.x);
-}
-
-// src/gptb_kernel/sgemm_kernel.cu:3-6
-extern "C" __global__ __launch_bounds__(256) void general_ptb_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N, int NORMAL_K,
-                                             GPTB_TRAILER)
-{
-    tk::sgemm_role(A, B, C, NORMAL_M, NORMAL_N, NORMAL_K, grid_dimension_x, grid_dimension_y, grid_dimension_z,
-                   (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
-                   (int)threadIdx.x - thread_base, (int)blockDim.x);
-}
-
-extern "C" __global__ void g_general_ptb_cp(int numatoms, float gridspacing, float *energygrid,
-                                            GPTB_TRAILER)
-{
-    tk::cp_role(numatoms, gridspacing, energygrid, grid_dimension_x, grid_dimension_y, grid_dimension_z,
-                (int)blockIdx.x, ptb_iter_block_step, ptb_start_block_pos, ptb_end_block_pos,
-                (int)threadIdx.x - thread_base, (int)blockDim.x);
 }
 
 // Counts the floats with bit patterns in [lo_bits, hi_bits) for which the short form of
@@ -298,15 +242,8 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ComputeRhoPhiGPU", (const void *)ComputeRhoPhiGPU, ctx);
     insert("ori_mrif", (const void *)ori_mrif, ctx);
     insert("ori_sgemm", (const void *)ori_sgemm, ctx);
-    insert("gptb_tzgemm", (const void *)general_ptb_tzgemm, ctx);
     insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);
     insert("tz_clear_words", (const void *)tz_clear_words, ctx);
-    insert("gptb_stencil", (const void *)general_ptb_stencil, ctx);
-    insert("gptb_lbm", (const void *)general_ptb_lbm, ctx);
-    insert("gptb_mriq", (const void *)g_general_ptb_mriq, ctx);
-    insert("gptb_cp", (const void *)g_general_ptb_cp, ctx);
-    insert("gptb_mrif", (const void *)general_ptb_mrif, ctx);
-    insert("gptb_sgemm", (const void *)general_ptb_sgemm, ctx);
     insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);
     insert("im2col", (const void *)im2col_gpu_kernel_, ctx);
     insert("convert_fp32_to_fp16", (const void *)convertFp32ToFp16_, ctx);
@@ -315,6 +252,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("maxpool2x2_nhwc", (const void *)maxpool2x2_nhwc, ctx);
     insert("pack_fc_input", (const void *)pack_fc_input, ctx);
     insert("pack_fc_input_pooled", (const void *)pack_fc_input_pooled, ctx);
+    tk_register_gptb_kernels(insert, ctx);
     tk_register_mix_kernels(insert, ctx);
     tk_register_large_kernels(insert, ctx);
     return TK_SUCCESS;

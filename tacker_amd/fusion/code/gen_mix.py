@@ -17,7 +17,7 @@ so two forms are emitted:
   reference does; a role that needs a barrier uses an LDS arrival counter
   private to its waves (``tk::RoleSpinSync``).
 """
-from kernel_code import ROLES, signature
+from kernel_code import ROLES, gptb_signature, signature
 
 
 def _params_text(sig_a, sig_b):
@@ -186,6 +186,33 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(
     meta = {"variant": variant, "symbol": name, "blocksize": threads, "group": wgs1 + wgs2,
             "share1": wgs1, "share2": wgs2, "kind": "wg"}
     return text, meta
+
+
+def generate_gptb(name):
+    """The plain GPTB kernel of one role (``src/gptb_kernel/<name>_kernel.cu`` of the reference): the
+    launch's workgroups are the role's persistent workgroups, ``thread_base`` shifts the thread index
+    (src/GPTBKernel.h:30-61).  Returns (text, symbol)."""
+    role = ROLES[name]
+    sig = gptb_signature(name)
+    call = role["call"].format(p="", block="(int)blockIdx.x", blocks="ptb_iter_block_step",
+                               tid="(int)threadIdx.x - thread_base", threads="(int)blockDim.x", extra="",
+                               stages="TZ_STAGES", stream_c="true")
+    symbol = role["gptb"]["symbol"]
+    attributes = role["gptb"]["attributes"] + " " if role["gptb"]["attributes"] else ""
+    setup = ""
+    if name == "tzgemm":
+        setup = ("    __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];\n"
+                 "    tk::WorkgroupSync sync;\n")
+    text = f"""// Generated by fusion/code/gen_run.py -- do not edit.
+// GPTB form of {name} ({role["gptb"]["cite"]}): block positions [ptb_start_block_pos,
+// ptb_end_block_pos) served by the ptb_iter_block_step workgroups of the launch.
+extern "C" __global__ {attributes}void {symbol}(
+    {_params_text(sig, [])})
+{{
+{_void_unused(sig, call)}{setup}    {call}
+}}
+"""
+    return text, symbol
 
 
 def generate_pair(be, candidates):

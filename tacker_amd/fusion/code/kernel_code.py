@@ -10,6 +10,9 @@ device functions.
 
 ``params``   -- (C type, name) in the order of the reference kernel's signature,
                without the 10-int GPTB trailer.
+``gptb``     -- the plain GPTB kernel of the role: its symbol (the reference's names,
+               src/main.cu:108-125: ``g_general_ptb_`` for mriq and cp), attributes in front
+               of ``void`` and the reference file that holds its counterpart.
 ``call``     -- format string of the role call; ``{p}`` is the parameter prefix,
                ``{block}``, ``{blocks}`` the role-local persistent-workgroup id
                and count, ``{tid}`` the role-local thread id, ``{threads}`` the
@@ -22,6 +25,8 @@ GPTB_RANGE = ["ptb_start_block_pos", "ptb_iter_block_step", "ptb_end_block_pos"]
 
 ROLES = {
     "tzgemm": {
+        "gptb": {"symbol": "general_ptb_tzgemm", "cite": "src/gptb_kernel/tzgemm_kernel.cu:430-448",
+                 "attributes": "__launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))"},
         "params": [("_Float16*", "A"), ("_Float16*", "B"), ("float*", "C"),
                    ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K")],
         "needs_sync": True,
@@ -31,6 +36,8 @@ ROLES = {
                  "tz_lds, sync);"),
     },
     "stencil": {
+        "gptb": {"symbol": "general_ptb_stencil", "cite": "src/gptb_kernel/stencil_kernel.cu:3-105",
+                 "attributes": "__launch_bounds__(256)"},
         "params": [("float", "c0"), ("float", "c1"), ("float*", "A0"), ("float*", "Anext"),
                    ("int", "nx"), ("int", "ny"), ("int", "nz")],
         "needs_sync": False,
@@ -39,6 +46,7 @@ ROLES = {
                  "{p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "lbm": {
+        "gptb": {"symbol": "general_ptb_lbm", "cite": "src/gptb_kernel/lbm_kernel.cu:3-178", "attributes": ""},
         "params": [("float*", "srcGrid"), ("float*", "dstGrid")],
         "needs_sync": False,
         "call": ("tk::lbm_role{extra}({p}srcGrid, {p}dstGrid, {p}grid_dimension_x, {p}grid_dimension_y, "
@@ -46,6 +54,7 @@ ROLES = {
                  "{p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "mriq": {
+        "gptb": {"symbol": "g_general_ptb_mriq", "cite": "src/gptb_kernel/mriq_kernel.cu:3-70", "attributes": ""},
         "params": [("int", "numK"), ("int", "kGlobalIndex"), ("float*", "x"), ("float*", "y"),
                    ("float*", "z"), ("float*", "Qr"), ("float*", "Qi")],
         "needs_sync": False,
@@ -54,6 +63,7 @@ ROLES = {
                  "{threads});"),
     },
     "mrif": {
+        "gptb": {"symbol": "general_ptb_mrif", "cite": "src/gptb_kernel/mrif_kernel.cu:6-93", "attributes": ""},
         "params": [("int", "numK"), ("int", "kGlobalIndex"), ("float*", "x"), ("float*", "y"),
                    ("float*", "z"), ("float*", "outR"), ("float*", "outI")],
         "needs_sync": False,
@@ -62,6 +72,8 @@ ROLES = {
                  "{threads});"),
     },
     "sgemm": {
+        "gptb": {"symbol": "general_ptb_sgemm", "cite": "src/gptb_kernel/sgemm_kernel.cu:3-66",
+                 "attributes": "__launch_bounds__(256)"},
         "params": [("float*", "A"), ("float*", "B"), ("float*", "C"),
                    ("int", "NORMAL_M"), ("int", "NORMAL_N"), ("int", "NORMAL_K")],
         "needs_sync": False,
@@ -70,6 +82,7 @@ ROLES = {
                  "{p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "cp": {
+        "gptb": {"symbol": "g_general_ptb_cp", "cite": "src/gptb_kernel/cp_kernel.cu:8-96", "attributes": ""},
         "params": [("int", "numatoms"), ("float", "gridspacing"), ("float*", "energygrid")],
         "needs_sync": False,
         "call": ("tk::cp_role({p}numatoms, {p}gridspacing, {p}energygrid, {p}grid_dimension_x, "
@@ -87,3 +100,11 @@ def signature(name, index):
     out = [(t, prefix + n) for t, n in ROLES[name]["params"]]
     out += [("int", prefix + n) for n in GPTB_DIMS + GPTB_RANGE]
     return prefix, out
+
+
+def gptb_signature(name):
+    """Parameter list of the plain GPTB kernel of role ``name``: ori params, 6 GPTB dims,
+    start/step/end, thread_base (src/GPTBKernel.h:30-61 of the reference appends them in this order)."""
+    out = list(ROLES[name]["params"])
+    out += [("int", n) for n in GPTB_DIMS + GPTB_RANGE + ["thread_base"]]
+    return out

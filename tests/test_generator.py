@@ -96,6 +96,35 @@ def test_emitted_dispatcher_signature(be, n_params):
     assert f"(int)threadIdx.x - 256" in wave
 
 
+@pytest.mark.parametrize("name,symbol,n_params", [
+    ("tzgemm", "general_ptb_tzgemm", 16), ("stencil", "general_ptb_stencil", 17), ("lbm", "general_ptb_lbm", 12),
+    ("mriq", "g_general_ptb_mriq", 17), ("mrif", "general_ptb_mrif", 17), ("cp", "g_general_ptb_cp", 13),
+    ("sgemm", "general_ptb_sgemm", 16)])
+def test_emitted_gptb_kernel_has_the_reference_name_and_parameter_list(name, symbol, n_params):
+    # src/gptb_kernel/<name>_kernel.cu: the original kernel's parameters, then 6 dims, start, step, end,
+    # thread_base (e.g. stencil_kernel.cu:3-5: 7 + 10; the names are what src/main.cu:108-125 registers)
+    text, got_symbol = gen_mix.generate_gptb(name)
+    sig = re.search(r"void (\w+)\(\s*(.*?)\)\s*\{", text, re.S)
+    names = [p.split()[-1] for p in sig.group(2).split(",")]
+    assert sig.group(1) == symbol == got_symbol and len(names) == n_params
+    assert names[-10:] == ["grid_dimension_x", "grid_dimension_y", "grid_dimension_z", "block_dimension_x",
+                           "block_dimension_y", "block_dimension_z", "ptb_start_block_pos", "ptb_iter_block_step",
+                           "ptb_end_block_pos", "thread_base"]
+    assert "(int)threadIdx.x - thread_base" in text and "(int)blockIdx.x, ptb_iter_block_step" in text
+    files = gen_run.generate()
+    assert files[f"gptb_kernel/{name}_kernel.hip"] == text
+    assert f'insert("gptb_{name}", (const void *){symbol}, ctx);' in files["gptb_kernel/gptb_kernels.inc"]
+
+
+def test_gptb_kernels_exist_only_as_generator_output():
+    # the library's translation unit includes the generated files and defines no general_ptb_ kernel of
+    # its own besides the variant of tzgemm whose workspace is an argument
+    text = open(os.path.join(ROOT, "tacker_amd", "csrc", "kernels", "kernels.hip")).read()
+    assert '#include "../gptb_kernel/gptb_kernels.inc"' in text
+    own = re.findall(r"void (g?_?general_ptb_\w+)\(", text)
+    assert own == ["general_ptb_tzgemm_scratch"]
+
+
 def test_kinfo_emitted_for_every_variant():
     kinfo = json.load(open(os.path.join(ROOT, "tacker_amd", "config", "kinfo-gfx950.json")))
     for be in gen_run.BE_KERNELS:
