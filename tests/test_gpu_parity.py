@@ -240,6 +240,42 @@ def test_tzgemm_on_the_global_operand_buffers():
         assert np.array_equal(host(own).view(np.uint32), got.view(np.uint32))
 
 
+def test_a_larger_workspace_replaces_the_bound_one_while_launches_are_queued():
+    # an allocator hands an output address out again for another shape: the workspace bound to it is too
+    # small, a larger one replaces it while launches on the old one are still queued (the old one stays
+    # allocated until the workspaces are released), and both shapes keep giving their own bits
+    ta.tzgemm_release_workspaces()
+    buf = torch.zeros(128 * 8192, device="cuda:0")
+    shapes = [(128, 128, 1024), (256, 512, 4608), (128, 8192, 1024)]
+    assert [ta.tzgemm_workspace_bytes(*s_) for s_ in shapes] == sorted(ta.tzgemm_workspace_bytes(*s_) for s_ in shapes)
+    ops, wants, kernels = [], [], []
+    for i, (M, N, K) in enumerate(shapes):
+        A, B = gemm_inputs(M, N, K, seed=60 + i)
+        ops.append((dev(A), dev(B)))
+        own = torch.zeros((M, N), device="cuda:0")
+        ta.gptb_tzgemm(ops[-1][0], ops[-1][1], own)
+        wants.append(host(own))
+    torch.cuda.synchronize()
+    for i, (M, N, K) in enumerate(shapes):
+        Cv = buf[:M * N].view(M, N)
+        assert Cv.data_ptr() == buf.data_ptr()
+        ori = ta.ori_tzgemm_create(ops[i][0], ops[i][1], Cv)      # binds, or replaces, the workspace of this address
+        g = ta.gptb_create(ori, 0, 0, 0, (M // 64) * (N // 64))
+        kernels.append((ori, g))
+        for _ in range(20):
+            g.execute()                                            # left queued: no synchronisation before the next shape
+    torch.cuda.synchronize()
+    assert np.array_equal(host(buf[:128 * 8192].view(128, 8192)).view(np.uint32), wants[2].view(np.uint32))
+    # the objects of the smaller shapes still work: they find the replacement through the table
+    for i in (0, 1, 2, 0):
+        M, N, K = shapes[i]
+        kernels[i][1].execute()
+        torch.cuda.synchronize()
+        assert np.array_equal(host(buf[:M * N].view(M, N)).view(np.uint32), wants[i].view(np.uint32)), shapes[i]
+    assert ta.spin_fail_flag() == 0
+    ta.tzgemm_release_workspaces()
+
+
 def test_tzgemm_shared_reduction_fused_equals_unfused():
     # conv5's shape with a best-effort kernel in the same launch: same bits as the GEMM alone
     M, N, K = 256, 512, 4608
