@@ -101,8 +101,8 @@ TK_API int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void 
 /* Fills the string-keyed device-function registry (the global `fmap` of
  * src/main.cu:108-159) without the host translation unit including device
  * sources: insert(key, function, ctx) is called once per kernel. Keys on the
- * hot path: ori_{stencil,lbm,mriq,mrif,cp,sgemm}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp,sgemm},
- * tzgemm_{stencil,lbm,mriq,mrif,cp,sgemm}, plus variant keys "<key>@<variant>". */
+ * hot path: ori_{stencil,lbm,mriq,mrif,cp,sgemm,fft}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp,sgemm,fft},
+ * tzgemm_{stencil,lbm,mriq,mrif,cp,sgemm,fft}, plus variant keys "<key>@<variant>". */
 typedef void (*tk_kernel_insert_fn)(const char *key, const void *func, void *ctx);
 TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx);
 
@@ -251,6 +251,18 @@ TK_API int tacker_gptb_sgemm(const float *A, const float *B, float *C, int M, in
                              int block_start, int block_end, int launch_grid, int launch_block,
                              tkStream_t stream);
 
+/* ori_fft / g_general_ptb_fft (src/ori_kernel/fft_kernel.cu:11-61, src/gptb_kernel/fft_kernel.cu:3-75):
+ * `batches` forward transforms of 256 complex points each, radix 2, in place; data holds
+ * batches x 256 (re, im) pairs of floats.  One block position per transform; a position past the
+ * batch wraps (position % batches).  A transform is served by one wavefront (launch_block a
+ * multiple of 64) where the reference launches 128 threads.  Twiddles are correctly rounded table
+ * values: results agree with the reference's within rounding (about 1e-5 absolute for inputs in
+ * [-1, 1]), not bit for bit. */
+#define TACKER_FFT_POINTS 256
+TK_API int tacker_ori_fft(float *data, int batches, tkStream_t stream);
+TK_API int tacker_gptb_fft(float *data, int batches, int block_start, int block_end, int launch_grid,
+                           int launch_block, tkStream_t stream);
+
 /* copyatomstoconstbuf (src/ori_kernel/cp_kernel.cu:159-179): host array of
  * count (<= 64) {x,y,z,q}; z is replaced by (zplane - z)^2 on the way. */
 TK_API int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane);
@@ -314,6 +326,11 @@ TK_API int tacker_mix_tzgemm_sgemm(const float *sA, const float *sB, float *sC, 
                                    int M, int N, int K, int tile_start, int tile_end,
                                    const char *variant, int launch_grid, int launch_block,
                                    tkStream_t stream);
+/* src/mix_kernel/tzgemm_fft.cu */
+TK_API int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_end, const void *A,
+                                 const void *B, float *C, int M, int N, int K, int tile_start,
+                                 int tile_end, const char *variant, int launch_grid, int launch_block,
+                                 tkStream_t stream);
 TK_API int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx,
                                 int voly, int be_start, int be_end, const void *A, const void *B,
                                 float *C, int M, int N, int K, int tile_start, int tile_end,
@@ -336,7 +353,7 @@ TK_API float tacker_fget_kernel_info(const char *kernel, const char *key);
 /* ---- object API: the class layer itself, one handle per C++ object ---------- */
 typedef void *tacker_kernel_t;
 
-/* createKernel (src/Creator.cu:21-337) for the names cp, lbm, mrif, mriq, sgemm, stencil,
+/* createKernel (src/Creator.cu:21-337) for the names cp, fft, lbm, mrif, mriq, sgemm, stencil,
  * tzgemm: the memoised GPTBKernel that owns seeded device buffers exactly as the
  * reference's Ori*Kernel::initParams builds them. Never destroy these. */
 TK_API tacker_kernel_t tacker_create_kernel(const char *name);
@@ -350,6 +367,7 @@ TK_API tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const fl
                                               const float *z, float *Qr, float *Qi, int numX);
 TK_API tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N,
                                                int K);
+TK_API tacker_kernel_t tacker_ori_fft_create(float *data, int batches);
 TK_API tacker_kernel_t tacker_ori_mrif_create(int numK, const float *x, const float *y,
                                               const float *z, float *outR, float *outI, int numX);
 TK_API tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid,

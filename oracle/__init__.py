@@ -48,6 +48,8 @@ def _declare(l):
                                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_stencil.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_sgemm_gptb.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 9
+    l.orc_fft_gptb.argtypes = [_f32p, C.c_int, C.c_int, C.c_int]
+    l.orc_fft_source.argtypes = [_f32p, C.c_int]
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
@@ -280,6 +282,28 @@ def sgemm(A, B, Cm, start=0, end=None, parts=1, W=None, chunk=SGEMM_K_CHUNK):
     assert W.dtype == np.float32 and W.flags["C_CONTIGUOUS"] and W.shape == (N, M)
     lib().orc_sgemm_gptb(A.reshape(-1), B.reshape(-1), out.reshape(-1), W.reshape(-1), M, N, K, gdx, gdy, parts,
                          chunk, start, end)
+    return out
+
+
+# --------------------------------------------------------------------------- fft
+FFT_N = 256
+
+
+def fft(data, start=0, end=None):
+    """Batched 256-point forward transforms, in place in the reference and returned here: data is
+    [batches][256][2] float32 (re, im); block positions [start, end), position p = batch entry p % batches."""
+    out = np.array(data, np.float32, order="C")
+    assert out.ndim == 3 and out.shape[1:] == (FFT_N, 2)
+    if end is None:
+        end = out.shape[0]
+    lib().orc_fft_gptb(out.reshape(-1), out.shape[0], start, end)
+    return out
+
+
+def fft_source(batches):
+    """The reference's input: rand() after srand(54321), scaled to [-1, 1]."""
+    out = np.zeros((batches, FFT_N, 2), np.float32)
+    lib().orc_fft_source(out.reshape(-1), out.size)
     return out
 
 

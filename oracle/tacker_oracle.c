@@ -749,3 +749,73 @@ ORC_API void orc_sgemm_gptb(const float *A, const float *B, float *C, float *W, 
         }
     }
 }
+
+/* ------------------------------------------------------------------ fft
+ * src/ori_kernel/fft_kernel.cu:11-61, src/header/fft_header.h:13-67 (g_general_ptb_fft:
+ * src/gptb_kernel/fft_kernel.cu:3-75): a block of FFT_T = 128 threads transforms 256 complex
+ * points in place.  Thread j holds v[r] = data[j + r*128], r = 0, 1; for Ns = 1, 2, .., 128:
+ * angle = -2 pi (j % Ns) / (Ns * 2) (evaluated in double, rounded to float), v[r] *= (cos(r*angle),
+ * sin(r*angle)) with the float cos and sin, butterfly (v0 + v1, v0 - v1), then every thread writes
+ * v[r] to work[expand(j, Ns, 2) + r*Ns] and reads v[r] = work[j + r*128] (expand(j, 128, 2) = j),
+ * expand(i, N1, N2) = (i / N1) * N1 * N2 + i % N1.  Complex product: (a.x b.x - a.y b.y,
+ * a.x b.y + a.y b.x).  The library's cosf/sinf stand for CUDA's: bits of the twiddles may differ
+ * from either device's.
+ *
+ * Positions [start, end): position p transforms batch entry p % grid. */
+ORC_API void orc_fft_gptb(float *data, int grid, int start, int end)
+{
+    enum { N = 256, T = 128 };
+    const double pi = 3.14159265358979323846;   /* M_PI of math.h */
+    for (int pos = start; pos < end; pos++) {
+        float *d = data + (size_t)(pos % grid) * N * 2;
+        float vx[T][2], vy[T][2];
+        for (int j = 0; j < T; j++)
+            for (int r = 0; r < 2; r++) {
+                vx[j][r] = d[2 * (j + r * T)];
+                vy[j][r] = d[2 * (j + r * T) + 1];
+            }
+        for (int Ns = 1; Ns < N; Ns *= 2) {
+            float sr[N], si[N];
+            for (int j = 0; j < T; j++) {
+                const float angle = (float)(-2 * pi * (j % Ns) / (Ns * 2));
+                for (int r = 0; r < 2; r++) {
+                    const float bx = cosf(r * angle), by = sinf(r * angle);
+                    const float ax = vx[j][r], ay = vy[j][r];
+                    const float p0 = ax * bx, p1 = ay * by, p2 = ax * by, p3 = ay * bx;
+                    vx[j][r] = p0 - p1;
+                    vy[j][r] = p2 + p3;
+                }
+                const float tx = vx[j][0], ty = vy[j][0];
+                vx[j][0] = tx + vx[j][1];
+                vy[j][0] = ty + vy[j][1];
+                vx[j][1] = tx - vx[j][1];
+                vy[j][1] = ty - vy[j][1];
+                const int idxD = (j / Ns) * Ns * 2 + (j % Ns);
+                for (int r = 0; r < 2; r++) {
+                    sr[idxD + r * Ns] = vx[j][r];
+                    si[idxD + r * Ns] = vy[j][r];
+                }
+            }
+            for (int j = 0; j < T; j++) {
+                const int idxS = (j / T) * T * 2 + (j % T);
+                for (int r = 0; r < 2; r++) {
+                    vx[j][r] = sr[idxS + r * T];
+                    vy[j][r] = si[idxS + r * T];
+                }
+            }
+        }
+        for (int j = 0; j < T; j++)
+            for (int r = 0; r < 2; r++) {
+                d[2 * (j + r * T)] = vx[j][r];
+                d[2 * (j + r * T) + 1] = vy[j][r];
+            }
+    }
+}
+
+/* source[i] = rand() / (float)RAND_MAX * 2 - 1 after srand(54321), x then y of each point
+ * (src/ori_kernel/fft_kernel.cu:93-103) */
+ORC_API void orc_fft_source(float *data, int values)
+{
+    srand(54321);
+    for (int i = 0; i < values; i++) data[i] = (rand() / (float)RAND_MAX) * 2 - 1;
+}

@@ -70,6 +70,9 @@ def _declare(lib):
     lib.tacker_ori_sgemm.argtypes = [vp, vp, vp, i, i, i, vp]
     lib.tacker_gptb_sgemm.argtypes = [vp, vp, vp, i, i, i, i, i, i, i, vp]
     lib.tacker_mix_tzgemm_sgemm.argtypes = [vp, vp, vp, i, i, i, i, i] + gemm
+    lib.tacker_ori_fft.argtypes = [vp, i, vp]
+    lib.tacker_gptb_fft.argtypes = [vp, i, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_fft.argtypes = [vp, i, i, i] + gemm
     lib.tacker_mix_tzgemm_cp.argtypes = [i, f, vp, i, i, i, i] + gemm
     lib.tacker_im2col.argtypes = [vp] + [i] * 11 + [vp, vp]
     lib.tacker_convert_fp32_to_fp16.argtypes = [vp, vp, i, vp]
@@ -79,7 +82,7 @@ def _declare(lib):
     lib.tacker_fget_kernel_info.restype = f
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
                  "tacker_ori_mriq_create", "tacker_ori_mrif_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
-                 "tacker_ori_sgemm_create",
+                 "tacker_ori_sgemm_create", "tacker_ori_fft_create",
                  "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
                  "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
@@ -89,6 +92,7 @@ def _declare(lib):
     lib.tacker_ori_mriq_create.argtypes = [i, vp, vp, vp, vp, vp, i]
     lib.tacker_ori_mrif_create.argtypes = [i, vp, vp, vp, vp, vp, i]
     lib.tacker_ori_sgemm_create.argtypes = [vp, vp, vp, i, i, i]
+    lib.tacker_ori_fft_create.argtypes = [vp, i]
     lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
     lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_gptb_create.argtypes = [vp, i, i, i, i]
@@ -459,6 +463,32 @@ def mix_tzgemm_sgemm(sA, sB, sC, A, B, Cm, be_start=0, be_end=None, tile_start=0
         "tacker_mix_tzgemm_sgemm")
 
 
+def _fft_batches(data):
+    """data: [batches][256][2] float32 device tensor (re, im), transformed in place"""
+    if data.dim() != 3 or tuple(data.shape[1:]) != (256, 2) or not data.is_contiguous():
+        raise ValueError("fft: data must be a contiguous [batches][256][2] float32 tensor")
+    return data.shape[0]
+
+
+def ori_fft(data, stream=None):
+    check(lib().tacker_ori_fft(_ptr(data), _fft_batches(data), _stream(stream)), "tacker_ori_fft")
+
+
+def gptb_fft(data, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    batches = _fft_batches(data)
+    check(lib().tacker_gptb_fft(_ptr(data), batches, start, batches if end is None else end, launch_grid,
+                                launch_block, _stream(stream)), "tacker_gptb_fft")
+
+
+def mix_tzgemm_fft(data, A, B, Cm, be_start=0, be_end=None, tile_start=0, tile_end=None, variant=None,
+                   launch_grid=0, launch_block=0, stream=None):
+    batches = _fft_batches(data)
+    check(lib().tacker_mix_tzgemm_fft(
+        _ptr(data), batches, be_start, batches if be_end is None else be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_fft")
+
+
 def mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, A, B, Cm, be_start=0, be_end=None, tile_start=0,
                     tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
     if be_end is None:
@@ -595,6 +625,10 @@ def ori_sgemm_create(sA, sB, sC):
     M, N, K = _sgemm_dims(sA, sB, sC)
     return KernelHandle(lib().tacker_ori_sgemm_create(_ptr(sA), _ptr(sB), _ptr(sC), M, N, K), "OriSGEMMKernel",
                         keep=(sA, sB, sC))
+
+
+def ori_fft_create(data):
+    return KernelHandle(lib().tacker_ori_fft_create(_ptr(data), _fft_batches(data)), "OriFFTKernel", keep=(data,))
 
 
 def ori_cp_create(numatoms, gridspacing, grid):

@@ -492,6 +492,33 @@ int tacker_gptb_sgemm(const float *A, const float *B, float *C, int M, int N, in
     return run_gptb_once(ori, block_start, block_end, launch_grid, launch_block, stream);
 }
 
+namespace {
+int check_fft(const float *data, int batches)
+{
+    static_assert(TACKER_FFT_POINTS == FFT_N, "public and device transform sizes must agree");
+    if (!data || batches <= 0) return fail(TK_ERROR_INVALID_VALUE, "fft: bad arguments");
+    if ((long long)batches * FFT_N >= (1ll << 30)) return fail(TK_ERROR_UNSUPPORTED, "fft: a batch of 2^30 points or more");
+    return TK_SUCCESS;
+}
+}  // namespace
+
+int tacker_ori_fft(float *data, int batches, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_fft(data, batches);
+    if (rc) return rc;
+    return run_once(new OriFFTKernel(0, data, batches), stream);
+}
+
+int tacker_gptb_fft(float *data, int batches, int block_start, int block_end, int launch_grid, int launch_block,
+                    tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_fft(data, batches);
+    if (rc) return rc;
+    return run_gptb_once(new OriFFTKernel(0, data, batches), block_start, block_end, launch_grid, launch_block, stream);
+}
+
 int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane)
 {
     REQUIRE_INIT();
@@ -618,6 +645,17 @@ int tacker_mix_tzgemm_sgemm(const float *sA, const float *sB, float *sC, int sM,
                         launch_block, stream);
 }
 
+int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_end, const void *A, const void *B, float *C,
+                          int M, int N, int K, int tile_start, int tile_end, const char *variant, int launch_grid,
+                          int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_fft(data, batches);
+    if (rc) return rc;
+    return run_mix_once(new OriFFTKernel(0, data, batches), be_start, be_end, A, B, C, M, N, K, tile_start, tile_end,
+                        variant, launch_grid, launch_block, stream);
+}
+
 int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, int be_start,
                          int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
                          int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
@@ -681,7 +719,7 @@ tacker_kernel_t tacker_create_kernel(const char *name)
         fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
         return nullptr;
     }
-    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "sgemm", "stencil", "tzgemm"};
+    static const char *known[] = {"cp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil", "tzgemm"};
     bool ok = false;
     for (auto k : known) ok |= (strcmp(k, name) == 0);
     if (!ok) {
@@ -723,6 +761,11 @@ tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y,
 {
     CREATE(check_mriq(numK, x, y, z, Qr, Qi, numX), new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX));
 }
+tacker_kernel_t tacker_ori_fft_create(float *data, int batches)
+{
+    CREATE(check_fft(data, batches), new OriFFTKernel(0, data, batches));
+}
+
 tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N, int K)
 {
     CREATE(check_sgemm(A, B, C, M, N, K), new OriSGEMMKernel(0, A, B, C, M, N, K));
@@ -1095,7 +1138,7 @@ tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const ch
         fail(TK_ERROR_INVALID_VALUE, "tacker_task_manager_create: bad arguments");
         return nullptr;
     }
-    static const char *known[] = {"cp", "lbm", "mrif", "mriq", "sgemm", "stencil"};
+    static const char *known[] = {"cp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"};
     bool ok1 = false, ok2 = !be2 || !*be2;
     for (auto k : known) {
         ok1 |= strcmp(k, be1) == 0;

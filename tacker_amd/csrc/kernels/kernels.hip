@@ -13,6 +13,7 @@
 #include "../../../include/tacker_amd.h"
 #include "cp_role.h"
 #include "dnn_kernels.h"
+#include "fft_role.h"
 #include "lbm_role.h"
 #include "mriq_role.h"
 #include "mrif_role.h"
@@ -98,6 +99,13 @@ extern "C" __global__ __launch_bounds__(128) void ori_sgemm(float *A, float *B, 
     __shared__ __align__(16) float stage[2][64];
     tk::sgemm_thread(A, B, C, nullptr, NORMAL_M, NORMAL_N, NORMAL_K, blockIdx.x * SGEMM_TILE_M + mid,
                      blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K, (tk::sgemm_lds_float *)&stage[mid >> 6][0]);
+}
+
+// grid (transforms), block 64: a wavefront per transform where the reference has a block of 128 threads
+// (src/ori_kernel/fft_kernel.cu:48-61)
+extern "C" __global__ __launch_bounds__(FFT_WAVE) void ori_fft(float *data)
+{
+    tk::fft_role<1>(data, (int)gridDim.x, (int)blockIdx.x, (int)gridDim.x, 0, (int)gridDim.x, (int)threadIdx.x, FFT_WAVE);
 }
 
 // grid (volx/128, voly/8), block (16,8)
@@ -242,6 +250,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ComputeRhoPhiGPU", (const void *)ComputeRhoPhiGPU, ctx);
     insert("ori_mrif", (const void *)ori_mrif, ctx);
     insert("ori_sgemm", (const void *)ori_sgemm, ctx);
+    insert("ori_fft", (const void *)ori_fft, ctx);
     insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);
     insert("tz_clear_words", (const void *)tz_clear_words, ctx);
     insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);

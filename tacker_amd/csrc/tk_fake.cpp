@@ -53,6 +53,7 @@ const std::vector<int> MRIQ = {I, I, P, P, P, P, P};
 const std::vector<int> MRIF = {I, I, P, P, P, P, P};
 const std::vector<int> CP = {I, F, P};
 const std::vector<int> SGEMM = {P, P, P, I, I, I};
+const std::vector<int> FFT = {P};
 const std::vector<int> TZ = {P, P, P, I, I, I};
 }  // namespace
 
@@ -188,6 +189,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ComputeRhoPhiGPU", {I, P, P, P, P, P, P});
         add("ori_mrif", MRIF);
         add("ori_sgemm", SGEMM);
+        add("ori_fft", FFT);
         add("gptb_tzgemm", cat(TZ, trailer(true)));
         add("gptb_tzgemm@large", cat(TZ, trailer(true)));
         add("gptb_tzgemm_scratch", cat(cat(TZ, {P}), trailer(true)));
@@ -198,6 +200,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("gptb_cp", cat(CP, trailer(true)));
         add("gptb_mrif", cat(MRIF, trailer(true)));
         add("gptb_sgemm", cat(SGEMM, trailer(true)));
+        add("gptb_fft", cat(FFT, trailer(true)));
         add("cp_inv_sqrt_selftest", {I, I, P});
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
@@ -207,7 +210,8 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("pack_fc_input", {P, 8, P, I, I, P});
         add("pack_fc_input_pooled", {P, I, I, I, P, I, I, P});
         const std::pair<const char *, const std::vector<int> *> bes[] = {
-            {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}, {"mrif", &MRIF}, {"sgemm", &SGEMM}};
+            {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}, {"mrif", &MRIF}, {"sgemm", &SGEMM},
+            {"fft", &FFT}};
         static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};
         for (auto &be : bes)
             for (auto v : variants)

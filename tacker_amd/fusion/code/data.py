@@ -58,6 +58,9 @@ KERNEL_INFO = {
     # 32 x 258 blocks of 128 rows x 16 columns of C x 16 parts of 256 k steps (4096 x 4128 x 4064)
     "sgemm": {"register": 64, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
               "ori_blks": 132096},
+    # 10240 transforms of 256 points, a wavefront each; 2 KiB of LDS per wavefront
+    "fft": {"register": 40, "shared_memory": 8192, "blocksize": 256, "solo_ptb_blks": 8,
+            "ori_blks": 10240},
     # 16384 blocks of 128 x 8 points x 4 parts of the unrolled x points
     "cp": {"register": 40, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
            "ori_blks": 65536},

@@ -49,7 +49,7 @@ def generate_wg_split(be, tz_wgs, be_wgs, threads=256):
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="sp.role_block", blocks="sp.role_blocks",
                                              tid="(int)threadIdx.x", stages="TZ_STAGES_WG", stream_c=_stream_c(be))
     be_call = ROLES[be]["call"].format(p=p_be, block="sp.role_block", blocks="sp.role_blocks",
-                                       tid="(int)threadIdx.x", threads=threads, extra="")
+                                       tid="(int)threadIdx.x", threads=threads, waves=threads // 64, extra="")
     name = mix_kernel_name(be, variant)
     text = f"""// {be}-tzgemm  workgroup split  {tz_wgs} tzgemm : {be_wgs} {be} workgroups per group
 extern "C" __global__ __launch_bounds__({threads}) void {name}(
@@ -88,7 +88,7 @@ def generate_wave_split(be, be_threads, tz_first=True):
     # enough loads in flight
     be_call = ROLES[be]["call"].format(p=p_be, block="be_block", blocks="be_blocks",
                                        tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads,
-                                       extra="<2>" if be == "lbm" else "")
+                                       waves=be_threads // 64, extra="<2>" if be == "lbm" else "")
     tz_cond = (f"threadIdx.x < {tz_threads}" if tz_first else f"threadIdx.x >= {be_threads}")
     name = mix_kernel_name(be, variant)
     unused = _void_unused(sig_be + sig_tz, tz_call + be_call + f"{p_be}ptb_iter_block_step")
@@ -155,9 +155,10 @@ def generate_be_pair(be1, be2, wgs1, wgs2, threads=256, order=False):
     p1, sig1 = signature(be1, 0)
     p2, sig2 = signature(be2, 1)
     block, blocks = ("(int)blockIdx.x", "(int)gridDim.x") if order else ("sp.role_block", "sp.role_blocks")
-    call1 = ROLES[be1]["call"].format(p=p1, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads, extra="")
+    call1 = ROLES[be1]["call"].format(p=p1, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads,
+                                      waves=threads // 64, extra="")
     call2 = ROLES[be2]["call"].format(p=p2, block=block, blocks=blocks, tid="(int)threadIdx.x", threads=threads,
-                                      extra="")
+                                      waves=threads // 64, extra="")
     name = be_pair_kernel_name(be1, be2, variant)
     if order:
         title = f"order split  {wgs1} of {wgs1 + wgs2} workgroups start with {be1}, the others with {be2}"
@@ -188,6 +189,10 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(
     return text, meta
 
 
+# wavefronts a GPTB launch of a role that sizes its LDS by them may have (__launch_bounds__(256))
+GPTB_MAX_WAVES = 4
+
+
 def generate_gptb(name):
     """The plain GPTB kernel of one role (``src/gptb_kernel/<name>_kernel.cu`` of the reference): the
     launch's workgroups are the role's persistent workgroups, ``thread_base`` shifts the thread index
@@ -195,7 +200,8 @@ def generate_gptb(name):
     role = ROLES[name]
     sig = gptb_signature(name)
     call = role["call"].format(p="", block="(int)blockIdx.x", blocks="ptb_iter_block_step",
-                               tid="(int)threadIdx.x - thread_base", threads="(int)blockDim.x", extra="",
+                               tid="(int)threadIdx.x - thread_base", threads="(int)blockDim.x", waves=GPTB_MAX_WAVES,
+                               extra="",
                                stages="TZ_STAGES", stream_c="true")
     symbol = role["gptb"]["symbol"]
     attributes = role["gptb"]["attributes"] + " " if role["gptb"]["attributes"] else ""

@@ -80,6 +80,10 @@ def make_inputs(np, torch, ta, be, small):
         shape = (32, 512) if small else (4096, 4096)
         grid = torch.zeros(shape, device="cuda:0")
         return ta.ori_cp_create(64, 0.1, grid), ta.cp_blocks(shape[1], shape[0]), [grid]
+    if be == "fft":
+        batches = 40 if small else 10240
+        data = torch.from_numpy(rng.uniform(-1, 1, (batches, 256, 2)).astype(np.float32)).cuda()
+        return ta.ori_fft_create(data), batches, [data]
     if be == "sgemm":
         M, N, K = (256, 48, 300) if small else (4096, 4128, 4064)
         A = torch.from_numpy(rng.uniform(0, 1, (K, M)).astype(np.float32)).cuda()

@@ -1,7 +1,7 @@
 """Role descriptions the generator stitches together.
 
 Each entry plays the part of one ``<kernel>_code.py`` of the reference
-(fusion/code/cp_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
+(fusion/code/cp_code.py, fft_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
 truncated tzgemm_code.py): the kernel's parameter list in reference order and
 how to call its device-side role.  The role bodies themselves live in
 ``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
@@ -16,7 +16,8 @@ device functions.
 ``call``     -- format string of the role call; ``{p}`` is the parameter prefix,
                ``{block}``, ``{blocks}`` the role-local persistent-workgroup id
                and count, ``{tid}`` the role-local thread id, ``{threads}`` the
-               role's thread count, ``{extra}`` role-specific trailing arguments.
+               role's thread count, ``{waves}`` that count in wavefronts (a compile-time
+               constant: it sizes the role's LDS), ``{extra}`` role-specific trailing arguments.
 """
 
 GPTB_DIMS = ["grid_dimension_x", "grid_dimension_y", "grid_dimension_z",
@@ -79,6 +80,14 @@ ROLES = {
         "needs_sync": False,
         "call": ("tk::sgemm_role({p}A, {p}B, {p}C, {p}NORMAL_M, {p}NORMAL_N, {p}NORMAL_K, {p}grid_dimension_x, "
                  "{p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, {p}ptb_start_block_pos, "
+                 "{p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+    "fft": {
+        "gptb": {"symbol": "g_general_ptb_fft", "cite": "src/gptb_kernel/fft_kernel.cu:39-75",
+                 "attributes": "__launch_bounds__(256)"},
+        "params": [("float*", "data")],
+        "needs_sync": False,
+        "call": ("tk::fft_role<{waves}>({p}data, {p}grid_dimension_x, {block}, {blocks}, {p}ptb_start_block_pos, "
                  "{p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "cp": {

@@ -76,10 +76,11 @@ def test_committed_generated_sources_are_fresh():
     assert rc.returncode == 0, rc.stdout + rc.stderr
 
 
-@pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27), ("sgemm", 30)])
+@pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27), ("sgemm", 30),
+                                         ("fft", 25)])
 def test_emitted_dispatcher_signature(be, n_params):
     # parameter count = the reference dispatcher's (src/mix_kernel/tzgemm_stencil.cu:281-283 31,
-    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27, tzgemm_sgemm.cu:303 30), order: be first
+    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27, tzgemm_sgemm.cu:303 30, tzgemm_fft.cu:988-996 25), order: be first
     text, meta = gen_mix.generate_wg_split(be, 1, 1)
     sig = re.search(r"void (\w+)\(\s*(.*?)\)\s*\{", text, re.S)
     params = [p.strip() for p in sig.group(2).split(",")]
@@ -99,7 +100,7 @@ def test_emitted_dispatcher_signature(be, n_params):
 @pytest.mark.parametrize("name,symbol,n_params", [
     ("tzgemm", "general_ptb_tzgemm", 16), ("stencil", "general_ptb_stencil", 17), ("lbm", "general_ptb_lbm", 12),
     ("mriq", "g_general_ptb_mriq", 17), ("mrif", "general_ptb_mrif", 17), ("cp", "g_general_ptb_cp", 13),
-    ("sgemm", "general_ptb_sgemm", 16)])
+    ("sgemm", "general_ptb_sgemm", 16), ("fft", "g_general_ptb_fft", 11)])
 def test_emitted_gptb_kernel_has_the_reference_name_and_parameter_list(name, symbol, n_params):
     # src/gptb_kernel/<name>_kernel.cu: the original kernel's parameters, then 6 dims, start, step, end,
     # thread_base (e.g. stencil_kernel.cu:3-5: 7 + 10; the names are what src/main.cu:108-125 registers)
@@ -139,9 +140,14 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
     files = gen_run.generate()
     kinfo = json.loads(files["../config/kinfo-gfx950.json"])
     pairs = gen_run.be_pairs()
-    assert pairs == [("cp", "lbm"), ("cp", "mrif"), ("cp", "mriq"), ("cp", "sgemm"), ("cp", "stencil"), ("lbm", "mrif"),
-                     ("lbm", "mriq"), ("lbm", "sgemm"), ("lbm", "stencil"), ("mrif", "mriq"), ("mrif", "sgemm"),
-                     ("mrif", "stencil"), ("mriq", "sgemm"), ("mriq", "stencil"), ("sgemm", "stencil")]
+    assert pairs == [("cp", "fft"), ("cp", "lbm"), ("cp", "mrif"), ("cp", "mriq"), ("cp", "sgemm"), ("cp", "stencil"),
+                     ("fft", "lbm"), ("fft", "mrif"), ("fft", "mriq"), ("fft", "sgemm"), ("fft", "stencil"),
+                     ("lbm", "mrif"), ("lbm", "mriq"), ("lbm", "sgemm"), ("lbm", "stencil"), ("mrif", "mriq"),
+                     ("mrif", "sgemm"), ("mrif", "stencil"), ("mriq", "sgemm"), ("mriq", "stencil"), ("sgemm", "stencil")]
+    # the fft pairs the reference ships: src/mix_kernel/{cp_fft_3_1,fft_lbm_6_1,fft_mriq_3_2,fft_sgemm_1_4,fft_stencil_5_3}.cu
+    sig = re.search(r"void fft_lbm_mix_wg_1_1\(\s*(.*?)\)\s*\{", files["mix_kernel/fft_lbm.hip"], re.S)
+    names = [q.split()[-1] for q in sig.group(1).split(",")]
+    assert len(names) == 21 and names[0] == "fft0_data" and names[10:12] == ["lbm1_srcGrid", "lbm1_dstGrid"]
     # the four sgemm pairs the reference ships: src/mix_kernel/{cp_sgemm_1_1,lbm_sgemm_1_7,mrif_sgemm_1_4,mriq_sgemm_1_2}.cu
     cp_sgemm = files["mix_kernel/cp_sgemm.hip"]
     sig = re.search(r"void cp_sgemm_mix_wg_1_1\(\s*(.*?)\)\s*\{", cp_sgemm, re.S)
@@ -161,7 +167,7 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
         assert f'insert("{a}_{b}", ' in files["mix_kernel/mix_kernels.inc"]
         # parameter order: the first kernel's list, then the second's
         assert text.index(f"{a}0_grid_dimension_x") < text.index(f"{b}1_grid_dimension_x")
-    assert "__shared__" not in files["mix_kernel/lbm_mriq.hip"]        # no role of a pair uses LDS
+    assert "__shared__" not in files["mix_kernel/lbm_mriq.hip"]        # LDS, where a role uses it, is the role's own
 
 
 def test_measured_load_ratios_travel_from_profile_ratio_to_the_schedulers_lookup(tmp_path, monkeypatch):
@@ -191,7 +197,7 @@ def test_measured_load_ratios_travel_from_profile_ratio_to_the_schedulers_lookup
     assert after["tzgemm_stencil"] == before["tzgemm_stencil"]          # pairs that were not measured keep theirs
     with pytest.raises(SystemExit):                                    # a pair the generator does not know
         bad = tmp_path / "bad.json"
-        bad.write_text(json.dumps({"stretch": 1.0, "device": "x", "pairs": {"tzgemm_fft": {"by_k": {}}}}))
+        bad.write_text(json.dumps({"stretch": 1.0, "device": "x", "pairs": {"tzgemm_cutcp": {"by_k": {}}}}))
         profile_ratio.apply(str(bad))
     kinfo_text = gen_run.generate()["../config/kinfo-gfx950.json"]
     kinfo = json.loads(kinfo_text)

@@ -806,9 +806,22 @@ def _small_be(name):
         sA, sB, sC0 = sgemm_inputs()
         sC = dev(sC0)
         return ta.ori_sgemm_create(dev(sA), dev(sB), sC), ta.sgemm_blocks(256, 48, 700), [sC]
+    if name == "fft":
+        data = dev(fft_inputs())
+        return ta.ori_fft_create(data), data.shape[0], [data]
     ta.cp_set_atoms(cp_atoms(), 0.0)
     g = torch.zeros((32, 512), device="cuda:0")
     return ta.ori_cp_create(64, 0.1, g), ta.cp_blocks(512, 32), [g]
+
+
+def fft_inputs():
+    return np.random.default_rng(36).uniform(-1, 1, (50, 256, 2)).astype(np.float32)
+
+
+def fft_close(got, want):
+    """|d| <= 1e-4 + 1e-5 |ref|: eight stages of fp32 butterflies on inputs in [-1, 1] (sums up to ~40) with
+    twiddles that differ from the C library's in the last place"""
+    return bool(np.all(np.abs(got.astype(np.float64) - want) <= 1e-4 + 1e-5 * np.abs(want)))
 
 
 def sgemm_inputs():
@@ -819,7 +832,8 @@ def sgemm_inputs():
 
 BE_PAIRS = [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"), ("lbm", "stencil"), ("mriq", "stencil"),
             ("cp", "mrif"), ("lbm", "mrif"), ("mrif", "mriq"), ("mrif", "stencil"), ("cp", "sgemm"), ("lbm", "sgemm"),
-            ("mrif", "sgemm"), ("mriq", "sgemm"), ("sgemm", "stencil")]
+            ("mrif", "sgemm"), ("mriq", "sgemm"), ("sgemm", "stencil"), ("cp", "fft"), ("fft", "lbm"), ("fft", "mrif"),
+            ("fft", "mriq"), ("fft", "sgemm"), ("fft", "stencil")]
 
 
 @pytest.mark.parametrize("first,second", BE_PAIRS)
@@ -847,7 +861,7 @@ def test_best_effort_pairs_fused_equals_unfused(first, second, variant):
 
 def _small_be_matches_oracle(name, outs):
     """the outputs of _small_be(name) after one full pass, against the oracle on the same seeded inputs:
-    bit-exact for stencil, lbm and cp, the float tolerance for the two MRI kernels"""
+    bit-exact for stencil, lbm, cp and sgemm, the float tolerances for the two MRI kernels and the FFT"""
     if name == "stencil":
         A0 = stencil_inputs(6, 20, 200, seed=31)
         return np.array_equal(host(outs[0]).view(np.uint32), oracle.stencil(C0, C1, A0, A0).view(np.uint32))
@@ -867,6 +881,8 @@ def _small_be_matches_oracle(name, outs):
         return mriq_close(host(outs[0]), tr.astype(np.float64)) and mriq_close(host(outs[1]), ti.astype(np.float64))
     if name == "sgemm":
         return np.array_equal(host(outs[0]).view(np.uint32), oracle.sgemm(*sgemm_inputs()).view(np.uint32))
+    if name == "fft":
+        return fft_close(host(outs[0]), oracle.fft(fft_inputs()).astype(np.float64))
     want = oracle.cp(oracle.cp_atoms_to_const(cp_atoms(), 0.0), np.zeros((32, 512), np.float32))
     return np.array_equal(host(outs[0]).view(np.uint32), want.view(np.uint32))
 
