@@ -101,6 +101,17 @@ def pair_leg(ta, torch, np, name, stream):
         label = "tzgemm 2048^3 + sgemm 4096x4128x4064 fp32 (reference mix tzgemm_sgemm)"
         reset = sC.zero_        # C = 2 C + 2 A B doubles with every pass: start every timed round from zero
         n = 50
+    elif name == "fft":     # Parboil FFT, 10240 transforms of 256 points (the Creator's instance, src/ori_kernel/fft_kernel.cu:87-115)
+        batches = 10240
+        source = torch.from_numpy(rng.uniform(-1, 1, (batches, 256, 2)).astype(np.float32)).cuda()
+        data = source.clone()
+        be_ori = ta.ori_fft_create(data)
+        nblk = batches
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "hbm", "algorithmic_bytes": 2.0 * batches * 256 * 8}
+        label = "tzgemm 2048^3 + fft 10240 x 256 points (reference mix tzgemm_fft)"
+        reset = lambda: data.copy_(source)   # in place: every pass multiplies the magnitudes by 16
+        n = 25
     elif name == "lbm":     # D3Q19, 120x120x150, rest equilibrium + noise, 5 % obstacle cells
         sx, sy, sz = 120, 120, 150
         cells = sx * sy * sz
@@ -445,10 +456,11 @@ def main():
     if not args.no_extras:
         out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
         out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream)
-                              for name in ("lbm", "mriq", "cp", "mrif", "sgemm")}
+                              for name in ("lbm", "mriq", "cp", "mrif", "sgemm", "fft")}
         if not args.no_lc:
             out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")
+            out["lc_colocation_fft"] = lc_leg(ta, torch, np, args.queries, "fft", "fft 10240 x 256 points")
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(A, B, A0, c0, c1)
     print(json.dumps(out))
