@@ -30,6 +30,13 @@
  *                         positions as orc_mriq.
  *   orc_cp*               single atom closed form, numpy float64 brute force,
  *                         ori_blks = 16384 held by fusion/code/kinfo.json.
+ *   orc_sgemm_gptb        float64 matrix product, integer operands (exact), one-hot A, the
+ *                         fused multiply-add per step against exact rationals, any
+ *                         ascending tiling of the position grid (tests/test_oracle_sgemm.py).
+ *   orc_fft*              the float64 transform (numpy's FFT and the defining sum), unit
+ *                         impulses = rows of the DFT matrix, pure tones, linearity,
+ *                         Parseval, position wrap; the input stream against the cp atoms'
+ *                         draw of the same seeded rand().
  *   orc_im2col            direct convolution brute force.
  *   orc_gptb_index        partition invariance (any launch grid covers every
  *                         block once).
