@@ -101,8 +101,8 @@ TK_API int tkModuleLaunchKernel(tkFunction_t f, tkDim3 grid, tkDim3 block, void 
 /* Fills the string-keyed device-function registry (the global `fmap` of
  * src/main.cu:108-159) without the host translation unit including device
  * sources: insert(key, function, ctx) is called once per kernel. Keys on the
- * hot path: ori_{stencil,lbm,mriq,mrif,cp,sgemm,fft}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp,sgemm,fft},
- * tzgemm_{stencil,lbm,mriq,mrif,cp,sgemm,fft}, plus variant keys "<key>@<variant>". */
+ * hot path: ori_{stencil,lbm,mriq,mrif,cp,sgemm,fft,cutcp}, gptb_{tzgemm,stencil,lbm,mriq,mrif,cp,sgemm,fft,cutcp},
+ * tzgemm_{stencil,lbm,mriq,mrif,cp,sgemm,fft,cutcp}, plus variant keys "<key>@<variant>". */
 typedef void (*tk_kernel_insert_fn)(const char *key, const void *func, void *ctx);
 TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx);
 
@@ -263,6 +263,34 @@ TK_API int tacker_ori_fft(float *data, int batches, tkStream_t stream);
 TK_API int tacker_gptb_fft(float *data, int batches, int block_start, int block_end, int launch_grid,
                            int launch_block, tkStream_t stream);
 
+/* prepare_input (src/header/cutcp_header.h:111-300): hashes natoms atoms {x, y, z, q} into bins of
+ * 4 x 4 x 4 Angstroms, 8 atoms to a bin, around a lattice of nx x ny x nz points of spacing h whose
+ * lowest corner is lo, and lists the bin offsets a region of 8 x 8 x 8 points has to visit for the
+ * given cutoff.  binDim[3], *padding (bins added on every side) and *nbr_len are always written;
+ * bins (binDim[0] * binDim[1] * binDim[2] * 32 floats, x fastest) and nbr (*nbr_len triples, at most
+ * 1331) when not NULL; counts[0] = atoms left out because their bin was full (the reference leaves
+ * those to the CPU), counts[1] = atoms outside the bins or without charge.  Host memory only. */
+TK_API int tacker_cutcp_prepare_input(const float *atoms, int natoms, const float lo[3], int nx, int ny,
+                                      int nz, float h, float cutoff, int binDim[3], int *padding,
+                                      float *bins, int *nbr, int *nbr_len, int counts[2]);
+/* cudaMemcpyToSymbol(NbrListLen / NbrList) (src/ori_kernel/cutcp_kernel.cu:241-242) */
+TK_API int tacker_cutcp_set_neighbours(const int *ijk, int len);
+/* ori_cutcp / general_ptb_cutcp (src/ori_kernel/cutcp_kernel.cu:19-158,
+ * src/gptb_kernel/cutcp_kernel.cu:12-183): the cutoff potential of the binned atoms on regions_x x
+ * regions_y x regions_z regions of 8 x 8 x 8 lattice points, 512 floats per region, region (x, y, z)
+ * at ((z regions_y + y) regions_x + x) * 512.  binZeroAddr points at bin (0, 0, 0) of the lattice,
+ * behind the padding bins (device memory, read only).  One block position per region, in the order
+ * of the reference's GPTB kernel (x slowest).  A wavefront serves half a region (launch_block a
+ * multiple of 64).  The hardware's reciprocal square root stands for CUDA's rsqrtf: results agree
+ * with the reference's within rounding, not bit for bit. */
+TK_API int tacker_ori_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2,
+                            float inv_cutoff2, float *regionZeroAddr, int regions_x, int regions_y,
+                            int regions_z, tkStream_t stream);
+TK_API int tacker_gptb_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2,
+                             float inv_cutoff2, float *regionZeroAddr, int regions_x, int regions_y,
+                             int regions_z, int block_start, int block_end, int launch_grid,
+                             int launch_block, tkStream_t stream);
+
 /* copyatomstoconstbuf (src/ori_kernel/cp_kernel.cu:159-179): host array of
  * count (<= 64) {x,y,z,q}; z is replaced by (zplane - z)^2 on the way. */
 TK_API int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane);
@@ -326,6 +354,13 @@ TK_API int tacker_mix_tzgemm_sgemm(const float *sA, const float *sB, float *sC, 
                                    int M, int N, int K, int tile_start, int tile_end,
                                    const char *variant, int launch_grid, int launch_block,
                                    tkStream_t stream);
+/* src/mix_kernel/tzgemm_cutcp.cu */
+TK_API int tacker_mix_tzgemm_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h,
+                                   float cutoff2, float inv_cutoff2, float *regionZeroAddr, int regions_x,
+                                   int regions_y, int regions_z, int be_start, int be_end, const void *A,
+                                   const void *B, float *C, int M, int N, int K, int tile_start,
+                                   int tile_end, const char *variant, int launch_grid, int launch_block,
+                                   tkStream_t stream);
 /* src/mix_kernel/tzgemm_fft.cu */
 TK_API int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_end, const void *A,
                                  const void *B, float *C, int M, int N, int K, int tile_start,
@@ -353,7 +388,7 @@ TK_API float tacker_fget_kernel_info(const char *kernel, const char *key);
 /* ---- object API: the class layer itself, one handle per C++ object ---------- */
 typedef void *tacker_kernel_t;
 
-/* createKernel (src/Creator.cu:21-337) for the names cp, fft, lbm, mrif, mriq, sgemm, stencil,
+/* createKernel (src/Creator.cu:21-337) for the names cp, cutcp, fft, lbm, mrif, mriq, sgemm, stencil,
  * tzgemm: the memoised GPTBKernel that owns seeded device buffers exactly as the
  * reference's Ori*Kernel::initParams builds them. Never destroy these. */
 TK_API tacker_kernel_t tacker_create_kernel(const char *name);
@@ -368,6 +403,9 @@ TK_API tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const fl
 TK_API tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N,
                                                int K);
 TK_API tacker_kernel_t tacker_ori_fft_create(float *data, int batches);
+TK_API tacker_kernel_t tacker_ori_cutcp_create(int binDim_x, int binDim_y, const float *binZeroAddr, float h,
+                                               float cutoff2, float inv_cutoff2, float *regionZeroAddr,
+                                               int regions_x, int regions_y, int regions_z);
 TK_API tacker_kernel_t tacker_ori_mrif_create(int numK, const float *x, const float *y,
                                               const float *z, float *outR, float *outI, int numX);
 TK_API tacker_kernel_t tacker_ori_cp_create(int numatoms, float gridspacing, float *energygrid,

@@ -48,6 +48,9 @@ def _declare(l):
                                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_stencil.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_sgemm_gptb.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 9
+    l.orc_cutcp_gptb.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_void_p, _i32p] + [C.c_int] * 6
+    l.orc_cutcp_prepare.argtypes = [_f32p, C.c_int, _f32p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, _i32p, _i32p,
+                                    C.c_void_p, C.c_void_p, _i32p]
     l.orc_fft_gptb.argtypes = [_f32p, C.c_int, C.c_int, C.c_int]
     l.orc_fft_source.argtypes = [_f32p, C.c_int]
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
@@ -283,6 +286,42 @@ def sgemm(A, B, Cm, start=0, end=None, parts=1, W=None, chunk=SGEMM_K_CHUNK):
     lib().orc_sgemm_gptb(A.reshape(-1), B.reshape(-1), out.reshape(-1), W.reshape(-1), M, N, K, gdx, gdy, parts,
                          chunk, start, end)
     return out
+
+
+# --------------------------------------------------------------------------- cutcp
+def cutcp_prepare(atoms, lo, nx, ny, nz, h, cutoff):
+    """prepare_input of the reference: dict with binDim (x, y, z), padding, bins [z][y][x][8][4] float32
+    (padding bins included), nbr [n][3] int32, extra, excluded."""
+    atoms = np.ascontiguousarray(atoms, np.float32).reshape(-1, 4)
+    lo = np.ascontiguousarray(lo, np.float32)
+    dims, pad, counts = np.zeros(3, np.int32), np.zeros(1, np.int32), np.zeros(2, np.int32)
+    nbr = np.zeros((1331, 3), np.int32)
+    n = lib().orc_cutcp_prepare(atoms.reshape(-1), len(atoms), lo, nx, ny, nz, h, cutoff, dims, pad, None,
+                                nbr.ctypes.data, counts)
+    if n < 0:
+        raise ValueError("cutcp: spacing or cutoff outside what the neighbour list covers")
+    bins = np.zeros((int(dims[2]), int(dims[1]), int(dims[0]), 8, 4), np.float32)
+    lib().orc_cutcp_prepare(atoms.reshape(-1), len(atoms), lo, nx, ny, nz, h, cutoff, dims, pad, bins.ctypes.data,
+                            nbr.ctypes.data, counts)
+    return {"binDim": tuple(int(d) for d in dims), "padding": int(pad[0]), "bins": bins, "nbr": nbr[:n].copy(),
+            "extra": int(counts[0]), "excluded": int(counts[1])}
+
+
+def cutcp(prep, h, cutoff2, inv_cutoff2, regions, start=0, end=None, out=None):
+    """Energies [regions z][y][x][8][8][8] float32 (point (x, y, z) of a region at [z][y][x]) of the block
+    positions [start, end) of a (regions x, y, z) grid; other regions keep what ``out`` holds (zeros)."""
+    rx, ry, rz = regions
+    bins = prep["bins"]
+    c = prep["padding"]
+    bdx, bdy = prep["binDim"][0], prep["binDim"][1]
+    zero = bins.ctypes.data + (((c * bdy + c) * bdx + c) * 32) * 4
+    res = np.zeros((rz, ry, rx, 8, 8, 8), np.float32) if out is None else np.array(out, np.float32, order="C")
+    if end is None:
+        end = rx * ry * rz
+    nbr = np.ascontiguousarray(prep["nbr"], np.int32)
+    lib().orc_cutcp_gptb(bdx, bdy, zero, h, cutoff2, inv_cutoff2, res.ctypes.data, nbr.reshape(-1), len(nbr), rx, ry, rz,
+                         start, end)
+    return res
 
 
 # --------------------------------------------------------------------------- fft

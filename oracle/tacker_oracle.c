@@ -826,3 +826,110 @@ ORC_API void orc_fft_source(float *data, int values)
     srand(54321);
     for (int i = 0; i < values; i++) data[i] = (rand() / (float)RAND_MAX) * 2 - 1;
 }
+
+/* ------------------------------------------------------------------ cutcp
+ * src/ori_kernel/cutcp_kernel.cu:19-158 (general_ptb_cutcp: src/gptb_kernel/cutcp_kernel.cu:12-183):
+ * thread (tx, ty, tz) of region (xr, yr, zr) owns the lattice points (8 xr + tx, 8 yr + ty + 2 e,
+ * 8 zr + tz), e = 0..3.  It walks the bins centre + nbr[n], n ascending, and in a bin the atoms until
+ * the first with charge 0:
+ *   dx = ax - x; dz = az - z; dxdz2 = dx*dx + dz*dz; dy = ay - y; r2 = dy*dy + dxdz2;
+ *   if (r2 < cutoff2) { s = 1 - r2 * inv_cutoff2; energy_e += aq * rsqrt(r2) * s * s; }  dy -= 2h; ...
+ * centre = floor((8 r + 4) * h / 4) per dimension.  1.0f / sqrtf stands for CUDA's rsqrtf (an
+ * approximation of about an ulp on either device).  Energies are stored, not accumulated.
+ *
+ * Positions [start, end): position p is region (p / (gdy gdz), (p / gdz) % gdy, p % gdz). */
+ORC_API void orc_cutcp_gptb(int binDim_x, int binDim_y, const float *binZero, float h, float cutoff2, float inv_cutoff2,
+                            float *regionZero, const int *nbr, int nbr_len, int gdx, int gdy, int gdz, int start, int end)
+{
+#pragma omp parallel for schedule(dynamic)
+    for (int pos = start; pos < end; pos++) {
+        const int xr = (pos / (gdy * gdz)) % gdx, yr = (pos / gdz) % gdy, zr = pos % gdz;
+        float *region = regionZero + (size_t)((zr * gdy + yr) * gdx + xr) * 512;
+        const int bx = (int)floorf((8 * xr + 4) * h * 0.25f);
+        const int by = (int)floorf((8 * yr + 4) * h * 0.25f);
+        const int bz = (int)floorf((8 * zr + 4) * h * 0.25f);
+        for (int tid = 0; tid < 128; tid++) {
+            const int tx = tid & 7, ty = (tid >> 3) & 1, tz = tid >> 4;
+            const float x = (8 * xr + tx) * h, y = (8 * yr + ty) * h, z = (8 * zr + tz) * h;
+            float energy[4] = {0.f, 0.f, 0.f, 0.f};
+            for (int n = 0; n < nbr_len; n++) {
+                const int i = bx + nbr[3 * n], j = by + nbr[3 * n + 1], k = bz + nbr[3 * n + 2];
+                const float *bin = binZero + ((long long)(k * binDim_y + j) * binDim_x + i) * 32;
+                for (int a = 0; a < 8; a++) {
+                    const float aq = bin[4 * a + 3];
+                    if (0.f == aq) break;
+                    const float dx = bin[4 * a] - x;
+                    const float dz = bin[4 * a + 2] - z;
+                    const float dxdz2 = dx * dx + dz * dz;
+                    float dy = bin[4 * a + 1] - y;
+                    for (int e = 0; e < 4; e++) {
+                        const float r2 = dy * dy + dxdz2;
+                        if (r2 < cutoff2) {
+                            const float s = (1.f - r2 * inv_cutoff2);
+                            energy[e] += aq * (1.0f / sqrtf(r2)) * s * s;
+                        }
+                        dy -= 2.0f * h;
+                    }
+                }
+            }
+            for (int e = 0; e < 4; e++) region[(tid >> 4) * 64 + (tid & 15) + 16 * e] = energy[e];
+        }
+    }
+}
+
+/* prepare_input (src/header/cutcp_header.h:111-300): bin dimensions, neighbour list and the atoms
+ * hashed into bins of 4 Angstroms, 8 to a bin, in the order given.  bins: binDim x*y*z * 32 floats,
+ * zeroed by the caller; nbr: room for 1331 triples.  Returns the neighbour count, -1 where the
+ * reference gives up.  counts: atoms whose bin was full, atoms outside or without charge. */
+ORC_API int orc_cutcp_prepare(const float *atoms, int natoms, const float *lo, int nx, int ny, int nz, float h,
+                              float cutoff, int *binDim, int *padding, float *bins, int *nbr, int *counts)
+{
+    const int lnx = 8 * (int)ceilf(nx / 8.f), lny = 8 * (int)ceilf(ny / 8.f), lnz = 8 * (int)ceilf(nz / 8.f);
+    const int c = (int)ceil(cutoff * 0.25f);
+    *padding = c;
+    binDim[0] = (int)ceil(lnx * h * 0.25f) + 2 * c;
+    binDim[1] = (int)ceil(lny * h * 0.25f) + 2 * c;
+    binDim[2] = (int)ceil(lnz * h * 0.25f) + 2 * c;
+    float s;
+    if (ceilf(4.f / (8 * h)) == floorf(4.f / (8 * h))) {
+        s = sqrtf(3);
+        if (2 * c + 1 > 11) return -1;
+    } else if (8 * h <= 2 * 4.f) {
+        s = 2.f * sqrtf(3);
+        if (2 * c + 3 > 11) return -1;
+    } else {
+        return -1;
+    }
+    const float r2 = (cutoff + s * 4.f) * (cutoff + s * 4.f);
+    int cnt = 0;
+    for (int k = -c; k <= c; k++)
+        for (int j = -c; j <= c; j++)
+            for (int i = -c; i <= c; i++) {
+                if ((i * i + j * j + k * k) * 4.f * 4.f >= r2) continue;
+                if (nbr) nbr[3 * cnt] = i, nbr[3 * cnt + 1] = j, nbr[3 * cnt + 2] = k;
+                cnt++;
+            }
+    if (!bins) return cnt;
+    const long long nbins = (long long)binDim[0] * binDim[1] * binDim[2];
+    int *fill = (int *)calloc((size_t)nbins, sizeof(int));
+    counts[0] = counts[1] = 0;
+    for (int n = 0; n < natoms; n++) {
+        const float px = atoms[4 * n] - lo[0], py = atoms[4 * n + 1] - lo[1], pz = atoms[4 * n + 2] - lo[2];
+        const float q = atoms[4 * n + 3];
+        const int i = (int)floorf(px * 0.25f), j = (int)floorf(py * 0.25f), k = (int)floorf(pz * 0.25f);
+        if (i >= -c && i < binDim[0] - c && j >= -c && j < binDim[1] - c && k >= -c && k < binDim[2] - c && q != 0) {
+            const long long index = ((long long)(k + c) * binDim[1] + (j + c)) * binDim[0] + (i + c);
+            if (fill[index] < 8) {
+                float *slot = bins + index * 32 + 4 * fill[index];
+                slot[0] = px, slot[1] = py, slot[2] = pz, slot[3] = q;
+                fill[index]++;
+            } else {
+                counts[0]++;
+            }
+        } else {
+            counts[1]++;
+        }
+    }
+    free(fill);
+    return cnt;
+}

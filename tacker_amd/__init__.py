@@ -70,6 +70,12 @@ def _declare(lib):
     lib.tacker_ori_sgemm.argtypes = [vp, vp, vp, i, i, i, vp]
     lib.tacker_gptb_sgemm.argtypes = [vp, vp, vp, i, i, i, i, i, i, i, vp]
     lib.tacker_mix_tzgemm_sgemm.argtypes = [vp, vp, vp, i, i, i, i, i] + gemm
+    cut = [i, i, vp, f, f, f, vp, i, i, i]
+    lib.tacker_cutcp_prepare_input.argtypes = [vp, i, vp, i, i, i, f, f, vp, vp, vp, vp, vp, vp]
+    lib.tacker_cutcp_set_neighbours.argtypes = [vp, i]
+    lib.tacker_ori_cutcp.argtypes = cut + [vp]
+    lib.tacker_gptb_cutcp.argtypes = cut + [i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_cutcp.argtypes = cut + [i, i] + gemm
     lib.tacker_ori_fft.argtypes = [vp, i, vp]
     lib.tacker_gptb_fft.argtypes = [vp, i, i, i, i, i, vp]
     lib.tacker_mix_tzgemm_fft.argtypes = [vp, i, i, i] + gemm
@@ -82,7 +88,7 @@ def _declare(lib):
     lib.tacker_fget_kernel_info.restype = f
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
                  "tacker_ori_mriq_create", "tacker_ori_mrif_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
-                 "tacker_ori_sgemm_create", "tacker_ori_fft_create",
+                 "tacker_ori_sgemm_create", "tacker_ori_fft_create", "tacker_ori_cutcp_create",
                  "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
                  "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
@@ -93,6 +99,7 @@ def _declare(lib):
     lib.tacker_ori_mrif_create.argtypes = [i, vp, vp, vp, vp, vp, i]
     lib.tacker_ori_sgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_ori_fft_create.argtypes = [vp, i]
+    lib.tacker_ori_cutcp_create.argtypes = cut
     lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
     lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_gptb_create.argtypes = [vp, i, i, i, i]
@@ -461,6 +468,71 @@ def mix_tzgemm_sgemm(sA, sB, sC, A, B, Cm, be_start=0, be_end=None, tile_start=0
         _ptr(sA), _ptr(sB), _ptr(sC), M, N, K, be_start, be_end,
         *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
         "tacker_mix_tzgemm_sgemm")
+
+
+class CutcpInput:
+    """prepare_input of the reference on host arrays, then on the device: the binned atoms (``bins``, with the
+    padding bins), the address of bin (0, 0, 0), the neighbour list loaded into the device table, and an
+    energy tensor [regions z][y][x][8][8][8] (``energies``)."""
+
+    def __init__(self, atoms, lo, nx, ny, nz, h, cutoff, regions=None):
+        import numpy as np
+        import torch
+        atoms = np.ascontiguousarray(atoms, np.float32).reshape(-1, 4)
+        lo = np.ascontiguousarray(lo, np.float32)
+        dims, pad, nlen, counts = (C.c_int * 3)(), C.c_int(), C.c_int(), (C.c_int * 2)()
+        args = (atoms.ctypes.data, len(atoms), lo.ctypes.data, nx, ny, nz, h, cutoff)
+        check(lib().tacker_cutcp_prepare_input(*args, dims, C.byref(pad), None, None, C.byref(nlen), counts),
+              "tacker_cutcp_prepare_input")
+        self.binDim = tuple(dims)
+        self.padding = pad.value
+        bins = np.zeros((dims[2], dims[1], dims[0], 8, 4), np.float32)
+        nbr = np.zeros((nlen.value, 3), np.int32)
+        check(lib().tacker_cutcp_prepare_input(*args, dims, C.byref(pad), bins.ctypes.data, nbr.ctypes.data,
+                                               C.byref(nlen), counts), "tacker_cutcp_prepare_input")
+        self.extra, self.excluded = counts[0], counts[1]
+        self.nbr = nbr
+        self.host_bins = bins
+        self.h = float(h)
+        self.bins = torch.from_numpy(bins).cuda()
+        c = self.padding
+        self.bin_zero = self.bins.data_ptr() + (((c * dims[1] + c) * dims[0] + c) * 32) * 4
+        self.regions = regions or (-(-nx // 8), -(-ny // 8), -(-nz // 8))
+        rx, ry, rz = self.regions
+        self.energies = torch.zeros((rz, ry, rx, 8, 8, 8), device="cuda:0")
+        self.load_neighbours()
+
+    def load_neighbours(self):
+        check(lib().tacker_cutcp_set_neighbours(self.nbr.ctypes.data, len(self.nbr)), "tacker_cutcp_set_neighbours")
+
+    def blocks(self):
+        return self.regions[0] * self.regions[1] * self.regions[2]
+
+    def args(self, cutoff2, inv_cutoff2, energies=None):
+        e = self.energies if energies is None else energies
+        return (self.binDim[0], self.binDim[1], self.bin_zero, self.h, cutoff2, inv_cutoff2, _ptr(e)) + tuple(self.regions)
+
+
+def ori_cutcp(inp, cutoff2, inv_cutoff2, energies=None, stream=None):
+    check(lib().tacker_ori_cutcp(*inp.args(cutoff2, inv_cutoff2, energies), _stream(stream)), "tacker_ori_cutcp")
+
+
+def gptb_cutcp(inp, cutoff2, inv_cutoff2, energies=None, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    check(lib().tacker_gptb_cutcp(*inp.args(cutoff2, inv_cutoff2, energies), start, inp.blocks() if end is None else end,
+                                  launch_grid, launch_block, _stream(stream)), "tacker_gptb_cutcp")
+
+
+def mix_tzgemm_cutcp(inp, cutoff2, inv_cutoff2, A, B, Cm, energies=None, be_start=0, be_end=None, tile_start=0,
+                     tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    check(lib().tacker_mix_tzgemm_cutcp(
+        *inp.args(cutoff2, inv_cutoff2, energies), be_start, inp.blocks() if be_end is None else be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_cutcp")
+
+
+def ori_cutcp_create(inp, cutoff2, inv_cutoff2, energies=None):
+    return KernelHandle(lib().tacker_ori_cutcp_create(*inp.args(cutoff2, inv_cutoff2, energies)), "OriCUTCPKernel",
+                        keep=(inp, energies))
 
 
 def _fft_batches(data):

@@ -46,6 +46,9 @@ GPTBKernel *createKernel(const std::string &name)
     if (name == "cp") {
         auto *ori = new OriCPKernel(10);
         k = new GPTBKernel(10, "cp", "gptb_cp", ori, gptbGrid(name), gptbBlock(name, 128), 0, oriBlocks(name, ori));
+    } else if (name == "cutcp") {
+        auto *ori = new OriCUTCPKernel(11);
+        k = new GPTBKernel(11, "cutcp", "gptb_cutcp", ori, gptbGrid(name), gptbBlock(name, 128), 0, oriBlocks(name, ori));
     } else if (name == "fft") {
         auto *ori = new OriFFTKernel(12);
         k = new GPTBKernel(12, "fft", "gptb_fft", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));

@@ -519,6 +519,70 @@ int tacker_gptb_fft(float *data, int batches, int block_start, int block_end, in
     return run_gptb_once(new OriFFTKernel(0, data, batches), block_start, block_end, launch_grid, launch_block, stream);
 }
 
+namespace {
+int check_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, const float *regionZeroAddr, int rx,
+                int ry, int rz)
+{
+    if (!binZeroAddr || !regionZeroAddr || binDim_x <= 0 || binDim_y <= 0 || !(h > 0) || rx <= 0 || ry <= 0 || rz <= 0)
+        return fail(TK_ERROR_INVALID_VALUE, "cutcp: bad arguments");
+    if ((long long)rx * ry * rz * REGION_SIZE >= (1ll << 31))
+        return fail(TK_ERROR_UNSUPPORTED, "cutcp: a lattice of 2^31 points or more");
+    return TK_SUCCESS;
+}
+}  // namespace
+
+int tacker_cutcp_prepare_input(const float *atoms, int natoms, const float lo[3], int nx, int ny, int nz, float h,
+                               float cutoff, int binDim[3], int *padding, float *bins, int *nbr, int *nbr_len,
+                               int counts[2])
+{
+    if ((natoms > 0 && !atoms) || natoms < 0 || !lo || nx <= 0 || ny <= 0 || nz <= 0 || !(h > 0) || !(cutoff > 0) || !binDim ||
+        !padding || !nbr_len)
+        return fail(TK_ERROR_INVALID_VALUE, "cutcp_prepare_input: bad arguments");
+    return guarded([&]() -> int {
+        CutcpBins out;
+        const char *why = nullptr;
+        if (!cutcpPrepareInput(atoms, natoms, lo, nx, ny, nz, h, cutoff, &out, &why)) return fail(TK_ERROR_UNSUPPORTED, why);
+        for (int d = 0; d < 3; ++d) binDim[d] = out.binDim[d];
+        *padding = out.padding;
+        *nbr_len = (int)out.nbrlist.size() / 3;
+        if (bins) std::copy(out.bins.begin(), out.bins.end(), bins);
+        if (nbr) std::copy(out.nbrlist.begin(), out.nbrlist.end(), nbr);
+        if (counts) counts[0] = out.extra, counts[1] = out.excluded;
+        return TK_SUCCESS;
+    });
+}
+
+int tacker_cutcp_set_neighbours(const int *ijk, int len)
+{
+    REQUIRE_INIT();
+    if (len < 0 || len > NBRLIST_MAXLEN || (len > 0 && !ijk))
+        return fail(TK_ERROR_INVALID_VALUE, "cutcp: neighbour list length out of range");
+    const int rc = cutcpSetNeighbours(ijk, len);
+    return rc ? fail(rc, "cutcp: loading the neighbour list failed") : rc;
+}
+
+int tacker_ori_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2, float inv_cutoff2,
+                     float *regionZeroAddr, int rx, int ry, int rz, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_cutcp(binDim_x, binDim_y, binZeroAddr, h, regionZeroAddr, rx, ry, rz);
+    if (rc) return rc;
+    return run_once(new OriCUTCPKernel(0, binDim_x, binDim_y, const_cast<float *>(binZeroAddr), h, cutoff2, inv_cutoff2,
+                                       regionZeroAddr, rx, ry, rz), stream);
+}
+
+int tacker_gptb_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2, float inv_cutoff2,
+                      float *regionZeroAddr, int rx, int ry, int rz, int block_start, int block_end, int launch_grid,
+                      int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_cutcp(binDim_x, binDim_y, binZeroAddr, h, regionZeroAddr, rx, ry, rz);
+    if (rc) return rc;
+    return run_gptb_once(new OriCUTCPKernel(0, binDim_x, binDim_y, const_cast<float *>(binZeroAddr), h, cutoff2,
+                                            inv_cutoff2, regionZeroAddr, rx, ry, rz),
+                         block_start, block_end, launch_grid, launch_block, stream);
+}
+
 int tacker_cp_set_atoms(const float *atoms_host, int count, float zplane)
 {
     REQUIRE_INIT();
@@ -645,6 +709,19 @@ int tacker_mix_tzgemm_sgemm(const float *sA, const float *sB, float *sC, int sM,
                         launch_block, stream);
 }
 
+int tacker_mix_tzgemm_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2,
+                            float inv_cutoff2, float *regionZeroAddr, int rx, int ry, int rz, int be_start, int be_end,
+                            const void *A, const void *B, float *C, int M, int N, int K, int tile_start, int tile_end,
+                            const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_cutcp(binDim_x, binDim_y, binZeroAddr, h, regionZeroAddr, rx, ry, rz);
+    if (rc) return rc;
+    return run_mix_once(new OriCUTCPKernel(0, binDim_x, binDim_y, const_cast<float *>(binZeroAddr), h, cutoff2,
+                                           inv_cutoff2, regionZeroAddr, rx, ry, rz),
+                        be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
 int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_end, const void *A, const void *B, float *C,
                           int M, int N, int K, int tile_start, int tile_end, const char *variant, int launch_grid,
                           int launch_block, tkStream_t stream)
@@ -719,7 +796,7 @@ tacker_kernel_t tacker_create_kernel(const char *name)
         fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
         return nullptr;
     }
-    static const char *known[] = {"cp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil", "tzgemm"};
+    static const char *known[] = {"cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil", "tzgemm"};
     bool ok = false;
     for (auto k : known) ok |= (strcmp(k, name) == 0);
     if (!ok) {
@@ -761,6 +838,14 @@ tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const float *y,
 {
     CREATE(check_mriq(numK, x, y, z, Qr, Qi, numX), new OriMRIQKernel(0, numK, x, y, z, Qr, Qi, numX));
 }
+tacker_kernel_t tacker_ori_cutcp_create(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2,
+                                        float inv_cutoff2, float *regionZeroAddr, int rx, int ry, int rz)
+{
+    CREATE(check_cutcp(binDim_x, binDim_y, binZeroAddr, h, regionZeroAddr, rx, ry, rz),
+           new OriCUTCPKernel(0, binDim_x, binDim_y, const_cast<float *>(binZeroAddr), h, cutoff2, inv_cutoff2,
+                              regionZeroAddr, rx, ry, rz));
+}
+
 tacker_kernel_t tacker_ori_fft_create(float *data, int batches)
 {
     CREATE(check_fft(data, batches), new OriFFTKernel(0, data, batches));
@@ -1138,7 +1223,7 @@ tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const ch
         fail(TK_ERROR_INVALID_VALUE, "tacker_task_manager_create: bad arguments");
         return nullptr;
     }
-    static const char *known[] = {"cp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"};
+    static const char *known[] = {"cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"};
     bool ok1 = false, ok2 = !be2 || !*be2;
     for (auto k : known) {
         ok1 |= strcmp(k, be1) == 0;

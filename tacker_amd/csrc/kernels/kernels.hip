@@ -12,6 +12,7 @@
 
 #include "../../../include/tacker_amd.h"
 #include "cp_role.h"
+#include "cutcp_role.h"
 #include "dnn_kernels.h"
 #include "fft_role.h"
 #include "lbm_role.h"
@@ -99,6 +100,20 @@ extern "C" __global__ __launch_bounds__(128) void ori_sgemm(float *A, float *B, 
     __shared__ __align__(16) float stage[2][64];
     tk::sgemm_thread(A, B, C, nullptr, NORMAL_M, NORMAL_N, NORMAL_K, blockIdx.x * SGEMM_TILE_M + mid,
                      blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K, (tk::sgemm_lds_float *)&stage[mid >> 6][0]);
+}
+
+// grid (regions along x, y, z), block (8,2,8): a wavefront per half region
+// (src/ori_kernel/cutcp_kernel.cu:19-158; zRegionIndex_t is not read there either)
+extern "C" __global__ __launch_bounds__(CUTCP_BLOCK_THREADS) void ori_cutcp(int binDim_x, int binDim_y, float *binZeroAddr,
+                                                                            float h, float cutoff2, float inv_cutoff2,
+                                                                            float *regionZeroAddr, int zRegionIndex_t)
+{
+    (void)zRegionIndex_t;
+    const int tid = (threadIdx.z * blockDim.y + threadIdx.y) * blockDim.x + threadIdx.x;
+    tk::cutcp_half_region(binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2, regionZeroAddr, (int)gridDim.x,
+                          (int)gridDim.y, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z,
+                          __builtin_amdgcn_readfirstlane(tid >> 6),
+                          (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
 }
 
 // grid (transforms), block 64: a wavefront per transform where the reference has a block of 128 threads
@@ -251,6 +266,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ori_mrif", (const void *)ori_mrif, ctx);
     insert("ori_sgemm", (const void *)ori_sgemm, ctx);
     insert("ori_fft", (const void *)ori_fft, ctx);
+    insert("ori_cutcp", (const void *)ori_cutcp, ctx);
     insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);
     insert("tz_clear_words", (const void *)tz_clear_words, ctx);
     insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);
@@ -284,6 +300,16 @@ extern "C" int tk_device_symbol(const char *name, const void **symbol, size_t *b
     if (__builtin_strcmp(name, "atominfo") == 0) {
         *symbol = (const void *)&atominfo;
         *bytes = sizeof(atominfo);
+        return TK_SUCCESS;
+    }
+    if (__builtin_strcmp(name, "NbrListLen") == 0) {
+        *symbol = (const void *)&NbrListLen;
+        *bytes = sizeof(NbrListLen);
+        return TK_SUCCESS;
+    }
+    if (__builtin_strcmp(name, "NbrList") == 0) {
+        *symbol = (const void *)&NbrList;
+        *bytes = sizeof(NbrList);
         return TK_SUCCESS;
     }
     if (__builtin_strcmp(name, "tz_ws_table") == 0) {

@@ -54,6 +54,7 @@ const std::vector<int> MRIF = {I, I, P, P, P, P, P};
 const std::vector<int> CP = {I, F, P};
 const std::vector<int> SGEMM = {P, P, P, I, I, I};
 const std::vector<int> FFT = {P};
+const std::vector<int> CUTCP = {I, I, P, F, F, F, P, I};
 const std::vector<int> TZ = {P, P, P, I, I, I};
 }  // namespace
 
@@ -81,7 +82,7 @@ int tkMemset(void *ptr, int value, size_t bytes) { memset(ptr, value, bytes); re
 int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset)
 {
     if (strcmp(symbol, "ck") && strcmp(symbol, "c_mrif") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail") &&
-        strcmp(symbol, "tz_ws_table"))
+        strcmp(symbol, "tz_ws_table") && strcmp(symbol, "NbrListLen") && strcmp(symbol, "NbrList"))
         return TK_ERROR_NOT_FOUND;
     auto &buf = g_symbols[symbol];
     if (buf.size() < offset + bytes) buf.resize(offset + bytes);
@@ -190,6 +191,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ori_mrif", MRIF);
         add("ori_sgemm", SGEMM);
         add("ori_fft", FFT);
+        add("ori_cutcp", CUTCP);
         add("gptb_tzgemm", cat(TZ, trailer(true)));
         add("gptb_tzgemm@large", cat(TZ, trailer(true)));
         add("gptb_tzgemm_scratch", cat(cat(TZ, {P}), trailer(true)));
@@ -201,6 +203,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("gptb_mrif", cat(MRIF, trailer(true)));
         add("gptb_sgemm", cat(SGEMM, trailer(true)));
         add("gptb_fft", cat(FFT, trailer(true)));
+        add("gptb_cutcp", cat(CUTCP, trailer(true)));
         add("cp_inv_sqrt_selftest", {I, I, P});
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
@@ -211,7 +214,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("pack_fc_input_pooled", {P, I, I, I, P, I, I, P});
         const std::pair<const char *, const std::vector<int> *> bes[] = {
             {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}, {"mrif", &MRIF}, {"sgemm", &SGEMM},
-            {"fft", &FFT}};
+            {"fft", &FFT}, {"cutcp", &CUTCP}};
         static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};
         for (auto &be : bes)
             for (auto v : variants)

@@ -18,7 +18,7 @@ namespace {
 thread_local std::string g_last_hip_error;
 std::mutex g_modules_mutex;
 std::vector<hipModule_t> g_modules;   // code objects loaded through tkModuleLoad
-const char *const kMirroredSymbols[] = {"ck", "c_mrif", "atominfo", "tz_ws_table", "tk_spin_fail"};
+const char *const kMirroredSymbols[] = {"ck", "c_mrif", "atominfo", "NbrListLen", "NbrList", "tz_ws_table", "tk_spin_fail"};
 
 int fold(hipError_t e, const char *what)
 {

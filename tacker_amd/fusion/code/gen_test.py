@@ -84,6 +84,13 @@ def make_inputs(np, torch, ta, be, small):
         batches = 40 if small else 10240
         data = torch.from_numpy(rng.uniform(-1, 1, (batches, 256, 2)).astype(np.float32)).cuda()
         return ta.ori_fft_create(data), batches, [data]
+    if be == "cutcp":
+        n, count = (24, 400) if small else (208, 70000)
+        atoms = np.empty((count, 4), np.float32)
+        atoms[:, :3] = rng.uniform(0, (n - 1) * 0.5, (count, 3))
+        atoms[:, 3] = rng.uniform(0.1, 1, count) * rng.choice([-1, 1], count)
+        inp = ta.CutcpInput(atoms, (0, 0, 0), n, n, n if small else 16, 0.5, 12.0)
+        return ta.ori_cutcp_create(inp, 144.0, 0.006944), inp.blocks(), [inp.energies]
     if be == "sgemm":
         M, N, K = (256, 48, 300) if small else (4096, 4128, 4064)
         A = torch.from_numpy(rng.uniform(0, 1, (K, M)).astype(np.float32)).cuda()

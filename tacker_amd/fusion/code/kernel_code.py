@@ -1,7 +1,7 @@
 """Role descriptions the generator stitches together.
 
 Each entry plays the part of one ``<kernel>_code.py`` of the reference
-(fusion/code/cp_code.py, fft_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
+(fusion/code/cp_code.py, cutcp_code.py, fft_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
 truncated tzgemm_code.py): the kernel's parameter list in reference order and
 how to call its device-side role.  The role bodies themselves live in
 ``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
@@ -89,6 +89,16 @@ ROLES = {
         "needs_sync": False,
         "call": ("tk::fft_role<{waves}>({p}data, {p}grid_dimension_x, {block}, {blocks}, {p}ptb_start_block_pos, "
                  "{p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+    "cutcp": {
+        "gptb": {"symbol": "general_ptb_cutcp", "cite": "src/gptb_kernel/cutcp_kernel.cu:12-183", "attributes": ""},
+        "params": [("int", "binDim_x"), ("int", "binDim_y"), ("float*", "binZeroAddr"), ("float", "h"),
+                   ("float", "cutoff2"), ("float", "inv_cutoff2"), ("float*", "regionZeroAddr"),
+                   ("int", "zRegionIndex_t")],
+        "needs_sync": False,
+        "call": ("tk::cutcp_role({p}binDim_x, {p}binDim_y, {p}binZeroAddr, {p}h, {p}cutoff2, {p}inv_cutoff2, "
+                 "{p}regionZeroAddr, {p}grid_dimension_x, {p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, "
+                 "{p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "cp": {
         "gptb": {"symbol": "g_general_ptb_cp", "cite": "src/gptb_kernel/cp_kernel.cu:8-96", "attributes": ""},

@@ -77,10 +77,10 @@ def test_committed_generated_sources_are_fresh():
 
 
 @pytest.mark.parametrize("be,n_params", [("stencil", 31), ("lbm", 26), ("mriq", 31), ("cp", 27), ("sgemm", 30),
-                                         ("fft", 25)])
+                                         ("fft", 25), ("cutcp", 32)])
 def test_emitted_dispatcher_signature(be, n_params):
     # parameter count = the reference dispatcher's (src/mix_kernel/tzgemm_stencil.cu:281-283 31,
-    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27, tzgemm_sgemm.cu:303 30, tzgemm_fft.cu:988-996 25), order: be first
+    # tzgemm_lbm.cu:352 26, tzgemm_mriq.cu:638 31, tzgemm_cp.cu:994 27, tzgemm_sgemm.cu:303 30, tzgemm_fft.cu:988-996 25, tzgemm_cutcp.cu:345-368 32), order: be first
     text, meta = gen_mix.generate_wg_split(be, 1, 1)
     sig = re.search(r"void (\w+)\(\s*(.*?)\)\s*\{", text, re.S)
     params = [p.strip() for p in sig.group(2).split(",")]
@@ -100,7 +100,8 @@ def test_emitted_dispatcher_signature(be, n_params):
 @pytest.mark.parametrize("name,symbol,n_params", [
     ("tzgemm", "general_ptb_tzgemm", 16), ("stencil", "general_ptb_stencil", 17), ("lbm", "general_ptb_lbm", 12),
     ("mriq", "g_general_ptb_mriq", 17), ("mrif", "general_ptb_mrif", 17), ("cp", "g_general_ptb_cp", 13),
-    ("sgemm", "general_ptb_sgemm", 16), ("fft", "g_general_ptb_fft", 11)])
+    ("sgemm", "general_ptb_sgemm", 16), ("fft", "g_general_ptb_fft", 11),
+    ("cutcp", "general_ptb_cutcp", 18)])
 def test_emitted_gptb_kernel_has_the_reference_name_and_parameter_list(name, symbol, n_params):
     # src/gptb_kernel/<name>_kernel.cu: the original kernel's parameters, then 6 dims, start, step, end,
     # thread_base (e.g. stencil_kernel.cu:3-5: 7 + 10; the names are what src/main.cu:108-125 registers)
@@ -140,10 +141,8 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
     files = gen_run.generate()
     kinfo = json.loads(files["../config/kinfo-gfx950.json"])
     pairs = gen_run.be_pairs()
-    assert pairs == [("cp", "fft"), ("cp", "lbm"), ("cp", "mrif"), ("cp", "mriq"), ("cp", "sgemm"), ("cp", "stencil"),
-                     ("fft", "lbm"), ("fft", "mrif"), ("fft", "mriq"), ("fft", "sgemm"), ("fft", "stencil"),
-                     ("lbm", "mrif"), ("lbm", "mriq"), ("lbm", "sgemm"), ("lbm", "stencil"), ("mrif", "mriq"),
-                     ("mrif", "sgemm"), ("mrif", "stencil"), ("mriq", "sgemm"), ("mriq", "stencil"), ("sgemm", "stencil")]
+    names = ["cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"]
+    assert pairs == [(a, b) for i, a in enumerate(names) for b in names[i + 1:]] and len(pairs) == 28
     # the fft pairs the reference ships: src/mix_kernel/{cp_fft_3_1,fft_lbm_6_1,fft_mriq_3_2,fft_sgemm_1_4,fft_stencil_5_3}.cu
     sig = re.search(r"void fft_lbm_mix_wg_1_1\(\s*(.*?)\)\s*\{", files["mix_kernel/fft_lbm.hip"], re.S)
     names = [q.split()[-1] for q in sig.group(1).split(",")]
@@ -197,7 +196,7 @@ def test_measured_load_ratios_travel_from_profile_ratio_to_the_schedulers_lookup
     assert after["tzgemm_stencil"] == before["tzgemm_stencil"]          # pairs that were not measured keep theirs
     with pytest.raises(SystemExit):                                    # a pair the generator does not know
         bad = tmp_path / "bad.json"
-        bad.write_text(json.dumps({"stretch": 1.0, "device": "x", "pairs": {"tzgemm_cutcp": {"by_k": {}}}}))
+        bad.write_text(json.dumps({"stretch": 1.0, "device": "x", "pairs": {"tzgemm_tpacf": {"by_k": {}}}}))
         profile_ratio.apply(str(bad))
     kinfo_text = gen_run.generate()["../config/kinfo-gfx950.json"]
     kinfo = json.loads(kinfo_text)

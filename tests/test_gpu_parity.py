@@ -809,9 +809,20 @@ def _small_be(name):
     if name == "fft":
         data = dev(fft_inputs())
         return ta.ori_fft_create(data), data.shape[0], [data]
+    if name == "cutcp":
+        inp = ta.CutcpInput(cutcp_atoms(), (0, 0, 0), 24, 16, 16, 0.5, 12.0)
+        return ta.ori_cutcp_create(inp, 144.0, 0.006944), inp.blocks(), [inp.energies]
     ta.cp_set_atoms(cp_atoms(), 0.0)
     g = torch.zeros((32, 512), device="cuda:0")
     return ta.ori_cp_create(64, 0.1, g), ta.cp_blocks(512, 32), [g]
+
+
+def cutcp_atoms():
+    rng = np.random.default_rng(37)
+    a = np.empty((300, 4), np.float32)
+    a[:, :3] = rng.uniform(0, 7.5, (300, 3))
+    a[:, 3] = rng.uniform(0.1, 1, 300) * rng.choice([-1, 1], 300)
+    return a
 
 
 def fft_inputs():
@@ -833,7 +844,8 @@ def sgemm_inputs():
 BE_PAIRS = [("cp", "lbm"), ("cp", "mriq"), ("cp", "stencil"), ("lbm", "mriq"), ("lbm", "stencil"), ("mriq", "stencil"),
             ("cp", "mrif"), ("lbm", "mrif"), ("mrif", "mriq"), ("mrif", "stencil"), ("cp", "sgemm"), ("lbm", "sgemm"),
             ("mrif", "sgemm"), ("mriq", "sgemm"), ("sgemm", "stencil"), ("cp", "fft"), ("fft", "lbm"), ("fft", "mrif"),
-            ("fft", "mriq"), ("fft", "sgemm"), ("fft", "stencil")]
+            ("fft", "mriq"), ("fft", "sgemm"), ("fft", "stencil"), ("cp", "cutcp"), ("cutcp", "fft"), ("cutcp", "lbm"),
+            ("cutcp", "mrif"), ("cutcp", "mriq"), ("cutcp", "sgemm"), ("cutcp", "stencil")]
 
 
 @pytest.mark.parametrize("first,second", BE_PAIRS)
@@ -883,6 +895,10 @@ def _small_be_matches_oracle(name, outs):
         return np.array_equal(host(outs[0]).view(np.uint32), oracle.sgemm(*sgemm_inputs()).view(np.uint32))
     if name == "fft":
         return fft_close(host(outs[0]), oracle.fft(fft_inputs()).astype(np.float64))
+    if name == "cutcp":
+        prep = oracle.cutcp_prepare(cutcp_atoms(), (0, 0, 0), 24, 16, 16, 0.5, 12.0)
+        want = oracle.cutcp(prep, 0.5, 144.0, 0.006944, (3, 2, 2)).astype(np.float64)
+        return bool(np.all(np.abs(host(outs[0]) - want) <= 2e-4 + 2e-5 * np.abs(want)))
     want = oracle.cp(oracle.cp_atoms_to_const(cp_atoms(), 0.0), np.zeros((32, 512), np.float32))
     return np.array_equal(host(outs[0]).view(np.uint32), want.view(np.uint32))
 

@@ -448,7 +448,7 @@ def test_create_mix_kernel_is_memoised_and_uses_the_creator_kernels(fake):
     assert (as_int(l["args"][8]), as_int(l["args"][10])) == (0, 18000)           # lbm rows of 120x120x150
     assert (as_int(l["args"][24]), as_int(l["args"][26])) == (0, 16384)          # mri-q: 1024 voxel blocks x 16 k chunks
     assert (as_int(l["args"][18]), as_int(l["args"][19])) == (1024, 16)          # its grid_dimension_x, _y
-    for bad in (b"mriq_lbm", b"lbm", b"tzgemm_stencil", b"cutcp_lbm"):
+    for bad in (b"mriq_lbm", b"lbm", b"tzgemm_stencil", b"lbm_tpacf"):
         assert not fake.tacker_create_mix_kernel(bad)
 
 
