@@ -101,6 +101,19 @@ def pair_leg(ta, torch, np, name, stream):
         label = "tzgemm 2048^3 + sgemm 4096x4128x4064 fp32 (reference mix tzgemm_sgemm)"
         reset = sC.zero_        # C = 2 C + 2 A B doubles with every pass: start every timed round from zero
         n = 50
+    elif name == "cutcp":   # cutoff Coulomb potential, the Creator's instance (src/ori_kernel/cutcp_kernel.cu:181-263)
+        n_pts, count = 208, 70000
+        atoms = np.empty((count, 4), np.float32)
+        atoms[:, :3] = rng.uniform(0, (n_pts - 1) * 0.5, (count, 3))
+        atoms[:, 3] = rng.uniform(0.1, 1, count) * rng.choice([-1, 1], count)
+        inp = ta.CutcpInput(atoms, (0, 0, 0), n_pts, n_pts, n_pts, 0.5, 12.0, regions=(26, 26, 2))
+        be_ori = ta.ori_cutcp_create(inp, 144.0, 0.006944)
+        nblk = inp.blocks()
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        # atom-point pairs: 335 neighbour bins of each of the 1352 regions, their atoms, 512 points
+        filled = float(np.count_nonzero(inp.host_bins[..., 3])) / inp.host_bins[..., 3].size * 8
+        work = {"bound": "valu", "pairs": nblk * 512.0 * len(inp.nbr) * filled}
+        label = "tzgemm 2048^3 + cutcp 208^3 lattice, 70000 atoms, 26x26x2 regions (reference mix tzgemm_cutcp)"
     elif name == "fft":     # Parboil FFT, 10240 transforms of 256 points (the Creator's instance, src/ori_kernel/fft_kernel.cu:87-115)
         batches = 10240
         source = torch.from_numpy(rng.uniform(-1, 1, (batches, 256, 2)).astype(np.float32)).cuda()
@@ -456,7 +469,7 @@ def main():
     if not args.no_extras:
         out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
         out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream)
-                              for name in ("lbm", "mriq", "cp", "mrif", "sgemm", "fft")}
+                              for name in ("lbm", "mriq", "cp", "mrif", "sgemm", "fft", "cutcp")}
         if not args.no_lc:
             out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")

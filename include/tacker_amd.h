@@ -279,10 +279,16 @@ TK_API int tacker_cutcp_set_neighbours(const int *ijk, int len);
  * src/gptb_kernel/cutcp_kernel.cu:12-183): the cutoff potential of the binned atoms on regions_x x
  * regions_y x regions_z regions of 8 x 8 x 8 lattice points, 512 floats per region, region (x, y, z)
  * at ((z regions_y + y) regions_x + x) * 512.  binZeroAddr points at bin (0, 0, 0) of the lattice,
- * behind the padding bins (device memory, read only).  One block position per region, in the order
- * of the reference's GPTB kernel (x slowest).  A wavefront serves half a region (launch_block a
+ * behind the padding bins (device memory, read only).  Block positions of the GPTB form: the regions
+ * in the order of the reference's GPTB kernel (x slowest) by the parts of TACKER_CUTCP_NBR_CHUNK
+ * entries of the neighbour list loaded last, position p adding part p / regions to region
+ * p % regions; a part other than the first goes on from the energies in memory.
+ * [0, tacker_cutcp_blocks(...)) equals ori_cutcp bit for bit, and so does any sequence of launches
+ * whose ranges tile it in ascending order.  A wavefront serves half a region (launch_block a
  * multiple of 64).  The hardware's reciprocal square root stands for CUDA's rsqrtf: results agree
  * with the reference's within rounding, not bit for bit. */
+#define TACKER_CUTCP_NBR_CHUNK 32
+TK_API int tacker_cutcp_blocks(int regions_x, int regions_y, int regions_z);
 TK_API int tacker_ori_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2,
                             float inv_cutoff2, float *regionZeroAddr, int regions_x, int regions_y,
                             int regions_z, tkStream_t stream);

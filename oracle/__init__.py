@@ -48,7 +48,7 @@ def _declare(l):
                                    C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_stencil.argtypes = [C.c_float, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_sgemm_gptb.argtypes = [_f32p, _f32p, _f32p, _f32p] + [C.c_int] * 9
-    l.orc_cutcp_gptb.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_void_p, _i32p] + [C.c_int] * 6
+    l.orc_cutcp_gptb.argtypes = [C.c_int, C.c_int, C.c_void_p, C.c_float, C.c_float, C.c_float, C.c_void_p, _i32p] + [C.c_int] * 7
     l.orc_cutcp_prepare.argtypes = [_f32p, C.c_int, _f32p, C.c_int, C.c_int, C.c_int, C.c_float, C.c_float, _i32p, _i32p,
                                     C.c_void_p, C.c_void_p, _i32p]
     l.orc_fft_gptb.argtypes = [_f32p, C.c_int, C.c_int, C.c_int]
@@ -307,20 +307,32 @@ def cutcp_prepare(atoms, lo, nx, ny, nz, h, cutoff):
             "extra": int(counts[0]), "excluded": int(counts[1])}
 
 
-def cutcp(prep, h, cutoff2, inv_cutoff2, regions, start=0, end=None, out=None):
-    """Energies [regions z][y][x][8][8][8] float32 (point (x, y, z) of a region at [z][y][x]) of the block
-    positions [start, end) of a (regions x, y, z) grid; other regions keep what ``out`` holds (zeros)."""
+CUTCP_NBR_CHUNK = 32
+
+
+def cutcp_positions(regions, nbr_len, chunk=CUTCP_NBR_CHUNK):
+    return regions[0] * regions[1] * regions[2] * max(1, -(-nbr_len // chunk))
+
+
+def cutcp(prep, h, cutoff2, inv_cutoff2, regions, start=0, end=None, out=None, parts=1, chunk=CUTCP_NBR_CHUNK):
+    """Energies [regions z][y][x][8][8][8] float32 (point (x, y, z) of a region at [z][y][x]) after the block
+    positions [start, end) of the (regions) x (parts) grid: parts=1, a position is a region's whole neighbour
+    list in ascending order (the reference's kernel); parts='chunks', the list is dealt round-robin into
+    ceil(len / chunk) parts and position p adds part p // regions (entries part, part + parts, ...) to region
+    p % regions, going on from the energies in ``out``.  Other regions keep what ``out`` holds (zeros)."""
     rx, ry, rz = regions
     bins = prep["bins"]
     c = prep["padding"]
     bdx, bdy = prep["binDim"][0], prep["binDim"][1]
     zero = bins.ctypes.data + (((c * bdy + c) * bdx + c) * 32) * 4
     res = np.zeros((rz, ry, rx, 8, 8, 8), np.float32) if out is None else np.array(out, np.float32, order="C")
-    if end is None:
-        end = rx * ry * rz
     nbr = np.ascontiguousarray(prep["nbr"], np.int32)
+    if parts == "chunks":
+        parts = max(1, -(-len(nbr) // chunk))
+    if end is None:
+        end = rx * ry * rz * parts
     lib().orc_cutcp_gptb(bdx, bdy, zero, h, cutoff2, inv_cutoff2, res.ctypes.data, nbr.reshape(-1), len(nbr), rx, ry, rz,
-                         start, end)
+                         parts, start, end)
     return res
 
 

@@ -837,42 +837,55 @@ ORC_API void orc_fft_source(float *data, int values)
  * centre = floor((8 r + 4) * h / 4) per dimension.  1.0f / sqrtf stands for CUDA's rsqrtf (an
  * approximation of about an ulp on either device).  Energies are stored, not accumulated.
  *
- * Positions [start, end): position p is region (p / (gdy gdz), (p / gdz) % gdy, p % gdz). */
+ * Positions [start, end) of a grid of regions (columns) by parts of the list (rows; parts = 1: a
+ * position is a region's whole list in ascending order, the reference's kernel): position p adds part
+ * (p / regions) % parts, the entries part, part + parts, part + 2 parts, ..., to region r = p % regions =
+ * (r / (gdy gdz), (r / gdz) % gdy, r % gdz).  Part 0 starts from zero, other parts from the energies
+ * the region holds.  Positions of one region are applied in ascending order. */
 ORC_API void orc_cutcp_gptb(int binDim_x, int binDim_y, const float *binZero, float h, float cutoff2, float inv_cutoff2,
-                            float *regionZero, const int *nbr, int nbr_len, int gdx, int gdy, int gdz, int start, int end)
+                            float *regionZero, const int *nbr, int nbr_len, int gdx, int gdy, int gdz, int parts,
+                            int start, int end)
 {
+    const int regions = gdx * gdy * gdz;
 #pragma omp parallel for schedule(dynamic)
-    for (int pos = start; pos < end; pos++) {
-        const int xr = (pos / (gdy * gdz)) % gdx, yr = (pos / gdz) % gdy, zr = pos % gdz;
+    for (int r = 0; r < regions; r++) {
+        const int xr = r / (gdy * gdz), yr = (r / gdz) % gdy, zr = r % gdz;
         float *region = regionZero + (size_t)((zr * gdy + yr) * gdx + xr) * 512;
         const int bx = (int)floorf((8 * xr + 4) * h * 0.25f);
         const int by = (int)floorf((8 * yr + 4) * h * 0.25f);
         const int bz = (int)floorf((8 * zr + 4) * h * 0.25f);
-        for (int tid = 0; tid < 128; tid++) {
-            const int tx = tid & 7, ty = (tid >> 3) & 1, tz = tid >> 4;
-            const float x = (8 * xr + tx) * h, y = (8 * yr + ty) * h, z = (8 * zr + tz) * h;
-            float energy[4] = {0.f, 0.f, 0.f, 0.f};
-            for (int n = 0; n < nbr_len; n++) {
-                const int i = bx + nbr[3 * n], j = by + nbr[3 * n + 1], k = bz + nbr[3 * n + 2];
-                const float *bin = binZero + ((long long)(k * binDim_y + j) * binDim_x + i) * 32;
-                for (int a = 0; a < 8; a++) {
-                    const float aq = bin[4 * a + 3];
-                    if (0.f == aq) break;
-                    const float dx = bin[4 * a] - x;
-                    const float dz = bin[4 * a + 2] - z;
-                    const float dxdz2 = dx * dx + dz * dz;
-                    float dy = bin[4 * a + 1] - y;
-                    for (int e = 0; e < 4; e++) {
-                        const float r2 = dy * dy + dxdz2;
-                        if (r2 < cutoff2) {
-                            const float s = (1.f - r2 * inv_cutoff2);
-                            energy[e] += aq * (1.0f / sqrtf(r2)) * s * s;
+        int first = start + ((r - start % regions) + regions) % regions;
+        for (int pos = first; pos < end; pos += regions) {
+            const int part = (pos / regions) % parts;
+            for (int tid = 0; tid < 128; tid++) {
+                const int tx = tid & 7, ty = (tid >> 3) & 1, tz = tid >> 4;
+                const float x = (8 * xr + tx) * h, y = (8 * yr + ty) * h, z = (8 * zr + tz) * h;
+                float *mine = region + (tid >> 4) * 64 + (tid & 15);
+                float energy[4] = {0.f, 0.f, 0.f, 0.f};
+                if (part > 0)
+                    for (int e = 0; e < 4; e++) energy[e] = mine[16 * e];
+                for (int n = part; n < nbr_len; n += parts) {
+                    const int i = bx + nbr[3 * n], j = by + nbr[3 * n + 1], k = bz + nbr[3 * n + 2];
+                    const float *bin = binZero + ((long long)(k * binDim_y + j) * binDim_x + i) * 32;
+                    for (int a = 0; a < 8; a++) {
+                        const float aq = bin[4 * a + 3];
+                        if (0.f == aq) break;
+                        const float dx = bin[4 * a] - x;
+                        const float dz = bin[4 * a + 2] - z;
+                        const float dxdz2 = dx * dx + dz * dz;
+                        float dy = bin[4 * a + 1] - y;
+                        for (int e = 0; e < 4; e++) {
+                            const float r2 = dy * dy + dxdz2;
+                            if (r2 < cutoff2) {
+                                const float s = (1.f - r2 * inv_cutoff2);
+                                energy[e] += aq * (1.0f / sqrtf(r2)) * s * s;
+                            }
+                            dy -= 2.0f * h;
                         }
-                        dy -= 2.0f * h;
                     }
                 }
+                for (int e = 0; e < 4; e++) mine[16 * e] = energy[e];
             }
-            for (int e = 0; e < 4; e++) region[(tid >> 4) * 64 + (tid & 15) + 16 * e] = energy[e];
         }
     }
 }

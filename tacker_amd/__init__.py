@@ -73,6 +73,7 @@ def _declare(lib):
     cut = [i, i, vp, f, f, f, vp, i, i, i]
     lib.tacker_cutcp_prepare_input.argtypes = [vp, i, vp, i, i, i, f, f, vp, vp, vp, vp, vp, vp]
     lib.tacker_cutcp_set_neighbours.argtypes = [vp, i]
+    lib.tacker_cutcp_blocks.argtypes = [i, i, i]
     lib.tacker_ori_cutcp.argtypes = cut + [vp]
     lib.tacker_gptb_cutcp.argtypes = cut + [i, i, i, i, vp]
     lib.tacker_mix_tzgemm_cutcp.argtypes = cut + [i, i] + gemm
@@ -506,7 +507,8 @@ class CutcpInput:
         check(lib().tacker_cutcp_set_neighbours(self.nbr.ctypes.data, len(self.nbr)), "tacker_cutcp_set_neighbours")
 
     def blocks(self):
-        return self.regions[0] * self.regions[1] * self.regions[2]
+        """block positions of the GPTB form: regions x parts of the neighbour list (as loaded last)"""
+        return lib().tacker_cutcp_blocks(*self.regions)
 
     def args(self, cutoff2, inv_cutoff2, energies=None):
         e = self.energies if energies is None else energies

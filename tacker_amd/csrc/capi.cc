@@ -561,6 +561,13 @@ int tacker_cutcp_set_neighbours(const int *ijk, int len)
     return rc ? fail(rc, "cutcp: loading the neighbour list failed") : rc;
 }
 
+int tacker_cutcp_blocks(int rx, int ry, int rz)
+{
+    static_assert(TACKER_CUTCP_NBR_CHUNK == CUTCP_NBR_CHUNK, "public and device chunk sizes must agree");
+    if (rx <= 0 || ry <= 0 || rz <= 0) return 0;
+    return rx * ry * rz * cutcpNeighbourParts();
+}
+
 int tacker_ori_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2, float inv_cutoff2,
                      float *regionZeroAddr, int rx, int ry, int rz, tkStream_t stream)
 {

@@ -12,3 +12,6 @@
 #define NBRLIST_MAXLEN (NBRLIST_DIM * NBRLIST_DIM * NBRLIST_DIM)
 // threads of the reference's block (8, 2, 8): each takes 4 points of its region, 2 apart in y
 #define CUTCP_BLOCK_THREADS 128
+// bins of the neighbour list one block position of the GPTB form walks (the reference's block stages
+// BIN_CACHE_MAXLEN bins at a time: the same granularity)
+#define CUTCP_NBR_CHUNK BIN_CACHE_MAXLEN

@@ -110,10 +110,13 @@ extern "C" __global__ __launch_bounds__(CUTCP_BLOCK_THREADS) void ori_cutcp(int 
 {
     (void)zRegionIndex_t;
     const int tid = (threadIdx.z * blockDim.y + threadIdx.y) * blockDim.x + threadIdx.x;
+    // the neighbour list in the order of the GPTB form's parts: entries p, p + parts, ... for p = 0, 1, ...
+    const int len = NbrListLen;
+    const int parts = max(1, (len + CUTCP_NBR_CHUNK - 1) / CUTCP_NBR_CHUNK);
     tk::cutcp_half_region(binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2, regionZeroAddr, (int)gridDim.x,
                           (int)gridDim.y, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z,
                           __builtin_amdgcn_readfirstlane(tid >> 6),
-                          (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+                          (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)), 0, parts, parts, len);
 }
 
 // grid (transforms), block 64: a wavefront per transform where the reference has a block of 128 threads

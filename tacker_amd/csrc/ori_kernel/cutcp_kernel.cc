@@ -76,12 +76,21 @@ bool cutcpPrepareInput(const float *atoms, int natoms, const float lo[3], int nx
     return true;
 }
 
+static int g_neighbour_len = 0;   // what the device table holds
+
 int cutcpSetNeighbours(const int *ijk, int len)
 {
     if (len < 0 || len > NBRLIST_MAXLEN) return TK_ERROR_INVALID_VALUE;
     int rc = tkMemcpyToSymbol("NbrListLen", &len, sizeof(int), 0);
     if (!rc && len) rc = tkMemcpyToSymbol("NbrList", ijk, (size_t)len * 3 * sizeof(int), 0);
+    if (!rc) g_neighbour_len = len;
     return rc;
+}
+
+int cutcpNeighbourParts()
+{
+    const int parts = (g_neighbour_len + CUTCP_NBR_CHUNK - 1) / CUTCP_NBR_CHUNK;
+    return parts < 1 ? 1 : parts;
 }
 
 OriCUTCPKernel::OriCUTCPKernel(int id)
@@ -145,7 +154,11 @@ void OriCUTCPKernel::bind(int rx, int ry, int rz)
 {
     if (rx <= 0 || ry <= 0 || rz <= 0) logger.ERROR("cutcp: the grid of regions must not be empty");
     OriCUTCPParamsStruct *p = CUTCPKernelParams;
-    launchGridDim = dim3(rx, ry, rz);
+    // Block positions: (x, y, z / parts) = the reference's grid of regions
+    // (src/ori_kernel/cutcp_kernel.cu:246-249), the parts of the neighbour list folded into z as the
+    // slowest index.  The natural launch below runs the regions, each through the whole list.
+    regionsZ = rz;
+    launchGridDim = dim3(rx, ry, rz * cutcpNeighbourParts());
     launchBlockDim = dim3(8, 2, 8);
     kernelParams = {&p->binDim_x, &p->binDim_y, &p->binZeroAddr, &p->h, &p->cutoff2, &p->inv_cutoff2, &p->regionZeroAddr,
                     &p->zRegionIndex_t};
@@ -158,6 +171,7 @@ void OriCUTCPKernel::bind(int rx, int ry, int rz)
 void OriCUTCPKernel::executeImpl(cudaStream_t stream)
 {
     if (!kernelFunc) logger.ERROR("load kernel {ori_cutcp} failed!");
-    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, launchGridDim.raw(), launchBlockDim.raw(),
+    const dim3 regions(launchGridDim.x, launchGridDim.y, regionsZ);
+    TK_SAFE_CALL(tkLaunchKernel(this->kernelFunc, regions.raw(), launchBlockDim.raw(),
                                 (void **)this->kernelParams.data(), 0, stream));
 }

@@ -38,6 +38,9 @@ bool cutcpPrepareInput(const float *atoms, int natoms, const float lo[3], int nx
                        CutcpBins *out, const char **why);
 // cudaMemcpyToSymbol(NbrListLen / NbrList) (src/ori_kernel/cutcp_kernel.cu:241-242)
 int cutcpSetNeighbours(const int *ijk, int len);
+// parts of CUTCP_NBR_CHUNK entries the neighbour list loaded last falls into (1 for an empty list):
+// the rows of the GPTB position grid of kernel objects built from now on
+int cutcpNeighbourParts();
 
 class OriCUTCPKernel : public Kernel {
 public:
@@ -46,6 +49,7 @@ public:
     // does not ship; here 70000 atoms with seeded uniform positions in the box and charges in [-1, 1).
     explicit OriCUTCPKernel(int id);
     // caller-owned bins and energies; the neighbour list must have been loaded (cutcpSetNeighbours)
+    // and must not change its number of parts while the object is in use
     OriCUTCPKernel(int id, int binDim_x, int binDim_y, float *binZeroAddr, float h, float cutoff2, float inv_cutoff2,
                    float *regionZeroAddr, int regions_x, int regions_y, int regions_z);
     ~OriCUTCPKernel() override;
@@ -61,4 +65,5 @@ private:
     void loadKernel() override {}
     void bind(int rx, int ry, int rz);
     OriCUTCPParamsStruct *CUTCPKernelParams = nullptr;
+    int regionsZ = 0;   // launchGridDim.z also counts the parts of the neighbour list
 };

@@ -61,9 +61,9 @@ KERNEL_INFO = {
     # 10240 transforms of 256 points, a wavefront each; 2 KiB of LDS per wavefront
     "fft": {"register": 40, "shared_memory": 8192, "blocksize": 256, "solo_ptb_blks": 8,
             "ori_blks": 10240},
-    # 26 x 26 x 2 regions of 8 x 8 x 8 lattice points, two wavefronts each
+    # 26 x 26 x 2 regions of 8 x 8 x 8 lattice points (two wavefronts each) x 11 parts of 32 neighbour bins
     "cutcp": {"register": 48, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
-              "ori_blks": 1352},
+              "ori_blks": 14872},
     # 16384 blocks of 128 x 8 points x 4 parts of the unrolled x points
     "cp": {"register": 40, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
            "ori_blks": 65536},

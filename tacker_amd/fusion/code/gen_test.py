@@ -89,7 +89,8 @@ def make_inputs(np, torch, ta, be, small):
         atoms = np.empty((count, 4), np.float32)
         atoms[:, :3] = rng.uniform(0, (n - 1) * 0.5, (count, 3))
         atoms[:, 3] = rng.uniform(0.1, 1, count) * rng.choice([-1, 1], count)
-        inp = ta.CutcpInput(atoms, (0, 0, 0), n, n, n if small else 16, 0.5, 12.0)
+        # the benchmark instance computes the two lowest layers of regions of the 208^3 lattice
+        inp = ta.CutcpInput(atoms, (0, 0, 0), n, n, n, 0.5, 12.0, regions=None if small else (26, 26, 2))
         return ta.ori_cutcp_create(inp, 144.0, 0.006944), inp.blocks(), [inp.energies]
     if be == "sgemm":
         M, N, K = (256, 48, 300) if small else (4096, 4128, 4064)

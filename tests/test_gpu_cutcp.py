@@ -3,7 +3,7 @@ src/gptb_kernel/cutcp_kernel.cu, src/mix_kernel/tzgemm_cutcp.cu): against the or
 bins within |d| <= 2e-4 + 2e-5 |ref| (the hardware's reciprocal square root here, 1 / sqrtf there, CUDA's
 rsqrtf in the reference: approximations of an ulp each, summed over hundreds of atoms) and against the
 float64 sum over the atom list; the natural launch, the GPTB form over any tiling of its positions and
-every fused variant give the same bits as each other; the host's binning equals the oracle's exactly."""
+every fused variant give the same bits as each other (positions = regions x parts of the neighbour list); the host's binning equals the oracle's exactly."""
 import numpy as np
 import pytest
 import torch
@@ -94,10 +94,13 @@ def test_any_tiling_of_the_positions_gives_the_one_kernel(seed):
         ta.gptb_cutcp(inp, C2, INV_C2, e, a, b, launch_grid=int(rng.choice([1, 5, 64, 256])),
                       launch_block=int(rng.choice([64, 128, 256])))
     assert np.array_equal(bits(e), bits(whole))
-    # a partial range writes its regions only, in the reference's position order (x slowest)
+    assert n == oracle.cutcp_positions(inp.regions, len(inp.nbr)) == inp.regions[0] * inp.regions[1] * inp.regions[2] * 11
+    # a partial range touches its regions only, in the reference's position order (x slowest); positions 1 and 2
+    # are the first part of the neighbour list (entries 0, 11, 22, ...) of regions 1 and 2
     e = torch.full_like(inp.energies, -3.0)
     ta.gptb_cutcp(inp, C2, INV_C2, e, 1, 3)
-    want = oracle.cutcp(prep, H, C2, INV_C2, inp.regions, 1, 3, out=np.full(tuple(e.shape), -3.0, np.float32))
+    want = oracle.cutcp(prep, H, C2, INV_C2, inp.regions, 1, 3, out=np.full(tuple(e.shape), -3.0, np.float32),
+                        parts="chunks")
     got = host(e)
     assert np.array_equal(got == -3.0, want == -3.0) and close(got, want)
 
@@ -135,7 +138,7 @@ def test_creator_object_is_the_references_instance_on_seeded_atoms():
     # (src/ori_kernel/cutcp_kernel.cu:181-263)
     k = ta.create_kernel("cutcp")
     info = k.info()
-    assert (info["ptb_start"], info["ptb_end"], info["ori_grid_x"], info["ori_grid_y"]) == (0, 26 * 26 * 2, 26, 26)
+    assert (info["ptb_start"], info["ptb_end"], info["ori_grid_x"], info["ori_grid_y"]) == (0, 26 * 26 * 2 * 11, 26, 26)
     assert (k.param(0, "int"), k.param(1, "int")) == (32, 32)
     assert abs(k.param(3, "float") - 0.5) < 1e-7 and abs(k.param(4, "float") - 144.0) < 1e-4
     assert abs(k.param(5, "float") - 0.006944) < 1e-8

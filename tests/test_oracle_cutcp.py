@@ -141,3 +141,44 @@ def test_positions_follow_the_gptb_index_and_leave_other_regions_alone():
     for a, b in ((0, 5), (5, 6), (6, 18)):
         tiled = oracle.cutcp(prep, H, 144.0, 0.006944, (3, 3, 2), a, b, out=tiled)
     assert np.array_equal(tiled, whole)
+
+
+def test_any_ascending_tiling_of_the_region_by_part_grid_is_the_one_walk():
+    # 335 neighbour bins dealt round-robin into 11 parts: position p adds part p // regions (entries part,
+    # part + 11, ...) to region p % regions, the energies resting in the output between parts
+    n = 24
+    atoms = atoms_in_box(600, (n - 1) * H, seed=5)
+    prep = oracle.cutcp_prepare(atoms, (0, 0, 0), n, n, 16, H, CUTOFF)
+    regions = (3, 3, 2)
+    whole = oracle.cutcp(prep, H, 144.0, 0.006944, regions)
+    total = oracle.cutcp_positions(regions, len(prep["nbr"]))
+    assert total == 18 * 11
+    rng = np.random.default_rng(6)
+    for _ in range(3):
+        cuts = sorted(set(rng.integers(0, total + 1, 5).tolist()) | {0, total})
+        out = np.full((2, 3, 3, 8, 8, 8), 7.0, np.float32)              # part 0 does not read what is there
+        for a, b in zip(cuts, cuts[1:]):
+            out = oracle.cutcp(prep, H, 144.0, 0.006944, regions, a, b, out=out, parts="chunks")
+        if _ == 0:
+            first = out
+        assert np.array_equal(out.view(np.uint32), first.view(np.uint32))     # whatever the tiling: the same bits
+        # ... and the one ascending walk of the reference up to the order of the additions
+        assert np.all(np.abs(out - whole) <= 1e-5 + 2e-6 * np.abs(whole))
+    # one position = one part of one region: float64 over the atoms of exactly those 32 bins
+    pos = 18 * 4 + 7                                                    # part 4 of region 7 = (x 1, y 0, z 1)
+    got = oracle.cutcp(prep, H, 144.0, 0.006944, regions, pos, pos + 1, parts="chunks")
+    # part 4 starts from the energies in memory (zero here) and adds its bins only: entries 4, 15, 26, ...
+    bins, c = prep["bins"], prep["padding"]
+    centre = [int(np.floor((8 * r + 4) * H * 0.25)) for r in (1, 0, 1)]
+    members = []
+    for i, j, k in prep["nbr"][4::11]:
+        slot = bins[centre[2] + k + c, centre[1] + j + c, centre[0] + i + c]
+        for a in slot:
+            if a[3] == 0:
+                break
+            members.append(a)
+    want = brute_force(np.array(members, np.float32).reshape(-1, 4), regions, H, 144.0, 0.006944)
+    assert len(members) > 10 and np.all(np.abs(got[1, 0, 1] - want[1, 0, 1]) <= 1e-4 + 2e-5 * np.abs(want[1, 0, 1]))
+    other = np.ones_like(got, bool)
+    other[1, 0, 1] = False
+    assert np.all(got[other] == 0.0)
