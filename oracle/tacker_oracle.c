@@ -33,6 +33,11 @@
  *   orc_sgemm_gptb        float64 matrix product, integer operands (exact), one-hot A, the
  *                         fused multiply-add per step against exact rationals, any
  *                         ascending tiling of the position grid (tests/test_oracle_sgemm.py).
+ *   orc_cutcp*            float64 sum over the atom list without bins, single-charge closed form and
+ *                         exact zero outside the cutoff, binning against a Python dictionary,
+ *                         neighbour list by its inequality, the 32 x 32 bin grid the reference
+ *                         hard-codes, any ascending tiling of the region-by-part grid
+ *                         (tests/test_oracle_cutcp.py).
  *   orc_fft*              the float64 transform (numpy's FFT and the defining sum), unit
  *                         impulses = rows of the DFT matrix, pure tones, linearity,
  *                         Parseval, position wrap; the input stream against the cp atoms'
