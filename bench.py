@@ -112,7 +112,7 @@ def pair_leg(ta, torch, np, name, stream):
         tz, tiles, flop = gemm(2048, 2048, 2048)
         # atom-point pairs: 335 neighbour bins of each of the 1352 regions, their atoms, 512 points
         filled = float(np.count_nonzero(inp.host_bins[..., 3])) / inp.host_bins[..., 3].size * 8
-        work = {"bound": "valu", "pairs": nblk * 512.0 * len(inp.nbr) * filled}
+        work = {"bound": "valu", "pairs": 26 * 26 * 2 * 512.0 * len(inp.nbr) * filled}
         label = "tzgemm 2048^3 + cutcp 208^3 lattice, 70000 atoms, 26x26x2 regions (reference mix tzgemm_cutcp)"
     elif name == "fft":     # Parboil FFT, 10240 transforms of 256 points (the Creator's instance, src/ori_kernel/fft_kernel.cu:87-115)
         batches = 10240
