@@ -354,6 +354,9 @@ def main():
                     help="skip the other pairs (configs 3, 4) and the co-location latency leg (config 5)")
     ap.add_argument("--queries", type=int, default=1000, help="latency-critical queries of the co-location leg")
     ap.add_argument("--no-lc", action="store_true", help="skip the co-location latency legs (config 5)")
+    ap.add_argument("--pairs", default="lbm,mriq,cp,mrif,sgemm,fft,cutcp",
+                    help="best-effort kernels of the other-pairs legs (comma separated); with a list of its own the "
+                         "tzgemm shapes leg is skipped too (profiling runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (no sharding, no collectives); use --gpus 1",
@@ -467,9 +470,9 @@ def main():
         "wall_s_timed_region": round(t_wall, 3),
     }
     if not args.no_extras:
-        out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
-        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream)
-                              for name in ("lbm", "mriq", "cp", "mrif", "sgemm", "fft", "cutcp")}
+        if args.pairs == ap.get_default("pairs"):
+            out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
+        out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in args.pairs.split(",") if name}
         if not args.no_lc:
             out["lc_colocation"] = lc_leg(ta, torch, np, args.queries)
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")
