@@ -119,3 +119,32 @@ def test_large_tile_gemm_and_a_fused_kernel_from_code_objects():
     assert np.array_equal(bits(s_got), oracle.stencil(C0, C1, A0, A0).view(np.uint32))
     assert np.array_equal(bits(c_got), bits(want))
     assert ta.spin_fail_flag() == 0
+
+
+def test_cutcp_and_fft_from_the_code_object():
+    # cutcp reads its neighbour list from two device symbols (NbrListLen, NbrList): the copies inside a code
+    # object follow the library's, whether the list was loaded before the object or after; fft carries its
+    # twiddle table in the object itself
+    rng = np.random.default_rng(61)
+    atoms = np.empty((300, 4), np.float32)
+    atoms[:, :3] = rng.uniform(0, 7.5, (300, 3))
+    atoms[:, 3] = rng.uniform(0.1, 1, 300)
+    inp = ta.CutcpInput(atoms, (0, 0, 0), 16, 16, 16, 0.5, 12.0)          # loads the list: the modules are already there
+    want = torch.zeros_like(inp.energies)
+    ta.gptb_cutcp(inp, 144.0, 0.006944, want)
+    for name in ("kernels", "kernels_after_cutcp"):
+        if name != "kernels":
+            ta.register_module(name, ta.CODE_OBJECT_PATH)                 # loaded after the list: filled at load
+        got = torch.full_like(inp.energies, -1.0)
+        k = ta.gptb_create(ta.ori_cutcp_create(inp, 144.0, 0.006944, got), 0, 0, 0, inp.blocks())
+        k.use_module(name, "general_ptb_cutcp")
+        k.execute()
+        assert np.array_equal(bits(got), bits(want)), name
+    d = rng.uniform(-1, 1, (70, 256, 2)).astype(np.float32)
+    a, b = dev(d), dev(d)
+    ta.gptb_fft(a)
+    k = ta.gptb_create(ta.ori_fft_create(b), 0, 0, 0, 70)
+    k.use_module("kernels", "g_general_ptb_fft")
+    k.execute()
+    assert np.array_equal(bits(a), bits(b))
+    assert ta.spin_fail_flag() == 0
