@@ -243,7 +243,7 @@ TK_API int tacker_gptb_mrif(int numK, const float *x, const float *y, const floa
  * library binds to C when a kernel object is built on it (tacker_tzgemm_release_workspaces frees
  * it).  [0, tacker_sgemm_blocks(M, N, K)) equals ori_sgemm bit for bit, and so does any sequence
  * of launches whose ranges tile it in ascending order. */
-#define TACKER_SGEMM_K_CHUNK 256
+#define TACKER_SGEMM_K_CHUNK 64
 TK_API int tacker_sgemm_blocks(int M, int N, int K);
 TK_API int tacker_ori_sgemm(const float *A, const float *B, float *C, int M, int N, int K,
                             tkStream_t stream);

@@ -255,7 +255,7 @@ def cp(atominfo, energygrid, gridspacing=0.1, start=0, end=None, parts=1):
 
 
 # --------------------------------------------------------------------------- sgemm
-SGEMM_K_CHUNK = 256
+SGEMM_K_CHUNK = 64
 
 
 def sgemm_positions(M, N, K, chunk=SGEMM_K_CHUNK):

@@ -9,4 +9,4 @@
 #define SGEMM_ALPHA 2.0f
 #define SGEMM_BETA 2.0f
 // k steps one block position of the GPTB form adds to its 128 x 16 partial results
-#define SGEMM_K_CHUNK 256
+#define SGEMM_K_CHUNK 64

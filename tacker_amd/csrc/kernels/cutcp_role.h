@@ -33,6 +33,14 @@ typedef __attribute__((address_space(4))) const float4_t cutcp_const_float4;
 // the same wherever the atoms are).  A range that does not start with part 0 goes on from the
 // energies in memory, where the range before it left them (a float stored and reloaded is unchanged,
 // so consecutive ranges give the bits of one walk through all parts).
+//
+// AHEAD = false: the atoms of a bin by scalar loads, issued when the bin's turn comes -- the faster
+// form when the SIMD has other waves to run meanwhile (the plain kernel: 300 against 330 us).
+// AHEAD = true: the 32 floats of a bin in 32 lanes of one register, fetched with one vector load
+// while the bin before it is walked, the atoms handed out with v_readlane -- a wave that has its
+// SIMD almost to itself (a slice of positions next to a GEMM) does not wait for the L2 once per
+// bin.  The atoms' bits, and so the results, are the same either way.
+template <bool AHEAD>
 __device__ __forceinline__ void cutcp_half_region(int binDim_x, int binDim_y, const float *binZeroAddr, float h,
                                                   float cutoff2, float inv_cutoff2, float *regionZeroAddr, int gdx,
                                                   int gdy, int xr, int yr, int zr, int half, int lane, int part_begin,
@@ -57,50 +65,82 @@ __device__ __forceinline__ void cutcp_half_region(int binDim_x, int binDim_y, co
         energy2 = mine[32];
         energy3 = mine[48];
     }
-    for (int part = part_begin; part < part_end; ++part) {
-        for (int n = part; n < len; n += parts) {
-            const int i = bx + NbrList[n][0];
-            const int j = by + NbrList[n][1];
-            const int k = bz + NbrList[n][2];
-            const long long bin = ((long long)(k * binDim_y + j) * binDim_x + i) * BIN_DEPTH;
-            // wave-uniform address of read-only data: scalar loads
-            const cutcp_const_float4 *atoms =
-                (const cutcp_const_float4 *)(reinterpret_cast<const float4_t *>(binZeroAddr) + bin);
+    const float4_t *bins = reinterpret_cast<const float4_t *>(binZeroAddr);
+    const auto bin_of = [&](int n) -> const float4_t * {
+        const int i = bx + NbrList[n][0];
+        const int j = by + NbrList[n][1];
+        const int k = bz + NbrList[n][2];
+        return bins + ((long long)(k * binDim_y + j) * binDim_x + i) * BIN_DEPTH;
+    };
+    const auto lane_of = [](float v, int l) -> float {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+    };
+// one atom {ax_, ay_, az_, aq_} (wave-uniform) against the lane's four points
+#define CUTCP_ATOM(ax_, ay_, az_, aq_)                                                            \
+    {                                                                                             \
+        const float dx = (ax_) - x;                                                               \
+        const float dz = (az_) - z;                                                               \
+        const float dxdz2 = dx * dx + dz * dz;                                                    \
+        float dy = (ay_) - y;                                                                     \
+        float r2 = dy * dy + dxdz2;                                                               \
+        if (r2 < cutoff2) {                                                                       \
+            const float s = (1.f - r2 * inv_cutoff2);                                             \
+            energy0 += (aq_) * __builtin_amdgcn_rsqf(r2) * s * s;                                 \
+        }                                                                                         \
+        dy -= two_h;                                                                              \
+        r2 = dy * dy + dxdz2;                                                                     \
+        if (r2 < cutoff2) {                                                                       \
+            const float s = (1.f - r2 * inv_cutoff2);                                             \
+            energy1 += (aq_) * __builtin_amdgcn_rsqf(r2) * s * s;                                 \
+        }                                                                                         \
+        dy -= two_h;                                                                              \
+        r2 = dy * dy + dxdz2;                                                                     \
+        if (r2 < cutoff2) {                                                                       \
+            const float s = (1.f - r2 * inv_cutoff2);                                             \
+            energy2 += (aq_) * __builtin_amdgcn_rsqf(r2) * s * s;                                 \
+        }                                                                                         \
+        dy -= two_h;                                                                              \
+        r2 = dy * dy + dxdz2;                                                                     \
+        if (r2 < cutoff2) {                                                                       \
+            const float s = (1.f - r2 * inv_cutoff2);                                             \
+            energy3 += (aq_) * __builtin_amdgcn_rsqf(r2) * s * s;                                 \
+        }                                                                                         \
+    }
+    if (AHEAD) {
+        // entry of the walk after (part, n): n + parts, or the first entry of the next part
+        int part = part_begin, n = part_begin;
+        while (part < part_end && n >= len) n = ++part;   // parts beyond a short list are empty
+        float cur = part < part_end ? reinterpret_cast<const float *>(bin_of(n))[lane & 31] : 0.f;
+        while (part < part_end) {
+            int part_next = part, n_next = n + parts;
+            while (part_next < part_end && n_next >= len) n_next = ++part_next;
+            const float nxt = part_next < part_end ? reinterpret_cast<const float *>(bin_of(n_next))[lane & 31] : 0.f;
 #pragma unroll
             for (int a = 0; a < BIN_DEPTH; ++a) {
-                const float4_t atom = atoms[a];
-                const float aq = atom.w;
+                const float aq = lane_of(cur, 4 * a + 3);
                 if (0.f == aq) break;   // no more atoms in this bin
-                const float dx = atom.x - x;
-                const float dz = atom.z - z;
-                const float dxdz2 = dx * dx + dz * dz;
-                float dy = atom.y - y;
-                float r2 = dy * dy + dxdz2;
-                if (r2 < cutoff2) {
-                    const float s = (1.f - r2 * inv_cutoff2);
-                    energy0 += aq * __builtin_amdgcn_rsqf(r2) * s * s;
-                }
-                dy -= two_h;
-                r2 = dy * dy + dxdz2;
-                if (r2 < cutoff2) {
-                    const float s = (1.f - r2 * inv_cutoff2);
-                    energy1 += aq * __builtin_amdgcn_rsqf(r2) * s * s;
-                }
-                dy -= two_h;
-                r2 = dy * dy + dxdz2;
-                if (r2 < cutoff2) {
-                    const float s = (1.f - r2 * inv_cutoff2);
-                    energy2 += aq * __builtin_amdgcn_rsqf(r2) * s * s;
-                }
-                dy -= two_h;
-                r2 = dy * dy + dxdz2;
-                if (r2 < cutoff2) {
-                    const float s = (1.f - r2 * inv_cutoff2);
-                    energy3 += aq * __builtin_amdgcn_rsqf(r2) * s * s;
+                CUTCP_ATOM(lane_of(cur, 4 * a), lane_of(cur, 4 * a + 1), lane_of(cur, 4 * a + 2), aq)
+            }
+            cur = nxt;
+            part = part_next;
+            n = n_next;
+        }
+    } else {
+        for (int part = part_begin; part < part_end; ++part) {
+            for (int n = part; n < len; n += parts) {
+                // wave-uniform address of read-only data: scalar loads
+                const cutcp_const_float4 *atoms = (const cutcp_const_float4 *)bin_of(n);
+#pragma unroll
+                for (int a = 0; a < BIN_DEPTH; ++a) {
+                    const float4_t atom = atoms[a];
+                    const float aq = atom.w;
+                    if (0.f == aq) break;   // no more atoms in this bin
+                    CUTCP_ATOM(atom.x, atom.y, atom.z, aq)
                 }
             }
         }
     }
+#undef CUTCP_ATOM
     mine[0] = energy0;
     mine[16] = energy1;
     mine[32] = energy2;
@@ -110,6 +150,7 @@ __device__ __forceinline__ void cutcp_half_region(int binDim_x, int binDim_y, co
 // One phase of a launch: regions [region_lo, region_hi) (in position order) each walk parts
 // [part_begin, part_end) of the neighbour list.  A wavefront serves the half regions it owns: first_owned,
 // first_owned + stride, ...
+template <bool AHEAD>
 __device__ __forceinline__ void cutcp_phase(int region_lo, int region_hi, int part_begin, int part_end, int parts,
                                             int len, int binDim_x,
                                             int binDim_y, const float *binZeroAddr, float h, float cutoff2,
@@ -124,8 +165,8 @@ __device__ __forceinline__ void cutcp_phase(int region_lo, int region_hi, int pa
         const int cu = __builtin_amdgcn_readfirstlane(c);
         const int r = cu >> 1;
         // region r of the reference's GPTB order, x slowest (src/gptb_kernel/cutcp_kernel.cu:61-63)
-        cutcp_half_region(binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2, regionZeroAddr, gdx, gdy,
-                          r / (gdy * gdz), (r / gdz) % gdy, r % gdz, cu & 1, lane, part_begin, part_end, parts, len);
+        cutcp_half_region<AHEAD>(binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2, regionZeroAddr, gdx, gdy,
+                                 r / (gdy * gdz), (r / gdz) % gdy, r % gdz, cu & 1, lane, part_begin, part_end, parts, len);
     }
 }
 
@@ -136,6 +177,7 @@ __device__ __forceinline__ void cutcp_phase(int region_lo, int region_hi, int pa
 // whole launch, which walks the rows in order, so the parts of a region are added in ascending order
 // without any synchronisation, whole rows that follow each other are one run through their parts, and
 // a range that runs past the grid wraps.
+template <bool AHEAD = false>
 __device__ __forceinline__ void cutcp_role(int binDim_x, int binDim_y, const float *binZeroAddr, float h, float cutoff2,
                                            float inv_cutoff2, float *regionZeroAddr, int grid_dimension_x,
                                            int grid_dimension_y, int grid_dimension_z, int role_block, int role_blocks,
@@ -155,7 +197,7 @@ __device__ __forceinline__ void cutcp_role(int binDim_x, int binDim_y, const flo
     const auto chunk_begin = [&](int row) { return row % gy; };
     const auto chunk_end = [&](int row) { return row % gy + 1; };
 #define CUTCP_PHASE(lo_, hi_, pb_, pe_)                                                                          \
-    cutcp_phase(lo_, hi_, pb_, pe_, gy, len, binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2,           \
+    cutcp_phase<AHEAD>(lo_, hi_, pb_, pe_, gy, len, binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2,           \
                 regionZeroAddr, grid_dimension_x, grid_dimension_y, gdz, first_owned, stride, lane)
     const int first_row = start / gx;
     const int last_row = (end - 1) / gx;

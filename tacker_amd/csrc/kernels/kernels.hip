@@ -91,15 +91,15 @@ extern "C" __global__ __launch_bounds__(256) void ori_mrif(int numK, int kGlobal
     tk::mrif_voxel(numK, x, y, z, outR, outI, blockIdx.x * KERNEL_FH_THREADS_PER_BLOCK + threadIdx.x);
 }
 
-// grid (M/128, N/16), block (16,8): a thread's row of C is its flattened id in the block
-// (src/ori_kernel/sgemm_kernel.cu:9-44)
-extern "C" __global__ __launch_bounds__(128) void ori_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N,
-                                                            int NORMAL_K)
+// grid (M/128, N/16), block (16,4): one wavefront where the reference has 128 threads, a lane owning the
+// rows of the reference's threads l and l + 64 (src/ori_kernel/sgemm_kernel.cu:9-44)
+extern "C" __global__ __launch_bounds__(64) void ori_sgemm(float *A, float *B, float *C, int NORMAL_M, int NORMAL_N,
+                                                           int NORMAL_K)
 {
     const int mid = threadIdx.y * blockDim.x + threadIdx.x;
-    __shared__ __align__(16) float stage[2][64];
+    __shared__ __align__(16) float stage[64];
     tk::sgemm_thread(A, B, C, nullptr, NORMAL_M, NORMAL_N, NORMAL_K, blockIdx.x * SGEMM_TILE_M + mid,
-                     blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K, (tk::sgemm_lds_float *)&stage[mid >> 6][0]);
+                     blockIdx.y * SGEMM_TILE_N, 0, NORMAL_K, (tk::sgemm_lds_float *)&stage[0]);
 }
 
 // grid (regions along x, y, z), block (8,2,8): a wavefront per half region
@@ -113,7 +113,7 @@ extern "C" __global__ __launch_bounds__(CUTCP_BLOCK_THREADS) void ori_cutcp(int 
     // the neighbour list in the order of the GPTB form's parts: entries p, p + parts, ... for p = 0, 1, ...
     const int len = NbrListLen;
     const int parts = max(1, (len + CUTCP_NBR_CHUNK - 1) / CUTCP_NBR_CHUNK);
-    tk::cutcp_half_region(binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2, regionZeroAddr, (int)gridDim.x,
+    tk::cutcp_half_region<false>(binDim_x, binDim_y, binZeroAddr, h, cutoff2, inv_cutoff2, regionZeroAddr, (int)gridDim.x,
                           (int)gridDim.y, (int)blockIdx.x, (int)blockIdx.y, (int)blockIdx.z,
                           __builtin_amdgcn_readfirstlane(tid >> 6),
                           (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)), 0, parts, parts, len);

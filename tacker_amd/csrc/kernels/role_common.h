@@ -133,6 +133,121 @@ struct RoleSpinSync {
     }
 };
 
+// RoleSpinSync that hands over to the hardware barrier once the waves of the other role have ended.
+//
+// The hardware barrier counts the waves of the workgroup that have not terminated.  While waves of
+// the other role run it cannot serve one role; once they have all ended it serves the waves that are
+// left, and it costs nothing where the arrival counter costs an LDS atomic and a poll per barrier (the
+// GEMM role's K loop runs a fifth slower on the counter).  Three LDS words: the arrival counter,
+// `alive` = waves of the other role that have not finished (each subtracts 1 when its work is done,
+// role_wave_done), and `switch_at`.  The role's first wave is the decider: when it has seen alive == 0
+// it writes the index of the barrier it is about to arrive at into switch_at, then arrives.  Every wave
+// reads switch_at after each barrier it passes on the counter and takes the hardware barrier for all
+// barriers behind index switch_at.  The write precedes the decider's arrival and LDS serves a wave's
+// operations in order, so every wave that passes barrier switch_at reads it, and waves that read it
+// earlier still take that barrier on the counter: all waves change over at the same barrier.  A wave
+// whose poll runs into its limit changes over too (and raises the failure word): from then on it can
+// only hold the others up at the hardware barrier until they give up as well, never spin on.
+struct RoleHandoverSync {
+    static constexpr bool kSplit = false;   // wait() is the whole barrier
+    unsigned counter_addr;   // LDS byte address of the three words
+    unsigned waves;
+    unsigned expected;       // arrivals that complete the current barrier = its index
+    unsigned gave_up;
+    unsigned *fail;
+    unsigned spin_limit;
+    unsigned hw;             // the same in all lanes: 1 = hardware barrier from now on
+    unsigned announce;       // the same in all lanes: decider has seen the other role's waves gone
+    unsigned decider;        // the same in all lanes: this is the role's first wave
+    __device__ __forceinline__ RoleHandoverSync(unsigned *words, unsigned w, bool first_wave, unsigned *f,
+                                                unsigned limit = (1u << 24))
+        : counter_addr((unsigned)(size_t)(__attribute__((address_space(3))) unsigned *)words), waves(w), expected(0),
+          gave_up(0), fail(f), spin_limit(limit), hw(0), announce(0), decider(first_wave ? 1u : 0u) {}
+
+    // what thread 0 of the workgroup stores before the roles part ways: no arrival, other_waves
+    // waves of the other role at work, no change-over in sight
+    static __device__ __forceinline__ void init(unsigned *words, unsigned other_waves)
+    {
+        words[0] = 0u;
+        words[1] = other_waves;
+        words[2] = 0x7fffffffu;
+    }
+
+    __device__ __forceinline__ void arrive() {}
+    // The hardware barrier is the path the K loop falls through; the counter's code sits out of its
+    // way.  (Every instruction at the barrier is a gap in the wave's MFMA stream: with the change-over
+    // test and the counter's code in line the loop ran 12 % slower than with the bare s_barrier.)
+    __device__ __forceinline__ void wait()
+    {
+        if (__builtin_expect(__builtin_amdgcn_readfirstlane(hw) != 0u, 1)) {
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            on_the_counter();
+        }
+    }
+    // arrive, poll until every wave of the role has, then look whether this was the barrier to change over at
+    __device__ __forceinline__ void on_the_counter()
+    {
+        expected += waves;
+        unsigned now, at, alive, left, uni;
+        unsigned long long saved_exec;
+        asm volatile("s_mov_b32 %[left], %[limit]\n\t"
+                     "v_readfirstlane_b32 %[uni], %[announce]\n\t"
+                     "s_mov_b64 %[saved], exec\n\t"
+                     "s_mov_b64 exec, 1\n\t"
+                     "s_cmp_eq_u32 %[uni], 0\n\t"
+                     "s_cbranch_scc1 8f\n\t"
+                     "ds_write_b32 %[addr], %[index] offset:8\n"
+                     "8:\n\t"
+                     "ds_add_u32 %[addr], %[one]\n\t"
+                     "s_mov_b64 exec, %[saved]\n"
+                     "4:\n\t"                              // poll
+                     "ds_read_b32 %[now], %[addr]\n\t"
+                     "s_waitcnt lgkmcnt(0)\n\t"
+                     "v_sub_u32 %[now], %[now], %[index]\n\t"
+                     "v_cmp_gt_i32 vcc, 0, %[now]\n\t"
+                     "s_cbranch_vccz 2f\n\t"
+                     "s_sub_u32 %[left], %[left], 1\n\t"
+                     "s_cmp_lg_u32 %[left], 0\n\t"
+                     "s_cbranch_scc1 4b\n"
+                     "2:\n\t"                              // passed (or gave up): change over from here?
+                     "ds_read_b32 %[at], %[addr] offset:8\n\t"
+                     "ds_read_b32 %[alive], %[addr] offset:4\n\t"
+                     "s_waitcnt lgkmcnt(0)\n\t"
+                     "v_sub_u32 %[at], %[index], %[at]\n\t"
+                     "v_cmp_le_i32 vcc, 0, %[at]\n\t"
+                     "v_cndmask_b32_e64 %[hw], 0, 1, vcc\n\t"
+                     "v_cmp_eq_u32 vcc, 0, %[alive]\n\t"
+                     "v_cndmask_b32_e64 %[announce], 0, 1, vcc"
+                     : [now] "=&v"(now), [at] "=&v"(at), [alive] "=&v"(alive), [left] "=&s"(left), [uni] "=&s"(uni),
+                       [saved] "=&s"(saved_exec), [hw] "=&v"(hw), [announce] "+v"(announce)
+                     : [addr] "v"(counter_addr), [index] "v"(expected), [one] "v"(1u), [limit] "s"(spin_limit)
+                     : "vcc", "scc", "memory");
+        announce &= decider;
+        const unsigned out_of_polls = (left == 0u);
+        gave_up |= out_of_polls;
+        hw |= out_of_polls;
+    }
+    __device__ __forceinline__ void sync()
+    {
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        wait();
+    }
+    __device__ __forceinline__ void finish()
+    {
+        if (gave_up && fail) __hip_atomic_fetch_or(fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
+
+// What a wave of the other role calls when its work is done (every wave of it, on every path): one
+// less to wait for before the hardware barrier can serve the role that synchronises.
+__device__ __forceinline__ void role_wave_done(unsigned *words)
+{
+    const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    if (lane == 0) __hip_atomic_fetch_sub(words + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+
 // Where a workgroup of a workgroup-split fused launch belongs.
 // The launch has gridDim.x = groups * (a + b) workgroups.  Hardware hands
 // consecutive workgroup ids to the 8 XCDs round-robin, so roles are assigned by

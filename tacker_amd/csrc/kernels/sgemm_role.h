@@ -40,20 +40,29 @@ namespace tk {
 typedef __attribute__((address_space(3))) float sgemm_lds_float;
 typedef __attribute__((address_space(3))) float4_t sgemm_lds_float4;
 
-// thread's row m, columns n0 .. n0 + 15, k in [k_begin, k_end); n0, k_begin, k_end wave-uniform;
-// stage: this wave's 64 floats of LDS
+// rows a lane owns of a block of C: one wavefront serves the 128 rows of a block
+#define SGEMM_ROWS_PER_LANE (SGEMM_TILE_M / 64)
+
+// The lane's rows m, m + 64 (the reference's threads m and m + 64 of the block), columns
+// n0 .. n0 + 15, k in [k_begin, k_end); n0, k_begin, k_end wave-uniform; stage: this wave's 64
+// floats of LDS.  Every value of B a wave reads back from LDS serves both rows.
 __device__ __forceinline__ void sgemm_thread(const float *__restrict__ A, const float *__restrict__ B,
                                              float *__restrict__ C, float *__restrict__ W, int M, int N, int K,
                                              int m, int n0, int k_begin, int k_end, sgemm_lds_float *stage)
 {
-    float c[SGEMM_TILE_N];
+    constexpr int R = SGEMM_ROWS_PER_LANE;
+    float c[R][SGEMM_TILE_N];
     const size_t t = (size_t)M * n0 + m;   // of C and of the workspace: column n0, row m
     if (k_begin == 0) {
 #pragma unroll
-        for (int i = 0; i < SGEMM_TILE_N; ++i) c[i] = 0.0f;
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int i = 0; i < SGEMM_TILE_N; ++i) c[r][i] = 0.0f;
     } else {
 #pragma unroll
-        for (int i = 0; i < SGEMM_TILE_N; ++i) c[i] = W[t + (size_t)i * M];
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int i = 0; i < SGEMM_TILE_N; ++i) c[r][i] = W[t + 64 * r + (size_t)i * M];
     }
     const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));   // whatever the block shape
     // 32-bit element indices (the host refuses matrices of 2^31 elements): fewer scalar registers
@@ -64,6 +73,16 @@ __device__ __forceinline__ void sgemm_thread(const float *__restrict__ A, const 
     int k = k_begin;
     // four k steps per iteration; the next iteration's values of A and B are on their way while
     // this one's are used
+#define SGEMM_READ_ROW(bv_, j_)                                                                   \
+    _Pragma("unroll") for (int q = 0; q < SGEMM_TILE_N / 4; ++q)                                  \
+        bv_[q] = *reinterpret_cast<const sgemm_lds_float4 *>(stage + SGEMM_TILE_N * (j_) + 4 * q);
+#define SGEMM_ROW_FMAS(a_, bv_, j_)                                                               \
+    _Pragma("unroll") for (int r = 0; r < R; ++r)                                                 \
+        _Pragma("unroll") for (int i = 0; i < SGEMM_TILE_N; ++i)                                  \
+            c[r][i] = __builtin_fmaf(a_[r][j_], bv_[i / 4][i % 4], c[r][i]);
+// Row k + j + 1 of the tile is read from LDS while row k + j is multiplied; the scheduling fences
+// keep the compiler from reading all four rows (and the next sets' loads) ahead, which costs
+// registers a fused kernel does not have.
 #define SGEMM_FOUR_STEPS(a_, b_)                                                                  \
     {                                                                                             \
         /* the wave's previous reads of the slot are behind it: LDS serves a wave in order */     \
@@ -71,83 +90,86 @@ __device__ __forceinline__ void sgemm_thread(const float *__restrict__ A, const 
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                    \
         __builtin_amdgcn_wave_barrier();                                                          \
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");                                    \
-        _Pragma("unroll") for (int j = 0; j < 4; ++j)                                             \
-        {                                                                                         \
-            float4_t bv[SGEMM_TILE_N / 4];   /* row k + j of the tile */                          \
-            _Pragma("unroll") for (int q = 0; q < SGEMM_TILE_N / 4; ++q)                          \
-                bv[q] = *reinterpret_cast<const sgemm_lds_float4 *>(stage + SGEMM_TILE_N * j + 4 * q); \
-            _Pragma("unroll") for (int i = 0; i < SGEMM_TILE_N; ++i)                              \
-                c[i] = __builtin_fmaf(a_[j], bv[i / 4][i % 4], c[i]);                             \
-        }                                                                                         \
+        float4_t bv0[SGEMM_TILE_N / 4], bv1[SGEMM_TILE_N / 4];                                    \
+        SGEMM_READ_ROW(bv0, 0)                                                                    \
+        SGEMM_READ_ROW(bv1, 1)                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        SGEMM_ROW_FMAS(a_, bv0, 0)                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        SGEMM_READ_ROW(bv0, 2)                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        SGEMM_ROW_FMAS(a_, bv1, 1)                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        SGEMM_READ_ROW(bv1, 3)                                                                    \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        SGEMM_ROW_FMAS(a_, bv0, 2)                                                                \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        SGEMM_ROW_FMAS(a_, bv1, 3)                                                                \
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");                                    \
         __builtin_amdgcn_wave_barrier();                                                          \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
     }
-// every register set walks its own index, 16 k steps at a time: the only strides are M, 2 M,
-// 3 M, 16 M and 16 N, which keeps the scalar registers of a fused kernel within reach
+// every register set walks its own index, 4 SGEMM_SETS k steps at a time: the only strides are M,
+// 2 M, 3 M and the sets' steps, which keeps the scalar registers of a fused kernel within reach
+#define SGEMM_SETS 2
 #define SGEMM_FETCH(a_, b_, ia_, ib_)                                                             \
-    _Pragma("unroll") for (int j = 0; j < 4; ++j) a_[j] = A[(ia_) + j * M];                       \
+    _Pragma("unroll") for (int r = 0; r < R; ++r)                                                 \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) a_[r][j] = A[(ia_) + 64 * r + j * M];       \
     b_ = B[ib_];                                                                                  \
-    ia_ += 16 * M;                                                                                \
-    ib_ += 16 * N;
+    ia_ += 4 * SGEMM_SETS * M;                                                                    \
+    ib_ += 4 * SGEMM_SETS * N;
     if (k + 4 <= k_end) {
-        // Four register sets take turns: the values of an iteration are fetched four iterations
-        // (16 k steps, a thousand cycles of this wave's own arithmetic) before they are used, so
-        // that a wave with a SIMD to itself -- a short slice next to a GEMM -- is bound by the ALUs
-        // and not by the round trip to the L2.
-        float a0[4], a1[4], a2[4], a3[4], b0, b1, b2, b3;
-        int ia0 = a_at, ia1 = a_at + 4 * M, ia2 = a_at + 8 * M, ia3 = a_at + 12 * M;
-        int ib0 = b_at, ib1 = b_at + 4 * N, ib2 = b_at + 8 * N, ib3 = b_at + 12 * N;
+        // SGEMM_SETS register sets take turns: the values of an iteration (four k steps) are fetched
+        // that many iterations before they are used, so that a wave with a SIMD to itself -- a short
+        // slice next to a GEMM -- is bound by the ALUs and not by the round trip to the L2.
+        constexpr int SETS = SGEMM_SETS;
+        float a[SETS][R][4], b[SETS];
+        int ia[SETS], ib[SETS];
         const int n_iter = (k_end - k) >> 2;
-        SGEMM_FETCH(a0, b0, ia0, ib0)
-        if (n_iter > 1) { SGEMM_FETCH(a1, b1, ia1, ib1) }
-        if (n_iter > 2) { SGEMM_FETCH(a2, b2, ia2, ib2) }
-        if (n_iter > 3) { SGEMM_FETCH(a3, b3, ia3, ib3) }
-        int it = 0;
-        for (; it + 8 <= n_iter; it += 4) {
-            SGEMM_FOUR_STEPS(a0, b0)
-            SGEMM_FETCH(a0, b0, ia0, ib0)
-            SGEMM_FOUR_STEPS(a1, b1)
-            SGEMM_FETCH(a1, b1, ia1, ib1)
-            SGEMM_FOUR_STEPS(a2, b2)
-            SGEMM_FETCH(a2, b2, ia2, ib2)
-            SGEMM_FOUR_STEPS(a3, b3)
-            SGEMM_FETCH(a3, b3, ia3, ib3)
+#pragma unroll
+        for (int s = 0; s < SETS; ++s) {
+            ia[s] = a_at + 4 * s * M;
+            ib[s] = b_at + 4 * s * N;
+            if (s < n_iter) { SGEMM_FETCH(a[s], b[s], ia[s], ib[s]) }
         }
-        // at most seven iterations left: those in the sets, then those fetched meanwhile
-        const int left = n_iter - it;
-        SGEMM_FOUR_STEPS(a0, b0)
-        if (left > 4) { SGEMM_FETCH(a0, b0, ia0, ib0) }
-        if (left > 1) {
-            SGEMM_FOUR_STEPS(a1, b1)
-            if (left > 5) { SGEMM_FETCH(a1, b1, ia1, ib1) }
+        for (int it = 0; it < n_iter; it += SETS) {
+#pragma unroll
+            for (int s = 0; s < SETS; ++s) {
+                if (it + s < n_iter) {   // wave-uniform
+                    SGEMM_FOUR_STEPS(a[s], b[s])
+                    if (it + s + SETS < n_iter) { SGEMM_FETCH(a[s], b[s], ia[s], ib[s]) }
+                }
+            }
         }
-        if (left > 2) {
-            SGEMM_FOUR_STEPS(a2, b2)
-            if (left > 6) { SGEMM_FETCH(a2, b2, ia2, ib2) }
-        }
-        if (left > 3) { SGEMM_FOUR_STEPS(a3, b3) }
-        if (left > 4) { SGEMM_FOUR_STEPS(a0, b0) }
-        if (left > 5) { SGEMM_FOUR_STEPS(a1, b1) }
-        if (left > 6) { SGEMM_FOUR_STEPS(a2, b2) }
         k += 4 * n_iter;
         a_at += 4 * n_iter * M;
     }
 #undef SGEMM_FETCH
 #undef SGEMM_FOUR_STEPS
+#undef SGEMM_READ_ROW
+#undef SGEMM_ROW_FMAS
     // what is left of a k range that is not a multiple of four: values of B by scalar loads
     for (; k < k_end; ++k) {
-        const float av = A[a_at];
         const float *b_row = B + (size_t)k * N + n0;
 #pragma unroll
-        for (int i = 0; i < SGEMM_TILE_N; ++i) c[i] = __builtin_fmaf(av, b_row[i], c[i]);
+        for (int r = 0; r < R; ++r) {
+            const float av = A[a_at + 64 * r];
+#pragma unroll
+            for (int i = 0; i < SGEMM_TILE_N; ++i) c[r][i] = __builtin_fmaf(av, b_row[i], c[r][i]);
+        }
         a_at += M;
     }
-    if (k_end == K) {
 #pragma unroll
-        for (int i = 0; i < SGEMM_TILE_N; ++i) C[t + (size_t)i * M] = C[t + (size_t)i * M] * SGEMM_BETA + SGEMM_ALPHA * c[i];
-    } else {
+    for (int r = 0; r < R; ++r) {
+        const size_t tr = t + 64 * r;
+        if (k_end == K) {
 #pragma unroll
-        for (int i = 0; i < SGEMM_TILE_N; ++i) W[t + (size_t)i * M] = c[i];
+            for (int i = 0; i < SGEMM_TILE_N; ++i)
+                C[tr + (size_t)i * M] = C[tr + (size_t)i * M] * SGEMM_BETA + SGEMM_ALPHA * c[r][i];
+        } else {
+#pragma unroll
+            for (int i = 0; i < SGEMM_TILE_N; ++i) W[tr + (size_t)i * M] = c[r][i];
+        }
     }
 }
 
@@ -170,7 +192,7 @@ __device__ __forceinline__ void sgemm_phase(int block_lo, int block_hi, int k_be
     int b = first_owned;
     if (b < block_lo) b += (block_lo - b + stride - 1) / stride * stride;
     for (; b < block_hi; b += stride) {
-        const int bu = __builtin_amdgcn_readfirstlane(b);   // the 128 threads of a group are whole waves
+        const int bu = __builtin_amdgcn_readfirstlane(b);   // a group is one wavefront
         sgemm_thread(A, B, C, W, M, N, K, (bu % grid_x) * SGEMM_TILE_M + t, (bu / grid_x) * SGEMM_TILE_N, k_begin, k_end,
                      stage);
     }
@@ -183,9 +205,9 @@ __device__ __forceinline__ void sgemm_role(const float *__restrict__ A, const fl
                                            int grid_dimension_y, int grid_dimension_z, int role_block, int role_blocks,
                                            int start, int end, int tid, int role_threads)
 {
-    const int groups_at_once = role_threads / SGEMM_TILE_M;
-    const int slot = tid / SGEMM_TILE_M;
-    const int t = tid % SGEMM_TILE_M;
+    const int groups_at_once = role_threads / 64;   // a wavefront per block
+    const int slot = tid / 64;
+    const int t = tid % 64;
     if (slot >= groups_at_once || start >= end) return;
     const int gx = grid_dimension_x * grid_dimension_y;   // blocks = columns of the position grid
     const int gy = grid_dimension_z;                      // k parts = its rows

@@ -62,7 +62,7 @@ void OriSGEMMKernel::bind()
     // launch below runs the (x, y) blocks, each through its whole k loop.
     const int parts = (p->NORMAL_K + SGEMM_K_CHUNK - 1) / SGEMM_K_CHUNK;
     launchGridDim = dim3(p->NORMAL_M / SGEMM_TILE_M, p->NORMAL_N / SGEMM_TILE_N, parts);
-    launchBlockDim = dim3(SGEMM_TILE_N, SGEMM_TILE_TB_HEIGHT, 1);
+    launchBlockDim = dim3(SGEMM_TILE_N, SGEMM_TILE_TB_HEIGHT / 2, 1);   // one wavefront: a lane owns two of the block's rows
     kernelParams = {&p->A, &p->B, &p->C, &p->NORMAL_M, &p->NORMAL_N, &p->NORMAL_K};
     this->smem = 0;
     if (parts > 1) sgemmWorkspaceFor(p->C, p->NORMAL_M, p->NORMAL_N);

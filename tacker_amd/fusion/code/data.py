@@ -55,9 +55,9 @@ KERNEL_INFO = {
     # 1024 blocks of 256 voxels x 16 chunks of 128 k records
     "mrif": {"register": 44, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
              "ori_blks": 16384},
-    # 32 x 258 blocks of 128 rows x 16 columns of C x 16 parts of 256 k steps (4096 x 4128 x 4064)
+    # 32 x 258 blocks of 128 rows x 16 columns of C x 64 parts of 64 k steps (4096 x 4128 x 4064)
     "sgemm": {"register": 64, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
-              "ori_blks": 132096},
+              "ori_blks": 528384},
     # 10240 transforms of 256 points, a wavefront each; 2 KiB of LDS per wavefront
     "fft": {"register": 40, "shared_memory": 8192, "blocksize": 256, "solo_ptb_blks": 8,
             "ori_blks": 10240},

@@ -15,7 +15,8 @@ so two forms are emitted:
 * ``wave`` -- wave split: every workgroup holds both roles, threads
   ``[0, t0)`` run the first kernel and ``[t0, t0 + t1)`` the second, the way the
   reference does; a role that needs a barrier uses an LDS arrival counter
-  private to its waves (``tk::RoleSpinSync``).
+  private to its waves until the other role's waves have ended, then the
+  hardware barrier (``tk::RoleHandoverSync``).
 """
 from kernel_code import ROLES, gptb_signature, signature
 
@@ -70,6 +71,12 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(
     return text, meta
 
 
+# Template arguments of a role inside a wave-split kernel, where few best-effort waves share the CU
+# with the GEMM: lbm takes two rows per wave to keep enough loads in flight, cutcp fetches every bin
+# of atoms a bin ahead instead of waiting for it.
+WAVE_SPLIT_EXTRA = {"lbm": "<2>", "cutcp": "<true>"}
+
+
 def generate_wave_split(be, be_threads, tz_first=True):
     """Wave-split fused kernel: 256 tzgemm threads + be_threads of ``be`` per workgroup."""
     variant = f"wave_{be_threads}"
@@ -84,11 +91,10 @@ def generate_wave_split(be, be_threads, tz_first=True):
     tz_call = ROLES["tzgemm"]["call"].format(p=p_tz, block="(int)blockIdx.x",
                                              blocks=f"{p_tz}ptb_iter_block_step",
                                              tid=f"(int)threadIdx.x - {tz_lo}", stages="TZ_STAGES", stream_c=_stream_c(be))
-    # few best-effort waves share the CU with the GEMM: lbm takes two rows per wave to keep
-    # enough loads in flight
+    # few best-effort waves share the CU with the GEMM: see WAVE_SPLIT_EXTRA
     be_call = ROLES[be]["call"].format(p=p_be, block="be_block", blocks="be_blocks",
                                        tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads,
-                                       waves=be_threads // 64, extra="<2>" if be == "lbm" else "")
+                                       waves=be_threads // 64, extra=WAVE_SPLIT_EXTRA.get(be, ""))
     tz_cond = (f"threadIdx.x < {tz_threads}" if tz_first else f"threadIdx.x >= {be_threads}")
     name = mix_kernel_name(be, variant)
     unused = _void_unused(sig_be + sig_tz, tz_call + be_call + f"{p_be}ptb_iter_block_step")
@@ -101,13 +107,14 @@ extern "C" __global__ __launch_bounds__({total}) void {name}(
     // flight before each read of the ring.
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES + 16];
     unsigned *tz_arrivals = reinterpret_cast<unsigned *>(tz_lds + TZ_LDS_BYTES);
-    if (threadIdx.x == 0) *tz_arrivals = 0u;
-    __syncthreads();   // the only workgroup-wide barrier: before the roles part ways
+    if (threadIdx.x == 0) tk::RoleHandoverSync::init(tz_arrivals, {be_threads // 64});
+    __syncthreads();   // the only barrier of all waves: before the roles part ways
     if ({tz_cond}) {{
         // One tzgemm wave per SIMD shares it with {be} waves: let the MFMA stream issue
         // whenever it is ready and the {be} waves fill the slots it leaves.
         __builtin_amdgcn_s_setprio(TK_GEMM_WAVE_PRIORITY);
-        tk::RoleSpinSync sync(tz_arrivals, {tz_threads // 64}, &tk_spin_fail);
+        // role barrier: an arrival counter in LDS while {be} waves run, the hardware barrier once they have ended
+        tk::RoleHandoverSync sync(tz_arrivals, {tz_threads // 64}, (int)threadIdx.x - {tz_lo} < 64, &tk_spin_fail);
         {tz_call}
     }} else {{
         // A GEMM that leaves at least half of the workgroups without a tile: the {be} blocks go
@@ -122,6 +129,7 @@ extern "C" __global__ __launch_bounds__({total}) void {name}(
         if (be_block >= 0) {{
             {be_call}
         }}
+        tk::role_wave_done(tz_arrivals);
     }}
 }}
 """

@@ -96,7 +96,7 @@ ROLES = {
                    ("float", "cutoff2"), ("float", "inv_cutoff2"), ("float*", "regionZeroAddr"),
                    ("int", "zRegionIndex_t")],
         "needs_sync": False,
-        "call": ("tk::cutcp_role({p}binDim_x, {p}binDim_y, {p}binZeroAddr, {p}h, {p}cutoff2, {p}inv_cutoff2, "
+        "call": ("tk::cutcp_role{extra}({p}binDim_x, {p}binDim_y, {p}binZeroAddr, {p}h, {p}cutoff2, {p}inv_cutoff2, "
                  "{p}regionZeroAddr, {p}grid_dimension_x, {p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, "
                  "{p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
     },

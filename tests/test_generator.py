@@ -93,7 +93,7 @@ def test_emitted_dispatcher_signature(be, n_params):
     assert names[-3:] == ["tzgemm1_ptb_start_block_pos", "tzgemm1_ptb_iter_block_step", "tzgemm1_ptb_end_block_pos"]
     assert meta["blocksize"] == 256 and meta["group"] == 2
     wave, wmeta = gen_mix.generate_wave_split(be, 256)
-    assert "RoleSpinSync" in wave and wave.count("__syncthreads()") == 1 and wmeta["blocksize"] == 512
+    assert "RoleHandoverSync" in wave and "role_wave_done" in wave and wave.count("__syncthreads()") == 1 and wmeta["blocksize"] == 512
     assert f"(int)threadIdx.x - 256" in wave
 
 

@@ -118,12 +118,12 @@ def test_partial_results_need_the_workspace_bound_to_c():
 
 def test_creator_object_at_the_reference_size_matches_the_oracle_on_sampled_blocks():
     # createKernel("sgemm"): 4096 x 4128 x 4064, A and B uniform [0,1) from the library's seeded generator, C = 0
-    # (src/ori_kernel/sgemm_kernel.cu:86-112); 132096 positions
+    # (src/ori_kernel/sgemm_kernel.cu:86-112); 528384 positions
     k = ta.create_kernel("sgemm")
     info = k.info()
     M, N, K = k.param(3, "int"), k.param(4, "int"), k.param(5, "int")
     assert (M, N, K) == (4096, 4128, 4064)
-    assert (info["ptb_start"], info["ptb_end"]) == (0, 32 * 258 * 16) and (info["ori_grid_x"], info["ori_grid_y"]) == (32, 258)
+    assert (info["ptb_start"], info["ptb_end"]) == (0, 32 * 258 * 64) and (info["ori_grid_x"], info["ori_grid_y"]) == (32, 258)
     assert ta.lib().tkMemset(k.param(2), 0, M * N * 4) == 0          # the object is memoised: start from C = 0
     k.execute()
     torch.cuda.synchronize()

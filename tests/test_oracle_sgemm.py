@@ -90,7 +90,7 @@ def test_launch_shapes_the_reference_holds():
     # kinfo's ori_blks 774 = 3 x 258, the M/10 run of fusion/code/kinfo.json
     assert oracle.sgemm_positions(4096, 4128, 4064, chunk=1 << 30) == 32 * 258
     assert oracle.sgemm_positions(384, 4128, 4064, chunk=1 << 30) == 774
-    assert oracle.sgemm_positions(4096, 4128, 4064) == 32 * 258 * 16
+    assert oracle.sgemm_positions(4096, 4128, 4064) == 32 * 258 * 64          # parts of 64 k steps
 
 
 @pytest.mark.parametrize("K", [256, 300, 700, 64])
@@ -99,7 +99,7 @@ def test_any_ascending_tiling_of_the_position_grid_is_one_kernel(K):
     A, B, C0 = inputs(M, N, K, seed=K)
     whole = oracle.sgemm(A, B, C0)
     total = oracle.sgemm_positions(M, N, K)
-    assert total == 2 * 3 * -(-K // 256)
+    assert total == 2 * 3 * -(-K // 64)
     assert np.array_equal(oracle.sgemm(A, B, C0, parts="chunks"), whole)
     rng = np.random.default_rng(K)
     for _ in range(4):
@@ -111,7 +111,7 @@ def test_any_ascending_tiling_of_the_position_grid_is_one_kernel(K):
     # a range that runs past the grid wraps to block 0, part 0: with several parts only the workspace changes,
     # with one part the block is updated a second time
     twice = oracle.sgemm(A, B, C0, start=0, end=total + 1, parts="chunks")
-    if K > 256:
+    if K > oracle.SGEMM_K_CHUNK:
         assert np.array_equal(twice, whole)
     else:
         assert np.array_equal(twice, oracle.sgemm(A, B, whole, start=0, end=1))
