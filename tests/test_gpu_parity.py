@@ -971,3 +971,35 @@ def test_random_fused_launches_equal_the_two_kernels_alone(seed):
     for g, w in zip(got, want):
         assert np.array_equal(g.view(np.uint32), w.view(np.uint32)), (name, (M, N, K), (t0, t1), (b0, b1), variant)
     assert ta.spin_fail_flag() == 0
+
+
+@pytest.mark.parametrize("variant", ["wave_256", "wave_512"])
+def test_gemm_role_barrier_hands_over_to_the_hardware_barrier_at_any_point(variant):
+    # In a wave-split kernel the GEMM role synchronises on an LDS arrival counter while best-effort waves run
+    # and on the hardware barrier once they have ended.  The change-over falls wherever the best-effort
+    # work happens to end: before the first tile (no blocks), in the middle of a tile, between tiles of a
+    # workgroup that has several (few workgroups launched), inside a shared reduction, or never (best-effort
+    # work that outlasts the GEMM).  Whatever the point, the GEMM's bits are those of the kernel alone.
+    for (M, N, K), grid in [((512, 512, 2048), 4), ((512, 512, 2048), 0), ((256, 384, 1024), 0), ((128, 128, 4608), 0)]:
+        A, B = gemm_inputs(M, N, K, seed=M + K)
+        dA, dB = dev(A), dev(B)
+        tiles = (M // 64) * (N // 64)
+        solo = torch.zeros((M, N), device="cuda:0")
+        ta.gptb_tzgemm(dA, dB, solo)
+        want_c = host(solo).view(np.uint32)
+        numK, numX = 512, 8192
+        k, phiR, phiI, xyz = mriq_inputs(numK, numX, seed=44)
+        ta.mriq_set_kvalues(np.concatenate([k, oracle.mriq_phimag(phiR, phiI)[:, None]], 1).astype(np.float32))
+        dx, dy, dz = (dev(v) for v in xyz)
+        nblk = ta.mriq_blocks(numK, numX)
+        ref_q = [torch.zeros(numX, device="cuda:0") for _ in range(2)]
+        ta.gptb_mriq(numK, dx, dy, dz, ref_q[0], ref_q[1])
+        for blocks in (0, 1, 3, nblk // 8, nblk // 2, nblk):
+            c = torch.full((M, N), -9.0, device="cuda:0")
+            q = [torch.zeros(numX, device="cuda:0") for _ in range(2)]
+            ta.mix_tzgemm_mriq(numK, dx, dy, dz, q[0], q[1], dA, dB, c, be_end=blocks, variant=variant, launch_grid=grid)
+            assert np.array_equal(host(c).view(np.uint32), want_c), ((M, N, K), grid, blocks)
+            if blocks == nblk:
+                assert np.array_equal(host(q[0]).view(np.uint32), host(ref_q[0]).view(np.uint32))
+                assert np.array_equal(host(q[1]).view(np.uint32), host(ref_q[1]).view(np.uint32))
+    assert ta.spin_fail_flag() == 0
