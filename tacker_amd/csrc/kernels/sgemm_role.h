@@ -9,17 +9,20 @@
 // alpha = beta = 2 (both products exact, so every way of contracting that line gives one result).
 //
 // gfx950: the reference stages an 8 x 16 tile of B in shared memory behind two barriers per 8 k
-// steps, shared by the block's 4 warps.  Here every wave stages its own copy -- 4 k rows x 16
-// columns = one float per lane, fetched with one vector load an iteration ahead, written to a
-// 256-byte slot of LDS and read back as 16 broadcast reads of 16 bytes -- so a wave is its own
+// steps, shared by the block's 4 warps.  Here one wavefront serves a block -- a lane owns the rows
+// of the reference's threads l and l + 64 -- and stages B for itself: 4 k rows x 16 columns = one
+// float per lane, fetched with one vector load two iterations ahead, written to a 256-byte slot of
+// LDS and read back row by row as broadcast reads of 16 bytes -- so a wave is its own
 // synchronisation domain: no barrier, and the role drops into the wave-split fused kernels like
-// the other vector roles (it adds 4 KiB of LDS to a kernel).  Per 4 k steps a wave issues two
-// vector loads, one LDS write, 16 LDS reads and 64 v_fmac_f32; the work is bound by the vector
-// ALUs (64 cycles per k step and wave).  Fetching the rows of B with scalar loads instead (they
-// are wave-uniform) was measured first and ran 4.8 times slower: every k row is another 64-byte
+// the other vector roles (it adds 4 KiB of LDS to a kernel).  Per 4 k steps a wave issues three
+// vector loads, one LDS write, 16 LDS reads and 128 v_fmac_f32: every value read back from LDS
+// serves two rows, which is what brings the LDS return path (16 bytes a lane and read) below the
+// time of the multiply-adds; with one row per lane the role was bound by it (2.5 ms against 2.0
+// for 4096 x 4128 x 4064).  Fetching the rows of B with scalar loads instead (they are
+// wave-uniform) was measured first and ran 4.8 times slower: every k row is another 64-byte
 // line, and the scalar cache serves its misses one after the other.
 //
-// Block positions.  A block's whole k loop is long (K = 4064: 4064 x 64 cycles, 110 us), so the
+// Block positions.  A block's whole k loop is long (K = 4064: 4064 x 128 cycles, 220 us), so the
 // GPTB position grid has a third dimension through the reference's own index reconstruction
 // (block_id_z = pos / (x y) % z): position p adds k part (p / (x y)) % z -- SGEMM_K_CHUNK k
 // steps -- to block p % (x y).  Between parts the 16 partial results of a thread rest in a
