@@ -309,7 +309,8 @@ def lc_leg(ta, torch, np, queries, be_name="stencil", be_label="stencil 512x512x
     torch.cuda.synchronize()
     co = np.array(tm.latencies())
     solo = np.array(tm.latencies(solo=True))
-    e2e = {k: np.array(tm.latencies(kind=k)) for k in ("e2e_solo", "e2e_colocated", "e2e_solo_wall", "e2e_colocated_wall")}
+    e2e = {k: np.array(tm.latencies(kind=k)) for k in ("e2e_solo", "e2e_colocated", "e2e_solo_wall", "e2e_colocated_wall",
+                                                             "e2e_graph", "e2e_graph_wall")}
     be_total = ta.create_kernel(be_name).info()["ptb_end"]
     out = {"workload": f"configs[4]: VGG16 batch 1 224x224 (convs and FCs on tzgemm) + {be_label} "
                        "blocks co-located by TaskManager (Aker mode, calibrated block counts)",
@@ -327,7 +328,8 @@ def lc_leg(ta, torch, np, queries, be_name="stencil", be_label="stencil 512x512x
            "lc_kernels_barred_from_fusion_at_end": tm.fusion_disabled()}
     out["p99_within_bound"] = bool(out["colocated_p99_ms"] <= out["qos_bound_ms"])
     # whole queries, one event pair (and the host clock) around all launches of a query, no
-    # synchronisation between kernels; the figures above are sums of per-kernel intervals
+    # synchronisation between kernels; the figures above are sums of per-kernel intervals.  graph_*: the
+    # solo query's launches recorded once and launched as one graph per query
     out["end_to_end"] = {"queries": int(len(e2e["e2e_solo"]))}
     for k, v in e2e.items():
         if len(v):

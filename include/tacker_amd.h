@@ -85,6 +85,17 @@ TK_API int tkEventRecord(tkEvent_t e, tkStream_t s);
 TK_API int tkEventSynchronize(tkEvent_t e);
 TK_API int tkEventElapsedTime(float *ms, tkEvent_t start, tkEvent_t stop);
 
+/* A stream's work recorded once and launched as one graph afterwards (no counterpart in the
+ * reference, whose query loop issues its launches one by one): everything enqueued on s between
+ * tkStreamBeginCapture and tkStreamEndCapture -- kernel launches of either kind; no synchronisation
+ * and no memory-set calls may fall in between, and s must not be the null stream -- becomes an
+ * executable graph that tkGraphLaunch enqueues as a whole. */
+typedef void *tkGraphExec_t;
+TK_API int tkStreamBeginCapture(tkStream_t s);
+TK_API int tkStreamEndCapture(tkStream_t s, tkGraphExec_t *exec);
+TK_API int tkGraphLaunch(tkGraphExec_t exec, tkStream_t s);
+TK_API int tkGraphExecDestroy(tkGraphExec_t exec);
+
 /* cudaLaunchKernel (src/GPTBKernel.h:109, src/MixKernel.h:100): func is a value
  * of the function registry, args is an array of pointers to each argument. */
 TK_API int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, size_t shmem,
@@ -512,6 +523,15 @@ TK_API int tacker_task_destroy(tacker_task_t task);
 /* Task::initExecution + every kernel's execute(stream) (the warm-up loop of
  * src/main.cu:290-297) */
 TK_API int tacker_task_execute(tacker_task_t task, tkStream_t stream);
+/* Task::initExecution alone (src/Task.h:24 of the reference; VGG16's copies the query's input to
+ * the device, synchronously) */
+TK_API int tacker_task_stage_input(tacker_task_t task);
+/* The task's launches recorded from `stream` into one graph (no counterpart in the reference, which
+ * launches a query kernel by kernel): every kernel's execute(stream) between tkStreamBeginCapture
+ * and tkStreamEndCapture, none of them run.  Call tacker_task_execute once before, so that no
+ * kernel still has a buffer to allocate; per query then tacker_task_stage_input + tkGraphLaunch.
+ * The graph holds the task's buffers by address: destroy it (tkGraphExecDestroy) before the task. */
+TK_API int tacker_task_capture(tacker_task_t task, tkStream_t stream, tkGraphExec_t *exec);
 TK_API int tacker_task_kernel_count(tacker_task_t task);
 /* name (up to name_cap bytes), mixable flag, getArgs() (up to 14 ints, count in *nargs) */
 TK_API int tacker_task_kernel_info(tacker_task_t task, int index, char *name, int name_cap,
@@ -573,7 +593,9 @@ TK_API float tacker_task_manager_be_mix_ms(tacker_task_manager_t tm);
 TK_API int tacker_task_manager_set_end_to_end(tacker_task_manager_t tm, int queries);
 /* which = 0: per-query latency of the co-located queries (sum of per-kernel intervals), 1: of the
  * solo profiling queries; end-to-end queries (tacker_task_manager_set_end_to_end): 2 co-located and
- * 3 solo by events, 4 co-located and 5 solo by the host clock */
+ * 3 solo by events, 4 co-located and 5 solo by the host clock; 6 and 7: the solo query recorded once
+ * from a stream and launched as one graph per query (tkStreamBeginCapture .. tkGraphLaunch), by
+ * events and by the host clock -- no counterpart in the reference, which launches kernel by kernel */
 TK_API int tacker_task_manager_latencies(tacker_task_manager_t tm, int which, float *out, int cap);
 
 /* the scheduler's arithmetic on its own (src/TaskManager.cu:586-640) */

@@ -136,6 +136,15 @@ def _declare(lib):
     lib.tkMemset.argtypes = [vp, i, C.c_size_t]
     lib.tacker_task_logits.argtypes = [vp, C.POINTER(vp), C.POINTER(C.c_long), C.POINTER(i)]
     lib.tacker_task_input.argtypes = [vp, C.POINTER(vp), C.POINTER(i)]
+    lib.tacker_task_stage_input.argtypes = [vp]
+    lib.tacker_task_capture.argtypes = [vp, vp, C.POINTER(vp)]
+    lib.tkStreamCreate.argtypes = [C.POINTER(vp)]
+    lib.tkStreamDestroy.argtypes = [vp]
+    lib.tkStreamSynchronize.argtypes = [vp]
+    lib.tkStreamBeginCapture.argtypes = [vp]
+    lib.tkStreamEndCapture.argtypes = [vp, C.POINTER(vp)]
+    lib.tkGraphLaunch.argtypes = [vp, vp]
+    lib.tkGraphExecDestroy.argtypes = [vp]
     lib.tacker_task_manager_create.restype = vp
     lib.tacker_task_manager_create.argtypes = [vp, cp, cp]
     lib.tacker_task_manager_destroy.argtypes = [vp]
@@ -814,6 +823,23 @@ REPORT_KEYS = ("lc_solo_ms", "be1_solo_ms", "be2_solo_ms", "be_blocks_executed",
                "be_task_finish_num", "n_colocated", "n_solo")
 
 
+class QueryGraph:
+    """A recorded query (tkGraphExec_t): ``launch(raw_stream)`` enqueues all its kernels at once."""
+
+    def __init__(self, library, handle):
+        self.l, self.h = library, handle
+
+    def launch(self, raw_stream):
+        rc = self.l.tkGraphLaunch(self.h, raw_stream)
+        if rc:
+            raise TackerError(f"tkGraphLaunch failed ({rc})")
+
+    def close(self):
+        if self.h:
+            self.l.tkGraphExecDestroy(self.h)
+            self.h = None
+
+
 class LcTask:
     """createTask(model): the latency-critical job (VGG16 at batch 1)."""
 
@@ -828,6 +854,21 @@ class LcTask:
         rc = self.l.tacker_task_execute(self.h, st)
         if rc:
             raise TackerError(f"task execute failed ({rc}): {self.l.tacker_last_error().decode()}")
+
+    def stage_input(self):
+        """Task::initExecution alone: the query's input copied to the device (synchronous)."""
+        rc = self.l.tacker_task_stage_input(self.h)
+        if rc:
+            raise TackerError(f"task stage_input failed ({rc}): {self.l.tacker_last_error().decode()}")
+
+    def capture(self, raw_stream):
+        """The task's launches recorded from ``raw_stream`` (a tkStream_t, not the null stream) into
+        a ``QueryGraph``; run ``execute`` once before so that every buffer exists."""
+        exec_ = C.c_void_p()
+        rc = self.l.tacker_task_capture(self.h, raw_stream, C.byref(exec_))
+        if rc:
+            raise TackerError(f"task capture failed ({rc}): {self.l.tacker_last_error().decode()}")
+        return QueryGraph(self.l, exec_)
 
     def kernels(self):
         out = []
@@ -927,7 +968,7 @@ class TaskManager:
         check(self.l.tacker_task_manager_set_end_to_end(self.h, queries), "set_end_to_end")
 
     LATENCY_KINDS = {"colocated": 0, "solo": 1, "e2e_colocated": 2, "e2e_solo": 3,
-                     "e2e_colocated_wall": 4, "e2e_solo_wall": 5}
+                     "e2e_colocated_wall": 4, "e2e_solo_wall": 5, "e2e_graph": 6, "e2e_graph_wall": 7}
 
     def latencies(self, solo=False, kind=None):
         """Per-query latencies in ms.  ``kind`` picks one of LATENCY_KINDS: the sums of per-kernel

@@ -53,6 +53,21 @@ void Task::executeTask(ExecutionMode mode, cudaStream_t stream)
     if (mode == ExecutionMode::Aker) recorder.recordTask(taskId, taskName);
 }
 
+tkGraphExec_t Task::captureQuery(cudaStream_t stream)
+{
+    tkGraphExec_t graph = nullptr;
+    TK_SAFE_CALL(tkStreamBeginCapture(stream));
+    try {
+        for (auto &kernel : kernels) kernel->execute(stream);
+    } catch (...) {   // a stream left recording would fail every later call on it
+        tkStreamEndCapture(stream, &graph);
+        if (graph) tkGraphExecDestroy(graph);
+        throw;
+    }
+    TK_SAFE_CALL(tkStreamEndCapture(stream, &graph));
+    return graph;
+}
+
 void Task::executeTask(ExecutionMode mode, int idx, cudaStream_t stream)
 {
     EventPair ev;

@@ -20,6 +20,11 @@ public:
     void executeTask(ExecutionMode mode, int idx, cudaStream_t stream);
     // stage the job's input (host -> device copy for a DNN query)
     virtual void initExecution() = 0;
+    // the job's launches recorded from `stream` (not the null stream) into one executable graph:
+    // every kernel's execute() once, none of them run.  The job must have run before, so that no
+    // kernel still has buffers to allocate, and the caller stages the input before each launch of
+    // the graph.  The caller destroys the graph (tkGraphExecDestroy).
+    tkGraphExec_t captureQuery(cudaStream_t stream);
 
     int taskId;
     std::string taskName;

@@ -69,6 +69,7 @@ struct TaskManagerReport {
     // pair of events, no synchronisation between kernels; and the same span on the host clock
     std::vector<float> e2e_colocated_ms, e2e_solo_ms;
     std::vector<float> e2e_colocated_wall_ms, e2e_solo_wall_ms;
+    std::vector<float> e2e_graph_ms, e2e_graph_wall_ms;   // the solo query launched as one captured graph
 };
 
 class TaskManager {

@@ -1164,6 +1164,27 @@ int tacker_task_execute(tacker_task_t h, tkStream_t stream)
     });
 }
 
+int tacker_task_stage_input(tacker_task_t h)
+{
+    Task *t = static_cast<Task *>(h);
+    if (!t) return fail(TK_ERROR_INVALID_VALUE, "null task");
+    return guarded([&]() -> int {
+        t->initExecution();
+        return TK_SUCCESS;
+    });
+}
+
+int tacker_task_capture(tacker_task_t h, tkStream_t stream, tkGraphExec_t *exec)
+{
+    Task *t = static_cast<Task *>(h);
+    if (!t || !exec) return fail(TK_ERROR_INVALID_VALUE, "null task or result");
+    if (!stream) return fail(TK_ERROR_INVALID_VALUE, "the null stream cannot record a graph");
+    return guarded([&]() -> int {
+        *exec = t->captureQuery(stream);
+        return TK_SUCCESS;
+    });
+}
+
 int tacker_task_kernel_count(tacker_task_t h)
 {
     Task *t = static_cast<Task *>(h);
@@ -1342,8 +1363,9 @@ int tacker_task_manager_latencies(tacker_task_manager_t h, int which, float *out
     if (!tm || !out) return -1;
     const std::vector<float> *all[] = {&tm->report.query_latency_ms,      &tm->report.solo_latency_ms,
                                        &tm->report.e2e_colocated_ms,      &tm->report.e2e_solo_ms,
-                                       &tm->report.e2e_colocated_wall_ms, &tm->report.e2e_solo_wall_ms};
-    if (which < 0 || which > 5) return -1;
+                                       &tm->report.e2e_colocated_wall_ms, &tm->report.e2e_solo_wall_ms,
+                                       &tm->report.e2e_graph_ms,          &tm->report.e2e_graph_wall_ms};
+    if (which < 0 || which > 7) return -1;
     const std::vector<float> &v = *all[which];
     const int n = std::min((int)v.size(), cap);
     memcpy(out, v.data(), (size_t)n * sizeof(float));

@@ -29,6 +29,13 @@ std::vector<FakeKernel *> &kernels()
     return k;
 }
 std::vector<Launch> g_launches;
+// stream capture: launches on the capturing stream are recorded, not "run"; a graph replays its record
+void *g_capturing = nullptr;
+std::vector<Launch> g_captured;
+struct FakeGraph {
+    std::vector<Launch> launches;
+};
+int g_graph_launches = 0;
 int g_fail_next_launch = 0;
 int g_cu_count = 256;
 float g_event_ms = 1.0f;
@@ -142,7 +149,39 @@ int tkLaunchKernel(const void *func, tkDim3 grid, tkDim3 block, void **args, siz
         const unsigned char *p = (const unsigned char *)args[i];
         l.args.emplace_back(p, p + k->arg_sizes[i]);
     }
-    g_launches.push_back(std::move(l));
+    if (g_capturing && stream == g_capturing) g_captured.push_back(std::move(l));
+    else g_launches.push_back(std::move(l));
+    return TK_SUCCESS;
+}
+
+int tkStreamBeginCapture(tkStream_t s)
+{
+    if (!s || g_capturing) return TK_ERROR_INVALID_VALUE;
+    g_capturing = s;
+    g_captured.clear();
+    return TK_SUCCESS;
+}
+int tkStreamEndCapture(tkStream_t s, tkGraphExec_t *exec)
+{
+    if (!s || s != g_capturing || !exec) return TK_ERROR_INVALID_VALUE;
+    g_capturing = nullptr;
+    *exec = new FakeGraph{std::move(g_captured)};
+    g_captured.clear();
+    return TK_SUCCESS;
+}
+int tkGraphLaunch(tkGraphExec_t exec, tkStream_t s)
+{
+    if (!exec) return TK_ERROR_INVALID_VALUE;
+    for (Launch l : static_cast<FakeGraph *>(exec)->launches) {
+        l.stream = s;
+        g_launches.push_back(std::move(l));
+    }
+    ++g_graph_launches;
+    return TK_SUCCESS;
+}
+int tkGraphExecDestroy(tkGraphExec_t exec)
+{
+    delete static_cast<FakeGraph *>(exec);
     return TK_SUCCESS;
 }
 
@@ -235,7 +274,8 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
 
 // ---- inspection interface for tests --------------------------------------
 TK_API int tk_fake_launch_count(void) { return (int)g_launches.size(); }
-TK_API void tk_fake_reset(void) { g_launches.clear(); g_fail_next_launch = 0; g_event_queue.clear(); }
+TK_API int tk_fake_graph_launch_count(void) { return g_graph_launches; }
+TK_API void tk_fake_reset(void) { g_launches.clear(); g_graph_launches = 0; g_fail_next_launch = 0; g_event_queue.clear(); }
 TK_API void tk_fake_fail_next_launches(int n) { g_fail_next_launch = n; }
 TK_API void tk_fake_set_cu_count(int n) { g_cu_count = n; }
 TK_API void tk_fake_set_event_ms(float ms) { g_event_ms = ms; }

@@ -166,6 +166,30 @@ int tkStreamSynchronize(tkStream_t s) { return FOLD(hipStreamSynchronize((hipStr
 int tkDeviceSynchronize(void) { return FOLD(hipDeviceSynchronize()); }
 int tkEventCreate(tkEvent_t *e) { return FOLD(hipEventCreate((hipEvent_t *)e)); }
 int tkEventDestroy(tkEvent_t e) { return FOLD(hipEventDestroy((hipEvent_t)e)); }
+int tkStreamBeginCapture(tkStream_t s)
+{
+    if (!s) return TK_ERROR_INVALID_VALUE;   // the null stream cannot be captured
+    return FOLD(hipStreamBeginCapture((hipStream_t)s, hipStreamCaptureModeThreadLocal));
+}
+int tkStreamEndCapture(tkStream_t s, tkGraphExec_t *exec)
+{
+    if (!s || !exec) return TK_ERROR_INVALID_VALUE;
+    hipGraph_t graph = nullptr;
+    int rc = FOLD(hipStreamEndCapture((hipStream_t)s, &graph));
+    if (rc) return rc;
+    hipGraphExec_t made = nullptr;
+    rc = FOLD(hipGraphInstantiate(&made, graph, nullptr, nullptr, 0));
+    (void)hipGraphDestroy(graph);
+    if (rc) return rc;
+    *exec = made;
+    return TK_SUCCESS;
+}
+int tkGraphLaunch(tkGraphExec_t exec, tkStream_t s)
+{
+    if (!exec) return TK_ERROR_INVALID_VALUE;
+    return FOLD(hipGraphLaunch((hipGraphExec_t)exec, (hipStream_t)s));
+}
+int tkGraphExecDestroy(tkGraphExec_t exec) { return exec ? FOLD(hipGraphExecDestroy((hipGraphExec_t)exec)) : TK_SUCCESS; }
 int tkEventRecord(tkEvent_t e, tkStream_t s) { return FOLD(hipEventRecord((hipEvent_t)e, (hipStream_t)s)); }
 int tkEventSynchronize(tkEvent_t e) { return FOLD(hipEventSynchronize((hipEvent_t)e)); }
 int tkEventElapsedTime(float *ms, tkEvent_t start, tkEvent_t stop)

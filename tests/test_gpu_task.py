@@ -1,5 +1,7 @@
 """GPU tests of the conv->GEMM helpers, the VGG16 latency-critical task and the
 TaskManager on the real device."""
+import ctypes as C
+
 import numpy as np
 import pytest
 import torch
@@ -254,6 +256,9 @@ def test_task_manager_colocation_keeps_lc_results_and_reports():
     for kind in ("e2e_solo", "e2e_colocated", "e2e_solo_wall", "e2e_colocated_wall"):
         got = tm.latencies(kind=kind)
         assert len(got) == 5 and all(0 < v < 50.0 for v in got), kind
+    for kind in ("e2e_graph", "e2e_graph_wall"):
+        got = tm.latencies(kind=kind)
+        assert len(got) == 5 and all(0 < v < 50.0 for v in got), kind
     assert min(tm.latencies(kind="e2e_solo")) < min(tm.latencies(solo=True))
     assert all(w >= e - 1e-3 for w, e in zip(tm.latencies(kind="e2e_solo_wall"), tm.latencies(kind="e2e_solo")))
     tm.set_end_to_end(0)
@@ -349,3 +354,39 @@ def test_create_kernel_objects_run_and_match_oracle_for_cp():
         ta.create_kernel(name).execute()
     torch.cuda.synchronize()
     assert ta.spin_fail_flag() == 0
+
+
+def test_a_recorded_query_gives_the_eager_logits_on_every_replay():
+    """The query's launches recorded once and launched as one graph: replayed several times, with the
+    input staged again, eager queries, other kernels and synchronisations between the replays, and
+    every replay's logits compared bit for bit with the eager query's."""
+    task = ta.LcTask("vgg16", 64, 64)
+    task.execute()
+    torch.cuda.synchronize()
+    p, stride, n = task.logits()
+    want = ta.device_to_host(p, (n, stride), np.float32)[:, 0].copy()
+    assert np.isfinite(want).all() and np.abs(want).max() > 0
+    l = ta.lib()
+    stream = C.c_void_p()
+    assert l.tkStreamCreate(C.byref(stream)) == 0
+    with pytest.raises(ta.TackerError, match="null stream"):
+        task.capture(None)
+    graph = task.capture(stream)
+    x = torch.randn(1 << 20, device="cuda")
+    for replay in range(6):
+        # wipe the logits so that a replay that ran nothing cannot pass on the last one's result
+        assert l.tkMemset(p, 0xFF, n * stride * 4) == 0
+        torch.cuda.synchronize()
+        task.stage_input()
+        graph.launch(stream)
+        assert l.tkStreamSynchronize(stream) == 0
+        got = ta.device_to_host(p, (n, stride), np.float32)[:, 0]
+        assert np.array_equal(got, want), replay
+        # the program's own eager work between replays: another query kernel by kernel, a library reduction
+        if replay % 2 == 0:
+            task.execute()
+        assert torch.isfinite(x.sum()).item()
+        torch.cuda.synchronize()
+    graph.close()
+    assert l.tkStreamDestroy(stream) == 0
+    task.close()

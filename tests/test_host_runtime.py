@@ -720,10 +720,45 @@ def test_task_manager_times_whole_queries_with_one_interval_each(fake, small_vgg
     sizes = [b - a for a, b in ranges]
     for q in range(1, 6):
         assert all(s <= c for s, c in zip(sizes[q * per_query:(q + 1) * per_query], sizes[:per_query]))
+    # the solo query as one graph: recorded once (its launches run nothing while recorded), then one
+    # graph launch a query, two of them untimed
+    assert fake.tk_fake_graph_launch_count() == 5
+    assert tm.latencies(kind="e2e_graph") == pytest.approx([0.01] * 3, rel=1e-4)
+    assert len(tm.latencies(kind="e2e_graph_wall")) == 3
+    graph_span = all_launches[fused[-1] + 1:]
+    per_graph = len(graph_span) // 5              # a layer may take more than one launch (operand lowering)
+    assert per_graph >= n and len(graph_span) == 5 * per_graph
+    keys = [l["key"] for l in graph_span]
+    assert all(keys[q * per_graph:(q + 1) * per_graph] == keys[:per_graph] for q in range(5))
+    assert not any(k.startswith("tzgemm_stencil") for k in keys)
     tm.set_end_to_end(0)
     tm.run("aker", raw_stream=None, second_stage=False)
     assert tm.latencies(kind="e2e_solo") == [] and tm.latencies(kind="e2e_colocated_wall") == []
+    assert tm.latencies(kind="e2e_graph") == []
     tm.close()
+
+
+def test_a_recorded_query_replays_the_launches_of_an_eager_one(fake, small_vgg):
+    small_vgg.execute(raw_stream=None)
+    fake.tk_fake_reset()
+    small_vgg.execute(raw_stream=None)
+    eager = [(l["key"], l["grid"], l["block"], l["args"]) for l in launches(fake)]
+    assert len(eager) >= len(small_vgg.kernels())
+    stream = C.c_void_p()
+    assert fake.tkStreamCreate(C.byref(stream)) == 0
+    fake.tk_fake_reset()
+    with pytest.raises(ta.TackerError, match="null stream"):
+        small_vgg.capture(None)
+    graph = small_vgg.capture(stream)
+    assert launches(fake) == []                      # recording runs nothing
+    for replay in range(3):
+        small_vgg.stage_input()
+        graph.launch(stream)
+        got = [(l["key"], l["grid"], l["block"], l["args"]) for l in launches(fake)]
+        assert got[replay * len(eager):] == eager
+    assert fake.tk_fake_graph_launch_count() == 3
+    graph.close()
+    assert fake.tkStreamDestroy(stream) == 0
 
 
 def test_task_manager_falls_back_to_solo_when_headroom_is_short(fake, small_vgg):
