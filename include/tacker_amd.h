@@ -274,6 +274,46 @@ TK_API int tacker_ori_fft(float *data, int batches, tkStream_t stream);
 TK_API int tacker_gptb_fft(float *data, int batches, int block_start, int block_end, int launch_grid,
                            int launch_block, tkStream_t stream);
 
+/* ori_nn / general_ptb_nn (src/ori_kernel/nn_kernel.cu:9-17, src/gptb_kernel/nn_kernel.cu:3-23;
+ * Rodinia nn): distances[i] = sqrtf((lat - lat_i)^2 + (lng - lng_i)^2) for numRecords records,
+ * locations = numRecords {lat, lng} pairs of floats (the reference's LatLong).  One block position
+ * per 256 records, tacker_nn_blocks(numRecords) of them.  fp32 in the order of the reference's
+ * source with an IEEE square root: bit-identical to a CPU evaluation. */
+TK_API int tacker_nn_blocks(int numRecords);
+TK_API int tacker_ori_nn(const float *locations, float *distances, int numRecords, float lat, float lng,
+                         tkStream_t stream);
+TK_API int tacker_gptb_nn(const float *locations, float *distances, int numRecords, float lat, float lng,
+                          int block_start, int block_end, int launch_grid, int launch_block,
+                          tkStream_t stream);
+
+/* ori_hot3d / general_ptb_hot3d (src/ori_kernel/hot3d_kernel.cu:9-60,
+ * src/gptb_kernel/hot3d_kernel.cu:3-62; Rodinia hotspot3D): one time step of nx x ny x nz cells,
+ * p = dissipated power, tIn / tOut = temperature before / after (distinct arrays), x fastest.  nx a
+ * multiple of 64, ny of 4, nz >= 2; (nx / 64) * (ny / 4) block positions of 64 x 4 columns.  The
+ * step's coefficients follow from the cell counts (src/ori_kernel/hot3d_kernel.cu:84-116);
+ * tacker_hot3d_coefficients writes {sdc, ce, cw, cn, cs, ct, cb, cc}.  fp32 in the order of the
+ * reference's source: bit-identical to a CPU evaluation. */
+TK_API int tacker_hot3d_coefficients(int nx, int ny, int nz, float out[8]);
+TK_API int tacker_ori_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz,
+                            tkStream_t stream);
+TK_API int tacker_gptb_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz,
+                             int block_start, int block_end, int launch_grid, int launch_block,
+                             tkStream_t stream);
+
+/* ori_path / general_ptb_path (src/ori_kernel/path_kernel.cu:9-86,
+ * src/gptb_kernel/path_kernel.cu:3-93; Rodinia pathfinder): `iteration` rows (1 .. 127) of
+ * results[x] = wall[row][x] + min(src[x-1], src[x], src[x+1]) starting at row startStep of the
+ * wall (the grid without its first row: (rows - 1) x cols ints), src and results rows of cols ints.
+ * tacker_path_blocks(cols, iteration) block positions of 256 - 2 * iteration result columns each,
+ * served by one wavefront each (launch_block a multiple of 64).  Integer work: the reference's
+ * bits. */
+TK_API int tacker_path_blocks(int cols, int iteration);
+TK_API int tacker_ori_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows,
+                           int startStep, tkStream_t stream);
+TK_API int tacker_gptb_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows,
+                            int startStep, int block_start, int block_end, int launch_grid,
+                            int launch_block, tkStream_t stream);
+
 /* prepare_input (src/header/cutcp_header.h:111-300): hashes natoms atoms {x, y, z, q} into bins of
  * 4 x 4 x 4 Angstroms, 8 atoms to a bin, around a lattice of nx x ny x nz points of spacing h whose
  * lowest corner is lo, and lists the bin offsets a region of 8 x 8 x 8 points has to visit for the
@@ -383,6 +423,20 @@ TK_API int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_
                                  const void *B, float *C, int M, int N, int K, int tile_start,
                                  int tile_end, const char *variant, int launch_grid, int launch_block,
                                  tkStream_t stream);
+/* src/mix_kernel/tzgemm_nn.cu, tzgemm_hot3d.cu, tzgemm_path.cu */
+TK_API int tacker_mix_tzgemm_nn(const float *locations, float *distances, int numRecords, float lat,
+                                float lng, int be_start, int be_end, const void *A, const void *B,
+                                float *C, int M, int N, int K, int tile_start, int tile_end,
+                                const char *variant, int launch_grid, int launch_block, tkStream_t stream);
+TK_API int tacker_mix_tzgemm_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz,
+                                   int be_start, int be_end, const void *A, const void *B, float *C, int M,
+                                   int N, int K, int tile_start, int tile_end, const char *variant,
+                                   int launch_grid, int launch_block, tkStream_t stream);
+TK_API int tacker_mix_tzgemm_path(int iteration, const int *wall, const int *src, int *results, int cols,
+                                  int rows, int startStep, int be_start, int be_end, const void *A,
+                                  const void *B, float *C, int M, int N, int K, int tile_start,
+                                  int tile_end, const char *variant, int launch_grid, int launch_block,
+                                  tkStream_t stream);
 TK_API int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx,
                                 int voly, int be_start, int be_end, const void *A, const void *B,
                                 float *C, int M, int N, int K, int tile_start, int tile_end,
@@ -420,6 +474,12 @@ TK_API tacker_kernel_t tacker_ori_mriq_create(int numK, const float *x, const fl
 TK_API tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N,
                                                int K);
 TK_API tacker_kernel_t tacker_ori_fft_create(float *data, int batches);
+TK_API tacker_kernel_t tacker_ori_nn_create(const float *locations, float *distances, int numRecords,
+                                            float lat, float lng);
+TK_API tacker_kernel_t tacker_ori_hot3d_create(const float *p, const float *tIn, float *tOut, int nx, int ny,
+                                               int nz);
+TK_API tacker_kernel_t tacker_ori_path_create(int iteration, const int *wall, const int *src, int *results,
+                                              int cols, int rows, int startStep);
 TK_API tacker_kernel_t tacker_ori_cutcp_create(int binDim_x, int binDim_y, const float *binZeroAddr, float h,
                                                float cutoff2, float inv_cutoff2, float *regionZeroAddr,
                                                int regions_x, int regions_y, int regions_z);

@@ -53,6 +53,12 @@ def _declare(l):
                                     C.c_void_p, C.c_void_p, _i32p]
     l.orc_fft_gptb.argtypes = [_f32p, C.c_int, C.c_int, C.c_int]
     l.orc_fft_source.argtypes = [_f32p, C.c_int]
+    l.orc_nn_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_float, C.c_float] + [C.c_int] * 5
+    l.orc_hot3d_gptb.argtypes = ([_f32p, _f32p, _f32p, C.c_float, C.c_int, C.c_int, C.c_int] + [C.c_float] * 7 +
+                                 [C.c_int] * 6)
+    l.orc_hot3d_coefficients.argtypes = [C.c_int, C.c_int, C.c_int, _f32p]
+    l.orc_path_gptb.argtypes = [C.c_int, _i32p, _i32p, _i32p] + [C.c_int] * 5
+    l.orc_path_source.argtypes = [_i32p, C.c_longlong]
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
@@ -355,6 +361,83 @@ def fft_source(batches):
     """The reference's input: rand() after srand(54321), scaled to [-1, 1]."""
     out = np.zeros((batches, FFT_N, 2), np.float32)
     lib().orc_fft_source(out.reshape(-1), out.size)
+    return out
+
+
+# --------------------------------------------------------------------------- Rodinia partners
+NN_BLOCK = 256
+HOT3D_TILE = (64, 4)
+PATH_BLOCK = 256
+
+
+def nn_blocks(num_records):
+    return (num_records - 1) // NN_BLOCK + 1 if num_records > 0 else 0
+
+
+def nn(locations, lat, lng, out=None, start=0, end=None, grid=None, block=NN_BLOCK):
+    """Distances of [n][2] float32 {lat, lng} records to (lat, lng); block positions [start, end) of
+    `block` records over a grid (gx, gy) (default: all blocks in x).  Records no position covers
+    keep `out`'s value (zeros if not given)."""
+    loc = np.ascontiguousarray(locations, np.float32)
+    n = loc.shape[0]
+    res = np.zeros(n, np.float32) if out is None else np.array(out, np.float32)
+    gx, gy = grid if grid is not None else ((n - 1) // block + 1, 1)
+    if end is None:
+        end = gx * gy
+    lib().orc_nn_gptb(loc.reshape(-1), res, n, np.float32(lat), np.float32(lng), gx, gy, block, start, end)
+    return res
+
+
+def hot3d_coefficients(nx, ny, nz):
+    out = np.zeros(8, np.float32)
+    lib().orc_hot3d_coefficients(nx, ny, nz, out)
+    return dict(zip(("sdc", "ce", "cw", "cn", "cs", "ct", "cb", "cc"), out))
+
+
+def hot3d_blocks(nx, ny):
+    return (nx // HOT3D_TILE[0]) * (ny // HOT3D_TILE[1])
+
+
+def hot3d(p, t_in, coeff=None, out=None, start=0, end=None):
+    """One hotspot3D step on [nz][ny][nx] float32 arrays; block positions [start, end) of 64 x 4
+    columns.  Cells no position covers keep `out`'s value (zeros if not given)."""
+    p = np.ascontiguousarray(p, np.float32)
+    t = np.ascontiguousarray(t_in, np.float32)
+    nz, ny, nx = t.shape
+    k = coeff or hot3d_coefficients(nx, ny, nz)
+    res = np.zeros_like(t) if out is None else np.array(out, np.float32)
+    gx, gy = -(-nx // HOT3D_TILE[0]), -(-ny // HOT3D_TILE[1])
+    if end is None:
+        end = gx * gy
+    f = np.float32
+    lib().orc_hot3d_gptb(p.reshape(-1), t.reshape(-1), res.reshape(-1), f(k["sdc"]), nx, ny, nz, f(k["ce"]), f(k["cw"]),
+                         f(k["cn"]), f(k["cs"]), f(k["ct"]), f(k["cb"]), f(k["cc"]), gx, gy, HOT3D_TILE[0],
+                         HOT3D_TILE[1], start, end)
+    return res
+
+
+def path_blocks(cols, iteration):
+    small = PATH_BLOCK - 2 * iteration
+    return -(-cols // small) if small > 0 and cols > 0 else 0
+
+
+def path(iteration, wall, src, out=None, start_step=0, start=0, end=None):
+    """`iteration` rows of pathfinder from row start_step of wall ([rows - 1][cols] int32, the grid
+    without its first row), src = [cols] int32; block positions [start, end).  Columns no position
+    covers keep `out`'s value (zeros if not given)."""
+    w = np.ascontiguousarray(wall, np.int32)
+    s = np.ascontiguousarray(src, np.int32)
+    cols = s.shape[0]
+    res = np.zeros(cols, np.int32) if out is None else np.array(out, np.int32)
+    if end is None:
+        end = path_blocks(cols, iteration)
+    lib().orc_path_gptb(iteration, w.reshape(-1), s, res, cols, start_step, iteration, start, end)
+    return res
+
+
+def path_source(rows, cols):
+    out = np.zeros((rows, cols), np.int32)
+    lib().orc_path_source(out.reshape(-1), out.size)
     return out
 
 

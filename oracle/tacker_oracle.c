@@ -42,6 +42,18 @@
  *                         impulses = rows of the DFT matrix, pure tones, linearity,
  *                         Parseval, position wrap; the input stream against the cp atoms'
  *                         draw of the same seeded rand().
+ *   orc_nn_gptb           3-4-5 and axis-aligned known answers, numpy float64 hypot, the float32
+ *                         vectorised evaluation, block wrap and the record-count tail, any tiling
+ *                         of the block positions (tests/test_oracle_rodinia.py).
+ *   orc_hot3d_gptb        the ambient temperature as a fixed point, a constant field's closed
+ *                         form T (1 - ct) + ct 80, heat content conserved inside an insulated
+ *                         chip but for the top face's term, an edge-padded numpy formulation
+ *                         in float64 and in float32, the coefficients against Rodinia's formulas
+ *                         in float64, any tiling of the positions.
+ *   orc_path_gptb         the textbook row-by-row dynamic programme over the whole grid (numpy),
+ *                         brute force over all paths on a tiny wall, window edges at both ends of
+ *                         the grid, column counts that are not a multiple of the window's yield,
+ *                         any tiling of the positions; the input stream against rand() % 10.
  *   orc_im2col            direct convolution brute force.
  *   orc_gptb_index        partition invariance (any launch grid covers every
  *                         block once).
@@ -950,4 +962,137 @@ ORC_API int orc_cutcp_prepare(const float *atoms, int natoms, const float *lo, i
     }
     free(fill);
     return cnt;
+}
+
+
+/* ------------------------------------------------------------------ nn
+ * src/ori_kernel/nn_kernel.cu:9-17 (general_ptb_nn: src/gptb_kernel/nn_kernel.cu:3-23): thread t of
+ * block (bx, by) owns record globalId = blockDim.x * (gridDim.x * by + bx) + t and writes
+ * sqrt((lat - r.lat) * (lat - r.lat) + (lng - r.lng) * (lng - r.lng)) in float if globalId <
+ * numRecords.  Positions [start, end): bx = p % gx, by = (p / gx) % gy. */
+ORC_API void orc_nn_gptb(const float *locations, float *distances, int numRecords, float lat, float lng, int gx,
+                         int gy, int bdx, int start, int end)
+{
+    for (int pos = start; pos < end; ++pos) {
+        const int bx = (int)((unsigned)pos % (unsigned)gx);
+        const int by = (int)(((unsigned)pos / (unsigned)gx) % (unsigned)gy);
+        for (int t = 0; t < bdx; ++t) {
+            const long long id = (long long)bdx * ((long long)gx * by + bx) + t;
+            if (id >= numRecords) continue;
+            const float dlat = lat - locations[2 * id];
+            const float dlng = lng - locations[2 * id + 1];
+            distances[id] = sqrtf(dlat * dlat + dlng * dlng);
+        }
+    }
+}
+
+/* ------------------------------------------------------------------ hot3d
+ * src/ori_kernel/hot3d_kernel.cu:9-60 (general_ptb_hot3d: src/gptb_kernel/hot3d_kernel.cu:3-62):
+ * thread (tx, ty) of block (bx, by) owns column i = bdx bx + tx, j = bdy by + ty and walks it from
+ * layer 0 up; the neighbour of an edge cell is the cell itself, below the bottom layer and above
+ * the top layer likewise.  Per cell, float, summed left to right:
+ *   cc t + cw W + ce E + cs S + cn N + cb below + ct above + sdc p + ct 80. */
+ORC_API void orc_hot3d_gptb(const float *p, const float *tIn, float *tOut, float sdc, int nx, int ny, int nz,
+                            float ce, float cw, float cn, float cs, float ct, float cb, float cc, int gx, int gy,
+                            int bdx, int bdy, int start, int end)
+{
+    const float amb_temp = 80.0f;
+    const long long xy = (long long)nx * ny;
+    for (int pos = start; pos < end; ++pos) {
+        const int bx = (int)((unsigned)pos % (unsigned)gx);
+        const int by = (int)(((unsigned)pos / (unsigned)gx) % (unsigned)gy);
+        for (int ty = 0; ty < bdy; ++ty)
+            for (int tx = 0; tx < bdx; ++tx) {
+                const int i = bdx * bx + tx, j = bdy * by + ty;
+                if (i >= nx || j >= ny) continue;
+                for (int k = 0; k < nz; ++k) {
+                    const long long c = i + (long long)j * nx + k * xy;
+                    const long long W = i == 0 ? c : c - 1, E = i == nx - 1 ? c : c + 1;
+                    const long long N = j == 0 ? c : c - nx, S = j == ny - 1 ? c : c + nx;
+                    const float below = tIn[k == 0 ? c : c - xy], above = tIn[k == nz - 1 ? c : c + xy];
+                    float v = cc * tIn[c];
+                    v = v + cw * tIn[W];
+                    v = v + ce * tIn[E];
+                    v = v + cs * tIn[S];
+                    v = v + cn * tIn[N];
+                    v = v + cb * below;
+                    v = v + ct * above;
+                    v = v + sdc * p[c];
+                    v = v + ct * amb_temp;
+                    tOut[c] = v;
+                }
+            }
+    }
+}
+
+/* the step's coefficients, src/ori_kernel/hot3d_kernel.cu:84-116 (float variables, double constants) */
+ORC_API void orc_hot3d_coefficients(int numCols, int numRows, int layers, float out[8])
+{
+    const float t_chip = 0.0005f, chip_height = 0.016f, chip_width = 0.016f;
+    float dx = chip_height / numRows, dy = chip_width / numCols, dz = t_chip / layers;
+    float Cap = 0.5 * 1.75e6 * t_chip * dx * dy;
+    float Rx = dy / (2.0 * 100 * t_chip * dx);
+    float Ry = dx / (2.0 * 100 * t_chip * dy);
+    float Rz = dz / (100 * dx * dy);
+    float max_slope = 3.0e6 / (0.5 * t_chip * 1.75e6);
+    float dt = 0.001 / max_slope;
+    float stepDivCap = dt / Cap;
+    float ce = stepDivCap / Rx, cn = stepDivCap / Ry, ct = stepDivCap / Rz;
+    float cc = 1.0 - (2.0 * ce + 2.0 * cn + 3.0 * ct);
+    out[0] = stepDivCap, out[1] = ce, out[2] = ce, out[3] = cn, out[4] = cn, out[5] = ct, out[6] = ct, out[7] = cc;
+}
+
+/* ------------------------------------------------------------------ path
+ * src/ori_kernel/path_kernel.cu:9-86 (general_ptb_path: src/gptb_kernel/path_kernel.cu:3-93):
+ * block bx works on the 256 columns from blkX = (256 - 2 iteration) bx - border; thread tx holds
+ * column blkX + tx.  prev[] starts as the source row where the column is on the grid.  Row i
+ * (0 <= i < iteration): threads with i + 1 <= tx <= 254 - i whose tx lies in [validXmin,
+ * validXmax] set result[tx] = min(prev[W], prev[tx], prev[E]) + wall[cols (startStep + i) + xidx],
+ * W = max(tx - 1, validXmin), E = min(tx + 1, validXmax); all but the last row then copy result to
+ * prev.  The threads that computed in the last row write result to gpuResults.
+ * Positions [start, end): bx = p (no wrap in the reference). */
+ORC_API void orc_path_gptb(int iteration, const int *wall, const int *src, int *results, int cols, int startStep,
+                           int border, int start, int end)
+{
+    enum { BS = 256 };
+    for (int bx = start; bx < end; ++bx) {
+        int prev[BS], result[BS], computed[BS];
+        const int small_block_cols = BS - iteration * 2;
+        const int blkX = small_block_cols * bx - border;
+        const int blkXmax = blkX + BS - 1;
+        const int validXmin = blkX < 0 ? -blkX : 0;
+        const int validXmax = blkXmax > cols - 1 ? BS - 1 - (blkXmax - cols + 1) : BS - 1;
+        for (int tx = 0; tx < BS; ++tx) {
+            const int xidx = blkX + tx;
+            prev[tx] = (xidx >= 0 && xidx <= cols - 1) ? src[xidx] : 0;
+            result[tx] = 0;
+            computed[tx] = 0;
+        }
+        for (int i = 0; i < iteration; ++i) {
+            for (int tx = 0; tx < BS; ++tx) {
+                computed[tx] = 0;
+                if (tx >= i + 1 && tx <= BS - i - 2 && tx >= validXmin && tx <= validXmax) {
+                    int W = tx - 1, E = tx + 1;
+                    if (W < validXmin) W = validXmin;
+                    if (E > validXmax) E = validXmax;
+                    int shortest = prev[W] <= prev[tx] ? prev[W] : prev[tx];
+                    shortest = shortest <= prev[E] ? shortest : prev[E];
+                    computed[tx] = 1;
+                    result[tx] = shortest + wall[(long long)cols * (startStep + i) + blkX + tx];
+                }
+            }
+            if (i == iteration - 1) break;
+            for (int tx = 0; tx < BS; ++tx)
+                if (computed[tx]) prev[tx] = result[tx];
+        }
+        for (int tx = 0; tx < BS; ++tx)
+            if (computed[tx]) results[blkX + tx] = result[tx];
+    }
+}
+
+/* the reference's grid: rand() % 10 after srand(9), row by row (src/ori_kernel/path_kernel.cu:113-119) */
+ORC_API void orc_path_source(int *cells, long long n)
+{
+    srand(9);
+    for (long long i = 0; i < n; ++i) cells[i] = rand() % 10;
 }

@@ -81,6 +81,18 @@ def _declare(lib):
     lib.tacker_gptb_fft.argtypes = [vp, i, i, i, i, i, vp]
     lib.tacker_mix_tzgemm_fft.argtypes = [vp, i, i, i] + gemm
     lib.tacker_mix_tzgemm_cp.argtypes = [i, f, vp, i, i, i, i] + gemm
+    lib.tacker_nn_blocks.argtypes = [i]
+    lib.tacker_ori_nn.argtypes = [vp, vp, i, f, f, vp]
+    lib.tacker_gptb_nn.argtypes = [vp, vp, i, f, f, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_nn.argtypes = [vp, vp, i, f, f, i, i] + gemm
+    lib.tacker_hot3d_coefficients.argtypes = [i, i, i, vp]
+    lib.tacker_ori_hot3d.argtypes = [vp, vp, vp, i, i, i, vp]
+    lib.tacker_gptb_hot3d.argtypes = [vp, vp, vp, i, i, i, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_hot3d.argtypes = [vp, vp, vp, i, i, i, i, i] + gemm
+    lib.tacker_path_blocks.argtypes = [i, i]
+    lib.tacker_ori_path.argtypes = [i, vp, vp, vp, i, i, i, vp]
+    lib.tacker_gptb_path.argtypes = [i, vp, vp, vp, i, i, i, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_path.argtypes = [i, vp, vp, vp, i, i, i, i, i] + gemm
     lib.tacker_im2col.argtypes = [vp] + [i] * 11 + [vp, vp]
     lib.tacker_convert_fp32_to_fp16.argtypes = [vp, vp, i, vp]
     lib.tacker_mnk_from_conv_args.argtypes = [C.POINTER(i), C.POINTER(i)]
@@ -90,6 +102,7 @@ def _declare(lib):
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
                  "tacker_ori_mriq_create", "tacker_ori_mrif_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
                  "tacker_ori_sgemm_create", "tacker_ori_fft_create", "tacker_ori_cutcp_create",
+                 "tacker_ori_nn_create", "tacker_ori_hot3d_create", "tacker_ori_path_create",
                  "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
                  "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
@@ -100,6 +113,9 @@ def _declare(lib):
     lib.tacker_ori_mrif_create.argtypes = [i, vp, vp, vp, vp, vp, i]
     lib.tacker_ori_sgemm_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_ori_fft_create.argtypes = [vp, i]
+    lib.tacker_ori_nn_create.argtypes = [vp, vp, i, f, f]
+    lib.tacker_ori_hot3d_create.argtypes = [vp, vp, vp, i, i, i]
+    lib.tacker_ori_path_create.argtypes = [i, vp, vp, vp, i, i, i]
     lib.tacker_ori_cutcp_create.argtypes = cut
     lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
     lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
@@ -570,6 +586,131 @@ def mix_tzgemm_fft(data, A, B, Cm, be_start=0, be_end=None, tile_start=0, tile_e
         _ptr(data), batches, be_start, batches if be_end is None else be_end,
         *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
         "tacker_mix_tzgemm_fft")
+
+
+# ---- Rodinia partners: nn, hot3d, path
+def nn_blocks(num_records):
+    return lib().tacker_nn_blocks(num_records)
+
+
+def _nn_records(locations, distances):
+    """locations: [n][2] float32 {lat, lng}; distances: [n] float32"""
+    if locations.dim() != 2 or locations.shape[1] != 2 or distances.numel() != locations.shape[0]:
+        raise ValueError("nn: locations must be [n][2] and distances [n]")
+    return locations.shape[0]
+
+
+def ori_nn(locations, distances, lat, lng, stream=None):
+    n = _nn_records(locations, distances)
+    check(lib().tacker_ori_nn(_ptr(locations), _ptr(distances), n, lat, lng, _stream(stream)), "tacker_ori_nn")
+
+
+def gptb_nn(locations, distances, lat, lng, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    n = _nn_records(locations, distances)
+    check(lib().tacker_gptb_nn(_ptr(locations), _ptr(distances), n, lat, lng, start,
+                               nn_blocks(n) if end is None else end, launch_grid, launch_block, _stream(stream)),
+          "tacker_gptb_nn")
+
+
+def mix_tzgemm_nn(locations, distances, lat, lng, A, B, Cm, be_start=0, be_end=None, tile_start=0, tile_end=None,
+                  variant=None, launch_grid=0, launch_block=0, stream=None):
+    n = _nn_records(locations, distances)
+    check(lib().tacker_mix_tzgemm_nn(
+        _ptr(locations), _ptr(distances), n, lat, lng, be_start, nn_blocks(n) if be_end is None else be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_nn")
+
+
+def ori_nn_create(locations, distances, lat, lng):
+    n = _nn_records(locations, distances)
+    return KernelHandle(lib().tacker_ori_nn_create(_ptr(locations), _ptr(distances), n, lat, lng), "OriNNKernel",
+                        keep=(locations, distances))
+
+
+def hot3d_coefficients(nx, ny, nz):
+    """{sdc, ce, cw, cn, cs, ct, cb, cc} of a step on nx x ny x nz cells, as float32 values."""
+    out = (C.c_float * 8)()
+    check(lib().tacker_hot3d_coefficients(nx, ny, nz, out), "tacker_hot3d_coefficients")
+    return dict(zip(("sdc", "ce", "cw", "cn", "cs", "ct", "cb", "cc"), [float(v) for v in out]))
+
+
+def hot3d_blocks(nx, ny):
+    return (nx // 64) * (ny // 4)
+
+
+def _hot3d_dims(p, t_in, t_out):
+    """p, t_in, t_out: [nz][ny][nx] float32"""
+    if t_in.dim() != 3 or tuple(p.shape) != tuple(t_in.shape) or tuple(t_out.shape) != tuple(t_in.shape):
+        raise ValueError("hot3d: p, t_in and t_out must be [nz][ny][nx] tensors of one shape")
+    nz, ny, nx = t_in.shape
+    return nx, ny, nz
+
+
+def ori_hot3d(p, t_in, t_out, stream=None):
+    check(lib().tacker_ori_hot3d(_ptr(p), _ptr(t_in), _ptr(t_out), *_hot3d_dims(p, t_in, t_out), _stream(stream)),
+          "tacker_ori_hot3d")
+
+
+def gptb_hot3d(p, t_in, t_out, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    nx, ny, nz = _hot3d_dims(p, t_in, t_out)
+    check(lib().tacker_gptb_hot3d(_ptr(p), _ptr(t_in), _ptr(t_out), nx, ny, nz, start,
+                                  hot3d_blocks(nx, ny) if end is None else end, launch_grid, launch_block,
+                                  _stream(stream)), "tacker_gptb_hot3d")
+
+
+def mix_tzgemm_hot3d(p, t_in, t_out, A, B, Cm, be_start=0, be_end=None, tile_start=0, tile_end=None, variant=None,
+                     launch_grid=0, launch_block=0, stream=None):
+    nx, ny, nz = _hot3d_dims(p, t_in, t_out)
+    check(lib().tacker_mix_tzgemm_hot3d(
+        _ptr(p), _ptr(t_in), _ptr(t_out), nx, ny, nz, be_start, hot3d_blocks(nx, ny) if be_end is None else be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_hot3d")
+
+
+def ori_hot3d_create(p, t_in, t_out):
+    return KernelHandle(lib().tacker_ori_hot3d_create(_ptr(p), _ptr(t_in), _ptr(t_out), *_hot3d_dims(p, t_in, t_out)),
+                        "OriHOT3DKernel", keep=(p, t_in, t_out))
+
+
+def path_blocks(cols, iteration):
+    return lib().tacker_path_blocks(cols, iteration)
+
+
+def _path_dims(wall, src, results):
+    """wall: [rows - 1][cols] int32 (the grid without its first row); src, results: [cols] int32"""
+    if wall.dim() != 2 or src.numel() != wall.shape[1] or results.numel() != wall.shape[1]:
+        raise ValueError("path: wall must be [rows - 1][cols], src and results [cols]")
+    return wall.shape[1], wall.shape[0] + 1
+
+
+def ori_path(iteration, wall, src, results, start_step=0, stream=None):
+    cols, rows = _path_dims(wall, src, results)
+    check(lib().tacker_ori_path(iteration, _ptr(wall), _ptr(src), _ptr(results), cols, rows, start_step,
+                                _stream(stream)), "tacker_ori_path")
+
+
+def gptb_path(iteration, wall, src, results, start_step=0, start=0, end=None, launch_grid=0, launch_block=0,
+              stream=None):
+    cols, rows = _path_dims(wall, src, results)
+    check(lib().tacker_gptb_path(iteration, _ptr(wall), _ptr(src), _ptr(results), cols, rows, start_step, start,
+                                 path_blocks(cols, iteration) if end is None else end, launch_grid, launch_block,
+                                 _stream(stream)), "tacker_gptb_path")
+
+
+def mix_tzgemm_path(iteration, wall, src, results, A, B, Cm, start_step=0, be_start=0, be_end=None, tile_start=0,
+                    tile_end=None, variant=None, launch_grid=0, launch_block=0, stream=None):
+    cols, rows = _path_dims(wall, src, results)
+    check(lib().tacker_mix_tzgemm_path(
+        iteration, _ptr(wall), _ptr(src), _ptr(results), cols, rows, start_step, be_start,
+        path_blocks(cols, iteration) if be_end is None else be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_path")
+
+
+def ori_path_create(iteration, wall, src, results, start_step=0):
+    cols, rows = _path_dims(wall, src, results)
+    return KernelHandle(lib().tacker_ori_path_create(iteration, _ptr(wall), _ptr(src), _ptr(results), cols, rows,
+                                                     start_step), "OriPATHKernel", keep=(wall, src, results))
 
 
 def mix_tzgemm_mriq(numK, x, y, z, Qr, Qi, A, B, Cm, be_start=0, be_end=None, tile_start=0,

@@ -49,6 +49,16 @@ GPTBKernel *createKernel(const std::string &name)
     } else if (name == "cutcp") {
         auto *ori = new OriCUTCPKernel(11);
         k = new GPTBKernel(11, "cutcp", "gptb_cutcp", ori, gptbGrid(name), gptbBlock(name, 128), 0, oriBlocks(name, ori));
+    } else if (name == "nn") {
+        // the reference gives all its Rodinia kernels the id 20 (src/Creator.cu:193-246)
+        auto *ori = new OriNNKernel(20);
+        k = new GPTBKernel(20, "nn", "gptb_nn", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
+    } else if (name == "hot3d") {
+        auto *ori = new OriHOT3DKernel(20);
+        k = new GPTBKernel(20, "hot3d", "gptb_hot3d", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
+    } else if (name == "path") {
+        auto *ori = new OriPATHKernel(20);
+        k = new GPTBKernel(20, "path", "gptb_path", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
     } else if (name == "fft") {
         auto *ori = new OriFFTKernel(12);
         k = new GPTBKernel(12, "fft", "gptb_fft", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));

@@ -520,6 +520,106 @@ int tacker_gptb_fft(float *data, int batches, int block_start, int block_end, in
 }
 
 namespace {
+int check_nn(const float *locations, float *distances, int numRecords)
+{
+    if (!locations || !distances || numRecords <= 0) return fail(TK_ERROR_INVALID_VALUE, "nn: bad arguments");
+    return TK_SUCCESS;
+}
+int check_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz)
+{
+    if (!p || !tIn || !tOut || nx <= 0 || ny <= 0 || nz <= 0 || tIn == tOut)
+        return fail(TK_ERROR_INVALID_VALUE, "hot3d: bad arguments");
+    if (nx % HOT3D_TILE_X || ny % HOT3D_TILE_Y || nz < 2)
+        return fail(TK_ERROR_UNSUPPORTED, "hot3d: nx must be a multiple of 64, ny of 4, and nz at least 2");
+    if ((long long)nx * ny * nz >= (1ll << 31)) return fail(TK_ERROR_UNSUPPORTED, "hot3d: a chip of 2^31 cells or more");
+    return TK_SUCCESS;
+}
+int check_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows, int startStep)
+{
+    if (!wall || !src || !results || cols <= 0 || rows <= 0 || startStep < 0 || src == results)
+        return fail(TK_ERROR_INVALID_VALUE, "path: bad arguments");
+    if (iteration < 1 || 2 * iteration * PATH_HALO >= PATH_BLOCK_SIZE)
+        return fail(TK_ERROR_UNSUPPORTED, "path: a pyramid of 1 .. 127 rows");
+    if ((long long)startStep + iteration > rows - 1)
+        return fail(TK_ERROR_INVALID_VALUE, "path: the pyramid reaches past the wall's last row");
+    if ((long long)cols * rows >= (1ll << 31)) return fail(TK_ERROR_UNSUPPORTED, "path: a wall of 2^31 cells or more");
+    return TK_SUCCESS;
+}
+}  // namespace
+
+int tacker_nn_blocks(int numRecords) { return nnBlocks(numRecords); }
+
+int tacker_ori_nn(const float *locations, float *distances, int numRecords, float lat, float lng, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_nn(locations, distances, numRecords);
+    if (rc) return rc;
+    return run_once(new OriNNKernel(0, (LatLong *)const_cast<float *>(locations), distances, numRecords, lat, lng), stream);
+}
+
+int tacker_gptb_nn(const float *locations, float *distances, int numRecords, float lat, float lng, int block_start,
+                   int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_nn(locations, distances, numRecords);
+    if (rc) return rc;
+    return run_gptb_once(new OriNNKernel(0, (LatLong *)const_cast<float *>(locations), distances, numRecords, lat, lng),
+                         block_start, block_end, launch_grid, launch_block, stream);
+}
+
+int tacker_hot3d_coefficients(int nx, int ny, int nz, float out[8])
+{
+    if (nx <= 0 || ny <= 0 || nz <= 0 || !out) return fail(TK_ERROR_INVALID_VALUE, "hot3d_coefficients: bad arguments");
+    OriHOT3DParamsStruct q{};
+    hot3dCoefficients(nx, ny, nz, &q);
+    const float v[8] = {q.sdc, q.ce, q.cw, q.cn, q.cs, q.ct, q.cb, q.cc};
+    for (int i = 0; i < 8; ++i) out[i] = v[i];
+    return TK_SUCCESS;
+}
+
+int tacker_ori_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_hot3d(p, tIn, tOut, nx, ny, nz);
+    if (rc) return rc;
+    return run_once(new OriHOT3DKernel(0, const_cast<float *>(p), const_cast<float *>(tIn), tOut, nx, ny, nz), stream);
+}
+
+int tacker_gptb_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz, int block_start,
+                      int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_hot3d(p, tIn, tOut, nx, ny, nz);
+    if (rc) return rc;
+    return run_gptb_once(new OriHOT3DKernel(0, const_cast<float *>(p), const_cast<float *>(tIn), tOut, nx, ny, nz),
+                         block_start, block_end, launch_grid, launch_block, stream);
+}
+
+int tacker_path_blocks(int cols, int iteration) { return pathBlocks(cols, iteration); }
+
+int tacker_ori_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows, int startStep,
+                    tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_path(iteration, wall, src, results, cols, rows, startStep);
+    if (rc) return rc;
+    return run_once(new OriPATHKernel(0, iteration, const_cast<int *>(wall), const_cast<int *>(src), results, cols, rows,
+                                      startStep),
+                    stream);
+}
+
+int tacker_gptb_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows, int startStep,
+                     int block_start, int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_path(iteration, wall, src, results, cols, rows, startStep);
+    if (rc) return rc;
+    return run_gptb_once(new OriPATHKernel(0, iteration, const_cast<int *>(wall), const_cast<int *>(src), results, cols,
+                                           rows, startStep),
+                         block_start, block_end, launch_grid, launch_block, stream);
+}
+
+namespace {
 int check_cutcp(int binDim_x, int binDim_y, const float *binZeroAddr, float h, const float *regionZeroAddr, int rx,
                 int ry, int rz)
 {
@@ -740,6 +840,41 @@ int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_end, co
                         variant, launch_grid, launch_block, stream);
 }
 
+int tacker_mix_tzgemm_nn(const float *locations, float *distances, int numRecords, float lat, float lng, int be_start,
+                         int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                         int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_nn(locations, distances, numRecords);
+    if (rc) return rc;
+    return run_mix_once(new OriNNKernel(0, (LatLong *)const_cast<float *>(locations), distances, numRecords, lat, lng),
+                        be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
+int tacker_mix_tzgemm_hot3d(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz, int be_start,
+                            int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                            int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_hot3d(p, tIn, tOut, nx, ny, nz);
+    if (rc) return rc;
+    return run_mix_once(new OriHOT3DKernel(0, const_cast<float *>(p), const_cast<float *>(tIn), tOut, nx, ny, nz),
+                        be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
+int tacker_mix_tzgemm_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows,
+                           int startStep, int be_start, int be_end, const void *A, const void *B, float *C, int M,
+                           int N, int K, int tile_start, int tile_end, const char *variant, int launch_grid,
+                           int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    const int rc = check_path(iteration, wall, src, results, cols, rows, startStep);
+    if (rc) return rc;
+    return run_mix_once(new OriPATHKernel(0, iteration, const_cast<int *>(wall), const_cast<int *>(src), results, cols,
+                                          rows, startStep),
+                        be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid, launch_block, stream);
+}
+
 int tacker_mix_tzgemm_cp(int numatoms, float gridspacing, float *energygrid, int volx, int voly, int be_start,
                          int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
                          int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
@@ -803,7 +938,8 @@ tacker_kernel_t tacker_create_kernel(const char *name)
         fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
         return nullptr;
     }
-    static const char *known[] = {"cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil", "tzgemm"};
+    static const char *known[] = {"cp",   "cutcp", "fft",  "hot3d", "lbm",     "mrif",
+                                  "mriq", "nn",    "path", "sgemm", "stencil", "tzgemm"};
     bool ok = false;
     for (auto k : known) ok |= (strcmp(k, name) == 0);
     if (!ok) {
@@ -856,6 +992,25 @@ tacker_kernel_t tacker_ori_cutcp_create(int binDim_x, int binDim_y, const float 
 tacker_kernel_t tacker_ori_fft_create(float *data, int batches)
 {
     CREATE(check_fft(data, batches), new OriFFTKernel(0, data, batches));
+}
+
+tacker_kernel_t tacker_ori_nn_create(const float *locations, float *distances, int numRecords, float lat, float lng)
+{
+    CREATE(check_nn(locations, distances, numRecords),
+           new OriNNKernel(0, (LatLong *)const_cast<float *>(locations), distances, numRecords, lat, lng));
+}
+
+tacker_kernel_t tacker_ori_hot3d_create(const float *p, const float *tIn, float *tOut, int nx, int ny, int nz)
+{
+    CREATE(check_hot3d(p, tIn, tOut, nx, ny, nz),
+           new OriHOT3DKernel(0, const_cast<float *>(p), const_cast<float *>(tIn), tOut, nx, ny, nz));
+}
+
+tacker_kernel_t tacker_ori_path_create(int iteration, const int *wall, const int *src, int *results, int cols, int rows,
+                                       int startStep)
+{
+    CREATE(check_path(iteration, wall, src, results, cols, rows, startStep),
+           new OriPATHKernel(0, iteration, const_cast<int *>(wall), const_cast<int *>(src), results, cols, rows, startStep));
 }
 
 tacker_kernel_t tacker_ori_sgemm_create(const float *A, const float *B, float *C, int M, int N, int K)
@@ -1251,14 +1406,22 @@ tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const ch
         fail(TK_ERROR_INVALID_VALUE, "tacker_task_manager_create: bad arguments");
         return nullptr;
     }
-    static const char *known[] = {"cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"};
-    bool ok1 = false, ok2 = !be2 || !*be2;
-    for (auto k : known) {
-        ok1 |= strcmp(k, be1) == 0;
-        if (be2) ok2 |= strcmp(k, be2) == 0;
-    }
-    if (!ok1 || !ok2) {
+    // fused pairs of two best-effort kernels exist within a family only (src/Creator.cu:341-640)
+    static const char *families[2][8] = {{"cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"},
+                                         {"hot3d", "nn", "path", nullptr, nullptr, nullptr, nullptr, nullptr}};
+    int family1 = -1, family2 = (!be2 || !*be2) ? -2 : -1;
+    for (int f = 0; f < 2; ++f)
+        for (auto k : families[f]) {
+            if (!k) continue;
+            if (strcmp(k, be1) == 0) family1 = f;
+            if (family2 == -1 && strcmp(k, be2) == 0) family2 = f;
+        }
+    if (family1 < 0 || family2 == -1) {
         fail(TK_ERROR_NOT_FOUND, "Creator: Kernel not found");
+        return nullptr;
+    }
+    if (family2 >= 0 && family2 != family1) {
+        fail(TK_ERROR_NOT_FOUND, std::string("Creator: no fused kernel of ") + be1 + " and " + be2);
         return nullptr;
     }
     return new TaskManager(static_cast<Task *>(lc_task), be1, be2 ? be2 : "");

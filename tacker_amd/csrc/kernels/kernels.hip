@@ -15,8 +15,11 @@
 #include "cutcp_role.h"
 #include "dnn_kernels.h"
 #include "fft_role.h"
+#include "hot3d_role.h"
 #include "lbm_role.h"
 #include "mriq_role.h"
+#include "nn_role.h"
+#include "path_role.h"
 #include "mrif_role.h"
 #include "sgemm_role.h"
 #include "stencil_role.h"
@@ -124,6 +127,65 @@ extern "C" __global__ __launch_bounds__(CUTCP_BLOCK_THREADS) void ori_cutcp(int 
 extern "C" __global__ __launch_bounds__(FFT_WAVE) void ori_fft(float *data)
 {
     tk::fft_role<1>(data, (int)gridDim.x, (int)blockIdx.x, (int)gridDim.x, 0, (int)gridDim.x, (int)threadIdx.x, FFT_WAVE);
+}
+
+// grid (blocks of 256 records, 1), block 256 (src/ori_kernel/nn_kernel.cu:9-17)
+extern "C" __global__ __launch_bounds__(NN_THREADS_PER_BLOCK) void ori_nn(LatLong *d_locations, float *d_distances,
+                                                                          int numRecords, float lat, float lng)
+{
+    const int blocks = (int)(gridDim.x * gridDim.y);
+    tk::nn_role(d_locations, d_distances, numRecords, lat, lng, (int)gridDim.x, (int)gridDim.y, (int)blockDim.x,
+                (int)(gridDim.x * blockIdx.y + blockIdx.x), blocks, 0, blocks, (int)threadIdx.x, (int)blockDim.x);
+}
+
+// grid (nx/64, ny/4), block (64,4) (src/ori_kernel/hot3d_kernel.cu:9-60)
+extern "C" __global__ __launch_bounds__(HOT3D_TILE_X *HOT3D_TILE_Y) void ori_hot3d(float *p, float *tIn, float *tOut,
+                                                                                  float sdc, int nx, int ny, int nz,
+                                                                                  float ce, float cw, float cn,
+                                                                                  float cs, float ct, float cb,
+                                                                                  float cc)
+{
+    const int blocks = (int)(gridDim.x * gridDim.y);
+    tk::hot3d_role(p, tIn, tOut, sdc, nx, ny, nz, ce, cw, cn, cs, ct, cb, cc, (int)gridDim.x, (int)gridDim.y,
+                   (int)blockDim.x, (int)blockDim.y, (int)(gridDim.x * blockIdx.y + blockIdx.x), blocks, 0, blocks,
+                   (int)(threadIdx.y * blockDim.x + threadIdx.x), (int)(blockDim.x * blockDim.y));
+}
+
+// grid (block positions), block 64: a wavefront per position where the reference means a block of
+// 256 threads (src/ori_kernel/path_kernel.cu:9-86)
+extern "C" __global__ __launch_bounds__(TK_WAVE_SIZE) void ori_path(int iteration, int *gpuWall, int *gpuSrc,
+                                                                    int *gpuResults, int cols, int rows, int startStep,
+                                                                    int border)
+{
+    (void)rows;
+    tk::path_role(iteration, gpuWall, gpuSrc, gpuResults, cols, startStep, border, (int)blockIdx.x, (int)gridDim.x, 0,
+                  (int)gridDim.x, (int)threadIdx.x, TK_WAVE_SIZE);
+}
+
+// Values that depend on (index, seed) only, for the default instances of the large kernels.
+__device__ __forceinline__ unsigned tk_fill_hash(unsigned long long i, unsigned seed)
+{
+    unsigned x = (unsigned)i ^ ((unsigned)(i >> 32) * 0x9E3779B9u) ^ seed;
+    x ^= x >> 16;
+    x *= 0x7feb352du;
+    x ^= x >> 15;
+    x *= 0x846ca68bu;
+    x ^= x >> 16;
+    return x;
+}
+extern "C" __global__ __launch_bounds__(256) void tk_fill_uniform(float *dst, unsigned long long n, unsigned seed,
+                                                                  float lo, float hi)
+{
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        dst[i] = lo + (hi - lo) * ((float)(tk_fill_hash(i, seed) >> 8) * (1.0f / 16777216.0f));
+}
+extern "C" __global__ __launch_bounds__(256) void tk_fill_int_mod(int *dst, unsigned long long n, unsigned seed,
+                                                                  int mod)
+{
+    const unsigned long long stride = (unsigned long long)gridDim.x * blockDim.x;
+    for (unsigned long long i = (unsigned long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+        dst[i] = (int)(tk_fill_hash(i, seed) % (unsigned)mod);
 }
 
 // grid (volx/128, voly/8), block (16,8)
@@ -270,6 +332,11 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ori_sgemm", (const void *)ori_sgemm, ctx);
     insert("ori_fft", (const void *)ori_fft, ctx);
     insert("ori_cutcp", (const void *)ori_cutcp, ctx);
+    insert("ori_nn", (const void *)ori_nn, ctx);
+    insert("ori_hot3d", (const void *)ori_hot3d, ctx);
+    insert("ori_path", (const void *)ori_path, ctx);
+    insert("fill_uniform", (const void *)tk_fill_uniform, ctx);
+    insert("fill_int_mod", (const void *)tk_fill_int_mod, ctx);
     insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);
     insert("tz_clear_words", (const void *)tz_clear_words, ctx);
     insert("cp_inv_sqrt_selftest", (const void *)cp_inv_sqrt_selftest, ctx);

@@ -61,6 +61,9 @@ const std::vector<int> MRIF = {I, I, P, P, P, P, P};
 const std::vector<int> CP = {I, F, P};
 const std::vector<int> SGEMM = {P, P, P, I, I, I};
 const std::vector<int> FFT = {P};
+const std::vector<int> NN = {P, P, I, F, F};
+const std::vector<int> HOT3D = {P, P, P, F, I, I, I, F, F, F, F, F, F, F};
+const std::vector<int> PATH = {I, P, P, P, I, I, I, I};
 const std::vector<int> CUTCP = {I, I, P, F, F, F, P, I};
 const std::vector<int> TZ = {P, P, P, I, I, I};
 }  // namespace
@@ -231,6 +234,11 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ori_sgemm", SGEMM);
         add("ori_fft", FFT);
         add("ori_cutcp", CUTCP);
+        add("ori_nn", NN);
+        add("ori_hot3d", HOT3D);
+        add("ori_path", PATH);
+        add("fill_uniform", {P, 8, I, F, F});
+        add("fill_int_mod", {P, 8, I, I});
         add("gptb_tzgemm", cat(TZ, trailer(true)));
         add("gptb_tzgemm@large", cat(TZ, trailer(true)));
         add("gptb_tzgemm_scratch", cat(cat(TZ, {P}), trailer(true)));
@@ -243,6 +251,9 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("gptb_sgemm", cat(SGEMM, trailer(true)));
         add("gptb_fft", cat(FFT, trailer(true)));
         add("gptb_cutcp", cat(CUTCP, trailer(true)));
+        add("gptb_nn", cat(NN, trailer(true)));
+        add("gptb_hot3d", cat(HOT3D, trailer(true)));
+        add("gptb_path", cat(PATH, trailer(true)));
         add("cp_inv_sqrt_selftest", {I, I, P});
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
@@ -255,18 +266,24 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
             {"stencil", &STENCIL}, {"lbm", &LBM}, {"mriq", &MRIQ}, {"cp", &CP}, {"mrif", &MRIF}, {"sgemm", &SGEMM},
             {"fft", &FFT}, {"cutcp", &CUTCP}};
         static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};
-        for (auto &be : bes)
-            for (auto v : variants)
-                add((std::string("tzgemm_") + be.first + v).c_str(),
-                    cat(cat(*be.second, trailer(false)), cat(TZ, trailer(false))));
+        // the Rodinia kernels pair with tzgemm and with each other only
+        const std::pair<const char *, const std::vector<int> *> rodinia[] = {{"nn", &NN}, {"hot3d", &HOT3D}, {"path", &PATH}};
+        for (auto *family : {&bes[0], &rodinia[0]})
+            for (auto *be = family; be != family + (family == &bes[0] ? 8 : 3); ++be)
+                for (auto v : variants)
+                    add((std::string("tzgemm_") + be->first + v).c_str(),
+                        cat(cat(*be->second, trailer(false)), cat(TZ, trailer(false))));
         // best-effort pairs, first < second alphabetically
         static const char *pair_variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1", "@ord_1_1", "@ord_1_2", "@ord_2_1"};
-        for (auto &a : bes)
-            for (auto &b : bes)
-                if (std::string(a.first) < std::string(b.first))
-                    for (auto v : pair_variants)
-                        add((std::string(a.first) + "_" + b.first + v).c_str(),
-                            cat(cat(*a.second, trailer(false)), cat(*b.second, trailer(false))));
+        for (auto *family : {&bes[0], &rodinia[0]}) {
+            const int n = family == &bes[0] ? 8 : 3;
+            for (auto *a = family; a != family + n; ++a)
+                for (auto *b = family; b != family + n; ++b)
+                    if (std::string(a->first) < std::string(b->first))
+                        for (auto v : pair_variants)
+                            add((std::string(a->first) + "_" + b->first + v).c_str(),
+                                cat(cat(*a->second, trailer(false)), cat(*b->second, trailer(false))));
+        }
     }
     for (auto *k : kernels()) insert(k->key.c_str(), k, ctx);
     return TK_SUCCESS;

@@ -64,6 +64,15 @@ KERNEL_INFO = {
     # 26 x 26 x 2 regions of 8 x 8 x 8 lattice points (two wavefronts each) x 11 parts of 32 neighbour bins
     "cutcp": {"register": 48, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
               "ori_blks": 14872},
+    # 2560000 blocks of 256 records
+    "nn": {"register": 32, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
+           "ori_blks": 2560000},
+    # 256 x 2048 patches of 64 x 4 columns, 8 layers each
+    "hot3d": {"register": 48, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
+              "ori_blks": 524288},
+    # 200 windows of 256 columns (6 result columns each), a wavefront each
+    "path": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 1,
+             "ori_blks": 200},
     # 16384 blocks of 128 x 8 points x 4 parts of the unrolled x points
     "cp": {"register": 40, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
            "ori_blks": 65536},

@@ -2,7 +2,8 @@
 
 Each entry plays the part of one ``<kernel>_code.py`` of the reference
 (fusion/code/cp_code.py, cutcp_code.py, fft_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
-truncated tzgemm_code.py): the kernel's parameter list in reference order and
+truncated tzgemm_code.py; the Rodinia kernels nn, hot3d and path have no such file there, their fused
+kernels are checked in under src/mix_kernel): the kernel's parameter list in reference order and
 how to call its device-side role.  The role bodies themselves live in
 ``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
 the reference's generated ``__global__`` functions call ``<a>_<b>_<k><i>()``
@@ -99,6 +100,37 @@ ROLES = {
         "call": ("tk::cutcp_role{extra}({p}binDim_x, {p}binDim_y, {p}binZeroAddr, {p}h, {p}cutoff2, {p}inv_cutoff2, "
                  "{p}regionZeroAddr, {p}grid_dimension_x, {p}grid_dimension_y, {p}grid_dimension_z, {block}, {blocks}, "
                  "{p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+    "nn": {
+        "gptb": {"symbol": "general_ptb_nn", "cite": "src/gptb_kernel/nn_kernel.cu:3-23",
+                 "attributes": "__launch_bounds__(256)"},
+        "params": [("LatLong*", "d_locations"), ("float*", "d_distances"), ("int", "numRecords"),
+                   ("float", "lat"), ("float", "lng")],
+        "needs_sync": False,
+        "call": ("tk::nn_role({p}d_locations, {p}d_distances, {p}numRecords, {p}lat, {p}lng, {p}grid_dimension_x, "
+                 "{p}grid_dimension_y, {p}block_dimension_x, {block}, {blocks}, {p}ptb_start_block_pos, "
+                 "{p}ptb_end_block_pos, {tid}, {threads});"),
+    },
+    "hot3d": {
+        "gptb": {"symbol": "general_ptb_hot3d", "cite": "src/gptb_kernel/hot3d_kernel.cu:3-62",
+                 "attributes": "__launch_bounds__(256)"},
+        "params": [("float*", "p"), ("float*", "tIn"), ("float*", "tOut"), ("float", "sdc"),
+                   ("int", "nx"), ("int", "ny"), ("int", "nz"), ("float", "ce"), ("float", "cw"),
+                   ("float", "cn"), ("float", "cs"), ("float", "ct"), ("float", "cb"), ("float", "cc")],
+        "needs_sync": False,
+        "call": ("tk::hot3d_role({p}p, {p}tIn, {p}tOut, {p}sdc, {p}nx, {p}ny, {p}nz, {p}ce, {p}cw, {p}cn, {p}cs, "
+                 "{p}ct, {p}cb, {p}cc, {p}grid_dimension_x, {p}grid_dimension_y, {p}block_dimension_x, "
+                 "{p}block_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "{threads});"),
+    },
+    "path": {
+        "gptb": {"symbol": "general_ptb_path", "cite": "src/gptb_kernel/path_kernel.cu:3-93",
+                 "attributes": "__launch_bounds__(256)"},
+        "params": [("int", "iteration"), ("int*", "gpuWall"), ("int*", "gpuSrc"), ("int*", "gpuResults"),
+                   ("int", "cols"), ("int", "rows"), ("int", "startStep"), ("int", "border")],
+        "needs_sync": False,
+        "call": ("tk::path_role({p}iteration, {p}gpuWall, {p}gpuSrc, {p}gpuResults, {p}cols, {p}startStep, "
+                 "{p}border, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, {threads});"),
     },
     "cp": {
         "gptb": {"symbol": "g_general_ptb_cp", "cite": "src/gptb_kernel/cp_kernel.cu:8-96", "attributes": ""},

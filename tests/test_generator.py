@@ -142,7 +142,14 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
     kinfo = json.loads(files["../config/kinfo-gfx950.json"])
     pairs = gen_run.be_pairs()
     names = ["cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"]
-    assert pairs == [(a, b) for i, a in enumerate(names) for b in names[i + 1:]] and len(pairs) == 28
+    parboil = [(a, b) for i, a in enumerate(names) for b in names[i + 1:]]
+    # the Rodinia kernels pair with each other only (src/Creator.cu:554-640, src/mix_kernel/{hot3d_nn,hot3d_path,nn_path}.cu)
+    rodinia = [("hot3d", "nn"), ("hot3d", "path"), ("nn", "path")]
+    assert pairs == sorted(parboil + rodinia) and len(pairs) == 31
+    sig = re.search(r"void hot3d_nn_mix_wg_1_1\(\s*(.*?)\)\s*\{", files["mix_kernel/hot3d_nn.hip"], re.S)
+    params = [q.split()[-1] for q in sig.group(1).split(",")]
+    assert len(params) == 23 + 14 and params[:3] == ["hot3d0_p", "hot3d0_tIn", "hot3d0_tOut"]      # hot3d_nn.cu:4-13
+    assert params[23:28] == ["nn1_d_locations", "nn1_d_distances", "nn1_numRecords", "nn1_lat", "nn1_lng"]
     # the fft pairs the reference ships: src/mix_kernel/{cp_fft_3_1,fft_lbm_6_1,fft_mriq_3_2,fft_sgemm_1_4,fft_stencil_5_3}.cu
     sig = re.search(r"void fft_lbm_mix_wg_1_1\(\s*(.*?)\)\s*\{", files["mix_kernel/fft_lbm.hip"], re.S)
     names = [q.split()[-1] for q in sig.group(1).split(",")]
