@@ -125,6 +125,37 @@ def pair_leg(ta, torch, np, name, stream):
         label = "tzgemm 2048^3 + fft 10240 x 256 points (reference mix tzgemm_fft)"
         reset = lambda: data.copy_(source)   # in place: every pass multiplies the magnitudes by 16
         n = 25
+    elif name == "nn":      # Rodinia nn, 256 x 2560000 records (the Creator's instance, src/ori_kernel/nn_kernel.cu:46)
+        records = 256 * 2560000
+        loc = torch.rand((records, 2), device="cuda:0") * 90.0
+        dist = torch.zeros(records, device="cuda:0")
+        be_ori = ta.ori_nn_create(loc, dist, 30.0, 90.0)
+        nblk = ta.nn_blocks(records)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "hbm", "algorithmic_bytes": 12.0 * records}
+        label = "tzgemm 2048^3 + nn 655360000 records (reference mix tzgemm_nn)"
+        n = 10
+    elif name == "hot3d":   # Rodinia hotspot3D, 16384 x 8192 x 8 cells (the Creator's instance, src/ori_kernel/hot3d_kernel.cu:80-82)
+        nx, ny, nz = 16384, 8192, 8
+        power = torch.rand((nz, ny, nx), device="cuda:0") * 0.01
+        t_in = torch.rand((nz, ny, nx), device="cuda:0") * 20.0 + 320.0
+        t_out = torch.zeros((nz, ny, nx), device="cuda:0")
+        be_ori = ta.ori_hot3d_create(power, t_in, t_out)
+        nblk = ta.hot3d_blocks(nx, ny)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "hbm", "algorithmic_bytes": 12.0 * nx * ny * nz}
+        label = "tzgemm 2048^3 + hotspot3D 16384x8192x8 (reference mix tzgemm_hot3d)"
+        n = 6
+    elif name == "path":    # Rodinia pathfinder, 1200 columns, pyramid of 125 rows (src/ori_kernel/path_kernel.cu:102)
+        cols, height = 1200, 125
+        wall = torch.from_numpy(rng.integers(0, 10, (height, cols), dtype=np.int32)).cuda()
+        src_row = torch.from_numpy(rng.integers(0, 10, cols, dtype=np.int32)).cuda()
+        result_row = torch.zeros(cols, dtype=torch.int32, device="cuda:0")
+        be_ori = ta.ori_path_create(height, wall, src_row, result_row)
+        nblk = ta.path_blocks(cols, height)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        work = {"bound": "valu", "pairs": 256.0 * nblk * height}   # column updates of the 200 windows
+        label = "tzgemm 2048^3 + pathfinder 1200 columns x 125 rows (reference mix tzgemm_path)"
     elif name == "lbm":     # D3Q19, 120x120x150, rest equilibrium + noise, 5 % obstacle cells
         sx, sy, sz = 120, 120, 150
         cells = sx * sy * sz
@@ -356,7 +387,7 @@ def main():
                     help="skip the other pairs (configs 3, 4) and the co-location latency leg (config 5)")
     ap.add_argument("--queries", type=int, default=1000, help="latency-critical queries of the co-location leg")
     ap.add_argument("--no-lc", action="store_true", help="skip the co-location latency legs (config 5)")
-    ap.add_argument("--pairs", default="lbm,mriq,cp,mrif,sgemm,fft,cutcp",
+    ap.add_argument("--pairs", default="lbm,mriq,cp,mrif,sgemm,fft,cutcp,nn,hot3d,path",
                     help="best-effort kernels of the other-pairs legs (comma separated); with a list of its own the "
                          "tzgemm shapes leg is skipped too (profiling runs)")
     args = ap.parse_args()

@@ -12,9 +12,13 @@
 // itself in the bottom layer and above the cell itself in the top layer -- so the output is
 // bit-identical to a CPU evaluation in the same order.
 //
-// gfx950: a lane reads its column's next layer and power value with coalesced 4-byte loads (a wave
-// covers one 256-byte row of the patch); the W/E/N/S values come from the lines its neighbours
-// just fetched.  The role's threads serve role_threads / (patch columns) positions at a time.
+// gfx950: for the reference's 64 x 4 patch a wavefront serves a position -- a lane takes 4 adjacent
+// columns of one row (16 lanes a row), so the next layer, the power and the rows to the north and
+// south come as 16-byte loads and the step leaves as 16-byte stores; only the two values beyond
+// the ends of the lane's four columns are single loads (from lines the wave fetched anyway).  The
+// wavefronts of a workgroup take positions next to each other in x, which makes the workgroup's
+// accesses 1 KiB runs per row.  Other patch shapes (and arrays that are not 16-byte aligned) take a
+// column per lane.
 #pragma once
 #include "role_common.h"
 #include "../header/hot3d_header.h"
@@ -61,6 +65,41 @@ __device__ __forceinline__ void hot3d_column(const float *__restrict__ p, const 
     tOut[c] = hot3d_cell(k, centre, tIn[W], tIn[E], tIn[S], tIn[N], below, above, p[c]);
 }
 
+// the reference's 64 x 4 patch (bx, by) by one wavefront: lane -> row lane / 16, columns 4 (lane % 16) .. + 3
+__device__ __forceinline__ void hot3d_patch_wave(const float *__restrict__ p, const float *__restrict__ tIn,
+                                                 float *__restrict__ tOut, const Hot3dCoefficients &k, int nx, int ny,
+                                                 int nz, int bx, int by, int lane)
+{
+    const int i = HOT3D_TILE_X * bx + 4 * (lane & 15);
+    const int j = HOT3D_TILE_Y * by + (lane >> 4);
+    if (i >= nx || j >= ny) return;
+    const long long xy = (long long)nx * ny;
+    long long c = i + (long long)j * nx;
+    // offsets of the neighbours relative to c, the same in every layer
+    const int w_off = (i == 0) ? 0 : -1;            // left of the first column
+    const int e_off = (i + 3 == nx - 1) ? 3 : 4;    // right of the fourth
+    const int n_off = (j == 0) ? 0 : -nx;
+    const int s_off = (j == ny - 1) ? 0 : nx;
+    float4 below, centre, above;
+    below = centre = *reinterpret_cast<const float4 *>(tIn + c);
+    for (int layer = 0; layer < nz; ++layer) {
+        above = layer < nz - 1 ? *reinterpret_cast<const float4 *>(tIn + c + xy) : centre;
+        const float4 north = *reinterpret_cast<const float4 *>(tIn + c + n_off);
+        const float4 south = *reinterpret_cast<const float4 *>(tIn + c + s_off);
+        const float4 power = *reinterpret_cast<const float4 *>(p + c);
+        const float west = tIn[c + w_off], east = tIn[c + e_off];
+        float4 out;
+        out.x = hot3d_cell(k, centre.x, west, centre.y, south.x, north.x, below.x, above.x, power.x);
+        out.y = hot3d_cell(k, centre.y, centre.x, centre.z, south.y, north.y, below.y, above.y, power.y);
+        out.z = hot3d_cell(k, centre.z, centre.y, centre.w, south.z, north.z, below.z, above.z, power.z);
+        out.w = hot3d_cell(k, centre.w, centre.z, east, south.w, north.w, below.w, above.w, power.w);
+        *reinterpret_cast<float4 *>(tOut + c) = out;
+        below = centre;
+        centre = above;
+        c += xy;
+    }
+}
+
 // Block positions [start, end) of the grid (grid_dimension_x, grid_dimension_y) of patches of
 // block_dimension_x x block_dimension_y columns are served by the role's role_blocks persistent
 // workgroups in turn; positions wrap as the reference's block_pos % grid_dimension_x,
@@ -77,6 +116,21 @@ __device__ __forceinline__ void hot3d_role(const float *__restrict__ p, const fl
         block_dimension_y <= 0 || nz < 2)
         return;
     const Hot3dCoefficients k{ce, cw, cn, cs, ct, cb, cc, sdc};
+    if (block_dimension_x == HOT3D_TILE_X && block_dimension_y == HOT3D_TILE_Y && nx % 4 == 0 &&
+        (((size_t)p | (size_t)tIn | (size_t)tOut) & 15) == 0) {
+        const int waves = role_threads / TK_WAVE_SIZE;
+        const int wave = tid / TK_WAVE_SIZE;
+        if (wave >= waves) return;
+        const int lane = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        // workgroup b takes positions (b + j role_blocks) waves + wave of the range, j = 0, 1, ...
+        for (long long pos = (long long)start + (long long)role_block * waves + wave; pos < end;
+             pos += (long long)role_blocks * waves) {
+            const unsigned q = (unsigned)pos;
+            hot3d_patch_wave(p, tIn, tOut, k, nx, ny, nz, (int)(q % (unsigned)grid_dimension_x),
+                             (int)((q / (unsigned)grid_dimension_x) % (unsigned)grid_dimension_y), lane);
+        }
+        return;
+    }
     const int patch = block_dimension_x * block_dimension_y;
     const int at_once = role_threads >= patch ? role_threads / patch : 1;
     const int group = role_threads >= patch ? tid / patch : 0;

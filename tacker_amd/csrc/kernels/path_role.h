@@ -13,17 +13,34 @@
 // that were computed in it are written to gpuResults.
 //
 // gfx950: a wavefront serves a position, a lane holds 4 consecutive columns of the window in
-// registers.  The neighbours across lanes come by lane shuffles, so the two block barriers a row
-// of the reference's block and its two shared arrays are gone; the rows of the wall, the only
-// memory traffic, are fetched PATH_ROWS_AHEAD rows ahead of the row being evaluated (the
-// dynamic programme itself is a dependent chain of `iteration` steps).
+// registers.  The neighbours across lanes come by a one-lane DPP shift of the wavefront, so the two
+// block barriers a row of the reference's block and its two shared arrays are gone.  The dynamic
+// programme is a dependent chain of `iteration` steps issued by one wavefront, so a step is kept to
+// a few instructions: every column is updated in every row without asking whether it still takes
+// part -- a column outside the shrinking pyramid holds a value nobody reads, since a column that
+// takes part in row i only reads columns that took part in row i - 1 -- and only the clamping at
+// the grid's two edges and the final store are predicated.  The rows of the wall, the only memory
+// traffic, are fetched PATH_ROWS_AHEAD rows ahead of the row being evaluated, from column indices
+// clamped to the grid so that no load needs a predicate either.
 #pragma once
 #include "role_common.h"
 #include "../header/path_header.h"
 
+#ifndef PATH_ROWS_AHEAD
 #define PATH_ROWS_AHEAD 8
+#endif
 
 namespace tk {
+
+// value of the lane below / above in the wavefront (the lane itself at the wavefront's ends)
+__device__ __forceinline__ int path_from_lane_below(int v)
+{
+    return __builtin_amdgcn_update_dpp(v, v, 0x138 /* wave_shr:1 */, 0xf, 0xf, false);
+}
+__device__ __forceinline__ int path_from_lane_above(int v)
+{
+    return __builtin_amdgcn_update_dpp(v, v, 0x130 /* wave_shl:1 */, 0xf, 0xf, false);
+}
 
 // one position, whole pyramid; lane = lane of the wavefront
 __device__ __forceinline__ void path_window(int iteration, const int *__restrict__ gpuWall,
@@ -38,63 +55,58 @@ __device__ __forceinline__ void path_window(int iteration, const int *__restrict
     const int validXmax = (blkXmax > cols - 1) ? PATH_BLOCK_SIZE - 1 - (blkXmax - cols + 1) : PATH_BLOCK_SIZE - 1;
     const int tx0 = C * lane;
 
-    int prev[C], result[C];
-    bool valid[C];
+    int prev[C];
+    unsigned column[C];   // unsigned: a load is a wave-uniform row pointer plus a 32-bit lane offset
+    bool at_min[C], at_max[C];
 #pragma unroll
     for (int k = 0; k < C; ++k) {
         const int tx = tx0 + k, xidx = blkX + tx;
-        valid[k] = tx >= validXmin && tx <= validXmax;
-        prev[k] = (xidx >= 0 && xidx <= cols - 1) ? gpuSrc[xidx] : 0;
-        result[k] = 0;
+        column[k] = (unsigned)(xidx < 0 ? 0 : (xidx > cols - 1 ? cols - 1 : xidx));   // on the grid, for the loads
+        at_min[k] = tx == validXmin;                                       // W clamps to the column itself
+        at_max[k] = tx == validXmax;                                       // E likewise
+        prev[k] = gpuSrc[column[k]];
     }
-    // row i of the wall for this lane's columns, where they take part in row i
-    auto fetch = [&](int i, int (&w)[C]) {
-        const long long row = (long long)cols * (startStep + i) + blkX;
-#pragma unroll
-        for (int k = 0; k < C; ++k) {
-            const int tx = tx0 + k;
-            const bool takes_part = i < iteration && valid[k] && tx >= i + 1 && tx <= PATH_BLOCK_SIZE - i - 2;
-            w[k] = takes_part ? gpuWall[row + tx] : 0;
-        }
-    };
+    const int *ahead = gpuWall + (long long)cols * startStep;   // the row the next fetch takes
     int wall[PATH_ROWS_AHEAD][C];
 #pragma unroll
-    for (int u = 0; u < PATH_ROWS_AHEAD; ++u) fetch(u, wall[u]);
-
-    bool computed[C];
+    for (int u = 0; u < PATH_ROWS_AHEAD; ++u)
+        if (u < iteration) {
 #pragma unroll
-    for (int k = 0; k < C; ++k) computed[k] = false;
+            for (int k = 0; k < C; ++k) wall[u][k] = ahead[column[k]];
+            ahead += cols;
+        }
     for (int base = 0; base < iteration; base += PATH_ROWS_AHEAD) {
 #pragma unroll
         for (int u = 0; u < PATH_ROWS_AHEAD; ++u) {
             const int i = base + u;
             if (i >= iteration) break;   // uniform
-            // the columns next to this lane's four
-            const int from_left = __shfl_up(prev[C - 1], 1);
-            const int from_right = __shfl_down(prev[0], 1);
+            const int from_left = path_from_lane_below(prev[C - 1]);
+            const int from_right = path_from_lane_above(prev[0]);
+            int next[C];
 #pragma unroll
             for (int k = 0; k < C; ++k) {
-                const int tx = tx0 + k;
-                computed[k] = valid[k] && tx >= i + 1 && tx <= PATH_BLOCK_SIZE - i - 2;
-                const int left_of = k == 0 ? from_left : prev[k - 1];
-                const int right_of = k == C - 1 ? from_right : prev[k + 1];
-                const int left = tx == validXmin ? prev[k] : left_of;      // W clamped to validXmin
-                const int right = tx == validXmax ? prev[k] : right_of;    // E clamped to validXmax
-                const int up = prev[k];
-                int shortest = left <= up ? left : up;
+                const int left = at_min[k] ? prev[k] : (k == 0 ? from_left : prev[k - 1]);
+                const int right = at_max[k] ? prev[k] : (k == C - 1 ? from_right : prev[k + 1]);
+                int shortest = left <= prev[k] ? left : prev[k];
                 shortest = shortest <= right ? shortest : right;
-                if (computed[k]) result[k] = shortest + wall[u][k];
+                next[k] = shortest + wall[u][k];
             }
-            if (i == iteration - 1) break;   // uniform
 #pragma unroll
-            for (int k = 0; k < C; ++k)
-                if (computed[k]) prev[k] = result[k];
-            fetch(i + PATH_ROWS_AHEAD, wall[u]);
+            for (int k = 0; k < C; ++k) prev[k] = next[k];
+            if (i + PATH_ROWS_AHEAD < iteration) {   // uniform
+#pragma unroll
+                for (int k = 0; k < C; ++k) wall[u][k] = ahead[column[k]];
+                ahead += cols;
+            }
         }
     }
+    // the columns that took part in the last row: the middle of the window, where it is on the grid
 #pragma unroll
-    for (int k = 0; k < C; ++k)
-        if (computed[k]) gpuResults[blkX + tx0 + k] = result[k];
+    for (int k = 0; k < C; ++k) {
+        const int tx = tx0 + k;
+        if (tx >= iteration && tx <= PATH_BLOCK_SIZE - 1 - iteration && tx >= validXmin && tx <= validXmax)
+            gpuResults[blkX + tx] = prev[k];
+    }
 }
 
 // Block positions [start, end) are served by the role's role_blocks x (role_threads / 64)

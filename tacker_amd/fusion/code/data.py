@@ -64,11 +64,13 @@ KERNEL_INFO = {
     # 26 x 26 x 2 regions of 8 x 8 x 8 lattice points (two wavefronts each) x 11 parts of 32 neighbour bins
     "cutcp": {"register": 48, "shared_memory": 0, "blocksize": 128, "solo_ptb_blks": 16,
               "ori_blks": 14872},
-    # 2560000 blocks of 256 records
-    "nn": {"register": 32, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
+    # 2560000 blocks of 256 records; a stream that wants many workgroups in flight (4.0 TB/s with 8 a CU,
+    # 4.95 with 32)
+    "nn": {"register": 48, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 32,
            "ori_blks": 2560000},
-    # 256 x 2048 patches of 64 x 4 columns, 8 layers each
-    "hot3d": {"register": 48, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
+    # 256 x 2048 patches of 64 x 4 columns, 8 layers each; 24 streams of 256-byte pieces per patch: fewer
+    # wavefronts in flight keep more of them in open memory pages (4.9 TB/s with 2 workgroups a CU, 3.9 with 8)
+    "hot3d": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 2,
               "ori_blks": 524288},
     # 200 windows of 256 columns (6 result columns each), a wavefront each
     "path": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 1,

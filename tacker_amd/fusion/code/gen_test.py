@@ -92,6 +92,23 @@ def make_inputs(np, torch, ta, be, small):
         # the benchmark instance computes the two lowest layers of regions of the 208^3 lattice
         inp = ta.CutcpInput(atoms, (0, 0, 0), n, n, n, 0.5, 12.0, regions=None if small else (26, 26, 2))
         return ta.ori_cutcp_create(inp, 144.0, 0.006944), inp.blocks(), [inp.energies]
+    if be == "nn":
+        records = 256 * 37 + 5 if small else 256 * 2560000
+        loc = torch.rand((records, 2), device="cuda:0") * 90.0
+        dist = torch.zeros(records, device="cuda:0")
+        return ta.ori_nn_create(loc, dist, 30.0, 90.0), ta.nn_blocks(records), [dist]
+    if be == "hot3d":
+        nx, ny, nz = (128, 16, 4) if small else (16384, 8192, 8)
+        power = torch.rand((nz, ny, nx), device="cuda:0") * 0.01
+        t_in = torch.rand((nz, ny, nx), device="cuda:0") * 20.0 + 320.0
+        t_out = torch.zeros((nz, ny, nx), device="cuda:0")
+        return ta.ori_hot3d_create(power, t_in, t_out), ta.hot3d_blocks(nx, ny), [t_out]
+    if be == "path":
+        cols, height = (700, 60) if small else (1200, 125)
+        wall = torch.from_numpy(rng.integers(0, 10, (height, cols), dtype=np.int32)).cuda()
+        src = torch.from_numpy(rng.integers(0, 10, cols, dtype=np.int32)).cuda()
+        out = torch.zeros(cols, dtype=torch.int32, device="cuda:0")
+        return ta.ori_path_create(height, wall, src, out), ta.path_blocks(cols, height), [out]
     if be == "sgemm":
         M, N, K = (256, 48, 300) if small else (4096, 4128, 4064)
         A = torch.from_numpy(rng.uniform(0, 1, (K, M)).astype(np.float32)).cuda()
