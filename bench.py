@@ -146,6 +146,22 @@ def pair_leg(ta, torch, np, name, stream):
         work = {"bound": "hbm", "algorithmic_bytes": 12.0 * nx * ny * nz}
         label = "tzgemm 2048^3 + hotspot3D 16384x8192x8 (reference mix tzgemm_hot3d)"
         n = 6
+    elif name == "lava":    # Rodinia lavaMD, 60^3 boxes of 100 particles (src/ori_kernel/lava_kernel.cu:163-175)
+        boxes1d = 60
+        particles = 100 * boxes1d ** 3
+        rv = torch.rand((particles, 4), device="cuda:0") * 0.9 + 0.1
+        qv = torch.rand(particles, device="cuda:0") * 0.9 + 0.1
+        fv = torch.zeros((particles, 4), device="cuda:0")
+        be_ori = ta.ori_lava_create(0.5, rv, qv, fv)
+        nblk = ta.lava_blocks(boxes1d)
+        tz, tiles, flop = gemm(2048, 2048, 2048)
+        # particle pairs: every box against itself and its neighbours (58^3 inner boxes have 26, faces fewer)
+        per_edge = [2 if c in (0, boxes1d - 1) else 3 for c in range(boxes1d)]
+        box_pairs = float(sum(per_edge)) ** 3
+        work = {"bound": "valu", "pairs": box_pairs * 100.0 * 100.0}
+        label = "tzgemm 2048^3 + lavaMD 60^3 boxes x 100 particles (reference mix tzgemm_lava)"
+        reset = fv.zero_        # the forces accumulate from launch to launch
+        n = 3
     elif name == "path":    # Rodinia pathfinder, 1200 columns, pyramid of 125 rows (src/ori_kernel/path_kernel.cu:102)
         cols, height = 1200, 125
         wall = torch.from_numpy(rng.integers(0, 10, (height, cols), dtype=np.int32)).cuda()
@@ -387,7 +403,7 @@ def main():
                     help="skip the other pairs (configs 3, 4) and the co-location latency leg (config 5)")
     ap.add_argument("--queries", type=int, default=1000, help="latency-critical queries of the co-location leg")
     ap.add_argument("--no-lc", action="store_true", help="skip the co-location latency legs (config 5)")
-    ap.add_argument("--pairs", default="lbm,mriq,cp,mrif,sgemm,fft,cutcp,nn,hot3d,path",
+    ap.add_argument("--pairs", default="lbm,mriq,cp,mrif,sgemm,fft,cutcp,nn,hot3d,path,lava",
                     help="best-effort kernels of the other-pairs legs (comma separated); with a list of its own the "
                          "tzgemm shapes leg is skipped too (profiling runs)")
     args = ap.parse_args()

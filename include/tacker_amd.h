@@ -314,6 +314,27 @@ TK_API int tacker_gptb_path(int iteration, const int *wall, const int *src, int 
                             int startStep, int block_start, int block_end, int launch_grid,
                             int launch_block, tkStream_t stream);
 
+/* ori_lava / general_ptb_lava (src/ori_kernel/lava_kernel.cu:9-141,
+ * src/gptb_kernel/lava_kernel.cu:3-140; Rodinia lavaMD): boxes1d^3 boxes of 100 particles; rv = per
+ * particle {v, x, y, z}, qv = its charge, fv = {potential, force x, y, z}, onto which every particle's
+ * sums over the particles of its own box and of the up to 26 boxes around it are added (rv and fv
+ * 16-byte aligned, distinct).  The box list (the reference's box_str array,
+ * src/ori_kernel/lava_kernel.cu:176-224) is built inside; tacker_lava_boxes writes it to a host
+ * buffer of boxes1d^3 * 656 bytes.  Block positions: boxes x 27 -- position p adds part
+ * (p / boxes) % 27 of box p % boxes (part 0 = the box itself, part k = its k-th neighbour), so
+ * ranges must be applied in ascending order to add a box's parts in the reference's order;
+ * tacker_lava_blocks = boxes1d^3 * 27.  A box is served by one wavefront (launch_block a multiple of
+ * 64) where the reference launches 128 threads.  fp32 in the order of the reference's source with
+ * the hardware's exponential: results agree with a CPU evaluation within rounding
+ * (|d| <= 2e-3 + 2e-5 |ref| for charges and coordinates in [0.1, 1]), not bit for bit. */
+TK_API int tacker_lava_blocks(int boxes1d);
+TK_API int tacker_lava_boxes(int boxes1d, void *out, size_t out_bytes);
+TK_API int tacker_ori_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv,
+                           tkStream_t stream);
+TK_API int tacker_gptb_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv,
+                            int block_start, int block_end, int launch_grid, int launch_block,
+                            tkStream_t stream);
+
 /* prepare_input (src/header/cutcp_header.h:111-300): hashes natoms atoms {x, y, z, q} into bins of
  * 4 x 4 x 4 Angstroms, 8 atoms to a bin, around a lattice of nx x ny x nz points of spacing h whose
  * lowest corner is lo, and lists the bin offsets a region of 8 x 8 x 8 points has to visit for the
@@ -423,7 +444,11 @@ TK_API int tacker_mix_tzgemm_fft(float *data, int batches, int be_start, int be_
                                  const void *B, float *C, int M, int N, int K, int tile_start,
                                  int tile_end, const char *variant, int launch_grid, int launch_block,
                                  tkStream_t stream);
-/* src/mix_kernel/tzgemm_nn.cu, tzgemm_hot3d.cu, tzgemm_path.cu */
+/* src/mix_kernel/tzgemm_nn.cu, tzgemm_hot3d.cu, tzgemm_path.cu, tzgemm_lava.cu */
+TK_API int tacker_mix_tzgemm_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv,
+                                  int be_start, int be_end, const void *A, const void *B, float *C, int M,
+                                  int N, int K, int tile_start, int tile_end, const char *variant,
+                                  int launch_grid, int launch_block, tkStream_t stream);
 TK_API int tacker_mix_tzgemm_nn(const float *locations, float *distances, int numRecords, float lat,
                                 float lng, int be_start, int be_end, const void *A, const void *B,
                                 float *C, int M, int N, int K, int tile_start, int tile_end,
@@ -478,6 +503,8 @@ TK_API tacker_kernel_t tacker_ori_nn_create(const float *locations, float *dista
                                             float lat, float lng);
 TK_API tacker_kernel_t tacker_ori_hot3d_create(const float *p, const float *tIn, float *tOut, int nx, int ny,
                                                int nz);
+TK_API tacker_kernel_t tacker_ori_lava_create(float alpha, int boxes1d, const float *rv, const float *qv,
+                                              float *fv);
 TK_API tacker_kernel_t tacker_ori_path_create(int iteration, const int *wall, const int *src, int *results,
                                               int cols, int rows, int startStep);
 TK_API tacker_kernel_t tacker_ori_cutcp_create(int binDim_x, int binDim_y, const float *binZeroAddr, float h,

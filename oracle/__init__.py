@@ -59,6 +59,8 @@ def _declare(l):
     l.orc_hot3d_coefficients.argtypes = [C.c_int, C.c_int, C.c_int, _f32p]
     l.orc_path_gptb.argtypes = [C.c_int, _i32p, _i32p, _i32p] + [C.c_int] * 5
     l.orc_path_source.argtypes = [_i32p, C.c_longlong]
+    l.orc_lava_boxes.argtypes = [C.c_int, C.c_void_p]
+    l.orc_lava_gptb.argtypes = [C.c_float, C.c_void_p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_lbm_gptb.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int]
     l.orc_lbm.argtypes = [_f32p, _f32p, C.c_int, C.c_int, C.c_int]
     l.orc_mriq_phimag.argtypes = [_f32p, _f32p, _f32p, C.c_int]
@@ -439,6 +441,37 @@ def path_source(rows, cols):
     out = np.zeros((rows, cols), np.int32)
     lib().orc_path_source(out.reshape(-1), out.size)
     return out
+
+
+LAVA_PARTS = 27
+LAVA_BOX = np.dtype([("x", "<i4"), ("y", "<i4"), ("z", "<i4"), ("number", "<i4"), ("offset", "<i8"), ("nn", "<i4"),
+                     ("pad", "<i4"), ("nei", [("x", "<i4"), ("y", "<i4"), ("z", "<i4"), ("number", "<i4"),
+                                              ("offset", "<i8")], 26)])
+
+
+def lava_boxes(boxes1d):
+    """The box list of a boxes1d^3 system as a structured array (the reference's box_str layout)."""
+    assert lib().orc_lava_box_bytes() == LAVA_BOX.itemsize == 656
+    out = np.zeros(boxes1d ** 3, LAVA_BOX)
+    lib().orc_lava_boxes(boxes1d, out.ctypes.data)
+    return out
+
+
+def lava_blocks(boxes1d):
+    return boxes1d ** 3 * LAVA_PARTS
+
+
+def lava(alpha, boxes1d, rv, qv, fv=None, start=0, end=None):
+    """lavaMD: rv [n][4] float32 {v, x, y, z}, qv [n] float32, n = 100 boxes1d^3; block positions
+    [start, end) of the boxes x 27 parts grid added onto fv (zeros if not given)."""
+    boxes = lava_boxes(boxes1d)
+    r = np.ascontiguousarray(rv, np.float32)
+    q = np.ascontiguousarray(qv, np.float32)
+    f = np.zeros_like(r) if fv is None else np.array(fv, np.float32)
+    if end is None:
+        end = lava_blocks(boxes1d)
+    lib().orc_lava_gptb(np.float32(alpha), boxes.ctypes.data, r.reshape(-1), q, f.reshape(-1), boxes1d ** 3, start, end)
+    return f
 
 
 # --------------------------------------------------------------------------- conv helpers

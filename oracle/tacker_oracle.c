@@ -54,6 +54,11 @@
  *                         brute force over all paths on a tiny wall, window edges at both ends of
  *                         the grid, column counts that are not a multiple of the window's yield,
  *                         any tiling of the positions; the input stream against rand() % 10.
+ *   orc_lava*             the neighbour lists by count (corner 7, edge 11, face 17, inside 26) and
+ *                         by symmetry, a float64 numpy evaluation of the same sums over the same
+ *                         lists, a single pair's closed form, equal charges => the forces of all
+ *                         particles sum to zero, any ascending tiling of the box-by-part grid
+ *                         (tests/test_oracle_rodinia.py).
  *   orc_im2col            direct convolution brute force.
  *   orc_gptb_index        partition invariance (any launch grid covers every
  *                         block once).
@@ -1095,4 +1100,78 @@ ORC_API void orc_path_source(int *cells, long long n)
 {
     srand(9);
     for (long long i = 0; i < n; ++i) cells[i] = rand() % 10;
+}
+
+
+/* ------------------------------------------------------------------ lava
+ * src/ori_kernel/lava_kernel.cu:9-141 (general_ptb_lava: src/gptb_kernel/lava_kernel.cu:3-140);
+ * the box list as src/ori_kernel/lava_kernel.cu:176-224 builds it.  Layouts of
+ * src/header/lava_header.h:16-45. */
+typedef struct { float v, x, y, z; } orc_four_vector;
+typedef struct { int x, y, z; int number; long offset; } orc_nei_str;
+typedef struct { int x, y, z; int number; long offset; int nn; orc_nei_str nei[26]; } orc_box_str;
+
+ORC_API int orc_lava_box_bytes(void) { return (int)sizeof(orc_box_str); }
+
+/* boxes1d^3 boxes, x fastest; the neighbours of a box in the order l (z), m (y), n (x) = -1, 0, 1 */
+ORC_API void orc_lava_boxes(int boxes1d, void *out)
+{
+    orc_box_str *box = (orc_box_str *)out;
+    int nh = 0;
+    for (int i = 0; i < boxes1d; i++)
+        for (int j = 0; j < boxes1d; j++)
+            for (int k = 0; k < boxes1d; k++) {
+                memset(&box[nh], 0, sizeof(orc_box_str));
+                box[nh].x = k, box[nh].y = j, box[nh].z = i;
+                box[nh].number = nh;
+                box[nh].offset = (long)nh * 100;
+                box[nh].nn = 0;
+                for (int l = -1; l < 2; l++)
+                    for (int m = -1; m < 2; m++)
+                        for (int n = -1; n < 2; n++) {
+                            const int inside = i + l >= 0 && j + m >= 0 && k + n >= 0 && i + l < boxes1d &&
+                                               j + m < boxes1d && k + n < boxes1d;
+                            if (!inside || (l == 0 && m == 0 && n == 0)) continue;
+                            orc_nei_str *ne = &box[nh].nei[box[nh].nn];
+                            ne->x = k + n, ne->y = j + m, ne->z = i + l;
+                            ne->number = ne->z * boxes1d * boxes1d + ne->y * boxes1d + ne->x;
+                            ne->offset = (long)ne->number * 100;
+                            box[nh].nn++;
+                        }
+                nh++;
+            }
+}
+
+/* Positions [start, end) of the grid boxes x 27: position p adds part (p / boxes) % 27 of box
+ * p % boxes (part 0 = the home box, part k = neighbour k - 1 of the list) onto fv, every home
+ * particle walking the part's 100 particles in order, all in float with expf. */
+ORC_API void orc_lava_gptb(float alpha, const void *boxes_, const float *rv_, const float *qv, float *fv_,
+                           int number_boxes, int start, int end)
+{
+    const orc_box_str *box = (const orc_box_str *)boxes_;
+    const orc_four_vector *rv = (const orc_four_vector *)rv_;
+    orc_four_vector *fv = (orc_four_vector *)fv_;
+    const float a2 = 2.0 * alpha * alpha;
+    for (int pos = start; pos < end; ++pos) {
+        const int bx = pos % number_boxes, k = (pos / number_boxes) % 27;
+        if (k >= 1 + box[bx].nn) continue;
+        const int pointer = k == 0 ? bx : box[bx].nei[k - 1].number;
+        const orc_four_vector *rA = rv + box[bx].offset, *rB = rv + box[pointer].offset;
+        const float *qB = qv + box[pointer].offset;
+        orc_four_vector *fA = fv + box[bx].offset;
+        for (int w = 0; w < 100; ++w)
+            for (int j = 0; j < 100; ++j) {
+                const float dot = rA[w].x * rB[j].x + rA[w].y * rB[j].y + rA[w].z * rB[j].z;
+                const float r2 = rA[w].v + rB[j].v - dot;
+                const float u2 = a2 * r2;
+                const float vij = expf(-u2);
+                const float fs = 2 * vij;
+                const float dx = rA[w].x - rB[j].x, dy = rA[w].y - rB[j].y, dz = rA[w].z - rB[j].z;
+                const float fxij = fs * dx, fyij = fs * dy, fzij = fs * dz;
+                fA[w].v += qB[j] * vij;
+                fA[w].x += qB[j] * fxij;
+                fA[w].y += qB[j] * fyij;
+                fA[w].z += qB[j] * fzij;
+            }
+    }
 }

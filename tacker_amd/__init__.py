@@ -89,6 +89,11 @@ def _declare(lib):
     lib.tacker_ori_hot3d.argtypes = [vp, vp, vp, i, i, i, vp]
     lib.tacker_gptb_hot3d.argtypes = [vp, vp, vp, i, i, i, i, i, i, i, vp]
     lib.tacker_mix_tzgemm_hot3d.argtypes = [vp, vp, vp, i, i, i, i, i] + gemm
+    lib.tacker_lava_blocks.argtypes = [i]
+    lib.tacker_lava_boxes.argtypes = [i, vp, C.c_size_t]
+    lib.tacker_ori_lava.argtypes = [f, i, vp, vp, vp, vp]
+    lib.tacker_gptb_lava.argtypes = [f, i, vp, vp, vp, i, i, i, i, vp]
+    lib.tacker_mix_tzgemm_lava.argtypes = [f, i, vp, vp, vp, i, i] + gemm
     lib.tacker_path_blocks.argtypes = [i, i]
     lib.tacker_ori_path.argtypes = [i, vp, vp, vp, i, i, i, vp]
     lib.tacker_gptb_path.argtypes = [i, vp, vp, vp, i, i, i, i, i, i, i, vp]
@@ -102,7 +107,7 @@ def _declare(lib):
     for name in ("tacker_create_kernel", "tacker_ori_stencil_create", "tacker_ori_lbm_create",
                  "tacker_ori_mriq_create", "tacker_ori_mrif_create", "tacker_ori_cp_create", "tacker_ori_tzgemm_create",
                  "tacker_ori_sgemm_create", "tacker_ori_fft_create", "tacker_ori_cutcp_create",
-                 "tacker_ori_nn_create", "tacker_ori_hot3d_create", "tacker_ori_path_create",
+                 "tacker_ori_nn_create", "tacker_ori_hot3d_create", "tacker_ori_path_create", "tacker_ori_lava_create",
                  "tacker_gptb_create", "tacker_mix_create", "tacker_be_pair_create",
                  "tacker_create_mix_kernel"):
         getattr(lib, name).restype = vp
@@ -116,6 +121,7 @@ def _declare(lib):
     lib.tacker_ori_nn_create.argtypes = [vp, vp, i, f, f]
     lib.tacker_ori_hot3d_create.argtypes = [vp, vp, vp, i, i, i]
     lib.tacker_ori_path_create.argtypes = [i, vp, vp, vp, i, i, i]
+    lib.tacker_ori_lava_create.argtypes = [f, i, vp, vp, vp]
     lib.tacker_ori_cutcp_create.argtypes = cut
     lib.tacker_ori_cp_create.argtypes = [i, f, vp, i, i]
     lib.tacker_ori_tzgemm_create.argtypes = [vp, vp, vp, i, i, i]
@@ -670,6 +676,45 @@ def mix_tzgemm_hot3d(p, t_in, t_out, A, B, Cm, be_start=0, be_end=None, tile_sta
 def ori_hot3d_create(p, t_in, t_out):
     return KernelHandle(lib().tacker_ori_hot3d_create(_ptr(p), _ptr(t_in), _ptr(t_out), *_hot3d_dims(p, t_in, t_out)),
                         "OriHOT3DKernel", keep=(p, t_in, t_out))
+
+
+def lava_blocks(boxes1d):
+    return lib().tacker_lava_blocks(boxes1d)
+
+
+def _lava_boxes1d(rv, qv, fv):
+    """rv, fv: [n][4] float32 {v, x, y, z}; qv: [n] float32; n = 100 boxes1d^3"""
+    n = qv.numel()
+    boxes1d = round((n / 100) ** (1 / 3))
+    if rv.dim() != 2 or rv.shape[1] != 4 or tuple(fv.shape) != tuple(rv.shape) or rv.shape[0] != n or \
+            100 * boxes1d ** 3 != n:
+        raise ValueError("lava: rv and fv must be [n][4], qv [n], n = 100 boxes1d^3")
+    return boxes1d
+
+
+def ori_lava(alpha, rv, qv, fv, stream=None):
+    check(lib().tacker_ori_lava(alpha, _lava_boxes1d(rv, qv, fv), _ptr(rv), _ptr(qv), _ptr(fv), _stream(stream)),
+          "tacker_ori_lava")
+
+
+def gptb_lava(alpha, rv, qv, fv, start=0, end=None, launch_grid=0, launch_block=0, stream=None):
+    b = _lava_boxes1d(rv, qv, fv)
+    check(lib().tacker_gptb_lava(alpha, b, _ptr(rv), _ptr(qv), _ptr(fv), start, lava_blocks(b) if end is None else end,
+                                 launch_grid, launch_block, _stream(stream)), "tacker_gptb_lava")
+
+
+def mix_tzgemm_lava(alpha, rv, qv, fv, A, B, Cm, be_start=0, be_end=None, tile_start=0, tile_end=None, variant=None,
+                    launch_grid=0, launch_block=0, stream=None):
+    b = _lava_boxes1d(rv, qv, fv)
+    check(lib().tacker_mix_tzgemm_lava(
+        alpha, b, _ptr(rv), _ptr(qv), _ptr(fv), be_start, lava_blocks(b) if be_end is None else be_end,
+        *_gemm_args(A, B, Cm, tile_start, tile_end, variant, launch_grid, launch_block, stream)),
+        "tacker_mix_tzgemm_lava")
+
+
+def ori_lava_create(alpha, rv, qv, fv):
+    return KernelHandle(lib().tacker_ori_lava_create(alpha, _lava_boxes1d(rv, qv, fv), _ptr(rv), _ptr(qv), _ptr(fv)),
+                        "OriLAVAKernel", keep=(rv, qv, fv))
 
 
 def path_blocks(cols, iteration):

@@ -56,6 +56,9 @@ GPTBKernel *createKernel(const std::string &name)
     } else if (name == "hot3d") {
         auto *ori = new OriHOT3DKernel(20);
         k = new GPTBKernel(20, "hot3d", "gptb_hot3d", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
+    } else if (name == "lava") {
+        auto *ori = new OriLAVAKernel(20);
+        k = new GPTBKernel(20, "lava", "gptb_lava", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));
     } else if (name == "path") {
         auto *ori = new OriPATHKernel(20);
         k = new GPTBKernel(20, "path", "gptb_path", ori, gptbGrid(name), gptbBlock(name, 256), 0, oriBlocks(name, ori));

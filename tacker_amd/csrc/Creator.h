@@ -11,13 +11,14 @@
 #include "ori_kernel/cutcp_kernel.h"
 #include "ori_kernel/fft_kernel.h"
 #include "ori_kernel/hot3d_kernel.h"
+#include "ori_kernel/lava_kernel.h"
 #include "ori_kernel/nn_kernel.h"
 #include "ori_kernel/path_kernel.h"
 #include "ori_kernel/sgemm_kernel.h"
 #include "ori_kernel/stencil_kernel.h"
 #include "tzgemm_kernel.h"
 
-// Memoised GPTB form of a best-effort kernel ("cp", "cutcp", "fft", "hot3d", "lbm", "mrif", "mriq", "nn", "path", "sgemm", "stencil") or
+// Memoised GPTB form of a best-effort kernel ("cp", "cutcp", "fft", "hot3d", "lava", "lbm", "mrif", "mriq", "nn", "path", "sgemm", "stencil") or
 // of the GEMM ("tzgemm"); an unknown name is logger.ERROR -> exit(1).
 GPTBKernel *createKernel(const std::string &name);
 

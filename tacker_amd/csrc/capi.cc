@@ -595,6 +595,58 @@ int tacker_gptb_hot3d(const float *p, const float *tIn, float *tOut, int nx, int
                          block_start, block_end, launch_grid, launch_block, stream);
 }
 
+namespace {
+int check_lava(int boxes1d, const float *rv, const float *qv, float *fv)
+{
+    if (!rv || !qv || !fv || rv == fv) return fail(TK_ERROR_INVALID_VALUE, "lava: bad arguments");
+    if (boxes1d < 1 || boxes1d > 128) return fail(TK_ERROR_UNSUPPORTED, "lava: 1 .. 128 boxes along an edge");
+    if ((((size_t)rv | (size_t)fv) & 15) != 0) return fail(TK_ERROR_INVALID_VALUE, "lava: rv and fv must be 16-byte aligned");
+    return TK_SUCCESS;
+}
+Kernel *new_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv, int *rc)
+{
+    Kernel *ori = nullptr;   // the box list is allocated and copied: not outside guarded()
+    *rc = guarded([&]() -> int {
+        ori = new OriLAVAKernel(0, alpha, boxes1d, (FOUR_VECTOR *)const_cast<float *>(rv), const_cast<float *>(qv),
+                                (FOUR_VECTOR *)fv);
+        return TK_SUCCESS;
+    });
+    return ori;
+}
+}  // namespace
+
+int tacker_lava_blocks(int boxes1d) { return boxes1d < 1 || boxes1d > 128 ? 0 : boxes1d * boxes1d * boxes1d * LAVA_PARTS; }
+
+int tacker_lava_boxes(int boxes1d, void *out, size_t out_bytes)
+{
+    if (boxes1d < 1 || boxes1d > 128 || !out) return fail(TK_ERROR_INVALID_VALUE, "lava_boxes: bad arguments");
+    const std::vector<box_str> boxes = lavaBoxes(boxes1d);
+    if (out_bytes < boxes.size() * sizeof(box_str)) return fail(TK_ERROR_INVALID_VALUE, "lava_boxes: buffer too small");
+    memcpy(out, boxes.data(), boxes.size() * sizeof(box_str));
+    return TK_SUCCESS;
+}
+
+int tacker_ori_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    int rc = check_lava(boxes1d, rv, qv, fv);
+    if (rc) return rc;
+    Kernel *ori = new_lava(alpha, boxes1d, rv, qv, fv, &rc);
+    if (rc) return rc;
+    return run_once(ori, stream);
+}
+
+int tacker_gptb_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv, int block_start,
+                     int block_end, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    int rc = check_lava(boxes1d, rv, qv, fv);
+    if (rc) return rc;
+    Kernel *ori = new_lava(alpha, boxes1d, rv, qv, fv, &rc);
+    if (rc) return rc;
+    return run_gptb_once(ori, block_start, block_end, launch_grid, launch_block, stream);
+}
+
 int tacker_path_blocks(int cols, int iteration) { return pathBlocks(cols, iteration); }
 
 int tacker_ori_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows, int startStep,
@@ -862,6 +914,19 @@ int tacker_mix_tzgemm_hot3d(const float *p, const float *tIn, float *tOut, int n
                         be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid, launch_block, stream);
 }
 
+int tacker_mix_tzgemm_lava(float alpha, int boxes1d, const float *rv, const float *qv, float *fv, int be_start,
+                           int be_end, const void *A, const void *B, float *C, int M, int N, int K, int tile_start,
+                           int tile_end, const char *variant, int launch_grid, int launch_block, tkStream_t stream)
+{
+    REQUIRE_INIT();
+    int rc = check_lava(boxes1d, rv, qv, fv);
+    if (rc) return rc;
+    Kernel *ori = new_lava(alpha, boxes1d, rv, qv, fv, &rc);
+    if (rc) return rc;
+    return run_mix_once(ori, be_start, be_end, A, B, C, M, N, K, tile_start, tile_end, variant, launch_grid,
+                        launch_block, stream);
+}
+
 int tacker_mix_tzgemm_path(int iteration, const int *wall, const int *src, int *results, int cols, int rows,
                            int startStep, int be_start, int be_end, const void *A, const void *B, float *C, int M,
                            int N, int K, int tile_start, int tile_end, const char *variant, int launch_grid,
@@ -938,7 +1003,7 @@ tacker_kernel_t tacker_create_kernel(const char *name)
         fail(TK_ERROR_INVALID_VALUE, "tacker_create_kernel: not initialised");
         return nullptr;
     }
-    static const char *known[] = {"cp",   "cutcp", "fft",  "hot3d", "lbm",     "mrif",
+    static const char *known[] = {"cp",   "cutcp", "fft", "hot3d", "lava",  "lbm",     "mrif",
                                   "mriq", "nn",    "path", "sgemm", "stencil", "tzgemm"};
     bool ok = false;
     for (auto k : known) ok |= (strcmp(k, name) == 0);
@@ -1004,6 +1069,13 @@ tacker_kernel_t tacker_ori_hot3d_create(const float *p, const float *tIn, float 
 {
     CREATE(check_hot3d(p, tIn, tOut, nx, ny, nz),
            new OriHOT3DKernel(0, const_cast<float *>(p), const_cast<float *>(tIn), tOut, nx, ny, nz));
+}
+
+tacker_kernel_t tacker_ori_lava_create(float alpha, int boxes1d, const float *rv, const float *qv, float *fv)
+{
+    CREATE(check_lava(boxes1d, rv, qv, fv),
+           new OriLAVAKernel(0, alpha, boxes1d, (FOUR_VECTOR *)const_cast<float *>(rv), const_cast<float *>(qv),
+                             (FOUR_VECTOR *)fv));
 }
 
 tacker_kernel_t tacker_ori_path_create(int iteration, const int *wall, const int *src, int *results, int cols, int rows,
@@ -1408,7 +1480,7 @@ tacker_task_manager_t tacker_task_manager_create(tacker_task_t lc_task, const ch
     }
     // fused pairs of two best-effort kernels exist within a family only (src/Creator.cu:341-640)
     static const char *families[2][8] = {{"cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"},
-                                         {"hot3d", "nn", "path", nullptr, nullptr, nullptr, nullptr, nullptr}};
+                                         {"hot3d", "lava", "nn", "path", nullptr, nullptr, nullptr, nullptr}};
     int family1 = -1, family2 = (!be2 || !*be2) ? -2 : -1;
     for (int f = 0; f < 2; ++f)
         for (auto k : families[f]) {

@@ -16,6 +16,7 @@
 #include "dnn_kernels.h"
 #include "fft_role.h"
 #include "hot3d_role.h"
+#include "lava_role.h"
 #include "lbm_role.h"
 #include "mriq_role.h"
 #include "nn_role.h"
@@ -160,6 +161,16 @@ extern "C" __global__ __launch_bounds__(TK_WAVE_SIZE) void ori_path(int iteratio
     (void)rows;
     tk::path_role(iteration, gpuWall, gpuSrc, gpuResults, cols, startStep, border, (int)blockIdx.x, (int)gridDim.x, 0,
                   (int)gridDim.x, (int)threadIdx.x, TK_WAVE_SIZE);
+}
+
+// grid (boxes), block 64: a wavefront per home box, all 27 parts of its work, where the reference
+// launches 128 threads (src/ori_kernel/lava_kernel.cu:9-141)
+extern "C" __global__ __launch_bounds__(TK_WAVE_SIZE) void ori_lava(par_str d_par_gpu, dim_str d_dim_gpu,
+                                                                    box_str *d_box_gpu, FOUR_VECTOR *d_rv_gpu,
+                                                                    float *d_qv_gpu, FOUR_VECTOR *d_fv_gpu)
+{
+    tk::lava_role(d_par_gpu, d_dim_gpu, d_box_gpu, d_rv_gpu, d_qv_gpu, d_fv_gpu, (int)gridDim.x, (int)blockIdx.x,
+                  (int)gridDim.x, 0, (int)gridDim.x * LAVA_PARTS, (int)threadIdx.x, TK_WAVE_SIZE);
 }
 
 // Values that depend on (index, seed) only, for the default instances of the large kernels.
@@ -335,6 +346,7 @@ extern "C" TK_API int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
     insert("ori_nn", (const void *)ori_nn, ctx);
     insert("ori_hot3d", (const void *)ori_hot3d, ctx);
     insert("ori_path", (const void *)ori_path, ctx);
+    insert("ori_lava", (const void *)ori_lava, ctx);
     insert("fill_uniform", (const void *)tk_fill_uniform, ctx);
     insert("fill_int_mod", (const void *)tk_fill_int_mod, ctx);
     insert("gptb_tzgemm_scratch", (const void *)general_ptb_tzgemm_scratch, ctx);

@@ -64,6 +64,7 @@ const std::vector<int> FFT = {P};
 const std::vector<int> NN = {P, P, I, F, F};
 const std::vector<int> HOT3D = {P, P, P, F, I, I, I, F, F, F, F, F, F, F};
 const std::vector<int> PATH = {I, P, P, P, I, I, I, I};
+const std::vector<int> LAVA = {4, 56, P, P, P, P};   // par_str and dim_str by value
 const std::vector<int> CUTCP = {I, I, P, F, F, F, P, I};
 const std::vector<int> TZ = {P, P, P, I, I, I};
 }  // namespace
@@ -237,6 +238,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("ori_nn", NN);
         add("ori_hot3d", HOT3D);
         add("ori_path", PATH);
+        add("ori_lava", LAVA);
         add("fill_uniform", {P, 8, I, F, F});
         add("fill_int_mod", {P, 8, I, I});
         add("gptb_tzgemm", cat(TZ, trailer(true)));
@@ -254,6 +256,7 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
         add("gptb_nn", cat(NN, trailer(true)));
         add("gptb_hot3d", cat(HOT3D, trailer(true)));
         add("gptb_path", cat(PATH, trailer(true)));
+        add("gptb_lava", cat(LAVA, trailer(true)));
         add("cp_inv_sqrt_selftest", {I, I, P});
         add("im2col", {I, P, I, I, I, I, I, I, I, I, I, I, I, I, P, I, I});
         add("convert_fp32_to_fp16", {P, P, I});
@@ -267,16 +270,16 @@ int tk_register_kernels(tk_kernel_insert_fn insert, void *ctx)
             {"fft", &FFT}, {"cutcp", &CUTCP}};
         static const char *variants[] = {"", "@wg_1_1", "@wg_1_2", "@wave_256", "@wave_512"};
         // the Rodinia kernels pair with tzgemm and with each other only
-        const std::pair<const char *, const std::vector<int> *> rodinia[] = {{"nn", &NN}, {"hot3d", &HOT3D}, {"path", &PATH}};
+        const std::pair<const char *, const std::vector<int> *> rodinia[] = {{"nn", &NN}, {"hot3d", &HOT3D}, {"path", &PATH}, {"lava", &LAVA}};
         for (auto *family : {&bes[0], &rodinia[0]})
-            for (auto *be = family; be != family + (family == &bes[0] ? 8 : 3); ++be)
+            for (auto *be = family; be != family + (family == &bes[0] ? 8 : 4); ++be)
                 for (auto v : variants)
                     add((std::string("tzgemm_") + be->first + v).c_str(),
                         cat(cat(*be->second, trailer(false)), cat(TZ, trailer(false))));
         // best-effort pairs, first < second alphabetically
         static const char *pair_variants[] = {"", "@wg_1_1", "@wg_1_2", "@wg_2_1", "@ord_1_1", "@ord_1_2", "@ord_2_1"};
         for (auto *family : {&bes[0], &rodinia[0]}) {
-            const int n = family == &bes[0] ? 8 : 3;
+            const int n = family == &bes[0] ? 8 : 4;
             for (auto *a = family; a != family + n; ++a)
                 for (auto *b = family; b != family + n; ++b)
                     if (std::string(a->first) < std::string(b->first))

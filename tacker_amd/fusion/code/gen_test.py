@@ -103,6 +103,13 @@ def make_inputs(np, torch, ta, be, small):
         t_in = torch.rand((nz, ny, nx), device="cuda:0") * 20.0 + 320.0
         t_out = torch.zeros((nz, ny, nx), device="cuda:0")
         return ta.ori_hot3d_create(power, t_in, t_out), ta.hot3d_blocks(nx, ny), [t_out]
+    if be == "lava":
+        boxes1d = 2 if small else 60
+        n = 100 * boxes1d ** 3
+        rv = torch.rand((n, 4), device="cuda:0") * 0.9 + 0.1
+        qv = torch.rand(n, device="cuda:0") * 0.9 + 0.1
+        fv = torch.zeros((n, 4), device="cuda:0")
+        return ta.ori_lava_create(0.5, rv, qv, fv), ta.lava_blocks(boxes1d), [fv]
     if be == "path":
         cols, height = (700, 60) if small else (1200, 125)
         wall = torch.from_numpy(rng.integers(0, 10, (height, cols), dtype=np.int32)).cuda()

@@ -2,7 +2,7 @@
 
 Each entry plays the part of one ``<kernel>_code.py`` of the reference
 (fusion/code/cp_code.py, cutcp_code.py, fft_code.py, lbm_code.py, mriq_code.py, mrif_code.py, sgemm_code.py, stencil_code.py and the
-truncated tzgemm_code.py; the Rodinia kernels nn, hot3d and path have no such file there, their fused
+truncated tzgemm_code.py; the Rodinia kernels nn, hot3d, lava and path have no such file there, their fused
 kernels are checked in under src/mix_kernel): the kernel's parameter list in reference order and
 how to call its device-side role.  The role bodies themselves live in
 ``csrc/kernels/*_role.h``; the generator emits dispatchers around them, the way
@@ -121,6 +121,16 @@ ROLES = {
         "call": ("tk::hot3d_role({p}p, {p}tIn, {p}tOut, {p}sdc, {p}nx, {p}ny, {p}nz, {p}ce, {p}cw, {p}cn, {p}cs, "
                  "{p}ct, {p}cb, {p}cc, {p}grid_dimension_x, {p}grid_dimension_y, {p}block_dimension_x, "
                  "{p}block_dimension_y, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
+                 "{threads});"),
+    },
+    "lava": {
+        "gptb": {"symbol": "general_ptb_lava", "cite": "src/gptb_kernel/lava_kernel.cu:3-140",
+                 "attributes": "__launch_bounds__(256)"},
+        "params": [("par_str", "d_par_gpu"), ("dim_str", "d_dim_gpu"), ("box_str*", "d_box_gpu"),
+                   ("FOUR_VECTOR*", "d_rv_gpu"), ("float*", "d_qv_gpu"), ("FOUR_VECTOR*", "d_fv_gpu")],
+        "needs_sync": False,
+        "call": ("tk::lava_role({p}d_par_gpu, {p}d_dim_gpu, {p}d_box_gpu, {p}d_rv_gpu, {p}d_qv_gpu, {p}d_fv_gpu, "
+                 "{p}grid_dimension_x, {block}, {blocks}, {p}ptb_start_block_pos, {p}ptb_end_block_pos, {tid}, "
                  "{threads});"),
     },
     "path": {

@@ -31,7 +31,7 @@ ROOT = os.path.abspath(os.path.join(HERE, "..", "..", ".."))
 DEFAULTS = os.path.join(HERE, "defaults.json")
 # reduction lengths of the VGG16 batch-1 layers after padding to 128, plus the benchmark's
 K_LADDER = (128, 640, 1152, 2048, 2304, 4096, 4608)
-PAIRS = ("stencil", "lbm", "mriq", "cp", "mrif", "sgemm", "fft", "cutcp", "nn", "hot3d", "path")
+PAIRS = ("stencil", "lbm", "mriq", "cp", "mrif", "sgemm", "fft", "cutcp", "nn", "hot3d", "path", "lava")
 TILES = 1024
 LADDER = 32          # best-effort block counts tried: N/1024, N/512, ..., N/64, then N/32, 2N/32, ..., N
 

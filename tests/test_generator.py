@@ -143,9 +143,14 @@ def test_best_effort_pairs_are_emitted_in_alphabetical_order_with_kinfo():
     pairs = gen_run.be_pairs()
     names = ["cp", "cutcp", "fft", "lbm", "mrif", "mriq", "sgemm", "stencil"]
     parboil = [(a, b) for i, a in enumerate(names) for b in names[i + 1:]]
-    # the Rodinia kernels pair with each other only (src/Creator.cu:554-640, src/mix_kernel/{hot3d_nn,hot3d_path,nn_path}.cu)
-    rodinia = [("hot3d", "nn"), ("hot3d", "path"), ("nn", "path")]
-    assert pairs == sorted(parboil + rodinia) and len(pairs) == 31
+    # the Rodinia kernels pair with each other only (src/Creator.cu:554-640,
+    # src/mix_kernel/{hot3d_lava,hot3d_nn,hot3d_path,lava_nn,lava_path,nn_path}.cu)
+    rodinia = [("hot3d", "lava"), ("hot3d", "nn"), ("hot3d", "path"), ("lava", "nn"), ("lava", "path"), ("nn", "path")]
+    assert pairs == sorted(parboil + rodinia) and len(pairs) == 34
+    sig = re.search(r"void lava_nn_mix_wg_1_1\(\s*(.*?)\)\s*\{", files["mix_kernel/lava_nn.hip"], re.S)
+    params = [q.split() for q in sig.group(1).split(",")]
+    assert [q[0] for q in params[:6]] == ["par_str", "dim_str", "box_str*", "FOUR_VECTOR*", "float*", "FOUR_VECTOR*"]  # lava_nn.cu:4-10
+    assert len(params) == 15 + 14
     sig = re.search(r"void hot3d_nn_mix_wg_1_1\(\s*(.*?)\)\s*\{", files["mix_kernel/hot3d_nn.hip"], re.S)
     params = [q.split()[-1] for q in sig.group(1).split(",")]
     assert len(params) == 23 + 14 and params[:3] == ["hot3d0_p", "hot3d0_tIn", "hot3d0_tOut"]      # hot3d_nn.cu:4-13

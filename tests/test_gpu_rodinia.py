@@ -1,8 +1,10 @@
-"""GPU parity of the Rodinia partners nn, hotspot3D and pathfinder (src/ori_kernel/{nn,hot3d,path}_kernel.cu,
-src/gptb_kernel/*, src/mix_kernel/tzgemm_{nn,hot3d,path}.cu, hot3d_nn.cu, hot3d_path.cu, nn_path.cu): bit for
-bit against the oracle -- fp32 in the reference's operation order for nn and hot3d, integers for path --
-for the natural launch, the GPTB form over any tiling of its positions, every fused variant with tzgemm and
-every fused pair among the three."""
+"""GPU parity of the Rodinia partners nn, hotspot3D, pathfinder and lavaMD
+(src/ori_kernel/{nn,hot3d,path,lava}_kernel.cu, src/gptb_kernel/*, src/mix_kernel/tzgemm_{nn,hot3d,path,lava}.cu,
+hot3d_nn.cu, hot3d_path.cu, nn_path.cu, hot3d_lava.cu, lava_nn.cu, lava_path.cu): bit for bit against the oracle
+-- fp32 in the reference's operation order for nn and hot3d, integers for path -- and within
+|d| <= 2e-3 + 2e-5 |ref| for lavaMD (the hardware's exponential against the C library's), for the natural
+launch, the GPTB form over any tiling of its positions, every fused variant with tzgemm and every fused pair
+among the four; every device form of the same lavaMD work gives the same bits as every other."""
 import numpy as np
 import pytest
 import torch
@@ -172,6 +174,78 @@ def test_path_walks_a_grid_pyramid_by_pyramid():
     assert np.array_equal(host(a), cur.astype(np.int32))
 
 
+# ----------------------------------------------------------------------------- lava
+def lava_inputs(boxes1d, seed=4):
+    rng = np.random.default_rng(seed)
+    n = 100 * boxes1d ** 3
+    return (rng.integers(1, 11, (n, 4)) / 10.0).astype(np.float32), (rng.integers(1, 11, n) / 10.0).astype(np.float32)
+
+
+def lava_close(got, want):
+    """|d| <= 2e-3 + 2e-5 |ref|: sums of up to 2700 terms of order 0.3 in fp32, the exponential from the
+    hardware's 2^x here and from expf there"""
+    return bool(np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 2e-3 + 2e-5 * np.abs(want)))
+
+
+@pytest.mark.parametrize("boxes1d", [1, 2, 3])
+def test_lava_forms_match_the_oracle(boxes1d):
+    rv, qv = lava_inputs(boxes1d, seed=boxes1d)
+    want = oracle.lava(0.5, boxes1d, rv, qv)
+    d_r, d_q = dev(rv), dev(qv)
+    out = [torch.zeros((rv.shape[0], 4), device="cuda:0") for _ in range(3)]
+    ta.ori_lava(0.5, d_r, d_q, out[0])
+    ta.gptb_lava(0.5, d_r, d_q, out[1])
+    ta.gptb_lava(0.5, d_r, d_q, out[2], launch_grid=3, launch_block=128)
+    assert lava_close(host(out[0]), want)
+    # a box is one wavefront's work whatever the launch: the three forms agree bit for bit
+    assert np.array_equal(bits(out[1]), bits(out[0])) and np.array_equal(bits(out[2]), bits(out[0]))
+    # float64 over the same neighbour lists
+    boxes = oracle.lava_boxes(boxes1d)
+    r, q = rv.astype(np.float64), qv.astype(np.float64)
+    b = boxes[len(boxes) // 2]
+    A = r[100 * b["number"]:100 * b["number"] + 100]
+    pot = np.zeros(100)
+    for other in [b["number"]] + b["nei"][:b["nn"]]["number"].tolist():
+        B = r[100 * other:100 * other + 100]
+        pot += np.exp(-0.5 * (A[:, None, 0] + B[None, :, 0] - A[:, 1:] @ B[:, 1:].T)) @ q[100 * other:100 * other + 100]
+    np.testing.assert_allclose(host(out[0])[100 * b["number"]:100 * b["number"] + 100, 0], pot, rtol=2e-5)
+    assert ta.lava_blocks(boxes1d) == oracle.lava_blocks(boxes1d)
+
+
+def test_lava_box_list_is_the_oracles():
+    for boxes1d in (1, 2, 5):
+        want = oracle.lava_boxes(boxes1d)
+        got = np.zeros(boxes1d ** 3, oracle.LAVA_BOX)
+        assert ta.lib().tacker_lava_boxes(boxes1d, got.ctypes.data, got.nbytes) == 0
+        assert got.tobytes() == want.tobytes()
+    assert ta.lib().tacker_lava_boxes(2, got.ctypes.data, 100) != 0        # buffer too small
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_lava_any_ascending_tiling_of_the_positions(seed):
+    rng = np.random.default_rng(400 + seed)
+    boxes1d = int(rng.choice([2, 3]))
+    rv, qv = lava_inputs(boxes1d, seed=seed)
+    n = ta.lava_blocks(boxes1d)
+    d_r, d_q = dev(rv), dev(qv)
+    whole = torch.zeros((rv.shape[0], 4), device="cuda:0")
+    ta.gptb_lava(0.5, d_r, d_q, whole)
+    cuts = sorted(set(rng.integers(0, n + 1, 4).tolist()) | {0, n})
+    out = torch.zeros((rv.shape[0], 4), device="cuda:0")
+    for a, b in zip(cuts, cuts[1:]):
+        ta.gptb_lava(0.5, d_r, d_q, out, a, b, launch_grid=int(rng.choice([1, 5, 64])),
+                     launch_block=int(rng.choice([64, 128, 256])))
+    assert np.array_equal(bits(out), bits(whole))
+    # one position: its box's forces move, on top of what the array held, and nothing else does
+    boxes = boxes1d ** 3
+    base = np.full((rv.shape[0], 4), 3.0, np.float32)
+    out = dev(base)
+    ta.gptb_lava(0.5, d_r, d_q, out, boxes + 1, boxes + 2)          # box 1, its first neighbour
+    want = oracle.lava(0.5, boxes1d, rv, qv, fv=base, start=boxes + 1, end=boxes + 2)
+    got = host(out)
+    assert lava_close(got, want) and np.array_equal(np.delete(got, np.s_[100:200], axis=0), np.delete(base, np.s_[100:200], axis=0))
+
+
 # ----------------------------------------------------------------------------- fused with tzgemm
 def _small(name):
     """(ori kernel, block positions, output tensor, oracle's output, dtype view)"""
@@ -183,6 +257,11 @@ def _small(name):
         p, t = hot3d_inputs(256, 24, 8, seed=42)
         out = torch.full((8, 24, 256), -1.0, device="cuda:0")
         return ta.ori_hot3d_create(dev(p), dev(t), out), ta.hot3d_blocks(256, 24), out, oracle.hot3d(p, t)
+    if name == "lava":
+        rv, qv = lava_inputs(2, seed=44)
+        out = torch.full((rv.shape[0], 4), -1.0, device="cuda:0")
+        return (ta.ori_lava_create(0.5, dev(rv), dev(qv), out), ta.lava_blocks(2), out,
+                oracle.lava(0.5, 2, rv, qv, fv=np.full((rv.shape[0], 4), -1.0, np.float32)))
     wall, src = path_inputs(1500, 101, seed=43)
     out = torch.full((1500,), -1, dtype=torch.int32, device="cuda:0")
     return (ta.ori_path_create(100, dev(wall), dev(src), out), ta.path_blocks(1500, 100), out,
@@ -190,10 +269,13 @@ def _small(name):
 
 
 def _same(t, want):
+    """the oracle's bits; for lava (float32 [n][4] sums) the stated tolerance"""
+    if t.dtype == torch.float32 and t.dim() == 2:
+        return lava_close(host(t), want)
     return np.array_equal(host(t).view(np.uint32), np.ascontiguousarray(want).view(np.uint32))
 
 
-@pytest.mark.parametrize("be", ["nn", "hot3d", "path"])
+@pytest.mark.parametrize("be", ["nn", "hot3d", "path", "lava"])
 @pytest.mark.parametrize("variant", [None, "wave_256", "wave_512", "wg_1_1", "wg_1_2"])
 def test_mix_with_tzgemm(be, variant):
     M, N, K = 256, 256, 256
@@ -207,6 +289,7 @@ def test_mix_with_tzgemm(be, variant):
     g_tz = ta.gptb_create(ta.ori_tzgemm_create(a, b, mix_c), 0, 0, 0, 16)
     ta.mix_create(g_be, g_tz, 0, n, 0, 16, variant=variant).execute()
     assert _same(out, want)
+    first_bits = bits(out).copy()
     assert np.array_equal(host(mix_c), host(solo_c))
     ok, fro, dmax = gemm_tolerance_ok(host(mix_c), oracle.tzgemm(A, B, f64=True), K)
     assert ok and fro <= 1e-5
@@ -216,12 +299,12 @@ def test_mix_with_tzgemm(be, variant):
     cut = max(1, n // 3)
     ta.mix_create(g_be, g_tz, 0, cut, 0, 5, variant=variant).execute()
     ta.mix_create(g_be, g_tz, cut, n, 5, 16, variant=variant).execute()
-    assert _same(out, want)
+    assert _same(out, want) and np.array_equal(bits(out), first_bits)      # the same bits however the range is cut
     assert np.array_equal(host(mix_c), host(solo_c))
     assert ta.spin_fail_flag() == 0
 
 
-RODINIA_PAIRS = [("hot3d", "nn"), ("hot3d", "path"), ("nn", "path")]
+RODINIA_PAIRS = [("hot3d", "nn"), ("hot3d", "path"), ("nn", "path"), ("hot3d", "lava"), ("lava", "nn"), ("lava", "path")]
 
 
 @pytest.mark.parametrize("first,second", RODINIA_PAIRS)
@@ -247,7 +330,7 @@ def test_pairs_among_the_three(first, second, variant):
 
 def test_create_mix_kernel_knows_the_reference_pairs():
     # src/Creator.cu:554-640
-    for name in ("hot3d_nn", "hot3d_path", "nn_path"):
+    for name in ("hot3d_nn", "hot3d_path", "nn_path", "hot3d_lava", "lava_nn", "lava_path"):
         assert ta.lib().tacker_get_kernel_info(name.encode(), b"blocksize") == 256
     for name in ("cp_nn", "hot3d_lbm", "path_stencil"):
         assert ta.lib().tacker_get_kernel_info(name.encode(), b"blocksize") == -32767
@@ -321,9 +404,46 @@ def test_creator_path_is_the_references_grid():
     assert ta.spin_fail_flag() == 0
 
 
+def test_creator_lava_is_the_references_system():
+    k = ta.create_kernel("lava")
+    info = k.info()
+    boxes = 60 ** 3
+    assert (info["ptb_start"], info["ptb_end"], info["ori_grid_x"]) == (0, boxes * 27, boxes)
+    # a slice of the launch: the first 2048 boxes against themselves and their first neighbour
+    n = 2048
+    lib = ta.lib()
+    fv_ptr, rv_ptr, qv_ptr = k.param(5), k.param(3), k.param(4)
+    assert lib.tkMemset(fv_ptr, 0, 16 * 100 * n) == 0
+    k.set_range(0, n)
+    k.execute()
+    k.set_range(boxes, boxes + n)
+    k.execute()
+    torch.cuda.synchronize()
+    k.set_range(0, boxes * 27)
+    rv = ta.device_to_host(rv_ptr, (100 * 60 * 60 * 2, 4), np.float32)          # the first two layers of boxes
+    qv = ta.device_to_host(qv_ptr, (100 * 60 * 60 * 2,), np.float32)
+    assert np.array_equal(rv.reshape(-1), _fill_uniform(np.arange(rv.size), 4301, 0.1, 1.0))
+    assert np.array_equal(qv, _fill_uniform(np.arange(qv.size), 4302, 0.1, 1.0))
+    got = ta.device_to_host(fv_ptr, (100 * n, 4), np.float32)
+    box_list = np.zeros(boxes, oracle.LAVA_BOX)
+    assert lib.tacker_lava_boxes(60, box_list.ctypes.data, box_list.nbytes) == 0
+    r, q = rv.astype(np.float64), qv.astype(np.float64)
+    for b in (0, 59, 60, 1000, n - 1):
+        A = r[100 * b:100 * b + 100]
+        pot = np.zeros(100)
+        for other in (b, int(box_list[b]["nei"][0]["number"])):
+            B = r[100 * other:100 * other + 100]
+            pot += np.exp(-0.5 * (A[:, None, 0] + B[None, :, 0] - A[:, 1:] @ B[:, 1:].T)) @ q[100 * other:100 * other + 100]
+        np.testing.assert_allclose(got[100 * b:100 * b + 100, 0], pot, rtol=2e-5)
+    assert ta.spin_fail_flag() == 0
+
+
 def test_bad_arguments_are_refused():
     lib = ta.lib()
     loc, out = dev(nn_inputs(10)), torch.zeros(10, device="cuda:0")
+    rv = torch.zeros((100, 4), device="cuda:0")
+    assert lib.tacker_ori_lava(0.5, 1, rv.data_ptr(), rv.data_ptr(), rv.data_ptr(), None) == 1       # in place
+    assert lib.tacker_ori_lava(0.5, 0, rv.data_ptr(), rv.data_ptr(), out.data_ptr(), None) != 0
     assert lib.tacker_ori_nn(None, out.data_ptr(), 10, 1.0, 1.0, None) == 1
     assert lib.tacker_ori_nn(loc.data_ptr(), out.data_ptr(), 0, 1.0, 1.0, None) == 1
     t = torch.zeros((2, 4, 64), device="cuda:0")

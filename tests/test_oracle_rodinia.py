@@ -199,3 +199,93 @@ def test_path_source_is_rand_mod_ten():
     assert np.array_equal(grid, oracle.path_source(3, 1200))
     counts = np.bincount(grid.reshape(-1), minlength=10)
     assert counts.min() > 280 and counts.max() < 440
+
+
+# ----------------------------------------------------------------------------- lava
+def _lava_inputs(boxes1d, seed=21, equal_charges=False):
+    rng = np.random.default_rng(seed)
+    n = 100 * boxes1d ** 3
+    rv = (rng.integers(1, 11, (n, 4)) / 10.0).astype(np.float32)       # 0.1 .. 1.0 as the reference draws them
+    qv = np.full(n, 0.5, np.float32) if equal_charges else (rng.integers(1, 11, n) / 10.0).astype(np.float32)
+    return rv, qv
+
+
+def _lava_float64(alpha, boxes1d, rv, qv):
+    """The same sums in float64, box pairs found from coordinates (not from the oracle's list)."""
+    r, q = rv.astype(np.float64), qv.astype(np.float64)
+    a2 = 2.0 * alpha * alpha
+    out = np.zeros_like(r)
+    coords = [(x, y, z) for z in range(boxes1d) for y in range(boxes1d) for x in range(boxes1d)]
+    for a, (ax, ay, az) in enumerate(coords):
+        A = r[100 * a:100 * a + 100]
+        for b, (bx, by, bz) in enumerate(coords):
+            if max(abs(ax - bx), abs(ay - by), abs(az - bz)) > 1:
+                continue
+            B, qB = r[100 * b:100 * b + 100], q[100 * b:100 * b + 100]
+            r2 = A[:, None, 0] + B[None, :, 0] - A[:, 1:] @ B[:, 1:].T
+            vij = np.exp(-a2 * r2)
+            out[100 * a:100 * a + 100, 0] += vij @ qB
+            for c in (1, 2, 3):
+                out[100 * a:100 * a + 100, c] += (2 * vij * (A[:, None, c] - B[None, :, c])) @ qB
+    return out
+
+
+def test_lava_box_list():
+    boxes = oracle.lava_boxes(4)
+    assert len(boxes) == 64
+    counts = np.bincount(boxes["nn"], minlength=27)
+    assert (counts[7], counts[11], counts[17], counts[26]) == (8, 24, 24, 8) and counts.sum() == 64
+    for b in boxes:
+        assert b["number"] == b["x"] + 4 * b["y"] + 16 * b["z"] and b["offset"] == 100 * b["number"]
+        nei = b["nei"][:b["nn"]]
+        assert len(set(nei["number"].tolist())) == b["nn"] and b["number"] not in nei["number"]
+        for ne in nei:
+            assert max(abs(ne["x"] - b["x"]), abs(ne["y"] - b["y"]), abs(ne["z"] - b["z"])) == 1
+            assert ne["number"] == ne["x"] + 4 * ne["y"] + 16 * ne["z"] and ne["offset"] == 100 * ne["number"]
+            assert b["number"] in boxes[ne["number"]]["nei"][:boxes[ne["number"]]["nn"]]["number"]     # symmetric
+    assert oracle.lava_boxes(1)["nn"].tolist() == [0]
+
+
+def test_lava_against_float64_and_closed_forms():
+    rv, qv = _lava_inputs(2)
+    got = oracle.lava(0.5, 2, rv, qv)
+    want = _lava_float64(0.5, 2, rv, qv)
+    assert np.all(np.abs(got - want) <= 2e-3 + 2e-5 * np.abs(want))          # 800 float32 additions per sum of ~250
+    # one box, particle 0 against the box: the potential term by hand
+    rv1, qv1 = _lava_inputs(1, seed=5)
+    one = oracle.lava(0.5, 1, rv1, qv1)
+    r = rv1.astype(np.float64)
+    r2 = r[0, 0] + r[:, 0] - r[:, 1:] @ r[0, 1:]
+    assert one[0, 0] == pytest.approx(float(np.sum(qv1 * np.exp(-0.5 * r2))), rel=1e-5)
+    # alpha enters as a2 = 2 alpha^2
+    other = oracle.lava(1.0, 1, rv1, qv1)
+    assert other[0, 0] == pytest.approx(float(np.sum(qv1 * np.exp(-2.0 * r2))), rel=1e-5)
+    # equal charges: every pair's forces cancel, so all forces sum to zero (the potentials do not)
+    rv, qv = _lava_inputs(3, seed=8, equal_charges=True)
+    f = oracle.lava(0.5, 3, rv, qv).astype(np.float64)
+    assert np.all(np.abs(f[:, 1:].sum(axis=0)) <= 1e-4 * np.abs(f[:, 1:]).sum(axis=0))
+    assert f[:, 0].min() > 0
+
+
+def test_lava_positions():
+    rv, qv = _lava_inputs(2, seed=13)
+    whole = oracle.lava(0.5, 2, rv, qv)
+    n = oracle.lava_blocks(2)
+    assert n == 8 * 27
+    # any ascending tiling adds the same terms in the same order
+    f = np.zeros_like(rv)
+    for a, b in ((0, 5), (5, 8), (8, 100), (100, n)):
+        f = oracle.lava(0.5, 2, rv, qv, fv=f, start=a, end=b)
+    assert np.array_equal(f.view(np.uint32), whole.view(np.uint32))
+    # row 0 is every box against itself; a 2^3 system has 7 neighbours a box: rows 8 .. 26 add nothing
+    self_only = oracle.lava(0.5, 2, rv, qv, start=0, end=8)
+    assert np.all(self_only[:, 0] > 0) and np.all(self_only[:, 0] < whole[:, 0])
+    assert np.array_equal(oracle.lava(0.5, 2, rv, qv, start=8 * 8, end=n), np.zeros_like(rv))
+    # one position touches its box only, and starts from what the array holds
+    base = np.full_like(rv, 3.0)
+    one = oracle.lava(0.5, 2, rv, qv, fv=base, start=8 + 3, end=8 + 4)             # box 3, its first neighbour
+    assert np.array_equal(np.delete(one, np.s_[300:400], axis=0), np.delete(base, np.s_[300:400], axis=0))
+    assert np.all(one[300:400, 0] > 3.0)
+    # positions past the grid wrap
+    again = oracle.lava(0.5, 2, rv, qv, fv=base, start=n + 8 + 3, end=n + 8 + 4)
+    assert np.array_equal(again, one)
