@@ -16,8 +16,8 @@ Method per (pair, K): GEMM 2048 x 2048 x K (1024 tiles, one 128x128 macro tile p
 t0 = fused launch with no best-effort block, t_be = the best-effort kernel alone (all N
 blocks).  For nb on a ladder of block counts, earned(nb) = t0 + t_be * nb / N - t_fused(nb)
 is the time one fused launch saves over the two serial launches (the quantity TaskManager
-credits, src/TaskManager.cu:626-640); the ladder runs N/1024, N/512, ..., N/64, then N/32, 2N/32, ..., N
-and stops once a launch is twice as long as allowed.  The ratio is nb / 1024 for the nb with the largest
+credits, src/TaskManager.cu:626-640); the ladder runs N/1024, N/512, ..., N/64 (from N/65536 for grids of
+a million positions and more), then N/32, 2N/32, ..., N and stops once a launch is twice as long as allowed.  The ratio is nb / 1024 for the nb with the largest
 earned time among those whose launch stays within (1 + stretch) * t0, i.e. the
 latency-critical GEMM is never stretched by more than that factor; 0 if nothing earns.
 """
@@ -38,8 +38,10 @@ LADDER = 32          # best-effort block counts tried: N/1024, N/512, ..., N/64,
 
 def ladder(be_total):
     """ascending block counts: a geometric run-up for kernels whose 1/32 is already longer than a GEMM
-    (sgemm: 2 ms for 528384 positions), then the linear ladder"""
-    counts = {be_total >> j for j in range(6, 11)} | {be_total * step // LADDER for step in range(1, LADDER + 1)}
+    (sgemm: 2 ms for 528384 positions; from 1/65536 for grids of a million positions and more -- lavaMD:
+    43 ms for 5832000), then the linear ladder"""
+    deepest = 17 if be_total >= 1 << 20 else 11
+    counts = {be_total >> j for j in range(6, deepest)} | {be_total * step // LADDER for step in range(1, LADDER + 1)}
     return sorted(c for c in counts if c > 0)
 
 
