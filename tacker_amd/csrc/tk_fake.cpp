@@ -85,11 +85,51 @@ const char *tkGetErrorString(int code)
 }
 int tkGetCuCount(int *cu_count) { *cu_count = g_cu_count; return TK_SUCCESS; }
 int tkGetDeviceName(char *buf, size_t len) { snprintf(buf, len, "fake device"); return TK_SUCCESS; }
-int tkMalloc(void **ptr, size_t bytes) { *ptr = calloc(1, bytes ? bytes : 1); return *ptr ? TK_SUCCESS : TK_ERROR_DEVICE; }
-int tkFree(void *ptr) { free(ptr); return TK_SUCCESS; }
-int tkMemcpy(void *dst, const void *src, size_t bytes, int) { memmove(dst, src, bytes); return TK_SUCCESS; }
-int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int, tkStream_t) { memmove(dst, src, bytes); return TK_SUCCESS; }
-int tkMemset(void *ptr, int value, size_t bytes) { memset(ptr, value, bytes); return TK_SUCCESS; }
+// Allocations come zeroed from calloc without their pages being touched; clearing one that nothing
+// has written yet would only touch them (the default instances of the large kernels clear gigabytes).
+namespace {
+std::map<char *, size_t> g_untouched;   // base -> bytes of allocations still as calloc left them
+void touched(void *dst)
+{
+    auto it = g_untouched.upper_bound(static_cast<char *>(dst));
+    if (it == g_untouched.begin()) return;
+    --it;
+    if (static_cast<char *>(dst) < it->first + it->second) g_untouched.erase(it);
+}
+}  // namespace
+int tkMalloc(void **ptr, size_t bytes)
+{
+    *ptr = calloc(1, bytes ? bytes : 1);
+    if (!*ptr) return TK_ERROR_DEVICE;
+    g_untouched[static_cast<char *>(*ptr)] = bytes ? bytes : 1;
+    return TK_SUCCESS;
+}
+int tkFree(void *ptr)
+{
+    g_untouched.erase(static_cast<char *>(ptr));
+    free(ptr);
+    return TK_SUCCESS;
+}
+int tkMemcpy(void *dst, const void *src, size_t bytes, int)
+{
+    touched(dst);
+    memmove(dst, src, bytes);
+    return TK_SUCCESS;
+}
+int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int, tkStream_t)
+{
+    touched(dst);
+    memmove(dst, src, bytes);
+    return TK_SUCCESS;
+}
+int tkMemset(void *ptr, int value, size_t bytes)
+{
+    auto it = g_untouched.find(static_cast<char *>(ptr));
+    if (value == 0 && it != g_untouched.end() && bytes <= it->second) return TK_SUCCESS;   // still all zero
+    touched(ptr);
+    memset(ptr, value, bytes);
+    return TK_SUCCESS;
+}
 int tkMemcpyToSymbol(const char *symbol, const void *src, size_t bytes, size_t offset)
 {
     if (strcmp(symbol, "ck") && strcmp(symbol, "c_mrif") && strcmp(symbol, "atominfo") && strcmp(symbol, "tk_spin_fail") &&

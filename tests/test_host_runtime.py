@@ -602,6 +602,28 @@ def test_task_manager_fuses_when_budget_allows(fake, small_vgg):
     assert rep["mix_times"] > 0 and rep["be_blocks_executed"] > 0
 
 
+def test_task_manager_with_the_rodinia_kernels_and_their_pairs(fake, small_vgg):
+    # nn rides with the layers, and the second stage fuses nn with pathfinder (src/Creator.cu:629-640: nn_path);
+    # a Rodinia kernel has no fused kernel with a Parboil one, which is refused where the reference exits
+    fake.tk_fake_set_event_ms(0.01)
+    tm = ta.TaskManager(small_vgg, "nn", "path", library=fake)
+    tm.configure(warmup=1, profile=2, verbose=0, qos_budget_ms=50.0, guard_ms=4.0, queries=1)
+    fake.tk_fake_reset()
+    rep = tm.run("aker", raw_stream=None, second_stage=True)
+    keys = [l["key"] for l in launches(fake)]
+    assert "nn_path" in keys and any(k.startswith("tzgemm_nn") for k in keys)
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_nn")]
+    assert all(len(l["args"]) == 5 + 9 + 6 + 9 for l in fused)            # nn's 5, its trailer, tzgemm's 6, its trailer
+    assert rep["mix_times"] > 0 and rep["be_blocks_executed"] > 0
+    tm.close()
+    for be1, be2 in (("nn", "lbm"), ("stencil", "path"), ("lava", "cp")):
+        with pytest.raises(ta.TackerError, match="no fused kernel"):
+            ta.TaskManager(small_vgg, be1, be2, library=fake)
+    for name in ("nn", "hot3d", "path", "lava"):
+        tm = ta.TaskManager(small_vgg, name, None, library=fake)
+        tm.close()
+
+
 def test_task_manager_second_stage_credits_the_fused_best_effort_pair(fake, small_vgg):
     # every timed region takes 10 us and holds 10 launches, of one best-effort kernel or of the fused pair:
     # the pair (1 us a launch) beats the two solo launches (1 + 1 us), so the budget left is worth twice as
