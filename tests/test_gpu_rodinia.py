@@ -438,6 +438,33 @@ def test_creator_lava_is_the_references_system():
     assert ta.spin_fail_flag() == 0
 
 
+def test_task_manager_colocates_the_rodinia_kernels():
+    # nn and hotspot3D blocks ride with VGG16's layers (tzgemm_nn, tzgemm_hot3d), the nn_path pair
+    # (src/mix_kernel/nn_path.cu) runs in the second stage; the query's logits stay the solo query's bits
+    task = ta.LcTask("vgg16", 64, 64)
+    task.execute()
+    torch.cuda.synchronize()
+    p, stride, n = task.logits()
+    solo_logits = ta.device_to_host(p, (n, stride), np.float32)[:, 0].copy()
+    tm = ta.TaskManager(task, "nn", "path")
+    tm.configure(qos_budget_ms=50.0, guard_ms=0.5, warmup=1, profile=3, queries=3, verbose=0)
+    rep = tm.run("aker", second_stage=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
+    assert rep["mixable_times"] == 16 and rep["be1_solo_ms"] > 0 and rep["n_colocated"] == 3
+    tm.close()
+    tm = ta.TaskManager(task, "hot3d", None)
+    tm.configure(qos_budget_ms=50.0, guard_ms=0.5, warmup=1, profile=3, queries=3, verbose=0)
+    rep = tm.run("aker", second_stage=False)
+    torch.cuda.synchronize()
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo_logits)
+    assert rep["n_colocated"] == 3 and ta.spin_fail_flag() == 0
+    tm.close()
+    with pytest.raises(ta.TackerError, match="no fused kernel"):
+        ta.TaskManager(task, "nn", "stencil")
+    task.close()
+
+
 def test_bad_arguments_are_refused():
     lib = ta.lib()
     loc, out = dev(nn_inputs(10)), torch.zeros(10, device="cuda:0")
