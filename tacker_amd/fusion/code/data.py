@@ -72,8 +72,10 @@ KERNEL_INFO = {
     # wavefronts in flight keep more of them in open memory pages (4.9 TB/s with 2 workgroups a CU, 3.9 with 8)
     "hot3d": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 2,
               "ori_blks": 524288},
-    # 216000 boxes of 100 particles (a wavefront each) x 27 parts (the home box and its neighbour slots)
-    "lava": {"register": 84, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 4,
+    # 216000 boxes of 100 particles (a wavefront each) x 27 parts (the home box and its neighbour slots);
+    # boxes on the faces have fewer neighbours: the more owner wavefronts, the evener their shares
+    # (42.4 ms with 4 workgroups a CU, 35.8 with 32)
+    "lava": {"register": 84, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 32,
              "ori_blks": 5832000},
     # 200 windows of 256 columns (6 result columns each), a wavefront each
     "path": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 1,
