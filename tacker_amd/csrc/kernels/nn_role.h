@@ -20,6 +20,11 @@
 #include "role_common.h"
 #include "../header/nn_header.h"
 
+// steps of loads a lane issues before its first store
+#ifndef NN_STEPS_IN_FLIGHT
+#define NN_STEPS_IN_FLIGHT 4
+#endif
+
 namespace tk {
 
 __device__ __forceinline__ float nn_distance(float2 r, float lat, float lng)
@@ -36,7 +41,7 @@ __device__ __forceinline__ void nn_positions(const float *__restrict__ records, 
                                              int grid_dimension_y, int width, int role_block, int role_blocks,
                                              int start, int end, int tid, int role_threads)
 {
-    constexpr int DEPTH = 4;
+    constexpr int DEPTH = NN_STEPS_IN_FLIGHT;
     typedef float vec_in __attribute__((ext_vector_type(2 * PER)));
     // lanes a position takes, positions served at once and this thread's place among them
     const int lanes = (width + PER - 1) / PER;
