@@ -1,5 +1,5 @@
-"""Committed golden vectors (tests/golden/kernels_small.npz): the oracle must keep
-reproducing them (CPU), and the HIP path must match them (GPU)."""
+"""Committed golden vectors (tests/golden/kernels_small.npz, kernels_partners.npz): the oracle must
+keep reproducing them (CPU), and the HIP path must match them (GPU)."""
 import os
 
 import numpy as np
@@ -8,6 +8,7 @@ import pytest
 import oracle
 
 G = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kernels_small.npz"))
+P = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "kernels_partners.npz"))
 C0, C1 = np.float32(1 / 6), np.float32(1 / 36)
 
 
@@ -79,3 +80,51 @@ def test_hip_path_matches_golden_vectors():
     ta.gptb_mrif(96, x, y, z, outR, outI)
     for got, want in ((host(outR), G["mrif_outR"]), (host(outI), G["mrif_outI"])):
         assert np.all(np.abs(got.astype(np.float64) - want) <= 1e-3 + 1e-4 * np.abs(want))
+
+
+def test_oracle_reproduces_the_partners_golden_vectors():
+    assert np.array_equal(oracle.sgemm(P["sgemm_A"], P["sgemm_B"], P["sgemm_C0"]), P["sgemm_C"])
+    assert np.array_equal(oracle.fft(P["fft_in"]), P["fft_out"])
+    prep = oracle.cutcp_prepare(P["cutcp_atoms"], (0, 0, 0), 16, 16, 8, 0.5, 12.0)
+    assert np.array_equal(oracle.cutcp(prep, 0.5, 144.0, 0.006944, (2, 2, 1)), P["cutcp_energies"])
+    assert np.array_equal(oracle.nn(P["nn_locations"], 30.0, 90.0), P["nn_distances"])
+    t1 = oracle.hot3d(P["hot3d_power"], P["hot3d_t0"])
+    assert np.array_equal(t1, P["hot3d_t1"]) and np.array_equal(oracle.hot3d(P["hot3d_power"], t1), P["hot3d_t2"])
+    assert np.array_equal(oracle.path(40, P["path_wall"], P["path_src"]), P["path_result"])
+    assert np.array_equal(oracle.lava(0.5, 2, P["lava_rv"], P["lava_qv"]), P["lava_fv"])
+
+
+@pytest.mark.gpu
+def test_hip_path_matches_the_partners_golden_vectors():
+    import torch
+    import tacker_amd as ta
+    from gpu_util import dev, host, setup
+    setup()
+
+    def close(got, want, atol, rtol):
+        return bool(np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= atol + rtol * np.abs(want)))
+
+    c = dev(P["sgemm_C0"])
+    ta.gptb_sgemm(dev(P["sgemm_A"]), dev(P["sgemm_B"]), c)
+    assert np.array_equal(host(c).view(np.uint32), P["sgemm_C"].view(np.uint32))
+    d = dev(P["fft_in"])
+    ta.gptb_fft(d)
+    assert close(host(d), P["fft_out"], 1e-4, 1e-5)
+    inp = ta.CutcpInput(P["cutcp_atoms"], (0, 0, 0), 16, 16, 8, 0.5, 12.0)
+    ta.gptb_cutcp(inp, 144.0, 0.006944)
+    assert close(host(inp.energies), P["cutcp_energies"], 2e-4, 2e-5)
+    dist = torch.zeros(700, device="cuda:0")
+    ta.gptb_nn(dev(P["nn_locations"]), dist, 30.0, 90.0)
+    assert np.array_equal(host(dist).view(np.uint32), P["nn_distances"].view(np.uint32))
+    t1, t2 = torch.zeros((4, 8, 64), device="cuda:0"), torch.zeros((4, 8, 64), device="cuda:0")
+    ta.gptb_hot3d(dev(P["hot3d_power"]), dev(P["hot3d_t0"]), t1)
+    ta.gptb_hot3d(dev(P["hot3d_power"]), t1, t2)
+    assert np.array_equal(host(t1).view(np.uint32), P["hot3d_t1"].view(np.uint32))
+    assert np.array_equal(host(t2).view(np.uint32), P["hot3d_t2"].view(np.uint32))
+    res = torch.zeros(300, dtype=torch.int32, device="cuda:0")
+    ta.gptb_path(40, dev(P["path_wall"]), dev(P["path_src"]), res)
+    assert np.array_equal(host(res), P["path_result"])
+    fv = torch.zeros((800, 4), device="cuda:0")
+    ta.gptb_lava(0.5, dev(P["lava_rv"]), dev(P["lava_qv"]), fv)
+    assert close(host(fv), P["lava_fv"], 2e-3, 2e-5)
+    assert ta.spin_fail_flag() == 0
