@@ -35,8 +35,8 @@ def launches(l):
         l.tk_fake_launch_dims(i, dims)
         args = []
         for a in range(l.tk_fake_launch_nargs(i)):
-            buf = C.create_string_buffer(8)
-            n = l.tk_fake_launch_arg(i, a, buf, 8)
+            buf = C.create_string_buffer(64)       # lavaMD passes a 56-byte struct by value
+            n = l.tk_fake_launch_arg(i, a, buf, 64)
             args.append(buf.raw[:n])
         out.append({"key": l.tk_fake_launch_key(i).decode(), "grid": tuple(dims[:3]), "block": tuple(dims[3:]),
                     "args": args, "by_driver": bool(l.tk_fake_launch_by_driver(i))})
@@ -267,6 +267,45 @@ def test_other_mix_vectors_have_reference_lengths(fake, be, n_be):
     # lbm_tzgemm_mix 11+15, mriq_tzgemm_mix and mrif_tzgemm_mix 16+15, cp_tzgemm_mix 12+15
     # (src/mix_kernel/tzgemm_{lbm,mriq,mrif,cp}.cu dispatcher signatures)
     assert l["key"] == f"tzgemm_{be}" and len(l["args"]) == n_be + 9 + 15
+
+
+@pytest.mark.parametrize("be,n_be", [("nn", 5), ("hot3d", 14), ("path", 8), ("lava", 6)])
+def test_rodinia_mix_and_gptb_vectors_have_reference_lengths(fake, be, n_be):
+    fake.tk_fake_reset()
+    buf = np.zeros(1 << 16, np.float32)
+    out = np.zeros(1 << 16, np.float32)
+    A = np.zeros((128, 128), np.float16)
+    Cm = np.zeros((128, 128), np.float32)
+    g = [A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 128, 128, 128, 0, 4, None, 0, 0, None]
+    p, q = buf.ctypes.data, out.ctypes.data
+    if be == "nn":
+        mix = fake.tacker_mix_tzgemm_nn(p, q, 1000, 30.0, 90.0, 0, 4, *g)
+        gptb = fake.tacker_gptb_nn(p, q, 1000, 30.0, 90.0, 0, 4, 0, 0, None)
+        dims = [4, 1, 1, 256, 1, 1]                      # 4 blocks of 256 records
+    elif be == "hot3d":
+        mix = fake.tacker_mix_tzgemm_hot3d(p, p, q, 128, 8, 4, 0, 4, *g)
+        gptb = fake.tacker_gptb_hot3d(p, p, q, 128, 8, 4, 0, 4, 0, 0, None)
+        dims = [2, 2, 1, 64, 4, 1]                       # 2 x 2 patches of 64 x 4 columns
+    elif be == "path":
+        mix = fake.tacker_mix_tzgemm_path(20, p, p, q, 500, 30, 0, 0, 3, *g)
+        gptb = fake.tacker_gptb_path(20, p, p, q, 500, 30, 0, 0, 3, 0, 0, None)
+        dims = [3, 1, 1, 64, 1, 1]                       # ceil(500 / 216) windows, a wavefront each
+    else:
+        mix = fake.tacker_mix_tzgemm_lava(0.5, 2, p, p, q, 0, 216, *g)
+        gptb = fake.tacker_gptb_lava(0.5, 2, p, p, q, 0, 216, 0, 0, None)
+        dims = [8, 1, 27, 64, 1, 1]                      # 8 boxes x 27 parts, a wavefront a box
+    assert mix == 0 and gptb == 0, fake.tacker_last_error()
+    l_mix, l_gptb = launches(fake)
+    # src/mix_kernel/tzgemm_{nn,hot3d,path,lava}.cu: the kernel's own parameters, its 9 GPTB ints, tzgemm's 15;
+    # src/gptb_kernel/{nn,hot3d,path,lava}_kernel.cu: the parameters and the 10-int trailer
+    assert l_mix["key"] == f"tzgemm_{be}" and len(l_mix["args"]) == n_be + 9 + 15
+    assert l_gptb["key"] == f"gptb_{be}" and len(l_gptb["args"]) == n_be + 10
+    assert [as_int(x) for x in l_gptb["args"][n_be:n_be + 6]] == dims
+    assert [as_int(x) for x in l_mix["args"][n_be:n_be + 6]] == dims
+    if be == "lava":
+        assert len(l_gptb["args"][0]) == 4 and len(l_gptb["args"][1]) == 56      # par_str and dim_str by value
+        assert struct.unpack("<f", l_gptb["args"][0])[0] == 0.5
+        assert struct.unpack("<4i5q", l_gptb["args"][1])[3:5] == (2, 8)          # boxes1d_arg, number_boxes
 
 
 def test_gptb_vector_is_restored_after_launch_and_after_failure(fake):
