@@ -227,3 +227,12 @@ def test_measured_load_ratios_travel_from_profile_ratio_to_the_schedulers_lookup
     # a K of the table, the base entry, linear extrapolation from 4096 beyond the table, and the block count
     # Aker mode gives a 1024-tile GEMM of K = 2304: tiles x ratio
     assert [float(v) for v in got[:3]] == [2.25, 5.25, 10.5] and int(got[3]) == int(1024 * 4.25)
+
+
+def test_profile_tools_import_without_a_gpu_and_know_every_kernel():
+    import profile_gptb
+    import profile_ratio
+    assert set(profile_ratio.PAIRS) == set(gen_run.BE_KERNELS)
+    assert profile_gptb.LADDER[-1] == 1.0 and list(profile_gptb.LADDER) == sorted(profile_gptb.LADDER)
+    # grids of a million positions and more get a finer run-up (lavaMD: 5832000 positions, 43 ms)
+    assert profile_ratio.ladder(5832000)[0] == 5832000 >> 16 and profile_ratio.ladder(528384)[0] == 528384 >> 10
