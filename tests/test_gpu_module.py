@@ -148,3 +148,40 @@ def test_cutcp_and_fft_from_the_code_object():
     k.execute()
     assert np.array_equal(bits(a), bits(b))
     assert ta.spin_fail_flag() == 0
+
+
+def test_the_rodinia_kernels_from_the_code_object():
+    # cuModuleGetFunction + cuLaunchKernel (src/ModuleCenter.cu) with structs passed by value (lavaMD's par_str,
+    # dim_str): the driver-style launch from the code object gives the registry launch's bits
+    rng = np.random.default_rng(62)
+    loc = dev(rng.uniform(0, 90, (3000, 2)).astype(np.float32))
+    want, got = torch.zeros(3000, device="cuda:0"), torch.full((3000,), -1.0, device="cuda:0")
+    ta.gptb_nn(loc, want, 30.0, 90.0)
+    k = ta.gptb_create(ta.ori_nn_create(loc, got, 30.0, 90.0), 0, 0, 0, ta.nn_blocks(3000))
+    k.use_module("kernels", "general_ptb_nn")
+    k.execute()
+    assert np.array_equal(bits(got), bits(want))
+    p, t = dev(rng.uniform(0, 0.01, (4, 8, 128)).astype(np.float32)), dev(rng.uniform(320, 340, (4, 8, 128)).astype(np.float32))
+    want, got = torch.zeros((4, 8, 128), device="cuda:0"), torch.full((4, 8, 128), -1.0, device="cuda:0")
+    ta.gptb_hot3d(p, t, want)
+    k = ta.gptb_create(ta.ori_hot3d_create(p, t, got), 0, 0, 0, ta.hot3d_blocks(128, 8))
+    k.use_module("kernels", "general_ptb_hot3d")
+    k.execute()
+    assert np.array_equal(bits(got), bits(want))
+    wall, src = dev(rng.integers(0, 10, (50, 900), dtype=np.int32)), dev(rng.integers(0, 10, 900, dtype=np.int32))
+    want = torch.zeros(900, dtype=torch.int32, device="cuda:0")
+    got = torch.full((900,), -1, dtype=torch.int32, device="cuda:0")
+    ta.gptb_path(50, wall, src, want)
+    k = ta.gptb_create(ta.ori_path_create(50, wall, src, got), 0, 0, 0, ta.path_blocks(900, 50))
+    k.use_module("kernels", "general_ptb_path")
+    k.execute()
+    assert np.array_equal(host(got), host(want))
+    rv = dev((rng.integers(1, 11, (800, 4)) / 10.0).astype(np.float32))
+    qv = dev((rng.integers(1, 11, 800) / 10.0).astype(np.float32))
+    want, got = torch.zeros((800, 4), device="cuda:0"), torch.zeros((800, 4), device="cuda:0")
+    ta.gptb_lava(0.5, rv, qv, want)
+    k = ta.gptb_create(ta.ori_lava_create(0.5, rv, qv, got), 0, 0, 0, ta.lava_blocks(2))
+    k.use_module("kernels", "general_ptb_lava")
+    k.execute()
+    assert np.array_equal(bits(got), bits(want))
+    assert ta.spin_fail_flag() == 0
