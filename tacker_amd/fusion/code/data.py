@@ -47,7 +47,8 @@ KERNEL_INFO = {
     # 1024 blocks of 64 x 4 columns x 8 runs of 8 centre planes
     "stencil": {"register": 48, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
                 "ori_blks": 8192},
-    "lbm": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
+    # 67.4 us with 16 workgroups a CU, 69.9 with 8 (profile_gptb.py)
+    "lbm": {"register": 64, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 16,
             "ori_blks": 18000},
     # 1024 blocks of 256 voxels x 16 chunks of 128 k records
     "mriq": {"register": 40, "shared_memory": 0, "blocksize": 256, "solo_ptb_blks": 8,
