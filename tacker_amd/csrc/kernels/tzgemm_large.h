@@ -21,7 +21,7 @@
 // for 256 x 256, and the ring is two buffers.  They are filled by LDS-direct loads
 // (global_load_lds_dwordx4: lane l's 16 bytes land at base + 16 l, so one load fills 8 rows),
 // each of which takes whole 128-byte lines from 8 matrix rows: the same loads taking 64 bytes
-// from 16 rows each move 55 GB/s into a CU, these 86 (microbench/feed_rate.hip).
+// from 16 rows each move 55 GB/s into a CU, these 86 (a stand-alone load-shape measurement).
 // An iteration multiplies one chunk, whose fragments the wave already holds in registers, and
 // meanwhile reads the fragments of the next chunk.  In the first iteration of a pair those come
 // from the same buffer, which was published an iteration ago: no wait, no barrier.  In the second
@@ -47,25 +47,10 @@
 #pragma once
 #include "tzgemm_role.h"
 
-// Measurement builds only (microbench/tzgemm_large_probe.hip): each macro takes one ingredient out
-// of the kernel (the loads or the barrier of the steady K loop, the C stores) -- the results are
-// wrong, the time says what the ingredient costs.
-#ifdef TZL_KNOCK_OUT_LOADS
-#define TZL_LOOP_LOAD(...)
-#else
 #define TZL_LOOP_LOAD(...) tz_load_to_lds(__VA_ARGS__)
-#endif
-#ifdef TZL_KNOCK_OUT_BARRIER
-#define TZL_LOOP_BARRIER()
-#else
 #define TZL_LOOP_BARRIER() __builtin_amdgcn_s_barrier()
-#endif
 #define TZL_LOOP_READ(dst_, src_) dst_ = src_
-#ifdef TZL_KNOCK_OUT_STORES
-#define TZL_STORE_IF(v_) if ((v_)[0] == 123.456f)   // never true for the probe's operands
-#else
 #define TZL_STORE_IF(v_)
-#endif
 
 namespace tk {
 

@@ -177,13 +177,7 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
                               (((q_) & 1) ? OPERAND_BYTES : 0);                                   \
         tz_load_to_lds((((q_) & 1) ? b_tile : a_tile) + uni_, (j_ & 1) ? src_odd : src_even, dst_); \
     }
-// loads issued from inside the steady K loop; a measurement build (microbench/fused_probe.hip)
-// takes them out to see what they cost (results wrong on purpose)
-#ifdef TZ_KNOCK_OUT_LOADS
-#define TZ_LOOP_ISSUE_ONE(chunk_, stage_, q_) {}
-#else
 #define TZ_LOOP_ISSUE_ONE(chunk_, stage_, q_) TZ_ISSUE_ONE(chunk_, stage_, q_)
-#endif
 #define TZ_ISSUE_CHUNK(chunk_, stage_)                                                            \
     _Pragma("unroll") for (int q = 0; q < LOADS_PER_CHUNK; ++q) TZ_ISSUE_ONE(chunk_, stage_, q)
 #define TZ_READ_FRAGS(fa_, fb_, stage_, seg_)                                                     \
@@ -193,13 +187,9 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         fa_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_a);                                 \
         fb_[i] = *reinterpret_cast<const half8_t *>(s_ + frag_b);                                 \
     }
-#ifdef TZ_KNOCK_OUT_MFMA   // measurement build: no MFMAs but the 4 of a split barrier's asm block
-#define TZ_MFMAS_ROWS(fa_, fb_, i0_, i1_)
-#else
 #define TZ_MFMAS_ROWS(fa_, fb_, i0_, i1_)                                                         \
     _Pragma("unroll") for (int i = i0_; i < i1_; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j) \
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[j], fa_[i], acc[i][j], 0, 0, 0);
-#endif
 #define TZ_MFMAS(fa_, fb_) TZ_MFMAS_ROWS(fa_, fb_, 0, 4)
 // Issue order inside one scheduling region: after each MFMA one LDS read (count_ of them),
 // then after each MFMA one LDS-direct load (count2_).  An MFMA occupies the matrix pipe for
@@ -212,13 +202,9 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
         __builtin_amdgcn_sched_group_barrier(mask_, 1, 0);                                        \
     }
 #define TZ_SCHED_DS_READ 0x100
-#ifdef TZ_KNOCK_OUT_MFMA
-#define TZ_MFMA_AT(fa_, fb_, n_)
-#else
 #define TZ_MFMA_AT(fa_, fb_, n_)                                                                  \
     acc[(n_) >> 2][(n_) & 3] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb_[(n_) & 3], fa_[(n_) >> 2], \
                                                                       acc[(n_) >> 2][(n_) & 3], 0, 0, 0);
-#endif
 // First k-step of a chunk multiplied while the chunk barrier completes; the reads of the
 // second k-step (into fn_, fbn_) ride in the shadow of the first 8 MFMAs, and loads 4..7 of
 // chunk tail_chunk_ (the half of a chunk the previous second k-step did not issue) follow one
