@@ -271,12 +271,21 @@ def pair_leg(ta, torch, np, name, stream):
     out["be_blocks"] = nblk
     if slice_blocks > 0:
         out["slice_speedup"] = round(out["slice_serial_us"] / out["slice_fused_us"], 4)
-    if out["be_us"] > 1.3 * out["gemm_us"]:
-        # the longer best-effort kernel spread over the GEMMs it rides with: n = T_be / T_gemm fused launches,
-        # each carrying the next 1/n of the block positions, against n GEMM launches plus the kernel alone
-        n_cur = max(1, int(round(out["be_us"] / out["gemm_us"])))
-        bounds = [nblk * i // n_cur for i in range(n_cur + 1)]
+    # what TaskManager credits a co-located slice with: the GEMM alone plus the slice at the whole kernel's
+    # rate (src/TaskManager.cu:626-640) -- the slice launched alone runs below that rate, which flatters
+    # slice_speedup
+    if slice_blocks > 0:
+        out["slice_serial_at_kernel_rate_us"] = round(out["gemm_us"] + out["be_us"] * slice_blocks / nblk, 2)
+        out["slice_speedup_at_kernel_rate"] = round(out["slice_serial_at_kernel_rate_us"] / out["slice_fused_us"], 4)
+    if out["be_us"] > 1.3 * out["gemm_us"] and slice_blocks > 0:
+        # The longer best-effort kernel spread over the GEMMs it rides with, the way the scheduler does it in
+        # Aker mode: consecutive fused launches, each carrying the next slice_blocks block positions (a cursor),
+        # against as many GEMM launches plus the best-effort kernel alone over the same positions.  At most 64
+        # launches are timed (the first 64 slices of kernels that need more).
+        n_cur = min(64, (nblk + slice_blocks - 1) // slice_blocks)
+        bounds = [min(nblk, slice_blocks * i) for i in range(n_cur + 1)]
         mix_cur = ta.mix_create(be, tz, 0, 0, 0, tiles)
+        be_part = be if bounds[-1] == nblk else ta.gptb_create(be_ori, 0, 0, 0, bounds[-1])
 
         def cursor_fused():
             for i in range(n_cur):
@@ -286,7 +295,7 @@ def pair_leg(ta, torch, np, name, stream):
         def cursor_serial():
             for _ in range(n_cur):
                 tz.execute(stream)
-            be.execute(stream)
+            be_part.execute(stream)
 
         n = 40 if n_cur <= 30 else 10
         cur = {"cursor_serial_us": [], "cursor_fused_us": []}
@@ -295,7 +304,20 @@ def pair_leg(ta, torch, np, name, stream):
             cur["cursor_fused_us"].append(timed(cursor_fused))
         out.update({key: round(statistics.median(v), 2) for key, v in cur.items()})
         out["cursor_launches"] = n_cur
+        out["cursor_blocks"] = bounds[-1]
         out["cursor_speedup"] = round(out["cursor_serial_us"] / out["cursor_fused_us"], 4)
+    # the scheduler's decisions for this pair (kinfo): Aker mode co-locates slice_blocks positions with a GEMM
+    # of this K (0 = never fuses it at this K); Tacker mode lets the whole kernel ride only if kinfo's measured
+    # whole-kernel gain says that it pays, and falls back to the Aker slice otherwise
+    whole = ta.lib().tacker_qos_whole_kernel_gain(name.encode())
+    out["scheduler"] = {"aker_slice_blocks": slice_blocks, "aker_fuses": bool(slice_blocks > 0),
+                        "kinfo_whole_kernel_gain": round(whole, 4), "tacker_fuses_whole_kernel": bool(whole >= 1.0)}
+    picked = []
+    if slice_blocks > 0:
+        picked.append(out.get("cursor_speedup", out["slice_speedup_at_kernel_rate"]))
+    if whole >= 1.0:
+        picked.append(out["speedup"])
+    out["scheduler"]["slowest_form_it_would_pick"] = round(min(picked), 4) if picked else None
     out["gemm_tflops_alone"] = round(flop / out["gemm_us"] / 1e6, 1)
     if work["bound"] == "hbm":
         out["be_gbps_alone"] = round(work["algorithmic_bytes"] / out["be_us"] / 1e3, 1)
@@ -351,6 +373,7 @@ def lc_leg(ta, torch, np, queries, be_name="stencil", be_label="stencil 512x512x
     tm = ta.TaskManager(task, be_name, be2_name)   # the second kernel only names the stage-2 pair (same family)
     tm.configure(qos_budget_ms=50.0, guard_ms=4.0, warmup=5, profile=min(500, queries), queries=queries, verbose=0)
     tm.set_calibration(True, 0.10)
+    tm.set_calibration_variants(("default", "wave_256"))   # per layer: the pair's default form or the 512-thread one
     tm.set_end_to_end(min(500, queries))
     rep = tm.run("aker", second_stage=True)
     torch.cuda.synchronize()
@@ -372,7 +395,9 @@ def lc_leg(ta, torch, np, queries, be_name="stencil", be_label="stencil 512x512x
            "be_blocks_per_query": rep["be_blocks_executed"], "time_earned_ms_per_query": round(rep["time_earned_ms"], 4),
            "be_work_ms_per_query": round(rep["be_blocks_executed"] * rep["be1_solo_ms"] / be_total, 4),
            "be_kernel_passes_completed": rep["be_task_finish_num"],
-           "lc_kernels_barred_from_fusion_at_end": tm.fusion_disabled()}
+           "lc_kernels_barred_from_fusion_at_end": tm.fusion_disabled(),
+           "layers_calibrated_to_the_512_thread_form": sum(1 for v, n in zip(tm.calibrated_variants(), tm.calibrated_blocks())
+                                                           if n > 0 and v == "wave_256")}
     out["p99_within_bound"] = bool(out["colocated_p99_ms"] <= out["qos_bound_ms"])
     # whole queries, one event pair (and the host clock) around all launches of a query, no
     # synchronisation between kernels; the figures above are sums of per-kernel intervals.  graph_*: the
@@ -485,39 +510,11 @@ def main():
     fused_launch_s = ms["fused"] / ITERATIONS * 1e-3
     speedup = ms["serial"] / ms["fused"]
     info = mix.info()
-    out = {
-        "metric": "fused-pair speedup vs serial (tzgemm 2048^3 + stencil 512x512x64, 100 iterations)",
-        "value": round(speedup, 4), "unit": "x", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms["fused"], 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16 in / f32 accumulate (tzgemm), f32 (stencil)",
-        "data": "synthetic (numpy default_rng(1337): A,B uniform[-1,1] -> f16; grid uniform[0,1])",
-        "config": {"workload": "configs[1]: fused tzgemm fp16 2048x2048x2048 + 7-point stencil fp32 "
-                               "512x512x64, c0=1/6, c1=1/36, 100 iterations",
-                   "fused_kernel": "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)"),
-                   "fused_grid": info["grid"], "fused_block": info["block"], "device": ta.device_name()},
-        "serial_ms_per_step": round(ms["serial"], 4),
-        "gemm_alone_ms_per_100": round(ms["gemm"], 4), "stencil_alone_ms_per_100": round(ms["stencil"], 4),
-        "overlap_efficiency": round(max(ms["gemm"], ms["stencil"]) / ms["fused"], 4),
-        "roofline": {"bound": "hbm", "achieved": round(fused_bytes / fused_launch_s / 1e9, 1),
-                     "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-                     "frac": round(fused_bytes / fused_launch_s / HBM_PEAK, 4),
-                     "traffic": FUSED_HBM_TRAFFIC_BYTES,
-                     "kernel": "stencil_tzgemm_mix (one fused launch: 1 GEMM + 1 sweep)",
-                     "algorithmic_bytes_per_launch": fused_bytes,
-                     "avg_launch_us": round(fused_launch_s * 1e6, 2)},
-        "roofline_mfma": {"bound": "mfma", "achieved": round(gemm_flop / fused_launch_s / 1e12, 1),
-                          "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s",
-                          "frac": round(gemm_flop / fused_launch_s / MFMA_F16_PEAK, 4),
-                          "flop_per_launch": gemm_flop},
-        "alone": {
-            "tzgemm": {"avg_launch_us": round(ms["gemm"] * 10, 2),
-                       "tflops": round(gemm_flop / (ms["gemm"] / ITERATIONS * 1e-3) / 1e12, 1),
-                       "frac_of_mfma_peak": round(gemm_flop / (ms["gemm"] / ITERATIONS * 1e-3) / MFMA_F16_PEAK, 4)},
-            "stencil": {"avg_launch_us": round(ms["stencil"] * 10, 2),
-                        "gbps": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / 1e9, 1),
-                        "frac_of_hbm_peak": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / HBM_PEAK, 4)}},
-        "wall_s_timed_region": round(t_wall, 3),
-    }
+    import statistics
+    per_step = [a / b for a, b in zip(samples["serial"], samples["fused"])]   # serial and fused jobs alternate inside a step
+    # Details first, headline last: a reader who keeps only the end of the line still has the metric,
+    # the roofline and the summaries of every pair.
+    out = {}
     if not args.no_extras:
         if args.pairs == ap.get_default("pairs"):
             out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
@@ -527,8 +524,71 @@ def main():
             out["lc_colocation_mriq"] = lc_leg(ta, torch, np, args.queries, "mriq", "mri-q numK 2048, numX 262144")
             out["lc_colocation_fft"] = lc_leg(ta, torch, np, args.queries, "fft", "fft 10240 x 256 points")
             out["lc_colocation_nn"] = lc_leg(ta, torch, np, args.queries, "nn", "nn 655360000 records", "path")
+    out["alone"] = {
+        "tzgemm": {"avg_launch_us": round(ms["gemm"] * 10, 2),
+                   "tflops": round(gemm_flop / (ms["gemm"] / ITERATIONS * 1e-3) / 1e12, 1),
+                   "frac_of_mfma_peak": round(gemm_flop / (ms["gemm"] / ITERATIONS * 1e-3) / MFMA_F16_PEAK, 4)},
+        "stencil": {"avg_launch_us": round(ms["stencil"] * 10, 2),
+                    "gbps": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / 1e9, 1),
+                    "frac_of_hbm_peak": round(stencil_bytes / (ms["stencil"] / ITERATIONS * 1e-3) / HBM_PEAK, 4)}}
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(A, B, A0, c0, c1)
+    if "tzgemm_shapes" in out:
+        # shape -> [tzgemm us, fraction of the MFMA peak, torch.matmul us]
+        out["tzgemm_shapes_summary"] = {k: [v["us"], v["frac_of_mfma_peak"], v["torch_matmul_us"]]
+                                        for k, v in out["tzgemm_shapes"].items()}
+    if "other_pairs" in out:
+        # pair -> [whole kernel fused, slice at the kernel's rate, cursor (the scheduler's slices), GEMM us, best-effort us,
+        #          serial us, fused us, slowest form the scheduler would pick]; speedups are serial / fused
+        out["pairs_summary"] = {k: [v["speedup"], v.get("slice_speedup_at_kernel_rate"), v.get("cursor_speedup"),
+                                    v["gemm_us"], v["be_us"], v["serial_us"], v["fused_us"],
+                                    v["scheduler"]["slowest_form_it_would_pick"]]
+                                for k, v in out["other_pairs"].items()}
+        out["pairs_summary"]["stencil"] = [round(speedup, 4), None, None, round(ms["gemm"] * 10, 2),
+                                           round(ms["stencil"] * 10, 2), round(ms["serial"] * 10, 2),
+                                           round(ms["fused"] * 10, 2), round(speedup, 4)]
+        losing = [k for k, v in out["pairs_summary"].items() if v[7] is not None and v[7] < 1.0]
+        out["pairs_the_scheduler_would_fuse_at_a_loss"] = losing
+    for key in ("lc_colocation", "lc_colocation_mriq", "lc_colocation_fft", "lc_colocation_nn"):
+        if key in out:
+            e = out[key]["end_to_end"]
+            # [solo p50, solo p99, co-located p50, co-located p99, bound, within bound, ms earned per query,
+            #  best-effort ms carried per query, fused layers]
+            out[key + "_summary"] = [e.get("solo_p50_ms"), e.get("solo_p99_ms"), e.get("colocated_p50_ms"),
+                                     e.get("colocated_p99_ms"), e.get("qos_bound_ms"), e.get("p99_within_bound"),
+                                     out[key]["time_earned_ms_per_query"], out[key]["be_work_ms_per_query"],
+                                     out[key]["mixed_launches_per_query"]]
+    out.update({
+        "wall_s_timed_region": round(t_wall, 3),
+        "overlap_efficiency": round(max(ms["gemm"], ms["stencil"]) / ms["fused"], 4),
+        "gemm_alone_ms_per_100": round(ms["gemm"], 4), "stencil_alone_ms_per_100": round(ms["stencil"], 4),
+        "roofline_mfma": {"bound": "mfma", "achieved": round(gemm_flop / fused_launch_s / 1e12, 1),
+                          "peak": MFMA_F16_PEAK / 1e12, "unit": "TFLOP/s",
+                          "frac": round(gemm_flop / fused_launch_s / MFMA_F16_PEAK, 4),
+                          "flop_per_launch": gemm_flop},
+        "roofline": {"bound": "hbm", "achieved": round(fused_bytes / fused_launch_s / 1e9, 1),
+                     "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                     "frac": round(fused_bytes / fused_launch_s / HBM_PEAK, 4),
+                     "traffic": FUSED_HBM_TRAFFIC_BYTES,
+                     "kernel": "stencil_tzgemm_mix (one fused launch: 1 GEMM + 1 sweep)",
+                     "algorithmic_bytes_per_launch": fused_bytes,
+                     "avg_launch_us": round(fused_launch_s * 1e6, 2)},
+        "config": {"workload": "configs[1]: fused tzgemm fp16 2048x2048x2048 + 7-point stencil fp32 "
+                               "512x512x64, c0=1/6, c1=1/36, 100 iterations",
+                   "fused_kernel": "tzgemm_stencil" + ("@" + args.variant if args.variant else " (kinfo default)"),
+                   "fused_grid": info["grid"], "fused_block": info["block"], "device": ta.device_name()},
+        "data": "synthetic (numpy default_rng(1337): A,B uniform[-1,1] -> f16; grid uniform[0,1])",
+        "dtype": "f16 in / f32 accumulate (tzgemm), f32 (stencil)",
+        "metric": "fused-pair speedup vs serial (tzgemm 2048^3 + stencil 512x512x64, 100 iterations)",
+        "unit": "x", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        # value = trimmed mean of the serial job / trimmed mean of the fused job; per step: the ratio of the
+        # two jobs of that step (they run back to back)
+        "value_per_step": {"min": round(min(per_step), 4), "median": round(statistics.median(per_step), 4),
+                           "max": round(max(per_step), 4)},
+        "serial_ms_per_step": round(ms["serial"], 4), "ms_per_step": round(ms["fused"], 4),
+        "value": round(speedup, 4),
+    })
     print(json.dumps(out))
     return 0
 

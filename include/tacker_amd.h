@@ -64,6 +64,10 @@ TK_API int tkGetDeviceName(char *buf, size_t len);
 
 TK_API int tkMalloc(void **ptr, size_t bytes);                           /* cudaMalloc */
 TK_API int tkFree(void *ptr);                                            /* cudaFree */
+/* How often tkMalloc and tkFree have been called in this process (either pointer may be null).
+ * No counterpart in the reference: a caller that must not allocate (stream capture, a serving
+ * loop) reads it before and after a call to see that the library kept to that. */
+TK_API int tkAllocationCalls(long long *mallocs, long long *frees);
 TK_API int tkMemcpy(void *dst, const void *src, size_t bytes, int kind); /* cudaMemcpy */
 TK_API int tkMemcpyAsync(void *dst, const void *src, size_t bytes, int kind, tkStream_t s);
 TK_API int tkMemset(void *ptr, int value, size_t bytes);                 /* cudaMemset */
@@ -141,10 +145,16 @@ TK_API int tacker_tzgemm_grid_dim(int m, int n, int k, int out[4]);
  * tacker_tzgemm_parts: the number of parts for (m, n, k) rounded as tacker_tzgemm_grid_dim
  * rounds them -- a function of the shape only, so fused and unfused launches add in the same
  * order. tacker_tzgemm_workspace_bytes: size of that workspace, 0 when parts == 1.
+ * A kernel object built on C is a user of C's binding until it is destroyed; a binding without
+ * users stays for the next object on the same C and is taken out (after a device synchronisation,
+ * least recently used first) when a new binding needs its place: at most 512 bindings, at most
+ * 1 GiB held by bindings without users.
+ * tacker_tzgemm_workspace_stats: bindings in the table, those with a user, bytes they hold.
  * tacker_tzgemm_release_workspaces: synchronises the device and frees them all; only when no
- * kernel object built on caller-owned operands is left. */
+ * kernel object that uses one is left. */
 TK_API int tacker_tzgemm_parts(int m, int n, int k);
 TK_API long long tacker_tzgemm_workspace_bytes(int m, int n, int k);
+TK_API int tacker_tzgemm_workspace_stats(int *bindings, int *in_use, long long *bytes);
 TK_API int tacker_tzgemm_release_workspaces(void);
 
 /* general_ptb_tzgemm through GPTBKernel (src/gptb_kernel/tzgemm_kernel.cu:430-449,
@@ -667,6 +677,14 @@ TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int 
  * tacker_task_manager_calibrated_blocks copies the counts of the last run (one per LC kernel). */
 TK_API int tacker_task_manager_set_calibration(tacker_task_manager_t tm, int on, float max_stretch);
 TK_API int tacker_task_manager_calibrated_blocks(tacker_task_manager_t tm, int *out, int cap);
+/* The calibration pass can also choose, per LC kernel, among generated forms of the fused kernel:
+ * `variants` is a comma-separated list of variant names ("default" = the form kinfo names for the
+ * pair, e.g. "default,wave_256"); forms the pair was not generated in are skipped.  A short layer
+ * can earn more in a form with fewer best-effort waves per workgroup (a 512-thread workgroup is
+ * cheaper to launch than a 768-thread one).  tacker_task_manager_calibrated_variant copies the form
+ * kept for LC kernel `kernel` in the last run ("" = default) and returns its length, -1 on error. */
+TK_API int tacker_task_manager_set_calibration_variants(tacker_task_manager_t tm, const char *variants);
+TK_API int tacker_task_manager_calibrated_variant(tacker_task_manager_t tm, int kernel, char *out, int cap);
 /* LC kernels barred from fusion at the end of the last run */
 TK_API int tacker_task_manager_fusion_disabled(tacker_task_manager_t tm);
 /* "[Mix] BE task1 + task2 took ..." (src/TaskManager.cu:693): average time of the fused launch of
@@ -687,6 +705,11 @@ TK_API int tacker_task_manager_latencies(tacker_task_manager_t tm, int which, fl
 
 /* the scheduler's arithmetic on its own (src/TaskManager.cu:586-640) */
 TK_API float tacker_qos_block_ratio(const char *be_name, int K_GLOBAL);
+/* No counterpart in the reference (its Tacker mode always fuses the whole best-effort kernel,
+ * src/TaskManager.cu:599): kinfo's measured gain (serial time / fused time) of a fused launch that
+ * carries the whole best-effort kernel, 1 when kinfo holds none. Below 1 the scheduler carries the
+ * Aker-mode slice in Tacker mode too. */
+TK_API float tacker_qos_whole_kernel_gain(const char *be_name);
 /* mode: 0 = Aker, 1 = Tacker (enum ExecutionMode) */
 TK_API int tacker_qos_colocated_blocks(int mode, const char *be_name, int tiles, int K_GLOBAL,
                                        int be_total_blocks);

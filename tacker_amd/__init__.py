@@ -160,6 +160,7 @@ def _declare(lib):
     lib.tacker_task_input.argtypes = [vp, C.POINTER(vp), C.POINTER(i)]
     lib.tacker_task_stage_input.argtypes = [vp]
     lib.tacker_task_capture.argtypes = [vp, vp, C.POINTER(vp)]
+    lib.tkAllocationCalls.argtypes = [C.POINTER(C.c_longlong), C.POINTER(C.c_longlong)]
     lib.tkStreamCreate.argtypes = [C.POINTER(vp)]
     lib.tkStreamDestroy.argtypes = [vp]
     lib.tkStreamSynchronize.argtypes = [vp]
@@ -179,10 +180,14 @@ def _declare(lib):
     lib.tacker_task_manager_set_calibration.argtypes = [vp, i, f]
     lib.tacker_task_manager_set_end_to_end.argtypes = [vp, i]
     lib.tacker_task_manager_calibrated_blocks.argtypes = [vp, vp, i]
+    lib.tacker_task_manager_set_calibration_variants.argtypes = [vp, cp]
+    lib.tacker_task_manager_calibrated_variant.argtypes = [vp, i, cp, i]
     lib.tacker_task_manager_be_mix_ms.argtypes = [vp]
     lib.tacker_task_manager_be_mix_ms.restype = f
     lib.tacker_qos_block_ratio.argtypes = [cp, i]
     lib.tacker_qos_block_ratio.restype = f
+    lib.tacker_qos_whole_kernel_gain.argtypes = [cp]
+    lib.tacker_qos_whole_kernel_gain.restype = f
     lib.tacker_qos_colocated_blocks.argtypes = [i, cp, i, i, i]
     lib.tacker_qos_must_run_solo.argtypes = [f, f, f, f]
     lib.tacker_qos_account.argtypes = [i, f, f, f, i, i, C.POINTER(f)]
@@ -798,6 +803,13 @@ def mnk_from_conv_args(args14):
     return list(out)
 
 
+def allocation_calls(library=None):
+    """(tkMalloc calls, tkFree calls) of the library since it was loaded"""
+    m, f = C.c_longlong(), C.c_longlong()
+    check((library or lib()).tkAllocationCalls(C.byref(m), C.byref(f)), "tkAllocationCalls")
+    return m.value, f.value
+
+
 def spin_fail_flag():
     v = C.c_int()
     check(lib().tacker_spin_fail_flag(C.byref(v)), "tacker_spin_fail_flag")
@@ -1139,10 +1151,25 @@ class TaskManager:
     def set_calibration(self, on=True, max_stretch=0.10):
         check(self.l.tacker_task_manager_set_calibration(self.h, 1 if on else 0, max_stretch), "set_calibration")
 
+    def set_calibration_variants(self, variants=("default", "wave_256")):
+        """forms of the fused kernel the calibration pass tries per LC kernel ("default" = kinfo's)"""
+        check(self.l.tacker_task_manager_set_calibration_variants(self.h, ",".join(variants).encode()),
+              "set_calibration_variants")
+
     def calibrated_blocks(self):
         buf = (C.c_int * 4096)()
         n = self.l.tacker_task_manager_calibrated_blocks(self.h, buf, 4096)
         return list(buf[:max(n, 0)])
+
+    def calibrated_variants(self):
+        """the form kept per LC kernel by the last calibrated run ("" = the pair's default)"""
+        out = []
+        buf = C.create_string_buffer(64)
+        for k in range(len(self.calibrated_blocks())):
+            if self.l.tacker_task_manager_calibrated_variant(self.h, k, buf, 64) < 0:
+                break
+            out.append(buf.value.decode())
+        return out
 
     def fusion_disabled(self):
         return self.l.tacker_task_manager_fusion_disabled(self.h)

@@ -100,10 +100,17 @@ float QosPolicy::blockRatio(const std::string &be_name, int K_GLOBAL)
     return block_ratio;
 }
 
+float QosPolicy::wholeKernelGain(const std::string &be_name)
+{
+    const float gain = fget_kernel_info("tzgemm_" + be_name, "whole_kernel_gain");
+    return gain == JSON_NOT_FOUND ? 1.0f : gain;
+}
+
 int QosPolicy::coLocatedBlocks(ExecutionMode mode, const std::string &be_name, int tiles, int K_GLOBAL,
                                int be_total_blocks)
 {
-    if (mode == ExecutionMode::Tacker) return be_total_blocks;   // the whole BE kernel rides along
+    // the whole BE kernel rides along, unless it is known to lose that way
+    if (mode == ExecutionMode::Tacker && wholeKernelGain(be_name) >= 1.0f) return be_total_blocks;
     return std::min(int(tiles * blockRatio(be_name, K_GLOBAL)), be_total_blocks);
 }
 
@@ -222,59 +229,70 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     }
 
     // launch of LC kernel idx fused with BE blocks [from, to) of be_kernel1
-    auto launch_mixed = [&](Kernel *lc_kernel, int from, int to) {
+    auto launch_mixed = [&](Kernel *lc_kernel, int from, int to, const std::string &variant = std::string()) {
         std::vector<int> args = lc_kernel->getArgs();
         std::vector<int> mnk = lc_kernel->mixable == 1 ? args : get_mnk_from_cudnn_args(args);
         if (auto *layer = dynamic_cast<LcGemmKernel *>(lc_kernel))
-            layer->executeMixed(be_kernel1, from, to, stream);   // the layer's own operands
+            layer->executeMixed(be_kernel1, from, to, stream, variant);   // the layer's own operands
         else if (lc_kernel->mixable == 1) mixcublasSgemm(mnk, be_kernel1, from, to, stream);
         else mixcudnnConvolutionForward(args, be_kernel1, from, to, stream);
     };
 
     // optional: measured block count per LC kernel instead of the kinfo table
     calibrated_blocks.clear();
+    calibrated_variant.clear();
     if (calibrate_blocks && mode == ExecutionMode::Aker && be_total > 0) {
         calibrated_blocks.assign(nk, 0);
+        calibrated_variant.assign(nk, "");
         std::vector<float> best_earned(nk, 0.0f);
-        std::vector<bool> over(nk, false);   // a smaller count already stretched this kernel too far
         const int first = be_kernel1->gptbParams.ptb_start_block_pos;
-        for (int divisor = 256; divisor >= 1; divisor /= 2) {
-            const int n = std::max(1, be_total / divisor);
-            std::vector<float> fused_ms(nk, 0.0f);
-            const int timed = 3;
-            for (int pass = -1; pass < timed; ++pass) {   // pass -1 warms up
-                lc_task->initExecution();
+        std::vector<std::string> forms;
+        for (const std::string &v : calibrate_variants)
+            if (v.empty() || get_kernel_info("tzgemm_" + be_task1_name + "@" + v, "blocksize") != JSON_NOT_FOUND)
+                forms.push_back(v);
+        if (forms.empty()) forms.push_back("");
+        for (const std::string &form : forms) {
+            std::vector<bool> over(nk, false);   // a smaller count already stretched this kernel too far
+            for (int divisor = 256; divisor >= 1; divisor /= 2) {
+                const int n = std::max(1, be_total / divisor);
+                std::vector<float> fused_ms(nk, 0.0f);
+                const int timed = 3;
+                for (int pass = -1; pass < timed; ++pass) {   // pass -1 warms up
+                    lc_task->initExecution();
+                    for (size_t idx = 0; idx < nk; ++idx) {
+                        Kernel *lc_kernel = lc_task->kernels[idx];
+                        if (lc_kernel->mixable == 0 || over[idx]) {
+                            lc_kernel->execute(stream);
+                            continue;
+                        }
+                        watch.start(stream);
+                        launch_mixed(lc_kernel, first, std::min(first + n, be_total), form);
+                        const float ms = watch.stop(stream);
+                        if (pass >= 0) fused_ms[idx] += ms / timed;
+                    }
+                }
                 for (size_t idx = 0; idx < nk; ++idx) {
-                    Kernel *lc_kernel = lc_task->kernels[idx];
-                    if (lc_kernel->mixable == 0 || over[idx]) {
-                        lc_kernel->execute(stream);
+                    if (lc_task->kernels[idx]->mixable == 0 || over[idx]) continue;
+                    const float alone = lc_kernel_time_vec[idx];
+                    if (fused_ms[idx] > (1.0f + calibrate_max_stretch) * alone) {
+                        over[idx] = true;
                         continue;
                     }
-                    watch.start(stream);
-                    launch_mixed(lc_kernel, first, std::min(first + n, be_total));
-                    const float ms = watch.stop(stream);
-                    if (pass >= 0) fused_ms[idx] += ms / timed;
-                }
-            }
-            for (size_t idx = 0; idx < nk; ++idx) {
-                if (lc_task->kernels[idx]->mixable == 0 || over[idx]) continue;
-                const float alone = lc_kernel_time_vec[idx];
-                if (fused_ms[idx] > (1.0f + calibrate_max_stretch) * alone) {
-                    over[idx] = true;
-                    continue;
-                }
-                const float earned = alone + report.be1_solo_ms * n / be_total - fused_ms[idx];
-                if (earned > best_earned[idx]) {
-                    best_earned[idx] = earned;
-                    calibrated_blocks[idx] = n;
+                    const float earned = alone + report.be1_solo_ms * n / be_total - fused_ms[idx];
+                    if (earned > best_earned[idx]) {
+                        best_earned[idx] = earned;
+                        calibrated_blocks[idx] = n;
+                        calibrated_variant[idx] = form;
+                    }
                 }
             }
         }
         if (verbose)
             for (size_t idx = 0; idx < nk; ++idx)
                 if (lc_task->kernels[idx]->mixable != 0)
-                    printf("[CAL] %s: %d blocks, earns %f ms\n", lc_task->kernels[idx]->kernelName.c_str(),
-                           calibrated_blocks[idx], best_earned[idx]);
+                    printf("[CAL] %s: %d blocks%s%s, earns %f ms\n", lc_task->kernels[idx]->kernelName.c_str(),
+                           calibrated_blocks[idx], calibrated_variant[idx].empty() ? "" : " in form ",
+                           calibrated_variant[idx].c_str(), best_earned[idx]);
     }
 
     // co-located queries: a cursor walks the BE kernel's blocks across launches
@@ -318,7 +336,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
                 }
                 const int end = std::min(be_cursor + cd_block_num, be_total);
                 cd_block_num = end - be_cursor;
-                launch_mixed(lc_kernel, be_cursor, end);
+                launch_mixed(lc_kernel, be_cursor, end, calibrated ? calibrated_variant[idx] : std::string());
                 be_cursor = end;
                 if (be_cursor >= be_total) {   // one pass over the BE kernel done
                     be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;
@@ -359,7 +377,8 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
                     continue;
                 }
                 const int end = std::min(be_cursor + carried[idx], be_total);
-                launch_mixed(lc_kernel, be_cursor, end);
+                launch_mixed(lc_kernel, be_cursor, end,
+                             calibrated_variant.empty() ? std::string() : calibrated_variant[idx]);
                 be_cursor = end >= be_total ? be_kernel1->gptbParams.ptb_start_block_pos : end;
             }
             const float ms = watch.stop(stream);   // waits for the query's last kernel

@@ -35,7 +35,13 @@ struct QosPolicy {
     // BE blocks per 64x64 GEMM tile for a GEMM of depth K_GLOBAL: kinfo entry
     // "tzgemm_<be>"[K]; when absent, the K=4096 entry scaled linearly by K (:593-598).
     static float blockRatio(const std::string &be_name, int K_GLOBAL);
-    // how many BE blocks ride along with a GEMM of `tiles` tiles (:599-600)
+    // kinfo entry "tzgemm_<be>"["whole_kernel_gain"]: serial time / fused time measured with the
+    // whole best-effort kernel in one fused launch; 1 when kinfo has none (the reference always
+    // fuses, and credits a launch only if it beat the solo launches, :696-700)
+    static float wholeKernelGain(const std::string &be_name);
+    // how many BE blocks ride along with a GEMM of `tiles` tiles (:599-600).  Tacker mode lets the
+    // whole kernel ride unless kinfo says that this loses against the two launches
+    // (wholeKernelGain < 1); it then carries the slice Aker mode would.
     static int coLocatedBlocks(ExecutionMode mode, const std::string &be_name, int tiles, int K_GLOBAL,
                                int be_total_blocks);
     // solo if the remaining budget cannot cover the rest of the query plus the guard (:586)
@@ -108,6 +114,12 @@ public:
     bool calibrate_blocks = false;
     float calibrate_max_stretch = 0.10f;
     std::vector<int> calibrated_blocks;   // per LC kernel, filled by the last calibrated run
+    // Forms of the fused kernel the calibration pass tries for every LC kernel ("" = the one kinfo
+    // names for the pair); it keeps, per LC kernel, the form and count that earned most.  A short
+    // layer can do better in a form with fewer best-effort waves per workgroup: the launch of a
+    // 512-thread workgroup costs less than that of a 768-thread one.
+    std::vector<std::string> calibrate_variants{""};
+    std::vector<std::string> calibrated_variant;   // per LC kernel, beside calibrated_blocks
     // Not in the reference (its latency of a query is the sum of per-kernel intervals, each
     // followed by a synchronisation, src/TaskManager.cu:620-624): after the co-located queries,
     // run this many more queries of each kind -- every kernel alone, and with the best-effort

@@ -227,6 +227,12 @@ int tacker_tzgemm_release_workspaces(void)
     });
 }
 
+int tacker_tzgemm_workspace_stats(int *bindings, int *in_use, long long *bytes)
+{
+    tzgemmWorkspaceStats(bindings, in_use, bytes);
+    return TK_SUCCESS;
+}
+
 int tacker_global_gemm_buffers(const void **A, const void **B, float **C, long long bytes[3])
 {
     if (!A || !B || !C || !bytes) return fail(TK_ERROR_INVALID_VALUE, "null output");
@@ -1563,6 +1569,34 @@ int tacker_task_manager_set_calibration(tacker_task_manager_t h, int on, float m
     return TK_SUCCESS;
 }
 
+int tacker_task_manager_set_calibration_variants(tacker_task_manager_t h, const char *variants)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || !variants) return fail(TK_ERROR_INVALID_VALUE, "bad task manager or list");
+    std::vector<std::string> forms;
+    std::string item;
+    for (const char *c = variants;; ++c) {
+        if (*c == ',' || *c == 0) {
+            forms.push_back(item == "default" ? std::string() : item);
+            item.clear();
+            if (*c == 0) break;
+        } else {
+            item.push_back(*c);
+        }
+    }
+    tm->calibrate_variants = forms;
+    return TK_SUCCESS;
+}
+
+int tacker_task_manager_calibrated_variant(tacker_task_manager_t h, int kernel, char *out, int cap)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || !out || cap < 1 || kernel < 0 || kernel >= (int)tm->calibrated_variant.size()) return -1;
+    const std::string &v = tm->calibrated_variant[(size_t)kernel];
+    snprintf(out, (size_t)cap, "%s", v.c_str());
+    return (int)v.size();
+}
+
 int tacker_task_manager_set_end_to_end(tacker_task_manager_t h, int queries)
 {
     TaskManager *tm = static_cast<TaskManager *>(h);
@@ -1608,6 +1642,7 @@ int tacker_task_manager_latencies(tacker_task_manager_t h, int which, float *out
 }
 
 float tacker_qos_block_ratio(const char *be_name, int K_GLOBAL) { return QosPolicy::blockRatio(be_name, K_GLOBAL); }
+float tacker_qos_whole_kernel_gain(const char *be_name) { return QosPolicy::wholeKernelGain(be_name ? be_name : ""); }
 
 int tacker_qos_colocated_blocks(int mode, const char *be_name, int tiles, int K_GLOBAL, int be_total_blocks)
 {

@@ -82,14 +82,15 @@ protected:
     }
 
 public:
-    void executeMixed(GPTBKernel *be, int be_start, int be_end, cudaStream_t stream) override
+    void executeMixed(GPTBKernel *be, int be_start, int be_end, cudaStream_t stream,
+                      const std::string &variant = "") override
     {
         before(stream);
         if (be_end <= be_start) {
             gptb_->execute(stream);
             return;
         }
-        std::unique_ptr<MixKernel> mix(createTzgemmMix(be, gptb_.get(), be_start, be_end, 0, tiles_, "", 0, 0));
+        std::unique_ptr<MixKernel> mix(createTzgemmMix(be, gptb_.get(), be_start, be_end, 0, tiles_, variant, 0, 0));
         mix->execute(stream);
     }
 

@@ -25,7 +25,9 @@ class LcGemmKernel : public Kernel {
 public:
     // the layer with blocks [be_start, be_end) of a best-effort kernel fused into
     // its GEMM launch (be_end <= be_start: the GEMM alone)
-    virtual void executeMixed(GPTBKernel *be, int be_start, int be_end, cudaStream_t stream) = 0;
+    // variant: which generated form of the fused kernel ("" = the one kinfo names for the pair)
+    virtual void executeMixed(GPTBKernel *be, int be_start, int be_end, cudaStream_t stream,
+                              const std::string &variant = "") = 0;
     // padded GEMM shape {M, N, K} actually launched
     virtual std::vector<int> gemmDims() const = 0;
     void initParams() override {}

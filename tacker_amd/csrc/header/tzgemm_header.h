@@ -104,9 +104,15 @@ TZ_HOST_DEVICE inline bool tz_use_large(int M, int N, int K)
 #define TZ_WS_TABLE_SLOTS 1024
 #define TZ_WS_TABLE_MAX_PROBES 16
 struct tz_ws_entry {
-    unsigned long long c;           // output buffer (device address), 0 = empty slot
+    unsigned long long c;           // key (below), 0 = empty slot, TZ_WS_TOMBSTONE = a binding that was taken out
     unsigned long long workspace;   // its workspace
 };
+#define TZ_WS_TOMBSTONE 1ull
+// Table keys of an output buffer C.  The two kinds of kernel that bind a workspace to their output
+// (tzgemm's shared reductions, sgemm's k parts) use different keys, so that they never share one:
+// an output buffer is at least 4-byte aligned, so C + 2 is no buffer's address.
+TZ_HOST_DEVICE inline unsigned long long tz_ws_key_tzgemm(const void *C) { return (unsigned long long)(size_t)C; }
+TZ_HOST_DEVICE inline unsigned long long tz_ws_key_sgemm(const void *C) { return (unsigned long long)(size_t)C + 2ull; }
 TZ_HOST_DEVICE inline unsigned tz_ws_hash(unsigned long long c)
 {
     return (unsigned)(((c >> 8) * 0x9E3779B97F4A7C15ull) >> 54) & (TZ_WS_TABLE_SLOTS - 1);

@@ -224,7 +224,7 @@ __device__ __forceinline__ void sgemm_role(const float *__restrict__ A, const fl
     float *W = nullptr;
     if (gy > 1) {
         // partial results rest in the workspace bound to C; without one nothing can be computed
-        W = reinterpret_cast<float *>(tz_find_workspace(C));
+        W = reinterpret_cast<float *>(tz_find_workspace(tz_ws_key_sgemm(C)));
         if (W == nullptr) {
             if (tid == 0 && role_block == 0)
                 __hip_atomic_fetch_or(&tk_spin_fail, TK_FAIL_WORKSPACE, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

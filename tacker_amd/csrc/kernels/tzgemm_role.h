@@ -49,12 +49,12 @@ __device__ tz_ws_entry tz_ws_table[TZ_WS_TABLE_SLOTS];
 
 namespace tk {
 
-// The workspace bound to output buffer C, nullptr if there is none.  C is a kernel argument, so
-// the probes are scalar loads; the host never lets a key sit more than TZ_WS_TABLE_MAX_PROBES
-// slots from its hash.
-__device__ __forceinline__ unsigned *tz_find_workspace(const float *C)
+// The workspace bound to a key of the table (tz_ws_key_*), nullptr if there is none.  The key comes
+// from a kernel argument, so the probes are scalar loads; the host never lets a key sit more than
+// TZ_WS_TABLE_MAX_PROBES slots from its hash, and a binding it takes out leaves a tombstone that
+// the probe walks past.
+__device__ __forceinline__ unsigned *tz_find_workspace(unsigned long long key)
 {
-    const unsigned long long key = (unsigned long long)(size_t)C;
     unsigned slot = tz_ws_hash(key);
     for (int probe = 0; probe < TZ_WS_TABLE_MAX_PROBES; ++probe) {
         const unsigned long long c = tz_ws_table[slot].c;
@@ -67,7 +67,7 @@ __device__ __forceinline__ unsigned *tz_find_workspace(const float *C)
 // ... for a GEMM of this shape: only the shapes whose reduction is shared by workgroups look.
 __device__ __forceinline__ unsigned *tz_workspace_of(const float *C, int M, int N, int K)
 {
-    return tz_ksplit_parts(M, N, K) > 1 ? tz_find_workspace(C) : nullptr;
+    return tz_ksplit_parts(M, N, K) > 1 ? tz_find_workspace(tz_ws_key_tzgemm(C)) : nullptr;
 }
 
 // Persistent-loop index -> macro tile (row, column).  With role_blocks a multiple
@@ -450,7 +450,9 @@ __device__ __forceinline__ int tz_opaque(int v)
 
 // Partial tiles travel between workgroups on other XCDs, whose L2s do not see each other's
 // lines.  Every access to them is an agent-scope access of its own (it goes through to the
-// memory side both XCDs share), so no cache has to be written back or dropped as a whole.
+// memory side both XCDs share), so no cache has to be written back or dropped as a whole; the
+// compiler is held to the order "partial tile, ticket" and "last ticket, reads" by a release and
+// an acquire fence at workgroup scope around them (tzgemm_role_ksplit).
 // A partial tile is 16 blocks of 64 x float4 (block = i * 4 + j of the accumulator set),
 // stored as two 8-byte halves per lane: [block][half][lane].
 typedef unsigned long long tz_u64;
@@ -604,12 +606,18 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
                 for (int i = 0; i < 4; ++i)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) tz_partial_store(my_partial, i * 4 + j, lane_here, acc[i][j]);
-                // the partial tile has arrived where the other XCDs read it before the ticket is drawn
+                // The partial tile before the ticket.  For the hardware: the stores above are agent-scope
+                // accesses (written through to the memory side all XCDs share) and the wave waits until
+                // every one of them has been acknowledged.  For the compiler: a release fence, so that no
+                // store can sink below the ticket.  The fence is at workgroup scope on purpose: at agent
+                // scope it is a write-back of the XCD's whole L2 (buffer_wbl2), 1 to 2 us on a layer of
+                // 11 to 14 us, for stores that have already left the L2.
                 __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));
-                asm volatile("" ::: "memory");
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
                 unsigned ticket = 0;
                 if (lane == 0)
                     ticket = __hip_atomic_fetch_add(workspace + pos, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
                 ticket = __builtin_amdgcn_readfirstlane(ticket);
                 // tell every wave whether this workgroup drew the last ticket: one word at the head of
                 // each wave's own LDS region (wave 0 is done with the partial tiles that were there)
@@ -622,6 +630,13 @@ __device__ __forceinline__ void tzgemm_role_ksplit(const _Float16 *__restrict__ 
             __builtin_amdgcn_readfirstlane(*(const __attribute__((address_space(3))) unsigned *)(lptr_t)mine) != 0u) {
             // last to arrive: add the partial tiles in part order.  Wave w takes rows 16w .. 16w+15 of
             // the tile; loads go out two parts at a time so that a batch is one trip to memory.
+            // The ticket before the reads.  Wave 0 drew the last ticket and told the others through LDS
+            // and the role barrier; every wave reads other workgroups' partial tiles itself.  For the
+            // compiler: an acquire fence, so that no load can rise above the flag.  For the hardware:
+            // the loads are agent-scope accesses of their own, which are served from the memory side,
+            // not from a line this XCD's L2 may hold.  At agent scope the fence is an invalidation of
+            // the whole L2 (buffer_inv), 5 to 6 us a layer.
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
             const tz_u64 *tile_parts = partial_tiles + (size_t)pos * parts * (TZ_PARTIAL_TILE_BYTES / 8);
             const int lane_here = tz_opaque(lane);
             float4_t sum[4];

@@ -26,6 +26,7 @@ OriSGEMMKernel::OriSGEMMKernel(int id, const float *A, const float *B, float *C,
 
 OriSGEMMKernel::~OriSGEMMKernel()
 {
+    if (holdsWorkspace) sgemmWorkspaceDone(SGEMMKernelParams->C);
     for (auto &ptr : cudaFreeList) tkErrCheck(tkFree(ptr));
     delete SGEMMKernelParams;
 }
@@ -65,7 +66,10 @@ void OriSGEMMKernel::bind()
     launchBlockDim = dim3(SGEMM_TILE_N, SGEMM_TILE_TB_HEIGHT / 2, 1);   // one wavefront: a lane owns two of the block's rows
     kernelParams = {&p->A, &p->B, &p->C, &p->NORMAL_M, &p->NORMAL_N, &p->NORMAL_K};
     this->smem = 0;
-    if (parts > 1) sgemmWorkspaceFor(p->C, p->NORMAL_M, p->NORMAL_N);
+    if (parts > 1 && !holdsWorkspace) {
+        sgemmWorkspaceFor(p->C, p->NORMAL_M, p->NORMAL_N);
+        holdsWorkspace = true;
+    }
     auto it = fmap.find("ori_sgemm");
     this->kernelFunc = it == fmap.end() ? nullptr : it->second;
     this->initialized = true;

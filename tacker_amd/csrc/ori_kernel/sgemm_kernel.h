@@ -15,8 +15,10 @@ struct OriSGEMMParamsStruct {
 
 // workspace of M x N floats bound to the output buffer C, where the partial results of a block
 // rest between the k parts of the GPTB form; entered into the device table kernels look C up in
-// (the one the GEMM role's shared reductions use) and kept until tzgemmReleaseWorkspaces()
+// (the one the GEMM role's shared reductions use, under a key of its own).  The caller is a user of
+// the binding until sgemmWorkspaceDone(C); bindings without users go when room is needed.
 void *sgemmWorkspaceFor(const float *C, int M, int N);
+void sgemmWorkspaceDone(const float *C);
 
 class OriSGEMMKernel : public Kernel {
 public:
@@ -38,4 +40,5 @@ private:
     void loadKernel() override {}
     void bind();
     OriSGEMMParamsStruct *SGEMMKernelParams = nullptr;
+    bool holdsWorkspace = false;
 };

@@ -97,8 +97,16 @@ void touched(void *dst)
     if (static_cast<char *>(dst) < it->first + it->second) g_untouched.erase(it);
 }
 }  // namespace
+static long long g_malloc_calls = 0, g_free_calls = 0;
+int tkAllocationCalls(long long *mallocs, long long *frees)
+{
+    if (mallocs) *mallocs = g_malloc_calls;
+    if (frees) *frees = g_free_calls;
+    return TK_SUCCESS;
+}
 int tkMalloc(void **ptr, size_t bytes)
 {
+    ++g_malloc_calls;
     *ptr = calloc(1, bytes ? bytes : 1);
     if (!*ptr) return TK_ERROR_DEVICE;
     g_untouched[static_cast<char *>(*ptr)] = bytes ? bytes : 1;
@@ -106,6 +114,7 @@ int tkMalloc(void **ptr, size_t bytes)
 }
 int tkFree(void *ptr)
 {
+    ++g_free_calls;
     g_untouched.erase(static_cast<char *>(ptr));
     free(ptr);
     return TK_SUCCESS;

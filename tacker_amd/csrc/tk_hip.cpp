@@ -4,6 +4,8 @@
 // tkGetErrorString.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include <cstring>
 #include <mutex>
 #include <string>
@@ -92,8 +94,25 @@ int tkGetDeviceName(char *buf, size_t len)
     return TK_SUCCESS;
 }
 
-int tkMalloc(void **ptr, size_t bytes) { return FOLD(hipMalloc(ptr, bytes)); }
-int tkFree(void *ptr) { return FOLD(hipFree(ptr)); }
+// calls of tkMalloc / tkFree since the library was loaded: what a caller that must not allocate
+// (a captured graph, a serving loop) checks around a call
+static std::atomic<long long> g_malloc_calls{0}, g_free_calls{0};
+int tkMalloc(void **ptr, size_t bytes)
+{
+    ++g_malloc_calls;
+    return FOLD(hipMalloc(ptr, bytes));
+}
+int tkFree(void *ptr)
+{
+    ++g_free_calls;
+    return FOLD(hipFree(ptr));
+}
+int tkAllocationCalls(long long *mallocs, long long *frees)
+{
+    if (mallocs) *mallocs = g_malloc_calls.load();
+    if (frees) *frees = g_free_calls.load();
+    return TK_SUCCESS;
+}
 int tkMemcpy(void *dst, const void *src, size_t bytes, int kind)
 {
     return FOLD(hipMemcpy(dst, src, bytes, kind_of(kind)));

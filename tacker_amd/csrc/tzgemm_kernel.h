@@ -50,13 +50,19 @@ inline std::vector<int> getTZGEMMGridDim(int m, int n, int k)
 void ensureGlobalGemmBuffers(int M_GLOBAL, int N_GLOBAL, int K_GLOBAL);
 
 // Workspace for GEMMs that write the buffer C: nullptr when the shape needs none, else a zeroed
-// device buffer of at least tz_workspace_bytes(M, N, K) that stays bound to C until
-// tzgemmReleaseWorkspaces (or until a larger one replaces it), entered into the device table
-// tz_ws_table where the kernels find it.  Launches that write the same C must not overlap anyway,
-// so they can share it; launches on different C never do.  Thread-safe.
+// device buffer of at least tz_workspace_bytes(M, N, K) bound to C (or a larger one that replaces
+// it), entered into the device table tz_ws_table where the kernels find it.  Launches that write
+// the same C must not overlap anyway, so they can share it; launches on different C never do.
+// The caller becomes a user of the binding until it calls tzgemmWorkspaceDone with the same
+// arguments; a binding without users stays for the next kernel object on the same C and is taken
+// out, least recently used first, when the table or the device memory such bindings may hold
+// (512 bindings, 1 GiB) is needed for a new one.  Thread-safe.
 void *tzgemmWorkspaceFor(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL);
-// Frees every such workspace after a device synchronisation.  Only when no kernel object built on
-// caller-owned operands is left (they keep the pointer they were given).
+void tzgemmWorkspaceDone(const float *C, int M_GLOBAL, int N_GLOBAL, int K_GLOBAL);
+// bindings in the table, those with a user, device bytes they hold (any pointer may be null)
+void tzgemmWorkspaceStats(int *bindings, int *in_use, long long *bytes);
+// Frees every workspace after a device synchronisation.  Only when no kernel object that uses one
+// is left.
 void tzgemmReleaseWorkspaces();
 
 class OriTZGEMMKernel : public Kernel {
@@ -77,7 +83,7 @@ public:
         useGlobals = false;
         this->initParams();
     }
-    ~OriTZGEMMKernel() override {}
+    ~OriTZGEMMKernel() override { dropWorkspace(); }
 
     void initParams() override
     {
@@ -86,8 +92,10 @@ public:
         N_GLOBAL = d[1];
         K_GLOBAL = d[2];
         ori_blks = d[3];
+        dropWorkspace();   // of an earlier initParams
         if (useGlobals) ensureGlobalGemmBuffers(M_GLOBAL, N_GLOBAL, K_GLOBAL);
         tzgemmWorkspaceFor(useGlobals ? ori_wmma_C : C_, M_GLOBAL, N_GLOBAL, K_GLOBAL);
+        ws_m = M_GLOBAL, ws_n = N_GLOBAL, ws_k = K_GLOBAL;
 
         launchGridDim = dim3(ori_blks, 1, 1);
         launchBlockDim = dim3(TZ_THREADS, 1, 1);
@@ -120,6 +128,14 @@ protected:
 
 private:
     void loadKernel() override {}
+    // this object is no longer a user of the workspace bound to its output buffer (the global C may
+    // have moved since: its bindings moved with it)
+    void dropWorkspace()
+    {
+        if (ws_m) tzgemmWorkspaceDone(useGlobals ? ori_wmma_C : C_, ws_m, ws_n, ws_k);
+        ws_m = ws_n = ws_k = 0;
+    }
+    int ws_m = 0, ws_n = 0, ws_k = 0;   // shape whose workspace this object holds a use of
     bool useGlobals;
     void *A_ = nullptr;
     void *B_ = nullptr;

@@ -20,6 +20,9 @@ credits, src/TaskManager.cu:626-640); the ladder runs N/1024, N/512, ..., N/64 (
 a million positions and more), then N/32, 2N/32, ..., N and stops once a launch is twice as long as allowed.  The ratio is nb / 1024 for the nb with the largest
 earned time among those whose launch stays within (1 + stretch) * t0, i.e. the
 latency-critical GEMM is never stretched by more than that factor; 0 if nothing earns.
+Per pair also `whole_kernel_gain`: the 2048^3 GEMM and the whole best-effort kernel as two launches
+over the one fused launch that carries both; below 1 the scheduler's Tacker mode, which would let
+the whole kernel ride, carries the slice of the table instead.
 """
 import argparse
 import json
@@ -36,16 +39,21 @@ TILES = 1024
 LADDER = 32          # best-effort block counts tried: N/1024, N/512, ..., N/64, then N/32, 2N/32, ..., N
 
 
-def ladder(be_total):
-    """ascending block counts: a geometric run-up for kernels whose 1/32 is already longer than a GEMM
+def ladder(be_total, points=0):
+    """points > 0: that many counts only, spread geometrically from N/64 to N (a quick check of the
+    method); otherwise
+    ascending block counts: a geometric run-up for kernels whose 1/32 is already longer than a GEMM
     (sgemm: 2 ms for 528384 positions; from 1/65536 for grids of a million positions and more -- lavaMD:
     43 ms for 5832000), then the linear ladder"""
+    if points > 0:
+        steps = max(points - 1, 1)
+        return sorted({max(1, int(round(be_total / 64 ** ((steps - i) / steps)))) for i in range(points)})
     deepest = 17 if be_total >= 1 << 20 else 11
     counts = {be_total >> j for j in range(6, deepest)} | {be_total * step // LADDER for step in range(1, LADDER + 1)}
     return sorted(c for c in counts if c > 0)
 
 
-def measure(out_path, stretch, launches, pairs=PAIRS):
+def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_points=0):
     sys.path.insert(0, ROOT)
     import torch
     import tacker_amd as ta
@@ -70,7 +78,7 @@ def measure(out_path, stretch, launches, pairs=PAIRS):
         be_total = be.info()["ptb_end"]
         be_us = timed(be)
         table = {}
-        for K in K_LADDER:
+        for K in k_ladder:
             A = (torch.rand((2048, K), device="cuda") * 2 - 1).half()
             B = (torch.rand((2048, K), device="cuda") * 2 - 1).half()
             Cm = torch.zeros((2048, 2048), device="cuda")
@@ -78,7 +86,7 @@ def measure(out_path, stretch, launches, pairs=PAIRS):
             mix = ta.mix_create(be, tz, 0, 0, 0, TILES)
             t0 = timed(mix)
             best = {"blocks": 0, "earned_us": 0.0, "fused_us": t0}
-            for nb in ladder(be_total):
+            for nb in ladder(be_total, ladder_points):
                 mix.set_range(0, nb, 0, TILES)
                 t = timed(mix)
                 earned = t0 + be_us * nb / be_total - t
@@ -92,8 +100,27 @@ def measure(out_path, stretch, launches, pairs=PAIRS):
             print(f"tzgemm_{be_name} K={K}: t0 {t0:.1f} us, best {best['blocks']} of {be_total} blocks "
                   f"(fused {best['fused_us']:.1f} us, earns {best['earned_us']:.1f} us) "
                   f"-> ratio {best['blocks'] / TILES:.4f}", flush=True)
+        # the whole best-effort kernel in one fused launch with the 2048^3 GEMM against the two launches
+        # (what TaskManager's Tacker mode does); the two are timed back to back, as they would run
+        A = (torch.rand((2048, 2048), device="cuda") * 2 - 1).half()
+        B = (torch.rand((2048, 2048), device="cuda") * 2 - 1).half()
+        Cm = torch.zeros((2048, 2048), device="cuda")
+        tz = ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, TILES)
+        whole = ta.mix_create(be, tz, 0, be_total, 0, TILES)
+
+        class Serial:
+            def execute(self):
+                tz.execute()
+                be.execute()
+
+        serial_us, whole_us = timed(Serial()), timed(whole)
+        print(f"tzgemm_{be_name} whole kernel: serial {serial_us:.1f} us, fused {whole_us:.1f} us "
+              f"-> gain {serial_us / whole_us:.4f}", flush=True)
         result["pairs"]["tzgemm_" + be_name] = {"be_total_blocks": be_total, "be_solo_us": round(be_us, 2),
-                                                "by_k": table}
+                                                "by_k": table,
+                                                "whole_kernel": {"serial_us": round(serial_us, 2),
+                                                                 "fused_us": round(whole_us, 2),
+                                                                 "gain": round(serial_us / whole_us, 4)}}
     with open(out_path, "w") as f:
         json.dump(result, f, indent=1)
     print("wrote", out_path)
@@ -110,6 +137,8 @@ def apply(in_path):
         entry = dflt[key]
         entry["ratio_by_k"] = {k: v["ratio"] for k, v in m["by_k"].items()}
         entry["block_ratio"] = m["by_k"]["4096"]["ratio"]
+        if "whole_kernel" in m:
+            entry["whole_kernel_gain"] = m["whole_kernel"]["gain"]
     dflt["ratio_provenance"] = {"stretch": meas["stretch"], "device": meas["device"],
                                 "method": "profile_ratio.py: GEMM 2048x2048xK; best-effort block count with "
                                           "the largest time earned over serial launches whose fused launch "
@@ -128,11 +157,15 @@ def main():
     ap.add_argument("--stretch", type=float, default=1.0,
                     help="largest tolerated stretch of the GEMM's launch (1.0 = at most twice as long)")
     ap.add_argument("--launches", type=int, default=100)
+    ap.add_argument("--k-ladder", default=",".join(str(k) for k in K_LADDER), help="reduction lengths to measure at")
+    ap.add_argument("--ladder-points", type=int, default=0,
+                    help="measure only this many block counts per K (N/64 .. N); 0 = the full ladder")
     ap.add_argument("--pairs", default=",".join(PAIRS),
                     help="best-effort kernels to measure (comma separated); --apply only touches those measured")
     args = ap.parse_args()
     if args.measure:
-        measure(args.measure, args.stretch, args.launches, tuple(args.pairs.split(",")))
+        measure(args.measure, args.stretch, args.launches, tuple(args.pairs.split(",")),
+                tuple(int(k) for k in args.k_ladder.split(",")), args.ladder_points)
     elif args.apply:
         apply(args.apply)
     else:

@@ -200,6 +200,131 @@ def test_workspace_table_slots_follow_the_hash_the_kernels_probe(fake):
     assert fake.tacker_tzgemm_release_workspaces() == 0
 
 
+def _ws_table(fake):
+    raw = C.create_string_buffer(1024 * 16)
+    n = fake.tk_fake_symbol(b"tz_ws_table", raw, len(raw))
+    words = struct.unpack(f"<{n // 8}Q", raw.raw[:n]) + (0,) * (2048 - n // 8)
+    return [(words[2 * i], words[2 * i + 1]) for i in range(1024)]
+
+
+def _ws_lookup(table, key):
+    """the device-side probe (csrc/kernels/tzgemm_role.h tz_find_workspace): stops at an empty slot,
+    walks past tombstones"""
+    slot = (((key >> 8) * 0x9E3779B97F4A7C15) % (1 << 64)) >> 54
+    for probe in range(16):
+        c, w = table[(slot + probe) % 1024]
+        if c == key:
+            return w
+        if c == 0:
+            return 0
+    return 0
+
+
+def _ws_stats(fake):
+    b, u, n = C.c_int(), C.c_int(), C.c_longlong()
+    fake.tacker_tzgemm_workspace_stats.argtypes = [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_longlong)]
+    assert fake.tacker_tzgemm_workspace_stats(C.byref(b), C.byref(u), C.byref(n)) == 0
+    return b.value, u.value, n.value
+
+
+def test_more_output_buffers_than_the_workspace_table_holds(fake):
+    """a caller whose output addresses keep changing: bindings nobody uses any more make room, least
+    recently used first, and every live key stays findable by the device-side probe"""
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+    A = np.zeros((256, 1024), np.float16)
+    outs = [np.zeros((256, 256), np.float32) for _ in range(700)]
+    for i, Cm in enumerate(outs):
+        assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 256, 256, 1024, 0, 16, 0, None) == 0, \
+            (i, fake.tacker_last_error())
+        table = _ws_table(fake)
+        assert _ws_lookup(table, Cm.ctypes.data) != 0, i
+    bindings, in_use, held = _ws_stats(fake)
+    assert bindings <= 512 and in_use == 0
+    assert held == bindings * fake.tacker_tzgemm_workspace_bytes(256, 256, 1024)
+    table = _ws_table(fake)
+    live = [Cm.ctypes.data for Cm in outs if _ws_lookup(table, Cm.ctypes.data)]
+    assert len(live) == bindings
+    assert outs[0].ctypes.data not in live and outs[-1].ctypes.data in live     # the oldest went first
+    assert sum(1 for c, _ in table if c == 1) > 0                               # tombstones mark what went
+    # a binding with a user is never taken: hold 40 kernel objects, then churn through 600 more buffers
+    held_objs = [fake.tacker_ori_tzgemm_create(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 256, 256, 1024)
+                 for Cm in outs[:40]]
+    assert all(held_objs)
+    more = [np.zeros((256, 256), np.float32) for _ in range(600)]
+    for Cm in more:
+        assert fake.tacker_gptb_tzgemm(A.ctypes.data, A.ctypes.data, Cm.ctypes.data, 256, 256, 1024, 0, 16, 0, None) == 0
+    table = _ws_table(fake)
+    assert all(_ws_lookup(table, Cm.ctypes.data) for Cm in outs[:40])
+    assert _ws_stats(fake)[1] == 40
+    for h in held_objs:
+        assert fake.tacker_kernel_destroy(h) == 0
+    assert _ws_stats(fake)[1] == 0
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+    assert _ws_stats(fake) == (0, 0, 0)
+
+
+def test_sgemm_and_tzgemm_on_one_output_buffer_never_share_a_workspace(fake):
+    """in any order of construction and launch: the two kinds of kernel bind under different keys, so
+    sgemm's partial sums can never lie where a tzgemm object expects its arrival counters at zero"""
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+    A16 = np.zeros((256, 1024), np.float16)
+    A32 = np.zeros((1024, 256), np.float32)
+    Cm = np.zeros((256, 256), np.float32)
+    fake.tacker_ori_tzgemm_create.restype = C.c_void_p
+    fake.tacker_ori_sgemm_create.restype = C.c_void_p
+    tz = fake.tacker_ori_tzgemm_create(A16.ctypes.data, A16.ctypes.data, Cm.ctypes.data, 256, 256, 1024)
+    sg = fake.tacker_ori_sgemm_create(A32.ctypes.data, A32.ctypes.data, Cm.ctypes.data, 256, 256, 1024)
+    assert tz and sg
+    table = _ws_table(fake)
+    w_tz, w_sg = _ws_lookup(table, Cm.ctypes.data), _ws_lookup(table, Cm.ctypes.data + 2)
+    assert w_tz and w_sg and w_tz != w_sg
+    assert _ws_stats(fake)[:2] == (2, 2)
+    # the older tzgemm object after the sgemm object, and a second tzgemm object: same workspace, still tzgemm's
+    tz2 = fake.tacker_ori_tzgemm_create(A16.ctypes.data, A16.ctypes.data, Cm.ctypes.data, 256, 256, 1024)
+    assert _ws_lookup(_ws_table(fake), Cm.ctypes.data) == w_tz
+    for h in (tz, sg, tz2):
+        assert fake.tacker_kernel_destroy(C.c_void_p(h)) == 0
+    assert _ws_stats(fake)[:2] == (2, 0)
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+
+
+def test_workspaces_of_the_global_output_buffer_follow_it_when_it_grows(fake):
+    """the global C is freed and allocated anew when a larger shape is created: its binding moves to the
+    new address (the kernel objects built on the global buffers keep a workspace) and nothing stays bound
+    to the freed one"""
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+    fake.tacker_ori_tzgemm_create.restype = C.c_void_p
+
+    def global_c():
+        a, b, c = C.c_void_p(), C.c_void_p(), C.c_void_p()
+        sizes = (C.c_longlong * 3)()
+        assert fake.tacker_global_gemm_buffers(C.byref(a), C.byref(b), C.byref(c), sizes) == 0
+        return c.value, sizes[2]
+
+    _, have = global_c()
+    side = 256
+    while 4 * side * side <= have:      # a shared-reduction shape larger than anything created so far
+        side *= 2
+    small = fake.tacker_ori_tzgemm_create(None, None, None, 256, 256, 1024)
+    assert small
+    c0, _ = global_c()
+    w0 = _ws_lookup(_ws_table(fake), c0)
+    assert w0
+    big = fake.tacker_ori_tzgemm_create(None, None, None, side, 128, 1024)
+    assert big
+    c1, have1 = global_c()
+    assert have1 >= 4 * side * 128
+    table = _ws_table(fake)
+    if c1 != c0:
+        assert _ws_lookup(table, c0) == 0
+    assert _ws_lookup(table, c1) != 0
+    assert _ws_stats(fake)[:2] == (1, 1)
+    for h in (small, big):
+        assert fake.tacker_kernel_destroy(C.c_void_p(h)) == 0
+    assert _ws_stats(fake)[1] == 0
+    assert fake.tacker_tzgemm_release_workspaces() == 0
+
+
 # ------------------------------------------------------------------ marshalling
 def test_gptb_stencil_parameter_vector(fake):
     fake.tk_fake_reset()
