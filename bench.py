@@ -311,11 +311,11 @@ def pair_leg(ta, torch, np, name, stream):
     # whole-kernel gain says that it pays, and falls back to the Aker slice otherwise
     whole = ta.lib().tacker_qos_whole_kernel_gain(name.encode())
     out["scheduler"] = {"aker_slice_blocks": slice_blocks, "aker_fuses": bool(slice_blocks > 0),
-                        "kinfo_whole_kernel_gain": round(whole, 4), "tacker_fuses_whole_kernel": bool(whole >= 1.0)}
+                        "kinfo_whole_kernel_gain": round(whole, 4), "tacker_fuses_whole_kernel": bool(whole >= 1.03)}
     picked = []
     if slice_blocks > 0:
         picked.append(out.get("cursor_speedup", out["slice_speedup_at_kernel_rate"]))
-    if whole >= 1.0:
+    if whole >= 1.03:    # QosPolicy::kWholeKernelGainMin
         picked.append(out["speedup"])
     out["scheduler"]["slowest_form_it_would_pick"] = round(min(picked), 4) if picked else None
     out["gemm_tflops_alone"] = round(flop / out["gemm_us"] / 1e6, 1)

@@ -110,7 +110,7 @@ int QosPolicy::coLocatedBlocks(ExecutionMode mode, const std::string &be_name, i
                                int be_total_blocks)
 {
     // the whole BE kernel rides along, unless it is known to lose that way
-    if (mode == ExecutionMode::Tacker && wholeKernelGain(be_name) >= 1.0f) return be_total_blocks;
+    if (mode == ExecutionMode::Tacker && wholeKernelGain(be_name) >= kWholeKernelGainMin) return be_total_blocks;
     return std::min(int(tiles * blockRatio(be_name, K_GLOBAL)), be_total_blocks);
 }
 

@@ -39,6 +39,8 @@ struct QosPolicy {
     // whole best-effort kernel in one fused launch; 1 when kinfo has none (the reference always
     // fuses, and credits a launch only if it beat the solo launches, :696-700)
     static float wholeKernelGain(const std::string &be_name);
+    // the gain from which on Tacker mode lets the whole kernel ride: 3 % clear of breaking even
+    static constexpr float kWholeKernelGainMin = 1.03f;
     // how many BE blocks ride along with a GEMM of `tiles` tiles (:599-600).  Tacker mode lets the
     // whole kernel ride unless kinfo says that this loses against the two launches
     // (wholeKernelGain < 1); it then carries the slice Aker mode would.

@@ -48,9 +48,7 @@
 #include "tzgemm_role.h"
 
 #define TZL_LOOP_LOAD(...) tz_load_to_lds(__VA_ARGS__)
-#define TZL_LOOP_BARRIER() __builtin_amdgcn_s_barrier()
 #define TZL_LOOP_READ(dst_, src_) dst_ = src_
-#define TZL_STORE_IF(v_)
 
 namespace tk {
 
@@ -69,17 +67,18 @@ __device__ __forceinline__ void tz_large_tile_of(int t, int tile_rows, int tile_
     mj = in_band / band;
 }
 
-// The role owns every wave of its workgroup (it synchronises with s_barrier).
+// Sync: the barrier among the role's four waves -- WorkgroupSync (the hardware barrier) when the
+// role owns every wave of its workgroup, RoleHandoverSync inside a wave-split fused kernel.
 // stream_c: C leaves with nontemporal stores.  Pays when C is larger than the caches can hold
 // until the memory has taken it (256 MiB at 8192 x 8192: plain stores push the operand panels out
 // of the L2s); below that plain stores are the faster ones -- the L2s and the memory-side cache
 // take the tile at once and write it back while the next kernel already runs (4096 x 4096 x 1024:
 // 37 instead of 43 us).
-template <int FM, int FN>
+template <int FM, int FN, class Sync>
 __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
                                                   float *__restrict__ C, int M, int N, int K, int role_block,
                                                   int role_blocks, int tile_start, int tile_end, int tid,
-                                                  char *lds, bool stream_c)
+                                                  char *lds, bool stream_c, Sync &sync)
 {
     typedef __attribute__((address_space(3))) void *lptr_t;
     constexpr int TM = 32 * FM, TN = 32 * FN;      // macro tile
@@ -91,12 +90,13 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
     constexpr int LB = TN / 8 / 4;                 // ... and B (one load = 8 rows of 128 bytes)
     constexpr int L = LA + LB;
     constexpr int FIRST = 8;                       // MFMAs of an iteration in front of the barrier
-    constexpr int READ_GAP = 3;                    // one LDS read per READ_GAP MFMAs
+    // one LDS read per READ_GAP MFMAs: 3 where the iteration is long enough, else as many as fit
+    constexpr int READ_GAP = (FM * FN - FIRST) / (FM + FN) >= 3 ? 3 : (FM * FN - FIRST) / (FM + FN);
     constexpr int LOAD_GAP = (FM * FN - FIRST) / L;
     static_assert(FM % 4 == 0 && FN % 4 == 0, "a wave tile is whole reference tiles");
     static_assert(LA <= 8 && LB <= 8, "eight row blocks of 8 per wave and operand at most");
     static_assert(L < 64, "vmcnt is a 6-bit counter");
-    static_assert((FM + FN) * READ_GAP <= FM * FN - FIRST && LOAD_GAP >= 1,
+    static_assert(READ_GAP >= 1 && (FM + FN) * READ_GAP <= FM * FN - FIRST && LOAD_GAP >= 1,
                   "an iteration slots its LDS reads and loads between the MFMAs behind the barrier");
     static_assert(2 * PAIR_BYTES <= TZ_LDS_BYTES, "the ring is two buffers");
 
@@ -195,8 +195,7 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
             __builtin_amdgcn_sched_barrier(0);                                                    \
         }                                                                                         \
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));                                              \
-        TZL_LOOP_BARRIER();                                                                       \
-        asm volatile("" ::: "memory");                                                            \
+        sync.wait();                                                                              \
         __builtin_amdgcn_sched_barrier(0);                                                        \
         _Pragma("unroll") for (int n = FIRST; n < FM * FN; ++n)                                   \
         {                                                                                         \
@@ -237,8 +236,7 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
             b_next += ROWB;
         }
         __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(L));
-        __builtin_amdgcn_s_barrier();
-        asm volatile("" ::: "memory");
+        sync.wait();
         half8_t fa0[FM], fb0[FN], fa1[FM], fb1[FN];
 #pragma unroll
         for (int i = 0; i < FM; ++i) fa0[i] = TZL_FRAG_A(0, frag_h0, i);
@@ -258,8 +256,7 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
         TZL_ITERATION_SECOND(fa1, fb1, fa0, fb0, 0, 1, false)
         TZL_ITERATION_FIRST(fa0, fb0, fa1, fb1, 1)
         _Pragma("unroll") for (int n = 0; n < FM * FN; ++n) { TZL_MFMA_AT(fa1, fb1, n) }
-        __builtin_amdgcn_s_barrier();   // every wave is done reading before the next tile refills the ring
-        asm volatile("" ::: "memory");
+        sync.wait();   // every wave is done reading before the next tile refills the ring
 
         // lane holds C[row0 + 16 i + lane % 16][col0 + 16 j + 4 (lane / 16) .. + 3]
         float *c_lane = C + (size_t)(mi * TM + wr * (FM * 16) + (lane & 15)) * N + mj * TN + wc * (FN * 16) +
@@ -276,11 +273,8 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
                     for (int j = 4 * rj; j < 4 * rj + 4; ++j) {
                         float4_t v = acc[i][j] * TZ_ALPHA;
                         float4_t *c_at = reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16);
-                        TZL_STORE_IF(v)
-                        {
-                            if (stream_c) __builtin_nontemporal_store(v, c_at);   // uniform
-                            else *c_at = v;
-                        }
+                        if (stream_c) __builtin_nontemporal_store(v, c_at);   // uniform
+                        else *c_at = v;
                     }
             }
         // The stores stay in flight while the next tile starts: they share the vmcnt counter with
@@ -293,6 +287,7 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
 #undef TZL_ITERATION_FIRST
 #undef TZL_ITERATION_SECOND
     }
+    sync.finish();
 }
 
 }  // namespace tk

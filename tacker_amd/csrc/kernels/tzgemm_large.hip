@@ -25,9 +25,10 @@ extern "C" __global__ __launch_bounds__(TZ_THREADS) __attribute__((amdgpu_waves_
     __shared__ __align__(16) char tz_lds[TZ_LDS_BYTES];
     // a launch on a shape the form does not cover (the host never makes one) computes nothing
     if (M_GLOBAL % TZ_LARGE_TILE || N_GLOBAL % TZ_LARGE_TILE || K_GLOBAL % 128) return;
+    tk::WorkgroupSync sync;
     tk::tzgemm_role_large<8, 8>(A, B, C, M_GLOBAL, N_GLOBAL, K_GLOBAL, (int)blockIdx.x, ptb_iter_block_step,
                                 ptb_start_block_pos, ptb_end_block_pos, (int)threadIdx.x - thread_base, tz_lds,
-                                (size_t)M_GLOBAL * (size_t)N_GLOBAL * sizeof(float) > TZ_LARGE_STREAM_C_BYTES);
+                                (size_t)M_GLOBAL * (size_t)N_GLOBAL * sizeof(float) > TZ_LARGE_STREAM_C_BYTES, sync);
 }
 
 extern "C" void tk_register_large_kernels(tk_kernel_insert_fn insert, void *ctx)

@@ -13,12 +13,13 @@ Two steps, because the GPU box and the build tree are different places:
     python profile_ratio.py --measure out.json          # on the GPU
     python profile_ratio.py --apply out.json            # rewrites defaults.json; then gen_run.py
 Method per (pair, K): GEMM 2048 x 2048 x K (1024 tiles, one 128x128 macro tile per CU).
-t0 = fused launch with no best-effort block, t_be = the best-effort kernel alone (all N
-blocks).  For nb on a ladder of block counts, earned(nb) = t0 + t_be * nb / N - t_fused(nb)
+t_gemm = the GEMM's own kernel alone, t_be = the best-effort kernel alone (all N blocks).
+For nb on a ladder of block counts, earned(nb) = t_gemm + t_be * nb / N - t_fused(nb)
 is the time one fused launch saves over the two serial launches (the quantity TaskManager
-credits, src/TaskManager.cu:626-640); the ladder runs N/1024, N/512, ..., N/64 (from N/65536 for grids of
+credits, src/TaskManager.cu:626-640); a count qualifies only if it earns at least min_gain
+(3 %) of those serial launches, so that a pair within the noise of breaking even is not fused; the ladder runs N/1024, N/512, ..., N/64 (from N/65536 for grids of
 a million positions and more), then N/32, 2N/32, ..., N and stops once a launch is twice as long as allowed.  The ratio is nb / 1024 for the nb with the largest
-earned time among those whose launch stays within (1 + stretch) * t0, i.e. the
+earned time among those whose launch stays within (1 + stretch) * t_gemm, i.e. the
 latency-critical GEMM is never stretched by more than that factor; 0 if nothing earns.
 Per pair also `whole_kernel_gain`: the 2048^3 GEMM and the whole best-effort kernel as two launches
 over the one fused launch that carries both; below 1 the scheduler's Tacker mode, which would let
@@ -53,7 +54,7 @@ def ladder(be_total, points=0):
     return sorted(c for c in counts if c > 0)
 
 
-def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_points=0):
+def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_points=0, min_gain=0.03):
     sys.path.insert(0, ROOT)
     import torch
     import tacker_amd as ta
@@ -62,7 +63,18 @@ def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_
     e0, e1 = ta.Event(), ta.Event()
 
     def timed(kernel):
-        for _ in range(10):
+        # Warm up for at least 5 ms of the kernel's own work before timing: after an allocation or a
+        # copy the GPU is back at idle clocks, and a kernel of 20 us timed over its first hundred
+        # launches reads up to a quarter too long -- which, for the GEMM alone, would be booked as
+        # time the fused launch "earns".
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(3):
+            kernel.execute()
+        e1.record()
+        e1.synchronize()
+        est_us = max(e0.elapsed_ms(e1) / 3 * 1e3, 1.0)
+        for _ in range(int(min(max(10, 5000.0 / est_us), 4 * launches))):
             kernel.execute()
         torch.cuda.synchronize()
         e0.record()
@@ -72,7 +84,7 @@ def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_
         e1.synchronize()
         return e0.elapsed_ms(e1) / launches * 1e3
 
-    result = {"stretch": stretch, "tiles": TILES, "device": ta.device_name(), "pairs": {}}
+    result = {"stretch": stretch, "min_gain": min_gain, "tiles": TILES, "device": ta.device_name(), "pairs": {}}
     for be_name in pairs:
         be = ta.create_kernel(be_name)
         be_total = be.info()["ptb_end"]
@@ -84,20 +96,23 @@ def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_
             Cm = torch.zeros((2048, 2048), device="cuda")
             tz = ta.gptb_create(ta.ori_tzgemm_create(A, B, Cm), 0, 0, 0, TILES)
             mix = ta.mix_create(be, tz, 0, 0, 0, TILES)
-            t0 = timed(mix)
+            t_gemm = timed(tz)           # the serial side: the GEMM's own kernel ...
+            t0 = timed(mix)              # ... which the fused kernel carrying nothing does not quite match
+            t_gemm = min(t_gemm, timed(tz))
             best = {"blocks": 0, "earned_us": 0.0, "fused_us": t0}
             for nb in ladder(be_total, ladder_points):
                 mix.set_range(0, nb, 0, TILES)
                 t = timed(mix)
-                earned = t0 + be_us * nb / be_total - t
-                if t <= (1 + stretch) * t0 and earned > best["earned_us"]:
+                serial = t_gemm + be_us * nb / be_total
+                earned = serial - t
+                if t <= (1 + stretch) * t_gemm and earned >= min_gain * serial and earned > best["earned_us"]:
                     best = {"blocks": nb, "earned_us": earned, "fused_us": t}
-                if t > 2 * (1 + stretch) * t0:      # more blocks only make the launch longer
+                if t > 2 * (1 + stretch) * t_gemm:      # more blocks only make the launch longer
                     break
             table[str(K)] = {"blocks": best["blocks"], "ratio": round(best["blocks"] / TILES, 4),
-                             "gemm_in_fused_us": round(t0, 2), "fused_us": round(best["fused_us"], 2),
+                             "gemm_us": round(t_gemm, 2), "gemm_in_fused_us": round(t0, 2), "fused_us": round(best["fused_us"], 2),
                              "earned_us": round(best["earned_us"], 2)}
-            print(f"tzgemm_{be_name} K={K}: t0 {t0:.1f} us, best {best['blocks']} of {be_total} blocks "
+            print(f"tzgemm_{be_name} K={K}: GEMM {t_gemm:.1f} us ({t0:.1f} in the fused kernel), best {best['blocks']} of {be_total} blocks "
                   f"(fused {best['fused_us']:.1f} us, earns {best['earned_us']:.1f} us) "
                   f"-> ratio {best['blocks'] / TILES:.4f}", flush=True)
         # the whole best-effort kernel in one fused launch with the 2048^3 GEMM against the two launches
@@ -139,11 +154,11 @@ def apply(in_path):
         entry["block_ratio"] = m["by_k"]["4096"]["ratio"]
         if "whole_kernel" in m:
             entry["whole_kernel_gain"] = m["whole_kernel"]["gain"]
-    dflt["ratio_provenance"] = {"stretch": meas["stretch"], "device": meas["device"],
+    dflt["ratio_provenance"] = {"stretch": meas["stretch"], "min_gain": meas.get("min_gain", 0.0), "device": meas["device"],
                                 "method": "profile_ratio.py: GEMM 2048x2048xK; best-effort block count with "
-                                          "the largest time earned over serial launches whose fused launch "
-                                          "stays within (1+stretch) of the launch without best-effort "
-                                          "blocks, divided by 1024 tiles"}
+                                          "the largest time earned over serial launches (at least min_gain of "
+                                          "them) whose fused launch stays within (1+stretch) of the GEMM "
+                                          "alone, divided by 1024 tiles"}
     with open(DEFAULTS, "w") as f:
         json.dump(dflt, f, indent=2)
         f.write("\n")
@@ -156,6 +171,8 @@ def main():
     ap.add_argument("--apply", metavar="IN.json")
     ap.add_argument("--stretch", type=float, default=1.0,
                     help="largest tolerated stretch of the GEMM's launch (1.0 = at most twice as long)")
+    ap.add_argument("--min-gain", type=float, default=0.03,
+                    help="a block count qualifies only if the fused launch saves this fraction of the serial launches")
     ap.add_argument("--launches", type=int, default=100)
     ap.add_argument("--k-ladder", default=",".join(str(k) for k in K_LADDER), help="reduction lengths to measure at")
     ap.add_argument("--ladder-points", type=int, default=0,
@@ -165,7 +182,7 @@ def main():
     args = ap.parse_args()
     if args.measure:
         measure(args.measure, args.stretch, args.launches, tuple(args.pairs.split(",")),
-                tuple(int(k) for k in args.k_ladder.split(",")), args.ladder_points)
+                tuple(int(k) for k in args.k_ladder.split(",")), args.ladder_points, args.min_gain)
     elif args.apply:
         apply(args.apply)
     else:

@@ -37,19 +37,20 @@ def test_load_ratio_sweep_measures_one_pair_on_a_four_point_ladder(tmp_path):
     assert set(pair["by_k"]) == {str(k) for k in ks}
     for k in ks:
         row = pair["by_k"][str(k)]
-        assert set(row) == {"blocks", "ratio", "gemm_in_fused_us", "fused_us", "earned_us"}
+        assert set(row) == {"blocks", "ratio", "gemm_us", "gemm_in_fused_us", "fused_us", "earned_us"}
         assert row["blocks"] in [0] + counts                  # a rung of the ladder, or nothing earns
         assert 0.0 <= row["ratio"] <= counts[-1] / 1024
         assert row["ratio"] == round(row["blocks"] / 1024, 4)
-        assert row["gemm_in_fused_us"] > 0 and row["fused_us"] >= row["gemm_in_fused_us"] * 0.9
-        assert row["fused_us"] <= 2.0 * row["gemm_in_fused_us"] * 1.001 or row["blocks"] == 0   # the stretch bound
+        assert row["gemm_us"] > 0 and row["gemm_in_fused_us"] > 0 and row["fused_us"] >= row["gemm_us"] * 0.9
+        assert row["fused_us"] <= 2.0 * row["gemm_us"] * 1.001 or row["blocks"] == 0   # the stretch bound
         assert row["earned_us"] >= 0.0
         if row["blocks"]:
             # what it claims to earn is what the two serial launches would cost minus the fused launch
-            serial = row["gemm_in_fused_us"] + pair["be_solo_us"] * row["blocks"] / total
+            serial = row["gemm_us"] + pair["be_solo_us"] * row["blocks"] / total
             assert abs(serial - row["fused_us"] - row["earned_us"]) <= 0.02 + 1e-3 * serial
+            assert row["earned_us"] >= meas["min_gain"] * serial - 0.02
     # a longer reduction is a longer GEMM
-    assert pair["by_k"]["2048"]["gemm_in_fused_us"] > pair["by_k"]["640"]["gemm_in_fused_us"]
+    assert pair["by_k"]["2048"]["gemm_us"] > pair["by_k"]["640"]["gemm_us"]
     whole = pair["whole_kernel"]
     assert whole["serial_us"] > 0 and whole["fused_us"] > 0
     assert abs(whole["gain"] - whole["serial_us"] / whole["fused_us"]) < 1e-3
