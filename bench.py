@@ -355,12 +355,20 @@ def gemm_leg(ta, torch, np, stream):
 
         ours = statistics.median(timed(lambda: tz.execute(stream)) for _ in range(3))
         lib = statistics.median(timed(lambda: torch.matmul(A, Bt)) for _ in range(3))
+        # the library with the output type tzgemm has (an fp32 C is twice the bytes of torch.matmul's fp16 C);
+        # None where this torch build does not offer it
+        try:
+            torch.mm(A, Bt, out_dtype=torch.float32)
+            lib32 = statistics.median(timed(lambda: torch.mm(A, Bt, out_dtype=torch.float32)) for _ in range(3))
+        except Exception:
+            lib32 = None
         flop = 2.0 * M * N * K
         out[f"{M}x{N}x{K}"] = {"us": round(ours, 2), "tflops": round(flop / ours / 1e6, 1),
                                "frac_of_mfma_peak": round(flop / (ours * 1e-6) / MFMA_F16_PEAK, 4),
                                "form": "256x256 tiles" if (M % 256 == 0 and N % 256 == 0 and (M // 256) * (N // 256) >= 256)
                                else "128x128 tiles",
-                               "torch_matmul_us": round(lib, 2), "torch_matmul_tflops": round(flop / lib / 1e6, 1)}
+                               "torch_matmul_us": round(lib, 2), "torch_matmul_tflops": round(flop / lib / 1e6, 1),
+                               "torch_mm_fp32_out_us": None if lib32 is None else round(lib32, 2)}
     return out
 
 
@@ -534,8 +542,8 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(A, B, A0, c0, c1)
     if "tzgemm_shapes" in out:
-        # shape -> [tzgemm us, fraction of the MFMA peak, torch.matmul us]
-        out["tzgemm_shapes_summary"] = {k: [v["us"], v["frac_of_mfma_peak"], v["torch_matmul_us"]]
+        # shape -> [tzgemm us, fraction of the MFMA peak, torch.matmul us (fp16 C), torch.mm us with an fp32 C]
+        out["tzgemm_shapes_summary"] = {k: [v["us"], v["frac_of_mfma_peak"], v["torch_matmul_us"], v["torch_mm_fp32_out_us"]]
                                         for k, v in out["tzgemm_shapes"].items()}
     if "other_pairs" in out:
         # pair -> [whole kernel fused, slice at the kernel's rate, cursor (the scheduler's slices), GEMM us, best-effort us,

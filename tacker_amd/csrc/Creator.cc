@@ -96,7 +96,18 @@ MixKernel *createTzgemmMix(GPTBKernel *be, GPTBKernel *tz, int be_start, int be_
                            int tile_end, const std::string &variant, int launch_grid, int launch_block)
 {
     const std::string base = "tzgemm_" + be->kernelName;
-    const std::string key = variant.empty() ? base : base + "@" + variant;
+    std::string key = variant.empty() ? base : base + "@" + variant;
+    if (variant.empty() && tz->kernel_) {
+        // a GEMM large enough for 256 x 128 tiles takes the form kinfo names for such shapes, if the pair has one
+        const std::vector<int> mnk = tz->kernel_->getArgs();
+        if (mnk.size() == 3) {
+            const std::vector<int> d = getTZGEMMGridDim(mnk[0], mnk[1], mnk[2]);
+            const std::string large = sget_kernel_info(base, "large_gemm_variant");
+            if (tz_use_large_fused(d[0], d[1], d[2]) && !large.empty() &&
+                get_kernel_info(base + "@" + large, "blocksize") != JSON_NOT_FOUND)
+                key = base + "@" + large;
+        }
+    }
     int per_cu = get_kernel_info(key, "gridsize");
     int bs = get_kernel_info(key, "blocksize");
     int group = get_kernel_info(key, "group");

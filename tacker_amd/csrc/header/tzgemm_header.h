@@ -96,6 +96,24 @@ TZ_HOST_DEVICE inline bool tz_use_large(int M, int N, int K)
            (long long)(M / TZ_LARGE_TILE) * (N / TZ_LARGE_TILE) >= TZ_LARGE_MIN_TILES;
 }
 
+// The GEMM role of a 512-thread fused kernel (variant wave_256_large) takes 256 x 128 tiles
+// (tzgemm_role_large_rot) for every shape they divide -- whole tiles, an even number of 64-k steps --
+// that is not one of the K-split forms', and the 128 x 128 form otherwise: tz_large_fused_fits, asked by the kernel.  The host picks that
+// variant by itself only where it pays, a tile for every CU: tz_use_large_fused.
+#define TZ_LARGE_FUSED_TILE_M 256
+#define TZ_LARGE_FUSED_TILE_N 128
+TZ_HOST_DEVICE inline bool tz_large_fused_fits(int M, int N, int K)
+{
+    // (not the shapes of the K-split forms: there the order of additions is another one, and a fused
+    // launch gives the bits of the plain kernel whatever its form)
+    return M % TZ_LARGE_FUSED_TILE_M == 0 && N % TZ_LARGE_FUSED_TILE_N == 0 && K % 128 == 0 && !tz_use_ksplit(M, N, K);
+}
+TZ_HOST_DEVICE inline bool tz_use_large_fused(int M, int N, int K)
+{
+    return tz_large_fused_fits(M, N, K) &&
+           (long long)(M / TZ_LARGE_FUSED_TILE_M) * (N / TZ_LARGE_FUSED_TILE_N) >= TZ_LARGE_MIN_TILES;
+}
+
 // Where a kernel finds the workspace of the output buffer it writes: a device-resident hash
 // table from C to workspace that the host fills when it binds one (open addressing, linear
 // probing, an entry is never moved or removed while kernels may run; key 0 = empty).  The

@@ -25,6 +25,7 @@
 #include "sgemm_role.h"
 #include "stencil_role.h"
 #include "tzgemm_role.h"
+#include "tzgemm_large.h"   // the large-tile GEMM role of the 512-thread fused kernels
 
 #define GPTB_TRAILER                                                                            \
     int grid_dimension_x, int grid_dimension_y, int grid_dimension_z, int block_dimension_x,    \

@@ -156,13 +156,16 @@ struct RoleHandoverSync {
     unsigned gave_up;
     unsigned *fail;
     unsigned spin_limit;
-    unsigned hw;             // the same in all lanes: 1 = hardware barrier from now on
-    unsigned announce;       // the same in all lanes: decider has seen the other role's waves gone
-    unsigned decider;        // the same in all lanes: this is the role's first wave
-    __device__ __forceinline__ RoleHandoverSync(unsigned *words, unsigned w, bool first_wave, unsigned *f,
+    // wave-uniform state, kept in scalar registers (every value below comes out of a readfirstlane):
+    unsigned hw;             // 1 = hardware barrier from now on
+    unsigned announce;       // decider has seen the other role's waves gone
+    unsigned decider;        // this is the role's first wave
+    // role_tid: the caller's thread index within the role (its first 64 threads are the decider wave)
+    __device__ __forceinline__ RoleHandoverSync(unsigned *words, unsigned w, int role_tid, unsigned *f,
                                                 unsigned limit = (1u << 24))
         : counter_addr((unsigned)(size_t)(__attribute__((address_space(3))) unsigned *)words), waves(w), expected(0),
-          gave_up(0), fail(f), spin_limit(limit), hw(0), announce(0), decider(first_wave ? 1u : 0u) {}
+          gave_up(0), fail(f), spin_limit(limit), hw(0), announce(0),
+          decider(__builtin_amdgcn_readfirstlane(role_tid) < 64 ? 1u : 0u) {}
 
     // what thread 0 of the workgroup stores before the roles part ways: no arrival, other_waves
     // waves of the other role at work, no change-over in sight
@@ -179,7 +182,7 @@ struct RoleHandoverSync {
     // test and the counter's code in line the loop ran 12 % slower than with the bare s_barrier.)
     __device__ __forceinline__ void wait()
     {
-        if (__builtin_expect(__builtin_amdgcn_readfirstlane(hw) != 0u, 1)) {
+        if (__builtin_expect(hw != 0u, 1)) {
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         } else {
@@ -190,13 +193,12 @@ struct RoleHandoverSync {
     __device__ __forceinline__ void on_the_counter()
     {
         expected += waves;
-        unsigned now, at, alive, left, uni;
+        unsigned now, at, alive, left, hw_lanes, announce_lanes;
         unsigned long long saved_exec;
         asm volatile("s_mov_b32 %[left], %[limit]\n\t"
-                     "v_readfirstlane_b32 %[uni], %[announce]\n\t"
                      "s_mov_b64 %[saved], exec\n\t"
                      "s_mov_b64 exec, 1\n\t"
-                     "s_cmp_eq_u32 %[uni], 0\n\t"
+                     "s_cmp_eq_u32 %[announce_in], 0\n\t"
                      "s_cbranch_scc1 8f\n\t"
                      "ds_write_b32 %[addr], %[index] offset:8\n"
                      "8:\n\t"
@@ -219,15 +221,16 @@ struct RoleHandoverSync {
                      "v_cmp_le_i32 vcc, 0, %[at]\n\t"
                      "v_cndmask_b32_e64 %[hw], 0, 1, vcc\n\t"
                      "v_cmp_eq_u32 vcc, 0, %[alive]\n\t"
-                     "v_cndmask_b32_e64 %[announce], 0, 1, vcc"
-                     : [now] "=&v"(now), [at] "=&v"(at), [alive] "=&v"(alive), [left] "=&s"(left), [uni] "=&s"(uni),
-                       [saved] "=&s"(saved_exec), [hw] "=&v"(hw), [announce] "+v"(announce)
-                     : [addr] "v"(counter_addr), [index] "v"(expected), [one] "v"(1u), [limit] "s"(spin_limit)
+                     "v_cndmask_b32_e64 %[announce_out], 0, 1, vcc"
+                     : [now] "=&v"(now), [at] "=&v"(at), [alive] "=&v"(alive), [left] "=&s"(left),
+                       [saved] "=&s"(saved_exec), [hw] "=&v"(hw_lanes), [announce_out] "=&v"(announce_lanes)
+                     : [addr] "v"(counter_addr), [index] "v"(expected), [one] "v"(1u), [limit] "s"(spin_limit),
+                       [announce_in] "s"(announce)
                      : "vcc", "scc", "memory");
-        announce &= decider;
+        announce = __builtin_amdgcn_readfirstlane(announce_lanes) & decider;
         const unsigned out_of_polls = (left == 0u);
         gave_up |= out_of_polls;
-        hw |= out_of_polls;
+        hw = __builtin_amdgcn_readfirstlane(hw_lanes) | out_of_polls;
     }
     __device__ __forceinline__ void sync()
     {

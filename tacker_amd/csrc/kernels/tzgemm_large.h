@@ -290,4 +290,258 @@ __device__ __forceinline__ void tzgemm_role_large(const _Float16 *__restrict__ A
     sync.finish();
 }
 
+// ---------------------------------------------------------------------------------------
+// The large-tile form for a wave-split fused kernel of 512 threads.  Two waves share a SIMD there
+// (one of the GEMM, one of the other role), so a lane has 256 registers and the tile is
+// 256 x 128: a wave tile of 128 x 64 = 8 x 4 accumulator tiles, 128 registers.  Same ring, same
+// loads, same LDS layout and the same bits as tzgemm_role_large (every element still sees its
+// chunks of 32 k in ascending order).  What differs is how the fragments are held: two register
+// sets of 8 + 4 fragments (96 registers) do not fit beside the accumulators, so there is ONE
+// set, and the 32 MFMAs of a chunk run in an order that lets every fragment be replaced as soon
+// as it is dead.  The order is two blocks of 4 rows of accumulator tiles, column by column
+// within a block:  MFMA n multiplies A fragment i = 4 (n / 16) + n % 4 with B fragment
+// j = n % 16 / 4.  Then
+//    A0..A3 are dead after MFMAs 12..15,  B0, B1, B2 after 19, 23, 27,
+//    A4..A7 after 28..31,                 B3 after 31,
+// and the next chunk needs A0..A3 and B0 from its MFMA 0 on, B1 from 4, B2 from 8, B3 from 12
+// and A4..A7 from 16.  So an iteration reads the next chunk's A0..A3, B0, B1, B2 behind its
+// own MFMAs 12, 14, 16, 18, 20, 23, 27 -- each at least 12 MFMAs before its first use -- and its
+// OWN B3, A4..A7 behind its MFMAs 0, 2, 4, 6, 7.  In a pair's second iteration the own-chunk
+// reads lie in front of the barrier (they read the buffer that is about to be refilled) and the
+// next-chunk reads and the 12 LDS-direct loads of the pair after next behind it, one memory
+// instruction per MFMA at most.
+// Against the 128 x 128 form of the fused kernels a workgroup moves 3/4 of the operand bytes per
+// flop through the CU's vector-memory path, and a 4096 x 4096 GEMM has its operands fetched 3
+// times over the 8 XCDs instead of 4.5 times.
+template <class Sync>
+__device__ __forceinline__ void tzgemm_role_large_rot(const _Float16 *__restrict__ A, const _Float16 *__restrict__ B,
+                                                      float *__restrict__ C, int M, int N, int K, int role_block,
+                                                      int role_blocks, int tile_start, int tile_end, int tid,
+                                                      char *lds, bool stream_c, Sync &sync)
+{
+    typedef __attribute__((address_space(3))) void *lptr_t;
+    constexpr int FM = 8, FN = 4;
+    constexpr int TM = 32 * FM, TN = 32 * FN;      // 256 x 128
+    constexpr int BK = 32;
+    constexpr int ROWB = 4 * BK;
+    constexpr int A_BYTES = TM * ROWB;
+    constexpr int B_BYTES = TN * ROWB;
+    constexpr int PAIR_BYTES = A_BYTES + B_BYTES;  // 48 KiB a buffer
+    // The ring in LDS: A of buffer 0, A of buffer 1, B of buffer 0, B of buffer 1.  With the two
+    // buffers of an operand next to each other every fragment read is "one of four lane addresses
+    // (operand, half) + an immediate below 64 KiB", and four address registers serve the loop.
+    constexpr int B_BASE = 2 * A_BYTES;
+    constexpr int LA = TM / 8 / 4;                 // 8 loads of A ...
+    constexpr int LB = TN / 8 / 4;                 // ... and 4 of B per wave and pair
+    constexpr int L = LA + LB;
+    constexpr int NM = FM * FN;                    // 32 MFMAs an iteration
+    constexpr int FIRST = 8;                       // MFMAs of a pair's second iteration in front of the barrier
+    static_assert(2 * PAIR_BYTES <= TZ_LDS_BYTES, "the ring is two buffers");
+
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave >> 1;
+    const int wc = wave & 1;
+    const int ref_cols = N / TZ_REF_TILE;
+    const int tile_rows = M / TM;
+    const int tile_cols = N / TN;
+    const int n_tiles = tile_rows * tile_cols;
+    const int npairs = K / (2 * BK);
+
+    // LDS-direct load q of an operand fills rows 8 (4 q + wave) .. + 7 of its area (tzgemm_role_large);
+    // here the row block 32 q is part of the wave-uniform base (scalar arithmetic) and one lane offset
+    // serves every load
+    const unsigned src_lane = (unsigned)(((lane >> 3) + 8 * wave) * K + (((lane & 7) ^ ((lane >> 4) | ((wave & 1) << 2))) * 8)) * 2u;
+    const size_t block_stride = (size_t)64 * (size_t)K;   // bytes between the rows of loads q and q + 1
+    const unsigned lds_dst = (unsigned)(size_t)(lptr_t)lds + wave * 1024;
+    const int frag_row = (lane & 15) * ROWB;
+    const int frag_h0 = frag_row + (((lane >> 4) ^ ((lane & 15) >> 1)) * 16);
+    const int frag_h1 = frag_row + (((4 + (lane >> 4)) ^ ((lane & 15) >> 1)) * 16);
+    const int off_a = wr * (FM * 16) * ROWB;
+    const int off_b = B_BASE + wc * (FN * 16) * ROWB;
+
+    for (int t = role_block; t < n_tiles; t += role_blocks) {
+        int mi, mj;
+        tz_large_tile_of(t, tile_rows, tile_cols, mi, mj);
+        const int ref_r0 = mi * (TM / TZ_REF_TILE) + wr * (FM / 4);
+        const int ref_c0 = mj * (TN / TZ_REF_TILE) + wc * (FN / 4);
+        {
+            const int r_first = mi * (TM / TZ_REF_TILE), c_first = mj * (TN / TZ_REF_TILE);
+            bool any = false;
+            for (int r = 0; r < TM / TZ_REF_TILE; ++r) {
+                const int p0 = (r_first + r) * ref_cols + c_first;
+                any |= p0 < tile_end && p0 + TN / TZ_REF_TILE > tile_start;
+            }
+            if (!any) continue;   // uniform over the workgroup
+        }
+        const char *a_tile = reinterpret_cast<const char *>(A + (size_t)(mi * TM) * K);
+        const char *b_tile = reinterpret_cast<const char *>(B + (size_t)(mj * TN) * K);
+
+#define TZR_LOAD(q_, buf_)                                                                        \
+    {                                                                                             \
+        if ((q_) < LA)                                                                            \
+            tz_load_to_lds(a_next + (size_t)(q_) * block_stride, src_lane, lds_dst + (buf_) * A_BYTES + (q_) * 4096); \
+        else                                                                                      \
+            tz_load_to_lds(b_next + (size_t)((q_) - LA) * block_stride, src_lane,                 \
+                           lds_dst + B_BASE + (buf_) * B_BYTES + ((q_) - LA) * 4096);             \
+    }
+#define TZR_FRAG_A(buf_, frag_, i_) \
+    *reinterpret_cast<const half8_t *>(lds + off_a + (frag_) + (buf_) * A_BYTES + (i_) * 16 * ROWB)
+#define TZR_FRAG_B(buf_, frag_, j_) \
+    *reinterpret_cast<const half8_t *>(lds + off_b + (frag_) + (buf_) * B_BYTES + (j_) * 16 * ROWB)
+// MFMA n of an iteration: accumulator tile (4 (n / 16) + n % 4, n % 16 / 4)
+#define TZR_MFMA(n_)                                                                              \
+    {                                                                                             \
+        constexpr int i_ = 4 * ((n_) / 16) + (n_) % 4, j_ = ((n_) % 16) / 4;                      \
+        acc[i_][j_] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j_], fa[i_], acc[i_][j_], 0, 0, 0); \
+    }
+// reads of the chunk that is being multiplied (half frag_ of buffer buf_): B3 and A4..A7, behind MFMA n_
+#define TZR_OWN_READS(n_, buf_, frag_)                                                            \
+    {                                                                                             \
+        if ((n_) == 0) fb[3] = TZR_FRAG_B(buf_, frag_, 3);                                        \
+        if ((n_) == 2) fa[4] = TZR_FRAG_A(buf_, frag_, 4);                                        \
+        if ((n_) == 4) fa[5] = TZR_FRAG_A(buf_, frag_, 5);                                        \
+        if ((n_) == 6) fa[6] = TZR_FRAG_A(buf_, frag_, 6);                                        \
+        if ((n_) == 7) fa[7] = TZR_FRAG_A(buf_, frag_, 7);                                        \
+    }
+// reads of the next chunk (half frag_ of buffer buf_): A0..A3, B0, B1, B2, behind MFMA n_
+#define TZR_NEXT_READS(n_, buf_, frag_)                                                           \
+    {                                                                                             \
+        if ((n_) == 12) fa[0] = TZR_FRAG_A(buf_, frag_, 0);                                       \
+        if ((n_) == 14) fa[1] = TZR_FRAG_A(buf_, frag_, 1);                                       \
+        if ((n_) == 16) fa[2] = TZR_FRAG_A(buf_, frag_, 2);                                       \
+        if ((n_) == 18) fa[3] = TZR_FRAG_A(buf_, frag_, 3);                                       \
+        if ((n_) == 20) fb[0] = TZR_FRAG_B(buf_, frag_, 0);                                       \
+        if ((n_) == 23) fb[1] = TZR_FRAG_B(buf_, frag_, 1);                                       \
+        if ((n_) == 27) fb[2] = TZR_FRAG_B(buf_, frag_, 2);                                       \
+    }
+// A pair's first iteration: its second chunk lies in the same buffer, published an iteration ago --
+// no wait and no barrier.
+#define TZR_ITERATION_FIRST(buf_)                                                                 \
+    {                                                                                             \
+        _Pragma("unroll") for (int n = 0; n < NM; ++n)                                            \
+        {                                                                                         \
+            TZR_MFMA_AT(n)                                                                        \
+            TZR_OWN_READS(n, buf_, frag_h0)                                                       \
+            TZR_NEXT_READS(n, buf_, frag_h1)                                                      \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
+    }
+// A pair's second iteration: behind the first MFMAs wait for this wave's loads of the next pair
+// and for its own LDS reads, and meet the other waves -- the next pair is then whole in nbuf_ and
+// nobody reads buf_ any more; read the next pair's first fragments and, if do_issue_, start the
+// loads of the pair after that into buf_.
+#define TZR_ITERATION_SECOND(buf_, nbuf_, do_issue_)                                              \
+    {                                                                                             \
+        _Pragma("unroll") for (int n = 0; n < FIRST; ++n)                                         \
+        {                                                                                         \
+            TZR_MFMA_AT(n)                                                                        \
+            TZR_OWN_READS(n, buf_, frag_h1)                                                       \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(0));                                              \
+        sync.sync();                                                                              \
+        __builtin_amdgcn_sched_barrier(0);                                                        \
+        _Pragma("unroll") for (int n = FIRST; n < NM; ++n)                                        \
+        {                                                                                         \
+            TZR_MFMA_AT(n)                                                                        \
+            TZR_NEXT_READS(n, nbuf_, frag_h0)                                                     \
+            if (do_issue_) {                                                                      \
+                constexpr int slot_[L] = {9, 11, 13, 15, 17, 19, 21, 22, 25, 26, 29, 31};         \
+                _Pragma("unroll") for (int q = 0; q < L; ++q)                                     \
+                    if (n == slot_[q]) TZR_LOAD(q, buf_)                                          \
+            }                                                                                     \
+            __builtin_amdgcn_sched_barrier(0);                                                    \
+        }                                                                                         \
+        if (do_issue_) {                                                                          \
+            a_next += ROWB;                                                                       \
+            b_next += ROWB;                                                                       \
+        }                                                                                         \
+    }
+// (the loop variable of an unrolled loop is a constant the MFMA's tile indices are computed from)
+#define TZR_MFMA_AT(n_)                                                                           \
+    {                                                                                             \
+        const int i_ = 4 * ((n_) / 16) + (n_) % 4, j_ = ((n_) % 16) / 4;                          \
+        acc[i_][j_] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fb[j_], fa[i_], acc[i_][j_], 0, 0, 0); \
+    }
+
+        float4_t acc[FM][FN];
+#pragma unroll
+        for (int i = 0; i < FM; ++i)
+#pragma unroll
+            for (int j = 0; j < FN; ++j) acc[i][j] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+        // fill both buffers (npairs >= 2 always), publish pair 0, fetch what its first chunk does
+        // not read itself
+        const char *a_next = a_tile, *b_next = b_tile;
+        for (int b = 0; b < 2; ++b) {
+            _Pragma("unroll") for (int q = 0; q < L; ++q) TZR_LOAD(q, b)
+            a_next += ROWB;
+            b_next += ROWB;
+        }
+        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(L));
+        sync.sync();
+        half8_t fa[FM], fb[FN];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) fa[i] = TZR_FRAG_A(0, frag_h0, i);
+#pragma unroll
+        for (int j = 0; j < 3; ++j) fb[j] = TZR_FRAG_B(0, frag_h0, j);
+
+        for (int p = 0; p + 2 < npairs; p += 2) {
+            TZR_ITERATION_FIRST(0)
+            TZR_ITERATION_SECOND(0, 1, true)
+            TZR_ITERATION_FIRST(1)
+            TZR_ITERATION_SECOND(1, 0, true)
+        }
+        // the last two pairs: nothing left to fetch, and behind the last chunk nothing left to read
+        TZR_ITERATION_FIRST(0)
+        TZR_ITERATION_SECOND(0, 1, false)
+        TZR_ITERATION_FIRST(1)
+        _Pragma("unroll") for (int n = 0; n < NM; ++n)
+        {
+            TZR_MFMA_AT(n)
+            TZR_OWN_READS(n, 1, frag_h1)
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        sync.sync();   // every wave is done reading before the next tile refills the ring
+
+        // (the lane's share of the address is formed here, from the lane number read afresh: nothing of
+        // it is kept in registers across the K loop)
+        int lane_here;
+        asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_here));
+        float *c_lane = C + (size_t)(mi * TM + wr * (FM * 16) + (lane_here & 15)) * N + mj * TN + wc * (FN * 16) +
+                        (lane_here >> 4) * 4;
+#pragma unroll
+        for (int ri = 0; ri < FM / 4; ++ri)
+#pragma unroll
+            for (int rj = 0; rj < FN / 4; ++rj) {
+                const int pos = (ref_r0 + ri) * ref_cols + ref_c0 + rj;
+                if (pos < tile_start || pos >= tile_end) continue;   // uniform over the wave
+#pragma unroll
+                for (int i = 4 * ri; i < 4 * ri + 4; ++i)
+#pragma unroll
+                    for (int j = 4 * rj; j < 4 * rj + 4; ++j) {
+                        float4_t v = acc[i][j] * TZ_ALPHA;
+                        float4_t *c_at = reinterpret_cast<float4_t *>(c_lane + (size_t)(i * 16) * N + j * 16);
+                        if (stream_c) __builtin_nontemporal_store(v, c_at);   // uniform
+                        else *c_at = v;
+                        // one tile at a time: scaled, stored, its registers free again (left to itself the
+                        // compiler scales all 32 tiles first, and 128 more registers do not exist here)
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+            }
+        // (the stores stay in flight while the next tile starts, as in tzgemm_role_large)
+#undef TZR_LOAD
+#undef TZR_FRAG_A
+#undef TZR_FRAG_B
+#undef TZR_MFMA
+#undef TZR_MFMA_AT
+#undef TZR_OWN_READS
+#undef TZR_NEXT_READS
+#undef TZR_ITERATION_FIRST
+#undef TZR_ITERATION_SECOND
+    }
+    sync.finish();
+}
+
 }  // namespace tk

@@ -77,9 +77,12 @@ extern "C" __global__ __launch_bounds__({threads}) void {name}(
 WAVE_SPLIT_EXTRA = {"lbm": "<2>", "cutcp": "<true>"}
 
 
-def generate_wave_split(be, be_threads, tz_first=True):
-    """Wave-split fused kernel: 256 tzgemm threads + be_threads of ``be`` per workgroup."""
-    variant = f"wave_{be_threads}"
+def generate_wave_split(be, be_threads, tz_first=True, large=False):
+    """Wave-split fused kernel: 256 tzgemm threads + be_threads of ``be`` per workgroup.
+
+    large: the 512-thread form whose GEMM role takes 256 x 128 tiles (tzgemm_role_large_rot) for
+    the shapes they divide (tz_large_fused_fits) and the 128 x 128 form for every other shape."""
+    variant = f"wave_{be_threads}_large" if large else f"wave_{be_threads}"
     tz_threads = 256
     total = tz_threads + be_threads
     p_be, sig_be = signature(be, 0)
@@ -95,6 +98,14 @@ def generate_wave_split(be, be_threads, tz_first=True):
     be_call = ROLES[be]["call"].format(p=p_be, block="be_block", blocks="be_blocks",
                                        tid=f"(int)threadIdx.x - {be_lo}", threads=be_threads,
                                        waves=be_threads // 64, extra=WAVE_SPLIT_EXTRA.get(be, ""))
+    if large:
+        if be_threads != 256:
+            raise ValueError("the large-tile GEMM role needs the registers of a 512-thread workgroup")
+        tz_call = (f"if (tz_large_fused_fits({p_tz}NORMAL_M, {p_tz}NORMAL_N, {p_tz}NORMAL_K))\n"
+                   f"            tk::tzgemm_role_large_rot({p_tz}A, {p_tz}B, {p_tz}C, {p_tz}NORMAL_M, {p_tz}NORMAL_N, {p_tz}NORMAL_K, "
+                   f"(int)blockIdx.x, {p_tz}ptb_iter_block_step, {p_tz}ptb_start_block_pos, {p_tz}ptb_end_block_pos, "
+                   f"(int)threadIdx.x - {tz_lo}, tz_lds, {_stream_c(be)}, sync);\n"
+                   f"        else\n            " + tz_call)
     tz_cond = (f"threadIdx.x < {tz_threads}" if tz_first else f"threadIdx.x >= {be_threads}")
     name = mix_kernel_name(be, variant)
     unused = _void_unused(sig_be + sig_tz, tz_call + be_call + f"{p_be}ptb_iter_block_step")
@@ -114,7 +125,7 @@ extern "C" __global__ __launch_bounds__({total}) void {name}(
         // whenever it is ready and the {be} waves fill the slots it leaves.
         __builtin_amdgcn_s_setprio(TK_GEMM_WAVE_PRIORITY);
         // role barrier: an arrival counter in LDS while {be} waves run, the hardware barrier once they have ended
-        tk::RoleHandoverSync sync(tz_arrivals, {tz_threads // 64}, (int)threadIdx.x - {tz_lo} < 64, &tk_spin_fail);
+        tk::RoleHandoverSync sync(tz_arrivals, {tz_threads // 64}, (int)threadIdx.x - {tz_lo}, &tk_spin_fail);
         {tz_call}
     }} else {{
         // A GEMM that leaves at least half of the workgroups without a tile: the {be} blocks go
@@ -236,5 +247,7 @@ def generate_pair(be, candidates):
             yield generate_wg_split(be, cand[1], cand[2])
         elif cand[0] == "wave":
             yield generate_wave_split(be, cand[1])
+        elif cand[0] == "wave_large":
+            yield generate_wave_split(be, cand[1], large=True)
         else:
             raise ValueError(cand)

@@ -14,7 +14,8 @@ Two steps, because the GPU box and the build tree are different places:
     python profile_ratio.py --apply out.json            # rewrites defaults.json; then gen_run.py
 Method per (pair, K): GEMM 2048 x 2048 x K (1024 tiles, one 128x128 macro tile per CU).
 t_gemm = the GEMM's own kernel alone, t_be = the best-effort kernel alone (all N blocks).
-For nb on a ladder of block counts, earned(nb) = t_gemm + t_be * nb / N - t_fused(nb)
+For nb on a ladder of block counts (every launch carrying the next nb positions of the kernel, so that
+no launch finds its data left in the caches by the one before), earned(nb) = t_gemm + t_be * nb / N - t_fused(nb)
 is the time one fused launch saves over the two serial launches (the quantity TaskManager
 credits, src/TaskManager.cu:626-640); a count qualifies only if it earns at least min_gain
 (3 %) of those serial launches, so that a pair within the noise of breaking even is not fused; the ladder runs N/1024, N/512, ..., N/64 (from N/65536 for grids of
@@ -84,6 +85,21 @@ def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_
         e1.synchronize()
         return e0.elapsed_ms(e1) / launches * 1e3
 
+    class Cursor:
+        """the fused kernel carrying nb block positions a launch, every launch the next nb of the kernel's
+        range (as TaskManager's cursor does): launched over one range again and again, a kernel that streams
+        its data would find it in the caches and its slice would look cheaper than it is"""
+
+        def __init__(self, mix, nb, total):
+            self.mix, self.nb, self.total, self.lo = mix, nb, total, 0
+
+        def execute(self):
+            if self.lo + self.nb > self.total:
+                self.lo = 0
+            self.mix.set_range(self.lo, self.lo + self.nb, 0, TILES)
+            self.mix.execute()
+            self.lo += self.nb
+
     result = {"stretch": stretch, "min_gain": min_gain, "tiles": TILES, "device": ta.device_name(), "pairs": {}}
     for be_name in pairs:
         be = ta.create_kernel(be_name)
@@ -101,8 +117,7 @@ def measure(out_path, stretch, launches, pairs=PAIRS, k_ladder=K_LADDER, ladder_
             t_gemm = min(t_gemm, timed(tz))
             best = {"blocks": 0, "earned_us": 0.0, "fused_us": t0}
             for nb in ladder(be_total, ladder_points):
-                mix.set_range(0, nb, 0, TILES)
-                t = timed(mix)
+                t = timed(Cursor(mix, nb, be_total))
                 serial = t_gemm + be_us * nb / be_total
                 earned = serial - t
                 if t <= (1 + stretch) * t_gemm and earned >= min_gain * serial and earned > best["earned_us"]:
