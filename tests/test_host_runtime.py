@@ -768,10 +768,15 @@ def test_task_manager_fuses_when_budget_allows(fake, small_vgg):
 
 def test_task_manager_with_the_rodinia_kernels_and_their_pairs(fake, small_vgg):
     # nn rides with the layers, and the second stage fuses nn with pathfinder (src/Creator.cu:629-640: nn_path);
-    # a Rodinia kernel has no fused kernel with a Parboil one, which is refused where the reference exits
+    # a Rodinia kernel has no fused kernel with a Parboil one, which is refused where the reference exits.
+    # (kinfo's measured load ratio of nn is 0 at every K on this GPU -- a stream earns nothing beside a GEMM --
+    # so it is the calibration pass that lets it ride here: on the fake every timed region takes the same time,
+    # and a fused launch that takes no longer than the layer alone earns its whole best-effort share)
     fake.tk_fake_set_event_ms(0.01)
+    assert fake.tacker_qos_colocated_blocks(0, b"nn", 1024, 2048, 2560000) == 0
     tm = ta.TaskManager(small_vgg, "nn", "path", library=fake)
     tm.configure(warmup=1, profile=2, verbose=0, qos_budget_ms=50.0, guard_ms=4.0, queries=1)
+    tm.set_calibration(True, 0.10)
     fake.tk_fake_reset()
     rep = tm.run("aker", raw_stream=None, second_stage=True)
     keys = [l["key"] for l in launches(fake)]
