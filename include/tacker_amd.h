@@ -665,8 +665,11 @@ TK_API int tacker_task_manager_run(tacker_task_manager_t tm, int mode, tkStream_
  * be_task_finish_num, n co-located latencies, n solo latencies} */
 TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
 /* No counterpart in the reference (its hot loop, src/TaskManager.cu:586-640, fuses every mixable
- * kernel of every query): an LC kernel whose fused launch lost against "LC alone, then the BE
- * share alone" `limit` times in a row is launched alone for the rest of the run (Aker mode only).
+ * kernel of every query): the manager keeps, per LC kernel, the average of what its fused launches
+ * earned against "LC alone, then the BE share alone" (losses included; mean of the first 16
+ * launches, exponential average of that memory afterwards) and launches the kernel alone once it
+ * has `limit` fused launches behind it and that average is negative, with one more fused launch
+ * every 64 queries (Aker mode only).  A kernel that always loses is barred after `limit` launches.
  * Default 3; 0 restores the reference's behaviour. */
 TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int limit);
 /* No counterpart in the reference (it takes tiles x block_ratio(K) from kinfo,
@@ -677,6 +680,15 @@ TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int 
  * tacker_task_manager_calibrated_blocks copies the counts of the last run (one per LC kernel). */
 TK_API int tacker_task_manager_set_calibration(tacker_task_manager_t tm, int on, float max_stretch);
 TK_API int tacker_task_manager_calibrated_blocks(tacker_task_manager_t tm, int *out, int cap);
+/* No counterpart in the reference.  With query_stretch > 0 the calibration pass chooses for the
+ * query as a whole: per LC kernel at most one of the (count, form) options it timed, such that
+ * what the fused launches add to their kernels sums to at most query_stretch of the query's solo
+ * time and the earned time is the largest possible (max_stretch of
+ * tacker_task_manager_set_calibration then only bounds a single kernel).  A layer that earns
+ * little for the latency it adds leaves its share to one that earns more.  0 (default): the best
+ * count per kernel.  passes (default 3, at least 1): timed fused launches per option; the slices
+ * of the timed launches advance through the best-effort kernel as the co-located queries' do. */
+TK_API int tacker_task_manager_set_calibration_budget(tacker_task_manager_t tm, float query_stretch, int passes);
 /* The calibration pass can also choose, per LC kernel, among generated forms of the fused kernel:
  * `variants` is a comma-separated list of variant names ("default" = the form kinfo names for the
  * pair, e.g. "default,wave_256"); forms the pair was not generated in are skipped.  A short layer

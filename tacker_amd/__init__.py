@@ -180,6 +180,7 @@ def _declare(lib):
     lib.tacker_task_manager_set_calibration.argtypes = [vp, i, f]
     lib.tacker_task_manager_set_end_to_end.argtypes = [vp, i]
     lib.tacker_task_manager_calibrated_blocks.argtypes = [vp, vp, i]
+    lib.tacker_task_manager_set_calibration_budget.argtypes = [vp, f, i]
     lib.tacker_task_manager_set_calibration_variants.argtypes = [vp, cp]
     lib.tacker_task_manager_calibrated_variant.argtypes = [vp, i, cp, i]
     lib.tacker_task_manager_be_mix_ms.argtypes = [vp]
@@ -1150,6 +1151,11 @@ class TaskManager:
 
     def set_calibration(self, on=True, max_stretch=0.10):
         check(self.l.tacker_task_manager_set_calibration(self.h, 1 if on else 0, max_stretch), "set_calibration")
+
+    def set_calibration_budget(self, query_stretch=0.15, passes=3):
+        """calibration chooses per query: the fused launches may add ``query_stretch`` of the query's solo
+        time in total (0 = the best count per kernel); ``passes`` timed launches per option"""
+        check(self.l.tacker_task_manager_set_calibration_budget(self.h, query_stretch, passes), "set_calibration_budget")
 
     def set_calibration_variants(self, variants=("default", "wave_256")):
         """forms of the fused kernel the calibration pass tries per LC kernel ("default" = kinfo's)"""

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <chrono>
+#include <cmath>
 #include <cstdio>
 #include <unordered_map>
 
@@ -246,17 +247,23 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         calibrated_variant.assign(nk, "");
         std::vector<float> best_earned(nk, 0.0f);
         const int first = be_kernel1->gptbParams.ptb_start_block_pos;
+        // every fused launch that was timed and kept its kernel within the per-kernel limit
+        struct Option { int n; std::string form; float cost_ms, earned_ms; };
+        std::vector<std::vector<Option>> options(nk);
         std::vector<std::string> forms;
         for (const std::string &v : calibrate_variants)
             if (v.empty() || get_kernel_info("tzgemm_" + be_task1_name + "@" + v, "blocksize") != JSON_NOT_FOUND)
                 forms.push_back(v);
         if (forms.empty()) forms.push_back("");
+        // the slices move through the best-effort kernel as they will in the co-located queries:
+        // a slice that was launched a moment ago is served from the caches and looks cheaper
+        int cal_cursor = first;
         for (const std::string &form : forms) {
             std::vector<bool> over(nk, false);   // a smaller count already stretched this kernel too far
             for (int divisor = 256; divisor >= 1; divisor /= 2) {
                 const int n = std::max(1, be_total / divisor);
                 std::vector<float> fused_ms(nk, 0.0f);
-                const int timed = 3;
+                const int timed = std::max(calibrate_passes, 1);
                 for (int pass = -1; pass < timed; ++pass) {   // pass -1 warms up
                     lc_task->initExecution();
                     for (size_t idx = 0; idx < nk; ++idx) {
@@ -265,8 +272,11 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
                             lc_kernel->execute(stream);
                             continue;
                         }
+                        if (cal_cursor + n > be_total) cal_cursor = first;
+                        const int from = cal_cursor, to = std::min(cal_cursor + n, be_total);
+                        cal_cursor = to;
                         watch.start(stream);
-                        launch_mixed(lc_kernel, first, std::min(first + n, be_total), form);
+                        launch_mixed(lc_kernel, from, to, form);
                         const float ms = watch.stop(stream);
                         if (pass >= 0) fused_ms[idx] += ms / timed;
                     }
@@ -279,12 +289,53 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
                         continue;
                     }
                     const float earned = alone + report.be1_solo_ms * n / be_total - fused_ms[idx];
+                    if (earned > 0.0f)
+                        options[idx].push_back({n, form, std::max(fused_ms[idx] - alone, 0.0f), earned});
                     if (earned > best_earned[idx]) {
                         best_earned[idx] = earned;
                         calibrated_blocks[idx] = n;
                         calibrated_variant[idx] = form;
                     }
                 }
+            }
+        }
+        if (calibrate_query_stretch > 0.0f) {
+            // A budget for the whole query instead of the best count per kernel: the launches to
+            // fuse, one option per kernel at most, that earn most while the query grows by at most
+            // calibrate_query_stretch of its solo time.  A short layer that earns a microsecond for
+            // five of latency then leaves its share of the budget to a layer that earns four for one.
+            // Exact by dynamic programming over the budget in steps of a thousandth.
+            const int steps = 1000;
+            const float budget_ms = calibrate_query_stretch * report.lc_solo_ms;
+            std::vector<float> best(steps + 1, 0.0f);
+            std::vector<std::vector<int>> pick(nk, std::vector<int>(steps + 1, -1));
+            for (size_t idx = 0; idx < nk; ++idx) {
+                std::vector<float> next(best);
+                for (size_t o = 0; o < options[idx].size(); ++o) {
+                    const Option &opt = options[idx][o];
+                    const int c = budget_ms > 0.0f ? (int)std::ceil(opt.cost_ms / budget_ms * steps) : 0;
+                    for (int u = c; u <= steps; ++u)
+                        if (best[u - c] + opt.earned_ms > next[u]) {
+                            next[u] = best[u - c] + opt.earned_ms;
+                            pick[idx][u] = (int)o;
+                        }
+                }
+                best.swap(next);
+            }
+            int u = steps;
+            for (int idx = (int)nk - 1; idx >= 0; --idx) {
+                const int o = pick[idx][u];
+                calibrated_blocks[idx] = 0;
+                calibrated_variant[idx] = "";
+                best_earned[idx] = 0.0f;
+                if (o < 0) continue;
+                // pick[idx][u] was set while kernel idx was added on top of the state of the kernels
+                // before it: walk back through that state
+                const Option &opt = options[idx][(size_t)o];
+                calibrated_blocks[idx] = opt.n;
+                calibrated_variant[idx] = opt.form;
+                best_earned[idx] = opt.earned_ms;
+                u -= budget_ms > 0.0f ? (int)std::ceil(opt.cost_ms / budget_ms * steps) : 0;
             }
         }
         if (verbose)
@@ -298,7 +349,19 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     // co-located queries: a cursor walks the BE kernel's blocks across launches
     int be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;
     float qos_headroom = policy.qos_budget_ms;
-    std::vector<int> strikes(nk, 0);   // consecutive fused launches of kernel i that did not pay
+    // What kernel i's fused launches earned so far (serial launches - fused launch, losses included):
+    // the mean of the first 16, an exponential average with that memory afterwards.  A kernel is
+    // barred once it has fusion_strikes_limit launches behind it and that average is negative --
+    // a kernel that always loses after exactly that many launches, one that earns a little on
+    // average not for a single slow launch (a timed region of 10-20 us jitters by more than a
+    // short layer earns).
+    std::vector<float> earn_mean(nk, 0.0f);
+    std::vector<int> earn_samples(nk, 0);
+    const int earn_memory = 16;
+    auto is_barred = [&](size_t idx) {
+        return mode == ExecutionMode::Aker && fusion_strikes_limit > 0 && earn_samples[idx] >= fusion_strikes_limit &&
+               earn_mean[idx] < 0.0f;
+    };
     std::vector<int> carried(nk, 0);   // best-effort blocks kernel i's launch carried in the last query
     for (int q = 0; q < queries; ++q) {
         lc_task->initExecution();
@@ -306,10 +369,10 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         // a barred kernel gets one more chance every fusion_retry_period queries; kernel i takes
         // its chance in the queries congruent to i, so that the retries (each a launch expected
         // to lose) are spread over queries instead of piling up in one slow query
+        std::vector<bool> retry(nk, false);
         if (fusion_retry_period > 0 && q >= fusion_retry_period)
             for (size_t idx = 0; idx < nk; ++idx)
-                if (q % fusion_retry_period == (int)(idx % (size_t)fusion_retry_period))
-                    strikes[idx] = std::min(strikes[idx], std::max(fusion_strikes_limit - 1, 0));
+                retry[idx] = q % fusion_retry_period == (int)(idx % (size_t)fusion_retry_period);
         long long cd_block_num_executed = 0;
         report.mix_times = 0;
         report.time_earned_ms = 0.0f;
@@ -318,8 +381,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             Kernel *lc_kernel = lc_task->kernels[idx];
             int cd_block_num = 0;
             watch.start(stream);
-            const bool barred = mode == ExecutionMode::Aker && fusion_strikes_limit > 0 &&
-                                strikes[idx] >= fusion_strikes_limit;
+            const bool barred = is_barred(idx) && !retry[idx];
             const bool calibrated = !calibrated_blocks.empty();
             if (policy.mustRunSolo(qos_headroom, lc_headroom_vec[idx]) || lc_kernel->mixable == 0 || barred ||
                 (calibrated && calibrated_blocks[idx] == 0)) {
@@ -350,7 +412,11 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             const QosPolicy::Outcome o = QosPolicy::account(mixed, duration, lc_kernel_time_vec[idx],
                                                             report.be1_solo_ms, cd_block_num, be_total);
             qos_headroom -= o.charged_ms;
-            if (mixed) strikes[idx] = o.counted_as_mixed ? 0 : strikes[idx] + 1;
+            if (mixed) {
+                const float earned = lc_kernel_time_vec[idx] + report.be1_solo_ms * cd_block_num / be_total - duration;
+                const int weight = std::min(++earn_samples[idx], earn_memory);
+                earn_mean[idx] += (earned - earn_mean[idx]) / weight;
+            }
             if (o.counted_as_mixed) {
                 cd_block_num_executed += cd_block_num;
                 report.mix_times++;
@@ -421,8 +487,13 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     }
     report.qos_headroom_left_ms = qos_headroom;
     report.fusion_disabled = 0;
-    if (fusion_strikes_limit > 0)
-        for (int v : strikes) report.fusion_disabled += v >= fusion_strikes_limit;
+    for (size_t idx = 0; idx < nk; ++idx) report.fusion_disabled += is_barred(idx);
+    if (verbose)
+        for (size_t idx = 0; idx < nk; ++idx)
+            if (earn_samples[idx] > 0)
+                printf("[MIX] %s: %d fused launches, earning %f ms on average at the end%s\n",
+                       lc_task->kernels[idx]->kernelName.c_str(), earn_samples[idx], earn_mean[idx],
+                       is_barred(idx) ? " (barred)" : "");
     report.stage1_be_ms = report.be_blocks_executed * report.be1_solo_ms / std::max(be_total, 1);
     if (verbose) {
         printf("execed be blks: %lld, mix times: %d/%d, time earned: %f\n", report.be_blocks_executed,

@@ -98,8 +98,9 @@ public:
     int profile_queries = 10;
     int queries = 5;
     bool verbose = true;
-    // Not in the reference: an LC kernel whose fused launch lost against "LC alone, then the
-    // BE share alone" this many times in a row is launched alone from then on (Aker mode).
+    // Not in the reference: an LC kernel whose fused launches lose on average against "LC alone,
+    // then the BE share alone" is launched alone (Aker mode), judged once it has this many fused
+    // launches behind it; a kernel that always loses is barred after exactly that many.
     // The static load ratios are measured on GEMMs that fill the GPU; layers with few tiles
     // can still lose, and every lost fusion stretches the LC query for nothing.  0 = never
     // stop (the reference's behaviour).
@@ -116,6 +117,13 @@ public:
     bool calibrate_blocks = false;
     float calibrate_max_stretch = 0.10f;
     std::vector<int> calibrated_blocks;   // per LC kernel, filled by the last calibrated run
+    // > 0: the calibration pass chooses for the query as a whole -- per kernel at most one of the
+    // timed (count, form) options, such that the sum of what the fused launches add to their
+    // kernels stays within calibrate_query_stretch of the query's solo time and the earned time
+    // is the largest possible; calibrate_max_stretch then only bounds what a single kernel may
+    // be stretched by (and ends the ladder of counts for it).  0: the best count per kernel.
+    float calibrate_query_stretch = 0.0f;
+    int calibrate_passes = 3;             // timed fused launches per (kernel, count, form)
     // Forms of the fused kernel the calibration pass tries for every LC kernel ("" = the one kinfo
     // names for the pair); it keeps, per LC kernel, the form and count that earned most.  A short
     // layer can do better in a form with fewer best-effort waves per workgroup: the launch of a

@@ -1569,6 +1569,15 @@ int tacker_task_manager_set_calibration(tacker_task_manager_t h, int on, float m
     return TK_SUCCESS;
 }
 
+int tacker_task_manager_set_calibration_budget(tacker_task_manager_t h, float query_stretch, int passes)
+{
+    TaskManager *tm = static_cast<TaskManager *>(h);
+    if (!tm || query_stretch < 0.0f || passes < 1) return fail(TK_ERROR_INVALID_VALUE, "bad task manager, stretch or passes");
+    tm->calibrate_query_stretch = query_stretch;
+    tm->calibrate_passes = passes;
+    return TK_SUCCESS;
+}
+
 int tacker_task_manager_set_calibration_variants(tacker_task_manager_t h, const char *variants)
 {
     TaskManager *tm = static_cast<TaskManager *>(h);

@@ -861,14 +861,19 @@ def test_task_manager_calibrates_block_counts_per_kernel(fake, small_vgg):
     # 9 block counts (1/256 ... 1) x (1 warm-up + 3 timed) passes of 16 fused launches, then 2 queries
     fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
     assert len(fused) == 9 * 4 * 16 + 2 * 16
-    ends = sorted({as_int(l["args"][15]) for l in fused[:9 * 4 * 16]})           # stencil ptb_end of the sweeps
-    assert ends == [32, 64, 128, 256, 512, 1024, 2048, 4096, 8192]
+    # the slices of the timed launches: 1/256 ... 1 of the kernel, each starting where the one before it ended
+    # (from the front again when the next would not fit), as the cursor of the co-located queries moves
+    sweeps = fused[:9 * 4 * 16]
+    spans = [(as_int(l["args"][13]), as_int(l["args"][15])) for l in sweeps]
+    assert sorted({e - b for b, e in spans}) == [32, 64, 128, 256, 512, 1024, 2048, 4096, 8192]
+    assert all(b2 == e1 or b2 == 0 for (_, e1), (b2, _) in zip(spans, spans[1:]))
+    assert len({b for b, e in spans if e - b == 32}) == 4 * 16                   # 64 different slices of 32
     # LC kernels alone take 10 us, every fused launch 12 us: 20 % over a 10 % allowance -> nothing is co-located
     cheap = [0.01] * (n * 2 + 1)
-    arr = (C.c_float * len(cheap))(*cheap)
+    arr, arr_len = (C.c_float * len(cheap))(*cheap), len(cheap)
     fake.tk_fake_reset()
     fake.tk_fake_set_event_ms(0.012)
-    fake.tk_fake_push_event_ms(arr, len(cheap))
+    fake.tk_fake_push_event_ms(arr, arr_len)
     rep = tm.run("aker", raw_stream=None, second_stage=False)
     assert tm.calibrated_blocks() == [0] * n and rep["mix_times"] == 0 and rep["be_blocks_executed"] == 0
     fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
@@ -876,9 +881,28 @@ def test_task_manager_calibrates_block_counts_per_kernel(fake, small_vgg):
     # 5 % over: allowed, and it pays from 1/16 of the kernel up (10 us * n/N > 0.5 us) -> again the whole kernel
     fake.tk_fake_reset()
     fake.tk_fake_set_event_ms(0.0105)
-    fake.tk_fake_push_event_ms(arr, len(cheap))
+    fake.tk_fake_push_event_ms(arr, arr_len)
     tm.run("aker", raw_stream=None, second_stage=False)
     assert all(tm.calibrated_blocks()[i] == 8192 for i in mixable)
+    # a budget for the query: every fused launch adds 0.5 us to its kernel and earns up to 9.5 us; with room
+    # for 3.5 such additions in the query, 3 kernels carry the whole best-effort kernel and 13 run alone
+    tm.set_calibration_budget(3.5 * 0.0005 / (n * 0.01), 2)
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.0105)
+    fake.tk_fake_push_event_ms(arr, arr_len)
+    rep = tm.run("aker", raw_stream=None, second_stage=False)
+    assert sorted(tm.calibrated_blocks()[i] for i in mixable) == [0] * 13 + [8192] * 3
+    assert rep["mix_times"] == 3 and rep["be_blocks_executed"] == 3 * 8192
+    fused = [l for l in launches(fake) if l["key"].startswith("tzgemm_stencil")]
+    assert len(fused) == 9 * 3 * 16 + 2 * 3                                      # 1 warm-up + 2 timed passes now
+    # room for all of them: the budget changes nothing
+    tm.set_calibration_budget(1.0, 3)
+    fake.tk_fake_reset()
+    fake.tk_fake_set_event_ms(0.0105)
+    fake.tk_fake_push_event_ms(arr, arr_len)
+    tm.run("aker", raw_stream=None, second_stage=False)
+    assert all(tm.calibrated_blocks()[i] == 8192 for i in mixable)
+    tm.set_calibration_budget(0.0, 3)
     tm.set_calibration(False, 0.10)                                              # back to the kinfo table
     fake.tk_fake_reset()
     fake.tk_fake_set_event_ms(0.01)
