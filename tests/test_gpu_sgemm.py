@@ -167,3 +167,43 @@ def test_an_output_address_sgemm_has_used_serves_a_shared_reduction_tzgemm_after
     ta.gptb_sgemm(dev(A), dev(B), c_s)
     assert np.array_equal(bits(c_s), oracle.sgemm(A, B, C0).view(np.uint32))
     assert ta.spin_fail_flag() == 0
+
+
+def test_kernel_objects_of_both_kinds_on_one_output_address_in_any_launch_order():
+    # a tzgemm object built on C, an sgemm object built on the same C afterwards, then launches in the
+    # order sgemm (a range that ends inside the reduction: running sums stay in its workspace), the
+    # older tzgemm object (its arrival counters must still be zero), the rest of sgemm (its sums must
+    # still be there): each kernel has a workspace of its own under the one address
+    M, N, K = 256, 512, 4608
+    assert ta.tzgemm_parts(M, N, K) > 1
+    buf = torch.zeros(M * N, device="cuda:0")
+    gA, gB = gemm_inputs(M, N, K, 78)
+    dA, dB = dev(gA), dev(gB)
+    c_t = buf.view(M, N)
+    tz = ta.gptb_create(ta.ori_tzgemm_create(dA, dB, c_t), 0, 0, 0, (M // 64) * (N // 64))
+    A, B, C0 = inputs(256, 512, 600, seed=10)
+    sA, sB = dev(A), dev(B)
+    c_s = buf.view(512, 256)
+    assert c_t.data_ptr() == c_s.data_ptr()
+    positions = ta.sgemm_blocks(256, 512, 600)
+    sg = ta.gptb_create(ta.ori_sgemm_create(sA, sB, c_s), 0, 0, 0, positions)
+    other = torch.full((M, N), -7.0, device="cuda:0")
+    ta.gptb_tzgemm(dA, dB, other)
+    want_s = oracle.sgemm(A, B, C0).view(np.uint32)
+    cut = positions // 2 + 3
+    stash = torch.empty_like(c_s)
+    for _ in range(2):                       # twice: whatever a round leaves behind serves the next
+        c_s.copy_(dev(C0))
+        sg.set_range(0, cut)
+        sg.execute()
+        stash.copy_(c_s)                     # sgemm's C so far (the tiles its range has finished)
+        c_t.fill_(-7.0)
+        tz.execute()
+        assert np.array_equal(host(c_t), host(other))
+        c_s.copy_(stash)
+        sg.set_range(cut, positions)
+        sg.execute()
+        assert np.array_equal(bits(c_s), want_s)
+    assert ta.spin_fail_flag() == 0
+    sg.close()
+    tz.close()
