@@ -30,11 +30,6 @@ typedef unsigned uint4_t __attribute__((ext_vector_type(4)));
 // deliberately left in flight -- the GEMM role keeps several chunks of
 // LDS-direct loads outstanding across its barriers and tracks them itself.
 struct WorkgroupSync {
-    // arrive() and wait() are the two halves of a barrier for code that can do useful
-    // work between "I am done" and "is everybody done"; the hardware barrier has no
-    // such split, so all of it happens in wait().
-    static constexpr bool kSplit = false;
-    __device__ __forceinline__ void arrive() {}
     __device__ __forceinline__ void wait()
     {
         __builtin_amdgcn_s_barrier();
@@ -48,92 +43,14 @@ struct WorkgroupSync {
     __device__ __forceinline__ void finish() {}
 };
 
-// Barrier among the waves of ONE role inside a workgroup that also hosts
-// another role (wave-split fused kernels).  gfx950 has a single hardware
-// barrier per workgroup and no named barriers, so a role-local barrier is an
-// LDS arrival counter: lane 0 of each wave adds 1, everybody polls until the
-// count reaches the number of arrivals expected so far.  All waves of a
-// workgroup are resident at the same time, so polling cannot starve a wave that
-// has yet to arrive.  The poll is bounded: after spin_limit polls the wave gives
-// up, raises *fail (a global word the host checks) and carries on, so a logic
-// error ends in a wrong answer plus a flag, never in waves that do not finish.
-struct RoleSpinSync {
-    static constexpr bool kSplit = true;
-    unsigned counter_addr;   // LDS byte address of the arrival counter (zero when the role starts)
-    unsigned waves;          // waves taking part
-    unsigned expected;       // arrivals that complete the current barrier
-    unsigned gave_up;        // nonzero once a poll ran into the limit
-    unsigned *fail;          // global flag, may be nullptr
-    unsigned spin_limit;
-    __device__ __forceinline__ RoleSpinSync(unsigned *c, unsigned w, unsigned *f,
-                                            unsigned limit = (1u << 24))
-        : counter_addr((unsigned)(size_t)(__attribute__((address_space(3))) unsigned *)c), waves(w),
-          expected(0), gave_up(0), fail(f), spin_limit(limit) {}
-
-    // Both halves are single asm blocks on purpose.  Written as C++ (an if for lane 0, a
-    // while for the poll) they put branches and a loop inside the caller's K loop, and the
-    // compiler's wait-count bookkeeping then loses track of the LDS-direct loads in flight
-    // and waits for all of them (vmcnt(0)) before the next LDS read -- which serialises the
-    // load ring.  As opaque blocks they leave the K loop a single basic block.
-
-    // "This wave is done with what the barrier protects."  The caller has already waited
-    // for its own LDS reads (lgkmcnt) and LDS-direct loads (vmcnt) as far as it needs.
-    __device__ __forceinline__ void arrive()
-    {
-        expected += waves;
-        unsigned long long saved_exec;
-        asm volatile("s_mov_b64 %0, exec\n\t"
-                     "s_mov_b64 exec, 1\n\t"
-                     "ds_add_u32 %1, %2\n\t"
-                     "s_mov_b64 exec, %0"
-                     : "=&s"(saved_exec)
-                     : "v"(counter_addr), "v"(1u)
-                     : "memory");
-    }
-    // Block until every wave of the role has arrived.  Work placed between arrive() and
-    // wait() hides the LDS round trip of the counter; the poll has no sleep in it because
-    // the other waves are at most a few hundred cycles behind.  The poll is bounded.
-    // seen: a value of the counter read after arrive() (the caller overlaps that read with
-    // its own work and hands the result in); a value from before the last arrival just polls.
-    __device__ __forceinline__ void wait(unsigned seen)
-    {
-        if ((int)(seen - expected) < 0) wait();
-    }
-    __device__ __forceinline__ void wait()
-    {
-        {
-            unsigned now, left;
-            asm volatile("s_mov_b32 %1, %4\n"
-                         "1:\n\t"
-                         "ds_read_b32 %0, %2\n\t"
-                         "s_waitcnt lgkmcnt(0)\n\t"
-                         "v_sub_u32 %0, %0, %3\n\t"
-                         "v_cmp_gt_i32 vcc, 0, %0\n\t"
-                         "s_cbranch_vccz 2f\n\t"
-                         "s_sub_u32 %1, %1, 1\n\t"
-                         "s_cmp_lg_u32 %1, 0\n\t"
-                         "s_cbranch_scc1 1b\n"
-                         "2:"
-                         : "=&v"(now), "=&s"(left)
-                         : "v"(counter_addr), "v"(expected), "s"(spin_limit)
-                         : "vcc", "scc", "memory");
-            gave_up |= (left == 0u);
-        }
-    }
-    __device__ __forceinline__ void sync()
-    {
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // LDS reads/writes of this wave are done
-        arrive();
-        wait();
-    }
-    // once, when the role is over: tell the host if any barrier was abandoned
-    __device__ __forceinline__ void finish()
-    {
-        if (gave_up && fail) __hip_atomic_fetch_or(fail, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-};
-
-// RoleSpinSync that hands over to the hardware barrier once the waves of the other role have ended.
+// Barrier among the waves of ONE role inside a workgroup that also hosts another role (wave-split
+// fused kernels).  gfx950 has a single hardware barrier per workgroup and no named barriers, so a
+// role-local barrier is an LDS arrival counter: lane 0 of each wave adds 1, everybody polls until
+// the count reaches the number of arrivals expected so far.  All waves of a workgroup are resident
+// at the same time, so polling cannot starve a wave that has yet to arrive.  The poll is bounded:
+// after spin_limit polls the wave gives up, raises *fail (a global word the host checks) and
+// carries on, so a logic error ends in a wrong answer plus a flag, never in waves that do not
+// finish.  The counter hands over to the hardware barrier once the waves of the other role have ended:
 //
 // The hardware barrier counts the waves of the workgroup that have not terminated.  While waves of
 // the other role run it cannot serve one role; once they have all ended it serves the waves that are
@@ -149,7 +66,6 @@ struct RoleSpinSync {
 // whose poll runs into its limit changes over too (and raises the failure word): from then on it can
 // only hold the others up at the hardware barrier until they give up as well, never spin on.
 struct RoleHandoverSync {
-    static constexpr bool kSplit = false;   // wait() is the whole barrier
     unsigned counter_addr;   // LDS byte address of the three words
     unsigned waves;
     unsigned expected;       // arrivals that complete the current barrier = its index
@@ -176,7 +92,6 @@ struct RoleHandoverSync {
         words[2] = 0x7fffffffu;
     }
 
-    __device__ __forceinline__ void arrive() {}
     // The hardware barrier is the path the K loop falls through; the counter's code sits out of its
     // way.  (Every instruction at the barrier is a gap in the wave's MFMA stream: with the change-over
     // test and the counter's code in line the loop ran 12 % slower than with the bare s_barrier.)

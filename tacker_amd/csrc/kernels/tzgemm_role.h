@@ -212,85 +212,31 @@ __device__ __forceinline__ void tzgemm_role_tiles(const _Float16 *__restrict__ A
 // the CU's vector-memory unit takes about 10 ns per load, a wave blocks at issue while the
 // unit's queue is full, and 32 loads issued right behind the barrier by the four waves at
 // once would stall the MFMAs queued behind them.
-// With a split barrier the wave announces itself after 12 of the 16 MFMAs (its reads of the
-// stage have landed by then); the last 4 and the first 8 MFMAs of the second k-step, which
-// need nothing from behind the barrier, hide the round trip of the arrival counter.
 #define TZ_FIRST_STEP_ACROSS_BARRIER(fa_, fb_, fn_, fbn_, vmcnt_, tail_chunk_, tail_stage_)       \
-    if constexpr (Sync::kSplit) {                                                                 \
-        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
-        TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
+    TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                                 \
+    TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    _Pragma("unroll") for (int q = 0; q < 8; ++q)                                                 \
+    {                                                                                             \
+        TZ_MFMA_AT(fa_, fb_, 8 + q)                                                               \
+        if ((q & 1) == 0 && (tail_chunk_) >= 0) TZ_LOOP_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q / 2) \
         __builtin_amdgcn_sched_barrier(0);                                                        \
-        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
-        {                                                                                         \
-            TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
-            if ((tail_chunk_) >= 0) TZ_LOOP_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q)            \
-            __builtin_amdgcn_sched_barrier(0);                                                    \
-        }                                                                                         \
-        __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
-        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
-        sync.arrive();                                                                            \
-        __builtin_amdgcn_sched_barrier(0);                                                        \
-        TZ_MFMAS_ROWS(fa_, fb_, 3, 4)                                                             \
-        TZ_MFMAS_ROWS(fn_, fbn_, 0, 1)                                                            \
-        __builtin_amdgcn_sched_barrier(0);                                                        \
-        {   /* counter read + 4 MFMAs + wait for the read, as one block: the compiler must */     \
-            /* not touch the destination register of the read while it is in flight       */     \
-            unsigned seen_;                                                                       \
-            asm volatile("ds_read_b32 %0, %5\n\t"                                                 \
-                         "v_mfma_f32_16x16x32_f16 %1, %6, %10, %1\n\t"                            \
-                         "v_mfma_f32_16x16x32_f16 %2, %7, %10, %2\n\t"                            \
-                         "v_mfma_f32_16x16x32_f16 %3, %8, %10, %3\n\t"                            \
-                         "v_mfma_f32_16x16x32_f16 %4, %9, %10, %4\n\t"                            \
-                         "s_waitcnt lgkmcnt(0)"                                                   \
-                         : "=&v"(seen_), "+v"(acc[1][0]), "+v"(acc[1][1]), "+v"(acc[1][2]),       \
-                           "+v"(acc[1][3])                                                        \
-                         : "v"(sync.counter_addr), "v"(fbn_[0]), "v"(fbn_[1]), "v"(fbn_[2]),      \
-                           "v"(fbn_[3]), "v"(fn_[1])                                              \
-                         : "memory");                                                             \
-            sync.wait(seen_);                                                                     \
-        }                                                                                         \
-    } else {                                                                                      \
-        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
-        TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
-        __builtin_amdgcn_sched_barrier(0);                                                        \
-        _Pragma("unroll") for (int q = 0; q < 8; ++q)                                             \
-        {                                                                                         \
-            TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
-            if ((q & 1) == 0 && (tail_chunk_) >= 0) TZ_LOOP_ISSUE_ONE(tail_chunk_, tail_stage_, 4 + q / 2) \
-            __builtin_amdgcn_sched_barrier(0);                                                    \
-        }                                                                                         \
-        __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                              \
-        __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                         \
-        sync.wait();                                                                              \
-    }
+    }                                                                                             \
+    __builtin_amdgcn_s_waitcnt(TK_LGKMCNT0_IMM);                                                  \
+    __builtin_amdgcn_s_waitcnt(TK_VMCNT_IMM(vmcnt_));                                             \
+    sync.wait();
 // Second k-step (what is left of it): the 8 reads of the next chunk's first k-step ride
 // between its first MFMAs and, if chunk_ >= 0, loads 0..3 of a new chunk follow; its loads
 // 4..7 go out with the next first k-step.
 #define TZ_SECOND_STEP(fa_, fb_, chunk_, stage_)                                                  \
-    if constexpr (Sync::kSplit) {                                                                 \
-        TZ_MFMAS_ROWS(fa_, fb_, 2, 3)                                                             \
-        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
-        {                                                                                         \
-            __builtin_amdgcn_sched_group_barrier(TZ_SCHED_DS_READ, 2, 0);                         \
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                    \
-        }                                                                                         \
+    TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                                 \
+    TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                        \
+    __builtin_amdgcn_sched_barrier(0);                                                            \
+    _Pragma("unroll") for (int q = 0; q < 8; ++q)                                                 \
+    {                                                                                             \
+        TZ_MFMA_AT(fa_, fb_, 8 + q)                                                               \
+        if ((q & 1) == 0 && (chunk_) >= 0) TZ_LOOP_ISSUE_ONE(chunk_, stage_, q / 2)               \
         __builtin_amdgcn_sched_barrier(0);                                                        \
-        _Pragma("unroll") for (int q = 0; q < 4; ++q)                                             \
-        {                                                                                         \
-            TZ_MFMA_AT(fa_, fb_, 12 + q)                                                          \
-            if ((chunk_) >= 0) TZ_LOOP_ISSUE_ONE(chunk_, stage_, q)                               \
-            __builtin_amdgcn_sched_barrier(0);                                                    \
-        }                                                                                         \
-    } else {                                                                                      \
-        TZ_MFMAS_ROWS(fa_, fb_, 0, 2)                                                             \
-        TZ_PAIR_MFMA_WITH(TZ_SCHED_DS_READ, 8)                                                    \
-        __builtin_amdgcn_sched_barrier(0);                                                        \
-        _Pragma("unroll") for (int q = 0; q < 8; ++q)                                             \
-        {                                                                                         \
-            TZ_MFMA_AT(fa_, fb_, 8 + q)                                                           \
-            if ((q & 1) == 0 && (chunk_) >= 0) TZ_LOOP_ISSUE_ONE(chunk_, stage_, q / 2)           \
-            __builtin_amdgcn_sched_barrier(0);                                                    \
-        }                                                                                         \
     }
 
         float4_t acc[4][4];
