@@ -665,12 +665,9 @@ TK_API int tacker_task_manager_run(tacker_task_manager_t tm, int mode, tkStream_
  * be_task_finish_num, n co-located latencies, n solo latencies} */
 TK_API int tacker_task_manager_report(tacker_task_manager_t tm, float out[13]);
 /* No counterpart in the reference (its hot loop, src/TaskManager.cu:586-640, fuses every mixable
- * kernel of every query): the manager keeps, per LC kernel, the average of what its fused launches
- * earned against "LC alone, then the BE share alone" (losses included; mean of the first 16
- * launches, exponential average of that memory afterwards) and launches the kernel alone once it
- * has `limit` fused launches behind it and that average is negative, with one more fused launch
- * every 64 queries (Aker mode only).  A kernel that always loses is barred after `limit` launches.
- * Default 3; 0 restores the reference's behaviour. */
+ * kernel of every query): an LC kernel whose fused launch lost against "LC alone, then the BE
+ * share alone" `limit` times in a row is launched alone from then on, with one more fused launch
+ * every 64 queries (Aker mode only).  Default 3; 0 restores the reference's behaviour. */
 TK_API int tacker_task_manager_set_fusion_strikes(tacker_task_manager_t tm, int limit);
 /* No counterpart in the reference (it takes tiles x block_ratio(K) from kinfo,
  * src/TaskManager.cu:593-600): with on != 0 an Aker-mode run first times, for every mixable LC

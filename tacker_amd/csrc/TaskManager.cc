@@ -349,19 +349,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     // co-located queries: a cursor walks the BE kernel's blocks across launches
     int be_cursor = be_kernel1->gptbParams.ptb_start_block_pos;
     float qos_headroom = policy.qos_budget_ms;
-    // What kernel i's fused launches earned so far (serial launches - fused launch, losses included):
-    // the mean of the first 16, an exponential average with that memory afterwards.  A kernel is
-    // barred once it has fusion_strikes_limit launches behind it and that average is negative --
-    // a kernel that always loses after exactly that many launches, one that earns a little on
-    // average not for a single slow launch (a timed region of 10-20 us jitters by more than a
-    // short layer earns).
-    std::vector<float> earn_mean(nk, 0.0f);
-    std::vector<int> earn_samples(nk, 0);
-    const int earn_memory = 16;
-    auto is_barred = [&](size_t idx) {
-        return mode == ExecutionMode::Aker && fusion_strikes_limit > 0 && earn_samples[idx] >= fusion_strikes_limit &&
-               earn_mean[idx] < 0.0f;
-    };
+    std::vector<int> strikes(nk, 0);   // consecutive fused launches of kernel i that did not pay
     std::vector<int> carried(nk, 0);   // best-effort blocks kernel i's launch carried in the last query
     for (int q = 0; q < queries; ++q) {
         lc_task->initExecution();
@@ -369,10 +357,10 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
         // a barred kernel gets one more chance every fusion_retry_period queries; kernel i takes
         // its chance in the queries congruent to i, so that the retries (each a launch expected
         // to lose) are spread over queries instead of piling up in one slow query
-        std::vector<bool> retry(nk, false);
         if (fusion_retry_period > 0 && q >= fusion_retry_period)
             for (size_t idx = 0; idx < nk; ++idx)
-                retry[idx] = q % fusion_retry_period == (int)(idx % (size_t)fusion_retry_period);
+                if (q % fusion_retry_period == (int)(idx % (size_t)fusion_retry_period))
+                    strikes[idx] = std::min(strikes[idx], std::max(fusion_strikes_limit - 1, 0));
         long long cd_block_num_executed = 0;
         report.mix_times = 0;
         report.time_earned_ms = 0.0f;
@@ -381,7 +369,8 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             Kernel *lc_kernel = lc_task->kernels[idx];
             int cd_block_num = 0;
             watch.start(stream);
-            const bool barred = is_barred(idx) && !retry[idx];
+            const bool barred = mode == ExecutionMode::Aker && fusion_strikes_limit > 0 &&
+                                strikes[idx] >= fusion_strikes_limit;
             const bool calibrated = !calibrated_blocks.empty();
             if (policy.mustRunSolo(qos_headroom, lc_headroom_vec[idx]) || lc_kernel->mixable == 0 || barred ||
                 (calibrated && calibrated_blocks[idx] == 0)) {
@@ -412,11 +401,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             const QosPolicy::Outcome o = QosPolicy::account(mixed, duration, lc_kernel_time_vec[idx],
                                                             report.be1_solo_ms, cd_block_num, be_total);
             qos_headroom -= o.charged_ms;
-            if (mixed) {
-                const float earned = lc_kernel_time_vec[idx] + report.be1_solo_ms * cd_block_num / be_total - duration;
-                const int weight = std::min(++earn_samples[idx], earn_memory);
-                earn_mean[idx] += (earned - earn_mean[idx]) / weight;
-            }
+            if (mixed) strikes[idx] = o.counted_as_mixed ? 0 : strikes[idx] + 1;
             if (o.counted_as_mixed) {
                 cd_block_num_executed += cd_block_num;
                 report.mix_times++;
@@ -487,13 +472,8 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
     }
     report.qos_headroom_left_ms = qos_headroom;
     report.fusion_disabled = 0;
-    for (size_t idx = 0; idx < nk; ++idx) report.fusion_disabled += is_barred(idx);
-    if (verbose)
-        for (size_t idx = 0; idx < nk; ++idx)
-            if (earn_samples[idx] > 0)
-                printf("[MIX] %s: %d fused launches, earning %f ms on average at the end%s\n",
-                       lc_task->kernels[idx]->kernelName.c_str(), earn_samples[idx], earn_mean[idx],
-                       is_barred(idx) ? " (barred)" : "");
+    if (fusion_strikes_limit > 0)
+        for (int v : strikes) report.fusion_disabled += v >= fusion_strikes_limit;
     report.stage1_be_ms = report.be_blocks_executed * report.be1_solo_ms / std::max(be_total, 1);
     if (verbose) {
         printf("execed be blks: %lld, mix times: %d/%d, time earned: %f\n", report.be_blocks_executed,

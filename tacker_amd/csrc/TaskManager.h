@@ -98,9 +98,8 @@ public:
     int profile_queries = 10;
     int queries = 5;
     bool verbose = true;
-    // Not in the reference: an LC kernel whose fused launches lose on average against "LC alone,
-    // then the BE share alone" is launched alone (Aker mode), judged once it has this many fused
-    // launches behind it; a kernel that always loses is barred after exactly that many.
+    // Not in the reference: an LC kernel whose fused launch lost against "LC alone, then the
+    // BE share alone" this many times in a row is launched alone from then on (Aker mode).
     // The static load ratios are measured on GEMMs that fill the GPU; layers with few tiles
     // can still lose, and every lost fusion stretches the LC query for nothing.  0 = never
     // stop (the reference's behaviour).
