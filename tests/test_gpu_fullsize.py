@@ -276,4 +276,24 @@ def test_config5_vgg16_224_colocated_queries_equal_the_solo_query():
     assert all(0 < v < 50.0 for v in tm.latencies())
     assert ta.spin_fail_flag() == 0
     tm.close()
+
+    # a budget for the whole query, both forms of the fused kernel, the stencil's large slices allowed:
+    # what the pass chooses stays inside the budget by its own figures, and the logits do not move
+    tm = ta.TaskManager(task, "stencil", "lbm")
+    tm.configure(qos_budget_ms=50.0, guard_ms=4.0, warmup=2, profile=20, queries=20, verbose=0)
+    tm.set_calibration(True, 1.5)
+    tm.set_calibration_budget(0.15, 2)
+    tm.set_calibration_variants(("default", "wave_256"))
+    tm.set_end_to_end(10)
+    rep = tm.run("aker", second_stage=False)
+    torch.cuda.synchronize()
+    blocks = tm.calibrated_blocks()
+    assert len(blocks) >= 16 and all(0 <= b <= 8192 for b in blocks)
+    assert all(v in ("", "wave_256") for v in tm.calibrated_variants())
+    assert np.array_equal(ta.device_to_host(p, (n, stride), np.float32)[:, 0], solo)
+    assert all(0 < v < 50.0 for v in tm.latencies())
+    solo_e2e = np.median(tm.latencies(kind="e2e_solo"))
+    assert np.median(tm.latencies(kind="e2e_colocated")) < 1.5 * solo_e2e
+    assert ta.spin_fail_flag() == 0
+    tm.close()
     task.close()
