@@ -26,7 +26,7 @@ MFMA_F16_PEAK = 2.5e15     # flop/s, dense fp16 MFMA
 # HBM-side bytes one fused launch moves, from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of this
 # file scaled by what the same counters read for a 64 MiB copy (x1.9988 and x1.0000); the summary with
 # the commands is profiles/pmc_hbm_traffic_bench_tzgemm2048_stencil512x512x64.txt
-FUSED_HBM_TRAFFIC_BYTES = 2.060e8
+FUSED_HBM_TRAFFIC_BYTES = 2.044e8
 
 GEMM_MNK = (2048, 2048, 2048)
 STENCIL_DIMS = (64, 512, 512)      # nz, ny, nx
