@@ -307,13 +307,18 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
             // Exact by dynamic programming over the budget in steps of a thousandth.
             const int steps = 1000;
             const float budget_ms = calibrate_query_stretch * report.lc_solo_ms;
+            // an option's cost in steps of the budget (steps + 1: does not fit)
+            auto cost_steps = [&](const Option &opt) {
+                if (budget_ms <= 0.0f) return opt.cost_ms > 0.0f ? steps + 1 : 0;
+                return (int)std::min(std::ceil(opt.cost_ms / budget_ms * steps), (float)(steps + 1));
+            };
             std::vector<float> best(steps + 1, 0.0f);
             std::vector<std::vector<int>> pick(nk, std::vector<int>(steps + 1, -1));
             for (size_t idx = 0; idx < nk; ++idx) {
                 std::vector<float> next(best);
                 for (size_t o = 0; o < options[idx].size(); ++o) {
                     const Option &opt = options[idx][o];
-                    const int c = budget_ms > 0.0f ? (int)std::ceil(opt.cost_ms / budget_ms * steps) : 0;
+                    const int c = cost_steps(opt);
                     for (int u = c; u <= steps; ++u)
                         if (best[u - c] + opt.earned_ms > next[u]) {
                             next[u] = best[u - c] + opt.earned_ms;
@@ -335,7 +340,7 @@ void TaskManager::run(ExecutionMode mode, cudaStream_t stream, bool with_second_
                 calibrated_blocks[idx] = opt.n;
                 calibrated_variant[idx] = opt.form;
                 best_earned[idx] = opt.earned_ms;
-                u -= budget_ms > 0.0f ? (int)std::ceil(opt.cost_ms / budget_ms * steps) : 0;
+                u -= cost_steps(opt);
             }
         }
         if (verbose)
