@@ -187,62 +187,53 @@ __device__ __forceinline__ void lbm_cell_pair(const float *__restrict__ src, flo
 #undef TK_LBM_SCATTER2
 }
 
-// Two rows at once, for a role that has few waves on its CU (inside a fused kernel): all 40
-// loads of both rows are issued before the first collision, so a wave has twice the bytes in
-// flight.  Each destination word has one writer whichever rows are paired, so the result is
-// the same as row by row.
-__device__ __forceinline__ void lbm_cell_pair_x2(const float *__restrict__ src, float *__restrict__ dst,
-                                                 int cells, int ca, int cb, int sx, int sxy)
+// N rows at once, for a role that has few waves on its CU (inside a fused kernel): all 20 N loads
+// of the rows are issued before the first collision, so a wave has N times the bytes in flight.
+// Each destination word has one writer whichever rows are taken together, so the result is the
+// same as row by row.
+template <int N>
+__device__ __forceinline__ void lbm_cell_pair_rows(const float *__restrict__ src, float *__restrict__ dst,
+                                                   int cells, const int (&c)[N], int sx, int sxy)
 {
-#define TK_LBM_LOAD(entry, dx, dy, dz, name)                                                          \
-    const lbm_pair_t name##_a = lbm_load_pair(src + cells * (entry) + ca);      \
-    const lbm_pair_t name##_b = lbm_load_pair(src + cells * (entry) + cb);
-    TK_LBM_DIRECTIONS(TK_LBM_LOAD)
+    lbm_pair_t in[N][20];
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+#define TK_LBM_LOAD(entry, dx, dy, dz, name) in[r][entry] = lbm_load_pair(src + cells * (entry) + c[r]);
+        TK_LBM_DIRECTIONS(TK_LBM_LOAD)
 #undef TK_LBM_LOAD
-    const lbm_pair_t flags_a = lbm_load_pair(src + cells * LBM_FLAGS + ca);
-    const lbm_pair_t flags_b = lbm_load_pair(src + cells * LBM_FLAGS + cb);
-#define TK_LBM_SCATTER_ROW(c_, entry, dx, dy, dz, v0_, v1_)                                \
+        in[r][LBM_FLAGS] = lbm_load_pair(src + cells * LBM_FLAGS + c[r]);
+    }
+    // a row is collided and scattered while the loads of the rows behind it are still on their way;
+    // the scheduling fences keep the rows' arithmetic apart (interleaved it needs more registers
+    // than a fused kernel has)
+#pragma unroll
+    for (int r = 0; r < N; ++r) {
+        __builtin_amdgcn_sched_barrier(0);
+#define TK_LBM_SPLIT(entry, dx, dy, dz, name) float name##0 = in[r][entry].x, name##1 = in[r][entry].y;
+        TK_LBM_DIRECTIONS(TK_LBM_SPLIT)
+#undef TK_LBM_SPLIT
+        lbm_collide(__float_as_uint(in[r][LBM_FLAGS].x), tempC0, tempN0, tempS0, tempE0, tempW0, tempT0, tempB0, tempNE0, tempNW0, tempSE0, tempSW0, tempNT0, tempNB0, tempST0, tempSB0, tempET0, tempEB0, tempWT0, tempWB0);
+        lbm_collide(__float_as_uint(in[r][LBM_FLAGS].y), tempC1, tempN1, tempS1, tempE1, tempW1, tempT1, tempB1, tempNE1, tempNW1, tempSE1, tempSW1, tempNT1, tempNB1, tempST1, tempSB1, tempET1, tempEB1, tempWT1, tempWB1);
+#define TK_LBM_SCATTER_ROW(entry, dx, dy, dz, name)                                        \
     do {                                                                                   \
-        const int t_ = (c_) + (dx) + (dy) * sx + (dz) * sxy;                               \
+        const int t_ = c[r] + (dx) + (dy) * sx + (dz) * sxy;                               \
         float *o_ = dst + cells * (entry) + t_;                                            \
         if (t_ >= 0 && t_ + 1 < cells) {                                                   \
-            lbm_store_pair(o_, lbm_pair_t{v0_, v1_});                    \
+            lbm_store_pair(o_, lbm_pair_t{name##0, name##1});                              \
         } else {                                                                           \
-            if (t_ >= 0 && t_ < cells) o_[0] = v0_;                                        \
-            if (t_ + 1 >= 0 && t_ + 1 < cells) o_[1] = v1_;                                \
+            if (t_ >= 0 && t_ < cells) o_[0] = name##0;                                    \
+            if (t_ + 1 >= 0 && t_ + 1 < cells) o_[1] = name##1;                            \
         }                                                                                  \
     } while (0);
-    // row a is collided and scattered while row b's loads are still on their way; the scheduling
-    // fences keep the two rows' arithmetic apart (interleaved it needs more registers than a fused
-    // kernel has)
-    __builtin_amdgcn_sched_barrier(0);
-    {
-#define TK_LBM_SPLIT(entry, dx, dy, dz, name) float name##0 = name##_a.x, name##1 = name##_a.y;
-        TK_LBM_DIRECTIONS(TK_LBM_SPLIT)
-#undef TK_LBM_SPLIT
-        lbm_collide(__float_as_uint(flags_a.x), tempC0, tempN0, tempS0, tempE0, tempW0, tempT0, tempB0, tempNE0, tempNW0, tempSE0, tempSW0, tempNT0, tempNB0, tempST0, tempSB0, tempET0, tempEB0, tempWT0, tempWB0);
-        lbm_collide(__float_as_uint(flags_a.y), tempC1, tempN1, tempS1, tempE1, tempW1, tempT1, tempB1, tempNE1, tempNW1, tempSE1, tempSW1, tempNT1, tempNB1, tempST1, tempSB1, tempET1, tempEB1, tempWT1, tempWB1);
-#define TK_LBM_SCATTER_A(entry, dx, dy, dz, name) TK_LBM_SCATTER_ROW(ca, entry, dx, dy, dz, name##0, name##1)
-        TK_LBM_DIRECTIONS(TK_LBM_SCATTER_A)
-#undef TK_LBM_SCATTER_A
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    {
-#define TK_LBM_SPLIT(entry, dx, dy, dz, name) float name##0 = name##_b.x, name##1 = name##_b.y;
-        TK_LBM_DIRECTIONS(TK_LBM_SPLIT)
-#undef TK_LBM_SPLIT
-        lbm_collide(__float_as_uint(flags_b.x), tempC0, tempN0, tempS0, tempE0, tempW0, tempT0, tempB0, tempNE0, tempNW0, tempSE0, tempSW0, tempNT0, tempNB0, tempST0, tempSB0, tempET0, tempEB0, tempWT0, tempWB0);
-        lbm_collide(__float_as_uint(flags_b.y), tempC1, tempN1, tempS1, tempE1, tempW1, tempT1, tempB1, tempNE1, tempNW1, tempSE1, tempSW1, tempNT1, tempNB1, tempST1, tempSB1, tempET1, tempEB1, tempWT1, tempWB1);
-#define TK_LBM_SCATTER_B(entry, dx, dy, dz, name) TK_LBM_SCATTER_ROW(cb, entry, dx, dy, dz, name##0, name##1)
-        TK_LBM_DIRECTIONS(TK_LBM_SCATTER_B)
-#undef TK_LBM_SCATTER_B
-    }
+        TK_LBM_DIRECTIONS(TK_LBM_SCATTER_ROW)
 #undef TK_LBM_SCATTER_ROW
+    }
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // grid_dimension_x = sy, grid_dimension_y = sz, block_dimension_x = sx
-// (src/ori_kernel/lbm_kernel.cu:218-222).  ROWS_PER_WAVE = 2: a wave takes two of its rows at a
-// time (see lbm_cell_pair_x2); which rows a wave owns is the same either way.
+// (src/ori_kernel/lbm_kernel.cu:218-222).  ROWS_PER_WAVE = N > 1: a wave takes N of its rows at a
+// time (see lbm_cell_pair_rows); which rows a wave owns is the same either way.
 template <int ROWS_PER_WAVE = 1>
 __device__ __forceinline__ void lbm_role(const float *__restrict__ src, float *__restrict__ dst,
                                          int grid_dimension_x, int grid_dimension_y,
@@ -271,13 +262,22 @@ __device__ __forceinline__ void lbm_role(const float *__restrict__ src, float *_
     }
     const unsigned stride = (unsigned)role_blocks * rows_at_once;
     unsigned pos = (unsigned)start + role_block * rows_at_once + row_slot;
-    if (ROWS_PER_WAVE == 2 && per_lane == 2) {
-        for (; pos + stride < (unsigned)end && pos + stride > pos; pos += 2 * stride) {
-            const unsigned pos_b = pos + stride;
-            const int row_a = (int)(pos % sy) * sx + (int)((pos / sy) % sz) * sxy;
-            const int row_b = (int)(pos_b % sy) * sx + (int)((pos_b / sy) % sz) * sxy;
-            for (int x = x_first; x < sx; x += x_step)
-                lbm_cell_pair_x2(src, dst, cells, x + row_a, x + row_b, sx, sxy);
+    if (ROWS_PER_WAVE > 1 && per_lane == 2) {
+        constexpr int N = ROWS_PER_WAVE > 1 ? ROWS_PER_WAVE : 2;
+        // while N more rows of this wave lie in the range (and the position does not wrap)
+        for (; (unsigned long long)pos + (unsigned long long)(N - 1) * stride < (unsigned)end; pos += N * stride) {
+            int row[N];
+#pragma unroll
+            for (int r = 0; r < N; ++r) {
+                const unsigned p = pos + (unsigned)r * stride;
+                row[r] = (int)(p % sy) * sx + (int)((p / sy) % sz) * sxy;
+            }
+            for (int x = x_first; x < sx; x += x_step) {
+                int c[N];
+#pragma unroll
+                for (int r = 0; r < N; ++r) c[r] = x + row[r];
+                lbm_cell_pair_rows<N>(src, dst, cells, c, sx, sxy);
+            }
         }
     }
     for (; pos < (unsigned)end; pos += stride) {

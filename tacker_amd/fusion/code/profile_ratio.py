@@ -165,15 +165,25 @@ def apply(in_path):
         if key not in dflt:
             raise SystemExit(f"{DEFAULTS} has no entry {key}: add the pair to the generator first")
         entry = dflt[key]
-        entry["ratio_by_k"] = {k: v["ratio"] for k, v in m["by_k"].items()}
-        entry["block_ratio"] = m["by_k"]["4096"]["ratio"]
+        ratios = {k: v["ratio"] for k, v in m["by_k"].items()}
+        # A pair's earnings change smoothly with K.  A K whose count clears the min_gain bar while both of
+        # its neighbours on the ladder earn nothing cleared it by the noise of the timings: not fused.
+        ks = sorted(ratios, key=int)
+        for i, k in enumerate(ks):
+            around = [ratios[ks[j]] for j in (i - 1, i + 1) if 0 <= j < len(ks)]
+            if ratios[k] > 0 and around and not any(r > 0 for r in around):
+                print(f"{key}: K = {k} earns alone among its neighbours ({m['by_k'][k]['ratio']}): taken as noise, ratio 0")
+                ratios[k] = 0.0
+        entry["ratio_by_k"] = ratios
+        entry["block_ratio"] = ratios["4096"]
         if "whole_kernel" in m:
             entry["whole_kernel_gain"] = m["whole_kernel"]["gain"]
     dflt["ratio_provenance"] = {"stretch": meas["stretch"], "min_gain": meas.get("min_gain", 0.0), "device": meas["device"],
                                 "method": "profile_ratio.py: GEMM 2048x2048xK; best-effort block count with "
                                           "the largest time earned over serial launches (at least min_gain of "
                                           "them) whose fused launch stays within (1+stretch) of the GEMM "
-                                          "alone, divided by 1024 tiles"}
+                                          "alone, divided by 1024 tiles; a K that earns while both "
+                                          "neighbouring K of the ladder do not is set to 0"}
     with open(DEFAULTS, "w") as f:
         json.dump(dflt, f, indent=2)
         f.write("\n")
