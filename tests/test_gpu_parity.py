@@ -382,6 +382,39 @@ def test_stencil_any_tiling_of_the_position_grid_is_one_sweep(shape, grid):
     assert np.array_equal(host(one), oracle.stencil_gptb(C0, C1, A0, np.full_like(A0, -3.0), s, e, gdz="runs"))
 
 
+@pytest.mark.parametrize("ny,grid", [(256, 8), (256, 64), (128, 16), (192, 32)])
+def test_stencil_slab_numbering_of_the_wide_form_is_one_sweep(ny, grid):
+    # ranges long enough for the plane-by-plane march: with 64 or 32 quad rows the tasks are numbered by
+    # XCD slabs (256 rows: for 4 and for 8 waves a workgroup; 128 rows: for 4 only), with 48 in the plain
+    # order; any tiling by ranges, in any order, gives the bits of one sweep, alone and fused
+    nz, nx = (66 if ny > 128 else 130), 512
+    A0 = stencil_inputs(nz, ny, nx, seed=ny + grid)
+    npos = ta.stencil_blocks(nx, ny, nz)
+    assert npos == 8 * (ny // 4) * ((nz - 2) // 8) and npos > 2048
+    want = oracle.stencil(C0, C1, A0, np.full_like(A0, -3.0))
+    a0 = dev(A0)
+    rng = np.random.default_rng(ny + grid)
+    cuts = sorted(set([0, npos] + [int(c) for c in rng.integers(1, npos, 3)]))
+    ranges = list(zip(cuts[:-1], cuts[1:]))
+    acc = torch.full_like(a0, -3.0)
+    for i in rng.permutation(len(ranges)):
+        ta.gptb_stencil(C0, C1, a0, acc, start=ranges[i][0], end=ranges[i][1], launch_grid=grid)
+    assert np.array_equal(host(acc), want)
+    whole = torch.full_like(a0, -3.0)
+    ta.gptb_stencil(C0, C1, a0, whole, launch_grid=grid)
+    assert np.array_equal(host(whole), want)
+    # the same ranges riding with a GEMM (8 best-effort waves a workgroup)
+    gA, gB = gemm_inputs(256, 256, 256, 5)
+    dA, dB = dev(gA), dev(gB)
+    Cm = torch.zeros((256, 256), device="cuda:0")
+    fused = torch.full_like(a0, -3.0)
+    for i in rng.permutation(len(ranges)):
+        ta.mix_tzgemm_stencil(C0, C1, a0, fused, dA, dB, Cm, be_start=ranges[i][0], be_end=ranges[i][1],
+                              variant="wave_512", launch_grid=grid)
+    assert np.array_equal(host(fused), want)
+    assert ta.spin_fail_flag() == 0
+
+
 def test_stencil_iterations_ping_pong():
     A0 = stencil_inputs(6, 16, 128)
     a, b = dev(A0), dev(A0)
