@@ -428,6 +428,79 @@ def lc_leg(ta, torch, np, queries, be_name="stencil", be_label="stencil 512x512x
     return out
 
 
+class PowerSampler:
+    """socket power from the driver's hwmon file (microwatts), sampled from a thread while a leg runs; None
+    where the file is absent or unreadable"""
+
+    def __init__(self):
+        import glob
+        self.files = glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input")
+        self.cap = None
+        for f in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"):
+            try:
+                self.cap = int(open(f).read()) / 1e6
+            except (OSError, ValueError):
+                pass
+        self.samples = []
+        self.stop = False
+        self.thread = None
+
+    def usable(self):
+        try:
+            return bool(self.files) and int(open(self.files[0]).read()) > 0
+        except (OSError, ValueError):
+            return False
+
+    def start(self):
+        import threading
+
+        def poll():
+            while not self.stop:
+                try:
+                    self.samples.append((time.perf_counter(), int(open(self.files[0]).read()) / 1e6))
+                except (OSError, ValueError):
+                    pass
+                time.sleep(0.02)
+        self.thread = threading.Thread(target=poll, daemon=True)
+        self.thread.start()
+
+    def mean_between(self, t0, t1):
+        w = [p for t, p in self.samples if t0 <= t <= t1]
+        return sum(w) / len(w) if w else None
+
+    def close(self):
+        self.stop = True
+        if self.thread:
+            self.thread.join()
+
+
+def power_leg(torch, job, seconds=1.5):
+    """config 2's four jobs again, each looped for `seconds` with the socket power sampled every 20 ms (the first
+    half second of a loop is left out: the sensor averages): is the fused launch held by the power limit?"""
+    sampler = PowerSampler()
+    if not sampler.usable():
+        return None
+    sampler.start()
+    out = {"cap_w": sampler.cap, "sensor": "hwmon power1_input, 20 ms samples, loops of %.1f s" % seconds}
+    for kind in ("gemm", "stencil", "serial", "fused"):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        n = 0
+        while time.perf_counter() - t0 < seconds:
+            job(kind)
+            torch.cuda.synchronize()
+            n += ITERATIONS
+        t1 = time.perf_counter()
+        w = sampler.mean_between(t0 + 0.5, t1)
+        us = (t1 - t0) / n * 1e6
+        out[kind] = {"mean_w": round(w, 0) if w else None, "us_per_iteration_incl_host": round(us, 2),
+                     "mj_per_iteration": round(w * us * 1e-3, 2) if w else None}
+    sampler.close()
+    if out["fused"]["mean_w"] and sampler.cap:
+        out["fused_frac_of_cap"] = round(out["fused"]["mean_w"] / sampler.cap, 3)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -528,6 +601,9 @@ def main():
     # the roofline and the summaries of every pair.
     out = {}
     if not args.no_extras:
+        power = power_leg(torch, job)
+        if power:
+            out["power"] = power
         if args.pairs == ap.get_default("pairs"):
             out["tzgemm_shapes"] = gemm_leg(ta, torch, np, stream)
         out["other_pairs"] = {name: pair_leg(ta, torch, np, name, stream) for name in args.pairs.split(",") if name}
@@ -570,6 +646,9 @@ def main():
                                      e.get("colocated_p99_ms"), e.get("qos_bound_ms"), e.get("p99_within_bound"),
                                      out[key]["time_earned_ms_per_query"], out[key]["be_work_ms_per_query"],
                                      out[key]["mixed_launches_per_query"], e.get("earned_ms_per_query")]
+    if "power" in out:
+        # [GEMM alone W, stencil alone W, serial job W, fused job W, cap W]: is the fused launch held by the power limit?
+        out["power_summary"] = [out["power"][k]["mean_w"] for k in ("gemm", "stencil", "serial", "fused")] + [out["power"]["cap_w"]]
     out.update({
         "wall_s_timed_region": round(t_wall, 3),
         "overlap_efficiency": round(max(ms["gemm"], ms["stencil"]) / ms["fused"], 4),
