@@ -229,6 +229,35 @@ def test_measured_load_ratios_travel_from_profile_ratio_to_the_schedulers_lookup
     assert [float(v) for v in got[:3]] == [2.25, 5.25, 10.5] and int(got[3]) == int(1024 * 4.25)
 
 
+def test_a_load_ratio_that_earns_alone_among_its_neighbours_is_taken_as_noise(tmp_path, monkeypatch, capsys):
+    # a K whose count cleared the bar while both neighbouring K of the ladder earn nothing is set to 0;
+    # positive neighbours keep each other, and so do the ends of the ladder next to a positive K
+    import shutil
+    import profile_ratio
+    dflt = tmp_path / "defaults.json"
+    shutil.copy(os.path.join(GEN, "defaults.json"), dflt)
+    monkeypatch.setattr(profile_ratio, "DEFAULTS", str(dflt))
+    ks = [str(k) for k in profile_ratio.K_LADDER]
+    def measured(ratios):
+        return {"stretch": 1.0, "min_gain": 0.03, "tiles": 1024, "device": "test double",
+                "pairs": {"tzgemm_lbm": {"by_k": {k: {"blocks": int(r * 1024), "ratio": r} for k, r in zip(ks, ratios)},
+                                         "whole_kernel": {"serial_us": 100.0, "fused_us": 98.0, "gain": 1.0204}}}}
+    src = tmp_path / "m.json"
+    src.write_text(json.dumps(measured([0.0, 0.0, 0.0, 1.5, 0.0, 1.5, 0.0])))
+    profile_ratio.apply(str(src))
+    lbm = json.loads(dflt.read_text())["tzgemm_lbm"]
+    assert set(lbm["ratio_by_k"].values()) == {0.0} and lbm["block_ratio"] == 0.0 and lbm["whole_kernel_gain"] == 1.0204
+    assert capsys.readouterr().out.count("taken as noise") == 2
+    src.write_text(json.dumps(measured([2.0, 0.0, 0.0, 1.5, 1.0, 0.0, 3.0])))
+    profile_ratio.apply(str(src))
+    lbm = json.loads(dflt.read_text())["tzgemm_lbm"]
+    assert [lbm["ratio_by_k"][k] for k in ks] == [0.0, 0.0, 0.0, 1.5, 1.0, 0.0, 0.0]
+    src.write_text(json.dumps(measured([2.0, 1.0, 0.0, 0.0, 0.0, 2.5, 3.0])))
+    profile_ratio.apply(str(src))
+    lbm = json.loads(dflt.read_text())["tzgemm_lbm"]
+    assert [lbm["ratio_by_k"][k] for k in ks] == [2.0, 1.0, 0.0, 0.0, 0.0, 2.5, 3.0] and lbm["block_ratio"] == 2.5
+
+
 def test_profile_tools_import_without_a_gpu_and_know_every_kernel():
     import profile_gptb
     import profile_ratio
